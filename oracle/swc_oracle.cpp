@@ -1,0 +1,262 @@
+// CPU oracle for the SWCompiler inference kernels.
+//
+// THIS FILE IS TEST INFRASTRUCTURE.  It is the checker that the HIP kernels are
+// compared against; it is never linked into, loaded by or called from the
+// shipped library.  Only tests/, __graft_entry__.smoke() and bench.py's
+// cpu_baseline leg may use it.
+//
+// Every function restates the arithmetic of one kernel of the reference's
+// generated-code support header (src/codegen/utils/kernels.h) such that each
+// output element sees exactly the same sequence of IEEE-754 operations as in
+// the reference; loops are reordered for cache locality only where that does
+// not change the per-element operation order.  Build without FMA contraction
+// (see oracle/Makefile: -ffp-contract=off, no -ffast-math) or results drift.
+//
+// Pinning status (what proves this file equals the reference):
+//   * every function below is compared bit-for-bit with the reference header
+//     itself, compiled from /root/reference into oracle/_ref/libswc_ref.so,
+//     on seeded inputs (tests/test_oracle_vs_ref.py, skipped when the
+//     reference tree is absent);
+//   * the outputs of that reference build are committed as fixtures under
+//     tests/golden/ and checked on every run (tests/test_oracle_golden.py);
+//   * the MNIST-8 known answer of the reference's test inputs and closed-form
+//     / invariant checks (tests/test_oracle_math.py).
+//   No function here is "parity unpinned".
+
+#include <cmath>
+#include <cstddef>
+#include <cstdint>
+#include <cstring>
+#include <sys/types.h>
+#include <utility>
+#include <vector>
+#include <algorithm>
+
+namespace {
+
+struct Dims4 {
+    size_t d0, d1, d2, d3;
+    explicit Dims4(const size_t *p) : d0(p[0]), d1(p[1]), d2(p[2]), d3(p[3]) {}
+    // row-major flat index, kernels.h:154-158
+    size_t at(size_t a, size_t b, size_t c, size_t d) const {
+        return ((a * d1 + b) * d2 + c) * d3 + d;
+    }
+};
+
+} // namespace
+
+extern "C" {
+
+// kernels.h:41-56.  C[i,j] starts at 0.f and receives fl(A[i,p]*B[p,j]) for
+// p = 0..k-1 in order, each product rounded to fp32 before the fp32 add.
+// The reference iterates p,j,i; here i,p,j — per element the order over p is
+// the same, so the bits are the same.
+void oracle_matrixMatrixMul_f(int m, int n, int k, const float *a, int lda,
+                              const float *b, int ldb, float *c, int ldc) {
+    for (int i = 0; i < m; ++i) {
+        float *crow = c + (size_t)i * ldc;
+        for (int j = 0; j < n; ++j) crow[j] = 0.f;
+        const float *arow = a + (size_t)i * lda;
+        for (int p = 0; p < k; ++p) {
+            const float av = arow[p];
+            const float *brow = b + (size_t)p * ldb;
+            for (int j = 0; j < n; ++j) crow[j] += av * brow[j];
+        }
+    }
+}
+
+// kernels.h:58-64.  All fp32: 1 - 2/(expf(2x)+1).
+void oracle_matrixTanh_f(int m, int n, const float *a, int lda, float *b,
+                         int ldb) {
+    for (int i = 0; i < m; ++i)
+        for (int j = 0; j < n; ++j) {
+            float e = expf(a[(size_t)i * lda + j] * 2);
+            b[(size_t)i * ldb + j] = 1 - 2 / (e + 1);
+        }
+}
+
+// kernels.h:88-103.  Row max via std::max starting from element 0 (so a NaN
+// in a later column is ignored and a NaN in column 0 sticks), expf of the
+// shifted value, sequential fp32 sum left to right, true division.
+void oracle_matrixSoftmax_f(int m, int n, const float *a, int lda, float *b,
+                            int ldb) {
+    for (int i = 0; i < m; ++i) {
+        const float *x = a + (size_t)i * lda;
+        float *y = b + (size_t)i * ldb;
+        float mx = x[0];
+        for (int j = 0; j < n; ++j) mx = (mx < x[j]) ? x[j] : mx;
+        float total = 0;
+        for (int j = 0; j < n; ++j) {
+            y[j] = expf(x[j] - mx);
+            total += y[j];
+        }
+        for (int j = 0; j < n; ++j) y[j] = y[j] / total;
+    }
+}
+
+// kernels.h:163-243 (conv2d_set_bias + conv2d_f), NHWC input, [oC,kH,kW,iC]
+// filter.  Each output starts at bias[co] and then receives the in-bounds taps
+// in (kx, ky, ci) order, product rounded to fp32 then added in fp32.  Only
+// pads[0] (top) and pads[1] (left) take part in the index arithmetic.  The
+// reference adds g*inCG to the last filter axis for group g; kept literally.
+void oracle_conv2d_f(float *output, const float *input, const float *filter,
+                     const float *bias, const size_t *odims,
+                     const size_t *idims, const size_t *fdims,
+                     const size_t * /*bdims*/, const size_t *kernels,
+                     const size_t *strides, const size_t *pads, size_t group) {
+    const Dims4 O(odims), I(idims), F(fdims);
+    const size_t cin_g = I.d3 / group, cout_g = O.d3 / group;
+    const ssize_t kh = kernels[0], kw = kernels[1];
+    const ssize_t sh = strides[0], sw = strides[1];
+    const ssize_t pt = pads[0], pl = pads[1];
+    for (size_t n = 0; n < I.d0; ++n)
+        for (size_t ox = 0; ox < O.d1; ++ox)
+            for (size_t oy = 0; oy < O.d2; ++oy)
+                for (size_t co = 0; co < O.d3; ++co) {
+                    const size_t g = co / cout_g;
+                    float acc = bias[co];
+                    for (ssize_t kx = 0; kx < kh; ++kx) {
+                        const ssize_t ix = (ssize_t)ox * sh - pt + kx;
+                        if (ix < 0 || ix >= (ssize_t)I.d1) continue;
+                        for (ssize_t ky = 0; ky < kw; ++ky) {
+                            const ssize_t iy = (ssize_t)oy * sw - pl + ky;
+                            if (iy < 0 || iy >= (ssize_t)I.d2) continue;
+                            const float *ip =
+                                input + I.at(n, ix, iy, g * cin_g);
+                            const float *fp =
+                                filter + F.at(co, kx, ky, g * cin_g);
+                            for (size_t ci = 0; ci < cin_g; ++ci)
+                                acc += ip[ci] * fp[ci];
+                        }
+                    }
+                    output[O.at(n, ox, oy, co)] = acc;
+                }
+}
+
+// kernels.h:323-377 (values) and the index bookkeeping of kernels.h:407-436.
+// The first in-bounds tap initialises the running maximum; a later tap
+// replaces it only when strictly greater (NaN never replaces; a NaN first tap
+// is never replaced).  A window with no in-bounds tap yields 0.
+// argmax (may be null) receives the flat NHWC input index of the chosen tap,
+// or -1 for an empty window.
+void oracle_maxpool_argmax_f(const float *input, float *output, int32_t *argmax,
+                             const size_t *idims, const size_t *odims,
+                             const size_t *kernels, const size_t *strides,
+                             const size_t *pads) {
+    const Dims4 I(idims), O(odims);
+    const ssize_t kh = kernels[0], kw = kernels[1];
+    const ssize_t sh = strides[0], sw = strides[1];
+    const ssize_t pt = pads[0], pl = pads[1];
+    for (size_t n = 0; n < I.d0; ++n)
+        for (size_t ox = 0; ox < O.d1; ++ox)
+            for (size_t oy = 0; oy < O.d2; ++oy)
+                for (size_t c = 0; c < I.d3; ++c) {
+                    bool have = false;
+                    float best = 0;
+                    int64_t where = -1;
+                    for (ssize_t kx = 0; kx < kh; ++kx) {
+                        const ssize_t ix = (ssize_t)ox * sh - pt + kx;
+                        if (ix < 0 || ix >= (ssize_t)I.d1) continue;
+                        for (ssize_t ky = 0; ky < kw; ++ky) {
+                            const ssize_t iy = (ssize_t)oy * sw - pl + ky;
+                            if (iy < 0 || iy >= (ssize_t)I.d2) continue;
+                            const size_t idx = I.at(n, ix, iy, c);
+                            const float v = input[idx];
+                            if (!have || v > best) {
+                                best = v;
+                                where = (int64_t)idx;
+                                have = true;
+                            }
+                        }
+                    }
+                    const size_t o = O.at(n, ox, oy, c);
+                    output[o] = best;
+                    if (argmax) argmax[o] = (int32_t)where;
+                }
+}
+
+void oracle_maxpool_f(const float *input, float *output, const size_t *idims,
+                      const size_t *odims, const size_t *kernels,
+                      const size_t *strides, const size_t *pads) {
+    oracle_maxpool_argmax_f(input, output, nullptr, idims, odims, kernels,
+                            strides, pads);
+}
+
+// kernels.h:496-517.  var[c]+epsilon is an fp32 add; std::pow(float,double)
+// promotes, so everything after it is double arithmetic, rounded to fp32 once
+// on the store: ((in-mean) -> double) * pow(.) * scale + bias.
+void oracle_batchnormalization_f(float *output, const float *input,
+                                 const float *mean, const float *var,
+                                 const float *scale, const float *bias,
+                                 const size_t *idims, float epsilon) {
+    const size_t C = idims[3];
+    const size_t rows = idims[0] * idims[1] * idims[2];
+    std::vector<double> rs(C);
+    for (size_t c = 0; c < C; ++c) {
+        const float ve = var[c] + epsilon;
+        rs[c] = std::pow((double)ve, -0.5);
+    }
+    for (size_t r = 0; r < rows; ++r) {
+        const float *x = input + r * C;
+        float *y = output + r * C;
+        for (size_t c = 0; c < C; ++c) {
+            const float centred = x[c] - mean[c];
+            y[c] = (float)((double)centred * rs[c] * (double)scale[c] +
+                           (double)bias[c]);
+        }
+    }
+}
+
+// kernels.h:542-552.
+void oracle_batchedadd_f(float *dest, const float *batch, const float *slice,
+                         size_t numSlice, size_t sliceSize) {
+    for (size_t r = 0; r < numSlice; ++r)
+        for (size_t j = 0; j < sliceSize; ++j)
+            dest[r * sliceSize + j] = batch[r * sliceSize + j] + slice[j];
+}
+
+// kernels.h:575-580.  (x > 0) ? x : 0 — so -0.0 -> +0.0 and NaN -> 0.
+void oracle_relu_f(const float *src, float *dest, size_t size) {
+    for (size_t i = 0; i < size; ++i) dest[i] = (src[i] > 0) ? src[i] : 0;
+}
+
+// kernels.h:592-596.
+void oracle_vecAdd_f(int size, const float *a, const float *b, float *c) {
+    for (int i = 0; i < size; ++i) c[i] = a[i] + b[i];
+}
+
+// kernels.h:601-613.  Top-k column indices per row, ordered by descending
+// (value, index) pairs: equal values list the larger index first.
+void oracle_argMax_i(const float *input, int *idx, int m, int n, int top_k) {
+    std::vector<int> order(n);
+    for (int i = 0; i < m; ++i) {
+        const float *row = input + (size_t)i * n;
+        for (int j = 0; j < n; ++j) order[j] = j;
+        std::stable_sort(order.begin(), order.end(), [row](int p, int q) {
+            if (row[p] > row[q]) return true;
+            if (row[q] > row[p]) return false;
+            return p > q;
+        });
+        for (int j = 0; j < top_k; ++j) idx[(size_t)i * top_k + j] = order[j];
+    }
+}
+
+// image.h:13-33: raw little-endian fp32 file, `offset` counted in elements.
+// Returns the number of elements copied, or -1 if the file cannot be read.
+long oracle_load_f(float *data, size_t size, size_t offset, const char *path);
+
+} // extern "C"
+
+#include <cstdio>
+extern "C" long oracle_load_f(float *data, size_t size, size_t offset,
+                              const char *path) {
+    FILE *f = std::fopen(path, "rb");
+    if (!f) return -1;
+    if (std::fseek(f, (long)(offset * sizeof(float)), SEEK_SET) != 0) {
+        std::fclose(f);
+        return -1;
+    }
+    size_t got = std::fread(data, sizeof(float), size, f);
+    std::fclose(f);
+    return got == size ? (long)got : -1;
+}
