@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Benchmark of the SWCompiler inference path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--headline-only] [--no-cpu]
+
+Headline workload (the configuration the metric is quoted on): the wide MLP,
+batch 4096 x 784 -> FC 4096 + ReLU -> FC 4096 + ReLU -> FC 10 -> softmax, fp32,
+as the HIP target emits it (bias and ReLU in the GEMM epilogue).  One step = one
+pass of that graph over one batch already resident in HBM.  Prints ONE JSON
+line; `value` is samples/s over exactly K timed steps.
+
+Also in the line:
+  roofline      the dominant kernel (the tiled fp32-MFMA GEMM: both of its
+                launches per step, 4096x784x4096 and 4096x4096x4096), timed
+                with HIP events on the library's stream inside the timed region
+  kernels       per-launch times of the headline graph
+  configs       the other synthetic configurations (samples/s and, per kernel,
+                TFLOP/s or GB/s with the fraction of the MI355X peak)
+  cpu_baseline  the reference's own CPU kernels (oracle/_ref, g++ -std=c++11 -O2,
+                one thread) on the first rows of the same batch
+
+The CPU checker is used only for the cpu_baseline leg.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+
+PEAK_TFLOPS_FP32_MFMA = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+class Timed:
+    """Proxy of the runtime that records a HIP event before and after every op."""
+
+    def __init__(self, rt):
+        self.rt = rt
+        self.log = []   # (op name, slot0, slot1, work dict)
+        self.slot = 0
+
+    def reset(self):
+        self.log, self.slot = [], 0
+
+    def _wrap(self, name, work_fn):
+        fn = getattr(self.rt, name)
+
+        def call(*a, **kw):
+            s0 = self.slot
+            self.slot += 2
+            self.rt.event_record(s0)
+            out = fn(*a, **kw)
+            self.rt.event_record(s0 + 1)
+            self.log.append((name, s0, s0 + 1, work_fn(out, *a, **kw)))
+            return out
+        return call
+
+    def __getattr__(self, name):
+        return self._wrap(name, WORK[name])
+
+    def results(self):
+        rows = []
+        for name, s0, s1, work in self.log:
+            ms = self.rt.event_elapsed_ms(s0, s1)
+            rows.append(dict(op=name, ms=ms, **work))
+        return rows
+
+
+def _gemm_work(res, a, b, *r, **kw):
+    m, k = a.shape
+    n = b.shape[1]
+    return dict(shape=f"{m}x{k}x{n}", flop=2.0 * m * n * k)
+
+
+def _conv_work(res, x, f, *r, **kw):
+    m = res.size // res.shape[3]
+    k = f.shape[1] * f.shape[2] * f.shape[3]
+    return dict(shape=f"{list(x.shape)}*{list(f.shape)}", flop=2.0 * m * f.shape[0] * k)
+
+
+def _bytes(per_in=0, per_out=0, n_in=1):
+    def fn(res, x, *r, **kw):
+        return dict(shape=str(list(x.shape)), bytes=float(x.size * per_in * n_in + res.size * per_out))
+    return fn
+
+
+# algorithmic work per op: GEMM 2mnk, conv 2*M*oC*K; bandwidth ops count every
+# input element read once and every output element written once (4 B each).
+WORK = {
+    "matrixMatrixMul": _gemm_work, "fcbias": _gemm_work, "conv2d": _conv_work,
+    "relu": _bytes(4, 4), "batchedadd": _bytes(4, 4), "vecAdd": _bytes(4, 4, n_in=2),
+    "batchnormalization": _bytes(4, 4), "maxpool": _bytes(4, 4), "matrixSoftmax": _bytes(4, 4),
+    "batchnormReluMaxpool": _bytes(4, 4),
+}
+
+
+def rate(row):
+    """adds achieved rate and roofline fraction to a kernel row"""
+    s = row["ms"] * 1e-3
+    if "flop" in row:
+        row["tflops"] = row["flop"] / s / 1e12
+        row["frac"] = row["tflops"] / PEAK_TFLOPS_FP32_MFMA
+        row["bound"] = "mfma"
+    else:
+        row["gbs"] = row["bytes"] / s / 1e9
+        row["frac"] = row["gbs"] / PEAK_HBM_GBS
+        row["bound"] = "hbm"
+    return row
+
+
+def merge_rows(all_rows):
+    """average per-launch rows of repeated steps (same op order every step)"""
+    n = len(all_rows)
+    out = []
+    for i, row in enumerate(all_rows[0]):
+        r = dict(row)
+        r["ms"] = sum(step[i]["ms"] for step in all_rows) / n
+        out.append(rate(r))
+    return out
+
+
+def run_config(rt, graphs, cfg, steps, warmup):
+    t = graphs.make_inputs(cfg)
+    dt = {k: rt.upload(v) for k, v in t.items()}
+    batch = graphs.batch_of(cfg, t)
+    ws = {}
+    for _ in range(max(warmup, 1)):
+        graphs.run(cfg, rt, dt, fused=True, ws=ws)
+    rt.sync()
+    timed = Timed(rt)
+    per_step = []
+    t0 = time.perf_counter()
+    rt.timer_begin()
+    for _ in range(steps):
+        timed.log = []
+        graphs.run(cfg, timed, dt, fused=True, ws=ws)
+        per_step.append(timed.log)
+    gpu_ms = rt.timer_end_ms()
+    rt.sync()
+    wall = time.perf_counter() - t0
+    # events were recorded into distinct slots per step; read them now
+    all_rows = []
+    for log in per_step:
+        timed.log = log
+        all_rows.append(timed.results())
+    rows = merge_rows(all_rows)
+    return dict(batch=batch, wall_s=wall, gpu_ms=gpu_ms, ms_per_step=wall * 1e3 / steps,
+                samples_per_s=batch * steps / wall, kernels=rows)
+
+
+def cpu_baseline(graphs, rows=64):
+    """The reference's CPU kernels on the first `rows` rows of the headline batch."""
+    from oracle import binding
+    if binding.ref_available():
+        be, kind = binding.load_ref(), "reference"
+    else:
+        be, kind = binding.load_oracle(), "port"
+    t = graphs.make_inputs(2)
+    t["x"] = np.ascontiguousarray(t["x"][:rows])
+    t0 = time.perf_counter()
+    graphs.run(2, be, t, fused=False)
+    dt = time.perf_counter() - t0
+    return dict(value=rows / dt, unit="samples/s", cores=1, kind=kind, seconds=dt,
+                sample=f"first {rows} of the 4096 rows of the same batch through the whole graph "
+                       f"(matrixMatrixMul_f, batchedadd_f, relu_f, matrixSoftmax_f as the reference emits them), "
+                       f"one thread, g++ -std=c++11 -O2; {os.cpu_count()} host cpus visible")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--headline-only", action="store_true", help="skip the other configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-rows", type=int, default=64)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (nothing is sharded); use --gpus 1")
+
+    from swcompiler_amd import graphs
+    from swcompiler_amd.hip import runtime
+    rt = runtime()
+
+    head = run_config(rt, graphs, 2, args.steps, args.warmup)
+    gemm = [r for r in head["kernels"] if r["op"] == "fcbias" and not r["shape"].endswith("x10")]
+    flop = sum(r["flop"] for r in gemm)
+    secs = sum(r["ms"] for r in gemm) * 1e-3
+    achieved = flop / secs / 1e12
+    out = {
+        "metric": "samples/s per graph; TFLOP/s (FC/conv) & GB/s (eltwise) vs MI355X roofline",
+        "value": head["samples_per_s"], "unit": "samples/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "wide MLP: batch 4096x784 -> FC4096+ReLU -> FC4096+ReLU -> FC10 -> softmax, fp32 "
+                               "(BASELINE.json configs[1]), fused epilogues",
+                   "global_batch": head["batch"], "device": rt.device_name()},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS_FP32_MFMA, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_TFLOPS_FP32_MFMA, "traffic": None,
+                     "kernel": "gemm_tiled<2,2,true> (both launches per step: 4096x784x4096 and 4096x4096x4096)",
+                     "flop_per_launch": flop / len(gemm), "avg_launch_ms": secs * 1e3 / len(gemm)},
+        "gpu_ms_per_step": head["gpu_ms"] / args.steps,
+        "kernels": head["kernels"],
+    }
+    if not args.headline_only:
+        others = {}
+        for cfg in (1, 3, 4, 5):
+            steps = max(5, min(args.steps, 20))
+            r = run_config(rt, graphs, cfg, steps, max(2, min(args.warmup, 5)))
+            others[f"cfg{cfg}"] = dict(batch=r["batch"], samples_per_s=r["samples_per_s"], ms_per_step=r["ms_per_step"],
+                                       gpu_ms_per_step=r["gpu_ms"] / steps, kernels=r["kernels"])
+        out["configs"] = others
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(graphs, args.cpu_rows)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

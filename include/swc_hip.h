@@ -1,0 +1,176 @@
+/*
+ * swc_hip.h — C ABI of libswc_hip, the MI355X (gfx950) runtime that generated
+ * SWCompiler host programs call.
+ *
+ * The reference has no runtime library: its generated Graph.cpp calls C
+ * functions of a header copied next to it (src/codegen/utils/kernels.h) on
+ * host memory.  Each op entry point below takes the SAME argument list, in the
+ * same order and with the same meaning, as the CPU function the reference's
+ * code generator emits for that op (file:line given per function), so that a
+ * generated call site differs only by the `swc_hip_` prefix.  Differences:
+ *   - every data pointer is a DEVICE pointer (from swc_hip_malloc, or any HIP
+ *     device allocation, e.g. a torch tensor's data_ptr());
+ *   - the small `const size_t*` shape arrays (dims, kernels, strides, pads) stay
+ *     HOST pointers, read before the call returns;
+ *   - every function returns 0 on success and a non-zero SWC_HIP_E* code on
+ *     failure, with a message kept for swc_hip_last_error().  (The reference's
+ *     convention is "ignore or exit", src/codegen/utils/image.h:17-20.)
+ *   - ops are asynchronous on one in-order HIP stream per process (the
+ *     reference's CUDA path uses one stream per GPU,
+ *     src/codegen/Codegen.cpp:166-172); call swc_hip_sync() before reading
+ *     results on the host.  swc_hip_d2h synchronises by itself.
+ * Nothing here allocates device memory except swc_hip_malloc.
+ * Layouts are the reference's: 4-D activations NHWC, conv filters
+ * [oC, kH, kW, iC], matrices row-major.  All data is fp32.
+ */
+#ifndef SWC_HIP_H_
+#define SWC_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    SWC_HIP_OK = 0,
+    SWC_HIP_EINVAL = 1,      /* bad argument (null pointer, negative size, shape mismatch) */
+    SWC_HIP_EUNSUPPORTED = 2,/* valid in the reference but not implemented here (e.g. group != 1) */
+    SWC_HIP_ERUNTIME = 3,    /* a HIP call failed; message holds hipGetErrorString */
+    SWC_HIP_ENOTINIT = 4     /* swc_hip_init has not succeeded in this process */
+};
+
+/* ---- runtime: replaces the cudaSetDevice/cudaMalloc/cudaMemcpy/cudaFree and
+ * stream set-up lines the reference prints (src/codegen/Codegen.cpp:154-172,
+ * 504-521, 1134-1169, 2499-2526). ---- */
+int swc_hip_init(int device);                 /* idempotent; selects device, creates the stream */
+int swc_hip_shutdown(void);                   /* destroys the stream; outstanding allocations stay valid */
+void *swc_hip_malloc(size_t bytes);           /* 256-byte aligned device memory, NULL on failure */
+int swc_hip_free(void *dptr);
+int swc_hip_h2d(void *dst_dev, const void *src_host, size_t bytes); /* ordered after prior ops, returns when done */
+int swc_hip_d2h(void *dst_host, const void *src_dev, size_t bytes); /* ordered after prior ops, returns when done */
+int swc_hip_d2d(void *dst_dev, const void *src_dev, size_t bytes);  /* async on the stream */
+int swc_hip_fill_f(float *dst_dev, float value, size_t count);      /* initTensorConstant/Zero, kernels.h:23-29 */
+int swc_hip_sync(void);
+const char *swc_hip_last_error(void);         /* message of the last failure on this thread ("" if none) */
+void *swc_hip_stream(void);                   /* the hipStream_t ops are launched on */
+int swc_hip_set_stream(void *hip_stream);     /* launch on a caller-owned stream (NULL: back to the library's own) */
+const char *swc_hip_device_name(void);        /* gcnArchName of the selected device */
+
+/* Event timing on the library's stream, for harnesses: begin/end bracket a
+ * region; elapsed returns milliseconds of the last closed region. */
+int swc_hip_timer_begin(void);
+int swc_hip_timer_end(void);                  /* records the end event and waits for it */
+float swc_hip_timer_elapsed_ms(void);
+/* Numbered events (slots 0..4095) recorded on the current stream, so a harness
+ * can time individual kernels inside a longer timed region. elapsed waits for
+ * `second` and returns milliseconds, or a negative value on error. */
+int swc_hip_event_record(int slot);
+float swc_hip_event_elapsed_ms(int first, int second);
+
+/* ---- ops: same arguments as the reference's CPU kernels ---- */
+
+/* kernels.h:41-56; emitted at Codegen.cpp:1334-1337 with lda=k, ldb=n, ldc=n.
+ * C[m,n] = A[m,k] * B[k,n], row-major, leading dimensions in elements. */
+int swc_hip_matrixMatrixMul_f(int m, int n, int k, const float *a, int lda,
+                              const float *b, int ldb, float *c, int ldc);
+
+/* kernels.h:542-552; emitted at Codegen.cpp:1513-1515.
+ * dest[r,j] = batch[r,j] + slice[j]. dest may alias batch. */
+int swc_hip_batchedadd_f(float *dest, const float *batch, const float *slice,
+                         size_t numSlice, size_t sliceSize);
+
+/* kernels.h:575-580; Codegen.cpp:2134-2135. dest = (src > 0) ? src : 0, bit-exact
+ * (-0 -> +0, NaN -> 0). dest may alias src. */
+int swc_hip_relu_f(const float *src, float *dest, size_t size);
+
+/* kernels.h:592-596; Codegen.cpp:1608-1610. c = a + b. c may alias a or b. */
+int swc_hip_vecAdd_f(int size, const float *a, const float *b, float *c);
+
+/* kernels.h:177-243; Codegen.cpp:1777-1782.  NHWC input idims[4], filter
+ * fdims = {oC,kH,kW,iC}, bias bdims = {oC}, output odims[4]; pads = {t,l,b,r} of
+ * which only t and l enter the index arithmetic (as in the reference); group
+ * must be 1.  out = bias + sum over in-bounds taps. */
+int swc_hip_conv2d_f(float *output, const float *input, const float *filter,
+                     const float *bias, const size_t *odims, const size_t *idims,
+                     const size_t *fdims, const size_t *bdims,
+                     const size_t *kernels, const size_t *strides,
+                     const size_t *pads, size_t group);
+
+/* kernels.h:496-517; Codegen.cpp:1910-1915.  NHWC, per-channel parameters,
+ * out = (in-mean)*pow(var+eps,-0.5)*scale+bias evaluated in double. */
+int swc_hip_batchnormalization_f(float *output, const float *input,
+                                 const float *mean, const float *var,
+                                 const float *scale, const float *bias,
+                                 const size_t *idims, float epsilon);
+
+/* kernels.h:323-377; Codegen.cpp:2033-2037.  NHWC window max, first maximum
+ * in (kx,ky) scan order wins, out-of-bounds taps skipped, bit-exact. */
+int swc_hip_maxpool_f(const float *input, float *output, const size_t *idims,
+                      const size_t *odims, const size_t *kernels,
+                      const size_t *strides, const size_t *pads);
+
+/* Same values as swc_hip_maxpool_f plus the flat NHWC input index of the
+ * chosen tap (-1 for a window with no in-bounds tap): the bookkeeping the
+ * reference keeps only inside maxpoolGrad_f (kernels.h:407-436). */
+int swc_hip_maxpool_argmax_f(const float *input, float *output, int32_t *argmax,
+                             const size_t *idims, const size_t *odims,
+                             const size_t *kernels, const size_t *strides,
+                             const size_t *pads);
+
+/* kernels.h:88-103; Codegen.cpp:2352-2354.  Row softmax of A[m,n]. b may alias a. */
+int swc_hip_matrixSoftmax_f(int m, int n, const float *a, int lda, float *b,
+                            int ldb);
+
+/* kernels.h:58-64; Codegen.cpp:2286-2296 (MatrixTanh). b = 1 - 2/(exp(2a)+1). */
+int swc_hip_matrixTanh_f(int m, int n, const float *a, int lda, float *b,
+                         int ldb);
+
+/* kernels.h:601-613; Codegen.cpp:2372-2385 (ArgMax op).  idx[m,top_k] = columns of the top_k largest
+ * values of each row, ties listing the larger column first. top_k <= 8. */
+int swc_hip_argMax_i(const float *input, int *idx, int m, int n, int top_k);
+
+/* ---- fused ops: what the HIP target emits when the graph allows.  Each equals
+ * the named sequence of reference kernels. ---- */
+
+/* MatrixMatrixFCBias kept un-lowered (the reference lowers it to
+ * matrixMatrixMul_f + batchedadd_f, src/op/dlOp/dlOpEinsum.cpp:154-237):
+ * C = A*B + bias[n], then ReLU if relu != 0. bias may be NULL (no bias). */
+int swc_hip_matrixMatrixFCBias_f(int m, int n, int k, const float *a, int lda,
+                                 const float *b, int ldb, const float *bias,
+                                 float *c, int ldc, int relu);
+
+/* vecAdd_f followed by relu_f. */
+int swc_hip_vecAddRelu_f(int size, const float *a, const float *b, float *c);
+
+/* batchnormalization_f followed by relu_f. */
+int swc_hip_batchnormRelu_f(float *output, const float *input, const float *mean,
+                            const float *var, const float *scale,
+                            const float *bias, const size_t *idims,
+                            float epsilon);
+
+/* batchnormalization_f, relu_f, then maxpool_f over the result (output has the
+ * pooled shape odims). */
+int swc_hip_batchnormReluMaxpool_f(float *output, const float *input,
+                                   const float *mean, const float *var,
+                                   const float *scale, const float *bias,
+                                   const size_t *idims, float epsilon,
+                                   const size_t *odims, const size_t *kernels,
+                                   const size_t *strides, const size_t *pads);
+
+/* conv2d_f, then optionally batchnormalization_f (when bn_mean != NULL; all four
+ * bn_* pointers must then be given), then optionally relu_f. */
+int swc_hip_conv2dFused_f(float *output, const float *input, const float *filter,
+                          const float *bias, const size_t *odims,
+                          const size_t *idims, const size_t *fdims,
+                          const size_t *bdims, const size_t *kernels,
+                          const size_t *strides, const size_t *pads,
+                          size_t group, const float *bn_mean,
+                          const float *bn_var, const float *bn_scale,
+                          const float *bn_bias, float epsilon, int relu);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SWC_HIP_H_ */

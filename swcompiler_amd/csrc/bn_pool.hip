@@ -1,0 +1,309 @@
+// batchnormalization_f (kernels.h:496-517), maxpool_f (kernels.h:323-377) and
+// their fusions, NHWC.  All are one pass over HBM; channels are the contiguous
+// axis, so a thread owns four consecutive channels (one 128-bit access) and
+// keeps their normalisation constants in registers while it walks rows.
+//
+// Arithmetic follows the reference exactly: var+eps is an fp32 add, everything
+// after it is double ((x-mean) widened, times (var+eps)^-1/2, times scale, plus
+// bias) with a single rounding to fp32 on the store.
+#include "common.hpp"
+
+using namespace swc_hip;
+
+namespace {
+
+constexpr int kThreads = 256;
+
+struct BnQuad {
+    float mean[4];
+    double rs[4];     // (var+eps)^-1/2
+    double scale[4];
+    double bias[4];
+};
+
+__device__ __forceinline__ void load_bn_quad(BnQuad &q, const float *mean, const float *var, const float *scale,
+                                             const float *bias, size_t c0, float eps) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        q.mean[i] = mean[c0 + i];
+        const float ve = var[c0 + i] + eps;
+        q.rs[i] = 1.0 / sqrt((double)ve);
+        q.scale[i] = (double)scale[c0 + i];
+        q.bias[i] = (double)bias[c0 + i];
+    }
+}
+
+template <bool RELU>
+__device__ __forceinline__ float bn1(float x, const BnQuad &q, int i) {
+    const float centred = x - q.mean[i];
+    const float y = (float)((double)centred * q.rs[i] * q.scale[i] + q.bias[i]);
+    return RELU ? ((y > 0.f) ? y : 0.f) : y;
+}
+
+template <bool RELU>
+__device__ __forceinline__ float4 bn4(float4 x, const BnQuad &q) {
+    return make_float4(bn1<RELU>(x.x, q, 0), bn1<RELU>(x.y, q, 1), bn1<RELU>(x.z, q, 2), bn1<RELU>(x.w, q, 3));
+}
+
+// The launch makes gridDim.x*kThreads a multiple of quads (= C/4), so the
+// channel quad of a thread never changes while it strides through the tensor.
+template <bool RELU>
+__global__ __launch_bounds__(kThreads) void bn_vec4(float *out, const float *in, const float *__restrict__ mean,
+                                                    const float *__restrict__ var, const float *__restrict__ scale,
+                                                    const float *__restrict__ bias, size_t total4, unsigned quads,
+                                                    float eps) {
+    const size_t g = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * kThreads;
+    if (g >= total4) return;
+    BnQuad q;
+    load_bn_quad(q, mean, var, scale, bias, (g % quads) * 4, eps);
+    const float4 *i4 = reinterpret_cast<const float4 *>(in);
+    float4 *o4 = reinterpret_cast<float4 *>(out);
+    size_t i = g;
+    // two independent loads in flight per thread
+    for (; i + step < total4; i += 2 * step) {
+        const float4 x0 = i4[i];
+        const float4 x1 = i4[i + step];
+        o4[i] = bn4<RELU>(x0, q);
+        o4[i + step] = bn4<RELU>(x1, q);
+    }
+    if (i < total4) o4[i] = bn4<RELU>(i4[i], q);
+}
+
+template <bool RELU>
+__global__ __launch_bounds__(kThreads) void bn_scalar(float *out, const float *in, const float *__restrict__ mean,
+                                                      const float *__restrict__ var, const float *__restrict__ scale,
+                                                      const float *__restrict__ bias, size_t total, size_t C,
+                                                      float eps) {
+    size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * kThreads;
+    for (; i < total; i += step) {
+        const size_t c = i % C;
+        const float ve = var[c] + eps;
+        const float centred = in[i] - mean[c];
+        const float y = (float)((double)centred * (1.0 / sqrt((double)ve)) * (double)scale[c] + (double)bias[c]);
+        out[i] = RELU ? ((y > 0.f) ? y : 0.f) : y;
+    }
+}
+
+struct PoolGeom {
+    int N, H, W, C, OH, OW, kh, kw, sh, sw, pt, pl;
+};
+
+// First in-bounds tap initialises, later taps replace only when strictly
+// greater (kernels.h:362-366).  `BN` applies batchnorm+relu to each tap first.
+template <bool ARGMAX, bool BN>
+__global__ __launch_bounds__(kThreads) void maxpool_vec4(const float *__restrict__ in, float *__restrict__ out,
+                                                         int32_t *__restrict__ arg, PoolGeom g, size_t total4,
+                                                         const float *__restrict__ mean, const float *__restrict__ var,
+                                                         const float *__restrict__ scale,
+                                                         const float *__restrict__ bias, float eps) {
+    const unsigned quads = g.C / 4;
+    const size_t gid = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * kThreads;
+    if (gid >= total4) return;
+    BnQuad q;
+    if (BN) load_bn_quad(q, mean, var, scale, bias, (gid % quads) * 4, eps);
+    const float4 *i4 = reinterpret_cast<const float4 *>(in);
+    for (size_t o = gid; o < total4; o += step) {
+        const unsigned cq = (unsigned)(o % quads);
+        size_t r = o / quads;
+        const int ox = (int)(r % g.OW);
+        r /= g.OW;
+        const int oy = (int)(r % g.OH);
+        const int n = (int)(r / g.OH);
+        float best[4] = {0.f, 0.f, 0.f, 0.f};
+        int32_t where[4] = {-1, -1, -1, -1};
+        bool have = false;
+        for (int ky = 0; ky < g.kh; ++ky) {
+            const int iy = oy * g.sh - g.pt + ky;
+            if (iy < 0 || iy >= g.H) continue;
+            for (int kx = 0; kx < g.kw; ++kx) {
+                const int ix = ox * g.sw - g.pl + kx;
+                if (ix < 0 || ix >= g.W) continue;
+                const size_t pix = ((size_t)n * g.H + iy) * g.W + ix;
+                float4 v4 = i4[pix * quads + cq];
+                if (BN) v4 = bn4<true>(v4, q);
+                const float v[4] = {v4.x, v4.y, v4.z, v4.w};
+                const int32_t flat = (int32_t)(pix * g.C + cq * 4);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    if (!have || v[c] > best[c]) {
+                        best[c] = v[c];
+                        if (ARGMAX) where[c] = flat + c;
+                    }
+                }
+                have = true;
+            }
+        }
+        reinterpret_cast<float4 *>(out)[o] = make_float4(best[0], best[1], best[2], best[3]);
+        if (ARGMAX) reinterpret_cast<int4 *>(arg)[o] = make_int4(where[0], where[1], where[2], where[3]);
+    }
+}
+
+template <bool ARGMAX, bool BN>
+__global__ __launch_bounds__(kThreads) void maxpool_scalar(const float *__restrict__ in, float *__restrict__ out,
+                                                           int32_t *__restrict__ arg, PoolGeom g, size_t total,
+                                                           const float *__restrict__ mean,
+                                                           const float *__restrict__ var,
+                                                           const float *__restrict__ scale,
+                                                           const float *__restrict__ bias, float eps) {
+    size_t o = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * kThreads;
+    for (; o < total; o += step) {
+        const int c = (int)(o % g.C);
+        size_t r = o / g.C;
+        const int ox = (int)(r % g.OW);
+        r /= g.OW;
+        const int oy = (int)(r % g.OH);
+        const int n = (int)(r / g.OH);
+        float best = 0.f;
+        int32_t where = -1;
+        bool have = false;
+        for (int ky = 0; ky < g.kh; ++ky) {
+            const int iy = oy * g.sh - g.pt + ky;
+            if (iy < 0 || iy >= g.H) continue;
+            for (int kx = 0; kx < g.kw; ++kx) {
+                const int ix = ox * g.sw - g.pl + kx;
+                if (ix < 0 || ix >= g.W) continue;
+                const size_t flat = (((size_t)n * g.H + iy) * g.W + ix) * g.C + c;
+                float v = in[flat];
+                if (BN) {
+                    const float ve = var[c] + eps;
+                    const float centred = v - mean[c];
+                    v = (float)((double)centred * (1.0 / sqrt((double)ve)) * (double)scale[c] + (double)bias[c]);
+                    v = (v > 0.f) ? v : 0.f;
+                }
+                if (!have || v > best) {
+                    best = v;
+                    where = (int32_t)flat;
+                    have = true;
+                }
+            }
+        }
+        out[o] = best;
+        if (ARGMAX) arg[o] = where;
+    }
+}
+
+// blocks such that blocks*kThreads is a multiple of `quads`
+unsigned quad_stable_blocks(size_t total4, unsigned quads, unsigned max_blocks) {
+    unsigned a = quads, b = kThreads;
+    while (b) { unsigned t = a % b; a = b; b = t; }
+    const unsigned unit = quads / a;  // blocks must be a multiple of this
+    size_t need = (total4 + kThreads - 1) / kThreads;
+    if (need > max_blocks) need = max_blocks;
+    size_t blocks = ((need + unit - 1) / unit) * unit;
+    if (blocks == 0) blocks = unit;
+    return (unsigned)blocks;
+}
+
+int check_dims4(const char *who, const size_t *d) {
+    for (int i = 0; i < 4; ++i)
+        if (d[i] > 0x7fffffffu) return fail(SWC_HIP_EINVAL, "%s: dimension %d too large", who, i);
+    return 0;
+}
+
+template <bool RELU>
+int launch_bn(const char *who, float *output, const float *input, const float *mean, const float *var,
+              const float *scale, const float *bias, const size_t *idims, float eps) {
+    if (!idims) return fail(SWC_HIP_EINVAL, "%s: null idims", who);
+    if (check_dims4(who, idims)) return SWC_HIP_EINVAL;
+    const size_t C = idims[3];
+    const size_t total = idims[0] * idims[1] * idims[2] * C;
+    if (total == 0) return SWC_HIP_OK;
+    if (!output || !input || !mean || !var || !scale || !bias) return fail(SWC_HIP_EINVAL, "%s: null pointer", who);
+    if (C % 4 == 0 && aligned16(output) && aligned16(input)) {
+        const size_t total4 = total / 4;
+        const unsigned quads = (unsigned)(C / 4);
+        const unsigned blocks = quad_stable_blocks((total4 + 3) / 4, quads, (unsigned)num_cus() * 16u);
+        bn_vec4<RELU><<<blocks, kThreads, 0, stream()>>>(output, input, mean, var, scale, bias, total4, quads, eps);
+    } else {
+        size_t blocks = (total + kThreads - 1) / kThreads;
+        if (blocks > 8192) blocks = 8192;
+        bn_scalar<RELU><<<(unsigned)blocks, kThreads, 0, stream()>>>(output, input, mean, var, scale, bias, total, C, eps);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(SWC_HIP_ERUNTIME, "%s: launch failed: %s", who, hipGetErrorString(e));
+    return SWC_HIP_OK;
+}
+
+template <bool ARGMAX, bool BN>
+int launch_pool(const char *who, const float *input, float *output, int32_t *argmax, const size_t *idims,
+                const size_t *odims, const size_t *kernels, const size_t *strides, const size_t *pads,
+                const float *mean, const float *var, const float *scale, const float *bias, float eps) {
+    if (!idims || !odims || !kernels || !strides || !pads) return fail(SWC_HIP_EINVAL, "%s: null shape array", who);
+    if (check_dims4(who, idims) || check_dims4(who, odims)) return SWC_HIP_EINVAL;
+    if (odims[0] != idims[0] || odims[3] != idims[3])
+        return fail(SWC_HIP_EINVAL, "%s: output batch/channels differ from input", who);
+    if (kernels[0] == 0 || kernels[1] == 0 || strides[0] == 0 || strides[1] == 0 || kernels[0] > 4096 ||
+        kernels[1] > 4096 || strides[0] > 4096 || strides[1] > 4096 || pads[0] > 4096 || pads[1] > 4096)
+        return fail(SWC_HIP_EINVAL, "%s: bad kernel/stride/pad", who);
+    // every window must start inside the padded input, as in the reference's shape rule
+    if (odims[1] && (odims[1] - 1) * strides[0] >= idims[1] + pads[0] + kernels[0])
+        return fail(SWC_HIP_EINVAL, "%s: output height inconsistent with input", who);
+    if (odims[2] && (odims[2] - 1) * strides[1] >= idims[2] + pads[1] + kernels[1])
+        return fail(SWC_HIP_EINVAL, "%s: output width inconsistent with input", who);
+    const size_t in_total = idims[0] * idims[1] * idims[2] * idims[3];
+    const size_t total = odims[0] * odims[1] * odims[2] * odims[3];
+    if (total == 0) return SWC_HIP_OK;
+    if (ARGMAX && in_total > 0x7fffffffu) return fail(SWC_HIP_EUNSUPPORTED, "%s: input too large for int32 indices", who);
+    if (!input || !output || (ARGMAX && !argmax)) return fail(SWC_HIP_EINVAL, "%s: null pointer", who);
+    if (BN && (!mean || !var || !scale || !bias)) return fail(SWC_HIP_EINVAL, "%s: null batchnorm parameter", who);
+    PoolGeom g{(int)idims[0], (int)idims[1], (int)idims[2], (int)idims[3], (int)odims[1], (int)odims[2],
+               (int)kernels[0], (int)kernels[1], (int)strides[0], (int)strides[1], (int)pads[0], (int)pads[1]};
+    const size_t C = idims[3];
+    if (C % 4 == 0 && aligned16(input) && aligned16(output) && (!ARGMAX || aligned16(argmax))) {
+        const size_t total4 = total / 4;
+        const unsigned blocks = quad_stable_blocks(total4, (unsigned)(C / 4), (unsigned)num_cus() * 32u);
+        maxpool_vec4<ARGMAX, BN><<<blocks, kThreads, 0, stream()>>>(input, output, argmax, g, total4, mean, var, scale, bias, eps);
+    } else {
+        size_t blocks = (total + kThreads - 1) / kThreads;
+        if (blocks > 8192) blocks = 8192;
+        maxpool_scalar<ARGMAX, BN><<<(unsigned)blocks, kThreads, 0, stream()>>>(input, output, argmax, g, total, mean, var, scale, bias, eps);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(SWC_HIP_ERUNTIME, "%s: launch failed: %s", who, hipGetErrorString(e));
+    return SWC_HIP_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+int swc_hip_batchnormalization_f(float *output, const float *input, const float *mean, const float *var,
+                                 const float *scale, const float *bias, const size_t *idims, float epsilon) {
+    SWC_REQUIRE_INIT();
+    return launch_bn<false>("swc_hip_batchnormalization_f", output, input, mean, var, scale, bias, idims, epsilon);
+}
+
+int swc_hip_batchnormRelu_f(float *output, const float *input, const float *mean, const float *var,
+                            const float *scale, const float *bias, const size_t *idims, float epsilon) {
+    SWC_REQUIRE_INIT();
+    return launch_bn<true>("swc_hip_batchnormRelu_f", output, input, mean, var, scale, bias, idims, epsilon);
+}
+
+int swc_hip_maxpool_f(const float *input, float *output, const size_t *idims, const size_t *odims,
+                      const size_t *kernels, const size_t *strides, const size_t *pads) {
+    SWC_REQUIRE_INIT();
+    return launch_pool<false, false>("swc_hip_maxpool_f", input, output, nullptr, idims, odims, kernels, strides, pads,
+                                     nullptr, nullptr, nullptr, nullptr, 0.f);
+}
+
+int swc_hip_maxpool_argmax_f(const float *input, float *output, int32_t *argmax, const size_t *idims,
+                             const size_t *odims, const size_t *kernels, const size_t *strides, const size_t *pads) {
+    SWC_REQUIRE_INIT();
+    return launch_pool<true, false>("swc_hip_maxpool_argmax_f", input, output, argmax, idims, odims, kernels, strides,
+                                    pads, nullptr, nullptr, nullptr, nullptr, 0.f);
+}
+
+int swc_hip_batchnormReluMaxpool_f(float *output, const float *input, const float *mean, const float *var,
+                                   const float *scale, const float *bias, const size_t *idims, float epsilon,
+                                   const size_t *odims, const size_t *kernels, const size_t *strides,
+                                   const size_t *pads) {
+    SWC_REQUIRE_INIT();
+    return launch_pool<false, true>("swc_hip_batchnormReluMaxpool_f", input, output, nullptr, idims, odims, kernels,
+                                    strides, pads, mean, var, scale, bias, epsilon);
+}
+
+} // extern "C"

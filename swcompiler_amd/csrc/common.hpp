@@ -1,0 +1,48 @@
+// Shared plumbing of libswc_hip: error record, stream access, launch checks.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+
+#include "swc_hip.h"
+
+namespace swc_hip {
+
+// Records a printf-style message for swc_hip_last_error() and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+// The stream every op launches on; nullptr until swc_hip_init succeeded.
+hipStream_t stream();
+bool ready();
+int num_cus();
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline unsigned ceil_div(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
+
+} // namespace swc_hip
+
+#define SWC_REQUIRE_INIT()                                                              \
+    do {                                                                                \
+        if (!swc_hip::ready())                                                          \
+            return swc_hip::fail(SWC_HIP_ENOTINIT, "%s: swc_hip_init has not been called", __func__); \
+    } while (0)
+
+#define SWC_ARG(cond)                                                                   \
+    do {                                                                                \
+        if (!(cond)) return swc_hip::fail(SWC_HIP_EINVAL, "%s: argument check failed: %s", __func__, #cond); \
+    } while (0)
+
+#define SWC_HIP_TRY(expr)                                                               \
+    do {                                                                                \
+        hipError_t e__ = (expr);                                                        \
+        if (e__ != hipSuccess)                                                          \
+            return swc_hip::fail(SWC_HIP_ERUNTIME, "%s: %s -> %s", __func__, #expr, hipGetErrorString(e__)); \
+    } while (0)
+
+// after a kernel launch
+#define SWC_LAUNCH_CHECK() SWC_HIP_TRY(hipGetLastError())

@@ -1,0 +1,240 @@
+// conv2d_f (kernels.h:177-243) as an implicit GEMM on fp32 MFMA, NHWC.
+//
+//   C[M, oC] = A[M, K] * F^T,  M = N*OH*OW (output pixels), K = kH*kW*iC,
+//   A[m, (ky,kx,ci)] = in[n, oy*sh - pt + ky, ox*sw - pl + kx, ci] (0 outside),
+//   F = filter viewed as [oC, K] — K is the contiguous axis of BOTH operands,
+//   and the output tensor [N,OH,OW,oC] is exactly C row-major, so nothing is
+//   ever materialised or transposed.  Bias, inference batchnorm and ReLU are
+//   applied to the accumulators before the single store.
+//
+// The tile machinery is mfma_tile.hpp's; only the global->LDS gather differs
+// from the FC GEMM.  When iC % 4 == 0 four consecutive k's lie in one tap, so
+// the gather uses 128-bit loads; otherwise (first layer, iC = 1 or 3) 32-bit.
+#include "common.hpp"
+#include "mfma_tile.hpp"
+
+using namespace swc_hip;
+using namespace swc_hip::mfma;
+
+namespace {
+
+struct ConvGeom {
+    int N, H, W, C;      // input NHWC
+    int OH, OW, OC;      // output
+    int kh, kw, sh, sw, pt, pl;
+    int M, K;            // GEMM view
+};
+
+template <int TM, int TN, bool VEC>
+__global__ __launch_bounds__(kThreads) void conv_igemm(const float *__restrict__ in, const float *__restrict__ filt,
+                                                       float *__restrict__ out, ConvGeom g, Epilogue ep) {
+    using T = Tile<TM, TN, true>;
+    extern __shared__ __align__(16) float lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const int M = g.M, N = g.OC, K = g.K;
+
+    int tile_m, tile_n;
+    tile_coords((M + T::BM - 1) / T::BM, (N + T::BN - 1) / T::BN, tile_m, tile_n);
+    const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    // VEC: thread owns rows (tid>>3) + 32*i of the A tile and k quad (tid&7).
+    // Top-left input coordinate of each owned output pixel, (-1<<20) if row >= M.
+    int iy0[T::kAVec], ix0[T::kAVec], img[T::kAVec];
+    if (VEC) {
+#pragma unroll
+        for (int i = 0; i < T::kAVec; ++i) {
+            const int m = m0 + (tid >> 3) + 32 * i;
+            if (m < M) {
+                const int ox = m % g.OW;
+                const int t = m / g.OW;
+                const int oy = t % g.OH;
+                img[i] = t / g.OH;
+                iy0[i] = oy * g.sh - g.pt;
+                ix0[i] = ox * g.sw - g.pl;
+            } else {
+                img[i] = 0;
+                iy0[i] = -(1 << 20);
+                ix0[i] = -(1 << 20);
+            }
+        }
+    }
+
+    constexpr int kAScalar = T::kAVec * 4, kBScalar = T::kBVec * 4;
+    float4 ra[T::kAVec], rb[T::kBVec];
+    float sa[VEC ? 1 : kAScalar], sb[VEC ? 1 : kBScalar];
+
+    auto load_global = [&](int k0) {
+        if (VEC) {
+            const int k = k0 + (tid & 7) * 4;
+            const int tap = k / g.C, ci = k - tap * g.C;
+            const int ky = tap / g.kw, kx = tap - ky * g.kw;
+#pragma unroll
+            for (int i = 0; i < T::kAVec; ++i) {
+                const int iy = iy0[i] + ky, ix = ix0[i] + kx;
+                const bool ok = k < K && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+                ra[i] = ok ? *reinterpret_cast<const float4 *>(
+                                 in + (((size_t)img[i] * g.H + iy) * g.W + ix) * g.C + ci)
+                           : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int i = 0; i < T::kBVec; ++i) {
+                const int col = n0 + (tid >> 3) + 32 * i;
+                rb[i] = (col < N && k < K) ? *reinterpret_cast<const float4 *>(filt + (size_t)col * K + k)
+                                           : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kAScalar; ++i) {
+                const int e = tid + kThreads * i;
+                const int m = m0 + e / BK, k = k0 + e % BK;
+                float v = 0.f;
+                if (m < M && k < K) {
+                    const int ox = m % g.OW;
+                    const int t = m / g.OW;
+                    const int oy = t % g.OH, n = t / g.OH;
+                    const int tap = k / g.C, ci = k - tap * g.C;
+                    const int ky = tap / g.kw, kx = tap - ky * g.kw;
+                    const int iy = oy * g.sh - g.pt + ky, ix = ox * g.sw - g.pl + kx;
+                    if (iy >= 0 && iy < g.H && ix >= 0 && ix < g.W)
+                        v = in[(((size_t)n * g.H + iy) * g.W + ix) * g.C + ci];
+                }
+                sa[i] = v;
+            }
+#pragma unroll
+            for (int i = 0; i < kBScalar; ++i) {
+                const int e = tid + kThreads * i;
+                const int col = n0 + e / BK, k = k0 + e % BK;
+                sb[i] = (col < N && k < K) ? filt[(size_t)col * K + k] : 0.f;
+            }
+        }
+    };
+    auto store_lds = [&](int stage) {
+        float *As = lds + stage * T::kStageFloats;
+        float *Bs = As + T::kAFloats;
+        if (VEC) {
+#pragma unroll
+            for (int i = 0; i < T::kAVec; ++i)
+                *reinterpret_cast<float4 *>(&As[((tid >> 3) + 32 * i) * kLdK + (tid & 7) * 4]) = ra[i];
+#pragma unroll
+            for (int i = 0; i < T::kBVec; ++i)
+                *reinterpret_cast<float4 *>(&Bs[((tid >> 3) + 32 * i) * kLdK + (tid & 7) * 4]) = rb[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < kAScalar; ++i) {
+                const int e = tid + kThreads * i;
+                As[(e / BK) * kLdK + e % BK] = sa[i];
+            }
+#pragma unroll
+            for (int i = 0; i < kBScalar; ++i) {
+                const int e = tid + kThreads * i;
+                Bs[(e / BK) * kLdK + e % BK] = sb[i];
+            }
+        }
+    };
+
+    const int nk = (K + BK - 1) / BK;
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) load_global((kt + 1) * BK);
+        const float *As = lds + cur * T::kStageFloats;
+        compute_slice<TM, TN, true>(As, As + T::kAFloats, acc, wave_m, wave_n, lane);
+        if (kt + 1 < nk) store_lds(cur ^ 1);
+        __syncthreads();
+    }
+    store_tile<TM, TN>(acc, out, (size_t)N, M, N, m0 + wave_m * 32 * TM, n0 + wave_n * 32 * TN, lane, ep);
+}
+
+template <int TM, int TN>
+int launch_conv(bool vec, const float *in, const float *filt, float *out, const ConvGeom &g, const Epilogue &ep) {
+    using T = Tile<TM, TN, true>;
+    const long tiles = (long)((g.M + T::BM - 1) / T::BM) * ((g.OC + T::BN - 1) / T::BN);
+    auto kern = vec ? conv_igemm<TM, TN, true> : conv_igemm<TM, TN, false>;
+    static bool attr_set[2] = {false, false};
+    if (!attr_set[vec]) {
+        SWC_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)T::kLdsBytes));
+        attr_set[vec] = true;
+    }
+    kern<<<(unsigned)tiles, kThreads, T::kLdsBytes, stream()>>>(in, filt, out, g, ep);
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
+}
+
+int conv_dispatch(const char *who, float *output, const float *input, const float *filter, const float *bias,
+                  const size_t *odims, const size_t *idims, const size_t *fdims, const size_t *kernels,
+                  const size_t *strides, const size_t *pads, size_t group, const Epilogue &ep_in) {
+    if (!odims || !idims || !fdims || !kernels || !strides || !pads)
+        return fail(SWC_HIP_EINVAL, "%s: null shape array", who);
+    if (group != 1) return fail(SWC_HIP_EUNSUPPORTED, "%s: group = %zu (only 1 is supported)", who, group);
+    for (int i = 0; i < 4; ++i)
+        if (odims[i] > 0x7fffffffu || idims[i] > 0x7fffffffu || fdims[i] > 0x7fffffffu)
+            return fail(SWC_HIP_EINVAL, "%s: dimension too large", who);
+    if (odims[0] != idims[0]) return fail(SWC_HIP_EINVAL, "%s: batch of output and input differ", who);
+    if (fdims[0] != odims[3] || fdims[3] != idims[3] || fdims[1] != kernels[0] || fdims[2] != kernels[1])
+        return fail(SWC_HIP_EINVAL, "%s: filter dims {%zu,%zu,%zu,%zu} do not match oC=%zu, kernels {%zu,%zu}, iC=%zu", who,
+                    fdims[0], fdims[1], fdims[2], fdims[3], odims[3], kernels[0], kernels[1], idims[3]);
+    if (strides[0] == 0 || strides[1] == 0 || strides[0] > 4096 || strides[1] > 4096 || pads[0] > 4096 ||
+        pads[1] > 4096 || kernels[0] == 0 || kernels[1] == 0)
+        return fail(SWC_HIP_EINVAL, "%s: bad kernel/stride/pad", who);
+    const size_t M = odims[0] * odims[1] * odims[2];
+    const size_t K = fdims[1] * fdims[2] * fdims[3];
+    if (M > 0x7fffffffu || K > 0x7fffffffu || M * odims[3] > (size_t)1 << 40)
+        return fail(SWC_HIP_EINVAL, "%s: problem too large", who);
+    if (M == 0 || odims[3] == 0) return SWC_HIP_OK;
+    if (!output || !input || !filter || !bias) return fail(SWC_HIP_EINVAL, "%s: null pointer", who);
+    ConvGeom g{(int)idims[0], (int)idims[1], (int)idims[2], (int)idims[3], (int)odims[1], (int)odims[2],
+               (int)odims[3], (int)kernels[0], (int)kernels[1], (int)strides[0], (int)strides[1], (int)pads[0],
+               (int)pads[1], (int)M, (int)K};
+    Epilogue ep = ep_in;
+    ep.bias = bias;
+    const bool vec = (g.C % 4 == 0) && aligned16(input) && aligned16(filter);
+    const long tiles_m128 = (M + 127) / 128;
+    if (g.OC > 64 && tiles_m128 * ((g.OC + 127) / 128) >= num_cus())
+        return launch_conv<2, 2>(vec, input, filter, output, g, ep);
+    if (tiles_m128 * ((g.OC + 63) / 64) >= num_cus()) return launch_conv<2, 1>(vec, input, filter, output, g, ep);
+    return launch_conv<1, 1>(vec, input, filter, output, g, ep);
+}
+
+} // namespace
+
+extern "C" {
+
+int swc_hip_conv2d_f(float *output, const float *input, const float *filter, const float *bias, const size_t *odims,
+                     const size_t *idims, const size_t *fdims, const size_t *bdims, const size_t *kernels,
+                     const size_t *strides, const size_t *pads, size_t group) {
+    SWC_REQUIRE_INIT();
+    (void)bdims;
+    Epilogue ep{nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
+    return conv_dispatch("swc_hip_conv2d_f", output, input, filter, bias, odims, idims, fdims, kernels, strides, pads,
+                         group, ep);
+}
+
+int swc_hip_conv2dFused_f(float *output, const float *input, const float *filter, const float *bias,
+                          const size_t *odims, const size_t *idims, const size_t *fdims, const size_t *bdims,
+                          const size_t *kernels, const size_t *strides, const size_t *pads, size_t group,
+                          const float *bn_mean, const float *bn_var, const float *bn_scale, const float *bn_bias,
+                          float epsilon, int relu) {
+    SWC_REQUIRE_INIT();
+    (void)bdims;
+    if (bn_mean || bn_var || bn_scale || bn_bias)
+        SWC_ARG(bn_mean && bn_var && bn_scale && bn_bias);
+    Epilogue ep{nullptr, bn_mean, bn_var, bn_scale, bn_bias, epsilon, relu};
+    return conv_dispatch("swc_hip_conv2dFused_f", output, input, filter, bias, odims, idims, fdims, kernels, strides,
+                         pads, group, ep);
+}
+
+} // extern "C"

@@ -1,0 +1,161 @@
+// fp32 MFMA block-tile core shared by the FC GEMM and the implicit-GEMM conv.
+//
+// A workgroup of 256 threads (4 wavefronts as 2x2) computes a BM x BN tile of
+// C = A*B, BM = 64*TM, BN = 64*TN; each wavefront owns a (32*TM) x (32*TN)
+// sub-tile as TM x TN accumulators of v_mfma_f32_32x32x2_f32 (16 VGPRs each).
+// K is consumed in slices of BK = 32 staged through LDS, double-buffered, with
+// the next slice's global loads issued before the current slice's MFMAs.
+//
+// Operand layout of v_mfma_f32_32x32x2_f32 (lane l of 64):
+//   A[i][kk]: i = l % 32, kk = l / 32        B[kk][j]: j = l % 32, kk = l / 32
+//   D[i][j] in VGPR v (0..15): j = l % 32, i = 8*(v/4) + 4*(l/32) + v%4
+// The sum over k is order-free, so within a group of 8 k's the half-wave
+// h = l/32 takes k = 4h..4h+3: a lane then needs four CONSECUTIVE k's of one
+// row of A, which is a single 128-bit LDS read when A is stored k-contiguous.
+//
+// LDS layouts (floats):
+//   k-contiguous operand (A always; B when given as [n][k], i.e. conv filters):
+//     rows of BK + 4 — the +4 shifts consecutive rows by 4 banks, so the eight
+//     lanes served together by a 128-bit read touch disjoint bank quads.
+//   n-contiguous B ([k][n], FC weights): rows of BN + 8 — the two half-waves
+//     read rows 4 apart; 4*(BN+8) = 32 (mod 64) puts them on opposite halves
+//     of the banks.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace swc_hip {
+namespace mfma {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int BK = 32;
+constexpr int kPadK = 4;
+constexpr int kLdK = BK + kPadK;   // row length of a k-contiguous tile
+
+template <int TM, int TN, bool B_NT>
+struct Tile {
+    static constexpr int BM = 64 * TM;
+    static constexpr int BN = 64 * TN;
+    static constexpr int kLdBn = BN + 8;                       // [k][n] layout of B
+    static constexpr int kAFloats = BM * kLdK;
+    static constexpr int kBFloats = B_NT ? BN * kLdK : BK * kLdBn;
+    static constexpr int kStageFloats = kAFloats + kBFloats;
+    static constexpr size_t kLdsBytes = 2u * kStageFloats * sizeof(float);
+    // float4 per thread per k-slice
+    static constexpr int kAVec = BM * BK / 4 / kThreads;       // = 2*TM
+    static constexpr int kBVec = BN * BK / 4 / kThreads;       // = 2*TN
+};
+
+// One k-slice of MFMAs for this wavefront.  As/Bs point at the current stage.
+template <int TM, int TN, bool B_NT>
+__device__ __forceinline__ void compute_slice(const float *__restrict__ As, const float *__restrict__ Bs,
+                                              v16f (&acc)[TM][TN], int wave_m, int wave_n, int lane) {
+    using T = Tile<TM, TN, B_NT>;
+    const int l32 = lane & 31;
+    const int h = lane >> 5;
+#pragma unroll
+    for (int kb = 0; kb < BK; kb += 8) {
+        float4 a[TM];
+        float bq[TN][4];
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+            a[tm] = *reinterpret_cast<const float4 *>(&As[(wave_m * 32 * TM + tm * 32 + l32) * kLdK + kb + 4 * h]);
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+            if (B_NT) {
+                const float4 v =
+                    *reinterpret_cast<const float4 *>(&Bs[(wave_n * 32 * TN + tn * 32 + l32) * kLdK + kb + 4 * h]);
+                bq[tn][0] = v.x; bq[tn][1] = v.y; bq[tn][2] = v.z; bq[tn][3] = v.w;
+            } else {
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+                    bq[tn][s] = Bs[(kb + 4 * h + s) * T::kLdBn + wave_n * 32 * TN + tn * 32 + l32];
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+                const float av = (s == 0) ? a[tm].x : (s == 1) ? a[tm].y : (s == 2) ? a[tm].z : a[tm].w;
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn)
+                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bq[tn][s], acc[tm][tn], 0, 0, 0);
+            }
+        }
+    }
+}
+
+// Per-column epilogue constants: out = f(acc + bias[col]) with optional
+// inference batchnorm (double arithmetic, as the reference's
+// batchnormalization_f) and optional ReLU.
+struct Epilogue {
+    const float *bias;      // may be null
+    const float *bn_mean;   // null: no batchnorm
+    const float *bn_var;
+    const float *bn_scale;
+    const float *bn_bias;
+    float eps;
+    int relu;
+};
+
+// Writes this wavefront's accumulators to C (row-major, leading dimension ldc).
+template <int TM, int TN>
+__device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], float *__restrict__ C, size_t ldc, int M, int N,
+                                           int row0, int col0, int lane, const Epilogue &ep) {
+    const int l32 = lane & 31;
+    const int h = lane >> 5;
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+        const int col = col0 + tn * 32 + l32;
+        if (col >= N) continue;
+        const float bias = ep.bias ? ep.bias[col] : 0.f;
+        float mean = 0.f;
+        double rs = 1.0, gamma = 1.0, beta = 0.0;
+        const bool bn = ep.bn_mean != nullptr;
+        if (bn) {
+            mean = ep.bn_mean[col];
+            const float ve = ep.bn_var[col] + ep.eps;
+            rs = 1.0 / sqrt((double)ve);
+            gamma = (double)ep.bn_scale[col];
+            beta = (double)ep.bn_bias[col];
+        }
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = row0 + tm * 32 + 8 * (v / 4) + 4 * h + (v % 4);
+                if (row >= M) continue;
+                float x = acc[tm][tn][v] + bias;
+                if (bn) {
+                    const float centred = x - mean;
+                    x = (float)((double)centred * rs * gamma + beta);
+                }
+                if (ep.relu) x = (x > 0.f) ? x : 0.f;
+                C[(size_t)row * ldc + col] = x;
+            }
+        }
+    }
+}
+
+// Workgroup id -> tile coordinates.  Workgroups are dealt round-robin to the 8
+// XCDs, each with its own L2; ids that land on one XCD are renumbered to be
+// consecutive, and consecutive ids walk the tile grid in column strips 8 tiles
+// tall, so the tiles resident on one XCD at a time share A rows and B columns.
+__device__ __forceinline__ void tile_coords(int tiles_m, int tiles_n, int &tile_m, int &tile_n) {
+    const int total = tiles_m * tiles_n;
+    int pid = blockIdx.x;
+    constexpr int kXcd = 8;
+    if (total % kXcd == 0) pid = (pid % kXcd) * (total / kXcd) + pid / kXcd;
+    constexpr int kGroup = 8;
+    const int per_group = kGroup * tiles_n;
+    const int group = pid / per_group;
+    const int first_m = group * kGroup;
+    const int rows = (tiles_m - first_m < kGroup) ? (tiles_m - first_m) : kGroup;
+    const int in_group = pid - group * per_group;
+    tile_m = first_m + in_group % rows;
+    tile_n = in_group / rows;
+}
+
+} // namespace mfma
+} // namespace swc_hip

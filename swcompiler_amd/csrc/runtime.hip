@@ -1,0 +1,225 @@
+// Runtime half of libswc_hip: device selection, the single in-order stream,
+// arena allocation and host<->device copies.  Replaces the cudaSetDevice /
+// cudaMalloc / cudaMemcpy / cudaStreamCreate lines the reference's code
+// generator prints (src/codegen/Codegen.cpp:154-172, 504-521, 1134-1169).
+#include "common.hpp"
+
+#include <cstring>
+#include <mutex>
+
+namespace swc_hip {
+namespace {
+
+thread_local char g_err[512] = "";
+constexpr int kEventSlots = 4096;
+
+struct State {
+    std::mutex mu;
+    bool ready = false;
+    int device = -1;
+    int cus = 0;
+    hipStream_t own = nullptr;   // created by init
+    hipStream_t cur = nullptr;   // where ops launch (own or caller's)
+    bool cur_is_own = true;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    float last_ms = -1.f;
+    hipEvent_t slots[kEventSlots] = {};
+    char arch[64] = "";
+} g;
+
+__global__ void fill_kernel(float *__restrict__ dst, float v, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) dst[i] = v;
+}
+
+} // namespace
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+void clear_error() { g_err[0] = 0; }
+hipStream_t stream() { return g.cur; }
+bool ready() { return g.ready; }
+int num_cus() { return g.cus; }
+
+} // namespace swc_hip
+
+using namespace swc_hip;
+
+extern "C" {
+
+int swc_hip_init(int device) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (g.ready) {
+        if (device != g.device)
+            return fail(SWC_HIP_EINVAL, "swc_hip_init: already initialised on device %d", g.device);
+        return SWC_HIP_OK;
+    }
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0)
+        return fail(SWC_HIP_ERUNTIME, "swc_hip_init: no HIP device (%s)",
+                    e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+    if (device < 0 || device >= count)
+        return fail(SWC_HIP_EINVAL, "swc_hip_init: device %d out of range [0,%d)", device, count);
+    SWC_HIP_TRY(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    SWC_HIP_TRY(hipGetDeviceProperties(&prop, device));
+    snprintf(g.arch, sizeof(g.arch), "%s", prop.gcnArchName);
+    if (std::strncmp(g.arch, "gfx950", 6) != 0)
+        return fail(SWC_HIP_EUNSUPPORTED, "swc_hip_init: kernels are built for gfx950 only, device is %s", g.arch);
+    g.cus = prop.multiProcessorCount;
+    SWC_HIP_TRY(hipStreamCreateWithFlags(&g.own, hipStreamNonBlocking));
+    SWC_HIP_TRY(hipEventCreate(&g.t0));
+    SWC_HIP_TRY(hipEventCreate(&g.t1));
+    g.cur = g.own;
+    g.cur_is_own = true;
+    g.device = device;
+    g.ready = true;
+    clear_error();
+    return SWC_HIP_OK;
+}
+
+int swc_hip_shutdown(void) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (!g.ready) return SWC_HIP_OK;
+    (void)hipStreamSynchronize(g.cur);
+    (void)hipEventDestroy(g.t0);
+    (void)hipEventDestroy(g.t1);
+    (void)hipStreamDestroy(g.own);
+    g.own = g.cur = nullptr;
+    g.t0 = g.t1 = nullptr;
+    g.ready = false;
+    g.device = -1;
+    return SWC_HIP_OK;
+}
+
+void *swc_hip_malloc(size_t bytes) {
+    if (!ready()) {
+        fail(SWC_HIP_ENOTINIT, "swc_hip_malloc: swc_hip_init has not been called");
+        return nullptr;
+    }
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+    if (e != hipSuccess) {
+        fail(SWC_HIP_ERUNTIME, "swc_hip_malloc(%zu): %s", bytes, hipGetErrorString(e));
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return p;
+}
+
+int swc_hip_free(void *dptr) {
+    SWC_REQUIRE_INIT();
+    if (!dptr) return SWC_HIP_OK;
+    SWC_HIP_TRY(hipStreamSynchronize(stream()));
+    SWC_HIP_TRY(hipFree(dptr));
+    return SWC_HIP_OK;
+}
+
+int swc_hip_h2d(void *dst, const void *src, size_t bytes) {
+    SWC_REQUIRE_INIT();
+    SWC_ARG(bytes == 0 || (dst && src));
+    if (!bytes) return SWC_HIP_OK;
+    SWC_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, stream()));
+    SWC_HIP_TRY(hipStreamSynchronize(stream()));
+    return SWC_HIP_OK;
+}
+
+int swc_hip_d2h(void *dst, const void *src, size_t bytes) {
+    SWC_REQUIRE_INIT();
+    SWC_ARG(bytes == 0 || (dst && src));
+    if (!bytes) return SWC_HIP_OK;
+    SWC_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, stream()));
+    SWC_HIP_TRY(hipStreamSynchronize(stream()));
+    return SWC_HIP_OK;
+}
+
+int swc_hip_d2d(void *dst, const void *src, size_t bytes) {
+    SWC_REQUIRE_INIT();
+    SWC_ARG(bytes == 0 || (dst && src));
+    if (!bytes) return SWC_HIP_OK;
+    SWC_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, stream()));
+    return SWC_HIP_OK;
+}
+
+int swc_hip_fill_f(float *dst, float value, size_t count) {
+    SWC_REQUIRE_INIT();
+    SWC_ARG(count == 0 || dst);
+    if (!count) return SWC_HIP_OK;
+    unsigned blocks = ceil_div(count, 256);
+    if (blocks > 4096u) blocks = 4096u;
+    fill_kernel<<<blocks, 256, 0, stream()>>>(dst, value, count);
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
+}
+
+int swc_hip_sync(void) {
+    SWC_REQUIRE_INIT();
+    SWC_HIP_TRY(hipStreamSynchronize(stream()));
+    return SWC_HIP_OK;
+}
+
+const char *swc_hip_last_error(void) { return g_err; }
+
+void *swc_hip_stream(void) { return (void *)g.cur; }
+
+int swc_hip_set_stream(void *s) {
+    SWC_REQUIRE_INIT();
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (s) {
+        g.cur = (hipStream_t)s;
+        g.cur_is_own = false;
+    } else {
+        g.cur = g.own;
+        g.cur_is_own = true;
+    }
+    return SWC_HIP_OK;
+}
+
+const char *swc_hip_device_name(void) { return g.arch; }
+
+int swc_hip_timer_begin(void) {
+    SWC_REQUIRE_INIT();
+    SWC_HIP_TRY(hipEventRecord(g.t0, stream()));
+    return SWC_HIP_OK;
+}
+
+int swc_hip_timer_end(void) {
+    SWC_REQUIRE_INIT();
+    SWC_HIP_TRY(hipEventRecord(g.t1, stream()));
+    SWC_HIP_TRY(hipEventSynchronize(g.t1));
+    float ms = 0.f;
+    SWC_HIP_TRY(hipEventElapsedTime(&ms, g.t0, g.t1));
+    g.last_ms = ms;
+    return SWC_HIP_OK;
+}
+
+float swc_hip_timer_elapsed_ms(void) { return g.last_ms; }
+
+int swc_hip_event_record(int slot) {
+    SWC_REQUIRE_INIT();
+    SWC_ARG(slot >= 0 && slot < kEventSlots);
+    if (!g.slots[slot]) SWC_HIP_TRY(hipEventCreate(&g.slots[slot]));
+    SWC_HIP_TRY(hipEventRecord(g.slots[slot], stream()));
+    return SWC_HIP_OK;
+}
+
+float swc_hip_event_elapsed_ms(int first, int second) {
+    if (!ready() || first < 0 || second < 0 || first >= kEventSlots || second >= kEventSlots ||
+        !g.slots[first] || !g.slots[second]) {
+        fail(SWC_HIP_EINVAL, "swc_hip_event_elapsed_ms: slot not recorded");
+        return -1.f;
+    }
+    if (hipEventSynchronize(g.slots[second]) != hipSuccess) return -1.f;
+    float ms = -1.f;
+    if (hipEventElapsedTime(&ms, g.slots[first], g.slots[second]) != hipSuccess) return -1.f;
+    return ms;
+}
+
+} // extern "C"

@@ -1,0 +1,178 @@
+// matrixSoftmax_f (kernels.h:88-103) and argMax_i (kernels.h:601-613).
+//
+// Softmax is one read and one write of the matrix (8 B/element): a 64-lane
+// wavefront owns a row, keeps it in registers as float4s, and reduces the row
+// maximum and the row sum with cross-lane shuffles; no LDS, no second read.
+// Rows that do not fit that scheme (n not a multiple of 4, unaligned, or more
+// than 64*4*kMaxVec columns) take the strided three-pass kernel, whose re-reads
+// hit cache because one row is a few KB.
+#include "common.hpp"
+
+using namespace swc_hip;
+
+namespace {
+
+constexpr int kWave = 64;
+constexpr int kRowsPerBlock = 4;  // wavefronts per block
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// exp(x) for x <= 0 through the hardware exp2; relative error ~2e-6 at x = -30,
+// far inside the 1e-4 contract.
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+
+// VEC = float4s per lane; row length n = 4*n4 with n4 <= 64*VEC.
+template <int VEC>
+__global__ __launch_bounds__(kWave *kRowsPerBlock) void softmax_rows_reg(const float *a, float *b, int m, int n4,
+                                                                         size_t lda, size_t ldb) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int row = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= m) return;
+    const float4 *src = reinterpret_cast<const float4 *>(a + (size_t)row * lda);
+    float4 *dst = reinterpret_cast<float4 *>(b + (size_t)row * ldb);
+    float4 v[VEC];
+    const float ninf = -__builtin_inff();
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) {
+        const int i = lane + u * kWave;
+        v[u] = (i < n4) ? src[i] : make_float4(ninf, ninf, ninf, ninf);
+    }
+    float mx = ninf;
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) mx = fmaxf(fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)), mx);
+    mx = wave_max(mx);
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) {
+        v[u].x = fast_exp(v[u].x - mx);
+        v[u].y = fast_exp(v[u].y - mx);
+        v[u].z = fast_exp(v[u].z - mx);
+        v[u].w = fast_exp(v[u].w - mx);
+        s += (v[u].x + v[u].y) + (v[u].z + v[u].w);   // padding lanes hold exp(-inf) = 0
+    }
+    s = wave_sum(s);
+    const float inv = 1.f / s;
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) {
+        const int i = lane + u * kWave;
+        if (i < n4) dst[i] = make_float4(v[u].x * inv, v[u].y * inv, v[u].z * inv, v[u].w * inv);
+    }
+}
+
+// any n, any alignment: wave per row, strided scalar accesses, three passes.
+__global__ __launch_bounds__(kWave *kRowsPerBlock) void softmax_rows_strided(const float *a, float *b, int m, int n,
+                                                                             size_t lda, size_t ldb) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int row = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= m) return;
+    const float *src = a + (size_t)row * lda;
+    float *dst = b + (size_t)row * ldb;
+    float mx = -__builtin_inff();
+    for (int j = lane; j < n; j += kWave) mx = fmaxf(mx, src[j]);
+    mx = wave_max(mx);
+    float s = 0.f;
+    for (int j = lane; j < n; j += kWave) s += fast_exp(src[j] - mx);
+    s = wave_sum(s);
+    const float inv = 1.f / s;
+    for (int j = lane; j < n; j += kWave) dst[j] = fast_exp(src[j] - mx) * inv;
+}
+
+// Small n (the classifier heads, n = 10): one lane per row would waste the
+// wave on strided loads; here a block stages 256 rows through registers with
+// each lane owning one row, which is fine because the whole matrix is tiny.
+__global__ __launch_bounds__(256) void softmax_rows_small(const float *a, float *b, int m, int n, size_t lda,
+                                                          size_t ldb) {
+    const int row = blockIdx.x * 256 + threadIdx.x;
+    if (row >= m) return;
+    const float *src = a + (size_t)row * lda;
+    float *dst = b + (size_t)row * ldb;
+    float mx = src[0];
+    for (int j = 1; j < n; ++j) mx = fmaxf(mx, src[j]);
+    float s = 0.f;
+    for (int j = 0; j < n; ++j) s += fast_exp(src[j] - mx);
+    const float inv = 1.f / s;
+    for (int j = 0; j < n; ++j) dst[j] = fast_exp(src[j] - mx) * inv;
+}
+
+// argMax_i: one lane per row; top_k <= 8 kept sorted in registers.  Order is
+// descending (value, column): a later column with an equal value goes first.
+constexpr int kMaxTopK = 8;
+__global__ __launch_bounds__(256) void argmax_rows(const float *in, int *idx, int m, int n, int top_k) {
+    const int row = blockIdx.x * 256 + threadIdx.x;
+    if (row >= m) return;
+    const float *src = in + (size_t)row * n;
+    float bv[kMaxTopK];
+    int bi[kMaxTopK];
+    int have = 0;
+    for (int j = 0; j < n; ++j) {
+        const float v = src[j];
+        // position of (v, j) among the kept ones
+        int pos = have;
+        for (int t = have - 1; t >= 0; --t) {
+            // (v,j) precedes (bv[t],bi[t]) when v > bv[t], or equal (j is always the larger column)
+            if (v > bv[t] || v == bv[t]) pos = t;
+            else break;
+        }
+        if (pos >= top_k) continue;
+        const int last = (have < top_k) ? have : top_k - 1;
+        for (int t = last; t > pos; --t) {
+            bv[t] = bv[t - 1];
+            bi[t] = bi[t - 1];
+        }
+        bv[pos] = v;
+        bi[pos] = j;
+        if (have < top_k) ++have;
+    }
+    for (int t = 0; t < top_k; ++t) idx[(size_t)row * top_k + t] = (t < have) ? bi[t] : 0;
+}
+
+} // namespace
+
+extern "C" {
+
+int swc_hip_matrixSoftmax_f(int m, int n, const float *a, int lda, float *b, int ldb) {
+    SWC_REQUIRE_INIT();
+    SWC_ARG(m >= 0 && n >= 0);
+    if (m == 0 || n == 0) return SWC_HIP_OK;
+    SWC_ARG(a && b && lda >= n && ldb >= n);
+    hipStream_t s = stream();
+    const bool vec_ok = (n % 4 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) && aligned16(a) && aligned16(b);
+    const int n4 = n / 4;
+    if (n <= 32) {
+        softmax_rows_small<<<ceil_div(m, 256), 256, 0, s>>>(a, b, m, n, lda, ldb);
+    } else if (vec_ok && n4 <= kWave * 8) {
+        const unsigned blocks = ceil_div(m, kRowsPerBlock);
+        const dim3 block(kWave * kRowsPerBlock);
+        if (n4 <= kWave * 1) softmax_rows_reg<1><<<blocks, block, 0, s>>>(a, b, m, n4, lda, ldb);
+        else if (n4 <= kWave * 2) softmax_rows_reg<2><<<blocks, block, 0, s>>>(a, b, m, n4, lda, ldb);
+        else if (n4 <= kWave * 4) softmax_rows_reg<4><<<blocks, block, 0, s>>>(a, b, m, n4, lda, ldb);
+        else softmax_rows_reg<8><<<blocks, block, 0, s>>>(a, b, m, n4, lda, ldb);
+    } else {
+        softmax_rows_strided<<<ceil_div(m, kRowsPerBlock), kWave * kRowsPerBlock, 0, s>>>(a, b, m, n, lda, ldb);
+    }
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
+}
+
+int swc_hip_argMax_i(const float *input, int *idx, int m, int n, int top_k) {
+    SWC_REQUIRE_INIT();
+    SWC_ARG(m >= 0 && n >= 0 && top_k >= 0);
+    if (m == 0 || top_k == 0) return SWC_HIP_OK;
+    SWC_ARG(input && idx && top_k <= n);
+    if (top_k > kMaxTopK)
+        return fail(SWC_HIP_EUNSUPPORTED, "swc_hip_argMax_i: top_k %d exceeds %d", top_k, kMaxTopK);
+    argmax_rows<<<ceil_div(m, 256), 256, 0, stream()>>>(input, idx, m, n, top_k);
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,320 @@
+"""ctypes binding of libswc_hip.so (C ABI declared in include/swc_hip.h).
+
+Method names and argument order mirror the reference's CPU kernels
+(src/codegen/utils/kernels.h) — the same correspondence the C ABI keeps — so a
+parity test reads like a call sequence of the reference's generated program.
+Data lives in DeviceArray objects (device memory + shape); numpy arrays cross
+only through upload()/download().
+
+No fallback: a missing library or device raises SwcHipError.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+EXPORTS = [
+    "swc_hip_init", "swc_hip_shutdown", "swc_hip_malloc", "swc_hip_free", "swc_hip_h2d", "swc_hip_d2h",
+    "swc_hip_d2d", "swc_hip_fill_f", "swc_hip_sync", "swc_hip_last_error", "swc_hip_stream",
+    "swc_hip_set_stream", "swc_hip_device_name", "swc_hip_timer_begin", "swc_hip_timer_end",
+    "swc_hip_timer_elapsed_ms", "swc_hip_event_record", "swc_hip_event_elapsed_ms", "swc_hip_matrixMatrixMul_f", "swc_hip_batchedadd_f", "swc_hip_relu_f",
+    "swc_hip_vecAdd_f", "swc_hip_conv2d_f", "swc_hip_batchnormalization_f", "swc_hip_maxpool_f",
+    "swc_hip_maxpool_argmax_f", "swc_hip_matrixSoftmax_f", "swc_hip_matrixTanh_f", "swc_hip_argMax_i",
+    "swc_hip_matrixMatrixFCBias_f", "swc_hip_vecAddRelu_f", "swc_hip_batchnormRelu_f",
+    "swc_hip_batchnormReluMaxpool_f", "swc_hip_conv2dFused_f",
+]
+
+
+class SwcHipError(RuntimeError):
+    pass
+
+
+def lib_path():
+    return os.path.join(_HERE, "libswc_hip.so")
+
+
+def load_library():
+    """dlopen the in-tree library; raises if it has not been built."""
+    path = lib_path()
+    if not os.path.exists(path):
+        raise SwcHipError(f"{path} is missing: build it with `python -m swcompiler_amd.build` "
+                          "(there is no CPU fallback)")
+    lib = C.CDLL(path)
+    vp, sz, i32, f32 = C.c_void_p, C.c_size_t, C.c_int, C.c_float
+    szp = C.POINTER(C.c_size_t)
+    sig = {
+        "swc_hip_init": (i32, [i32]),
+        "swc_hip_shutdown": (i32, []),
+        "swc_hip_malloc": (vp, [sz]),
+        "swc_hip_free": (i32, [vp]),
+        "swc_hip_h2d": (i32, [vp, vp, sz]),
+        "swc_hip_d2h": (i32, [vp, vp, sz]),
+        "swc_hip_d2d": (i32, [vp, vp, sz]),
+        "swc_hip_fill_f": (i32, [vp, f32, sz]),
+        "swc_hip_sync": (i32, []),
+        "swc_hip_last_error": (C.c_char_p, []),
+        "swc_hip_stream": (vp, []),
+        "swc_hip_set_stream": (i32, [vp]),
+        "swc_hip_device_name": (C.c_char_p, []),
+        "swc_hip_timer_begin": (i32, []),
+        "swc_hip_timer_end": (i32, []),
+        "swc_hip_timer_elapsed_ms": (f32, []),
+        "swc_hip_event_record": (i32, [i32]),
+        "swc_hip_event_elapsed_ms": (f32, [i32, i32]),
+        "swc_hip_matrixMatrixMul_f": (i32, [i32, i32, i32, vp, i32, vp, i32, vp, i32]),
+        "swc_hip_batchedadd_f": (i32, [vp, vp, vp, sz, sz]),
+        "swc_hip_relu_f": (i32, [vp, vp, sz]),
+        "swc_hip_vecAdd_f": (i32, [i32, vp, vp, vp]),
+        "swc_hip_conv2d_f": (i32, [vp, vp, vp, vp, szp, szp, szp, szp, szp, szp, szp, sz]),
+        "swc_hip_batchnormalization_f": (i32, [vp, vp, vp, vp, vp, vp, szp, f32]),
+        "swc_hip_maxpool_f": (i32, [vp, vp, szp, szp, szp, szp, szp]),
+        "swc_hip_maxpool_argmax_f": (i32, [vp, vp, vp, szp, szp, szp, szp, szp]),
+        "swc_hip_matrixSoftmax_f": (i32, [i32, i32, vp, i32, vp, i32]),
+        "swc_hip_matrixTanh_f": (i32, [i32, i32, vp, i32, vp, i32]),
+        "swc_hip_argMax_i": (i32, [vp, vp, i32, i32, i32]),
+        "swc_hip_matrixMatrixFCBias_f": (i32, [i32, i32, i32, vp, i32, vp, i32, vp, vp, i32, i32]),
+        "swc_hip_vecAddRelu_f": (i32, [i32, vp, vp, vp]),
+        "swc_hip_batchnormRelu_f": (i32, [vp, vp, vp, vp, vp, vp, szp, f32]),
+        "swc_hip_batchnormReluMaxpool_f": (i32, [vp, vp, vp, vp, vp, vp, szp, f32, szp, szp, szp, szp]),
+        "swc_hip_conv2dFused_f": (i32, [vp, vp, vp, vp, szp, szp, szp, szp, szp, szp, szp, sz,
+                                        vp, vp, vp, vp, f32, i32]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = res, args
+    return lib
+
+
+def _dims(seq):
+    return (C.c_size_t * len(seq))(*[int(v) for v in seq])
+
+
+def pool_out_dims(idims, kernels, strides, pads):
+    """src/op/dlOp/dlOp.cpp:195-196: o = (i + pad_begin + pad_end - k) / s + 1, pads = {t,l,b,r}."""
+    n, h, w, c = idims
+    return (n, (h + pads[0] + pads[2] - kernels[0]) // strides[0] + 1,
+            (w + pads[1] + pads[3] - kernels[1]) // strides[1] + 1, c)
+
+
+class DeviceArray:
+    """A device allocation with a shape and dtype (float32 or int32)."""
+
+    def __init__(self, rt, shape, dtype=np.float32):
+        self.rt = rt
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+        self.size = int(np.prod(self.shape)) if self.shape else 1
+        self.nbytes = self.size * self.dtype.itemsize
+        self.ptr = rt._malloc(self.nbytes)
+
+    def reshape(self, *shape):
+        view = object.__new__(DeviceArray)
+        view.__dict__.update(self.__dict__)
+        shape = tuple(shape[0]) if len(shape) == 1 and not np.isscalar(shape[0]) else tuple(shape)
+        if -1 in shape:
+            known = int(np.prod([s for s in shape if s != -1]))
+            shape = tuple(self.size // known if s == -1 else s for s in shape)
+        view.shape = tuple(int(s) for s in shape)
+        assert int(np.prod(view.shape)) == self.size
+        view._base = self  # keep the owner alive; views never free
+        return view
+
+    def numpy(self):
+        return self.rt.download(self)
+
+    def offset_view(self, first, shape):
+        """A view starting `first` elements in (to exercise unaligned pointers)."""
+        view = self.reshape(self.shape)
+        view.shape = tuple(int(s) for s in shape)
+        view.size = int(np.prod(view.shape))
+        assert first + view.size <= self.size
+        view.nbytes = view.size * self.dtype.itemsize
+        view.ptr = self.ptr + first * self.dtype.itemsize
+        return view
+
+    def free(self):
+        if getattr(self, "_base", None) is None and self.ptr:
+            self.rt._free(self.ptr)
+        self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class SwcHip:
+    """One process-wide runtime: device 0 unless told otherwise."""
+
+    def __init__(self, device=0):
+        self.lib = load_library()
+        self._check(self.lib.swc_hip_init(device), "swc_hip_init")
+
+    # -- plumbing --------------------------------------------------------
+    def _check(self, rc, what):
+        if rc != 0:
+            raise SwcHipError(f"{what} failed ({rc}): {self.lib.swc_hip_last_error().decode()}")
+
+    def _malloc(self, nbytes):
+        p = self.lib.swc_hip_malloc(nbytes)
+        if not p:
+            raise SwcHipError(self.lib.swc_hip_last_error().decode())
+        return p
+
+    def _free(self, ptr):
+        self.lib.swc_hip_free(ptr)
+
+    def device_name(self):
+        return self.lib.swc_hip_device_name().decode()
+
+    def empty(self, shape, dtype=np.float32):
+        return DeviceArray(self, shape, dtype)
+
+    def upload(self, host):
+        host = np.ascontiguousarray(host)
+        assert host.dtype in (np.float32, np.int32)
+        d = DeviceArray(self, host.shape, host.dtype)
+        self._check(self.lib.swc_hip_h2d(d.ptr, host.ctypes.data, host.nbytes), "swc_hip_h2d")
+        return d
+
+    def download(self, d):
+        host = np.empty(d.shape, d.dtype)
+        self._check(self.lib.swc_hip_d2h(host.ctypes.data, d.ptr, d.nbytes), "swc_hip_d2h")
+        return host
+
+    def sync(self):
+        self._check(self.lib.swc_hip_sync(), "swc_hip_sync")
+
+    def timer_begin(self):
+        self._check(self.lib.swc_hip_timer_begin(), "swc_hip_timer_begin")
+
+    def timer_end_ms(self):
+        self._check(self.lib.swc_hip_timer_end(), "swc_hip_timer_end")
+        return float(self.lib.swc_hip_timer_elapsed_ms())
+
+    def event_record(self, slot):
+        self._check(self.lib.swc_hip_event_record(slot), "swc_hip_event_record")
+
+    def event_elapsed_ms(self, first, second):
+        ms = float(self.lib.swc_hip_event_elapsed_ms(first, second))
+        if ms < 0:
+            raise SwcHipError("swc_hip_event_elapsed_ms failed: " + self.lib.swc_hip_last_error().decode())
+        return ms
+
+    # -- ops (device in, device out) -------------------------------------
+    def matrixMatrixMul(self, a, b, out=None):
+        m, k = a.shape
+        k2, n = b.shape
+        assert k == k2
+        out = out if out is not None else self.empty((m, n))
+        self._check(self.lib.swc_hip_matrixMatrixMul_f(m, n, k, a.ptr, k, b.ptr, n, out.ptr, n), "matrixMatrixMul_f")
+        return out
+
+    def batchedadd(self, batch, slice_, out=None):
+        rows, cols = batch.shape
+        out = out if out is not None else self.empty(batch.shape)
+        self._check(self.lib.swc_hip_batchedadd_f(out.ptr, batch.ptr, slice_.ptr, rows, cols), "batchedadd_f")
+        return out
+
+    def fcbias(self, a, w, bias, relu=False, out=None):
+        m, k = a.shape
+        k2, n = w.shape
+        assert k == k2
+        out = out if out is not None else self.empty((m, n))
+        self._check(self.lib.swc_hip_matrixMatrixFCBias_f(m, n, k, a.ptr, k, w.ptr, n,
+                                                          bias.ptr if bias is not None else None,
+                                                          out.ptr, n, int(relu)), "matrixMatrixFCBias_f")
+        return out
+
+    def relu(self, x, out=None):
+        out = out if out is not None else self.empty(x.shape)
+        self._check(self.lib.swc_hip_relu_f(x.ptr, out.ptr, x.size), "relu_f")
+        return out
+
+    def vecAdd(self, a, b, out=None, relu=False):
+        assert a.shape == b.shape
+        out = out if out is not None else self.empty(a.shape)
+        fn = self.lib.swc_hip_vecAddRelu_f if relu else self.lib.swc_hip_vecAdd_f
+        self._check(fn(a.size, a.ptr, b.ptr, out.ptr), "vecAdd_f")
+        return out
+
+    def matrixTanh(self, a, out=None):
+        m, n = a.shape
+        out = out if out is not None else self.empty(a.shape)
+        self._check(self.lib.swc_hip_matrixTanh_f(m, n, a.ptr, n, out.ptr, n), "matrixTanh_f")
+        return out
+
+    def matrixSoftmax(self, a, out=None):
+        m, n = a.shape
+        out = out if out is not None else self.empty(a.shape)
+        self._check(self.lib.swc_hip_matrixSoftmax_f(m, n, a.ptr, n, out.ptr, n), "matrixSoftmax_f")
+        return out
+
+    def argMax(self, x, top_k):
+        m, n = x.shape
+        out = self.empty((m, top_k), np.int32)
+        self._check(self.lib.swc_hip_argMax_i(x.ptr, out.ptr, m, n, top_k), "argMax_i")
+        return out
+
+    def conv2d(self, x, filt, bias, kernels=None, strides=(1, 1), pads=(0, 0, 0, 0), group=1, bn=None,
+               eps=1e-5, relu=False, out=None):
+        """bn = (mean, var, scale, bias) DeviceArrays to fuse inference batchnorm."""
+        if kernels is None:
+            kernels = filt.shape[1:3]
+        n, oh, ow, _ = pool_out_dims(x.shape, kernels, strides, pads)
+        odims = (n, oh, ow, filt.shape[0])
+        out = out if out is not None else self.empty(odims)
+        shp = (_dims(odims), _dims(x.shape), _dims(filt.shape), _dims(bias.shape), _dims(kernels),
+               _dims(strides), _dims(pads))
+        if bn is None and not relu:
+            rc = self.lib.swc_hip_conv2d_f(out.ptr, x.ptr, filt.ptr, bias.ptr, *shp, group)
+        else:
+            ptrs = [p.ptr for p in bn] if bn is not None else [None] * 4
+            rc = self.lib.swc_hip_conv2dFused_f(out.ptr, x.ptr, filt.ptr, bias.ptr, *shp, group, *ptrs,
+                                                eps, int(relu))
+        self._check(rc, "conv2d_f")
+        return out
+
+    def batchnormalization(self, x, mean, var, scale, bias, eps, relu=False, out=None):
+        out = out if out is not None else self.empty(x.shape)
+        fn = self.lib.swc_hip_batchnormRelu_f if relu else self.lib.swc_hip_batchnormalization_f
+        self._check(fn(out.ptr, x.ptr, mean.ptr, var.ptr, scale.ptr, bias.ptr, _dims(x.shape), eps),
+                    "batchnormalization_f")
+        return out
+
+    def maxpool(self, x, kernels, strides, pads=(0, 0, 0, 0), out=None):
+        odims = pool_out_dims(x.shape, kernels, strides, pads)
+        out = out if out is not None else self.empty(odims)
+        self._check(self.lib.swc_hip_maxpool_f(x.ptr, out.ptr, _dims(x.shape), _dims(odims), _dims(kernels),
+                                               _dims(strides), _dims(pads)), "maxpool_f")
+        return out
+
+    def maxpool_argmax(self, x, kernels, strides, pads=(0, 0, 0, 0)):
+        odims = pool_out_dims(x.shape, kernels, strides, pads)
+        out, idx = self.empty(odims), self.empty(odims, np.int32)
+        self._check(self.lib.swc_hip_maxpool_argmax_f(x.ptr, out.ptr, idx.ptr, _dims(x.shape), _dims(odims),
+                                                      _dims(kernels), _dims(strides), _dims(pads)),
+                    "maxpool_argmax_f")
+        return out, idx
+
+    def batchnormReluMaxpool(self, x, mean, var, scale, bias, eps, kernels, strides, pads=(0, 0, 0, 0), out=None):
+        odims = pool_out_dims(x.shape, kernels, strides, pads)
+        out = out if out is not None else self.empty(odims)
+        self._check(self.lib.swc_hip_batchnormReluMaxpool_f(out.ptr, x.ptr, mean.ptr, var.ptr, scale.ptr, bias.ptr,
+                                                            _dims(x.shape), eps, _dims(odims), _dims(kernels),
+                                                            _dims(strides), _dims(pads)), "batchnormReluMaxpool_f")
+        return out
+
+
+_RT = None
+
+
+def runtime():
+    """The process-wide SwcHip instance (created on first use)."""
+    global _RT
+    if _RT is None:
+        _RT = SwcHip(0)
+    return _RT

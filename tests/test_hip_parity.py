@@ -1,0 +1,340 @@
+"""Parity of the HIP kernels (through the C ABI) against the CPU oracle.
+
+Bit-exact: relu, vecAdd, batchedadd, maxpool (values and chosen tap).
+Within 1e-4 relative: GEMM/FC, conv, batchnorm, softmax, tanh.  For batchnorm,
+softmax and tanh that is the strict element-wise |g-w|/|w|.  For the
+contractions (GEMM, conv) the HIP kernels add the k products in a different
+order than the oracle's sequential fp32 loop, and two fp32 orders of one dot
+product differ by ~k*eps*sum|a||b| however small the cancelled result is; so
+  * on non-negative operands (no cancellation) the strict element-wise relative
+    error is asserted, and
+  * on signed operands the error is taken relative to sum_k|a_ik||b_kj| (+|bias|)
+    (tests/util.py scaled_err),
+both against 1e-4, and integer-valued operands (exact in any order) are asserted
+bit-exact.
+"""
+import itertools
+import os
+
+import numpy as np
+import pytest
+
+from tests.util import assert_bit_exact, rel_err, scaled_err, strict_rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from swcompiler_amd.hip import runtime
+    return runtime()
+
+
+def up(rt, *arrays):
+    return [rt.upload(a) for a in arrays]
+
+
+# ------------------------------------------------------------ elementwise
+@pytest.mark.parametrize("n", [0, 1, 3, 4, 1031, 4096, (1 << 20) + 5])
+def test_relu_add_bit_exact(rt, oracle, n):
+    print("case relu/add n =", n, flush=True)
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(np.float32)
+    y = rng.standard_normal(n).astype(np.float32)
+    if n >= 8:
+        x[:8] = [0.0, -0.0, np.nan, np.inf, -np.inf, 1e-45, -1e-45, 3.0]
+        y[:8] = [-0.0, -0.0, 1.0, -np.inf, -np.inf, 1e-45, 1e-45, -3.0]
+    dx, dy = up(rt, x, y)
+    assert_bit_exact(rt.relu(dx).numpy(), oracle.relu(x), "relu")
+    assert_bit_exact(rt.vecAdd(dx, dy).numpy(), oracle.vecAdd(x, y), "vecAdd")
+    assert_bit_exact(rt.vecAdd(dx, dy, relu=True).numpy(), oracle.relu(oracle.vecAdd(x, y)), "vecAddRelu")
+
+
+def test_relu_unaligned_and_in_place(rt, oracle):
+    x = np.random.default_rng(0).standard_normal(5000).astype(np.float32)
+    d = rt.upload(x)
+    v = d.offset_view(1, (4099,))
+    out = rt.empty((5000,))
+    o = out.offset_view(3, (4099,))
+    rt.relu(v, out=o)
+    assert_bit_exact(o.numpy(), oracle.relu(x[1:4100]), "unaligned relu")
+    rt.relu(d, out=d)
+    assert_bit_exact(d.numpy(), oracle.relu(x), "in-place relu")
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (8, 512), (33, 10), (256, 500), (7, 4096)])
+def test_batchedadd_bit_exact(rt, oracle, rows, cols):
+    rng = np.random.default_rng(rows * cols)
+    a = rng.standard_normal((rows, cols)).astype(np.float32)
+    b = rng.standard_normal(cols).astype(np.float32)
+    da, db = up(rt, a, b)
+    assert_bit_exact(rt.batchedadd(da, db).numpy(), oracle.batchedadd(a, b), "batchedadd")
+
+
+def test_tanh(rt, oracle, golden):
+    x = golden["tanh_x"]
+    got = rt.matrixTanh(rt.upload(x)).numpy()
+    assert np.max(np.abs(got - golden["tanh_y"])) < 1e-6
+    assert rel_err(got, oracle.matrixTanh(x)) < TOL
+
+
+# ------------------------------------------------------------------ GEMM
+GEMM_SHAPES = [(1, 1, 1), (7, 13, 5), (33, 100, 17), (8, 784, 512), (64, 96, 130), (130, 70, 257),
+               (256, 800, 500), (200, 512, 128), (129, 33, 129), (64, 300, 10), (8, 512, 10),
+               (256, 500, 10), (100, 4096, 10), (17, 37, 16), (300, 64, 20)]
+
+
+@pytest.mark.parametrize("m,k,n", GEMM_SHAPES)
+def test_gemm_vs_oracle(rt, oracle, m, k, n):
+    print(f"case gemm {m}x{k}x{n}", flush=True)
+    rng = np.random.default_rng(m * 1000003 + k * 1009 + n)
+    a = rng.uniform(0, 1, (m, k)).astype(np.float32)
+    b = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32)
+    bias = rng.uniform(-0.01, 0.01, n).astype(np.float32)
+    da, db, dbias = up(rt, a, b, bias)
+    want = oracle.matrixMatrixMul(a, b)
+    mag = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64) + np.abs(bias)
+    assert scaled_err(rt.matrixMatrixMul(da, db).numpy(), want, mag) < TOL
+    assert scaled_err(rt.fcbias(da, db, dbias).numpy(), oracle.batchedadd(want, bias), mag) < TOL
+    assert scaled_err(rt.fcbias(da, db, dbias, relu=True).numpy(), oracle.relu(oracle.batchedadd(want, bias)), mag) < TOL
+    # no cancellation: strict element-wise relative error
+    bp = np.abs(b)
+    assert strict_rel_err(rt.matrixMatrixMul(da, rt.upload(bp)).numpy(), oracle.matrixMatrixMul(a, bp)) < TOL
+
+
+@pytest.mark.parametrize("m,k,n", [(70, 45, 90), (130, 260, 136), (40, 64, 12), (128, 128, 128)])
+def test_gemm_integer_valued_is_exact(rt, m, k, n):
+    """Small integers make every partial sum exact in fp32, so any summation
+    order must give the same bits; catches a wrong fragment/lane mapping."""
+    rng = np.random.default_rng(m + k + n)
+    a = rng.integers(-8, 9, (m, k)).astype(np.float32)
+    b = rng.integers(-8, 9, (k, n)).astype(np.float32)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    da, db = up(rt, a, b)
+    assert_bit_exact(rt.matrixMatrixMul(da, db).numpy(), want, "integer gemm")
+
+
+@pytest.mark.parametrize("tag", ["a", "b", "c", "d", "e"])
+def test_gemm_golden(rt, golden, tag):
+    da, db, dbias = up(rt, golden[f"gemm_{tag}_a"], golden[f"gemm_{tag}_b"], golden[f"gemm_{tag}_bias"])
+    a, b = golden[f"gemm_{tag}_a"], golden[f"gemm_{tag}_b"]
+    mag = np.abs(a).astype(np.float64) @ np.abs(b) + np.abs(golden[f"gemm_{tag}_bias"])
+    assert scaled_err(rt.matrixMatrixMul(da, db).numpy(), golden[f"gemm_{tag}_c"], mag) < TOL
+    assert scaled_err(rt.fcbias(da, db, dbias).numpy(), golden[f"gemm_{tag}_cb"], mag) < TOL
+
+
+def test_gemm_full_size_rows(rt, oracle):
+    """4096x4096x4096 (the GEMM-bound layer of the wide MLP): the oracle is run
+    on 12 sampled rows of A, which fixes those rows of C exactly."""
+    rng = np.random.default_rng(42)
+    m = k = n = 4096
+    a = rng.uniform(0, 1, (m, k)).astype(np.float32)
+    b = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32)
+    bias = rng.uniform(-0.01, 0.01, n).astype(np.float32)
+    da, db, dbias = up(rt, a, b, bias)
+    got = rt.fcbias(da, db, dbias, relu=True).numpy()
+    rows = np.array([0, 1, 31, 32, 63, 64, 127, 128, 2047, 2048, 4094, 4095])
+    want = oracle.relu(oracle.batchedadd(oracle.matrixMatrixMul(a[rows], b), bias))
+    mag = a[rows].astype(np.float64) @ np.abs(b) + np.abs(bias)
+    assert scaled_err(got[rows], want, mag) < TOL
+    bp = np.abs(b)
+    assert strict_rel_err(rt.matrixMatrixMul(da, rt.upload(bp)).numpy()[rows], oracle.matrixMatrixMul(a[rows], bp)) < TOL
+    # linearity in A over the whole output: (2A)B == 2(AB) exactly in fp32
+    got2 = rt.matrixMatrixMul(rt.upload(a * np.float32(2)), db).numpy()
+    assert_bit_exact(got2, rt.matrixMatrixMul(da, db).numpy() * np.float32(2), "scaling by 2")
+
+
+# ------------------------------------------------------------------ conv
+CONVS = [((2, 9, 9, 3), (4, 3, 3, 3), (1, 1), (1, 1, 1, 1)),
+         ((2, 28, 28, 1), (20, 5, 5, 1), (1, 1), (0, 0, 0, 0)),
+         ((2, 12, 12, 20), (50, 5, 5, 20), (1, 1), (0, 0, 0, 0)),
+         ((1, 14, 14, 64), (64, 3, 3, 64), (1, 1), (1, 1, 1, 1)),
+         ((1, 14, 14, 64), (128, 3, 3, 64), (1, 1), (1, 1, 1, 1)),
+         ((2, 15, 13, 8), (6, 3, 5, 8), (2, 3), (1, 2, 1, 2)),
+         ((1, 10, 10, 3), (4, 7, 7, 3), (2, 2), (3, 3, 3, 3)),
+         ((3, 5, 5, 16), (8, 1, 1, 16), (1, 1), (0, 0, 0, 0)),
+         ((1, 8, 7, 4), (3, 3, 2, 4), (1, 2), (2, 0, 1, 1)),
+         ((4, 28, 28, 128), (128, 3, 3, 128), (1, 1), (1, 1, 1, 1)),
+         ((2, 56, 56, 64), (64, 3, 3, 64), (1, 1), (1, 1, 1, 1))]
+
+
+@pytest.mark.parametrize("idims,fdims,strides,pads", CONVS)
+def test_conv_vs_oracle(rt, oracle, idims, fdims, strides, pads):
+    print("case conv", idims, fdims, strides, pads, flush=True)
+    rng = np.random.default_rng(sum(idims) * 131 + sum(fdims))
+    x = rng.standard_normal(idims).astype(np.float32)
+    f = (rng.standard_normal(fdims) / np.sqrt(np.prod(fdims[1:]))).astype(np.float32)
+    b = (rng.standard_normal(fdims[0]) * 0.1).astype(np.float32)
+    c = fdims[0]
+    mean, beta = (rng.standard_normal(c) * 0.1).astype(np.float32), (rng.standard_normal(c) * 0.1).astype(np.float32)
+    var, gamma = rng.uniform(0.5, 2, c).astype(np.float32), rng.uniform(0.5, 1.5, c).astype(np.float32)
+    dx, df, db, dm, dv, dg, dbe = up(rt, x, f, b, mean, var, gamma, beta)
+    want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
+    mag = oracle.conv2d(np.abs(x), np.abs(f), np.abs(b), fdims[1:3], strides, pads)   # sum of |terms|
+    got = rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy()
+    assert got.shape == want.shape
+    assert scaled_err(got, want, mag) < TOL
+    assert scaled_err(rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True).numpy(), oracle.relu(want), mag) < TOL
+    want_bn = oracle.relu(oracle.batchnormalization(want, mean, var, gamma, beta, 1e-5))
+    got_bn = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, bn=(dm, dv, dg, dbe), eps=1e-5, relu=True).numpy()
+    mag_bn = (mag + np.abs(mean)) * (gamma / np.sqrt(var + 1e-5)) + np.abs(beta)
+    assert scaled_err(got_bn, want_bn, mag_bn) < TOL
+    # no cancellation: strict element-wise relative error
+    xp, fp = np.abs(x), np.abs(f)
+    assert strict_rel_err(rt.conv2d(rt.upload(xp), rt.upload(fp), db, fdims[1:3], strides, pads, relu=True).numpy(),
+                          oracle.relu(oracle.conv2d(xp, fp, b, fdims[1:3], strides, pads))) < TOL
+
+
+def test_conv_integer_valued_is_exact(rt):
+    rng = np.random.default_rng(9)
+    for idims, fdims, pads in [((2, 9, 10, 8), (40, 3, 3, 8), (1, 1, 1, 1)), ((1, 12, 12, 3), (70, 5, 5, 3), (2, 2, 2, 2))]:
+        x = rng.integers(-4, 5, idims).astype(np.float32)
+        f = rng.integers(-4, 5, fdims).astype(np.float32)
+        b = rng.integers(-4, 5, fdims[0]).astype(np.float32)
+        n, h, w, ci = idims
+        co, kh, kw, _ = fdims
+        xp = np.zeros((n, h + 2 * pads[0], w + 2 * pads[1], ci), np.int64)
+        xp[:, pads[0]:pads[0] + h, pads[1]:pads[1] + w] = x
+        oh, ow = h + 2 * pads[0] - kh + 1, w + 2 * pads[1] - kw + 1
+        want = np.zeros((n, oh, ow, co), np.int64) + b.astype(np.int64)
+        for ky, kx in itertools.product(range(kh), range(kw)):
+            want += xp[:, ky:ky + oh, kx:kx + ow] @ f[:, ky, kx].astype(np.int64).T
+        got = rt.conv2d(*up(rt, x, f, b), fdims[1:3], (1, 1), pads).numpy()
+        assert_bit_exact(got, want.astype(np.float32), "integer conv")
+
+
+@pytest.mark.parametrize("tag", ["p1", "k5", "s2", "asym", "k1", "c64"])
+def test_conv_golden(rt, golden, tag):
+    x, f, b, sp = (golden[f"conv_{tag}_{k}"] for k in ("x", "f", "b", "sp"))
+    st, pd = tuple(int(v) for v in sp[:2]), tuple(int(v) for v in sp[2:])
+    got = rt.conv2d(*up(rt, x, f, b), f.shape[1:3], st, pd).numpy()
+    from oracle.binding import load_oracle
+    mag = load_oracle().conv2d(np.abs(x), np.abs(f), np.abs(b), f.shape[1:3], st, pd)
+    assert scaled_err(got, golden[f"conv_{tag}_y"], mag) < TOL
+
+
+def test_conv_rejects_groups(rt):
+    from swcompiler_amd.hip import SwcHipError
+    x, f, b = up(rt, np.zeros((1, 4, 4, 4), np.float32), np.zeros((4, 1, 1, 4), np.float32), np.zeros(4, np.float32))
+    with pytest.raises(SwcHipError, match="group"):
+        rt.conv2d(x, f, b, group=2)
+
+
+# ------------------------------------------------------- batchnorm / pool
+@pytest.mark.parametrize("idims", [(2, 5, 5, 8), (1, 3, 4, 130), (3, 7, 7, 20), (2, 4, 4, 3), (4, 28, 28, 128), (1, 1, 1, 1)])
+def test_batchnorm(rt, oracle, idims):
+    rng = np.random.default_rng(sum(idims))
+    c = idims[3]
+    x = rng.standard_normal(idims).astype(np.float32)
+    mean, beta = (rng.standard_normal(c) * 0.1).astype(np.float32), (rng.standard_normal(c) * 0.1).astype(np.float32)
+    var, gamma = rng.uniform(0.5, 2, c).astype(np.float32), rng.uniform(0.5, 1.5, c).astype(np.float32)
+    dx, dm, dv, dg, db = up(rt, x, mean, var, gamma, beta)
+    want = oracle.batchnormalization(x, mean, var, gamma, beta, 1e-5)
+    got = rt.batchnormalization(dx, dm, dv, dg, db, 1e-5).numpy()
+    # double arithmetic on both sides: at most the last bit may differ (pow vs 1/sqrt)
+    assert np.max(np.abs(got.view(np.int32).astype(np.int64) - want.view(np.int32))) <= 1
+    assert strict_rel_err(got, want) < TOL
+    got_r = rt.batchnormalization(dx, dm, dv, dg, db, 1e-5, relu=True).numpy()
+    assert_bit_exact(got_r, oracle.relu(got), "fused relu of the same bn values")
+
+
+POOLS = [((2, 8, 8, 5), (2, 2), (2, 2), (0, 0, 0, 0)), ((1, 9, 9, 3), (3, 3), (3, 3), (0, 0, 0, 0)),
+         ((2, 7, 9, 4), (3, 3), (2, 2), (1, 1, 1, 1)), ((1, 7, 7, 2), (2, 2), (2, 2), (0, 0, 0, 0)),
+         ((3, 24, 24, 20), (2, 2), (2, 2), (0, 0, 0, 0)), ((2, 8, 8, 50), (2, 2), (2, 2), (0, 0, 0, 0)),
+         ((2, 28, 28, 128), (2, 2), (2, 2), (0, 0, 0, 0)), ((1, 9, 9, 8), (3, 2), (1, 3), (0, 1, 0, 1))]
+
+
+@pytest.mark.parametrize("idims,k,s,p", POOLS)
+def test_maxpool_bit_exact_with_first_max(rt, oracle, idims, k, s, p):
+    print("case pool", idims, k, s, p, flush=True)
+    rng = np.random.default_rng(sum(idims) + k[0])
+    x = (np.round(rng.standard_normal(idims) * 2) / 2).astype(np.float32)  # many ties
+    x.flat[::17] = np.float32(-0.0)
+    x.flat[5::29] = np.nan
+    x.flat[7::31] = -np.inf
+    want, want_idx = oracle.maxpool_argmax(x, k, s, p)
+    dx = rt.upload(x)
+    assert_bit_exact(rt.maxpool(dx, k, s, p).numpy(), want, "maxpool")
+    got, idx = rt.maxpool_argmax(dx, k, s, p)
+    assert_bit_exact(got.numpy(), want, "maxpool(argmax variant)")
+    assert_bit_exact(idx.numpy(), want_idx, "argmax")
+
+
+@pytest.mark.parametrize("tag", ["k2", "k3s3", "k3s2p1", "odd"])
+def test_maxpool_golden(rt, golden, tag):
+    x = golden[f"pool_{tag}_x"]
+    ksp = [int(v) for v in golden[f"pool_{tag}_ksp"]]
+    got, idx = rt.maxpool_argmax(rt.upload(x), ksp[:2], ksp[2:4], ksp[4:])
+    assert_bit_exact(got.numpy(), golden[f"pool_{tag}_y"], "maxpool golden")
+    scat = np.zeros(x.size, np.float32)
+    np.add.at(scat, idx.numpy().ravel(), np.arange(1, got.size + 1, dtype=np.float32))
+    assert_bit_exact(scat.reshape(x.shape), golden[f"pool_{tag}_scatter"], "chosen tap golden")
+
+
+def test_bn_relu_maxpool_fused_equals_sequence(rt, oracle):
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((2, 16, 16, 64)).astype(np.float32)
+    c = 64
+    mean, beta = (rng.standard_normal(c) * 0.1).astype(np.float32), (rng.standard_normal(c) * 0.1).astype(np.float32)
+    var, gamma = rng.uniform(0.5, 2, c).astype(np.float32), rng.uniform(0.5, 1.5, c).astype(np.float32)
+    dx, dm, dv, dg, db = up(rt, x, mean, var, gamma, beta)
+    seq = rt.maxpool(rt.batchnormalization(dx, dm, dv, dg, db, 1e-5, relu=True), (2, 2), (2, 2)).numpy()
+    fused = rt.batchnormReluMaxpool(dx, dm, dv, dg, db, 1e-5, (2, 2), (2, 2)).numpy()
+    assert_bit_exact(fused, seq, "bn+relu+pool fused vs sequence")
+    want = oracle.maxpool(oracle.relu(oracle.batchnormalization(x, mean, var, gamma, beta, 1e-5)), (2, 2), (2, 2))
+    assert rel_err(fused, want) < TOL
+
+
+# --------------------------------------------------------------- softmax
+@pytest.mark.parametrize("m,n,sigma", [(8, 10, 1.0), (5, 1000, 3.0), (3, 1, 1.0), (4, 67, 30.0), (64, 1000, 3.0),
+                                       (9, 256, 3.0), (7, 2048, 3.0), (3, 5000, 3.0), (4096, 10, 2.0), (33, 36, 5.0)])
+def test_softmax(rt, oracle, m, n, sigma):
+    print(f"case softmax {m}x{n}", flush=True)
+    x = (np.random.default_rng(m * n).standard_normal((m, n)) * sigma).astype(np.float32)
+    want = oracle.matrixSoftmax(x)
+    got = rt.matrixSoftmax(rt.upload(x)).numpy()
+    nz = want > 1e-30  # exp underflow region: both sides are ~0, relative error is undefined there
+    assert strict_rel_err(got[nz], want[nz]) < TOL
+    assert np.all(got[~nz] < 1e-29)
+    assert np.allclose(got.sum(1, dtype=np.float64), 1, atol=1e-5)
+
+
+def test_softmax_golden_and_argmax(rt, oracle, golden):
+    for tag in "abcd":
+        got = rt.matrixSoftmax(rt.upload(golden[f"softmax_{tag}_x"])).numpy()
+        want = golden[f"softmax_{tag}_y"]
+        nz = want > 1e-30
+        assert strict_rel_err(got[nz], want[nz]) < TOL
+    x = golden["argmax_x"]
+    assert_bit_exact(rt.argMax(rt.upload(x), 3).numpy(), golden["argmax_top3"], "argMax ties")
+    z = np.round(np.random.default_rng(5).standard_normal((300, 10)) * 2).astype(np.float32)
+    for k in (1, 3, 8):
+        assert_bit_exact(rt.argMax(rt.upload(z), k).numpy(), oracle.argMax(z, k), f"argMax top{k}")
+
+
+def test_mnist8_known_answer(rt, golden):
+    """test/input of the reference: FCBias -> Tanh -> FCBias -> Softmax -> ArgMax = 5 0 4 1 9 2 1 3."""
+    d = os.path.join(HERE, "golden", "mnist8")
+    ld = lambda n, shape: np.fromfile(os.path.join(d, n), np.float32).reshape(shape)
+    img, w0, b0 = ld("mnist_images_8.bin", (8, 784)), ld("mlp_weight0.bin", (784, 512)), ld("mlp_bias0.bin", (512,))
+    w1, b1 = ld("mlp_weight1.bin", (512, 10)), ld("mlp_bias1.bin", (10,))
+    dimg, dw0, db0, dw1, db1 = up(rt, img, w0, b0, w1, b1)
+    h = rt.matrixTanh(rt.fcbias(dimg, dw0, db0))
+    prob = rt.matrixSoftmax(rt.fcbias(h, dw1, db1))
+    assert rt.argMax(prob, 1).numpy().ravel().tolist() == [5, 0, 4, 1, 9, 2, 1, 3]
+    assert_bit_exact(rt.argMax(prob, 3).numpy(), golden["mnist8_top3"], "top3")
+    assert strict_rel_err(prob.numpy(), golden["mnist8_prob"]) < TOL
+
+
+def test_error_paths(rt):
+    from swcompiler_amd.hip import SwcHipError
+    a = rt.upload(np.zeros((4, 4), np.float32))
+    with pytest.raises(SwcHipError):
+        rt._check(rt.lib.swc_hip_matrixMatrixMul_f(4, 4, 4, None, 4, a.ptr, 4, a.ptr, 4), "null a")
+    with pytest.raises(SwcHipError):
+        rt._check(rt.lib.swc_hip_matrixMatrixMul_f(4, 4, 4, a.ptr, 2, a.ptr, 4, a.ptr, 4), "lda < k")
+    with pytest.raises(SwcHipError):
+        rt._check(rt.lib.swc_hip_relu_f(None, a.ptr, 16), "null src")
+    assert rt.lib.swc_hip_relu_f(None, None, 0) == 0

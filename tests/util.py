@@ -44,3 +44,18 @@ def strict_rel_err(got, want):
     want = np.asarray(want, np.float64)
     den = np.where(want == 0, 1.0, np.abs(want))
     return float(np.max(np.abs(got - want) / den)) if want.size else 0.0
+
+
+def scaled_err(got, want, scale):
+    """max |g-w| / scale, element-wise, for contractions: `scale` is the sum of
+    the magnitudes of the accumulated terms, sum_k |a_ik||b_kj| (+|bias|).  Two
+    fp32 evaluations of one dot product in different orders differ by up to
+    ~k*eps of THAT quantity whatever the size of the (possibly cancelled)
+    result, so it is the denominator a relative tolerance on a contraction can
+    be held to; for sums without cancellation it equals the plain relative
+    error."""
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    scale = np.asarray(scale, np.float64)
+    scale = np.where(scale == 0, 1.0, scale)
+    return float(np.max(np.abs(got - want) / scale)) if want.size else 0.0
