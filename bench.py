@@ -179,6 +179,9 @@ def main():
     ap.add_argument("--headline-only", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=64)
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch relu_f on 2^26 floats three times: a plain 256 MiB-in/256 MiB-out pass whose "
+                         "FETCH_SIZE/WRITE_SIZE readings calibrate the counters for the traffic figures")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (nothing is sharded); use --gpus 1")
@@ -187,11 +190,24 @@ def main():
     from swcompiler_amd.hip import runtime
     rt = runtime()
 
+    if args.calibrate:
+        x = rt.upload(np.ones(1 << 26, np.float32))
+        y = rt.empty(x.shape)
+        for _ in range(3):
+            rt.relu(x, out=y)
+        rt.sync()
+        x.free()
+        y.free()
+
     head = run_config(rt, graphs, 2, args.steps, args.warmup)
     gemm = [r for r in head["kernels"] if r["op"] == "fcbias" and not r["shape"].endswith("x10")]
     flop = sum(r["flop"] for r in gemm)
     secs = sum(r["ms"] for r in gemm) * 1e-3
     achieved = flop / secs / 1e12
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):   # measured separately under rocprofv3 --pmc; see profiles/
+        traffic = json.load(open(tpath)).get("gemm_tiled<2,2,true>", {}).get("bytes_per_launch")
     out = {
         "metric": "samples/s per graph; TFLOP/s (FC/conv) & GB/s (eltwise) vs MI355X roofline",
         "value": head["samples_per_s"], "unit": "samples/s", "n_gpus": 1, "steps": args.steps,
@@ -201,7 +217,7 @@ def main():
                                "(BASELINE.json configs[1]), fused epilogues",
                    "global_batch": head["batch"], "device": rt.device_name()},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS_FP32_MFMA, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_TFLOPS_FP32_MFMA, "traffic": None,
+                     "frac": achieved / PEAK_TFLOPS_FP32_MFMA, "traffic": traffic,
                      "kernel": "gemm_tiled<2,2,true> (both launches per step: 4096x784x4096 and 4096x4096x4096)",
                      "flop_per_launch": flop / len(gemm), "avg_launch_ms": secs * 1e3 / len(gemm)},
         "gpu_ms_per_step": head["gpu_ms"] / args.steps,
