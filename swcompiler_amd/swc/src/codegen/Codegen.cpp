@@ -1,0 +1,410 @@
+// CPU code generator and the machinery shared with the HIP target.
+#include "Codegen.h"
+
+#include <cassert>
+#include <cstdlib>
+#include <fstream>
+#include <iomanip>
+
+#include "../graphIR/IRGraph.h"
+#include "../graphIR/OpNode.h"
+#include "../graphIR/TensorNode.h"
+#include "../op/ops.h"
+
+namespace swc {
+namespace codegen {
+
+using namespace swc::op;
+
+// ------------------------------------------------------------------ helpers
+uint64_t MemoryAllocator::allocate(Tensor *t, uint64_t bytes) {
+    const uint64_t start = (used_ + alignment_ - 1) / alignment_ * alignment_;
+    if (start + bytes > capacity_) {
+        SWLOG_ERROR << "arena " << base_ << " exhausted: need " << start + bytes << " of " << capacity_ << std::endl;
+        std::abort();
+    }
+    offsets_[t] = start;
+    used_ = start + bytes;
+    return start;
+}
+
+std::string MakefileBuilder::generate() const {
+    std::ostringstream os;
+    os << "all: " << target_ << "\n";
+    os << "CXX := " << cxx_ << "\n";
+    os << "CXXFLAGS :=";
+    for (auto &f : flags_) os << " " << f;
+    for (auto &d : incs_) os << " -I" << d;
+    os << "\nLDFLAGS :=";
+    for (auto &d : libDirs_) os << " -L" << d << " -Wl,-rpath," << d;
+    for (auto &l : libs_) os << " -l" << l;
+    os << "\n" << target_ << ":";
+    for (auto &s : srcs_) os << " " << s;
+    os << "\n\t$(CXX) $(CXXFLAGS) $^ $(LDFLAGS) -o $@\n";
+    os << "run: " << target_ << "\n\t" << runCmd_ << "\n";
+    os << "clean:\n\trm -f " << target_ << "\n";
+    return os.str();
+}
+
+static std::string deviceTag(const Device &d) {
+    return (d.type == DeviceType::GPU ? "gpu" : "cpu") + std::to_string(d.id);
+}
+
+// [d0, d1*d2*...]
+static std::pair<size_t, size_t> rowsCols(const std::vector<size_t> &dims) {
+    size_t cols = 1;
+    for (size_t i = 1; i < dims.size(); ++i) cols *= dims[i];
+    return {dims.empty() ? 0 : dims[0], cols};
+}
+
+std::string Codegen::arrayDef(const std::string &name, const std::vector<size_t> &v) {
+    std::ostringstream os;
+    os << "const size_t " << name << "[] = {";
+    for (size_t i = 0; i < v.size(); ++i) os << (i ? ", " : "") << v[i];
+    os << "};\n";
+    return os.str();
+}
+
+std::string Codegen::getTypeString(Tensor *t) const {
+    switch (t->getDataType()) {
+    case DataType::Double_t: return "double";
+    case DataType::Int8_t: return "char";
+    case DataType::Int32_t: return "int";
+    default: return "float";
+    }
+}
+
+static Tensor *T(IRNode *n) { return static_cast<TensorNode *>(n)->getTensor(); }
+
+std::string Codegen::nameOf(IRNode *tensorNode) { return tensors_name_map_.at(T(tensorNode)); }
+
+std::string Codegen::UniqueName(std::string name) {
+    for (char &c : name)
+        if (c == '/' || c == '.' || c == '-') c = '_';
+    auto it = names_map_.find(name);
+    if (it == names_map_.end()) {
+        names_map_[name] = 0;
+        return name;
+    }
+    std::string u;
+    do u = name + std::to_string(++it->second);
+    while (names_map_.count(u));
+    names_map_[u] = 0;
+    return u;
+}
+
+// ------------------------------------------------------------------- set-up
+Codegen::Codegen(IRGraph *graph) : graph_(graph) { config_ = graph->getConfig(); }
+Codegen::Codegen(IRGraph *graph, Config &config) : graph_(graph), config_(config) {}
+
+void Codegen::codeGenInit() {
+    mem_allocators_.clear();
+    dev_allocator_map_.clear();
+    tensors_name_map_.clear();
+    tensors_offset_map_.clear();
+    decl_order_.clear();
+    names_map_.clear();
+    headerWriter_.clear();
+    writer_.clear();
+    // one arena per device that can appear in a label
+    for (Device d : {Device(0, DeviceType::CPU, 0), Device(0, DeviceType::GPU, config_.hip_device)}) {
+        const uint64_t align = d.type == DeviceType::GPU ? devices::HipDevice().arenaAlignment : 64;
+        auto a = std::make_shared<MemoryAllocator>(d, deviceTag(d) + "_baseptr", UINT64_MAX, align);
+        mem_allocators_.push_back(a);
+        dev_allocator_map_[d] = a.get();
+    }
+    makefile_builder_ = MakefileBuilder();
+    swmakefile_builder_ = MakefileBuilder();
+    initMakefileBuilder();
+}
+
+void Codegen::initMakefileBuilder() {
+    // the reference's generated Makefile: g++ -std=c++11 -O2 (src/codegen/MakefileBuilder.h:34)
+    makefile_builder_.setCXXCompiler("/usr/bin/c++");
+    makefile_builder_.addCXXFlag("-std=c++11");
+    makefile_builder_.addCXXFlag("-O2");
+    makefile_builder_.addIncDir("/usr/local/include");
+    makefile_builder_.addCXXSrc("Graph.cpp");
+    swmakefile_builder_.setCXXCompiler("mpiCC");
+    swmakefile_builder_.addCXXFlag("-O2");
+}
+
+void Codegen::emitHeader() {
+    headerWriter_ << "// Graph.cpp -- generated from an IRGraph with " << graph_->tensorNodeNum() << " tensor nodes and "
+                  << graph_->opNodeNum() << " op nodes (CPU target)\n";
+    headerWriter_ << "#include <iostream>\n#include <random>\n#include <cstdlib>\n#include <cmath>\n"
+                  << "#include <sys/time.h>\n#include <sys/types.h>\n"
+                  << "#include \"utils/image.h\"\n#include \"utils/kernels.h\"\n";
+    if (config_.use_dataloader) headerWriter_ << "#include \"utils/DataLoader.h\"\n";
+}
+
+void Codegen::emitEnvInit() {
+    if (config_.cuda || config_.mkldnn || config_.mpi) {
+        SWLOG_ERROR << "the cuda / mkldnn / mpi targets are not part of this build; use Config::hip" << std::endl;
+        std::abort();
+    }
+}
+void Codegen::emitEnvFinalize() { writer_ << "return 0;\n"; }
+
+// ------------------------------------------------------------------ driver
+std::string Codegen::generate() {
+    codeGenInit();
+    emitHeader();
+    headerWriter_ << "using namespace std;\n";
+    writer_ << "#define TIME_MS(a,b)     (1000.0*((b).tv_sec-(a).tv_sec)+0.001*((b).tv_usec-(a).tv_usec))\n";
+    writer_ << "\nint main(int argc, char** argv) {\n";
+    writer_.indentInc();
+    writer_ << "struct timeval ts,te;\n(void)ts; (void)te; (void)argc; (void)argv;\n";
+    emitEnvInit();
+    writer_ << "\n// variable declaration and initiation\n";
+    emitMemAllocs();
+    writer_ << "\n// call op routine functions\n";
+    emitExecute();
+    emitOutputDump();
+    writer_ << "\n// free memory\n";
+    emitMemFree();
+    emitEnvFinalize();
+    writer_.indentDec();
+    writer_ << "}\n";
+
+    const std::string code = headerWriter_.get_code() + writer_.get_code();
+    std::ofstream("Graph.cpp") << code;
+    std::ofstream("G_Makefile") << makefile_builder_.generate();
+    swmakefile_builder_.addCXXSrc("Graph.cpp");
+    std::ofstream("SW_Makefile") << swmakefile_builder_.generate();
+    return code;
+}
+
+void Codegen::emitMemAllocs() {
+    allocateMemAddr();
+    emitVarDeclarations();
+    emitMemAllocations();
+    emitTensorAddresses();
+    emitTensorInitializations();
+}
+
+// Every distinct Tensor gets a name and an offset in the arena of its label's
+// device, in topological order.  The output of a Reshape shares its input's
+// storage.
+void Codegen::allocateMemAddr() {
+    for (int i = 0; i < graph_->topologyNum(); ++i)
+        for (int j = 0; j < graph_->getNumInTopoLevel(i); ++j) {
+            IRNode *node = graph_->getNodeInTopo(i, j);
+            if (node->nodeType() != TENSOR_NODE) continue;
+            auto *tn = static_cast<TensorNode *>(node);
+            Tensor *t = tn->getTensor();
+            if (tensors_name_map_.count(t)) continue;
+            const Device dev = tn->getLabel()->getDeviceLabel();
+            auto it = dev_allocator_map_.find(dev);
+            if (it == dev_allocator_map_.end()) {
+                SWLOG_ERROR << "no arena for the device of tensor " << tn->name() << std::endl;
+                std::abort();
+            }
+            MemoryAllocator *arena = it->second;
+            uint64_t off;
+            IRNode *producer = tn->parentNum() ? tn->getParentNode(0) : nullptr;
+            if (producer && static_cast<OpNode *>(producer)->getOp()->getOpName() == "Reshape" &&
+                tensors_offset_map_.count(T(producer->getParentNode(0))) &&
+                producer->getParentNode(0)->getLabel()->getDeviceLabel() == dev) {
+                off = tensors_offset_map_.at(T(producer->getParentNode(0))).second;
+                arena->alias(t, off);
+            } else {
+                off = arena->allocate(t, t->getSizeInBytes());
+            }
+            tensors_name_map_[t] = UniqueName(tn->name());
+            tensors_offset_map_[t] = {arena->getBasePtrName(), off};
+            decl_order_.push_back(tn);
+        }
+}
+
+void Codegen::emitVarDeclarations() {
+    for (auto &a : mem_allocators_)
+        if (a->getMemAllocated()) writer_ << "char *" << a->getBasePtrName() << ";\n";
+    for (TensorNode *tn : decl_order_)
+        writer_ << getTypeString(tn->getTensor()) << " *" << tensors_name_map_.at(tn->getTensor()) << ";\n";
+    writer_ << "\n";
+}
+
+void Codegen::emitMemAllocations() {
+    for (auto &a : mem_allocators_) {
+        if (!a->getMemAllocated()) continue;
+        if (a->getDevice().type != DeviceType::CPU) {
+            SWLOG_ERROR << "the CPU generator met a GPU-labelled tensor; use HipCodegen (Config::hip)" << std::endl;
+            std::abort();
+        }
+        writer_ << a->getBasePtrName() << " = (char*)malloc(" << a->getMemAllocated() << ");\n";
+    }
+    writer_ << "\n";
+}
+
+void Codegen::emitTensorAddresses() {
+    for (TensorNode *tn : decl_order_) {
+        Tensor *t = tn->getTensor();
+        const auto &where = tensors_offset_map_.at(t);
+        writer_ << tensors_name_map_.at(t) << " = reinterpret_cast<" << getTypeString(t) << "*>(" << where.first
+                << " + " << where.second << ");\n";
+    }
+    writer_ << "\n";
+}
+
+void Codegen::emitTensorInitializations() {
+    for (TensorNode *tn : decl_order_) {
+        Tensor *t = tn->getTensor();
+        const std::string name = tensors_name_map_.at(t);
+        const TensorInitInfo info = t->getTensorInitInfo();
+        switch (t->getTensorInitType()) {
+        case TensorInitType::XAVIER:
+            writer_ << "initTensorXavier(" << name << ", " << t->size() << ", " << info.getFilterSize() << ");\n";
+            break;
+        case TensorInitType::CONSTANT:
+            writer_ << "initTensorConstant(" << name << ", " << t->size() << ", " << info.getConstant() << ");\n";
+            break;
+        case TensorInitType::ZERO:
+            writer_ << "initTensorZero(" << name << ", " << t->size() << ");\n";
+            break;
+        case TensorInitType::FILE:
+            writer_ << "load(" << name << ", " << t->size() << ", " << info.getOffset() << ", \"" << info.getFilePath()
+                    << "\");\n";
+            break;
+        case TensorInitType::PARENTOP:
+            dispatchOpNode(static_cast<OpNode *>(tn->getParentNode(0)));
+            break;
+        default:
+            break;
+        }
+    }
+    writer_ << "\n";
+}
+
+void Codegen::emitExecute() {
+    if (config_.time_iters) {
+        writer_ << "gettimeofday(&ts, NULL);\n";
+        writer_ << "for (size_t swc_iter = 0; swc_iter < " << config_.time_iters << "; swc_iter++) {\n";
+        writer_.indentInc();
+    }
+    emitFuncCalls();
+    if (config_.time_iters) {
+        writer_.indentDec();
+        writer_ << "}\n";
+        writer_ << "gettimeofday(&te, NULL);\n";
+        writer_ << "std::cout << \"swc_time_ms_per_iter \" << TIME_MS(ts, te) / " << config_.time_iters
+                << " << std::endl;\n";
+    }
+}
+
+void Codegen::emitFuncCalls() {
+    for (int i = 0; i < graph_->topologyNum(); ++i)
+        for (int j = 0; j < graph_->getNumInTopoLevel(i); ++j) {
+            IRNode *node = graph_->getNodeInTopo(i, j);
+            if (node->nodeType() != OP_NODE) continue;
+            auto *op = static_cast<OpNode *>(node);
+            if (op->isRunOnce()) continue;   // emitted with the initialisations
+            writer_ << "// topology(" << i << ", " << j << "): " << op->name() << " : " << op->getOp()->getOpName()
+                    << "\n";
+            dispatchOpNode(op);
+        }
+}
+
+void Codegen::dispatchOpNode(OpNode *op) {
+    if (!op->runable()) return;
+    if (op->getLabel()->getDeviceLabel().type != DeviceType::CPU) {
+        SWLOG_ERROR << "op " << op->name() << " is labelled for a GPU; the CPU generator cannot emit it" << std::endl;
+        std::abort();
+    }
+    emitFuncCall(op);
+}
+
+void Codegen::emitMemFree() {
+    for (auto &a : mem_allocators_)
+        if (a->getMemAllocated() && a->getDevice().type == DeviceType::CPU)
+            writer_ << "free(" << a->getBasePtrName() << ");\n";
+}
+
+// Writes every output-marked tensor that lives on the host to "<name>.bin".
+void Codegen::emitOutputDump() {
+    if (!config_.dump_outputs) return;
+    writer_ << "\n// dump graph outputs\n";
+    for (TensorNode *tn : decl_order_) {
+        if (!tn->getLabel()->getIsOut() || tn->getLabel()->getDeviceLabel().type != DeviceType::CPU) continue;
+        Tensor *t = tn->getTensor();
+        writer_ << "store(" << tensors_name_map_.at(t) << ", " << t->size() << ", \"" << tensors_name_map_.at(t)
+                << ".bin\");\n";
+    }
+}
+
+// ------------------------------------------------------------ CPU emitters
+// One call per op node: the kernel name and argument order of the reference's
+// generator for the same op type (file:line of the reference given per case).
+void Codegen::emitFuncCall(OpNode *op) {
+    const std::string type = op->getOp()->getOpName();
+    const std::string nm = op->name();
+    auto in = [&](int i) { return op->getParentNode(i); };
+    auto out = [&](int i) { return op->getChildNode(i); };
+
+    if (type == "MatrixMatrixMul") {   // Codegen.cpp:1334-1337
+        const size_t m = T(in(0))->getDim(0), k = T(in(1))->getDim(0), n = T(in(1))->getDim(1);
+        writer_ << "matrixMatrixMul_f(" << m << ", " << n << ", " << k << ", " << nameOf(in(0)) << ", " << k << ", "
+                << nameOf(in(1)) << ", " << n << ", " << nameOf(out(0)) << ", " << n << ");\n";
+    } else if (type == "MatrixVectorAdd" || type == "BatchedAdd") {   // Codegen.cpp:1513-1515
+        auto rc = rowsCols(T(in(0))->getDims());
+        assert(rc.second == T(in(1))->size() && "bias length != row length");
+        writer_ << "batchedadd_f(" << nameOf(out(0)) << ", " << nameOf(in(0)) << ", " << nameOf(in(1)) << ", "
+                << rc.first << ", " << rc.second << ");\n";
+    } else if (type == "Reshape" || type == "Dropout") {   // Codegen.cpp:1480-1485 (pointer alias)
+        writer_ << nameOf(out(0)) << " = " << nameOf(in(0)) << ";\n";
+    } else if (type == "MatrixTanh") {   // Codegen.cpp:2293-2295
+        const size_t m = T(in(0))->getDim(0), n = T(in(0))->getDim(1);
+        writer_ << "matrixTanh_f(" << m << ", " << n << ", " << nameOf(in(0)) << ", " << n << ", " << nameOf(out(0))
+                << ", " << n << ");\n";
+    } else if (type == "MatrixSoftmax") {   // Codegen.cpp:2352-2354
+        const size_t m = T(in(0))->getDim(0), n = T(in(0))->getDim(1);
+        writer_ << "matrixSoftmax_f(" << m << ", " << n << ", " << nameOf(in(0)) << ", " << n << ", "
+                << nameOf(out(0)) << ", " << n << ");\n";
+    } else if (type == "ElementAdd") {   // Codegen.cpp:1608-1610
+        writer_ << "vecAdd_f(" << T(in(0))->size() << ", " << nameOf(in(0)) << ", " << nameOf(in(1)) << ", "
+                << nameOf(out(0)) << ");\n";
+    } else if (type == "Relu") {   // Codegen.cpp:2134-2135
+        writer_ << "relu_f(" << nameOf(in(0)) << ", " << nameOf(out(0)) << ", " << T(in(0))->size() << ");\n";
+    } else if (type == "Conv2d") {   // Codegen.cpp:1761-1782
+        auto *conv = static_cast<Conv2dOp *>(op->getOp());
+        writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims()) << arrayDef(nm + "_outDims", T(out(0))->getDims())
+                << arrayDef(nm + "_filterDims", T(in(1))->getDims()) << arrayDef(nm + "_biasDims", T(in(2))->getDims())
+                << arrayDef(nm + "_filterSizes", conv->getKernels()) << arrayDef(nm + "_strides", conv->getStrides())
+                << arrayDef(nm + "_pads", conv->getPads());
+        writer_ << "conv2d_f(" << nameOf(out(0)) << ", " << nameOf(in(0)) << ", " << nameOf(in(1)) << ", "
+                << nameOf(in(2)) << ", " << nm << "_outDims, " << nm << "_inDims, " << nm << "_filterDims, " << nm
+                << "_biasDims, " << nm << "_filterSizes, " << nm << "_strides, " << nm << "_pads, "
+                << conv->getGroup() << ");\n";
+    } else if (type == "BatchNormalization") {   // Codegen.cpp:1832-1837,1907-1915: parents in, scale, bias, mean, var
+        const float eps = static_cast<BatchNormalizationOp *>(op->getOp())->getEpsilon();
+        writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims());
+        writer_ << "batchnormalization_f(" << nameOf(out(0)) << ", " << nameOf(in(0)) << ", " << nameOf(in(3)) << ", "
+                << nameOf(in(4)) << ", " << nameOf(in(1)) << ", " << nameOf(in(2)) << ", " << nm << "_inDims, "
+                << std::setprecision(12) << eps << ");\n";
+    } else if (type == "MaxPool") {   // Codegen.cpp:2020-2037
+        auto *pool = static_cast<MaxPoolOp *>(op->getOp());
+        writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims()) << arrayDef(nm + "_outDims", T(out(0))->getDims())
+                << arrayDef(nm + "_filterSizes", pool->getKernels()) << arrayDef(nm + "_strides", pool->getStrides())
+                << arrayDef(nm + "_pads", pool->getPads());
+        writer_ << "maxpool_f(" << nameOf(in(0)) << ", " << nameOf(out(0)) << ", " << nm << "_inDims, " << nm
+                << "_outDims, " << nm << "_filterSizes, " << nm << "_strides, " << nm << "_pads);\n";
+    } else if (type == "ArgMax") {   // Codegen.cpp:2372-2385
+        const int topK = static_cast<ArgMaxOp *>(op->getOp())->getTopK();
+        writer_ << "argMax_i(" << nameOf(in(0)) << ", " << nameOf(out(0)) << ", " << T(in(0))->getDim(0) << ", "
+                << T(in(0))->getDim(1) << ", " << topK << ");\n";
+    } else if (type == "Accuracy") {   // Codegen.cpp:2387-2398
+        writer_ << "accuracy_i(" << nameOf(in(0)) << ", " << nameOf(in(1)) << ", " << nameOf(out(0)) << ", "
+                << T(in(0))->getDim(0) << ", " << T(in(0))->getDim(1) << ");\n";
+    } else if (type == "Debug") {   // Codegen.cpp:2401-2412
+        Tensor *a = T(in(0));
+        writer_ << "printMatrix(" << nameOf(in(0)) << ", " << a->getDim(0) << ", "
+                << (a->getNDim() == 2 ? a->getDim(1) : 1) << ");\n";
+        if (op->childNum()) writer_ << nameOf(out(0)) << " = " << nameOf(in(0)) << ";\n";
+    } else {
+        SWLOG_ERROR << "no CPU emitter for op type " << type << " (node " << nm << ")" << std::endl;
+        std::abort();
+    }
+}
+
+} // namespace codegen
+} // namespace swc

@@ -1,0 +1,62 @@
+#include "Engine.h"
+
+#include <cstdlib>
+
+#include "../codegen/Codegen.h"
+#include "../graphIR/IRGraph.h"
+#include "../graphIR/OpNode.h"
+#include "../graphIR/TensorNode.h"
+#include "../pass/passes.h"
+
+namespace swc {
+
+using namespace pass;
+
+void Engine::compile() {
+    const Config cfg = graph_->getConfig();
+    if (cfg.train_mode || cfg.mpi || cfg.mkldnn || cfg.cuda) {
+        SWLOG_ERROR << "Engine: only the inference pipeline (CPU or Config::hip) is part of this build" << std::endl;
+        std::abort();
+    }
+    runInferPasses();
+    if (cfg.hip) transformForHIP();
+}
+
+// labeling -> lowering -> labeling (new nodes) -> renaming, then refresh the
+// derived views and mark the outputs (reference order: src/engine/Engine.cpp:61-86)
+void Engine::runInferPasses() {
+    LabelingPass labeling(graph_);
+    LoweringPass lowering(graph_);
+    RenamingNodePass renaming(graph_);
+    PassManager pm;
+    pm.add(&labeling);
+    pm.add(&lowering);
+    pm.add(&labeling);
+    pm.add(&renaming);
+    pm.run();
+    graph_->findInOut();
+    graph_->updateTopology();
+    graph_->setOutMark();
+}
+
+void Engine::transformForHIP() {
+    const Config cfg = graph_->getConfig();
+    if (cfg.hip_fusion) {
+        HipFusionPass fusion(graph_);
+        fusion.run();
+    }
+    DeviceMemoryLoweringPass placement(graph_, cfg.hip_device);
+    placement.run();
+    LabelingPass labeling(graph_);
+    labeling.run();
+    graph_->findInOut();
+    graph_->updateTopology();
+}
+
+std::string Engine::genCode() {
+    Config cfg = graph_->getConfig();
+    if (!generator_) generator_ = cfg.hip ? new codegen::HipCodegen(graph_, cfg) : new codegen::Codegen(graph_, cfg);
+    return generator_->generate();
+}
+
+} // namespace swc

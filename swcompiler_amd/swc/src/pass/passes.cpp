@@ -1,0 +1,313 @@
+#include "passes.h"
+
+#include <cassert>
+#include <set>
+#include <unordered_set>
+
+#include "../graphIR/OpNode.h"
+#include "../graphIR/TensorNode.h"
+#include "../op/ops.h"
+
+namespace swc {
+namespace pass {
+
+using namespace swc::op;
+
+void Optimizer::runOptimizer() {
+    PassManager pm;
+    LabelingPass labeling(_graph);
+    LoweringPass lowering(_graph);
+    pm.add(&labeling);
+    pm.add(&lowering);
+    pm.add(&labeling);
+    pm.run();
+}
+
+// ------------------------------------------------------------------ labeling
+void LabelingPass::run() {
+    const Config cfg = _graph->getConfig();
+    for (int i = 0; i < _graph->tensorNodeNum(); ++i) {
+        TensorNode *t = _graph->getTensorNode(i);
+        Label *l = t->getLabel();
+        l->setNodeNameLabel(t->name());
+        l->setTypeNameLabel("Tensor");
+        if (t->getTensor()) {
+            l->setTraining(t->getTraining());
+            l->setTensorInitTypeLabel(t->getTensor()->getTensorInitType());
+        }
+    }
+    for (int i = 0; i < _graph->opNodeNum(); ++i) {
+        OpNode *o = _graph->getOpNode(i);
+        Label *l = o->getLabel();
+        l->setNodeNameLabel(o->name());
+        const std::string type = o->getOp()->getOpName();
+        l->setTypeNameLabel(type);
+        if (!cfg.enable_lowering) continue;
+        // FC without bias always becomes a plain GEMM.  FC with bias is split
+        // into GEMM + bias-add only for targets without a fused kernel: the CPU
+        // generator; MKL-DNN and the HIP target keep it whole.
+        if (type == "MatrixMatrixFC") l->setLowerMark();
+        else if (type == "MatrixMatrixFCBias" && !cfg.mkldnn && !cfg.hip) l->setLowerMark();
+    }
+}
+
+// ------------------------------------------------------------------ lowering
+void LoweringPass::run() {
+    // lowering edits the op list, so collect first
+    std::vector<OpNode *> marked;
+    for (int i = 0; i < _graph->opNodeNum(); ++i)
+        if (_graph->getOpNode(i)->getLabel()->getLowerMark()) marked.push_back(_graph->getOpNode(i));
+    for (OpNode *o : marked) {
+        o->getLabel()->clearLowerMark();
+        o->getOp()->lowering(_graph, o);
+    }
+}
+
+// ------------------------------------------------------------------ renaming
+std::string UniqueName::operator()(const std::string &in) {
+    assert(!in.empty());
+    std::string base = in;
+    for (char &c : base)
+        if (c == '/' || c == '.' || c == '-') c = '_';
+    std::string name = base;
+    auto it = seen_.find(base);
+    if (it != seen_.end())
+        do name = base + std::to_string(++it->second);
+        while (seen_.count(name));
+    seen_[name] = 0;
+    return name;
+}
+
+void RenamingNodePass::run() {
+    for (int i = 0; i < _graph->tensorNodeNum(); ++i) {
+        TensorNode *t = _graph->getTensorNode(i);
+        t->setName(unique_(t->name()));
+    }
+    for (int i = 0; i < _graph->opNodeNum(); ++i) {
+        OpNode *o = _graph->getOpNode(i);
+        o->setName(unique_(o->name()));
+    }
+}
+
+// --------------------------------------------------------------- elimination
+void EliminationPass::run() {
+    // live = everything from which an output-marked node is reachable
+    std::unordered_set<IRNode *> live;
+    std::vector<IRNode *> work;
+    auto seed = [&](IRNode *n) {
+        if (n->getLabel()->getIsOut() && live.insert(n).second) work.push_back(n);
+    };
+    for (int i = 0; i < _graph->tensorNodeNum(); ++i) seed(_graph->getTensorNode(i));
+    for (int i = 0; i < _graph->opNodeNum(); ++i) seed(_graph->getOpNode(i));
+    while (!work.empty()) {
+        IRNode *n = work.back();
+        work.pop_back();
+        for (IRNode *p : n->getParentNodes())
+            if (live.insert(p).second) work.push_back(p);
+    }
+    std::vector<TensorNode *> deadT;
+    std::vector<OpNode *> deadO;
+    for (int i = 0; i < _graph->tensorNodeNum(); ++i)
+        if (!live.count(_graph->getTensorNode(i))) deadT.push_back(_graph->getTensorNode(i));
+    for (int i = 0; i < _graph->opNodeNum(); ++i)
+        if (!live.count(_graph->getOpNode(i))) deadO.push_back(_graph->getOpNode(i));
+    auto detach = [](IRNode *n) {
+        while (n->parentNum()) n->destroyUpperNode(n->getParentNode(0));
+        while (n->childNum()) n->getChildNode(0)->destroyUpperNode(n);
+    };
+    for (auto *t : deadT) {
+        detach(t);
+        _graph->delTensorNode(t);
+    }
+    for (auto *o : deadO) {
+        detach(o);
+        _graph->delOpNode(o);
+    }
+    _graph->findInOut();
+    _graph->updateTopology();
+}
+
+// -------------------------------------------------------------------- fusion
+namespace {
+
+bool isType(IRNode *n, const char *type) {
+    return n->nodeType() == OP_NODE && static_cast<OpNode *>(n)->getOp()->getOpName() == type;
+}
+
+// the op consuming `producer`'s only output, if that output has exactly one
+// consumer, is not a graph output and the consumer has the wanted type
+OpNode *soleConsumer(OpNode *producer, const char *type, IRGraph *g) {
+    if (producer->childNum() != 1) return nullptr;
+    IRNode *t = producer->getChildNode(0);
+    if (t->childNum() != 1 || t->getLabel()->getIsOut()) return nullptr;
+    for (IRNode *lo : g->getLogicalOutNodes())
+        if (lo == t) return nullptr;
+    IRNode *c = t->getChildNode(0);
+    if (!isType(c, type) || c->getParentNode(0) != t) return nullptr;
+    return static_cast<OpNode *>(c);
+}
+
+// Replaces producer -> mid -> consumer -> out by fusedNode -> out, where
+// fusedNode takes producer's operands followed by consumer's operands 1.. .
+void splice(IRGraph *g, OpNode *producer, OpNode *consumer, Op *fusedOp) {
+    auto *mid = static_cast<TensorNode *>(producer->getChildNode(0));
+    auto *out = static_cast<TensorNode *>(consumer->getChildNode(0));
+    auto *fused = new OpNode(producer->name(), fusedOp);
+    *fused->getLabel() = *producer->getLabel();
+    fused->getLabel()->setTypeNameLabel(fusedOp->getOpName());
+    std::vector<IRNode *> operands(producer->getParentNodes());
+    for (int i = 1; i < consumer->parentNum(); ++i) operands.push_back(consumer->getParentNode(i));
+    while (producer->parentNum()) producer->destroyUpperNode(producer->getParentNode(0));
+    mid->destroyUpperNode(producer);
+    while (consumer->parentNum()) consumer->destroyUpperNode(consumer->getParentNode(0));
+    out->destroyUpperNode(consumer);
+    for (IRNode *p : operands) fused->exlinkUpperNode(p);
+    out->exlinkUpperNode(fused);
+    g->delOpNode(producer);
+    g->delOpNode(consumer);
+    g->delTensorNode(mid);
+    g->pushOpNode(fused);
+}
+
+} // namespace
+
+void HipFusionPass::run() {
+    bool changed = true;
+    while (changed) {
+        changed = false;
+        for (int i = 0; i < _graph->opNodeNum() && !changed; ++i) {
+            OpNode *o = _graph->getOpNode(i);
+            const std::string type = o->getOp()->getOpName();
+            if (type == "MatrixMatrixFCBias") {
+                if (OpNode *r = soleConsumer(o, "Relu", _graph)) {
+                    splice(_graph, o, r, new MatrixMatrixFCBiasReluOp());
+                    changed = true;
+                }
+            } else if (type == "Conv2d") {
+                auto *conv = static_cast<Conv2dOp *>(o->getOp());
+                auto k = conv->getKernels(), s = conv->getStrides(), p = conv->getPads();
+                if (conv->getGroup() != 1) continue;
+                if (OpNode *bn = soleConsumer(o, "BatchNormalization", _graph)) {
+                    const float eps = static_cast<BatchNormalizationOp *>(bn->getOp())->getEpsilon();
+                    splice(_graph, o, bn, new Conv2dBatchNormOp(k, s, p, eps, false));
+                    changed = true;
+                } else if (OpNode *r = soleConsumer(o, "Relu", _graph)) {
+                    splice(_graph, o, r, new Conv2dWithActivationOp(k, s, p, SWC_ACTIVATION_RELU));
+                    changed = true;
+                }
+            } else if (type == "Conv2dBatchNorm") {
+                auto *cb = static_cast<Conv2dBatchNormOp *>(o->getOp());
+                if (cb->hasRelu()) continue;
+                if (OpNode *r = soleConsumer(o, "Relu", _graph)) {
+                    auto k = cb->getKernels(), s = cb->getStrides(), p = cb->getPads();
+                    splice(_graph, o, r, new Conv2dBatchNormOp(k, s, p, cb->getEpsilon(), true));
+                    changed = true;
+                }
+            } else if (type == "BatchNormalization") {
+                if (OpNode *r = soleConsumer(o, "Relu", _graph)) {
+                    const float eps = static_cast<BatchNormalizationOp *>(o->getOp())->getEpsilon();
+                    splice(_graph, o, r, new BatchNormalizationReluOp(eps));
+                    changed = true;
+                }
+            } else if (type == "ElementAdd") {
+                if (OpNode *r = soleConsumer(o, "Relu", _graph)) {
+                    splice(_graph, o, r, new ElementAddReluOp());
+                    changed = true;
+                }
+            }
+            if (changed) ++fused_;
+        }
+    }
+    _graph->findInOut();
+    _graph->updateTopology();
+}
+
+// ---------------------------------------------------------- device placement
+bool DeviceMemoryLoweringPass::runsOnGpu(const std::string &t) {
+    static const std::set<std::string> gpu = {
+        "MatrixMatrixMul", "MatrixVectorAdd", "BatchedAdd", "MatrixMatrixFCBias", "MatrixMatrixFCBiasRelu",
+        "Reshape", "MatrixTanh", "MatrixSoftmax", "ElementAdd", "ElementAddRelu", "Relu", "Dropout",
+        "Conv2d", "Conv2dWithActivation", "Conv2dBatchNorm", "MaxPool", "BatchNormalization",
+        "BatchNormalizationRelu", "ArgMax"};
+    return gpu.count(t) != 0;
+}
+
+void DeviceMemoryLoweringPass::run() {
+    const Device gpu(0, DeviceType::GPU, device_);
+    const Config cfg = _graph->getConfig();
+
+    std::vector<OpNode *> ops;
+    for (int i = 0; i < _graph->opNodeNum(); ++i) ops.push_back(_graph->getOpNode(i));
+
+    // 1. label compute ops and what they produce
+    for (OpNode *o : ops) {
+        if (!runsOnGpu(o->getOp()->getOpName())) continue;
+        o->getLabel()->setDeviceLabel(gpu);
+        for (IRNode *c : o->getChildNodes()) c->getLabel()->setDeviceLabel(gpu);
+    }
+    auto onGpu = [&](IRNode *n) { return n->getLabel()->getDeviceLabel() == gpu; };
+
+    std::vector<TensorNode *> tensors;
+    for (int i = 0; i < _graph->tensorNodeNum(); ++i) tensors.push_back(_graph->getTensorNode(i));
+
+    for (TensorNode *t : tensors) {
+        if (!onGpu(t)) {
+            // 2. host tensor read by GPU ops: device twin + Scatter
+            std::vector<IRNode *> gpuReaders;
+            for (IRNode *c : t->getChildNodes())
+                if (onGpu(c) && std::find(gpuReaders.begin(), gpuReaders.end(), c) == gpuReaders.end())
+                    gpuReaders.push_back(c);
+            if (gpuReaders.empty()) continue;
+            auto *twin = new TensorNode(t->name() + "_dev", t->getTensor()->clone());
+            twin->getTensor()->setTensorInit(TensorInitType::NONE);
+            twin->getLabel()->setDeviceLabel(gpu);
+            auto *scatter = new OpNode(t->name() + "_h2d", new ScatterOp());
+            scatter->getLabel()->setDeviceLabel(gpu);
+            scatter->getLabel()->setTypeNameLabel("Scatter");
+            const bool perIteration = cfg.use_dataloader &&
+                                      (t == _graph->getInferDataNode() || t == _graph->getInferLabelNode());
+            const bool parameter = t->parentNum() == 0 && !perIteration;
+            if (parameter) {
+                scatter->setRunOnce();
+                twin->getTensor()->setTensorInit(TensorInitType::PARENTOP);
+            }
+            for (IRNode *reader : gpuReaders) t->replaceUseKeepOrder(reader, twin);
+            scatter->exlinkUpperNode(t);
+            twin->exlinkUpperNode(scatter);
+            _graph->pushOpNode(scatter);
+            _graph->pushTensorNode(twin);
+            ++scatters_;
+        } else {
+            // 3. GPU tensor that leaves the device: host twin + Gather
+            std::vector<IRNode *> hostReaders;
+            for (IRNode *c : t->getChildNodes())
+                if (!onGpu(c) && std::find(hostReaders.begin(), hostReaders.end(), c) == hostReaders.end())
+                    hostReaders.push_back(c);
+            bool isOutput = t->getLabel()->getIsOut() != 0 || t->childNum() == 0;
+            for (IRNode *lo : _graph->getLogicalOutNodes())
+                if (lo == t) isOutput = true;
+            if (hostReaders.empty() && !isOutput) continue;
+            auto *twin = new TensorNode(t->name() + "_host", t->getTensor()->clone());
+            twin->getTensor()->setTensorInit(TensorInitType::NONE);
+            twin->getLabel()->setDeviceLabel(Device());
+            auto *gather = new OpNode(t->name() + "_d2h", new GatherOp());
+            gather->getLabel()->setDeviceLabel(gpu);
+            gather->getLabel()->setTypeNameLabel("Gather");
+            for (IRNode *reader : hostReaders) t->replaceUseKeepOrder(reader, twin);
+            gather->exlinkUpperNode(t);
+            twin->exlinkUpperNode(gather);
+            if (isOutput) {
+                twin->getLabel()->setIsOut(1);
+                t->getLabel()->setIsOut(0);
+            }
+            _graph->pushOpNode(gather);
+            _graph->pushTensorNode(twin);
+            ++gathers_;
+        }
+    }
+    _graph->findInOut();
+    _graph->updateTopology();
+}
+
+} // namespace pass
+} // namespace swc

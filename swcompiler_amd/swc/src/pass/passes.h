@@ -1,0 +1,100 @@
+// The graph passes of the inference pipeline.
+//
+//   LabelingPass             type-name labels + lowering marks       (reference: src/pass/LabelingPass.h:34-125)
+//   LoweringPass             Op::lowering on marked nodes            (src/pass/LoweringPass.h:34-59)
+//   RenamingNodePass         C-identifier-safe unique node names     (src/pass/RenamingNodePass.h:23-83)
+//   EliminationPass          dead-node removal from the output marks (src/pass/EliminationPass.cpp:34-154)
+//   HipFusionPass            NEW: chains -> one fused libswc_hip call
+//   DeviceMemoryLoweringPass NEW: places compute on GPU 0, inserts host<->device transfer nodes
+#ifndef SWC_PASSES_H_
+#define SWC_PASSES_H_
+#include <string>
+#include <unordered_map>
+
+#include "OptimizePass.h"
+
+namespace swc {
+class OpNode;
+class TensorNode;
+namespace pass {
+
+class LabelingPass : public OptimizePass {
+  public:
+    explicit LabelingPass(IRGraph *graph) : OptimizePass(graph) {}
+    void run() override;
+};
+
+class LoweringPass : public OptimizePass {
+  public:
+    explicit LoweringPass(IRGraph *graph) : OptimizePass(graph) {}
+    void run() override;
+};
+
+// '/', '.', '-' become '_'; a repeated name gets the smallest unused numeric suffix.
+class UniqueName {
+    std::unordered_map<std::string, int> seen_;
+
+  public:
+    std::string operator()(const std::string &name);
+    void clear() { seen_.clear(); }
+};
+
+class RenamingNodePass : public OptimizePass {
+    UniqueName unique_;
+
+  public:
+    explicit RenamingNodePass(IRGraph *graph) : OptimizePass(graph) {}
+    void setGraph(IRGraph *graph) {
+        _graph = graph;
+        unique_.clear();
+    }
+    void run() override;
+};
+
+class EliminationPass : public OptimizePass {
+  public:
+    explicit EliminationPass(IRGraph *graph) : OptimizePass(graph) {}
+    void run() override;
+};
+
+// Rewrites, wherever the intermediate tensor has a single consumer and is not a
+// graph output:
+//   MatrixMatrixFCBias -> Relu                    => MatrixMatrixFCBiasRelu
+//   Conv2d -> BatchNormalization [-> Relu]        => Conv2dBatchNorm(relu)
+//   Conv2d -> Relu                                => Conv2dWithActivation(RELU)
+//   BatchNormalization -> Relu                    => BatchNormalizationRelu
+//   ElementAdd -> Relu                            => ElementAddRelu
+// Each right-hand side is one kernel launch of libswc_hip whose result equals
+// the left-hand sequence of reference kernels.
+class HipFusionPass : public OptimizePass {
+    int fused_{0};
+
+  public:
+    explicit HipFusionPass(IRGraph *graph) : OptimizePass(graph) {}
+    void run() override;
+    int fusedCount() const { return fused_; }
+};
+
+// Device placement for the single-GPU HIP target.  Every op libswc_hip
+// implements is labelled Device{0, GPU, id} together with its outputs; every
+// host tensor read by a GPU op gets a device twin fed by a ScatterOp (run-once
+// when the tensor is a parameter, i.e. has an initialiser and is not the
+// per-iteration data/label input); every GPU tensor that is a graph output or
+// is read by a host op (Debug, Accuracy) gets a host twin fed by a GatherOp.
+// After the pass the graph itself says where each buffer lives and where each
+// transfer happens; the code generator only walks it.
+class DeviceMemoryLoweringPass : public OptimizePass {
+    int device_;
+    int scatters_{0}, gathers_{0};
+
+  public:
+    DeviceMemoryLoweringPass(IRGraph *graph, int device = 0) : OptimizePass(graph), device_(device) {}
+    void run() override;
+    static bool runsOnGpu(const std::string &typeName);
+    int scatterCount() const { return scatters_; }
+    int gatherCount() const { return gathers_; }
+};
+
+} // namespace pass
+} // namespace swc
+#endif

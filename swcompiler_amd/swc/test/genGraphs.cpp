@@ -1,0 +1,243 @@
+// Builds one of the benchmark graphs through the SWC API, compiles it for the
+// CPU or the HIP target and writes Graph.cpp + G_Makefile into the current
+// directory.  User-level code: only `SWC.h` and the DSL macros, in the style of
+// the reference's test/engine/testEngineMLPInfer.cpp.
+//
+//   genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse]
+//   model: mnist8 | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
+//
+// Every parameter/input tensor is initialised from "<name>.bin" in the
+// directory the generated program runs in; outputs are dumped to "<name>.bin".
+#include <cstdlib>
+#include <iostream>
+#include <string>
+
+#include "SWC.h"
+
+using namespace swc;
+using namespace swc::op;
+using namespace std;
+
+static void fromFile(Tensor *t, const string &name) { t->setTensorInit(TensorInitType::FILE, name + ".bin"); }
+
+// x -> FCBias(w,b) [-> Relu] -> returns the output tensor node
+static TensorNode *fc(IRGraph *g, const string &name, TensorNode *x, size_t k, size_t n, bool relu) {
+    auto *w = new TensorNode(name + "_w", new Tensor({k, n}));
+    auto *b = new TensorNode(name + "_b", new Tensor({n}));
+    fromFile(w->getTensor(), name + "_w");
+    fromFile(b->getTensor(), name + "_b");
+    auto *op = new OpNode(name, new MatrixMatrixFCBiasOp());
+    op->exlinkUpperNode(x, w, b);
+    auto *y = new TensorNode(name + "_out", new Tensor({x->getDims()[0], n}), op);
+    g->pushTensorNode(w, b, y);
+    g->pushOpNode(op);
+    if (!relu) return y;
+    auto *r = new OpNode(name + "_relu", new ReluOp());
+    r->exlinkUpperNode(y);
+    auto *z = new TensorNode(name + "_act", new Tensor({x->getDims()[0], n}), r);
+    g->pushTensorNode(z);
+    g->pushOpNode(r);
+    return z;
+}
+
+static TensorNode *unary(IRGraph *g, const string &name, Op *op, TensorNode *x) {
+    auto *o = new OpNode(name, op);
+    o->exlinkUpperNode(x);
+    auto *y = new TensorNode(name + "_out", new Tensor(new TensorShape(x->getDims())), o);
+    g->pushOpNode(o);
+    g->pushTensorNode(y);
+    return y;
+}
+
+static TensorNode *conv(IRGraph *g, const string &name, TensorNode *x, size_t oc, size_t k, size_t pad) {
+    const size_t ic = x->getDims()[3];
+    auto *f = new TensorNode(name + "_f", new Tensor({oc, k, k, ic}));
+    auto *b = new TensorNode(name + "_b", new Tensor({oc}));
+    fromFile(f->getTensor(), name + "_f");
+    fromFile(b->getTensor(), name + "_b");
+    vector<size_t> kernels{k, k}, strides{1, 1}, pads{pad, pad, pad, pad};
+    DYOP(c, Conv2dOp, kernels, strides, pads);
+    c->setName(name);
+    LINKUPPER(c, x, f, b);
+    auto *y = new TensorNode(name + "_out", new Tensor({0}), c);   // shape filled in by initTensorNodes()
+    g->pushTensorNode(f, b, y);
+    g->pushOpNode(c);
+    return y;
+}
+
+static TensorNode *bn(IRGraph *g, const string &name, TensorNode *x) {
+    const size_t c = x->getDims().size() == 4 && x->getDims()[3] ? x->getDims()[3] : 0;
+    TensorNode *p[4];
+    const char *suffix[4] = {"_scale", "_bias", "_mean", "_var"};
+    for (int i = 0; i < 4; ++i) {
+        p[i] = new TensorNode(name + suffix[i], new Tensor({c}));
+        fromFile(p[i]->getTensor(), name + suffix[i]);
+        g->pushTensorNode(p[i]);
+    }
+    auto *o = new OpNode(name, new BatchNormalizationOp(1e-5f));
+    o->exlinkUpperNode(x, p[0], p[1], p[2], p[3]);
+    auto *y = new TensorNode(name + "_out", new Tensor({0}), o);
+    g->pushOpNode(o);
+    g->pushTensorNode(y);
+    return y;
+}
+
+static TensorNode *pool(IRGraph *g, const string &name, TensorNode *x) {
+    vector<size_t> kernels{2, 2}, strides{2, 2}, pads{0, 0, 0, 0};
+    auto *o = new OpNode(name, new MaxPoolOp(kernels, strides, pads));
+    o->exlinkUpperNode(x);
+    auto *y = new TensorNode(name + "_out", new Tensor({0}), o);
+    g->pushOpNode(o);
+    g->pushTensorNode(y);
+    return y;
+}
+
+static TensorNode *lazyUnary(IRGraph *g, const string &name, Op *op, TensorNode *x) {
+    auto *o = new OpNode(name, op);
+    o->exlinkUpperNode(x);
+    auto *y = new TensorNode(name + "_out", new Tensor({0}), o);
+    g->pushOpNode(o);
+    g->pushTensorNode(y);
+    return y;
+}
+
+int main(int argc, char **argv) {
+    if (argc < 3) {
+        cerr << "usage: genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse]\n";
+        return 2;
+    }
+    const string model = argv[1], target = argv[2];
+    const size_t batch = argc > 3 ? strtoul(argv[3], nullptr, 10) : 0;
+    const size_t iters = argc > 4 ? strtoul(argv[4], nullptr, 10) : 0;
+    const bool nofuse = argc > 5 && string(argv[5]) == "nofuse";
+
+    G(graph);
+    TensorNode *out = nullptr;
+
+    if (model == "mnist8") {
+        // the reference's MNIST example: FCBias -> Tanh -> FCBias -> Softmax -> ArgMax(3) -> print
+        TENSOR(data0, 8, 784);
+        TENSOR(weight0, 784, 512);
+        TENSOR(bias0, 512);
+        INIT(data0, TensorInitType::FILE, "mnist_images_8.bin");
+        INIT(weight0, TensorInitType::FILE, "mlp_weight0.bin");
+        INIT(bias0, TensorInitType::FILE, "mlp_bias0.bin");
+        OP(fc0, MatrixMatrixFCBiasOp);
+        LINKUPPER(fc0, data0, weight0, bias0);
+        TENSOR(data1, 8, 512);
+        LINKUPPER(data1, fc0);
+        OP(tanh0, MatrixTanhOp);
+        LINKUPPER(tanh0, data1);
+        TENSOR(data2, 8, 512);
+        LINKUPPER(data2, tanh0);
+        TENSOR(weight1, 512, 10);
+        TENSOR(bias1, 10);
+        INIT(weight1, TensorInitType::FILE, "mlp_weight1.bin");
+        INIT(bias1, TensorInitType::FILE, "mlp_bias1.bin");
+        OP(fc1, MatrixMatrixFCBiasOp);
+        LINKUPPER(fc1, data2, weight1, bias1);
+        TENSOR(data3, 8, 10);
+        LINKUPPER(data3, fc1);
+        OP(softmax, MatrixSoftmaxOp);
+        LINKUPPER(softmax, data3);
+        TENSOR(data4, 8, 10);
+        LINKUPPER(data4, softmax);
+        auto *argmax_o = new OpNode("argmax", new ArgMaxOp(3));
+        argmax_o->exlinkUpperNode(data4);
+        auto *top3_t = new TensorNode("top3", new Tensor({8, 3}, DataType::Int32_t), argmax_o);
+        auto *print_o = new OpNode("print", new DebugOp());
+        print_o->exlinkUpperNode(top3_t);
+        GpT(graph, data0, weight0, bias0, data1, data2, weight1, bias1, data3, data4, top3_t);
+        GpO(graph, fc0, tanh0, fc1, softmax, argmax_o, print_o);
+        graph->addLogicalOutNodes(data4, top3_t);   // dump the probabilities and the top-3 table
+    } else if (model == "cfg1" || model == "cfg2") {
+        const bool wide = model == "cfg2";
+        const size_t b = batch ? batch : (wide ? 4096 : 8), hidden = wide ? 4096 : 512;
+        auto *x = new TensorNode("x", new Tensor({b, 784}));
+        fromFile(x->getTensor(), "x");
+        graph->pushTensorNode(x);
+        TensorNode *h = fc(graph, "fc1", x, 784, hidden, true);
+        if (wide) h = fc(graph, "fc2", h, hidden, hidden, true);
+        h = fc(graph, wide ? "fc3" : "fc2", h, hidden, 10, false);
+        out = unary(graph, "softmax", new MatrixSoftmaxOp(), h);
+    } else if (model == "cfg3") {
+        const size_t b = batch ? batch : 256;
+        auto *x = new TensorNode("x", new Tensor({b, 28, 28, 1}));
+        fromFile(x->getTensor(), "x");
+        graph->pushTensorNode(x);
+        TensorNode *h = conv(graph, "conv1", x, 20, 5, 0);
+        graph->initTensorNodes();
+        h = pool(graph, "pool1", lazyUnary(graph, "relu1", new ReluOp(), h));
+        graph->initTensorNodes();
+        h = conv(graph, "conv2", h, 50, 5, 0);
+        h = pool(graph, "pool2", lazyUnary(graph, "relu2", new ReluOp(), h));
+        graph->initTensorNodes();
+        h = fc(graph, "fc1", h, 800, 500, true);   // 4-D input: read as [b, 4*4*50]
+        h = fc(graph, "fc2", h, 500, 10, false);
+        out = unary(graph, "softmax", new MatrixSoftmaxOp(), h);
+    } else if (model == "cfg4") {
+        const size_t b = batch ? batch : 32;
+        auto *x = new TensorNode("x", new Tensor({b, 56, 56, 64}));
+        fromFile(x->getTensor(), "x");
+        graph->pushTensorNode(x);
+        const size_t oc[4] = {64, 128, 128, 128};
+        TensorNode *h = x;
+        for (int i = 0; i < 4; ++i) {
+            const string n = to_string(i + 1);
+            h = conv(graph, "conv" + n, h, oc[i], 3, 1);
+            graph->initTensorNodes();
+            h = lazyUnary(graph, "relu" + n, new ReluOp(), bn(graph, "bn" + n, h));
+            if (i == 1 || i == 3) h = pool(graph, "pool" + n, h);
+            graph->initTensorNodes();
+        }
+        out = h;
+    } else if (model == "cfg5a") {
+        const size_t rows = batch ? batch : 65536;
+        auto *x = new TensorNode("logits", new Tensor({rows, 1000}));
+        fromFile(x->getTensor(), "logits");
+        graph->pushTensorNode(x);
+        out = unary(graph, "softmax", new MatrixSoftmaxOp(), x);
+    } else if (model == "cfg5b" || model == "cfg5c") {
+        const size_t b = batch ? batch : 256;
+        auto *p = new TensorNode("p", new Tensor({b, 32, 32, 256}));
+        fromFile(p->getTensor(), "p");
+        graph->pushTensorNode(p);
+        if (model == "cfg5b") {
+            auto *q = new TensorNode("q", new Tensor({b, 32, 32, 256}));
+            fromFile(q->getTensor(), "q");
+            OP(add, ElementAddOp);
+            LINKUPPER(add, p, q);
+            auto *s = new TensorNode("sum", new Tensor({b, 32, 32, 256}), add);
+            graph->pushTensorNode(q, s);
+            graph->pushOpNode(add);
+            out = unary(graph, "relu", new ReluOp(), s);
+        } else {
+            TensorNode *h = bn(graph, "bn", p);
+            graph->initTensorNodes();
+            h = lazyUnary(graph, "relu", new ReluOp(), h);
+            out = pool(graph, "pool", h);
+            graph->initTensorNodes();
+        }
+    } else {
+        cerr << "unknown model " << model << "\n";
+        return 2;
+    }
+    (void)out;
+
+    graph->initTensorNodes();
+    graph->findInOut();
+    graph->updateTopology();
+
+    Config config;
+    config.hip = target == "hip";
+    config.hip_fusion = !nofuse;
+    config.time_iters = iters;
+    config.dump_outputs = true;
+    graph->setConfig(config);
+
+    Engine engine(graph);
+    engine.compile();
+    string code = engine.genCode();
+    cout << code;
+    return 0;
+}

@@ -1,0 +1,188 @@
+"""The compiler side: SWC API -> passes -> CPU / HIP code generators.
+
+CPU (no GPU needed): graphs built through the SWC API compile, the CPU program
+calls the reference's kernels in the reference's order (checked by running it
+against the reference's own utils/kernels.h where the reference tree exists,
+else against the oracle through oracle/compat) and its outputs equal the
+oracle's graph run bit for bit; the HIP program has the expected structure and
+builds against include/swc_hip.h + libswc_hip.so.
+GPU: the HIP program runs on the MI355X and matches the oracle.
+"""
+import os
+import re
+import shutil
+import subprocess
+
+import numpy as np
+import pytest
+
+from swcompiler_amd import graphs
+from tests.util import assert_bit_exact, rel_err, strict_rel_err
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SWC = os.path.join(ROOT, "swcompiler_amd", "swc")
+GEN = os.path.join(SWC, "test", "bin", "genGraphs")
+REF_UTILS = "/root/reference/src/codegen"
+TOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def gen():
+    if not os.path.exists(GEN):
+        subprocess.check_call(["make", "-C", SWC, "-j8"], stdout=subprocess.DEVNULL)
+    return GEN
+
+
+def file_map(cfg, t):
+    """graphs.make_inputs key -> file stem read by the programs genGraphs builds"""
+    m = {}
+    for k in t:
+        if k in ("x", "logits", "p", "q"):
+            m[k] = k
+        elif re.fullmatch(r"w\d", k):
+            m[k] = f"fc{k[1]}_w"
+        elif re.fullmatch(r"b\d", k):
+            m[k] = f"fc{k[1]}_b"
+        elif re.fullmatch(r"f\d", k):
+            m[k] = f"conv{k[1]}_f"
+        elif re.fullmatch(r"cb\d", k):
+            m[k] = f"conv{k[2]}_b"
+        elif k.startswith("bn"):
+            m[k] = k
+    return m
+
+
+def write_inputs(cfg, t, workdir):
+    for k, stem in file_map(cfg, t).items():
+        t[k].tofile(os.path.join(workdir, stem + ".bin"))
+
+
+def generate(gen, model, target, workdir, batch=0, iters=0, nofuse=False):
+    args = [gen, model, target, str(batch), str(iters)] + (["nofuse"] if nofuse else [])
+    code = subprocess.run(args, cwd=workdir, check=True, capture_output=True, text=True).stdout
+    assert open(os.path.join(workdir, "Graph.cpp")).read() == code
+    return code
+
+
+def build_cpu(workdir):
+    if os.path.isdir(REF_UTILS):   # the reference's own image.h / kernels.h
+        cmd = ["g++", "-std=c++11", "-O2", "-w", "-I", REF_UTILS, "Graph.cpp", "-o", "net_cpu.bin"]
+    else:
+        odir = os.path.join(ROOT, "oracle")
+        cmd = ["g++", "-std=c++11", "-O2", "-I", os.path.join(odir, "compat"), "-I", os.path.join(ROOT, "include"),
+               "Graph.cpp", "-L", odir, "-Wl,-rpath," + odir, "-loracle", "-o", "net_cpu.bin"]
+    subprocess.check_call(cmd, cwd=workdir)
+    return os.path.join(workdir, "net_cpu.bin")
+
+
+def build_hip(workdir):
+    libdir = os.path.join(ROOT, "swcompiler_amd")
+    subprocess.check_call(["g++", "-std=c++11", "-O2", "-I", os.path.join(ROOT, "include"), "Graph.cpp", "-L", libdir,
+                           "-Wl,-rpath," + libdir, "-lswc_hip", "-o", "net_hip.bin"], cwd=workdir)
+    return os.path.join(workdir, "net_hip.bin")
+
+
+MODELS = [("cfg1", 1, 8, "softmax_out"), ("cfg2", 2, 16, "softmax_out"), ("cfg3", 3, 4, "softmax_out"),
+          ("cfg4", 4, 1, "pool4_out"), ("cfg5a", 5, 1, "softmax_out"), ("cfg5b", 5, 1, "relu_out"),
+          ("cfg5c", 5, 1, "pool_out")]
+
+
+def oracle_run(oracle, model, cfg, t):
+    out = graphs.run(cfg, oracle, t, fused=False)
+    return out[model[-1]] if cfg == 5 else out
+
+
+def model_batch(model, batch):
+    return batch * 256 if model == "cfg5a" else batch   # cfg5a counts softmax rows
+
+
+@pytest.mark.parametrize("model,cfg,batch,outname", MODELS)
+def test_cpu_program_equals_oracle_bit_for_bit(gen, oracle, tmp_path, model, cfg, batch, outname):
+    t = graphs.make_inputs(cfg, batch)
+    write_inputs(cfg, t, tmp_path)
+    code = generate(gen, model, "cpu", tmp_path, model_batch(model, batch))
+    assert "swc_hip" not in code and '#include "utils/kernels.h"' in code
+    if model in ("cfg1", "cfg2", "cfg3"):   # FCBias is lowered exactly as the reference does it
+        assert "matrixMatrixMul_f(" in code and "batchedadd_f(" in code and "_mm_out" in code
+    exe = build_cpu(tmp_path)
+    subprocess.check_call([exe], cwd=tmp_path, stdout=subprocess.DEVNULL)
+    want = oracle_run(oracle, model, cfg, t)
+    got = np.fromfile(os.path.join(tmp_path, outname + ".bin"), np.float32).reshape(want.shape)
+    assert_bit_exact(got, want, model)
+
+
+def test_mnist8_cpu_program_prints_the_reference_labels(gen, tmp_path, golden):
+    for f in os.listdir(os.path.join(ROOT, "tests", "golden", "mnist8")):
+        shutil.copy(os.path.join(ROOT, "tests", "golden", "mnist8", f), tmp_path)
+    generate(gen, "mnist8", "cpu", tmp_path)
+    exe = build_cpu(tmp_path)
+    out = subprocess.run([exe], cwd=tmp_path, check=True, capture_output=True, text=True).stdout
+    rows = [[int(v) for v in line.split()] for line in out.strip().splitlines()]
+    assert [r[0] for r in rows] == [5, 0, 4, 1, 9, 2, 1, 3]
+    assert_bit_exact(np.array(rows, np.int32), golden["mnist8_top3"], "printed top-3")
+
+
+def test_hip_program_structure_and_build(gen, tmp_path):
+    code = generate(gen, "cfg4", "hip", tmp_path, 2)
+    # fused: four conv+bn+relu launches, two pools, nothing else on the device
+    assert code.count("swc_hip_conv2dFused_f(") == 4 and "swc_hip_batchnorm" not in code and "swc_hip_relu_f" not in code
+    assert code.count("swc_hip_maxpool_f(") == 2
+    # every device tensor sits on a 256-byte boundary of the arena
+    offs = [int(v) for v in re.findall(r"gpu0_baseptr \+ (\d+)\)", code)]
+    assert offs and all(o % 256 == 0 for o in offs)
+    # parameters are uploaded once, before the op calls; the result comes back once, after them
+    body = code[code.index("// call op routine functions"):]
+    assert "swc_hip_h2d" not in body and body.count("swc_hip_d2h(") == 1
+    assert code.count("swc_hip_h2d(") == 1 + 4 * 6   # x + per layer filter, bias, 4 bn params
+    build_hip(tmp_path)
+
+    unfused = generate(gen, "cfg4", "hip", tmp_path, 2, nofuse=True)
+    assert unfused.count("swc_hip_conv2d_f(") == 4 and unfused.count("swc_hip_batchnormalization_f(") == 4
+    assert unfused.count("swc_hip_relu_f(") == 4
+
+    mlp = generate(gen, "cfg2", "hip", tmp_path, 64)
+    assert mlp.count("swc_hip_matrixMatrixFCBias_f(") == 3 and "swc_hip_batchedadd_f" not in mlp
+    assert re.search(r"swc_hip_matrixMatrixFCBias_f\(64, 4096, 784, .*, 1\)\);", mlp)
+    lenet = generate(gen, "cfg3", "hip", tmp_path, 4)
+    assert lenet.count("swc_hip_conv2dFused_f(") == 2 and "swc_hip_matrixMatrixFCBias_f(4, 500, 800" in lenet
+    timed = generate(gen, "cfg5b", "hip", tmp_path, 1, iters=10)
+    assert "swc_hip_vecAddRelu_f(" in timed and "swc_time_ms_per_iter" in timed and "swc_iter < 10" in timed
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("model,cfg,batch,outname", MODELS)
+@pytest.mark.parametrize("nofuse", [False, True])
+def test_hip_program_matches_oracle(gen, oracle, tmp_path, model, cfg, batch, outname, nofuse):
+    print(f"case generated {model} batch {batch} nofuse={nofuse}", flush=True)
+    t = graphs.make_inputs(cfg, batch)
+    write_inputs(cfg, t, tmp_path)
+    generate(gen, model, "hip", tmp_path, model_batch(model, batch), nofuse=nofuse)
+    exe = build_hip(tmp_path)
+    subprocess.run([exe], cwd=tmp_path, check=True, timeout=120, stdout=subprocess.DEVNULL)
+    want = oracle_run(oracle, model, cfg, t)
+    got = np.fromfile(os.path.join(tmp_path, outname + "_host.bin"), np.float32).reshape(want.shape)
+    if model == "cfg5b":
+        assert_bit_exact(got, want, model)
+    elif model == "cfg4":
+        assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < TOL
+    elif model == "cfg5c":
+        assert rel_err(got, want) < TOL
+    else:
+        nz = want > 1e-30
+        assert strict_rel_err(got[nz], want[nz]) < 5 * TOL
+
+
+@pytest.mark.gpu
+def test_mnist8_hip_program_prints_the_reference_labels(gen, tmp_path, golden):
+    for f in os.listdir(os.path.join(ROOT, "tests", "golden", "mnist8")):
+        shutil.copy(os.path.join(ROOT, "tests", "golden", "mnist8", f), tmp_path)
+    generate(gen, "mnist8", "hip", tmp_path)
+    exe = build_hip(tmp_path)
+    out = subprocess.run([exe], cwd=tmp_path, check=True, capture_output=True, text=True, timeout=120).stdout
+    rows = [[int(v) for v in line.split()] for line in out.strip().splitlines()]
+    assert [r[0] for r in rows] == [5, 0, 4, 1, 9, 2, 1, 3]
+    assert_bit_exact(np.array(rows, np.int32), golden["mnist8_top3"], "printed top-3")
+    prob = np.fromfile(os.path.join(tmp_path, "data4_host.bin"), np.float32).reshape(8, 10)
+    assert strict_rel_err(prob, golden["mnist8_prob"]) < TOL
+    top3 = np.fromfile(os.path.join(tmp_path, "top3_host.bin"), np.int32).reshape(8, 3)
+    assert_bit_exact(top3, golden["mnist8_top3"], "dumped top-3")
