@@ -11,7 +11,10 @@
 // from the FC GEMM.  When iC % 4 == 0 four consecutive k's lie in one tap, so
 // the gather uses 128-bit loads; otherwise (first layer, iC = 1 or 3) 32-bit.
 #include "common.hpp"
+#include "mfma_dma.hpp"
 #include "mfma_tile.hpp"
+#include <cstdlib>
+#include <cstring>
 
 using namespace swc_hip;
 using namespace swc_hip::mfma;
@@ -49,8 +52,14 @@ __global__ __launch_bounds__(kThreads) void conv_igemm(const float *__restrict__
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
     // VEC: thread owns rows (tid>>3) + 32*i of the A tile and k quad (tid&7).
-    // Top-left input coordinate of each owned output pixel, (-1<<20) if row >= M.
-    int iy0[T::kAVec], ix0[T::kAVec], img[T::kAVec];
+    // Per owned output pixel: element offset of its window's top-left tap
+    // (channel 0) and that tap's input coordinates; rows >= M get coordinates
+    // far outside the image so every tap fails the bounds test.
+    long row_off[T::kAVec];
+    int iy0[T::kAVec], ix0[T::kAVec];
+    // The k position of this thread's quad, kept as (ky, kx, ci) and advanced by
+    // BK per slice without divisions; tap_off = ((ky*W + kx)*C + ci).
+    int ky = 0, kx = 0, ci = 0, kpos = 0;
     if (VEC) {
 #pragma unroll
         for (int i = 0; i < T::kAVec; ++i) {
@@ -59,39 +68,54 @@ __global__ __launch_bounds__(kThreads) void conv_igemm(const float *__restrict__
                 const int ox = m % g.OW;
                 const int t = m / g.OW;
                 const int oy = t % g.OH;
-                img[i] = t / g.OH;
+                const int img = t / g.OH;
                 iy0[i] = oy * g.sh - g.pt;
                 ix0[i] = ox * g.sw - g.pl;
+                row_off[i] = (((long)img * g.H + iy0[i]) * g.W + ix0[i]) * g.C;
             } else {
-                img[i] = 0;
                 iy0[i] = -(1 << 20);
                 ix0[i] = -(1 << 20);
+                row_off[i] = 0;
             }
         }
+        kpos = (tid & 7) * 4;
+        const int tap = kpos / g.C;
+        ci = kpos - tap * g.C;
+        ky = tap / g.kw;
+        kx = tap - ky * g.kw;
     }
 
     constexpr int kAScalar = T::kAVec * 4, kBScalar = T::kBVec * 4;
     float4 ra[T::kAVec], rb[T::kBVec];
     float sa[VEC ? 1 : kAScalar], sb[VEC ? 1 : kBScalar];
 
+    // VEC path: loads the slice at the thread's current (ky,kx,ci), then steps
+    // the position by BK.  Slices are visited strictly in order.
     auto load_global = [&](int k0) {
         if (VEC) {
-            const int k = k0 + (tid & 7) * 4;
-            const int tap = k / g.C, ci = k - tap * g.C;
-            const int ky = tap / g.kw, kx = tap - ky * g.kw;
+            const bool k_ok = kpos < K;
+            const long tap_off = ((long)ky * g.W + kx) * g.C + ci;
 #pragma unroll
             for (int i = 0; i < T::kAVec; ++i) {
                 const int iy = iy0[i] + ky, ix = ix0[i] + kx;
-                const bool ok = k < K && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
-                ra[i] = ok ? *reinterpret_cast<const float4 *>(
-                                 in + (((size_t)img[i] * g.H + iy) * g.W + ix) * g.C + ci)
+                const bool ok = k_ok && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
+                ra[i] = ok ? *reinterpret_cast<const float4 *>(in + row_off[i] + tap_off)
                            : make_float4(0.f, 0.f, 0.f, 0.f);
             }
 #pragma unroll
             for (int i = 0; i < T::kBVec; ++i) {
                 const int col = n0 + (tid >> 3) + 32 * i;
-                rb[i] = (col < N && k < K) ? *reinterpret_cast<const float4 *>(filt + (size_t)col * K + k)
-                                           : make_float4(0.f, 0.f, 0.f, 0.f);
+                rb[i] = (col < N && k_ok) ? *reinterpret_cast<const float4 *>(filt + (size_t)col * K + kpos)
+                                          : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+            kpos += BK;
+            ci += BK;
+            while (ci >= g.C) {
+                ci -= g.C;
+                if (++kx == g.kw) {
+                    kx = 0;
+                    ++ky;
+                }
             }
         } else {
 #pragma unroll
@@ -103,11 +127,11 @@ __global__ __launch_bounds__(kThreads) void conv_igemm(const float *__restrict__
                     const int ox = m % g.OW;
                     const int t = m / g.OW;
                     const int oy = t % g.OH, n = t / g.OH;
-                    const int tap = k / g.C, ci = k - tap * g.C;
-                    const int ky = tap / g.kw, kx = tap - ky * g.kw;
-                    const int iy = oy * g.sh - g.pt + ky, ix = ox * g.sw - g.pl + kx;
+                    const int tap = k / g.C, cc = k - tap * g.C;
+                    const int kyy = tap / g.kw, kxx = tap - kyy * g.kw;
+                    const int iy = oy * g.sh - g.pt + kyy, ix = ox * g.sw - g.pl + kxx;
                     if (iy >= 0 && iy < g.H && ix >= 0 && ix < g.W)
-                        v = in[(((size_t)n * g.H + iy) * g.W + ix) * g.C + ci];
+                        v = in[(((size_t)n * g.H + iy) * g.W + ix) * g.C + cc];
                 }
                 sa[i] = v;
             }
@@ -158,6 +182,139 @@ __global__ __launch_bounds__(kThreads) void conv_igemm(const float *__restrict__
     store_tile<TM, TN>(acc, out, (size_t)N, M, N, m0 + wave_m * 32 * TM, n0 + wave_n * 32 * TN, lane, ep);
 }
 
+// Direct-to-LDS variant (mfma_dma.hpp): the im2col gather is expressed as one
+// 32-bit byte offset per lane per load — out-of-image taps and rows past M get
+// the out-of-range offset and arrive in LDS as zeros.  Needs iC % 4 == 0,
+// 16-byte-aligned tensors and input/filter below 2 GiB.
+template <int TM, int TN, int STAGES>
+__global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ in, const float *__restrict__ filt,
+                                                     float *__restrict__ out, ConvGeom g, unsigned in_bytes,
+                                                     unsigned filt_bytes, Epilogue ep) {
+#if __HIP_DEVICE_COMPILE__   // the host pass only needs the launch stub
+    using T = DmaTile<TM, TN, true, STAGES>;
+    extern __shared__ __align__(16) float lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int M = g.M, N = g.OC, K = g.K;
+
+    int tile_m, tile_n;
+    tile_coords((M + T::BM - 1) / T::BM, (N + T::BN - 1) / T::BN, tile_m, tile_n);
+    const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(in, in_bytes);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(filt, filt_bytes);
+
+    // Per load, the output pixel this lane gathers for: element offset of its
+    // window's top-left tap (may be negative) and that tap's coordinates; rows
+    // past M get coordinates no tap can bring back inside the image.
+    int row_off[T::kALoads], iy0[T::kALoads], ix0[T::kALoads], f_base[T::kBLoads];
+#pragma unroll
+    for (int j = 0; j < T::kALoads; ++j) {
+        const int m = m0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
+        if (m < M) {
+            const int ox = m % g.OW;
+            const int t = m / g.OW;
+            const int oy = t % g.OH;
+            const int img = t / g.OH;
+            iy0[j] = oy * g.sh - g.pt;
+            ix0[j] = ox * g.sw - g.pl;
+            row_off[j] = ((img * g.H + iy0[j]) * g.W + ix0[j]) * g.C;
+        } else {
+            iy0[j] = ix0[j] = -(1 << 20);
+            row_off[j] = 0;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < T::kBLoads; ++j) {
+        const int n = n0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
+        f_base[j] = n < N ? n * K * 4 : kOutOfRange;
+    }
+    // k position of this lane's chunk, as (ky, kx, ci), stepped by BK per slice
+    int kpos = kc_chunk(lane) * 4;
+    int ky, kx, ci;
+    {
+        const int tap = kpos / g.C;
+        ci = kpos - tap * g.C;
+        ky = tap / g.kw;
+        kx = tap - ky * g.kw;
+    }
+    int va[T::kALoads], vb[T::kBLoads];
+    auto next_offsets = [&]() {   // offsets of the next slice in order
+        const bool k_ok = kpos < K;
+        const int tap_off = (ky * g.W + kx) * g.C + ci;
+#pragma unroll
+        for (int j = 0; j < T::kALoads; ++j) {
+            const bool ok = k_ok && (unsigned)(iy0[j] + ky) < (unsigned)g.H && (unsigned)(ix0[j] + kx) < (unsigned)g.W;
+            va[j] = ok ? (row_off[j] + tap_off) * 4 : kOutOfRange;
+        }
+#pragma unroll
+        for (int j = 0; j < T::kBLoads; ++j)
+            vb[j] = (k_ok && f_base[j] != kOutOfRange) ? f_base[j] + kpos * 4 : kOutOfRange;
+        kpos += BK;
+        ci += BK;
+        while (ci >= g.C) {
+            ci -= g.C;
+            if (++kx == g.kw) {
+                kx = 0;
+                ++ky;
+            }
+        }
+    };
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) {
+        next_offsets();
+        float *wr = lds + s * T::kStageFloats;
+#pragma unroll
+        for (int j = 0; j < T::kALoads; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t *)(wr + (4 * j + wave) * 256), 16, va[j], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < T::kBLoads; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_t *)(wr + T::kAFloats + (4 * j + wave) * 256), 16,
+                                                     vb[j], 0, 0, 0);
+    }
+    const int nk = (K + BK - 1) / BK;
+    int rd_stage = 0, wr_stage = STAGES - 1;
+    for (int kt = 0; kt < nk; ++kt) {
+        ring_sync<(STAGES - 2) * T::kLoads>();
+        next_offsets();
+        dma_step<TM, TN, true, STAGES>(lds + wr_stage * T::kStageFloats, lds + rd_stage * T::kStageFloats, rsrc_a,
+                                       rsrc_b, va, vb, acc, wave, lane);
+        rd_stage = rd_stage + 1 == STAGES ? 0 : rd_stage + 1;
+        wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
+    }
+    wait_vmcnt<0>();   // the trailing dummy loads still target this workgroup's LDS
+    store_tile<TM, TN>(acc, out, (size_t)N, M, N, m0 + (wave >> 1) * 32 * TM, n0 + (wave & 1) * 32 * TN, lane, ep);
+#endif
+}
+
+template <int TM, int TN, int STAGES>
+int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGeom &g, size_t in_bytes,
+                    size_t filt_bytes, const Epilogue &ep) {
+    using T = DmaTile<TM, TN, true, STAGES>;
+    const long tiles = (long)((g.M + T::BM - 1) / T::BM) * ((g.OC + T::BN - 1) / T::BN);
+    auto kern = conv_dma<TM, TN, STAGES>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        SWC_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)T::kLdsBytes));
+        attr_set = true;
+    }
+    kern<<<(unsigned)tiles, kThreads, T::kLdsBytes, stream()>>>(in, filt, out, g, (unsigned)in_bytes,
+                                                                 (unsigned)filt_bytes, ep);
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
+}
+
 template <int TM, int TN>
 int launch_conv(bool vec, const float *in, const float *filt, float *out, const ConvGeom &g, const Epilogue &ep) {
     using T = Tile<TM, TN, true>;
@@ -202,6 +359,30 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
     Epilogue ep = ep_in;
     ep.bias = bias;
     const bool vec = (g.C % 4 == 0) && aligned16(input) && aligned16(filter);
+    const size_t in_bytes = idims[0] * idims[1] * idims[2] * idims[3] * 4, filt_bytes = odims[3] * K * 4;
+    const bool dma_ok = vec && in_bytes < kMaxDmaBytes && filt_bytes < kMaxDmaBytes;
+    const char *force = getenv("SWC_HIP_CONV");   // forces a kernel variant (tests, tuning): reg22 reg21 reg12 reg11 | 22_2 21_3 12_3 11_3 11_4
+    if (force) {
+        if (!strcmp(force, "reg22")) return launch_conv<2, 2>(vec, input, filter, output, g, ep);
+        if (!strcmp(force, "reg21")) return launch_conv<2, 1>(vec, input, filter, output, g, ep);
+        if (!strcmp(force, "reg12")) return launch_conv<1, 2>(vec, input, filter, output, g, ep);
+        if (!strcmp(force, "reg11")) return launch_conv<1, 1>(vec, input, filter, output, g, ep);
+        if (dma_ok) {
+            if (!strcmp(force, "22_2")) return launch_conv_dma<2, 2, 2>(input, filter, output, g, in_bytes, filt_bytes, ep);
+            if (!strcmp(force, "21_3")) return launch_conv_dma<2, 1, 3>(input, filter, output, g, in_bytes, filt_bytes, ep);
+            if (!strcmp(force, "12_3")) return launch_conv_dma<1, 2, 3>(input, filter, output, g, in_bytes, filt_bytes, ep);
+            if (!strcmp(force, "11_3")) return launch_conv_dma<1, 1, 3>(input, filter, output, g, in_bytes, filt_bytes, ep);
+            if (!strcmp(force, "11_4")) return launch_conv_dma<1, 1, 4>(input, filter, output, g, in_bytes, filt_bytes, ep);
+        }
+    }
+    if (dma_ok) {
+        // 64x128 tiles once they fill the chip (wide layers), 64x64 otherwise: the
+        // layers here are tens of microseconds long, many small tiles balance the
+        // 256 CUs better than few large ones
+        if (g.OC > 64 && ((M + 63) / 64) * ((g.OC + 127) / 128) >= (size_t)num_cus())
+            return launch_conv_dma<1, 2, 3>(input, filter, output, g, in_bytes, filt_bytes, ep);
+        return launch_conv_dma<1, 1, 3>(input, filter, output, g, in_bytes, filt_bytes, ep);
+    }
     const long tiles_m128 = (M + 127) / 128;
     if (g.OC > 64 && tiles_m128 * ((g.OC + 127) / 128) >= num_cus())
         return launch_conv<2, 2>(vec, input, filter, output, g, ep);

