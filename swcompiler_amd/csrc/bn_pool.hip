@@ -47,7 +47,11 @@ __device__ __forceinline__ float4 bn4(float4 x, const BnQuad &q) {
 
 // The launch makes gridDim.x*kThreads a multiple of quads (= C/4), so the
 // channel quad of a thread never changes while it strides through the tensor.
-template <bool RELU>
+// Each trip issues kBnUnroll independent 128-bit loads before anything else, and
+// the per-thread constants (four channels' parameters, a double 1/sqrt each) are
+// computed while the first trip's loads are in flight.
+constexpr int kBnUnroll = 4;
+template <bool RELU, bool NT>
 __global__ __launch_bounds__(kThreads) void bn_vec4(float *out, const float *in, const float *__restrict__ mean,
                                                     const float *__restrict__ var, const float *__restrict__ scale,
                                                     const float *__restrict__ bias, size_t total4, unsigned quads,
@@ -55,19 +59,25 @@ __global__ __launch_bounds__(kThreads) void bn_vec4(float *out, const float *in,
     const size_t g = (size_t)blockIdx.x * kThreads + threadIdx.x;
     const size_t step = (size_t)gridDim.x * kThreads;
     if (g >= total4) return;
-    BnQuad q;
-    load_bn_quad(q, mean, var, scale, bias, (g % quads) * 4, eps);
     const float4 *i4 = reinterpret_cast<const float4 *>(in);
     float4 *o4 = reinterpret_cast<float4 *>(out);
+    float4 x[kBnUnroll];
+#pragma unroll
+    for (int u = 0; u < kBnUnroll; ++u)
+        if (g + u * step < total4) x[u] = ld4<NT>(i4 + g + u * step);
+    BnQuad q;
+    load_bn_quad(q, mean, var, scale, bias, (g % quads) * 4, eps);
     size_t i = g;
-    // two independent loads in flight per thread
-    for (; i + step < total4; i += 2 * step) {
-        const float4 x0 = i4[i];
-        const float4 x1 = i4[i + step];
-        o4[i] = bn4<RELU>(x0, q);
-        o4[i + step] = bn4<RELU>(x1, q);
+    while (true) {
+#pragma unroll
+        for (int u = 0; u < kBnUnroll; ++u)
+            if (i + u * step < total4) st4<NT>(o4 + i + u * step, bn4<RELU>(x[u], q));
+        i += kBnUnroll * step;
+        if (i >= total4) break;
+#pragma unroll
+        for (int u = 0; u < kBnUnroll; ++u)
+            if (i + u * step < total4) x[u] = ld4<NT>(i4 + i + u * step);
     }
-    if (i < total4) o4[i] = bn4<RELU>(i4[i], q);
 }
 
 template <bool RELU>
@@ -92,7 +102,7 @@ struct PoolGeom {
 
 // First in-bounds tap initialises, later taps replace only when strictly
 // greater (kernels.h:362-366).  `BN` applies batchnorm+relu to each tap first.
-template <bool ARGMAX, bool BN>
+template <bool ARGMAX, bool BN, bool NT>
 __global__ __launch_bounds__(kThreads) void maxpool_vec4(const float *__restrict__ in, float *__restrict__ out,
                                                          int32_t *__restrict__ arg, PoolGeom g, size_t total4,
                                                          const float *__restrict__ mean, const float *__restrict__ var,
@@ -122,7 +132,7 @@ __global__ __launch_bounds__(kThreads) void maxpool_vec4(const float *__restrict
                 const int ix = ox * g.sw - g.pl + kx;
                 if (ix < 0 || ix >= g.W) continue;
                 const size_t pix = ((size_t)n * g.H + iy) * g.W + ix;
-                float4 v4 = i4[pix * quads + cq];
+                float4 v4 = ld4<NT>(i4 + pix * quads + cq);
                 if (BN) v4 = bn4<true>(v4, q);
                 const float v[4] = {v4.x, v4.y, v4.z, v4.w};
                 const int32_t flat = (int32_t)(pix * g.C + cq * 4);
@@ -136,8 +146,8 @@ __global__ __launch_bounds__(kThreads) void maxpool_vec4(const float *__restrict
                 have = true;
             }
         }
-        reinterpret_cast<float4 *>(out)[o] = make_float4(best[0], best[1], best[2], best[3]);
-        if (ARGMAX) reinterpret_cast<int4 *>(arg)[o] = make_int4(where[0], where[1], where[2], where[3]);
+        st4<NT>(reinterpret_cast<float4 *>(out) + o, make_float4(best[0], best[1], best[2], best[3]));
+        if (ARGMAX) st4i<NT>(reinterpret_cast<int4 *>(arg) + o, make_int4(where[0], where[1], where[2], where[3]));
     }
 }
 
@@ -216,8 +226,11 @@ int launch_bn(const char *who, float *output, const float *input, const float *m
     if (C % 4 == 0 && aligned16(output) && aligned16(input)) {
         const size_t total4 = total / 4;
         const unsigned quads = (unsigned)(C / 4);
-        const unsigned blocks = quad_stable_blocks((total4 + 3) / 4, quads, (unsigned)num_cus() * 16u);
-        bn_vec4<RELU><<<blocks, kThreads, 0, stream()>>>(output, input, mean, var, scale, bias, total4, quads, eps);
+        const unsigned blocks = quad_stable_blocks((total4 + kBnUnroll - 1) / kBnUnroll, quads, (unsigned)num_cus() * 64u);
+        if (total * sizeof(float) >= kStreamingBytes)
+            bn_vec4<RELU, true><<<blocks, kThreads, 0, stream()>>>(output, input, mean, var, scale, bias, total4, quads, eps);
+        else
+            bn_vec4<RELU, false><<<blocks, kThreads, 0, stream()>>>(output, input, mean, var, scale, bias, total4, quads, eps);
     } else {
         size_t blocks = (total + kThreads - 1) / kThreads;
         if (blocks > 8192) blocks = 8192;
@@ -255,8 +268,11 @@ int launch_pool(const char *who, const float *input, float *output, int32_t *arg
     const size_t C = idims[3];
     if (C % 4 == 0 && aligned16(input) && aligned16(output) && (!ARGMAX || aligned16(argmax))) {
         const size_t total4 = total / 4;
-        const unsigned blocks = quad_stable_blocks(total4, (unsigned)(C / 4), (unsigned)num_cus() * 32u);
-        maxpool_vec4<ARGMAX, BN><<<blocks, kThreads, 0, stream()>>>(input, output, argmax, g, total4, mean, var, scale, bias, eps);
+        const unsigned blocks = quad_stable_blocks(total4, (unsigned)(C / 4), (unsigned)num_cus() * 128u);
+        if (in_total * sizeof(float) >= kStreamingBytes)
+            maxpool_vec4<ARGMAX, BN, true><<<blocks, kThreads, 0, stream()>>>(input, output, argmax, g, total4, mean, var, scale, bias, eps);
+        else
+            maxpool_vec4<ARGMAX, BN, false><<<blocks, kThreads, 0, stream()>>>(input, output, argmax, g, total4, mean, var, scale, bias, eps);
     } else {
         size_t blocks = (total + kThreads - 1) / kThreads;
         if (blocks > 8192) blocks = 8192;

@@ -24,6 +24,38 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 inline unsigned ceil_div(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
 
+// Tensors at least this large are streamed with non-temporal loads and stores:
+// they cannot stay in the 4 MB-per-XCD L2 / 256 MB infinity cache anyway, and
+// marking the traffic as streaming measured ~10 % more HBM bandwidth on MI355X.
+// Smaller tensors keep normal caching so the next kernel finds them on chip.
+constexpr size_t kStreamingBytes = (size_t)64 << 20;
+
+typedef float swc_f4 __attribute__((ext_vector_type(4)));
+typedef int swc_i4 __attribute__((ext_vector_type(4)));
+template <bool NT> __device__ __forceinline__ float4 ld4(const float4 *p) {
+    if (NT) {
+        const swc_f4 v = __builtin_nontemporal_load(reinterpret_cast<const swc_f4 *>(p));
+        return make_float4(v.x, v.y, v.z, v.w);
+    }
+    return *p;
+}
+template <bool NT> __device__ __forceinline__ void st4(float4 *p, float4 r) {
+    if (NT) {
+        const swc_f4 v = {r.x, r.y, r.z, r.w};
+        __builtin_nontemporal_store(v, reinterpret_cast<swc_f4 *>(p));
+    } else {
+        *p = r;
+    }
+}
+template <bool NT> __device__ __forceinline__ void st4i(int4 *p, int4 r) {
+    if (NT) {
+        const swc_i4 v = {r.x, r.y, r.z, r.w};
+        __builtin_nontemporal_store(v, reinterpret_cast<swc_i4 *>(p));
+    } else {
+        *p = r;
+    }
+}
+
 } // namespace swc_hip
 
 #define SWC_REQUIRE_INIT()                                                              \

@@ -1,7 +1,8 @@
 // Bandwidth-bound flat kernels: relu_f, vecAdd_f, their fusion, batchedadd_f,
-// matrixTanh_f.  One pass over HBM with 128-bit accesses; every thread issues
-// UNROLL independent 16-byte loads per operand before the first use so that a
-// CU keeps enough bytes in flight to cover HBM latency.
+// matrixTanh_f.  One pass over HBM with 128-bit accesses, one float4 per
+// operand per thread and as many 256-thread workgroups as that takes (the
+// measured optimum on MI355X: deeper per-thread unrolling lowered bandwidth);
+// large tensors use non-temporal accesses.
 #include "common.hpp"
 
 using namespace swc_hip;
@@ -9,7 +10,7 @@ using namespace swc_hip;
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kUnroll = 4;                            // float4 per thread per operand
+constexpr int kUnroll = 1;                            // float4 per thread per operand
 constexpr size_t kBlockElems = (size_t)kThreads * kUnroll * 4;
 
 // (x > 0) ? x : 0 of kernels.h:578, kept as a compare+select: a max() would
@@ -41,7 +42,7 @@ __device__ __forceinline__ float4 apply4(float4 a, float4 b) {
 }
 
 // n4 = number of whole float4; elements [4*n4, n) are the scalar tail, done by block 0.
-template <class Op>
+template <class Op, bool NT>
 __global__ __launch_bounds__(kThreads) void flat_vec4(const float *a, const float *b,
                                                       float *out, size_t n4, size_t n) {
     const float4 *a4 = reinterpret_cast<const float4 *>(a);
@@ -53,14 +54,14 @@ __global__ __launch_bounds__(kThreads) void flat_vec4(const float *a, const floa
     for (int u = 0; u < kUnroll; ++u) {
         const size_t i = base + (size_t)u * kThreads;
         if (i < n4) {
-            va[u] = a4[i];
-            if (Op::kInputs == 2) vb[u] = b4[i];
+            va[u] = ld4<NT>(a4 + i);
+            if (Op::kInputs == 2) vb[u] = ld4<NT>(b4 + i);
         }
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         const size_t i = base + (size_t)u * kThreads;
-        if (i < n4) o4[i] = apply4<Op>(va[u], Op::kInputs == 2 ? vb[u] : va[u]);
+        if (i < n4) st4<NT>(o4 + i, apply4<Op>(va[u], Op::kInputs == 2 ? vb[u] : va[u]));
     }
     if (blockIdx.x == 0) {
         const size_t i = n4 * 4 + threadIdx.x;
@@ -86,7 +87,10 @@ int launch_flat(const char *who, const float *a, const float *b, float *out, siz
         const size_t n4 = n / 4;
         const size_t blocks = (n4 + (size_t)kThreads * kUnroll - 1) / ((size_t)kThreads * kUnroll);
         if (blocks > 0x7fffffffu) return fail(SWC_HIP_EINVAL, "%s: size %zu too large", who, n);
-        flat_vec4<Op><<<(unsigned)blocks, kThreads, 0, stream()>>>(a, b, out, n4, n);
+        if (n * sizeof(float) >= kStreamingBytes)
+            flat_vec4<Op, true><<<(unsigned)blocks, kThreads, 0, stream()>>>(a, b, out, n4, n);
+        else
+            flat_vec4<Op, false><<<(unsigned)blocks, kThreads, 0, stream()>>>(a, b, out, n4, n);
     } else {
         size_t blocks = (n + kThreads - 1) / kThreads;
         if (blocks > 65536) blocks = 65536;

@@ -31,7 +31,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
 
 // VEC = float4s per lane; row length n = 4*n4 with n4 <= 64*VEC.
-template <int VEC>
+template <int VEC, bool NT>
 __global__ __launch_bounds__(kWave *kRowsPerBlock) void softmax_rows_reg(const float *a, float *b, int m, int n4,
                                                                          size_t lda, size_t ldb) {
     const int lane = threadIdx.x & (kWave - 1);
@@ -44,7 +44,7 @@ __global__ __launch_bounds__(kWave *kRowsPerBlock) void softmax_rows_reg(const f
 #pragma unroll
     for (int u = 0; u < VEC; ++u) {
         const int i = lane + u * kWave;
-        v[u] = (i < n4) ? src[i] : make_float4(ninf, ninf, ninf, ninf);
+        v[u] = (i < n4) ? ld4<NT>(src + i) : make_float4(ninf, ninf, ninf, ninf);
     }
     float mx = ninf;
 #pragma unroll
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(kWave *kRowsPerBlock) void softmax_rows_reg(const f
 #pragma unroll
     for (int u = 0; u < VEC; ++u) {
         const int i = lane + u * kWave;
-        if (i < n4) dst[i] = make_float4(v[u].x * inv, v[u].y * inv, v[u].z * inv, v[u].w * inv);
+        if (i < n4) st4<NT>(dst + i, make_float4(v[u].x * inv, v[u].y * inv, v[u].z * inv, v[u].w * inv));
     }
 }
 
@@ -152,10 +152,17 @@ int swc_hip_matrixSoftmax_f(int m, int n, const float *a, int lda, float *b, int
     } else if (vec_ok && n4 <= kWave * 8) {
         const unsigned blocks = ceil_div(m, kRowsPerBlock);
         const dim3 block(kWave * kRowsPerBlock);
-        if (n4 <= kWave * 1) softmax_rows_reg<1><<<blocks, block, 0, s>>>(a, b, m, n4, lda, ldb);
-        else if (n4 <= kWave * 2) softmax_rows_reg<2><<<blocks, block, 0, s>>>(a, b, m, n4, lda, ldb);
-        else if (n4 <= kWave * 4) softmax_rows_reg<4><<<blocks, block, 0, s>>>(a, b, m, n4, lda, ldb);
-        else softmax_rows_reg<8><<<blocks, block, 0, s>>>(a, b, m, n4, lda, ldb);
+        const bool nt = (size_t)m * n * sizeof(float) >= kStreamingBytes;
+#define SWC_SOFTMAX_LAUNCH(V)                                                                       \
+    do {                                                                                            \
+        if (nt) softmax_rows_reg<V, true><<<blocks, block, 0, s>>>(a, b, m, n4, lda, ldb);          \
+        else softmax_rows_reg<V, false><<<blocks, block, 0, s>>>(a, b, m, n4, lda, ldb);            \
+    } while (0)
+        if (n4 <= kWave * 1) SWC_SOFTMAX_LAUNCH(1);
+        else if (n4 <= kWave * 2) SWC_SOFTMAX_LAUNCH(2);
+        else if (n4 <= kWave * 4) SWC_SOFTMAX_LAUNCH(4);
+        else SWC_SOFTMAX_LAUNCH(8);
+#undef SWC_SOFTMAX_LAUNCH
     } else {
         softmax_rows_strided<<<ceil_div(m, kRowsPerBlock), kWave * kRowsPerBlock, 0, s>>>(a, b, m, n, lda, ldb);
     }
