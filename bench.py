@@ -10,7 +10,7 @@ pass of that graph over one batch already resident in HBM.  Prints ONE JSON
 line; `value` is samples/s over exactly K timed steps.
 
 Also in the line:
-  roofline      the dominant kernel (the tiled fp32-MFMA GEMM: both of its
+  roofline      the dominant kernel (the tiled fp32-MFMA GEMM gemm_dma<2,2,2>: both of its
                 launches per step, 4096x784x4096 and 4096x4096x4096), timed
                 with HIP events on the library's stream inside the timed region
   kernels       per-launch times of the headline graph
@@ -207,7 +207,7 @@ def main():
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):   # measured separately under rocprofv3 --pmc; see profiles/
-        traffic = json.load(open(tpath)).get("gemm_tiled<2,2,true>", {}).get("bytes_per_launch")
+        traffic = json.load(open(tpath)).get("gemm_dma<2,2,2>", {}).get("bytes_per_launch")
     out = {
         "metric": "samples/s per graph; TFLOP/s (FC/conv) & GB/s (eltwise) vs MI355X roofline",
         "value": head["samples_per_s"], "unit": "samples/s", "n_gpus": 1, "steps": args.steps,
@@ -218,7 +218,7 @@ def main():
                    "global_batch": head["batch"], "device": rt.device_name()},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS_FP32_MFMA, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_TFLOPS_FP32_MFMA, "traffic": traffic,
-                     "kernel": "gemm_tiled<2,2,true> (both launches per step: 4096x784x4096 and 4096x4096x4096)",
+                     "kernel": "gemm_dma<2,2,2> (both launches per step: 4096x784x4096 and 4096x4096x4096)",
                      "flop_per_launch": flop / len(gemm), "avg_launch_ms": secs * 1e3 / len(gemm)},
         "gpu_ms_per_step": head["gpu_ms"] / args.steps,
         "kernels": head["kernels"],

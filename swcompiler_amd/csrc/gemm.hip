@@ -220,6 +220,7 @@ __global__ __launch_bounds__(kThreads) void gemm_dma(const float *__restrict__ A
 // --------------------------------------------------------------- skinny GEMM
 typedef float v4f __attribute__((ext_vector_type(4)));
 constexpr int kSkinnyMaxWaves = 16;
+constexpr int kSkinnyUnroll = 4;
 
 // v_mfma_f32_16x16x4_f32: A[i][kk] i = l%16, kk = l/16; B[kk][j] j = l%16, kk = l/16;
 // D[i][j] in VGPR v: j = l%16, i = 4*(l/16) + v.
@@ -239,23 +240,30 @@ __global__ __launch_bounds__(64 * kSkinnyMaxWaves) void gemm_skinny(const float 
     const bool col_ok = i < N;   // as B operand, lane's column j = i
     const float *arow = A + (size_t)(row_ok ? row : 0) * lda;
     v4f acc = {0.f, 0.f, 0.f, 0.f};
-    for (int k0 = wave * 32; k0 < K; k0 += waves * 32) {
-        const int k = k0 + q * 8;
-        float a[8], b[8];
-        if (VEC) {   // K % 4 == 0: each float4 is wholly inside or outside
-            const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
-            const float4 lo = (row_ok && k < K) ? *reinterpret_cast<const float4 *>(arow + k) : z;
-            const float4 hi = (row_ok && k + 4 < K) ? *reinterpret_cast<const float4 *>(arow + k + 4) : z;
-            a[0] = lo.x; a[1] = lo.y; a[2] = lo.z; a[3] = lo.w;
-            a[4] = hi.x; a[5] = hi.y; a[6] = hi.z; a[7] = hi.w;
-        } else {
+    // kSkinnyUnroll groups of 32 k per trip: all of a trip's loads are issued
+    // before its first MFMA, so a wavefront keeps 8 KB of A in flight.
+    for (int kbase = wave * 32; kbase < K; kbase += waves * 32 * kSkinnyUnroll) {
+        float a[kSkinnyUnroll][8], b[kSkinnyUnroll][8];
 #pragma unroll
-            for (int s = 0; s < 8; ++s) a[s] = (row_ok && k + s < K) ? arow[k + s] : 0.f;
+        for (int u = 0; u < kSkinnyUnroll; ++u) {
+            const int k = kbase + u * waves * 32 + q * 8;
+            if (VEC) {   // K % 4 == 0: each float4 is wholly inside or outside
+                const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+                const float4 lo = (row_ok && k < K) ? ld4<true>(reinterpret_cast<const float4 *>(arow + k)) : z;
+                const float4 hi = (row_ok && k + 4 < K) ? ld4<true>(reinterpret_cast<const float4 *>(arow + k + 4)) : z;
+                a[u][0] = lo.x; a[u][1] = lo.y; a[u][2] = lo.z; a[u][3] = lo.w;
+                a[u][4] = hi.x; a[u][5] = hi.y; a[u][6] = hi.z; a[u][7] = hi.w;
+            } else {
+#pragma unroll
+                for (int s = 0; s < 8; ++s) a[u][s] = (row_ok && k + s < K) ? arow[k + s] : 0.f;
+            }
+#pragma unroll
+            for (int s = 0; s < 8; ++s) b[u][s] = (col_ok && k + s < K) ? B[(size_t)(k + s) * ldb + i] : 0.f;
         }
 #pragma unroll
-        for (int s = 0; s < 8; ++s) b[s] = (col_ok && k + s < K) ? B[(size_t)(k + s) * ldb + i] : 0.f;
+        for (int u = 0; u < kSkinnyUnroll; ++u)
 #pragma unroll
-        for (int s = 0; s < 8; ++s) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[s], b[s], acc, 0, 0, 0);
+            for (int s = 0; s < 8; ++s) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u][s], b[u][s], acc, 0, 0, 0);
     }
 #pragma unroll
     for (int v = 0; v < 4; ++v) part[wave][4 * q + v][i] = acc[v];

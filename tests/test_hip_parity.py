@@ -338,3 +338,41 @@ def test_error_paths(rt):
     with pytest.raises(SwcHipError):
         rt._check(rt.lib.swc_hip_relu_f(None, a.ptr, 16), "null src")
     assert rt.lib.swc_hip_relu_f(None, None, 0) == 0
+
+
+# ------------------------------------------------- every kernel variant
+# SWC_HIP_GEMM / SWC_HIP_CONV force a tile shape / pipeline variant; the library
+# reads them on every call.  "reg*" = register-staged kernels (the path taken for
+# unaligned shapes and for operands beyond the 2 GiB reach of 32-bit buffer
+# offsets), "TMTN_S" = direct-to-LDS kernels with an S-stage ring.
+@pytest.mark.parametrize("variant", ["reg", "22_2", "22_3", "21_3", "12_3", "11_3", "11_4"])
+def test_gemm_every_variant(rt, oracle, variant, monkeypatch):
+    print("case gemm variant", variant, flush=True)
+    monkeypatch.setenv("SWC_HIP_GEMM", variant)
+    rng = np.random.default_rng(11)
+    for m, k, n in [(300, 200, 260), (128, 64, 128), (70, 36, 132), (64, 4, 64)]:
+        a = rng.integers(-8, 9, (m, k)).astype(np.float32)
+        b = rng.integers(-8, 9, (k, n)).astype(np.float32)
+        bias = rng.integers(-8, 9, n).astype(np.float32)
+        want = np.maximum((a.astype(np.int64) @ b.astype(np.int64) + bias.astype(np.int64)), 0).astype(np.float32)
+        got = rt.fcbias(*up(rt, a, b, bias), relu=True).numpy()
+        assert_bit_exact(got, want, f"integer gemm {m}x{k}x{n} variant {variant}")
+    a = rng.uniform(0, 1, (257, 516)).astype(np.float32)
+    b = rng.uniform(0, 1, (516, 260)).astype(np.float32)
+    assert strict_rel_err(rt.matrixMatrixMul(*up(rt, a, b)).numpy(), oracle.matrixMatrixMul(a, b)) < TOL
+
+
+@pytest.mark.parametrize("variant", ["reg22", "reg21", "reg12", "reg11", "22_2", "21_3", "12_3", "11_3", "11_4"])
+def test_conv_every_variant(rt, oracle, variant, monkeypatch):
+    print("case conv variant", variant, flush=True)
+    monkeypatch.setenv("SWC_HIP_CONV", variant)
+    rng = np.random.default_rng(12)
+    for idims, fdims, strides, pads in [((2, 9, 10, 8), (40, 3, 3, 8), (1, 1), (1, 1, 1, 1)),
+                                        ((1, 13, 11, 20), (70, 5, 5, 20), (2, 1), (2, 2, 2, 2)),
+                                        ((3, 6, 6, 64), (130, 3, 3, 64), (1, 1), (1, 1, 1, 1))]:
+        x = rng.integers(-4, 5, idims).astype(np.float32)
+        f = rng.integers(-4, 5, fdims).astype(np.float32)
+        b = rng.integers(-4, 5, fdims[0]).astype(np.float32)
+        want = oracle.relu(oracle.conv2d(x, f, b, fdims[1:3], strides, pads))   # exact: integer-valued
+        got = rt.conv2d(*up(rt, x, f, b), fdims[1:3], strides, pads, relu=True).numpy()
+        assert_bit_exact(got, want, f"integer conv {idims} variant {variant}")
