@@ -13,9 +13,12 @@
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <iostream>
+#include <initializer_list>
 #include <random>
 #include <string>
+#include <vector>
 
 template <typename T> inline unsigned load(T *data, size_t size, size_t offset, const std::string &path) {
     std::FILE *f = std::fopen(path.c_str(), "rb");
@@ -71,5 +74,87 @@ inline void accuracy_i(const int *pred, const int *label, int *accum, int m, int
             }
     }
 }
+
+// Record reader of the generated batch loop: a file of `sample_num` records
+// <label><data>, where a label is one byte (ONE_BYTE_AS_INT) or a 4-byte float
+// read as an integer class (FOUR_BYTES_AS_FLOAT), and data elements are bytes or
+// 4-byte floats likewise.  next() fills one mini-batch (label_shape[0] records)
+// and returns false once `epochs` passes over the file are done; a trailing
+// partial batch is dropped.  Same constructor and next()/shift() as the
+// reference's src/codegen/utils/DataLoader.h:56-63.
+#ifndef SWC_BYTES_PROTO_DEFINED
+#define SWC_BYTES_PROTO_DEFINED
+enum BytesProto { ONE_BYTE_AS_INT, FOUR_BYTES_AS_FLOAT };
+#endif
+
+class DataLoader {
+    std::FILE *file_{nullptr};
+    std::string path_;
+    BytesProto labelProto_, dataProto_;
+    size_t epochs_, samples_, batch_, dataPerSample_{1};
+    size_t cursor_{0}, epoch_{0};
+    std::vector<unsigned char> raw_;
+
+    static size_t width(BytesProto p) { return p == ONE_BYTE_AS_INT ? 1 : 4; }
+    void rewindFile() {
+        std::rewind(file_);
+        cursor_ = 0;
+    }
+    template <typename T> static void decode(const unsigned char *src, BytesProto p, size_t n, T *dst) {
+        for (size_t i = 0; i < n; ++i) {
+            if (p == ONE_BYTE_AS_INT) {
+                dst[i] = (T)src[i];
+            } else {
+                float f;
+                std::memcpy(&f, src + 4 * i, 4);
+                dst[i] = (T)f;
+            }
+        }
+    }
+
+  public:
+    DataLoader(const std::string &filename, BytesProto label_proto, BytesProto data_proto, size_t epochs,
+               size_t sample_num, const std::initializer_list<size_t> &label_shape,
+               const std::initializer_list<size_t> &data_shape)
+        : path_(filename), labelProto_(label_proto), dataProto_(data_proto), epochs_(epochs), samples_(sample_num),
+          batch_(*label_shape.begin()) {
+        size_t i = 0;
+        for (size_t d : data_shape)
+            if (i++ > 0) dataPerSample_ *= d;
+        file_ = std::fopen(path_.c_str(), "rb");
+        if (!file_) {
+            std::cout << "Error loading " << path_ << "\n";
+            std::exit(EXIT_FAILURE);
+        }
+        raw_.resize(width(labelProto_) + width(dataProto_) * dataPerSample_);
+    }
+    ~DataLoader() {
+        if (file_) std::fclose(file_);
+    }
+    DataLoader(const DataLoader &) = delete;
+    DataLoader &operator=(const DataLoader &) = delete;
+
+    bool next(int *label_batch, float *data_batch) {
+        if (cursor_ + batch_ > samples_) {
+            if (++epoch_ >= epochs_) return false;
+            rewindFile();
+            if (batch_ > samples_) return false;
+        }
+        if (epoch_ >= epochs_) return false;
+        for (size_t s = 0; s < batch_; ++s) {
+            if (std::fread(raw_.data(), 1, raw_.size(), file_) != raw_.size()) return false;
+            decode(raw_.data(), labelProto_, 1, label_batch + s);
+            decode(raw_.data() + width(labelProto_), dataProto_, dataPerSample_, data_batch + s * dataPerSample_);
+        }
+        cursor_ += batch_;
+        return true;
+    }
+    // skip n mini-batches
+    void shift(size_t n) {
+        const size_t skip = n * batch_;
+        std::fseek(file_, (long)(skip * raw_.size()), SEEK_CUR);
+        cursor_ += skip;
+    }
+};
 
 #endif /* SWC_HOST_UTILS_H_ */

@@ -180,7 +180,49 @@ void Codegen::emitMemAllocs() {
     emitVarDeclarations();
     emitMemAllocations();
     emitTensorAddresses();
+    if (config_.use_dataloader) emitInferDataLoaderInit();
     emitTensorInitializations();
+}
+
+static std::string bracedDims(const std::vector<size_t> &dims) {
+    std::ostringstream os;
+    os << "{";
+    for (size_t i = 0; i < dims.size(); ++i) os << (i ? ", " : "") << dims[i];
+    os << "}";
+    return os.str();
+}
+
+// Reference: src/codegen/Codegen.cpp:930-951.  One epoch over
+// Config::dataloader_samples records of Config::dataloader_src, mini-batch =
+// dim 0 of the label tensor.
+void Codegen::emitInferDataLoaderInit() {
+    TensorNode *label = graph_->getInferLabelNode();
+    TensorNode *data = graph_->getInferDataNode();
+    if (!label || !data) {
+        SWLOG_ERROR << "Config::use_dataloader needs IRGraph::setInferDataNodes(label, data)" << std::endl;
+        std::abort();
+    }
+    auto proto = [](BytesProto p) { return p == ONE_BYTE_AS_INT ? "ONE_BYTE_AS_INT" : "FOUR_BYTES_AS_FLOAT"; };
+    writer_ << "std::string dataloader_infer_source = \"" << config_.dataloader_src << "\";\n";
+    writer_ << "DataLoader loader(dataloader_infer_source, " << proto(config_.label_bytes) << ", "
+            << proto(config_.data_bytes) << ", 1, " << config_.dataloader_samples << ", " << bracedDims(label->getDims())
+            << ", " << bracedDims(data->getDims()) << ");\n";
+    writer_ << "size_t iter = 0;\n\n";
+}
+
+// Reference: src/codegen/Codegen.cpp:815-854.
+void Codegen::emitPrintGraphOutputs() {
+    writer_ << "\nif (iter % " << config_.display << " == 0) {\n";
+    writer_.indentInc();
+    writer_ << "std::cout << \"iterations \" << iter << \"\\n\";\n";
+    for (TensorNode *tn : graph_->getDisplayTensorNodes()) {
+        Tensor *t = tn->getTensor();
+        writer_ << "// " << tn->name() << "\n";
+        writer_ << "printMatrix(" << tensors_name_map_.at(t) << ", " << t->getDim(0) << ", "
+                << (t->getNDim() == 2 ? t->getDim(1) : 1) << ");\n";
+    }
+    writer_.indentDec();
+    writer_ << "}\n";
 }
 
 // Every distinct Tensor gets a name and an offset in the arena of its label's
@@ -277,6 +319,17 @@ void Codegen::emitTensorInitializations() {
 }
 
 void Codegen::emitExecute() {
+    if (config_.use_dataloader) {   // reference: src/codegen/Codegen.cpp:979-993, 1020-1030
+        writer_ << "while(loader.next(" << nameOf(graph_->getInferLabelNode()) << ", "
+                << nameOf(graph_->getInferDataNode()) << ")) {\n";
+        writer_.indentInc();
+        emitFuncCalls();
+        writer_ << "\niter++;\n";
+        if (config_.display > 0) emitPrintGraphOutputs();
+        writer_.indentDec();
+        writer_ << "} //while\n";
+        return;
+    }
     if (config_.time_iters) {
         writer_ << "gettimeofday(&ts, NULL);\n";
         writer_ << "for (size_t swc_iter = 0; swc_iter < " << config_.time_iters << "; swc_iter++) {\n";

@@ -124,8 +124,9 @@ class Codegen {
     virtual void emitExecute();
     virtual void emitFuncCalls();
     virtual void emitMemFree();
-    virtual void emitDataLoaderInit() {}
-    virtual void emitInferDataLoaderInit() {}
+    virtual void emitDataLoaderInit() {}          // training loader: not part of the inference build
+    virtual void emitInferDataLoaderInit();        // `DataLoader loader(...)` + iteration counter
+    void emitPrintGraphOutputs();                  // every Config::display iterations: the display tensors
 
     void codeGenInit();
     void emitMemAllocs();

@@ -119,6 +119,13 @@ void HipCodegen::emitTensorInitializations() {
 }
 
 void HipCodegen::emitExecute() {
+    if (config_.use_dataloader) {
+        // the batch loop of the CPU target; the per-iteration Scatter of the data
+        // tensor and the Gather in front of each host op are ordinary op nodes
+        Codegen::emitExecute();
+        writer_ << "SWC_HIP_CHECK(swc_hip_sync());\n";
+        return;
+    }
     if (config_.time_iters) {
         // one untimed pass (first-touch, code load), then the timed loop
         writer_ << "// warm-up pass\n";

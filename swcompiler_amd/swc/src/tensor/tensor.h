@@ -121,9 +121,6 @@ class Tensor {
         initInfo_.setFilePath(std::move(file));
         initInfo_.setOffset(offset);
     }
-    void setTensorInit(TensorInitType type, const char *file, size_t offset = 0) {
-        setTensorInit(type, std::string(file), offset);
-    }
     void setTensorInit(TensorInitType type, TensorInitInfo info) {
         initType_ = type;
         initInfo_ = std::move(info);

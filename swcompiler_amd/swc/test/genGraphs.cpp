@@ -4,7 +4,8 @@
 // the reference's test/engine/testEngineMLPInfer.cpp.
 //
 //   genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse]
-//   model: mnist8 | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
+//   model: mnist8 | mnist_loader | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
+//   mnist_loader: [batch] is the number of records in mnist_labels_images.bin
 //
 // Every parameter/input tensor is initialised from "<name>.bin" in the
 // directory the generated program runs in; outputs are dumped to "<name>.bin".
@@ -150,6 +151,47 @@ int main(int argc, char **argv) {
         GpT(graph, data0, weight0, bias0, data1, data2, weight1, bias1, data3, data4, top3_t);
         GpO(graph, fc0, tanh0, fc1, softmax, argmax_o, print_o);
         graph->addLogicalOutNodes(data4, top3_t);   // dump the probabilities and the top-3 table
+    } else if (model == "mnist_loader") {
+        // the reference's test/engine/testEngineMLPInfer.cpp: batch loop over a record file,
+        // FCBias -> Tanh -> FCBias -> Softmax -> ArgMax(1) -> Accuracy, counters printed at the end
+        TENSOR(data0, 8, 784);
+        TENSOR(weight0, 784, 512);
+        TENSOR(bias0, 512);
+        INIT(weight0, TensorInitType::FILE, "mlp_weight0.bin");
+        INIT(bias0, TensorInitType::FILE, "mlp_bias0.bin");
+        OP(fc0, MatrixMatrixFCBiasOp);
+        LINKUPPER(fc0, data0, weight0, bias0);
+        TENSOR(data1, 8, 512);
+        LINKUPPER(data1, fc0);
+        OP(tanh0, MatrixTanhOp);
+        LINKUPPER(tanh0, data1);
+        TENSOR(data2, 8, 512);
+        LINKUPPER(data2, tanh0);
+        TENSOR(weight1, 512, 10);
+        TENSOR(bias1, 10);
+        INIT(weight1, TensorInitType::FILE, "mlp_weight1.bin");
+        INIT(bias1, TensorInitType::FILE, "mlp_bias1.bin");
+        OP(fc1, MatrixMatrixFCBiasOp);
+        LINKUPPER(fc1, data2, weight1, bias1);
+        TENSOR(data3, 8, 10);
+        LINKUPPER(data3, fc1);
+        Tensor *labelt = new Tensor({8}, DataType::Int32_t);
+        TensorNode *label = new TensorNode("selected", labelt);
+        OP(softmax, MatrixSoftmaxOp);
+        LINKUPPER(softmax, data3);
+        TENSOR(data4, 8, 10);
+        LINKUPPER(data4, softmax);
+        auto *argmax_o = new OpNode("argmax", new ArgMaxOp(1));
+        argmax_o->exlinkUpperNode(data4);
+        auto *top1_t = new TensorNode("top1", new Tensor({8, 1}, DataType::Int32_t), argmax_o);
+        OP(accuracy_o, AccuracyOp);
+        LINKUPPER(accuracy_o, top1_t, label);
+        auto *accuracy_t = new TensorNode("accur", new Tensor({1, 2}, DataType::Int32_t), accuracy_o);
+        accuracy_t->getTensor()->setTensorInit(TensorInitType::CONSTANT, 0);
+        GpT(graph, data0, weight0, bias0, data1, data2, weight1, bias1, data3, data4, label, top1_t, accuracy_t);
+        GpO(graph, fc0, tanh0, fc1, softmax, argmax_o, accuracy_o);
+        graph->setInferDataNodes(label, data0);
+        graph->addDisplayTensorNodes(accuracy_t);
     } else if (model == "cfg1" || model == "cfg2") {
         const bool wide = model == "cfg2";
         const size_t b = batch ? batch : (wide ? 4096 : 8), hidden = wide ? 4096 : 512;
@@ -233,6 +275,14 @@ int main(int argc, char **argv) {
     config.hip_fusion = !nofuse;
     config.time_iters = iters;
     config.dump_outputs = true;
+    if (model == "mnist_loader") {
+        config.use_dataloader = true;
+        config.dataloader_src = "mnist_labels_images.bin";
+        config.label_bytes = BytesProto::ONE_BYTE_AS_INT;
+        config.data_bytes = BytesProto::FOUR_BYTES_AS_FLOAT;
+        config.dataloader_samples = batch;
+        config.display = batch / 8;   // print once, after the last mini-batch
+    }
     graph->setConfig(config);
 
     Engine engine(graph);

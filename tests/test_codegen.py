@@ -64,9 +64,12 @@ def generate(gen, model, target, workdir, batch=0, iters=0, nofuse=False):
     return code
 
 
-def build_cpu(workdir):
-    if os.path.isdir(REF_UTILS):   # the reference's own image.h / kernels.h
-        cmd = ["g++", "-std=c++11", "-O2", "-w", "-I", REF_UTILS, "Graph.cpp", "-o", "net_cpu.bin"]
+def build_cpu(workdir, with_loader=False, force_compat=False):
+    if os.path.isdir(REF_UTILS) and not force_compat:   # the reference's own image.h / kernels.h (/ DataLoader)
+        cmd = ["g++", "-std=c++11", "-O2", "-w", "-I", REF_UTILS, "Graph.cpp"]
+        if with_loader:
+            cmd.append(os.path.join(REF_UTILS, "utils", "DataLoader.cpp"))
+        cmd += ["-o", "net_cpu.bin"]
     else:
         odir = os.path.join(ROOT, "oracle")
         cmd = ["g++", "-std=c++11", "-O2", "-I", os.path.join(odir, "compat"), "-I", os.path.join(ROOT, "include"),
@@ -186,3 +189,78 @@ def test_mnist8_hip_program_prints_the_reference_labels(gen, tmp_path, golden):
     assert strict_rel_err(prob, golden["mnist8_prob"]) < TOL
     top3 = np.fromfile(os.path.join(tmp_path, "top3_host.bin"), np.int32).reshape(8, 3)
     assert_bit_exact(top3, golden["mnist8_top3"], "dumped top-3")
+
+
+# ------------------------------------------------------ batch loop (dataloader)
+def write_record_file(tmp_path, samples, seed=5):
+    """`samples` records of <1-byte label><784 fp32>; half of the images are the reference's eight
+    MNIST digits (so some predictions are right), the rest noise."""
+    d = os.path.join(ROOT, "tests", "golden", "mnist8")
+    for f in os.listdir(d):
+        shutil.copy(os.path.join(d, f), tmp_path)
+    img8 = np.fromfile(os.path.join(d, "mnist_images_8.bin"), np.float32).reshape(8, 784)
+    lab8 = [5, 0, 4, 1, 9, 2, 1, 3]
+    rng = np.random.default_rng(seed)
+    images, labels = [], []
+    for i in range(samples):
+        if i % 2 == 0:
+            j = int(rng.integers(0, 8))
+            images.append(img8[j])
+            labels.append(lab8[j])
+        else:
+            images.append(rng.uniform(0, 1, 784).astype(np.float32))
+            labels.append(int(rng.integers(0, 10)))
+    with open(os.path.join(tmp_path, "mnist_labels_images.bin"), "wb") as f:
+        for lab, img in zip(labels, images):
+            f.write(bytes([lab]))
+            f.write(np.asarray(img, np.float32).tobytes())
+    return np.stack(images), np.array(labels)
+
+
+def expected_counters(oracle, images, labels):
+    d = os.path.join(ROOT, "tests", "golden", "mnist8")
+    ld = lambda n, shape: np.fromfile(os.path.join(d, n), np.float32).reshape(shape)
+    w0, b0, w1, b1 = ld("mlp_weight0.bin", (784, 512)), ld("mlp_bias0.bin", (512,)), ld("mlp_weight1.bin", (512, 10)), ld("mlp_bias1.bin", (10,))
+    n = (len(images) // 8) * 8
+    prob = oracle.matrixSoftmax(oracle.fcbias(oracle.matrixTanh(oracle.fcbias(images[:n], w0, b0)), w1, b1))
+    right = int((oracle.argMax(prob, 1).ravel() == labels[:n]).sum())
+    return right, n
+
+
+def parse_counters(stdout):
+    lines = stdout.strip().splitlines()
+    assert lines[-2].startswith("iterations"), stdout
+    return tuple(int(v) for v in lines[-1].split())
+
+
+@pytest.mark.parametrize("compat", [False, True])
+def test_batch_loop_cpu_program(gen, oracle, tmp_path, compat):
+    """compat=False: the reference's DataLoader.cpp and kernels (where the reference tree exists);
+    compat=True: this repository's DataLoader (include/swc_host_utils.h) and the oracle."""
+    images, labels = write_record_file(tmp_path, 44)   # 5 mini-batches of 8, 4 records left over
+    code = generate(gen, "mnist_loader", "cpu", tmp_path, 44)
+    assert "while(loader.next(selected, data0))" in code and "DataLoader loader(" in code
+    exe = build_cpu(tmp_path, with_loader=True, force_compat=compat)
+    out = subprocess.run([exe], cwd=tmp_path, check=True, capture_output=True, text=True).stdout
+    assert parse_counters(out) == expected_counters(oracle, images, labels)
+    assert parse_counters(out)[1] == 40 and parse_counters(out)[0] >= 15
+
+
+def test_batch_loop_hip_program_structure(gen, tmp_path):
+    code = generate(gen, "mnist_loader", "hip", tmp_path, 44)
+    body = code[code.index("while(loader.next(selected, data0))"):]
+    # inside the loop: the data batch goes up, the top-1 table comes back, accuracy runs on the host
+    assert body.count("swc_hip_h2d(") == 1 and "swc_hip_h2d(data0_dev, data0" in body
+    assert body.count("swc_hip_d2h(") == 1 and "accuracy_i(top1_host, selected, accur" in body
+    # before the loop: the four parameter uploads
+    assert code[:code.index("while(loader")].count("swc_hip_h2d(") == 4
+    build_hip(tmp_path)
+
+
+@pytest.mark.gpu
+def test_batch_loop_hip_program(gen, oracle, tmp_path):
+    images, labels = write_record_file(tmp_path, 44)
+    generate(gen, "mnist_loader", "hip", tmp_path, 44)
+    exe = build_hip(tmp_path)
+    out = subprocess.run([exe], cwd=tmp_path, check=True, capture_output=True, text=True, timeout=120).stdout
+    assert parse_counters(out) == expected_counters(oracle, images, labels)
