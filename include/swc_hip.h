@@ -119,6 +119,20 @@ int swc_hip_maxpool_argmax_f(const float *input, float *output, int32_t *argmax,
                              const size_t *kernels, const size_t *strides,
                              const size_t *pads);
 
+/* kernels.h:444-493; Codegen.cpp:2038-2044.  NHWC window average: fp32 sum of the
+ * in-bounds taps in scan order divided by kh*kw (padding counts as zeros), bit-exact. */
+int swc_hip_avgpool_f(const float *input, float *output, const size_t *idims,
+                      const size_t *odims, const size_t *kernels,
+                      const size_t *strides, const size_t *pads);
+
+/* kernels.h:519-540; Codegen.cpp:2255-2284.  Axis permutation: output axis a is
+ * input axis shuffle[a], odims[a] = idims[shuffle[a]]; 4 resp. 2 entries per array.
+ * output must not alias input. */
+int swc_hip_transpose4d_f(const float *input, float *output, const size_t *idims,
+                          const size_t *odims, const size_t *shuffle);
+int swc_hip_transpose2d_f(const float *input, float *output, const size_t *idims,
+                          const size_t *odims, const size_t *shuffle);
+
 /* kernels.h:88-103; Codegen.cpp:2352-2354.  Row softmax of A[m,n]. b may alias a. */
 int swc_hip_matrixSoftmax_f(int m, int n, const float *a, int lda, float *b,
                             int ldb);

@@ -133,6 +133,23 @@ class CpuKernels:
                               _dims(kernels), _dims(strides), _dims(pads))
         return out
 
+    def avgpool(self, x, kernels, strides, pads=(0, 0, 0, 0)):
+        x = np.ascontiguousarray(x, np.float32)
+        odims = pool_out_dims(x.shape, kernels, strides, pads)
+        out = np.empty(odims, np.float32)
+        self._fn("avgpool_f")(_fp(x), _fp(out), _dims(x.shape), _dims(odims),
+                              _dims(kernels), _dims(strides), _dims(pads))
+        return out
+
+    def transpose(self, x, shuffle):
+        """out axis a = in axis shuffle[a] (2-D or 4-D)."""
+        x = np.ascontiguousarray(x, np.float32)
+        odims = tuple(x.shape[s] for s in shuffle)
+        out = np.empty(odims, np.float32)
+        fn = self._fn("transpose4d_f" if x.ndim == 4 else "transpose2d_f")
+        fn(_fp(x), _fp(out), _dims(x.shape), _dims(odims), _dims(shuffle))
+        return out
+
     def maxpool_argmax(self, x, kernels, strides, pads=(0, 0, 0, 0)):
         """values + flat NHWC input index of the first maximum (oracle only)."""
         x = np.ascontiguousarray(x, np.float32)

@@ -46,6 +46,16 @@ void ref_maxpoolGrad_f(float *ig, const float *og, const float *i,
                        const size_t *s, const size_t *p) {
     maxpoolGrad_f(ig, og, i, id, od, k, s, p);
 }
+void ref_avgpool_f(const float *i, float *o, const size_t *id, const size_t *od,
+                   const size_t *k, const size_t *s, const size_t *p) {
+    avgpool_f(i, o, id, od, k, s, p);
+}
+void ref_transpose4d_f(const float *i, float *o, const size_t *id, const size_t *od, const size_t *sh) {
+    transpose4d_f(i, o, id, od, sh);
+}
+void ref_transpose2d_f(const float *i, float *o, const size_t *id, const size_t *od, const size_t *sh) {
+    transpose2d_f(i, o, id, od, sh);
+}
 void ref_batchnormalization_f(float *o, const float *i, const float *mean,
                               const float *var, const float *scale,
                               const float *bias, const size_t *id, float eps) {

@@ -182,6 +182,57 @@ void oracle_maxpool_f(const float *input, float *output, const size_t *idims,
                             strides, pads);
 }
 
+// kernels.h:444-493.  Sum of the in-bounds taps in (kx, ky) order, fp32, divided
+// by kernel_h*kernel_w whatever the number of in-bounds taps (so padded borders
+// are averaged as if the padding were zeros).
+void oracle_avgpool_f(const float *input, float *output, const size_t *idims,
+                      const size_t *odims, const size_t *kernels,
+                      const size_t *strides, const size_t *pads) {
+    const Dims4 I(idims), O(odims);
+    const ssize_t kh = kernels[0], kw = kernels[1];
+    const ssize_t sh = strides[0], sw = strides[1];
+    const ssize_t pt = pads[0], pl = pads[1];
+    const float count = (float)(kernels[0] * kernels[1]);
+    for (size_t n = 0; n < I.d0; ++n)
+        for (size_t ox = 0; ox < O.d1; ++ox)
+            for (size_t oy = 0; oy < O.d2; ++oy)
+                for (size_t c = 0; c < I.d3; ++c) {
+                    float sum = 0;
+                    for (ssize_t kx = 0; kx < kh; ++kx) {
+                        const ssize_t ix = (ssize_t)ox * sh - pt + kx;
+                        if (ix < 0 || ix >= (ssize_t)I.d1) continue;
+                        for (ssize_t ky = 0; ky < kw; ++ky) {
+                            const ssize_t iy = (ssize_t)oy * sw - pl + ky;
+                            if (iy < 0 || iy >= (ssize_t)I.d2) continue;
+                            sum += input[I.at(n, ix, iy, c)];
+                        }
+                    }
+                    output[O.at(n, ox, oy, c)] = sum / count;
+                }
+}
+
+// kernels.h:519-540.  out[idx[shuffle[0]], idx[shuffle[1]], ...] = in[idx]:
+// output axis a is input axis shuffle[a].
+void oracle_transpose4d_f(const float *input, float *output, const size_t *idims,
+                          const size_t *odims, const size_t *shuffle) {
+    const Dims4 I(idims), O(odims);
+    size_t idx[4];
+    for (idx[0] = 0; idx[0] < I.d0; ++idx[0])
+        for (idx[1] = 0; idx[1] < I.d1; ++idx[1])
+            for (idx[2] = 0; idx[2] < I.d2; ++idx[2])
+                for (idx[3] = 0; idx[3] < I.d3; ++idx[3])
+                    output[O.at(idx[shuffle[0]], idx[shuffle[1]], idx[shuffle[2]], idx[shuffle[3]])] =
+                        input[I.at(idx[0], idx[1], idx[2], idx[3])];
+}
+
+void oracle_transpose2d_f(const float *input, float *output, const size_t *idims,
+                          const size_t *odims, const size_t *shuffle) {
+    size_t idx[2];
+    for (idx[0] = 0; idx[0] < idims[0]; ++idx[0])
+        for (idx[1] = 0; idx[1] < idims[1]; ++idx[1])
+            output[idx[shuffle[0]] * odims[1] + idx[shuffle[1]]] = input[idx[0] * idims[1] + idx[1]];
+}
+
 // kernels.h:496-517.  var[c]+epsilon is an fp32 add; std::pow(float,double)
 // promotes, so everything after it is double arithmetic, rounded to fp32 once
 // on the store: ((in-mean) -> double) * pow(.) * scale + bias.

@@ -196,6 +196,64 @@ __global__ __launch_bounds__(kThreads) void maxpool_scalar(const float *__restri
     }
 }
 
+// avgpool_f (kernels.h:444-493): fp32 sum of the in-bounds taps in (ky, kx) scan
+// order, divided by kh*kw (IEEE division) — the same operations in the same
+// order as the reference, so the result is bit-exact.
+template <bool NT>
+__global__ __launch_bounds__(kThreads) void avgpool_vec4(const float *__restrict__ in, float *__restrict__ out,
+                                                         PoolGeom g, size_t total4) {
+    const unsigned quads = g.C / 4;
+    const size_t step = (size_t)gridDim.x * kThreads;
+    const float4 *i4 = reinterpret_cast<const float4 *>(in);
+    const float count = (float)(g.kh * g.kw);
+    for (size_t o = (size_t)blockIdx.x * kThreads + threadIdx.x; o < total4; o += step) {
+        const unsigned cq = (unsigned)(o % quads);
+        size_t r = o / quads;
+        const int ox = (int)(r % g.OW);
+        r /= g.OW;
+        const int oy = (int)(r % g.OH);
+        const int n = (int)(r / g.OH);
+        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int ky = 0; ky < g.kh; ++ky) {
+            const int iy = oy * g.sh - g.pt + ky;
+            if (iy < 0 || iy >= g.H) continue;
+            for (int kx = 0; kx < g.kw; ++kx) {
+                const int ix = ox * g.sw - g.pl + kx;
+                if (ix < 0 || ix >= g.W) continue;
+                const float4 v = ld4<NT>(i4 + (((size_t)n * g.H + iy) * g.W + ix) * quads + cq);
+                sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+            }
+        }
+        st4<NT>(reinterpret_cast<float4 *>(out) + o,
+                make_float4(sum.x / count, sum.y / count, sum.z / count, sum.w / count));
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void avgpool_scalar(const float *__restrict__ in, float *__restrict__ out,
+                                                           PoolGeom g, size_t total) {
+    const size_t step = (size_t)gridDim.x * kThreads;
+    const float count = (float)(g.kh * g.kw);
+    for (size_t o = (size_t)blockIdx.x * kThreads + threadIdx.x; o < total; o += step) {
+        const int c = (int)(o % g.C);
+        size_t r = o / g.C;
+        const int ox = (int)(r % g.OW);
+        r /= g.OW;
+        const int oy = (int)(r % g.OH);
+        const int n = (int)(r / g.OH);
+        float sum = 0.f;
+        for (int ky = 0; ky < g.kh; ++ky) {
+            const int iy = oy * g.sh - g.pt + ky;
+            if (iy < 0 || iy >= g.H) continue;
+            for (int kx = 0; kx < g.kw; ++kx) {
+                const int ix = ox * g.sw - g.pl + kx;
+                if (ix < 0 || ix >= g.W) continue;
+                sum += in[(((size_t)n * g.H + iy) * g.W + ix) * g.C + c];
+            }
+        }
+        out[o] = sum / count;
+    }
+}
+
 // blocks such that blocks*kThreads is a multiple of `quads`
 unsigned quad_stable_blocks(size_t total4, unsigned quads, unsigned max_blocks) {
     unsigned a = quads, b = kThreads;
@@ -311,6 +369,40 @@ int swc_hip_maxpool_argmax_f(const float *input, float *output, int32_t *argmax,
     SWC_REQUIRE_INIT();
     return launch_pool<true, false>("swc_hip_maxpool_argmax_f", input, output, argmax, idims, odims, kernels, strides,
                                     pads, nullptr, nullptr, nullptr, nullptr, 0.f);
+}
+
+int swc_hip_avgpool_f(const float *input, float *output, const size_t *idims, const size_t *odims,
+                      const size_t *kernels, const size_t *strides, const size_t *pads) {
+    SWC_REQUIRE_INIT();
+    const char *who = "swc_hip_avgpool_f";
+    if (!idims || !odims || !kernels || !strides || !pads) return fail(SWC_HIP_EINVAL, "%s: null shape array", who);
+    if (check_dims4(who, idims) || check_dims4(who, odims)) return SWC_HIP_EINVAL;
+    if (odims[0] != idims[0] || odims[3] != idims[3])
+        return fail(SWC_HIP_EINVAL, "%s: output batch/channels differ from input", who);
+    if (kernels[0] == 0 || kernels[1] == 0 || strides[0] == 0 || strides[1] == 0 || kernels[0] > 4096 ||
+        kernels[1] > 4096 || strides[0] > 4096 || strides[1] > 4096 || pads[0] > 4096 || pads[1] > 4096)
+        return fail(SWC_HIP_EINVAL, "%s: bad kernel/stride/pad", who);
+    const size_t in_total = idims[0] * idims[1] * idims[2] * idims[3];
+    const size_t total = odims[0] * odims[1] * odims[2] * odims[3];
+    if (total == 0) return SWC_HIP_OK;
+    SWC_ARG(input && output);
+    PoolGeom g{(int)idims[0], (int)idims[1], (int)idims[2], (int)idims[3], (int)odims[1], (int)odims[2],
+               (int)kernels[0], (int)kernels[1], (int)strides[0], (int)strides[1], (int)pads[0], (int)pads[1]};
+    if (idims[3] % 4 == 0 && aligned16(input) && aligned16(output)) {
+        const size_t total4 = total / 4;
+        size_t blocks = (total4 + kThreads - 1) / kThreads;
+        if (blocks > (size_t)num_cus() * 128) blocks = (size_t)num_cus() * 128;
+        if (in_total * sizeof(float) >= kStreamingBytes)
+            avgpool_vec4<true><<<(unsigned)blocks, kThreads, 0, stream()>>>(input, output, g, total4);
+        else
+            avgpool_vec4<false><<<(unsigned)blocks, kThreads, 0, stream()>>>(input, output, g, total4);
+    } else {
+        size_t blocks = (total + kThreads - 1) / kThreads;
+        if (blocks > 8192) blocks = 8192;
+        avgpool_scalar<<<(unsigned)blocks, kThreads, 0, stream()>>>(input, output, g, total);
+    }
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
 }
 
 int swc_hip_batchnormReluMaxpool_f(float *output, const float *input, const float *mean, const float *var,

@@ -21,7 +21,8 @@ EXPORTS = [
     "swc_hip_set_stream", "swc_hip_device_name", "swc_hip_timer_begin", "swc_hip_timer_end",
     "swc_hip_timer_elapsed_ms", "swc_hip_event_record", "swc_hip_event_elapsed_ms", "swc_hip_matrixMatrixMul_f", "swc_hip_batchedadd_f", "swc_hip_relu_f",
     "swc_hip_vecAdd_f", "swc_hip_conv2d_f", "swc_hip_batchnormalization_f", "swc_hip_maxpool_f",
-    "swc_hip_maxpool_argmax_f", "swc_hip_matrixSoftmax_f", "swc_hip_matrixTanh_f", "swc_hip_argMax_i",
+    "swc_hip_maxpool_argmax_f", "swc_hip_avgpool_f", "swc_hip_transpose4d_f", "swc_hip_transpose2d_f",
+    "swc_hip_matrixSoftmax_f", "swc_hip_matrixTanh_f", "swc_hip_argMax_i",
     "swc_hip_matrixMatrixFCBias_f", "swc_hip_vecAddRelu_f", "swc_hip_batchnormRelu_f",
     "swc_hip_batchnormReluMaxpool_f", "swc_hip_conv2dFused_f",
 ]
@@ -71,6 +72,9 @@ def load_library():
         "swc_hip_batchnormalization_f": (i32, [vp, vp, vp, vp, vp, vp, szp, f32]),
         "swc_hip_maxpool_f": (i32, [vp, vp, szp, szp, szp, szp, szp]),
         "swc_hip_maxpool_argmax_f": (i32, [vp, vp, vp, szp, szp, szp, szp, szp]),
+        "swc_hip_avgpool_f": (i32, [vp, vp, szp, szp, szp, szp, szp]),
+        "swc_hip_transpose4d_f": (i32, [vp, vp, szp, szp, szp]),
+        "swc_hip_transpose2d_f": (i32, [vp, vp, szp, szp, szp]),
         "swc_hip_matrixSoftmax_f": (i32, [i32, i32, vp, i32, vp, i32]),
         "swc_hip_matrixTanh_f": (i32, [i32, i32, vp, i32, vp, i32]),
         "swc_hip_argMax_i": (i32, [vp, vp, i32, i32, i32]),
@@ -290,6 +294,21 @@ class SwcHip:
         out = out if out is not None else self.empty(odims)
         self._check(self.lib.swc_hip_maxpool_f(x.ptr, out.ptr, _dims(x.shape), _dims(odims), _dims(kernels),
                                                _dims(strides), _dims(pads)), "maxpool_f")
+        return out
+
+    def avgpool(self, x, kernels, strides, pads=(0, 0, 0, 0), out=None):
+        odims = pool_out_dims(x.shape, kernels, strides, pads)
+        out = out if out is not None else self.empty(odims)
+        self._check(self.lib.swc_hip_avgpool_f(x.ptr, out.ptr, _dims(x.shape), _dims(odims), _dims(kernels),
+                                               _dims(strides), _dims(pads)), "avgpool_f")
+        return out
+
+    def transpose(self, x, shuffle, out=None):
+        """out axis a = in axis shuffle[a] (2-D or 4-D)."""
+        odims = tuple(x.shape[s] for s in shuffle)
+        out = out if out is not None else self.empty(odims)
+        fn = self.lib.swc_hip_transpose4d_f if len(x.shape) == 4 else self.lib.swc_hip_transpose2d_f
+        self._check(fn(x.ptr, out.ptr, _dims(x.shape), _dims(odims), _dims(shuffle)), "transpose_f")
         return out
 
     def maxpool_argmax(self, x, kernels, strides, pads=(0, 0, 0, 0)):

@@ -441,6 +441,24 @@ void Codegen::emitFuncCall(OpNode *op) {
                 << arrayDef(nm + "_pads", pool->getPads());
         writer_ << "maxpool_f(" << nameOf(in(0)) << ", " << nameOf(out(0)) << ", " << nm << "_inDims, " << nm
                 << "_outDims, " << nm << "_filterSizes, " << nm << "_strides, " << nm << "_pads);\n";
+    } else if (type == "AveragePool") {   // Codegen.cpp:2020-2044
+        auto *pool = static_cast<AvgPoolOp *>(op->getOp());
+        writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims()) << arrayDef(nm + "_outDims", T(out(0))->getDims())
+                << arrayDef(nm + "_filterSizes", pool->getKernels()) << arrayDef(nm + "_strides", pool->getStrides())
+                << arrayDef(nm + "_pads", pool->getPads());
+        writer_ << "avgpool_f(" << nameOf(in(0)) << ", " << nameOf(out(0)) << ", " << nm << "_inDims, " << nm
+                << "_outDims, " << nm << "_filterSizes, " << nm << "_strides, " << nm << "_pads);\n";
+    } else if (type == "Transpose") {   // Codegen.cpp:2255-2284 (which hard-codes the shuffle {1,0}; the op's own is used here)
+        auto *tr = static_cast<TransposeOp *>(op->getOp());
+        const int nd = T(in(0))->getNDim();
+        if ((nd != 2 && nd != 4) || (int)tr->getShuffle().size() != nd) {
+            SWLOG_ERROR << "Transpose " << nm << ": only 2-D and 4-D tensors with a full shuffle" << std::endl;
+            std::abort();
+        }
+        writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims()) << arrayDef(nm + "_outDims", T(out(0))->getDims())
+                << arrayDef(nm + "_shuffle", tr->getShuffle());
+        writer_ << (nd == 2 ? "transpose2d_f(" : "transpose4d_f(") << nameOf(in(0)) << ", " << nameOf(out(0)) << ", "
+                << nm << "_inDims, " << nm << "_outDims, " << nm << "_shuffle);\n";
     } else if (type == "ArgMax") {   // Codegen.cpp:2372-2385
         const int topK = static_cast<ArgMaxOp *>(op->getOp())->getTopK();
         writer_ << "argMax_i(" << nameOf(in(0)) << ", " << nameOf(out(0)) << ", " << T(in(0))->getDim(0) << ", "

@@ -267,6 +267,25 @@ void HipCodegen::emitHipCall(OpNode *op) {
         writer_ << "SWC_HIP_CHECK(swc_hip_maxpool_f(" << nameOf(in(0)) << ", " << nameOf(out(0)) << ", " << nm
                 << "_inDims, " << nm << "_outDims, " << nm << "_filterSizes, " << nm << "_strides, " << nm
                 << "_pads));\n";
+    } else if (type == "AveragePool") {
+        auto *pool = static_cast<AvgPoolOp *>(op->getOp());
+        writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims()) << arrayDef(nm + "_outDims", T(out(0))->getDims())
+                << arrayDef(nm + "_filterSizes", pool->getKernels()) << arrayDef(nm + "_strides", pool->getStrides())
+                << arrayDef(nm + "_pads", pool->getPads());
+        writer_ << "SWC_HIP_CHECK(swc_hip_avgpool_f(" << nameOf(in(0)) << ", " << nameOf(out(0)) << ", " << nm
+                << "_inDims, " << nm << "_outDims, " << nm << "_filterSizes, " << nm << "_strides, " << nm
+                << "_pads));\n";
+    } else if (type == "Transpose") {
+        auto *tr = static_cast<TransposeOp *>(op->getOp());
+        const int nd = T(in(0))->getNDim();
+        if ((nd != 2 && nd != 4) || (int)tr->getShuffle().size() != nd) {
+            SWLOG_ERROR << "Transpose " << nm << ": only 2-D and 4-D tensors with a full shuffle" << std::endl;
+            std::abort();
+        }
+        writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims()) << arrayDef(nm + "_outDims", T(out(0))->getDims())
+                << arrayDef(nm + "_shuffle", tr->getShuffle());
+        writer_ << "SWC_HIP_CHECK(swc_hip_" << (nd == 2 ? "transpose2d_f(" : "transpose4d_f(") << nameOf(in(0)) << ", "
+                << nameOf(out(0)) << ", " << nm << "_inDims, " << nm << "_outDims, " << nm << "_shuffle));\n";
     } else if (type == "ArgMax") {
         const int topK = static_cast<ArgMaxOp *>(op->getOp())->getTopK();
         writer_ << "SWC_HIP_CHECK(swc_hip_argMax_i(" << nameOf(in(0)) << ", " << nameOf(out(0)) << ", "

@@ -71,6 +71,16 @@ void MaxPoolOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *shape) {
     const auto idims = dimsOfParent(node, 0);
     shape->setShape(windowedShape(idims, kernels_, strides_, pads_, idims[3]));
 }
+void AvgPoolOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *shape) {
+    const auto idims = dimsOfParent(node, 0);
+    shape->setShape(windowedShape(idims, kernels_, strides_, pads_, idims[3]));
+}
+void TransposeOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *shape) {
+    const auto idims = dimsOfParent(node, 0);
+    std::vector<size_t> odims;
+    for (size_t s : shuffle_) odims.push_back(idims.at(s));
+    shape->setShape(odims);
+}
 std::string Conv2dOp::getOpInfo() {
     return Op::getOpInfo() + "kernels: " + join(kernels_) + "\\nstrides: " + join(strides_) + "\\npads: " +
            join(pads_) + "\\n";

@@ -115,6 +115,27 @@ class MaxPoolOp : public Op {
     std::string getOpInfo() override;
     void outTensorShapeGen(OpNode *node, size_t index, TensorShape *shape) override;
 };
+class AvgPoolOp : public Op {           // sum of in-bounds taps / (kh*kw)
+    std::vector<size_t> kernels_, strides_, pads_;
+
+  public:
+    AvgPoolOp() : Op(DL_OP, 1, 1, "AveragePool") {}
+    AvgPoolOp(std::vector<size_t> &kernels, std::vector<size_t> &strides, std::vector<size_t> &pads)
+        : Op(DL_OP, 1, 1, "AveragePool"), kernels_(kernels), strides_(strides), pads_(pads) {}
+    std::vector<size_t> getPads() const { return pads_; }
+    std::vector<size_t> getKernels() const { return kernels_; }
+    std::vector<size_t> getStrides() const { return strides_; }
+    void outTensorShapeGen(OpNode *node, size_t index, TensorShape *shape) override;
+};
+// Axis permutation: output axis a is input axis shuffle[a] (NCHW2NHWC, NHWC2NCHW, {1,0}).
+class TransposeOp : public Op {
+    std::vector<size_t> shuffle_;
+
+  public:
+    TransposeOp(const std::initializer_list<size_t> &shuffle) : Op(DL_OP, 1, 1, "Transpose"), shuffle_(shuffle) {}
+    std::vector<size_t> getShuffle() const { return shuffle_; }
+    void outTensorShapeGen(OpNode *node, size_t index, TensorShape *shape) override;
+};
 class BatchNormalizationOp : public Op {   // parents: input, scale, bias, mean, var
     float epsilon_;
 

@@ -227,7 +227,8 @@ bool DeviceMemoryLoweringPass::runsOnGpu(const std::string &t) {
     static const std::set<std::string> gpu = {
         "MatrixMatrixMul", "MatrixVectorAdd", "BatchedAdd", "MatrixMatrixFCBias", "MatrixMatrixFCBiasRelu",
         "Reshape", "MatrixTanh", "MatrixSoftmax", "ElementAdd", "ElementAddRelu", "Relu", "Dropout",
-        "Conv2d", "Conv2dWithActivation", "Conv2dBatchNorm", "MaxPool", "BatchNormalization",
+        "Conv2d", "Conv2dWithActivation", "Conv2dBatchNorm", "MaxPool", "AveragePool", "Transpose",
+        "BatchNormalization",
         "BatchNormalizationRelu", "ArgMax"};
     return gpu.count(t) != 0;
 }

@@ -4,7 +4,7 @@
 // the reference's test/engine/testEngineMLPInfer.cpp.
 //
 //   genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse]
-//   model: mnist8 | mnist_loader | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
+//   model: mnist8 | mnist_loader | nchw | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
 //   mnist_loader: [batch] is the number of records in mnist_labels_images.bin
 //
 // Every parameter/input tensor is initialised from "<name>.bin" in the
@@ -192,6 +192,40 @@ int main(int argc, char **argv) {
         GpO(graph, fc0, tanh0, fc1, softmax, argmax_o, accuracy_o);
         graph->setInferDataNodes(label, data0);
         graph->addDisplayTensorNodes(accuracy_t);
+    } else if (model == "nchw") {
+        // an NCHW-trained block at the import boundary: data NCHW -> NHWC, filter OIHW -> OHWI
+        // (the reference's importer inserts TransposeOp(NCHW2NHWC) the same way,
+        // src/importer/Caffe2Importer.cpp:220-229), conv + relu + average pool, result back to NCHW
+        const size_t b = batch ? batch : 2;
+        auto *x = new TensorNode("x", new Tensor({b, 8, 12, 12}, DataType::Float_t, layout_nchw));
+        auto *w = new TensorNode("w", new Tensor({16, 8, 3, 3}, DataType::Float_t, layout_nchw));
+        auto *cb = new TensorNode("cb", new Tensor({16}));
+        fromFile(x->getTensor(), "x");
+        fromFile(w->getTensor(), "w");
+        fromFile(cb->getTensor(), "cb");
+        auto *tx = new OpNode("x_to_nhwc", new TransposeOp(NCHW2NHWC));
+        tx->exlinkUpperNode(x);
+        auto *xh = new TensorNode("x_nhwc", new Tensor({0}), tx);
+        auto *tw = new OpNode("w_to_ohwi", new TransposeOp(NCHW2NHWC));
+        tw->exlinkUpperNode(w);
+        auto *wh = new TensorNode("w_ohwi", new Tensor({0}), tw);
+        vector<size_t> kernels{3, 3}, strides{1, 1}, pads{1, 1, 1, 1};
+        DYOP(conv0, Conv2dOp, kernels, strides, pads);
+        LINKUPPER(conv0, xh, wh, cb);
+        auto *y = new TensorNode("conv0_out", new Tensor({0}), conv0);
+        graph->pushTensorNode(x, w, cb, xh, wh, y);
+        graph->pushOpNode(tx, tw, conv0);
+        graph->initTensorNodes();
+        TensorNode *h = lazyUnary(graph, "relu0", new ReluOp(), y);
+        vector<size_t> pk{2, 2}, ps{2, 2}, pp{0, 0, 0, 0};
+        auto *ap = new OpNode("avgpool0", new AvgPoolOp(pk, ps, pp));
+        ap->exlinkUpperNode(h);
+        auto *pooled = new TensorNode("avgpool0_out", new Tensor({0}), ap);
+        auto *back = new OpNode("to_nchw", new TransposeOp(NHWC2NCHW));
+        back->exlinkUpperNode(pooled);
+        out = new TensorNode("y_nchw", new Tensor({0}), back);
+        graph->pushTensorNode(pooled, out);
+        graph->pushOpNode(ap, back);
     } else if (model == "cfg1" || model == "cfg2") {
         const bool wide = model == "cfg2";
         const size_t b = batch ? batch : (wide ? 4096 : 8), hidden = wide ? 4096 : 512;

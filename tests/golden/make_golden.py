@@ -76,6 +76,18 @@ def main():
         og = np.arange(1, y.size + 1, dtype=F).reshape(y.shape)
         g[f"pool_{tag}_scatter"] = ref.maxpoolGrad(x, og, kernels, strides, pads)
 
+    # avgpool / transpose (reuse the pool inputs without the non-finite values)
+    for tag, (idims, kernels, strides, pads) in pools.items():
+        x = rng.standard_normal(idims).astype(F)
+        g[f"avg_{tag}_x"] = x
+        g[f"avg_{tag}_y"] = ref.avgpool(x, kernels, strides, pads)
+    x = rng.standard_normal((2, 3, 5, 7)).astype(F)
+    g["tr4_x"] = x
+    for tag, sh in {"nchw2nhwc": (0, 2, 3, 1), "nhwc2nchw": (0, 3, 1, 2), "rev": (3, 2, 1, 0)}.items():
+        g[f"tr4_{tag}_y"] = ref.transpose(x, sh)
+    g["tr2_x"] = rng.standard_normal((5, 9)).astype(F)
+    g["tr2_y"] = ref.transpose(g["tr2_x"], (1, 0))
+
     # batchnorm
     for tag, idims in {"a": (2, 5, 5, 8), "b": (1, 3, 4, 130)}.items():
         c = idims[3]

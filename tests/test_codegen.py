@@ -264,3 +264,42 @@ def test_batch_loop_hip_program(gen, oracle, tmp_path):
     exe = build_hip(tmp_path)
     out = subprocess.run([exe], cwd=tmp_path, check=True, capture_output=True, text=True, timeout=120).stdout
     assert parse_counters(out) == expected_counters(oracle, images, labels)
+
+
+# ------------------------------------------- layout ops at an NCHW import boundary
+def nchw_block_expected(oracle, x, w, cb):
+    xh, wh = oracle.transpose(x, (0, 2, 3, 1)), oracle.transpose(w, (0, 2, 3, 1))
+    y = oracle.relu(oracle.conv2d(xh, wh, cb, (3, 3), (1, 1), (1, 1, 1, 1)))
+    return oracle.transpose(oracle.avgpool(y, (2, 2), (2, 2)), (0, 3, 1, 2))
+
+
+def nchw_inputs(tmp_path):
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((2, 8, 12, 12)).astype(np.float32)
+    w = (rng.standard_normal((16, 8, 3, 3)) / 8).astype(np.float32)
+    cb = (rng.standard_normal(16) * 0.1).astype(np.float32)
+    for name, a in (("x", x), ("w", w), ("cb", cb)):
+        a.tofile(os.path.join(tmp_path, name + ".bin"))
+    return x, w, cb
+
+
+def test_nchw_block_cpu_program(gen, oracle, tmp_path):
+    x, w, cb = nchw_inputs(tmp_path)
+    code = generate(gen, "nchw", "cpu", tmp_path, 2)
+    assert code.count("transpose4d_f(") == 3 and "avgpool_f(" in code
+    subprocess.check_call([build_cpu(tmp_path)], cwd=tmp_path, stdout=subprocess.DEVNULL)
+    want = nchw_block_expected(oracle, x, w, cb)
+    got = np.fromfile(os.path.join(tmp_path, "y_nchw.bin"), np.float32).reshape(want.shape)
+    assert want.shape == (2, 16, 6, 6)
+    assert_bit_exact(got, want, "nchw block")
+
+
+@pytest.mark.gpu
+def test_nchw_block_hip_program(gen, oracle, tmp_path):
+    x, w, cb = nchw_inputs(tmp_path)
+    code = generate(gen, "nchw", "hip", tmp_path, 2)
+    assert code.count("swc_hip_transpose4d_f(") == 3 and "swc_hip_avgpool_f(" in code and "swc_hip_conv2dFused_f(" in code
+    subprocess.run([build_hip(tmp_path)], cwd=tmp_path, check=True, timeout=120, stdout=subprocess.DEVNULL)
+    want = nchw_block_expected(oracle, x, w, cb)
+    got = np.fromfile(os.path.join(tmp_path, "y_nchw_host.bin"), np.float32).reshape(want.shape)
+    assert rel_err(got, want) < TOL

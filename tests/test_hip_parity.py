@@ -273,6 +273,36 @@ def test_maxpool_golden(rt, golden, tag):
     assert_bit_exact(scat.reshape(x.shape), golden[f"pool_{tag}_scatter"], "chosen tap golden")
 
 
+@pytest.mark.parametrize("idims,k,s,p", POOLS)
+def test_avgpool_bit_exact(rt, oracle, idims, k, s, p):
+    x = np.random.default_rng(sum(idims)).standard_normal(idims).astype(np.float32)
+    assert_bit_exact(rt.avgpool(rt.upload(x), k, s, p).numpy(), oracle.avgpool(x, k, s, p), "avgpool")
+
+
+@pytest.mark.parametrize("shape,shuffle", [((2, 3, 5, 7), (0, 2, 3, 1)), ((2, 3, 5, 7), (0, 3, 1, 2)),
+                                           ((2, 3, 5, 7), (3, 2, 1, 0)), ((4, 64, 33, 35), (0, 2, 3, 1)),
+                                           ((4, 33, 35, 64), (0, 3, 1, 2)), ((3, 4, 5, 6), (1, 0, 2, 3)),
+                                           ((2, 40, 3, 50), (2, 3, 0, 1)), ((5, 9), (1, 0)), ((130, 257), (1, 0)),
+                                           ((7, 11), (0, 1)), ((1, 224, 224, 3), (0, 3, 1, 2))])
+def test_transpose_bit_exact(rt, oracle, shape, shuffle):
+    print("case transpose", shape, shuffle, flush=True)
+    x = np.random.default_rng(len(shape)).standard_normal(shape).astype(np.float32)
+    got = rt.transpose(rt.upload(x), shuffle).numpy()
+    assert_bit_exact(got, oracle.transpose(x, shuffle), "transpose vs oracle")
+    assert_bit_exact(got, np.ascontiguousarray(np.transpose(x, shuffle)), "transpose vs numpy")
+
+
+def test_transpose_golden(rt, golden):
+    x = rt.upload(golden["tr4_x"])
+    for tag, sh in {"nchw2nhwc": (0, 2, 3, 1), "nhwc2nchw": (0, 3, 1, 2), "rev": (3, 2, 1, 0)}.items():
+        assert_bit_exact(rt.transpose(x, sh).numpy(), golden[f"tr4_{tag}_y"], tag)
+    assert_bit_exact(rt.transpose(rt.upload(golden["tr2_x"]), (1, 0)).numpy(), golden["tr2_y"], "2d")
+    for tag in ("k2", "k3s3", "k3s2p1", "odd"):
+        ksp = [int(v) for v in golden[f"pool_{tag}_ksp"]]
+        got = rt.avgpool(rt.upload(golden[f"avg_{tag}_x"]), ksp[:2], ksp[2:4], ksp[4:]).numpy()
+        assert_bit_exact(got, golden[f"avg_{tag}_y"], "avgpool golden " + tag)
+
+
 def test_bn_relu_maxpool_fused_equals_sequence(rt, oracle):
     rng = np.random.default_rng(77)
     x = rng.standard_normal((2, 16, 16, 64)).astype(np.float32)

@@ -46,6 +46,21 @@ def test_maxpool_values_and_chosen_tap(oracle, golden, tag):
     assert_bit_exact(scat.reshape(x.shape), golden[f"pool_{tag}_scatter"], "argmax scatter")
 
 
+@pytest.mark.parametrize("tag", ["k2", "k3s3", "k3s2p1", "odd"])
+def test_avgpool(oracle, golden, tag):
+    ksp = [int(v) for v in golden[f"pool_{tag}_ksp"]]
+    y = oracle.avgpool(golden[f"avg_{tag}_x"], ksp[:2], ksp[2:4], ksp[4:])
+    assert_bit_exact(y, golden[f"avg_{tag}_y"], "avgpool")
+
+
+def test_transpose(oracle, golden):
+    x = golden["tr4_x"]
+    for tag, sh in {"nchw2nhwc": (0, 2, 3, 1), "nhwc2nchw": (0, 3, 1, 2), "rev": (3, 2, 1, 0)}.items():
+        assert_bit_exact(oracle.transpose(x, sh), golden[f"tr4_{tag}_y"], tag)
+        assert_bit_exact(oracle.transpose(x, sh), np.transpose(x, sh), tag + " vs numpy")
+    assert_bit_exact(oracle.transpose(golden["tr2_x"], (1, 0)), golden["tr2_y"], "2d")
+
+
 @pytest.mark.parametrize("tag", ["a", "b"])
 def test_batchnorm(oracle, golden, tag):
     g = lambda k: golden[f"bn_{tag}_{k}"]
