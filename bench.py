@@ -14,6 +14,8 @@ Also in the line:
                 launches per step, 4096x784x4096 and 4096x4096x4096), timed
                 with HIP events on the library's stream inside the timed region
   kernels       per-launch times of the headline graph
+  graph_replay  the same K steps replayed as one HIP graph per step (no per-kernel
+                events in the loop): what a launch-bound small graph gains
   configs       the other synthetic configurations (samples/s and, per kernel,
                 TFLOP/s or GB/s with the fraction of the MI355X peak)
   cpu_baseline  the reference's own CPU kernels (oracle/_ref, g++ -std=c++11 -O2,
@@ -149,8 +151,20 @@ def run_config(rt, graphs, cfg, steps, warmup):
         timed.log = log
         all_rows.append(timed.results())
     rows = merge_rows(all_rows)
+    # the same step as one HIP graph: K replays, nothing else in the loop
+    handle = rt.capture(lambda: graphs.run(cfg, rt, dt, fused=True, ws=ws))
+    for _ in range(3):
+        rt.graph_launch(handle)
+    rt.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        rt.graph_launch(handle)
+    rt.sync()
+    graph_wall = time.perf_counter() - t0
+    rt.graph_destroy(handle)
     return dict(batch=batch, wall_s=wall, gpu_ms=gpu_ms, ms_per_step=wall * 1e3 / steps,
-                samples_per_s=batch * steps / wall, kernels=rows)
+                samples_per_s=batch * steps / wall, kernels=rows,
+                graph_replay=dict(ms_per_step=graph_wall * 1e3 / steps, samples_per_s=batch * steps / graph_wall))
 
 
 def cpu_baseline(graphs, rows=64):
@@ -221,6 +235,7 @@ def main():
                      "kernel": "gemm_dma<2,2,2> (both launches per step: 4096x784x4096 and 4096x4096x4096)",
                      "flop_per_launch": flop / len(gemm), "avg_launch_ms": secs * 1e3 / len(gemm)},
         "gpu_ms_per_step": head["gpu_ms"] / args.steps,
+        "graph_replay": head["graph_replay"],
         "kernels": head["kernels"],
     }
     if not args.headline_only:
@@ -229,7 +244,8 @@ def main():
             steps = max(5, min(args.steps, 20))
             r = run_config(rt, graphs, cfg, steps, max(2, min(args.warmup, 5)))
             others[f"cfg{cfg}"] = dict(batch=r["batch"], samples_per_s=r["samples_per_s"], ms_per_step=r["ms_per_step"],
-                                       gpu_ms_per_step=r["gpu_ms"] / steps, kernels=r["kernels"])
+                                       gpu_ms_per_step=r["gpu_ms"] / steps, graph_replay=r["graph_replay"],
+                                       kernels=r["kernels"])
         out["configs"] = others
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(graphs, args.cpu_rows)

@@ -69,6 +69,17 @@ float swc_hip_timer_elapsed_ms(void);
 int swc_hip_event_record(int slot);
 float swc_hip_event_elapsed_ms(int first, int second);
 
+/* HIP graphs: the ops issued between begin and end are recorded instead of run;
+ * launch replays them with a single submission (the launch-bound small graphs —
+ * batch-8 MLP, LeNet — spend most of their time between kernels otherwise).
+ * Run the sequence once eagerly first (kernels configure themselves on first
+ * use).  h2d/d2h/sync and the timers must not be called while capturing.  The
+ * recorded launches keep the pointers and shapes they were issued with. */
+int swc_hip_graph_begin(void);
+int swc_hip_graph_end(void **graph_out);      /* returns an executable graph handle */
+int swc_hip_graph_launch(void *graph);        /* async on the stream */
+int swc_hip_graph_destroy(void *graph);
+
 /* ---- ops: same arguments as the reference's CPU kernels ---- */
 
 /* kernels.h:41-56; emitted at Codegen.cpp:1334-1337 with lda=k, ldb=n, ldc=n.

@@ -24,6 +24,7 @@ struct State {
     hipEvent_t t0 = nullptr, t1 = nullptr;
     float last_ms = -1.f;
     hipEvent_t slots[kEventSlots] = {};
+    bool capturing = false;
     char arch[64] = "";
 } g;
 
@@ -201,6 +202,45 @@ int swc_hip_timer_end(void) {
 }
 
 float swc_hip_timer_elapsed_ms(void) { return g.last_ms; }
+
+// ---- HIP graphs: capture the op sequence once, replay it with one launch ----
+int swc_hip_graph_begin(void) {
+    SWC_REQUIRE_INIT();
+    if (g.capturing) return fail(SWC_HIP_EINVAL, "swc_hip_graph_begin: a capture is already open");
+    SWC_HIP_TRY(hipStreamBeginCapture(stream(), hipStreamCaptureModeRelaxed));
+    g.capturing = true;
+    return SWC_HIP_OK;
+}
+
+int swc_hip_graph_end(void **graph_out) {
+    SWC_REQUIRE_INIT();
+    SWC_ARG(graph_out);
+    if (!g.capturing) return fail(SWC_HIP_EINVAL, "swc_hip_graph_end: no capture is open");
+    g.capturing = false;
+    hipGraph_t graph = nullptr;
+    SWC_HIP_TRY(hipStreamEndCapture(stream(), &graph));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return fail(SWC_HIP_ERUNTIME, "swc_hip_graph_end: hipGraphInstantiate -> %s", hipGetErrorString(e));
+    *graph_out = (void *)exec;
+    return SWC_HIP_OK;
+}
+
+int swc_hip_graph_launch(void *graph) {
+    SWC_REQUIRE_INIT();
+    SWC_ARG(graph);
+    SWC_HIP_TRY(hipGraphLaunch((hipGraphExec_t)graph, stream()));
+    return SWC_HIP_OK;
+}
+
+int swc_hip_graph_destroy(void *graph) {
+    SWC_REQUIRE_INIT();
+    if (!graph) return SWC_HIP_OK;
+    SWC_HIP_TRY(hipStreamSynchronize(stream()));
+    SWC_HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph));
+    return SWC_HIP_OK;
+}
 
 int swc_hip_event_record(int slot) {
     SWC_REQUIRE_INIT();

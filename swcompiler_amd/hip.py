@@ -19,7 +19,8 @@ EXPORTS = [
     "swc_hip_init", "swc_hip_shutdown", "swc_hip_malloc", "swc_hip_free", "swc_hip_h2d", "swc_hip_d2h",
     "swc_hip_d2d", "swc_hip_fill_f", "swc_hip_sync", "swc_hip_last_error", "swc_hip_stream",
     "swc_hip_set_stream", "swc_hip_device_name", "swc_hip_timer_begin", "swc_hip_timer_end",
-    "swc_hip_timer_elapsed_ms", "swc_hip_event_record", "swc_hip_event_elapsed_ms", "swc_hip_matrixMatrixMul_f", "swc_hip_batchedadd_f", "swc_hip_relu_f",
+    "swc_hip_timer_elapsed_ms", "swc_hip_event_record", "swc_hip_event_elapsed_ms", "swc_hip_graph_begin",
+    "swc_hip_graph_end", "swc_hip_graph_launch", "swc_hip_graph_destroy", "swc_hip_matrixMatrixMul_f", "swc_hip_batchedadd_f", "swc_hip_relu_f",
     "swc_hip_vecAdd_f", "swc_hip_conv2d_f", "swc_hip_batchnormalization_f", "swc_hip_maxpool_f",
     "swc_hip_maxpool_argmax_f", "swc_hip_avgpool_f", "swc_hip_transpose4d_f", "swc_hip_transpose2d_f",
     "swc_hip_matrixSoftmax_f", "swc_hip_matrixTanh_f", "swc_hip_argMax_i",
@@ -64,6 +65,10 @@ def load_library():
         "swc_hip_timer_elapsed_ms": (f32, []),
         "swc_hip_event_record": (i32, [i32]),
         "swc_hip_event_elapsed_ms": (f32, [i32, i32]),
+        "swc_hip_graph_begin": (i32, []),
+        "swc_hip_graph_end": (i32, [C.POINTER(vp)]),
+        "swc_hip_graph_launch": (i32, [vp]),
+        "swc_hip_graph_destroy": (i32, [vp]),
         "swc_hip_matrixMatrixMul_f": (i32, [i32, i32, i32, vp, i32, vp, i32, vp, i32]),
         "swc_hip_batchedadd_f": (i32, [vp, vp, vp, sz, sz]),
         "swc_hip_relu_f": (i32, [vp, vp, sz]),
@@ -207,6 +212,23 @@ class SwcHip:
         if ms < 0:
             raise SwcHipError("swc_hip_event_elapsed_ms failed: " + self.lib.swc_hip_last_error().decode())
         return ms
+
+    def capture(self, fn):
+        """Records the ops `fn()` issues into a HIP graph; returns a handle for graph_launch()."""
+        self._check(self.lib.swc_hip_graph_begin(), "swc_hip_graph_begin")
+        try:
+            fn()
+        finally:
+            handle = C.c_void_p()
+            rc = self.lib.swc_hip_graph_end(C.byref(handle))
+        self._check(rc, "swc_hip_graph_end")
+        return handle
+
+    def graph_launch(self, handle):
+        self._check(self.lib.swc_hip_graph_launch(handle), "swc_hip_graph_launch")
+
+    def graph_destroy(self, handle):
+        self._check(self.lib.swc_hip_graph_destroy(handle), "swc_hip_graph_destroy")
 
     # -- ops (device in, device out) -------------------------------------
     def matrixMatrixMul(self, a, b, out=None):

@@ -172,6 +172,7 @@ class HipCodegen : public Codegen {
     void dispatchOpNode(OpNode *op) override;
     void emitHipCall(OpNode *op);
     void emitTransfer(OpNode *op, bool toDevice);
+    void emitDeviceOpsOnly();   // the op sequence without transfers and host ops (what a HIP graph records)
 };
 
 } // namespace codegen

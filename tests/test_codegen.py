@@ -57,8 +57,8 @@ def write_inputs(cfg, t, workdir):
         t[k].tofile(os.path.join(workdir, stem + ".bin"))
 
 
-def generate(gen, model, target, workdir, batch=0, iters=0, nofuse=False):
-    args = [gen, model, target, str(batch), str(iters)] + (["nofuse"] if nofuse else [])
+def generate(gen, model, target, workdir, batch=0, iters=0, nofuse=False, graph=False):
+    args = [gen, model, target, str(batch), str(iters)] + (["nofuse"] if nofuse else []) + (["graph"] if graph else [])
     code = subprocess.run(args, cwd=workdir, check=True, capture_output=True, text=True).stdout
     assert open(os.path.join(workdir, "Graph.cpp")).read() == code
     return code
@@ -303,3 +303,21 @@ def test_nchw_block_hip_program(gen, oracle, tmp_path):
     want = nchw_block_expected(oracle, x, w, cb)
     got = np.fromfile(os.path.join(tmp_path, "y_nchw_host.bin"), np.float32).reshape(want.shape)
     assert rel_err(got, want) < TOL
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("graph", [False, True])
+def test_timed_hip_program(gen, oracle, tmp_path, graph):
+    """Config::time_iters (and Config::hip_graph): the program still produces the right output and
+    prints a per-iteration time."""
+    t = graphs.make_inputs(3, 8)
+    write_inputs(3, t, tmp_path)
+    code = generate(gen, "cfg3", "hip", tmp_path, 8, iters=20, graph=graph)
+    assert ("swc_hip_graph_launch(swc_graph)" in code) == graph
+    exe = build_hip(tmp_path)
+    out = subprocess.run([exe], cwd=tmp_path, check=True, capture_output=True, text=True, timeout=120).stdout
+    ms = float(re.search(r"swc_time_ms_per_iter ([0-9.eE+-]+)", out).group(1))
+    assert 0 < ms < 50
+    want = oracle_run(oracle, "cfg3", 3, t)
+    got = np.fromfile(os.path.join(tmp_path, "softmax_out_host.bin"), np.float32).reshape(want.shape)
+    assert strict_rel_err(got, want) < 5 * TOL

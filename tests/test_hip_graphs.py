@@ -132,3 +132,33 @@ def test_full_size_properties(rt, oracle):
     sub["x"] = t4["x"][[0, 31]]
     want = graphs.run(4, oracle, sub, fused=False)
     assert np.max(np.abs(got[[0, 31]] - want)) / np.max(np.abs(want)) < TOL  # chain: max norm, see test_cfg4_conv_block
+
+
+@pytest.mark.parametrize("cfg,batch", [(1, None), (3, 16), (4, 2)])
+def test_hip_graph_replay_equals_eager(rt, cfg, batch):
+    """One step captured into a HIP graph; every replay — with eager work and
+    synchronisations of the program's own in between — must reproduce the eager
+    result bit for bit (same kernels, same launch parameters)."""
+    t = graphs.make_inputs(cfg, batch)
+    dt = to_dev(rt, t)
+    ws = {}
+    out = graphs.run(cfg, rt, dt, fused=True, ws=ws)   # eager pass: sets up kernels, allocates outputs
+    eager = out.numpy().copy()
+    handle = rt.capture(lambda: graphs.run(cfg, rt, dt, fused=True, ws=ws))
+    scratch = rt.upload(np.ones(1000, np.float32))
+    for i in range(4):
+        rt.lib.swc_hip_fill_f(out.ptr, 0.0, out.size)          # wipe the output so a no-op replay would show
+        rt.relu(scratch, out=scratch)                            # unrelated eager work between replays
+        rt.sync()
+        rt.graph_launch(handle)
+        assert_bit_exact(out.numpy(), eager, f"replay {i}")
+    # new input values through the same graph
+    x2 = (t["x"] * np.float32(0.5)).astype(np.float32)
+    rt._check(rt.lib.swc_hip_h2d(dt["x"].ptr, x2.ctypes.data, x2.nbytes), "h2d")
+    rt.graph_launch(handle)
+    replay2 = out.numpy().copy()
+    t2 = dict(dt)
+    eager2 = graphs.run(cfg, rt, t2, fused=True, ws=ws).numpy()
+    assert_bit_exact(replay2, eager2, "replay on new input")
+    assert not np.array_equal(replay2, eager)
+    rt.graph_destroy(handle)
