@@ -315,6 +315,130 @@ int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGe
     return SWC_HIP_OK;
 }
 
+// ------------------------------------------------------------ small direct conv
+// First layers (iC = 1 or 3, a handful of output channels) have K = kH*kW*iC of
+// a few dozen: far too short for the MFMA pipeline, and iC % 4 != 0 rules out
+// 128-bit gathers.  One thread per output pixel keeps all oC accumulators in
+// registers, walks the taps in the reference's (ky, kx, ci) order and adds
+// fl(x*w) with separate fp32 multiply and add starting from the bias — the very
+// operation sequence of conv2d_f, so this path is bit-exact.  The filter is
+// staged in LDS as [k][oC] and read as wavefront-uniform broadcasts.
+constexpr int kDirectMaxK = 128;
+constexpr int kDirectMaxOC = 32;
+
+template <int OCQ>   // output channels rounded up to 4*OCQ
+__global__ __launch_bounds__(256) void conv_direct(const float *__restrict__ in, const float *__restrict__ filt,
+                                                   const float *__restrict__ bias, float *__restrict__ out,
+                                                   ConvGeom g, Epilogue ep) {
+#pragma clang fp contract(off)   // x*w and the add must round separately, as in the reference's -O2 x86 code
+    constexpr int OCP = 4 * OCQ;
+    __shared__ __align__(16) float w[kDirectMaxK * OCP];
+    __shared__ float bsh[OCP], mean_sh[OCP], slope_sh[OCP], beta_sh[OCP];
+    __shared__ float stage[256 * OCP];
+    const int K = g.K, OC = g.OC;
+    for (int i = threadIdx.x; i < K * OCP; i += 256) {
+        const int k = i / OCP, oc = i - k * OCP;
+        w[i] = oc < OC ? filt[(size_t)oc * K + k] : 0.f;
+    }
+    const bool bn = ep.bn_mean != nullptr;
+    if (threadIdx.x < OCP) {
+        const int oc = threadIdx.x;
+        bsh[oc] = oc < OC ? bias[oc] : 0.f;
+        if (bn && oc < OC) {
+            mean_sh[oc] = ep.bn_mean[oc];
+            slope_sh[oc] = (float)((double)ep.bn_scale[oc] / sqrt((double)(ep.bn_var[oc] + ep.eps)));
+            beta_sh[oc] = ep.bn_bias[oc];
+        }
+    }
+    __syncthreads();
+    const int m = blockIdx.x * 256 + threadIdx.x;
+    const bool active = m < g.M;
+    const int mm = active ? m : 0;
+    const int ox = mm % g.OW;
+    const int t = mm / g.OW;
+    const int oy = t % g.OH;
+    const int img = t / g.OH;
+    float acc[OCP];
+#pragma unroll
+    for (int oc = 0; oc < OCP; ++oc) acc[oc] = bsh[oc];
+    // For a fixed ky the taps (kx, ci) are L = kw*C consecutive floats of one input
+    // row (NHWC).  They are fetched eight at a time — all loads of a group issued
+    // before the first multiply — so the pixel's ~K dependent load latencies
+    // shrink to K/8.
+    const int L = g.kw * g.C;
+    const int ix0 = ox * g.sw - g.pl;
+    for (int ky = 0; ky < g.kh; ++ky) {
+        const int iy = oy * g.sh - g.pt + ky;
+        if ((unsigned)iy >= (unsigned)g.H) continue;   // whole kernel row outside: skipped, as in the reference
+        const float *row = in + (((long)img * g.H + iy) * g.W + ix0) * g.C;
+        const int kbase = ky * L;
+        for (int j0 = 0; j0 < L; j0 += 8) {
+            float xv[8];
+            bool ok[8];
+            int kx = j0 / g.C, ci = j0 - kx * g.C;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                ok[u] = j0 + u < L && (unsigned)(ix0 + kx) < (unsigned)g.W;
+                xv[u] = ok[u] ? row[j0 + u] : 0.f;
+                if (++ci == g.C) {
+                    ci = 0;
+                    ++kx;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (!ok[u]) continue;
+                const float x = xv[u];
+                const float4 *wk = reinterpret_cast<const float4 *>(&w[(kbase + j0 + u) * OCP]);
+#pragma unroll
+                for (int q = 0; q < OCQ; ++q) {
+                    const float4 wv = wk[q];
+                    acc[4 * q + 0] += x * wv.x;
+                    acc[4 * q + 1] += x * wv.y;
+                    acc[4 * q + 2] += x * wv.z;
+                    acc[4 * q + 3] += x * wv.w;
+                }
+            }
+        }
+    }
+    // Results go through LDS as the [pixel][oC] block they form in the output, so
+    // that the global stores are contiguous across the workgroup (a thread's own
+    // oC values are only 4*oC bytes apart from its neighbour's).
+    if (active) {
+#pragma unroll
+        for (int oc = 0; oc < OCP; ++oc) {
+            if (oc >= OC) break;
+            float v = acc[oc];
+            if (bn) v = fmaf(v - mean_sh[oc], slope_sh[oc], beta_sh[oc]);
+            if (ep.relu) v = (v > 0.f) ? v : 0.f;
+            stage[threadIdx.x * OC + oc] = v;
+        }
+    }
+    __syncthreads();
+    const int first = blockIdx.x * 256;
+    const int pixels = (g.M - first < 256) ? (g.M - first) : 256;
+    float *o = out + (size_t)first * OC;
+    for (int i = threadIdx.x; i < pixels * OC; i += 256) o[i] = stage[i];
+}
+
+int launch_conv_direct(const float *in, const float *filt, const float *bias, float *out, const ConvGeom &g,
+                       const Epilogue &ep) {
+    const unsigned blocks = ceil_div((size_t)g.M, 256);
+    const int ocq = (g.OC + 3) / 4;
+    switch (ocq) {
+    case 1: conv_direct<1><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
+    case 2: conv_direct<2><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
+    case 3: conv_direct<3><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
+    case 4: conv_direct<4><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
+    case 5: conv_direct<5><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
+    case 6: conv_direct<6><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
+    case 7: conv_direct<7><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
+    default: conv_direct<8><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
+    }
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
+}
+
 template <int TM, int TN>
 int launch_conv(bool vec, const float *in, const float *filt, float *out, const ConvGeom &g, const Epilogue &ep) {
     using T = Tile<TM, TN, true>;
@@ -375,6 +499,8 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
             if (!strcmp(force, "11_4")) return launch_conv_dma<1, 1, 4>(input, filter, output, g, in_bytes, filt_bytes, ep);
         }
     }
+    if (!(force && !strncmp(force, "reg", 3)) && g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0)
+        return launch_conv_direct(input, filter, bias, output, g, ep);
     if (dma_ok) {
         // 64x128 tiles once they fill the chip (wide layers), 64x64 otherwise: the
         // layers here are tens of microseconds long, many small tiles balance the

@@ -406,3 +406,20 @@ def test_conv_every_variant(rt, oracle, variant, monkeypatch):
         want = oracle.relu(oracle.conv2d(x, f, b, fdims[1:3], strides, pads))   # exact: integer-valued
         got = rt.conv2d(*up(rt, x, f, b), fdims[1:3], strides, pads, relu=True).numpy()
         assert_bit_exact(got, want, f"integer conv {idims} variant {variant}")
+
+
+@pytest.mark.parametrize("idims,fdims,strides,pads", [((4, 28, 28, 1), (20, 5, 5, 1), (1, 1), (0, 0, 0, 0)),
+                                                      ((2, 9, 9, 3), (4, 3, 3, 3), (1, 1), (1, 1, 1, 1)),
+                                                      ((1, 17, 13, 3), (32, 5, 3, 3), (2, 1), (2, 1, 2, 1)),
+                                                      ((3, 8, 8, 2), (7, 7, 7, 1 + 1), (3, 3), (3, 3, 3, 3))])
+def test_small_direct_conv_is_bit_exact(rt, oracle, idims, fdims, strides, pads):
+    """First-layer shapes (iC not a multiple of 4, K <= 128, oC <= 32) run the direct kernel, which
+    performs the reference's own sequence of fp32 multiplies and adds per output."""
+    rng = np.random.default_rng(sum(idims) + sum(fdims))
+    x = rng.standard_normal(idims).astype(np.float32)
+    f = rng.standard_normal(fdims).astype(np.float32)
+    b = rng.standard_normal(fdims[0]).astype(np.float32)
+    want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
+    dx, df, db = up(rt, x, f, b)
+    assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy(), want, "direct conv")
+    assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True).numpy(), oracle.relu(want), "direct conv + relu")
