@@ -127,6 +127,35 @@ void EliminationPass::run() {
     _graph->updateTopology();
 }
 
+// -------------------------------------------------------- transpose cancelling
+void ElimTransposePass::run() {
+    for (int i = 0; i < _graph->opNodeNum(); ++i) {
+        OpNode *first = _graph->getOpNode(i);
+        auto *t1 = dynamic_cast<TransposeOp *>(first->getOp());
+        if (!t1 || first->parentNum() != 1 || first->childNum() != 1) continue;
+        IRNode *source = first->getParentNode(0);
+        IRNode *mid = first->getChildNode(0);
+        const std::vector<size_t> a = t1->getShuffle();
+        std::vector<IRNode *> readers(mid->getChildNodes());
+        for (IRNode *r : readers) {
+            if (r->nodeType() != OP_NODE) continue;
+            auto *second = static_cast<OpNode *>(r);
+            auto *t2 = dynamic_cast<TransposeOp *>(second->getOp());
+            if (!t2 || second->childNum() != 1) continue;
+            const std::vector<size_t> b = t2->getShuffle();
+            bool inverse = a.size() == b.size();
+            for (size_t k = 0; inverse && k < b.size(); ++k) inverse = b[k] < a.size() && a[b[k]] == k;
+            if (!inverse) continue;
+            IRNode *result = second->getChildNode(0);
+            std::vector<IRNode *> users(result->getChildNodes());
+            for (IRNode *u : users) result->replaceUseKeepOrder(u, source);
+            ++cancelled_;
+        }
+    }
+    _graph->findInOut();
+    _graph->updateTopology();
+}
+
 // -------------------------------------------------------------------- fusion
 namespace {
 

@@ -4,6 +4,7 @@
 //   LoweringPass             Op::lowering on marked nodes            (src/pass/LoweringPass.h:34-59)
 //   RenamingNodePass         C-identifier-safe unique node names     (src/pass/RenamingNodePass.h:23-83)
 //   EliminationPass          dead-node removal from the output marks (src/pass/EliminationPass.cpp:34-154)
+//   ElimTransposePass        cancels inverse transpose pairs         (src/pass/ElimTransposePass.h:23-88)
 //   HipFusionPass            NEW: chains -> one fused libswc_hip call
 //   DeviceMemoryLoweringPass NEW: places compute on GPU 0, inserts host<->device transfer nodes
 #ifndef SWC_PASSES_H_
@@ -55,6 +56,18 @@ class EliminationPass : public OptimizePass {
   public:
     explicit EliminationPass(IRGraph *graph) : OptimizePass(graph) {}
     void run() override;
+};
+
+// Transpose(a) followed by Transpose(b) with a[b[i]] == i is the identity: the
+// readers of the second result are rewired to the first operand (the pair itself
+// is left for EliminationPass).  Reference: src/pass/ElimTransposePass.h:23-88.
+class ElimTransposePass : public OptimizePass {
+    int cancelled_{0};
+
+  public:
+    explicit ElimTransposePass(IRGraph *graph) : OptimizePass(graph) {}
+    void run() override;
+    int cancelledCount() const { return cancelled_; }
 };
 
 // Rewrites, wherever the intermediate tensor has a single consumer and is not a

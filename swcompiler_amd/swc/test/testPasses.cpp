@@ -1,0 +1,203 @@
+// Self-checking unit tests of the graph IR and the passes (no code is generated).
+// Exit status 0 = all checks passed; prints the failing check otherwise.
+#include <cstdlib>
+#include <iostream>
+
+#include "SWC.h"
+
+using namespace swc;
+using namespace swc::op;
+using namespace swc::pass;
+using namespace std;
+
+static int failures = 0;
+#define CHECK(cond)                                                                  \
+    do {                                                                             \
+        if (!(cond)) {                                                               \
+            cerr << __FILE__ << ":" << __LINE__ << ": CHECK failed: " #cond << endl; \
+            ++failures;                                                              \
+        }                                                                            \
+    } while (0)
+
+static int countOps(IRGraph *g, const string &type) {
+    int n = 0;
+    for (int i = 0; i < g->opNodeNum(); ++i) n += g->getOpNode(i)->getOp()->getOpName() == type;
+    return n;
+}
+
+static void testTopologyAndShapes() {
+    TENSOR(x, 4, 10, 10, 3);
+    TENSOR(f, 8, 3, 3, 3);
+    TENSOR(b, 8);
+    vector<size_t> k{3, 3}, s{2, 2}, p{1, 1, 1, 1};
+    DYOP(conv, Conv2dOp, k, s, p);
+    LINKUPPER(conv, x, f, b);
+    auto *y = new TensorNode("y", new Tensor({0}), conv);
+    vector<size_t> pk{2, 2}, ps{2, 2}, pp{0, 0, 0, 0};
+    DYOP(pool, MaxPoolOp, pk, ps, pp);
+    LINKUPPER(pool, y);
+    auto *z = new TensorNode("z", new Tensor({0}), pool);
+    G(g);
+    GpT(g, x, f, b, y, z);
+    GpO(g, conv, pool);
+    g->initTensorNodes();
+    g->findInOut();
+    g->updateTopology();
+    // (10 + 1 + 1 - 3) / 2 + 1 = 5 ; pooled (5 - 2) / 2 + 1 = 2
+    CHECK((y->getDims() == vector<size_t>{4, 5, 5, 8}));
+    CHECK((z->getDims() == vector<size_t>{4, 2, 2, 8}));
+    CHECK(y->getTensor()->getMemLayoutTag() == "nhwc");
+    CHECK(g->inNodeNum() == 3 && g->outNodeNum() == 1 && g->getOutNode(0) == z);
+    CHECK(g->topologyNum() == 5 && conv->topologyId() == 1 && z->topologyId() == 4);
+    CHECK(g->getNodeByName("pool") == pool && g->getNodeByName("nope") == nullptr);
+    IRGraph *c = g->clone();
+    CHECK(c->tensorNodeNum() == 5 && c->opNodeNum() == 2 && c->topologyNum() == 5);
+    CHECK(c->getTensorNode(0) != x && c->getTensorNode(0)->getTensor() != x->getTensor());
+    auto *cconv = static_cast<OpNode *>(c->getNodeByName("conv"));
+    CHECK(cconv->parentNum() == 3 && cconv->getParentNode(1)->name() == "f");
+}
+
+static void testLoweringAndRenaming() {
+    TENSOR(x, 8, 4, 4, 2);   // rank 4: FC views it as [8, 32]
+    TENSOR(w, 32, 16);
+    TENSOR(b, 16);
+    OP(fc, MatrixMatrixFCBiasOp);
+    LINKUPPER(fc, x, w, b);
+    TENSOR(y, 8, 16);
+    LINKUPPER(y, fc);
+    G(g);
+    GpT(g, x, w, b, y);
+    GpO(g, fc);
+    g->findInOut();
+    g->updateTopology();
+    Config cpu;
+    g->setConfig(cpu);
+    Engine e(g);
+    e.compile();
+    CHECK(countOps(g, "MatrixMatrixFCBias") == 0 && countOps(g, "MatrixMatrixMul") == 1);
+    CHECK(countOps(g, "MatrixVectorAdd") == 1 && countOps(g, "Reshape") == 1);
+    auto *mm = static_cast<OpNode *>(g->getNodeByName("fc_mm"));
+    CHECK(mm && mm->getParentNode(0)->name() == "x_reshape" && mm->getParentNode(1) == w);
+    CHECK(static_cast<TensorNode *>(mm->getParentNode(0))->getDims() == (vector<size_t>{8, 32}));
+    CHECK(g->getNodeByName("fc_mm_out") != nullptr && y->getParentNode(0)->name() == "fc_add");
+    CHECK(y->getLabel()->getIsOut() == 1);
+
+    UniqueName un;
+    CHECK(un("a/b.c-d") == "a_b_c_d" && un("a_b_c_d") == "a_b_c_d1" && un("a_b_c_d") == "a_b_c_d2");
+}
+
+static void testFusionAndPlacement() {
+    TENSOR(x, 2, 8, 8, 4);
+    TENSOR(f, 8, 3, 3, 4);
+    TENSOR(cb, 8);
+    x_Tensor->setTensorInit(TensorInitType::FILE, "x.bin");
+    f_Tensor->setTensorInit(TensorInitType::FILE, "f.bin");
+    cb_Tensor->setTensorInit(TensorInitType::ZERO);
+    vector<size_t> k{3, 3}, s{1, 1}, p{1, 1, 1, 1};
+    DYOP(conv, Conv2dOp, k, s, p);
+    LINKUPPER(conv, x, f, cb);
+    TENSOR(c, 2, 8, 8, 8);
+    LINKUPPER(c, conv);
+    TensorNode *bnp[4];
+    const char *names[4] = {"scale", "bias", "mean", "var"};
+    for (int i = 0; i < 4; ++i) {
+        bnp[i] = new TensorNode(names[i], new Tensor({8}));
+        bnp[i]->getTensor()->setTensorInit(TensorInitType::CONSTANT, 1);
+    }
+    DYOP(bn, BatchNormalizationOp, 1e-5f);
+    LINKUPPER(bn, c, bnp[0], bnp[1], bnp[2], bnp[3]);
+    TENSOR(n, 2, 8, 8, 8);
+    LINKUPPER(n, bn);
+    OP(relu, ReluOp);
+    LINKUPPER(relu, n);
+    TENSOR(r, 2, 8, 8, 8);
+    LINKUPPER(r, relu);
+    auto *print = new OpNode("print", new DebugOp());
+    print->exlinkUpperNode(r);
+    G(g);
+    GpT(g, x, f, cb, c, bnp[0], bnp[1], bnp[2], bnp[3], n, r);
+    GpO(g, conv, bn, relu, print);
+    g->findInOut();
+    g->updateTopology();
+    Config hip;
+    hip.hip = true;
+    g->setConfig(hip);
+    Engine e(g);
+    e.compile();
+    CHECK(countOps(g, "Conv2dBatchNorm") == 1 && countOps(g, "Conv2d") == 0);
+    CHECK(countOps(g, "BatchNormalization") == 0 && countOps(g, "Relu") == 0);
+    auto *fused = static_cast<OpNode *>(g->getNodeByName("conv"));
+    CHECK(fused && fused->parentNum() == 7 && static_cast<Conv2dBatchNormOp *>(fused->getOp())->hasRelu());
+    CHECK(fused->getParentNode(0)->name() == "x_dev" && fused->getParentNode(3)->name() == "scale_dev");
+    CHECK(fused->getLabel()->getDeviceLabel().type == DeviceType::GPU);
+    CHECK(countOps(g, "Scatter") == 7 && countOps(g, "Gather") == 1);
+    for (int i = 0; i < g->opNodeNum(); ++i)
+        if (g->getOpNode(i)->getOp()->getOpName() == "Scatter") CHECK(g->getOpNode(i)->isRunOnce());
+    // the host op reads the gathered twin, the device tensor keeps its GPU label
+    CHECK(print->getParentNode(0)->name() == "r_host" && r->getLabel()->getDeviceLabel().type == DeviceType::GPU);
+    CHECK(print->getLabel()->getDeviceLabel().type == DeviceType::CPU);
+}
+
+static void testElimination() {
+    TENSOR(x, 2, 3, 4, 5);
+    auto *t1 = new OpNode("t1", new TransposeOp(NCHW2NHWC));
+    t1->exlinkUpperNode(x);
+    auto *m = new TensorNode("m", new Tensor({0}), t1);
+    auto *t2 = new OpNode("t2", new TransposeOp(NHWC2NCHW));
+    t2->exlinkUpperNode(m);
+    auto *back = new TensorNode("back", new Tensor({0}), t2);
+    OP(relu, ReluOp);
+    LINKUPPER(relu, back);
+    auto *y = new TensorNode("y", new Tensor({0}), relu);
+    // a dead branch
+    OP(dead, ReluOp);
+    LINKUPPER(dead, x);
+    auto *dz = new TensorNode("dz", new Tensor({0}), dead);
+    G(g);
+    GpT(g, x, m, back, y, dz);
+    GpO(g, t1, t2, relu, dead);
+    g->initTensorNodes();
+    CHECK((m->getDims() == vector<size_t>{2, 4, 5, 3}) && (back->getDims() == vector<size_t>{2, 3, 4, 5}));
+    g->findInOut();
+    g->updateTopology();
+    SETOUT(g, y);
+    dz->getLabel()->setIsOut(0);
+    ElimTransposePass et(g);
+    et.run();
+    CHECK(et.cancelledCount() == 1 && relu->getParentNode(0) == x);
+    EliminationPass dce(g);
+    dce.run();
+    CHECK(g->opNodeNum() == 1 && g->getOpNode(0) == relu);
+    CHECK(g->tensorNodeNum() == 2 && g->getNodeByName("m") == nullptr && g->getNodeByName("dz") == nullptr);
+    // a non-inverse pair stays
+    TENSOR(a, 2, 3, 4, 5);
+    auto *u1 = new OpNode("u1", new TransposeOp(NCHW2NHWC));
+    u1->exlinkUpperNode(a);
+    auto *am = new TensorNode("am", new Tensor({0}), u1);
+    auto *u2 = new OpNode("u2", new TransposeOp(NCHW2NHWC));
+    u2->exlinkUpperNode(am);
+    auto *ab = new TensorNode("ab", new Tensor({0}), u2);
+    OP(r2, ReluOp);
+    LINKUPPER(r2, ab);
+    auto *ay = new TensorNode("ay", new Tensor({0}), r2);
+    G(h);
+    GpT(h, a, am, ab, ay);
+    GpO(h, u1, u2, r2);
+    h->initTensorNodes();
+    ElimTransposePass et2(h);
+    et2.run();
+    CHECK(et2.cancelledCount() == 0 && r2->getParentNode(0) == ab);
+}
+
+int main() {
+    testTopologyAndShapes();
+    testLoweringAndRenaming();
+    testFusionAndPlacement();
+    testElimination();
+    if (failures) {
+        cerr << failures << " check(s) failed" << endl;
+        return 1;
+    }
+    cout << "all pass checks ok" << endl;
+    return 0;
+}

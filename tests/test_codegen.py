@@ -321,3 +321,12 @@ def test_timed_hip_program(gen, oracle, tmp_path, graph):
     want = oracle_run(oracle, "cfg3", 3, t)
     got = np.fromfile(os.path.join(tmp_path, "softmax_out_host.bin"), np.float32).reshape(want.shape)
     assert strict_rel_err(got, want) < 5 * TOL
+
+
+def test_graph_ir_and_passes_cpp_unit_tests(gen):
+    """swcompiler_amd/swc/test/testPasses.cpp: topology, shape inference, clone, FC lowering, renaming,
+    fusion, device placement, transpose cancelling and dead-node elimination, checked in C++."""
+    exe = os.path.join(SWC, "test", "bin", "testPasses")
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0, out.stderr
+    assert "all pass checks ok" in out.stdout
