@@ -88,8 +88,7 @@ void HipCodegen::emitTensorInitializations() {
         const bool onGpu = tn->getLabel()->getDeviceLabel().type == DeviceType::GPU;
         const TensorInitInfo info = t->getTensorInitInfo();
         switch (t->getTensorInitType()) {
-        case TensorInitType::PARENTOP:
-            uploads.push_back(static_cast<OpNode *>(tn->getParentNode(0)));
+        case TensorInitType::PARENTOP:   // filled by its run-once producer, below
             break;
         case TensorInitType::CONSTANT:
         case TensorInitType::ZERO: {
@@ -113,6 +112,13 @@ void HipCodegen::emitTensorInitializations() {
             break;
         }
     }
+    // every run-once op (parameter uploads), in topological order; runable() lets each through once
+    for (int i = 0; i < graph_->topologyNum(); ++i)
+        for (int j = 0; j < graph_->getNumInTopoLevel(i); ++j) {
+            IRNode *node = graph_->getNodeInTopo(i, j);
+            if (node->nodeType() == OP_NODE && static_cast<OpNode *>(node)->isRunOnce())
+                uploads.push_back(static_cast<OpNode *>(node));
+        }
     if (!uploads.empty()) writer_ << "// one-time parameter upload\n";
     for (OpNode *u : uploads) dispatchOpNode(u);
     writer_ << "\n";

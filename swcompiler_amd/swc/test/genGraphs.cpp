@@ -4,7 +4,7 @@
 // the reference's test/engine/testEngineMLPInfer.cpp.
 //
 //   genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse|graph]
-//   model: mnist8 | mnist_loader | nchw | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
+//   model: mnist8 | mnist_loader | nchw | manual | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
 //   mnist_loader: [batch] is the number of records in mnist_labels_images.bin
 //
 // Every parameter/input tensor is initialised from "<name>.bin" in the
@@ -193,6 +193,59 @@ int main(int argc, char **argv) {
         GpO(graph, fc0, tanh0, fc1, softmax, argmax_o, accuracy_o);
         graph->setInferDataNodes(label, data0);
         graph->addDisplayTensorNodes(accuracy_t);
+    } else if (model == "manual") {
+        // placement written out by hand, the way the reference's test/cuda/testGPUInfer.cpp does it:
+        // device twins, ScatterOp / GatherOp nodes, Label::setDeviceLabel, run-once parameter uploads,
+        // and the code generator injected with Engine::setCodegenerator — no Config::hip, no placement pass
+        const size_t b = batch ? batch : 16;
+        const Device gpu0(0, DeviceType::GPU, 0);
+        TENSOR(x, b, 64);
+        TENSOR(w, 64, 24);
+        TENSOR(bias, 24);
+        INIT(x, TensorInitType::FILE, "x.bin");
+        INIT(w, TensorInitType::FILE, "w.bin");
+        INIT(bias, TensorInitType::FILE, "bias.bin");
+        TENSOR(x_d, b, 64);
+        TENSOR(w_d, 64, 24);
+        TENSOR(bias_d, 24);
+        OP(up_x, ScatterOp);
+        OP(up_w, ScatterOp);
+        OP(up_b, ScatterOp);
+        up_w->setRunOnce();
+        up_b->setRunOnce();
+        LINKUPPER(up_x, x);
+        LINKUPPER(x_d, up_x);
+        LINKUPPER(up_w, w);
+        LINKUPPER(w_d, up_w);
+        LINKUPPER(up_b, bias);
+        LINKUPPER(bias_d, up_b);
+        OP(fc, MatrixMatrixFCBiasOp);
+        LINKUPPER(fc, x_d, w_d, bias_d);
+        TENSOR(y_d, b, 24);
+        LINKUPPER(y_d, fc);
+        OP(act, MatrixTanhOp);
+        LINKUPPER(act, y_d);
+        TENSOR(z_d, b, 24);
+        LINKUPPER(z_d, act);
+        OP(down, GatherOp);
+        LINKUPPER(down, z_d);
+        TENSOR(z, b, 24);
+        LINKUPPER(z, down);
+        for (IRNode *n : {(IRNode *)x_d, (IRNode *)w_d, (IRNode *)bias_d, (IRNode *)y_d, (IRNode *)z_d, (IRNode *)up_x,
+                          (IRNode *)up_w, (IRNode *)up_b, (IRNode *)fc, (IRNode *)act, (IRNode *)down})
+            n->getLabel()->setDeviceLabel(gpu0);
+        GpT(graph, x, w, bias, x_d, w_d, bias_d, y_d, z_d, z);
+        GpO(graph, up_x, up_w, up_b, fc, act, down);
+        graph->findInOut();
+        graph->updateTopology();
+        Config config;
+        config.dump_outputs = true;
+        graph->setConfig(config);
+        Engine engine(graph);
+        engine.compile();   // CPU-target passes: FCBias is lowered to MatrixMatrixMul + MatrixVectorAdd, on the GPU label
+        engine.setCodegenerator(new codegen::HipCodegen(graph, config));
+        cout << engine.genCode();
+        return 0;
     } else if (model == "nchw") {
         // an NCHW-trained block at the import boundary: data NCHW -> NHWC, filter OIHW -> OHWI
         // (the reference's importer inserts TransposeOp(NCHW2NHWC) the same way,

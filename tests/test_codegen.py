@@ -330,3 +330,35 @@ def test_graph_ir_and_passes_cpp_unit_tests(gen):
     out = subprocess.run([exe], capture_output=True, text=True)
     assert out.returncode == 0, out.stderr
     assert "all pass checks ok" in out.stdout
+
+
+# ------------------------------------------------ placement written by hand
+def manual_inputs(tmp_path):
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((16, 64)).astype(np.float32)
+    w = (rng.standard_normal((64, 24)) / 8).astype(np.float32)
+    b = (rng.standard_normal(24) * 0.1).astype(np.float32)
+    for name, a in (("x", x), ("w", w), ("bias", b)):
+        a.tofile(os.path.join(tmp_path, name + ".bin"))
+    return x, w, b
+
+
+def test_manual_placement_structure(gen, tmp_path):
+    manual_inputs(tmp_path)
+    code = generate(gen, "manual", "hip", tmp_path, 16)
+    # the hand-placed graph went through the CPU-target passes: FCBias lowered, on the device
+    assert "swc_hip_matrixMatrixMul_f(16, 24, 64, x_d, 64, w_d, 24, fc_mm_out, 24)" in code
+    assert "swc_hip_batchedadd_f(y_d, fc_mm_out, bias_d, 16, 24)" in code and "swc_hip_matrixTanh_f(" in code
+    head, body = code.split("// call op routine functions")
+    assert head.count("swc_hip_h2d(") == 2 and body.count("swc_hip_h2d(x_d, x,") == 1 and body.count("swc_hip_d2h(z, z_d,") == 1
+    build_hip(tmp_path)
+
+
+@pytest.mark.gpu
+def test_manual_placement_runs(gen, oracle, tmp_path):
+    x, w, b = manual_inputs(tmp_path)
+    generate(gen, "manual", "hip", tmp_path, 16)
+    subprocess.run([build_hip(tmp_path)], cwd=tmp_path, check=True, timeout=120, stdout=subprocess.DEVNULL)
+    want = oracle.matrixTanh(oracle.fcbias(x, w, b))
+    got = np.fromfile(os.path.join(tmp_path, "z.bin"), np.float32).reshape(want.shape)
+    assert rel_err(got, want) < TOL
