@@ -10,12 +10,16 @@ pass of that graph over one batch already resident in HBM.  Prints ONE JSON
 line; `value` is samples/s over exactly K timed steps.
 
 Also in the line:
-  roofline      the dominant kernel (the tiled fp32-MFMA GEMM gemm_dma<2,2,2>: both of its
+  roofline      the dominant kernel (the tiled fp32-MFMA GEMM gemm_dma2<2,4,4,2,false,8>: both of its
                 launches per step, 4096x784x4096 and 4096x4096x4096), timed
                 with HIP events on the library's stream inside the timed region
   kernels       per-launch times of the headline graph
   graph_replay  the same K steps replayed as one HIP graph per step (no per-kernel
                 events in the loop): what a launch-bound small graph gains
+  incl_transfers  the step with the input batch uploaded and the result downloaded
+                each time (never the headline value)
+  peaks_measured  fp32 MFMA rate of a register-only loop and a streaming copy on this
+                device, beside the datasheet peaks the fractions are computed from
   configs       the other synthetic configurations (samples/s and, per kernel,
                 TFLOP/s or GB/s with the fraction of the MI355X peak)
   cpu_baseline  the reference's own CPU kernels (oracle/_ref, g++ -std=c++11 -O2,
@@ -36,6 +40,7 @@ import numpy as np  # noqa: E402
 
 PEAK_TFLOPS_FP32_MFMA = 157.3
 PEAK_HBM_GBS = 8000.0
+ROOFLINE_KERNEL = "gemm_dma2<2,4,4,2,false,8>"   # 256x256 tiles, eight wavefronts: what both large FCs dispatch to
 
 
 class Timed:
@@ -121,9 +126,54 @@ def merge_rows(all_rows):
     out = []
     for i, row in enumerate(all_rows[0]):
         r = dict(row)
-        r["ms"] = sum(step[i]["ms"] for step in all_rows) / n
+        times = sorted(step[i]["ms"] for step in all_rows)
+        r["ms"] = sum(times) / n          # the average: what the rates below are computed from
+        r["ms_median"] = times[n // 2]
+        r["ms_min"] = times[0]
         out.append(rate(r))
     return out
+
+
+def with_transfers(rt, graphs, cfg, steps):
+    """The same step with the input batch uploaded and the result downloaded every step
+    (pageable host memory, synchronous copies: what a generated program's batch loop does)."""
+    t = graphs.make_inputs(cfg)
+    dt = {k: rt.upload(v) for k, v in t.items()}
+    batch = graphs.batch_of(cfg, t)
+    ws = {}
+    out = graphs.run(cfg, rt, dt, fused=True, ws=ws)
+    host_out = np.empty(out.shape, np.float32)
+    rt.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        rt.upload_into(dt["x"], t["x"])
+        out = graphs.run(cfg, rt, dt, fused=True, ws=ws)
+        rt.download_into(host_out, out)
+    wall = time.perf_counter() - t0
+    return dict(samples_per_s=batch * steps / wall, ms_per_step=wall * 1e3 / steps,
+                h2d_bytes=int(t["x"].nbytes), d2h_bytes=int(host_out.nbytes))
+
+
+def measured_peaks(rt):
+    """What this device sustains on the two rooflines: a register-only fp32 MFMA loop
+    (short and ~10 ms long: the clock settles lower under sustained matrix load) and a
+    256 MiB-in / 256 MiB-out streaming pass (relu_f)."""
+    short = rt.probe_mfma_tflops(200)
+    long_ = rt.probe_mfma_tflops(20000)
+    x = rt.upload(np.ones(1 << 26, np.float32))
+    y = rt.empty(x.shape)
+    rt.relu(x, out=y)
+    times = []
+    for i in range(10):
+        rt.event_record(0)
+        rt.relu(x, out=y)
+        rt.event_record(1)
+        times.append(rt.event_elapsed_ms(0, 1))
+    x.free()
+    y.free()
+    return dict(mfma_f32_tflops_short=short[0], mfma_f32_short_ms=short[1], mfma_f32_tflops_sustained=long_[0],
+                mfma_f32_sustained_ms=long_[1], stream_copy_gbs=2 * (1 << 28) / (min(times) * 1e-3) / 1e9,
+                datasheet=dict(mfma_f32_tflops=PEAK_TFLOPS_FP32_MFMA, hbm_gbs=PEAK_HBM_GBS))
 
 
 def run_config(rt, graphs, cfg, steps, warmup):
@@ -221,7 +271,7 @@ def main():
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):   # measured separately under rocprofv3 --pmc; see profiles/
-        traffic = json.load(open(tpath)).get("gemm_dma<2,2,2>", {}).get("bytes_per_launch")
+        traffic = json.load(open(tpath)).get(ROOFLINE_KERNEL, {}).get("bytes_per_launch")
     out = {
         "metric": "samples/s per graph; TFLOP/s (FC/conv) & GB/s (eltwise) vs MI355X roofline",
         "value": head["samples_per_s"], "unit": "samples/s", "n_gpus": 1, "steps": args.steps,
@@ -232,12 +282,15 @@ def main():
                    "global_batch": head["batch"], "device": rt.device_name()},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS_FP32_MFMA, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_TFLOPS_FP32_MFMA, "traffic": traffic,
-                     "kernel": "gemm_dma<2,2,2> (both launches per step: 4096x784x4096 and 4096x4096x4096)",
+                     "kernel": ROOFLINE_KERNEL + " (both launches per step: 4096x784x4096 and 4096x4096x4096)",
                      "flop_per_launch": flop / len(gemm), "avg_launch_ms": secs * 1e3 / len(gemm)},
         "gpu_ms_per_step": head["gpu_ms"] / args.steps,
         "graph_replay": head["graph_replay"],
+        "incl_transfers": with_transfers(rt, graphs, 2, max(5, min(args.steps, 20))),
         "kernels": head["kernels"],
     }
+    if not args.headline_only:
+        out["peaks_measured"] = measured_peaks(rt)
     if not args.headline_only:
         others = {}
         for cfg in (1, 3, 4, 5):

@@ -69,6 +69,14 @@ float swc_hip_timer_elapsed_ms(void);
 int swc_hip_event_record(int slot);
 float swc_hip_event_elapsed_ms(int first, int second);
 
+/* Diagnostic without a counterpart in the reference: runs `iters` rounds of 16
+ * independent v_mfma_f32_32x32x2_f32 per wavefront on two workgroups per CU and
+ * returns the elapsed milliseconds and the flop executed, so a harness can print
+ * the fp32 matrix rate the device sustains beside the datasheet figure.
+ * scratch_dev: device buffer of at least 512 * (number of CUs) floats. */
+int swc_hip_probe_mfma_f32(float *scratch_dev, size_t scratch_floats, int iters,
+                           float *ms_out, double *flop_out);
+
 /* HIP graphs: the ops issued between begin and end are recorded instead of run;
  * launch replays them with a single submission (the launch-bound small graphs —
  * batch-8 MLP, LeNet — spend most of their time between kernels otherwise).

@@ -293,6 +293,7 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
         wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
     }
     wait_vmcnt<0>();   // the trailing dummy loads still target this workgroup's LDS
+    acc_settle(acc);
     store_tile<TM, TN>(acc, out, (size_t)N, M, N, m0 + (wave >> 1) * 32 * TM, n0 + (wave & 1) * 32 * TN, lane, ep);
 #endif
 }

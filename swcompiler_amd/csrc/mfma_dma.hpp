@@ -115,6 +115,10 @@ __device__ __forceinline__ void compute_slice_swz(const float *__restrict__ As, 
 #pragma unroll
     for (int g = 0; g < BK / 8; ++g) {
         if (g + 1 < BK / 8) load_frag_swz<TM, TN, B_NT>(frag[(g + 1) & 1], As, Bs, g + 1, wave_m, wave_n, l32, h);
+        // Without this fence the scheduler sinks each LDS read to just before its
+        // first use (one or two MFMAs of cover, then a wait); with it the reads of
+        // group g+1 have the whole of group g's MFMAs to complete.
+        __builtin_amdgcn_sched_barrier(0);
         const Frag<TM, TN> &f = frag[g & 1];
 #pragma unroll
         for (int s = 0; s < 4; ++s)
@@ -122,7 +126,8 @@ __device__ __forceinline__ void compute_slice_swz(const float *__restrict__ As, 
             for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
                 for (int tn = 0; tn < TN; ++tn)
-                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[tm][s], f.b[tn][s], acc[tm][tn], 0, 0, 0);
+                    mfma_acc(acc[tm][tn], f.a[tm][s], f.b[tn][s]);
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -157,6 +162,59 @@ template <int PENDING> __device__ __forceinline__ void ring_sync() {
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
+}
+
+// ---- ring with the hand-over in the middle of a slice (STAGES >= 3) ----
+// The step above stops the matrix pipe at every slice boundary: barrier, issue
+// loads, read the first fragments, and only then the next MFMA — and the
+// wavefronts that share a SIMD reach their boundaries together, so nothing
+// fills the gap.  Here the barrier sits after the first group of MFMAs of a
+// slice instead: it certifies that slice kt+1 has landed (every wave waited for
+// its own part) and that slice kt-1 is no longer read by anyone, whose stage
+// then receives slice kt+STAGES-1.  The boundary itself needs no
+// synchronisation any more, so the first fragments of slice kt+1 are fetched
+// before the last MFMA group of slice kt, like any other group.
+// frag[0] holds group 0 of `rd` on entry and group 0 of `nx` on exit.
+template <int TM, int TN, bool B_NT, int STAGES>
+__device__ __forceinline__ void dma_step_mid(float *__restrict__ wr, const float *__restrict__ rd,
+                                             const float *__restrict__ nx, __amdgpu_buffer_rsrc_t rsrc_a,
+                                             __amdgpu_buffer_rsrc_t rsrc_b,
+                                             const int (&voff_a)[DmaTile<TM, TN, B_NT, STAGES>::kALoads],
+                                             const int (&voff_b)[DmaTile<TM, TN, B_NT, STAGES>::kBLoads],
+                                             v16f (&acc)[TM][TN], Frag<TM, TN> (&frag)[2], int wave, int lane) {
+    using T = DmaTile<TM, TN, B_NT, STAGES>;
+    static_assert(STAGES >= 3, "the slice being loaded, the one being read and the next must be distinct stages");
+    const int l32 = lane & 31;
+    const int h = lane >> 5;
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+#pragma unroll
+    for (int g = 0; g < BK / 8; ++g) {
+        if (g == 1) {
+            ring_sync<(STAGES - 3) * T::kLoads>();
+#pragma unroll
+            for (int j = 0; j < T::kALoads; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t *)(wr + (4 * j + wave) * 256), 16,
+                                                         voff_a[j], 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < T::kBLoads; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_t *)(wr + T::kAFloats + (4 * j + wave) * 256),
+                                                         16, voff_b[j], 0, 0, 0);
+        }
+        if (g + 1 < BK / 8)
+            load_frag_swz<TM, TN, B_NT>(frag[(g + 1) & 1], rd, rd + T::kAFloats, g + 1, wave_m, wave_n, l32, h);
+        else
+            load_frag_swz<TM, TN, B_NT>(frag[0], nx, nx + T::kAFloats, 0, wave_m, wave_n, l32, h);
+        __builtin_amdgcn_sched_barrier(0);   // reads stay ahead of this group's MFMAs (see compute_slice_swz)
+        const Frag<TM, TN> &f = frag[g & 1];
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn)
+                    mfma_acc(acc[tm][tn], f.a[tm][s], f.b[tn][s]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
 }
 
 #endif  // __HIP_DEVICE_COMPILE__

@@ -47,6 +47,35 @@ struct Tile {
     static constexpr int kBVec = BN * BK / 4 / kThreads;       // = 2*TN
 };
 
+// One v_mfma_f32_32x32x2_f32 with the accumulator held in the AGPR half of the
+// register file.  With accumulators in ordinary VGPRs every LDS or memory read
+// that returns into VGPRs competes with the matrix core's accumulator traffic
+// and stalls it (a 128-bit LDS read per four MFMAs costs ~10 % of the MFMA rate
+// on MI355X, 3 % with AGPR accumulators); the compiler picks the VGPR form
+// whenever registers are plentiful, so the choice is made here.  Written as
+// inline assembly, the instruction is opaque to the compiler's hazard
+// recogniser: the loop needs nothing (an accumulator is only ever read by the
+// next MFMA that accumulates into it, which the hardware interlocks), but the
+// first ordinary read of the results must be preceded by acc_settle().
+__device__ __forceinline__ void mfma_acc(v16f &acc, float a, float b) {
+#if __HIP_DEVICE_COMPILE__
+    asm("v_mfma_f32_32x32x2_f32 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+#endif
+}
+
+// Wait states between the last MFMA and the first read of its result (a
+// 16-pass MFMA needs 18; the data dependences on acc keep this after the MFMAs).
+template <int TM, int TN>
+__device__ __forceinline__ void acc_settle(v16f (&acc)[TM][TN]) {
+#if __HIP_DEVICE_COMPILE__
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));   // every accumulator's chain ends before the nops
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" : "+a"(acc[TM - 1][TN - 1]));
+#endif
+}
+
 // Fragments of one group of 8 k's: a lane's four consecutive k's of each of its
 // TM rows of A and TN columns of B.
 template <int TM, int TN>
@@ -115,40 +144,67 @@ struct Epilogue {
 };
 
 // Writes this wavefront's accumulators to C (row-major, leading dimension ldc).
-template <int TM, int TN>
-__device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], float *__restrict__ C, size_t ldc, int M, int N,
-                                           int row0, int col0, int lane, const Epilogue &ep) {
+// One store instruction covers two rows of 32 consecutive floats (two full
+// 128-byte lines).  GUARD = false is the path of a sub-tile that lies wholly
+// inside the matrix: no per-row control flow, so the 16*TM*TN stores issue back
+// to back.  (On this target stores and loads share one outstanding-operation
+// counter; a branch per row makes the compiler wait for that counter — i.e. for
+// the previous store to be acknowledged — before every store.)  The guarded
+// path first waits for the per-column parameters explicitly, after which its
+// row blocks have no load to wait for either.
+template <int TM, int TN, bool GUARD>
+__device__ __forceinline__ void store_tile_impl(const v16f (&acc)[TM][TN], float *__restrict__ C, size_t ldc, int M,
+                                                int N, int row0, int col0, int lane, const Epilogue &ep) {
     const int l32 = lane & 31;
     const int h = lane >> 5;
+    const bool bn = ep.bn_mean != nullptr;
+    float bias[TN], mean[TN], slope[TN], beta[TN];
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
         const int col = col0 + tn * 32 + l32;
-        if (col >= N) continue;
-        const float bias = ep.bias ? ep.bias[col] : 0.f;
+        const bool ok = !GUARD || col < N;
+        bias[tn] = (ep.bias && ok) ? ep.bias[col] : 0.f;
         // batchnorm folded to one fp32 multiply-add per element: the slope
         // scale*(var+eps)^-1/2 is formed in double and rounded once; the result is
         // within 2 ulp of the reference's all-double evaluation
-        float mean = 0.f, slope = 1.f, beta = 0.f;
-        const bool bn = ep.bn_mean != nullptr;
-        if (bn) {
-            mean = ep.bn_mean[col];
+        mean[tn] = 0.f, slope[tn] = 1.f, beta[tn] = 0.f;
+        if (bn && ok) {
+            mean[tn] = ep.bn_mean[col];
             const float ve = ep.bn_var[col] + ep.eps;
-            slope = (float)((double)ep.bn_scale[col] / sqrt((double)ve));
-            beta = ep.bn_bias[col];
+            slope[tn] = (float)((double)ep.bn_scale[col] / sqrt((double)ve));
+            beta[tn] = ep.bn_bias[col];
         }
+    }
+#if __HIP_DEVICE_COMPILE__
+    if (GUARD) __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): the parameter loads above are complete
+#endif
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+        const int col = col0 + tn * 32 + l32;
+        if (GUARD && col >= N) continue;
+        float *__restrict__ p = C + (size_t)(row0 + 4 * h) * ldc + col;
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int row = row0 + tm * 32 + 8 * (v / 4) + 4 * h + (v % 4);
-                if (row >= M) continue;
-                float x = acc[tm][tn][v] + bias;
-                if (bn) x = fmaf(x - mean, slope, beta);
+                const int r = tm * 32 + 8 * (v / 4) + (v % 4);   // row relative to row0 + 4*h
+                if (GUARD && row0 + 4 * h + r >= M) continue;
+                float x = acc[tm][tn][v] + bias[tn];
+                if (bn) x = fmaf(x - mean[tn], slope[tn], beta[tn]);
                 if (ep.relu) x = (x > 0.f) ? x : 0.f;
-                C[(size_t)row * ldc + col] = x;
+                p[(size_t)r * ldc] = x;
             }
         }
     }
+}
+
+template <int TM, int TN>
+__device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], float *__restrict__ C, size_t ldc, int M, int N,
+                                           int row0, int col0, int lane, const Epilogue &ep) {
+    if (row0 + 32 * TM <= M && col0 + 32 * TN <= N)   // wavefront-uniform
+        store_tile_impl<TM, TN, false>(acc, C, ldc, M, N, row0, col0, lane, ep);
+    else
+        store_tile_impl<TM, TN, true>(acc, C, ldc, M, N, row0, col0, lane, ep);
 }
 
 // Workgroup id -> tile coordinates.  Workgroups are dealt round-robin to the 8

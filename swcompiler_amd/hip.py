@@ -20,7 +20,8 @@ EXPORTS = [
     "swc_hip_d2d", "swc_hip_fill_f", "swc_hip_sync", "swc_hip_last_error", "swc_hip_stream",
     "swc_hip_set_stream", "swc_hip_device_name", "swc_hip_timer_begin", "swc_hip_timer_end",
     "swc_hip_timer_elapsed_ms", "swc_hip_event_record", "swc_hip_event_elapsed_ms", "swc_hip_graph_begin",
-    "swc_hip_graph_end", "swc_hip_graph_launch", "swc_hip_graph_destroy", "swc_hip_matrixMatrixMul_f", "swc_hip_batchedadd_f", "swc_hip_relu_f",
+    "swc_hip_graph_end", "swc_hip_graph_launch", "swc_hip_graph_destroy", "swc_hip_probe_mfma_f32",
+    "swc_hip_matrixMatrixMul_f", "swc_hip_batchedadd_f", "swc_hip_relu_f",
     "swc_hip_vecAdd_f", "swc_hip_conv2d_f", "swc_hip_batchnormalization_f", "swc_hip_maxpool_f",
     "swc_hip_maxpool_argmax_f", "swc_hip_avgpool_f", "swc_hip_transpose4d_f", "swc_hip_transpose2d_f",
     "swc_hip_matrixSoftmax_f", "swc_hip_matrixTanh_f", "swc_hip_argMax_i",
@@ -69,6 +70,7 @@ def load_library():
         "swc_hip_graph_end": (i32, [C.POINTER(vp)]),
         "swc_hip_graph_launch": (i32, [vp]),
         "swc_hip_graph_destroy": (i32, [vp]),
+        "swc_hip_probe_mfma_f32": (i32, [vp, sz, i32, C.POINTER(f32), C.POINTER(C.c_double)]),
         "swc_hip_matrixMatrixMul_f": (i32, [i32, i32, i32, vp, i32, vp, i32, vp, i32]),
         "swc_hip_batchedadd_f": (i32, [vp, vp, vp, sz, sz]),
         "swc_hip_relu_f": (i32, [vp, vp, sz]),
@@ -193,6 +195,25 @@ class SwcHip:
         host = np.empty(d.shape, d.dtype)
         self._check(self.lib.swc_hip_d2h(host.ctypes.data, d.ptr, d.nbytes), "swc_hip_d2h")
         return host
+
+    def upload_into(self, d, host):
+        """h2d into an existing allocation of the same size"""
+        host = np.ascontiguousarray(host)
+        assert host.nbytes == d.nbytes
+        self._check(self.lib.swc_hip_h2d(d.ptr, host.ctypes.data, host.nbytes), "swc_hip_h2d")
+
+    def download_into(self, host, d):
+        assert host.nbytes == d.nbytes and host.flags.c_contiguous
+        self._check(self.lib.swc_hip_d2h(host.ctypes.data, d.ptr, d.nbytes), "swc_hip_d2h")
+
+    def probe_mfma_tflops(self, iters=2000):
+        """fp32 MFMA rate a register-only loop sustains (TFLOP/s) and its duration in ms"""
+        scratch = self.empty((512 * 512,))
+        ms, flop = C.c_float(), C.c_double()
+        self._check(self.lib.swc_hip_probe_mfma_f32(scratch.ptr, scratch.size, iters, C.byref(ms), C.byref(flop)),
+                    "swc_hip_probe_mfma_f32")
+        scratch.free()
+        return flop.value / (ms.value * 1e-3) / 1e12, ms.value
 
     def sync(self):
         self._check(self.lib.swc_hip_sync(), "swc_hip_sync")

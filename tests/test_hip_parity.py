@@ -374,8 +374,13 @@ def test_error_paths(rt):
 # SWC_HIP_GEMM / SWC_HIP_CONV force a tile shape / pipeline variant; the library
 # reads them on every call.  "reg*" = register-staged kernels (the path taken for
 # unaligned shapes and for operands beyond the 2 GiB reach of 32-bit buffer
-# offsets), "TMTN_S" = direct-to-LDS kernels with an S-stage ring.
-@pytest.mark.parametrize("variant", ["reg", "22_2", "22_3", "21_3", "12_3", "11_3", "11_4"])
+# offsets), "TMTN_S[m]" = direct-to-LDS kernels with an S-stage ring (m: ring hand-over in
+# mid-slice), "TMTNwWM_S[m][x8]" = the column-interleaved kernels (x8: eight wavefronts).
+GEMM_VARIANTS = ["reg", "22_2", "22_3", "21_3", "12_3", "11_3", "11_4", "11_3m", "21_3m",
+                 "24w4_2x8", "14w4_2", "14w4_3m", "24w2_3m", "22w2_2"]
+
+
+@pytest.mark.parametrize("variant", GEMM_VARIANTS)
 def test_gemm_every_variant(rt, oracle, variant, monkeypatch):
     print("case gemm variant", variant, flush=True)
     monkeypatch.setenv("SWC_HIP_GEMM", variant)
@@ -390,6 +395,13 @@ def test_gemm_every_variant(rt, oracle, variant, monkeypatch):
     a = rng.uniform(0, 1, (257, 516)).astype(np.float32)
     b = rng.uniform(0, 1, (516, 260)).astype(np.float32)
     assert strict_rel_err(rt.matrixMatrixMul(*up(rt, a, b)).numpy(), oracle.matrixMatrixMul(a, b)) < TOL
+    # tiles on every edge of a 256x256 grid, K not a multiple of the slice, bias without ReLU
+    m, k, n = 520, 100, 776
+    a = rng.integers(-8, 9, (m, k)).astype(np.float32)
+    b = rng.integers(-8, 9, (k, n)).astype(np.float32)
+    bias = rng.integers(-8, 9, n).astype(np.float32)
+    want = (a.astype(np.int64) @ b.astype(np.int64) + bias.astype(np.int64)).astype(np.float32)
+    assert_bit_exact(rt.fcbias(*up(rt, a, b, bias), relu=False).numpy(), want, f"integer gemm {m}x{k}x{n} variant {variant}")
 
 
 @pytest.mark.parametrize("variant", ["reg22", "reg21", "reg12", "reg11", "22_2", "21_3", "12_3", "11_3", "11_4"])
