@@ -186,7 +186,7 @@ __global__ __launch_bounds__(kThreads) void conv_igemm(const float *__restrict__
 // 32-bit byte offset per lane per load — out-of-image taps and rows past M get
 // the out-of-range offset and arrive in LDS as zeros.  Needs iC % 4 == 0,
 // 16-byte-aligned tensors and input/filter below 2 GiB.
-template <int TM, int TN, int STAGES>
+template <int TM, int TN, int STAGES, bool MID = false>
 __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ in, const float *__restrict__ filt,
                                                      float *__restrict__ out, ConvGeom g, unsigned in_bytes,
                                                      unsigned filt_bytes, Epilogue ep) {
@@ -284,13 +284,28 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
     }
     const int nk = (K + BK - 1) / BK;
     int rd_stage = 0, wr_stage = STAGES - 1;
-    for (int kt = 0; kt < nk; ++kt) {
-        ring_sync<(STAGES - 2) * T::kLoads>();
-        next_offsets();
-        dma_step<TM, TN, true, STAGES>(lds + wr_stage * T::kStageFloats, lds + rd_stage * T::kStageFloats, rsrc_a,
-                                       rsrc_b, va, vb, acc, wave, lane);
-        rd_stage = rd_stage + 1 == STAGES ? 0 : rd_stage + 1;
-        wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
+    if constexpr (MID) {   // ring hand-over after the first MFMA group of a slice (dma_step_mid)
+        ring_sync<(STAGES - 2) * T::kLoads>();   // slice 0 has landed
+        Frag<TM, TN> frag[2];
+        load_frag_swz<TM, TN, true>(frag[0], lds, lds + T::kAFloats, 0, wave >> 1, wave & 1, lane & 31, lane >> 5);
+        for (int kt = 0; kt < nk; ++kt) {
+            next_offsets();
+            const int nx_stage = rd_stage + 1 == STAGES ? 0 : rd_stage + 1;
+            dma_step_mid<TM, TN, true, STAGES>(lds + wr_stage * T::kStageFloats, lds + rd_stage * T::kStageFloats,
+                                               lds + nx_stage * T::kStageFloats, rsrc_a, rsrc_b, va, vb, acc, frag,
+                                               wave, lane);
+            rd_stage = nx_stage;
+            wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
+        }
+    } else {
+        for (int kt = 0; kt < nk; ++kt) {
+            ring_sync<(STAGES - 2) * T::kLoads>();
+            next_offsets();
+            dma_step<TM, TN, true, STAGES>(lds + wr_stage * T::kStageFloats, lds + rd_stage * T::kStageFloats, rsrc_a,
+                                           rsrc_b, va, vb, acc, wave, lane);
+            rd_stage = rd_stage + 1 == STAGES ? 0 : rd_stage + 1;
+            wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
+        }
     }
     wait_vmcnt<0>();   // the trailing dummy loads still target this workgroup's LDS
     acc_settle(acc);
@@ -298,12 +313,12 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
 #endif
 }
 
-template <int TM, int TN, int STAGES>
+template <int TM, int TN, int STAGES, bool MID = false>
 int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGeom &g, size_t in_bytes,
                     size_t filt_bytes, const Epilogue &ep) {
     using T = DmaTile<TM, TN, true, STAGES>;
     const long tiles = (long)((g.M + T::BM - 1) / T::BM) * ((g.OC + T::BN - 1) / T::BN);
-    auto kern = conv_dma<TM, TN, STAGES>;
+    auto kern = conv_dma<TM, TN, STAGES, MID>;
     static bool attr_set = false;
     if (!attr_set) {
         SWC_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -486,7 +501,7 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
     const bool vec = (g.C % 4 == 0) && aligned16(input) && aligned16(filter);
     const size_t in_bytes = idims[0] * idims[1] * idims[2] * idims[3] * 4, filt_bytes = odims[3] * K * 4;
     const bool dma_ok = vec && in_bytes < kMaxDmaBytes && filt_bytes < kMaxDmaBytes;
-    const char *force = getenv("SWC_HIP_CONV");   // forces a kernel variant (tests, tuning): reg22 reg21 reg12 reg11 | 22_2 21_3 12_3 11_3 11_4
+    const char *force = getenv("SWC_HIP_CONV");   // forces a kernel variant (tests, tuning): reg22 reg21 reg12 reg11 | 22_2 21_3 12_3 11_3 11_4 | 11_3m 21_3m 12_3m 22_3m (m: ring hand-over in mid-slice)
     if (force) {
         if (!strcmp(force, "reg22")) return launch_conv<2, 2>(vec, input, filter, output, g, ep);
         if (!strcmp(force, "reg21")) return launch_conv<2, 1>(vec, input, filter, output, g, ep);
@@ -498,17 +513,24 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
             if (!strcmp(force, "12_3")) return launch_conv_dma<1, 2, 3>(input, filter, output, g, in_bytes, filt_bytes, ep);
             if (!strcmp(force, "11_3")) return launch_conv_dma<1, 1, 3>(input, filter, output, g, in_bytes, filt_bytes, ep);
             if (!strcmp(force, "11_4")) return launch_conv_dma<1, 1, 4>(input, filter, output, g, in_bytes, filt_bytes, ep);
+            if (!strcmp(force, "11_3m")) return launch_conv_dma<1, 1, 3, true>(input, filter, output, g, in_bytes, filt_bytes, ep);
+            if (!strcmp(force, "21_3m")) return launch_conv_dma<2, 1, 3, true>(input, filter, output, g, in_bytes, filt_bytes, ep);
+            if (!strcmp(force, "12_3m")) return launch_conv_dma<1, 2, 3, true>(input, filter, output, g, in_bytes, filt_bytes, ep);
+            if (!strcmp(force, "22_3m")) return launch_conv_dma<2, 2, 3, true>(input, filter, output, g, in_bytes, filt_bytes, ep);
         }
     }
     if (!(force && !strncmp(force, "reg", 3)) && g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0)
         return launch_conv_direct(input, filter, bias, output, g, ep);
     if (dma_ok) {
-        // 64x128 tiles once they fill the chip (wide layers), 64x64 otherwise: the
-        // layers here are tens of microseconds long, many small tiles balance the
-        // 256 CUs better than few large ones
-        if (g.OC > 64 && ((M + 63) / 64) * ((g.OC + 127) / 128) >= (size_t)num_cus())
+        // These layers last 80-160 us: how evenly the tiles divide over the 256 CUs matters as much as
+        // the tile's own efficiency.  64x64 tiles (ring hand-over in mid-slice) while there are at least
+        // eight of them per CU; below that 64x128 tiles for wide layers, which halve the count but keep
+        // two workgroups per CU busy to the end (measured: 105 vs 100 TFLOP/s for 56x56x64->128,
+        // 85 vs 90 for 28x28x128->128).
+        const size_t tiles64 = ((M + 63) / 64) * ((g.OC + 63) / 64);
+        if (tiles64 < 8 * (size_t)num_cus() && g.OC > 64 && ((M + 63) / 64) * ((g.OC + 127) / 128) >= (size_t)num_cus())
             return launch_conv_dma<1, 2, 3>(input, filter, output, g, in_bytes, filt_bytes, ep);
-        return launch_conv_dma<1, 1, 3>(input, filter, output, g, in_bytes, filt_bytes, ep);
+        return launch_conv_dma<1, 1, 3, true>(input, filter, output, g, in_bytes, filt_bytes, ep);
     }
     const long tiles_m128 = (M + 127) / 128;
     if (g.OC > 64 && tiles_m128 * ((g.OC + 127) / 128) >= num_cus())

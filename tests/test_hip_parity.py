@@ -404,7 +404,7 @@ def test_gemm_every_variant(rt, oracle, variant, monkeypatch):
     assert_bit_exact(rt.fcbias(*up(rt, a, b, bias), relu=False).numpy(), want, f"integer gemm {m}x{k}x{n} variant {variant}")
 
 
-@pytest.mark.parametrize("variant", ["reg22", "reg21", "reg12", "reg11", "22_2", "21_3", "12_3", "11_3", "11_4"])
+@pytest.mark.parametrize("variant", ["reg22", "reg21", "reg12", "reg11", "22_2", "21_3", "12_3", "11_3", "11_4", "11_3m", "21_3m", "12_3m", "22_3m"])
 def test_conv_every_variant(rt, oracle, variant, monkeypatch):
     print("case conv variant", variant, flush=True)
     monkeypatch.setenv("SWC_HIP_CONV", variant)
