@@ -162,7 +162,7 @@ class CpuKernels:
         return out, idx
 
     def maxpoolGrad(self, x, out_grad, kernels, strides, pads=(0, 0, 0, 0)):
-        """reference build only: scatter out_grad to the chosen taps."""
+        """scatter out_grad to the taps the windows selected (kernels.h:380-442)"""
         x = np.ascontiguousarray(x, np.float32)
         out_grad = np.ascontiguousarray(out_grad, np.float32)
         ig = np.empty_like(x)
@@ -187,6 +187,81 @@ class CpuKernels:
         self._fn("argMax_i")(_fp(x), idx.ctypes.data_as(_i32p), C.c_int(m),
                              C.c_int(n), C.c_int(top_k))
         return idx
+
+    # ---- training kernels ---------------------------------------------
+    def matrixTrans(self, a):
+        a = np.ascontiguousarray(a, np.float32)
+        m, n = a.shape
+        out = np.empty((n, m), np.float32)
+        self._fn("matrixTrans_f")(C.c_int(m), C.c_int(n), _fp(a), C.c_int(n), _fp(out), C.c_int(m))
+        return out
+
+    def matrixTanhGrad(self, out, out_grad):
+        """(tanh output, gradient of it) -> gradient of the tanh input"""
+        out = np.ascontiguousarray(out, np.float32)
+        out_grad = np.ascontiguousarray(out_grad, np.float32)
+        m, n = out.shape
+        ig = np.empty_like(out)
+        self._fn("matrixTanhGrad_f")(C.c_int(m), C.c_int(n), _fp(ig), C.c_int(n), _fp(out), C.c_int(n),
+                                     _fp(out_grad), C.c_int(n))
+        return ig
+
+    def matrixSoftmaxWithLoss(self, a, selected):
+        a = np.ascontiguousarray(a, np.float32)
+        selected = np.ascontiguousarray(selected, np.int32)
+        m, n = a.shape
+        out = np.empty_like(a)
+        loss = np.zeros(1, np.float32)
+        self._fn("matrixSoftmaxWithLoss_f")(C.c_int(m), C.c_int(n), _fp(a), C.c_int(n), _fp(out), C.c_int(n),
+                                            selected.ctypes.data_as(_i32p), _fp(loss))
+        return out, loss[0]
+
+    def matrixSoftmaxGrad(self, prob, selected, with_loss=False):
+        prob = np.ascontiguousarray(prob, np.float32)
+        selected = np.ascontiguousarray(selected, np.int32)
+        m, n = prob.shape
+        ig = np.empty_like(prob)
+        name = "matrixSoftmaxWithLossGrad_f" if with_loss and self.has("matrixSoftmaxWithLossGrad_f") else "matrixSoftmaxGrad_f"
+        self._fn(name)(C.c_int(m), C.c_int(n), _fp(ig), C.c_int(n), _fp(prob), C.c_int(n),
+                       selected.ctypes.data_as(_i32p))
+        return ig
+
+    def conv2dGrad(self, x, filt, out_grad, kernels=None, strides=(1, 1), pads=(0, 0, 0, 0), group=1):
+        """-> (input gradient, filter gradient, bias gradient)"""
+        x = np.ascontiguousarray(x, np.float32)
+        filt = np.ascontiguousarray(filt, np.float32)
+        out_grad = np.ascontiguousarray(out_grad, np.float32)
+        if kernels is None:
+            kernels = filt.shape[1:3]
+        ig, fg, bg = np.empty_like(x), np.empty_like(filt), np.empty(filt.shape[0], np.float32)
+        self._fn("conv2dGrad_f")(_fp(ig), _fp(fg), _fp(bg), _fp(out_grad), _fp(x), _fp(filt), _dims(out_grad.shape),
+                                 _dims(x.shape), _dims(filt.shape), _dims(bg.shape), _dims(kernels), _dims(strides),
+                                 _dims(pads), C.c_size_t(group))
+        return ig, fg, bg
+
+    def batchedreduceadd(self, batch):
+        """one sum per row (slice) of a 2-D array"""
+        batch = np.ascontiguousarray(batch, np.float32)
+        ns, ss = batch.shape
+        out = np.empty(ns, np.float32)
+        self._fn("batchedreduceadd_f")(_fp(out), _fp(batch), C.c_size_t(ns), C.c_size_t(ss))
+        return out
+
+    def sgd(self, w, dw, mom, lr, decay, momentum, batch):
+        """-> (updated weights, updated momentum buffer); inputs are not modified"""
+        w = np.array(w, np.float32, copy=True, order="C")
+        mom = np.array(mom, np.float32, copy=True, order="C")
+        dw = np.ascontiguousarray(dw, np.float32)
+        self._fn("sgd_f")(C.c_size_t(w.size), _fp(w), _fp(w), _fp(dw), _fp(mom), C.c_float(lr), C.c_float(decay),
+                          C.c_float(momentum), C.c_size_t(batch))
+        return w, mom
+
+    def reluGrad(self, src, dest_grad):
+        src = np.ascontiguousarray(src, np.float32)
+        dest_grad = np.ascontiguousarray(dest_grad, np.float32)
+        out = np.empty_like(src)
+        self._fn("reluGrad_f")(_fp(out), _fp(src), _fp(dest_grad), C.c_size_t(src.size))
+        return out
 
 
 def build(force=False):

@@ -69,4 +69,28 @@ void ref_vecAdd_f(int n, float *a, float *b, float *c) { vecAdd_f(n, a, b, c); }
 void ref_argMax_i(const float *in, int *idx, int m, int n, int k) {
     argMax_i(in, idx, m, n, k);
 }
+void ref_matrixTrans_f(int m, int n, const float *a, int lda, float *b, int ldb) { matrixTrans_f(m, n, a, lda, b, ldb); }
+void ref_matrixTanhGrad_f(int m, int n, float *a, int lda, const float *b, int ldb, const float *c, int ldc) {
+    matrixTanhGrad_f(m, n, a, lda, b, ldb, c, ldc);
+}
+void ref_matrixSoftmaxWithLoss_f(int m, int n, const float *a, int lda, float *b, int ldb, const int *sel, float *loss) {
+    matrixSoftmaxWithLoss_f(m, n, a, lda, b, ldb, sel, loss);
+}
+void ref_matrixSoftmaxGrad_f(int m, int n, float *a, int lda, const float *b, int ldb, const int *sel) {
+    matrixSoftmaxGrad_f(m, n, a, lda, b, ldb, sel);
+}
+void ref_matrixSoftmaxWithLossGrad_f(int m, int n, float *a, int lda, const float *b, int ldb, const int *sel) {
+    matrixSoftmaxWithLossGrad_f(m, n, a, lda, b, ldb, sel);
+}
+void ref_conv2dGrad_f(float *ig, float *fg, float *bg, const float *og, const float *i, const float *f,
+                      const size_t *od, const size_t *id, const size_t *fd, const size_t *bd, const size_t *k,
+                      const size_t *s, const size_t *p, size_t group) {
+    conv2dGrad_f(ig, fg, bg, og, i, f, od, id, fd, bd, k, s, p, group);
+}
+void ref_batchedreduceadd_f(float *d, const float *b, size_t ns, size_t ss) { batchedreduceadd_f(d, b, ns, ss); }
+void ref_sgd_f(size_t size, float *out, float *w, float *dw, float *mom, float lr, float decay, float momentum,
+               size_t batch) {
+    sgd_f(size, out, w, dw, mom, lr, decay, momentum, batch);
+}
+void ref_reluGrad_f(float *sg, const float *s, const float *dg, size_t n) { reluGrad_f(sg, s, dg, n); }
 }

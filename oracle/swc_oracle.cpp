@@ -1,4 +1,4 @@
-// CPU oracle for the SWCompiler inference kernels.
+// CPU oracle for the SWCompiler inference kernels and the training kernels next to them.
 //
 // THIS FILE IS TEST INFRASTRUCTURE.  It is the checker that the HIP kernels are
 // compared against; it is never linked into, loaded by or called from the
@@ -15,12 +15,14 @@
 // Pinning status (what proves this file equals the reference):
 //   * every function below is compared bit-for-bit with the reference header
 //     itself, compiled from /root/reference into oracle/_ref/libswc_ref.so,
-//     on seeded inputs (tests/test_oracle_vs_ref.py, skipped when the
-//     reference tree is absent);
+//     on seeded inputs (tests/test_oracle_vs_ref.py, tests/test_oracle_training.py,
+//     skipped when the reference tree is absent);
 //   * the outputs of that reference build are committed as fixtures under
 //     tests/golden/ and checked on every run (tests/test_oracle_golden.py);
 //   * the MNIST-8 known answer of the reference's test inputs and closed-form
-//     / invariant checks (tests/test_oracle_math.py).
+//     / invariant checks (tests/test_oracle_math.py); each gradient kernel is
+//     checked as the derivative of its forward kernel by differences in float64
+//     (tests/test_oracle_training.py).
 //   No function here is "parity unpinned".
 
 #include <cmath>
@@ -295,6 +297,161 @@ void oracle_argMax_i(const float *input, int *idx, int m, int n, int top_k) {
 // image.h:13-33: raw little-endian fp32 file, `offset` counted in elements.
 // Returns the number of elements copied, or -1 if the file cannot be read.
 long oracle_load_f(float *data, size_t size, size_t offset, const char *path);
+
+
+// ---------------------------------------------------------------- training
+// The kernels a generated TRAINING program calls next to the inference ones
+// (Codegen.cpp:1518-1531, 1785-1830, 2047-2079, 2138-2148, 2357-2465, 2466-2489).
+
+// kernels.h:68-76.  B[n,m] = A[m,n]^T.
+void oracle_matrixTrans_f(int m, int n, const float *a, int lda, float *b, int ldb) {
+    for (int i = 0; i < n; ++i)
+        for (int j = 0; j < m; ++j) b[(size_t)i * ldb + j] = a[(size_t)j * lda + i];
+}
+
+// kernels.h:79-86.  A = (1 - B*B) * C with B the tanh output and C the incoming
+// gradient: fl(fl(1 - fl(B*B)) * C).
+void oracle_matrixTanhGrad_f(int m, int n, float *a, int lda, const float *b, int ldb, const float *c, int ldc) {
+    for (int i = 0; i < m; ++i)
+        for (int j = 0; j < n; ++j) {
+            const float bb = b[(size_t)i * ldb + j];
+            a[(size_t)i * lda + j] = (1 - bb * bb) * c[(size_t)i * ldc + j];
+        }
+}
+
+// kernels.h:105-129.  Row softmax as matrixSoftmax_f plus the mean
+// cross-entropy: loss = (1/m) * sum_i [ logf(sum_i * expf(max_i)) - A(i, selected[i]) ],
+// accumulated over rows in order in fp32.
+void oracle_matrixSoftmaxWithLoss_f(int m, int n, const float *a, int lda, float *b, int ldb, const int *selected,
+                                    float *loss) {
+    *loss = 0;
+    for (int i = 0; i < m; ++i) {
+        const float *arow = a + (size_t)i * lda;
+        float *brow = b + (size_t)i * ldb;
+        float max_ = arow[0];
+        for (int j = 0; j < n; ++j) max_ = std::max(max_, arow[j]);
+        float sum = 0;
+        for (int j = 0; j < n; ++j) {
+            brow[j] = expf(arow[j] - max_);
+            sum += brow[j];
+        }
+        for (int j = 0; j < n; ++j) brow[j] = brow[j] / sum;
+        *loss += logf(sum * expf(max_)) - arow[selected[i]];
+    }
+    *loss /= m;
+}
+
+// kernels.h:133-151 (matrixSoftmaxGrad_f and matrixSoftmaxWithLossGrad_f are the
+// same loop).  A = B - onehot(selected).
+void oracle_matrixSoftmaxGrad_f(int m, int n, float *a, int lda, const float *b, int ldb, const int *selected) {
+    for (int i = 0; i < m; ++i)
+        for (int j = 0; j < n; ++j) {
+            const float delta = (selected[i] == j);
+            a[(size_t)i * lda + j] = b[(size_t)i * ldb + j] - delta;
+        }
+}
+
+// kernels.h:245-319.  All three gradients start at zero and are accumulated in
+// fp32 in the loop order n, g, co, kx, ky, ox, oy, ci; the bias gradient takes
+// outputG once per output element, at tap (0,0) and after the bounds test — so an
+// output pixel whose first tap lies in the padding does not contribute (with
+// padding this is not the full bias gradient; it is what the reference computes).
+// Loop order is kept as in
+// the reference: the per-element operation order of inputG and filterG depends on it.
+void oracle_conv2dGrad_f(float *inputG, float *filterG, float *biasG, const float *outputG, const float *input,
+                         const float *filter, const size_t *odims, const size_t *idims, const size_t *fdims,
+                         const size_t *bdims, const size_t *kernels, const size_t *strides, const size_t *pads,
+                         size_t group) {
+    (void)bdims;
+    const Dims4 od(odims), id(idims), fd(fdims);
+    const size_t batch = id.d0, inC = id.d3, oC = od.d3;
+    const size_t inCG = inC / group, oCG = oC / group;
+    const size_t kh = kernels[0], kw = kernels[1], sh = strides[0], sw = strides[1], pt = pads[0], pl = pads[1];
+    std::fill(inputG, inputG + id.d0 * id.d1 * id.d2 * id.d3, 0.f);
+    std::fill(filterG, filterG + fd.d0 * fd.d1 * fd.d2 * fd.d3, 0.f);
+    std::fill(biasG, biasG + oC, 0.f);
+    for (size_t n = 0; n < batch; ++n)
+        for (size_t g = 0; g < group; ++g)
+            for (size_t co = g * oCG; co < (g + 1) * oCG; ++co)
+                for (size_t kx = 0; kx < kh; ++kx)
+                    for (size_t ky = 0; ky < kw; ++ky) {
+                        const size_t fbase = fd.at(co, kx, ky, g * inCG);
+                        for (size_t ox = 0; ox < od.d1; ++ox)
+                            for (size_t oy = 0; oy < od.d2; ++oy) {
+                                const ssize_t ix = (ssize_t)ox * sh - pt + kx;
+                                const ssize_t iy = (ssize_t)oy * sw - pl + ky;
+                                if (ix < 0 || ix >= (ssize_t)id.d1 || iy < 0 || iy >= (ssize_t)id.d2) continue;
+                                const size_t ibase = id.at(n, ix, iy, g * inCG);
+                                const float og = outputG[od.at(n, ox, oy, co)];
+                                for (size_t ci = 0; ci < inCG; ++ci) {
+                                    inputG[ibase + ci] += filter[fbase + ci] * og;
+                                    filterG[fbase + ci] += input[ibase + ci] * og;
+                                }
+                                if (kx == 0 && ky == 0) biasG[co] += og;
+                            }
+                    }
+}
+
+// kernels.h:380-442.  inputG starts at zero; every output element adds its
+// gradient to the input element its window selected (first maximum in scan
+// order; a window with no in-bounds tap selects element (0,0) of the image, as
+// the reference's uninitialised max_ix/max_iy = 0 do), in (n, ox, oy, c) order.
+void oracle_maxpoolGrad_f(float *inputG, const float *outputG, const float *input, const size_t *idims,
+                          const size_t *odims, const size_t *kernels, const size_t *strides, const size_t *pads) {
+    const Dims4 id(idims), od(odims);
+    const size_t kh = kernels[0], kw = kernels[1], sh = strides[0], sw = strides[1];
+    std::fill(inputG, inputG + id.d0 * id.d1 * id.d2 * id.d3, 0.f);
+    for (size_t n = 0; n < id.d0; ++n)
+        for (size_t ox = 0; ox < od.d1; ++ox)
+            for (size_t oy = 0; oy < od.d2; ++oy)
+                for (size_t c = 0; c < id.d3; ++c) {
+                    const ssize_t ixb = (ssize_t)(ox * sh) - (ssize_t)pads[0];
+                    const ssize_t iyb = (ssize_t)(oy * sw) - (ssize_t)pads[1];
+                    bool uninit = true;
+                    float mx = 0;
+                    size_t mix = 0, miy = 0;
+                    for (size_t kx = 0; kx < kh; ++kx)
+                        for (size_t ky = 0; ky < kw; ++ky) {
+                            const ssize_t ix = ixb + (ssize_t)kx, iy = iyb + (ssize_t)ky;
+                            if (ix < 0 || ix >= (ssize_t)id.d1 || iy < 0 || iy >= (ssize_t)id.d2) continue;
+                            const float v = input[id.at(n, ix, iy, c)];
+                            if (uninit || v > mx) {
+                                mx = v;
+                                mix = ix;
+                                miy = iy;
+                                uninit = false;
+                            }
+                        }
+                    inputG[id.at(n, mix, miy, c)] += outputG[od.at(n, ox, oy, c)];
+                }
+}
+
+// kernels.h:554-563.  dest[n] = sum of slice n (sliceSize consecutive floats), in
+// order, in fp32 — a sum per ROW of the [numSlice, sliceSize] matrix, numSlice results.
+void oracle_batchedreduceadd_f(float *dest, const float *batch, size_t numSlice, size_t sliceSize) {
+    for (size_t n = 0; n < numSlice; ++n) {
+        float sum = 0;
+        for (size_t i = 0; i < sliceSize; ++i) sum += batch[n * sliceSize + i];
+        dest[n] = sum;
+    }
+}
+
+// kernels.h:565-573.  neglr = -lr / batch (fp32);
+// negDelta = fl(fl(fl(fl(w*decay) + dw) * neglr) + fl(mom*momentum)); mom = negDelta; out += negDelta.
+void oracle_sgd_f(size_t size, float *out, float *w, float *dw, float *dw_mom, float lr, float decay, float momentum,
+                  size_t batch) {
+    const float neglr = -lr / batch;
+    for (size_t i = 0; i < size; ++i) {
+        const float negDelta = (w[i] * decay + dw[i]) * neglr + dw_mom[i] * momentum;
+        dw_mom[i] = negDelta;
+        out[i] += negDelta;
+    }
+}
+
+// kernels.h:586-590.  srcGrad = (src > 0) ? destGrad : 0.
+void oracle_reluGrad_f(float *srcGrad, const float *src, const float *destGrad, size_t size) {
+    for (size_t i = 0; i < size; ++i) srcGrad[i] = (src[i] > 0) ? destGrad[i] : 0;
+}
 
 } // extern "C"
 

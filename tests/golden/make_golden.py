@@ -22,6 +22,60 @@ OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "kernels_golden.n
 F = np.float32
 
 
+def training(ref, g):
+    """fixtures of the training kernels (their own random stream, so the arrays above never change)"""
+    rng = np.random.default_rng(0x7EA1)
+    convs = {
+        "p1": ((2, 9, 9, 4), (5, 3, 3, 4), (1, 1), (1, 1, 1, 1)),
+        "s2": ((2, 11, 10, 6), (7, 3, 3, 6), (2, 2), (1, 1, 1, 1)),
+        "k5": ((1, 12, 12, 1), (5, 5, 5, 1), (1, 1), (0, 0, 0, 0)),
+        "asym": ((1, 8, 7, 4), (3, 3, 2, 4), (1, 2), (2, 0, 1, 1)),
+        "c32": ((2, 6, 6, 32), (16, 3, 3, 32), (1, 1), (1, 1, 1, 1)),
+    }
+    for tag, (idims, fdims, strides, pads) in convs.items():
+        x = rng.standard_normal(idims).astype(F)
+        f = (rng.standard_normal(fdims) / np.sqrt(fdims[1] * fdims[2] * fdims[3])).astype(F)
+        y = ref.conv2d(x, f, np.zeros(fdims[0], F), fdims[1:3], strides, pads)
+        og = rng.standard_normal(y.shape).astype(F)
+        g[f"cgrad_{tag}_x"], g[f"cgrad_{tag}_f"], g[f"cgrad_{tag}_og"] = x, f, og
+        g[f"cgrad_{tag}_sp"] = np.array(list(strides) + list(pads), np.int64)
+        g[f"cgrad_{tag}_ig"], g[f"cgrad_{tag}_fg"], g[f"cgrad_{tag}_bg"] = ref.conv2dGrad(x, f, og, fdims[1:3], strides, pads)
+    # maxpool gradient with real-valued gradients; overlapping windows accumulate (k3s1, k3s2p1)
+    pools = {"k2": ((2, 8, 8, 5), (2, 2), (2, 2), (0, 0, 0, 0)), "k3s2p1": ((2, 7, 9, 4), (3, 3), (2, 2), (1, 1, 1, 1)),
+             "k3s1": ((1, 6, 6, 3), (3, 3), (1, 1), (1, 1, 1, 1))}
+    for tag, (idims, kernels, strides, pads) in pools.items():
+        x = np.round(rng.standard_normal(idims) * 2).astype(F) / F(2)
+        y = ref.maxpool(x, kernels, strides, pads)
+        og = rng.standard_normal(y.shape).astype(F)
+        g[f"pgrad_{tag}_x"], g[f"pgrad_{tag}_og"] = x, og
+        g[f"pgrad_{tag}_ksp"] = np.array(list(kernels) + list(strides) + list(pads), np.int64)
+        g[f"pgrad_{tag}_ig"] = ref.maxpoolGrad(x, og, kernels, strides, pads)
+    # softmax with loss, its gradient
+    for tag, (m, n, sigma) in {"a": (8, 10, 1.0), "b": (5, 1000, 3.0), "c": (33, 67, 10.0)}.items():
+        x = (rng.standard_normal((m, n)) * sigma).astype(F)
+        sel = rng.integers(0, n, m).astype(np.int32)
+        p, loss = ref.matrixSoftmaxWithLoss(x, sel)
+        g[f"swl_{tag}_x"], g[f"swl_{tag}_sel"], g[f"swl_{tag}_p"], g[f"swl_{tag}_loss"] = x, sel, p, np.array([loss], F)
+        g[f"swl_{tag}_grad"] = ref.matrixSoftmaxGrad(p, sel, with_loss=True)
+    # tanh gradient, transpose, relu gradient (with specials), row sums, sgd
+    t = ref.matrixTanh((rng.standard_normal((6, 40)) * 2).astype(F))
+    og = rng.standard_normal(t.shape).astype(F)
+    g["tanhgrad_y"], g["tanhgrad_og"], g["tanhgrad_ig"] = t, og, ref.matrixTanhGrad(t, og)
+    a = rng.standard_normal((37, 53)).astype(F)
+    g["mtrans_x"], g["mtrans_y"] = a, ref.matrixTrans(a)
+    x = rng.standard_normal(1031).astype(F)
+    x[:8] = [0.0, -0.0, np.nan, np.inf, -np.inf, 1e-45, -1e-45, 3.0]
+    dg = rng.standard_normal(1031).astype(F)
+    dg[8:12] = [np.nan, np.inf, -0.0, 0.0]
+    g["relugrad_x"], g["relugrad_dg"], g["relugrad_sg"] = x, dg, ref.reluGrad(x, dg)
+    b = rng.standard_normal((19, 300)).astype(F)
+    g["rowsum_x"], g["rowsum_y"] = b, ref.batchedreduceadd(b)
+    w, dw, mom = (rng.standard_normal(777).astype(F) for _ in range(3))
+    g["sgd_w"], g["sgd_dw"], g["sgd_mom"] = w, dw, mom
+    g["sgd_params"] = np.array([0.01, 0.0005, 0.9, 16], np.float64)
+    g["sgd_w1"], g["sgd_mom1"] = ref.sgd(w, dw, mom, 0.01, 0.0005, 0.9, 16)
+
+
 def main():
     ref = load_ref()
     rng = np.random.default_rng(0x5C0DE)
@@ -135,6 +189,8 @@ def main():
     h = ref.matrixTanh(ref.fcbias(img, w0, b0))
     g["mnist8_prob"] = ref.matrixSoftmax(ref.fcbias(h, w1, b1))
     g["mnist8_top3"] = ref.argMax(g["mnist8_prob"], 3)
+
+    training(ref, g)
 
     np.savez_compressed(OUT, **g)
     print("wrote", OUT, os.path.getsize(OUT), "bytes,", len(g), "arrays")
