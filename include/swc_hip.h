@@ -19,7 +19,10 @@
  *     reference's CUDA path uses one stream per GPU,
  *     src/codegen/Codegen.cpp:166-172); call swc_hip_sync() before reading
  *     results on the host.  swc_hip_d2h synchronises by itself.
- * Nothing here allocates device memory except swc_hip_malloc.
+ * Nothing here allocates device memory except swc_hip_malloc and, when no
+ * workspace has been provided, the two ops that need scratch memory
+ * (swc_hip_conv2dGrad_f, swc_hip_matrixSoftmaxWithLoss_f; see
+ * swc_hip_set_workspace).
  * Layouts are the reference's: 4-D activations NHWC, conv filters
  * [oC, kH, kW, iC], matrices row-major.  All data is fp32.
  */
@@ -53,6 +56,14 @@ int swc_hip_d2h(void *dst_host, const void *src_dev, size_t bytes); /* ordered a
 int swc_hip_d2d(void *dst_dev, const void *src_dev, size_t bytes);  /* async on the stream */
 int swc_hip_fill_f(float *dst_dev, float value, size_t count);      /* initTensorConstant/Zero, kernels.h:23-29 */
 int swc_hip_sync(void);
+/* Scratch device memory for the ops that need some (conv2dGrad_f: the
+ * transposed gradient and operand copies, up to about twice the size of its
+ * largest argument; matrixSoftmaxWithLoss_f: 4*m bytes).  A generated program
+ * reserves a slot of its arena and passes it here once; without this call the
+ * library allocates a buffer of its own on first need and grows it on demand
+ * (not possible while a graph is being recorded).  dptr NULL, bytes 0: back to
+ * the library's own buffer.  The buffer is shared by all ops on the stream. */
+int swc_hip_set_workspace(void *dptr, size_t bytes);
 const char *swc_hip_last_error(void);         /* message of the last failure on this thread ("" if none) */
 void *swc_hip_stream(void);                   /* the hipStream_t ops are launched on */
 int swc_hip_set_stream(void *hip_stream);     /* launch on a caller-owned stream (NULL: back to the library's own) */
@@ -163,6 +174,63 @@ int swc_hip_matrixTanh_f(int m, int n, const float *a, int lda, float *b,
 /* kernels.h:601-613; Codegen.cpp:2372-2385 (ArgMax op).  idx[m,top_k] = columns of the top_k largest
  * values of each row, ties listing the larger column first. top_k <= 8. */
 int swc_hip_argMax_i(const float *input, int *idx, int m, int n, int top_k);
+
+/* ---- training kernels: same arguments as the reference's; `selected` and `loss`
+ * are device pointers like every other data pointer ---- */
+
+/* kernels.h:68-76 (the generator emits transpose2d_f for MatrixTranspose, Codegen.cpp:2220-2284; matrixTrans_f is
+ * the hand-written form of the same operation with leading dimensions).  b[n,m] = a[m,n]^T. */
+int swc_hip_matrixTrans_f(int m, int n, const float *a, int lda, float *b, int ldb);
+
+/* kernels.h:79-86; Codegen.cpp:2414-2427.  a = (1 - b*b) * c: b the tanh output,
+ * c the gradient arriving at it, a the gradient of the tanh input.  Bit-exact. */
+int swc_hip_matrixTanhGrad_f(int m, int n, float *a, int lda, const float *b, int ldb,
+                             const float *c, int ldc);
+
+/* kernels.h:105-129; Codegen.cpp:2357-2370.  b = row softmax of a (as
+ * matrixSoftmax_f); *loss = mean over rows of logf(sum*expf(max)) - a[row, selected[row]],
+ * the rows added in order in fp32.  b may alias a. */
+int swc_hip_matrixSoftmaxWithLoss_f(int m, int n, const float *a, int lda, float *b, int ldb,
+                                    const int *selected, float *loss);
+
+/* kernels.h:133-151; Codegen.cpp:2429-2465.  a = b - onehot(selected): the
+ * gradient of the SUM (not the mean) of the rows' losses.  Bit-exact. */
+int swc_hip_matrixSoftmaxGrad_f(int m, int n, float *a, int lda, const float *b, int ldb,
+                                const int *selected);
+int swc_hip_matrixSoftmaxWithLossGrad_f(int m, int n, float *a, int lda, const float *b, int ldb,
+                                        const int *selected);
+
+/* kernels.h:245-319; Codegen.cpp:1785-1830.  Gradients of conv2d_f with respect to
+ * input, filter and bias from the gradient of its output; all three are
+ * overwritten.  biasG follows the reference literally: an output pixel whose
+ * first tap (0,0) lies in the padding does not contribute.  group must be 1. */
+int swc_hip_conv2dGrad_f(float *inputG, float *filterG, float *biasG, const float *outputG,
+                         const float *input, const float *filter, const size_t *odims,
+                         const size_t *idims, const size_t *fdims, const size_t *bdims,
+                         const size_t *kernels, const size_t *strides, const size_t *pads,
+                         size_t group);
+
+/* kernels.h:380-442; Codegen.cpp:2047-2079.  inputG = 0, then every output
+ * element adds its gradient to the input element its window selected (first
+ * maximum in scan order), in the reference's accumulation order: bit-exact,
+ * also for overlapping windows. */
+int swc_hip_maxpoolGrad_f(float *inputG, const float *outputG, const float *input,
+                          const size_t *idims, const size_t *odims, const size_t *kernels,
+                          const size_t *strides, const size_t *pads);
+
+/* kernels.h:554-563; Codegen.cpp:1517-1531.  dest[s] = sum of slice s (sliceSize
+ * consecutive floats of batch) added in order in fp32 — one result per ROW of the
+ * [numSlice, sliceSize] matrix, exactly as the reference computes it (its call
+ * site passes a dest of sliceSize floats; dest must hold numSlice).  Bit-exact. */
+int swc_hip_batchedreduceadd_f(float *dest, const float *batch, size_t numSlice, size_t sliceSize);
+
+/* kernels.h:565-573; Codegen.cpp:2468-2489.  neglr = -lr/batch;
+ * d = (w*decay + dw)*neglr + dw_mom*momentum; dw_mom = d; out += d.  out may be w.  Bit-exact. */
+int swc_hip_sgd_f(size_t size, float *out, float *w, float *dw, float *dw_mom, float lr,
+                  float decay, float momentum, size_t batch);
+
+/* kernels.h:586-590; Codegen.cpp:2138-2148.  srcGrad = (src > 0) ? destGrad : 0.  Bit-exact. */
+int swc_hip_reluGrad_f(float *srcGrad, const float *src, const float *destGrad, size_t size);
 
 /* ---- fused ops: what the HIP target emits when the graph allows.  Each equals
  * the named sequence of reference kernels. ---- */

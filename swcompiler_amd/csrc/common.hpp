@@ -19,6 +19,8 @@ void clear_error();
 hipStream_t stream();
 bool ready();
 int num_cus();
+// Scratch device memory for the current op (see runtime.hip); nullptr with the error recorded on failure.
+void *workspace(size_t bytes, const char *who);
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -12,6 +12,7 @@
 // the gather uses 128-bit loads; otherwise (first layer, iC = 1 or 3) 32-bit.
 #include "common.hpp"
 #include "mfma_dma.hpp"
+#include "mfma_dma2.hpp"
 #include "mfma_tile.hpp"
 #include <cstdlib>
 #include <cstring>
@@ -359,7 +360,7 @@ __global__ __launch_bounds__(256) void conv_direct(const float *__restrict__ in,
     const bool bn = ep.bn_mean != nullptr;
     if (threadIdx.x < OCP) {
         const int oc = threadIdx.x;
-        bsh[oc] = oc < OC ? bias[oc] : 0.f;
+        bsh[oc] = (oc < OC && bias) ? bias[oc] : 0.f;
         if (bn && oc < OC) {
             mean_sh[oc] = ep.bn_mean[oc];
             slope_sh[oc] = (float)((double)ep.bn_scale[oc] / sqrt((double)(ep.bn_var[oc] + ep.eps)));
@@ -473,7 +474,8 @@ int launch_conv(bool vec, const float *in, const float *filt, float *out, const 
 
 int conv_dispatch(const char *who, float *output, const float *input, const float *filter, const float *bias,
                   const size_t *odims, const size_t *idims, const size_t *fdims, const size_t *kernels,
-                  const size_t *strides, const size_t *pads, size_t group, const Epilogue &ep_in) {
+                  const size_t *strides, const size_t *pads, size_t group, const Epilogue &ep_in,
+                  bool bias_optional = false) {
     if (!odims || !idims || !fdims || !kernels || !strides || !pads)
         return fail(SWC_HIP_EINVAL, "%s: null shape array", who);
     if (group != 1) return fail(SWC_HIP_EUNSUPPORTED, "%s: group = %zu (only 1 is supported)", who, group);
@@ -492,7 +494,7 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
     if (M > 0x7fffffffu || K > 0x7fffffffu || M * odims[3] > (size_t)1 << 40)
         return fail(SWC_HIP_EINVAL, "%s: problem too large", who);
     if (M == 0 || odims[3] == 0) return SWC_HIP_OK;
-    if (!output || !input || !filter || !bias) return fail(SWC_HIP_EINVAL, "%s: null pointer", who);
+    if (!output || !input || !filter || (!bias && !bias_optional)) return fail(SWC_HIP_EINVAL, "%s: null pointer", who);
     ConvGeom g{(int)idims[0], (int)idims[1], (int)idims[2], (int)idims[3], (int)odims[1], (int)odims[2],
                (int)odims[3], (int)kernels[0], (int)kernels[1], (int)strides[0], (int)strides[1], (int)pads[0],
                (int)pads[1], (int)M, (int)K};
@@ -539,6 +541,329 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
     return launch_conv<1, 1>(vec, input, filter, output, g, ep);
 }
 
+// =================================================================== gradients
+// conv2dGrad_f (kernels.h:245-319), group 1.  Three independent results:
+//
+//   inputG  [N,H,W,iC]   = sum over (co,ky,kx) filter[co,ky,kx,ci] * outputG[n,oy,ox,co]
+//       For stride 1 this is itself a convolution — of outputG with the filter
+//       turned by 180 degrees and its channel axes swapped, padded by
+//       (kh-1-pt, kw-1-pl) — and runs on the forward kernels above; the turned
+//       filter is built in the workspace.  Other strides: a direct gather.
+//   filterG [oC,kh,kw,iC] = outputG^T [oC, M] * im2col(input) [M, kh*kw*iC]
+//       A GEMM whose K is the pixel count M (10^4..10^5) and whose result is
+//       small: it runs on the column-interleaved kernel body (mfma_dma2.hpp)
+//       with the im2col matrix gathered on the fly as the B operand, outputG
+//       transposed once into the workspace so that M is the contiguous axis of
+//       the A operand, and K split over blockIdx.y; the splits' partial results
+//       are summed in split order by a second kernel (deterministic).
+//   biasG   [oC]          = column sums of outputG over the pixels whose first
+//       tap (0,0) is inside the image (the reference adds it after the bounds
+//       test of that tap); two passes, partial sums in the workspace.
+//
+// inputG and filterG are sums of the same fp32 products as the reference's, in
+// a different order.
+
+// turned[ci][ky][kx][co] = filter[co][kh-1-ky][kw-1-kx][ci]
+__global__ __launch_bounds__(256) void turn_filter(const float *__restrict__ filt, float *__restrict__ turned, int OC,
+                                                   int kh, int kw, int C) {
+    const int total = OC * kh * kw * C;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
+        const int co = i % OC;
+        int t = i / OC;
+        const int kx = t % kw;
+        t /= kw;
+        const int ky = t % kh;
+        const int ci = t / kh;
+        turned[i] = filt[((co * kh + (kh - 1 - ky)) * kw + (kw - 1 - kx)) * C + ci];
+    }
+}
+
+// any stride: one thread per input element gathers the taps that reach it
+__global__ __launch_bounds__(256) void dgrad_direct(float *__restrict__ ig, const float *__restrict__ og,
+                                                    const float *__restrict__ filt, ConvGeom g) {
+    const size_t total = (size_t)g.N * g.H * g.W * g.C;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const int ci = (int)(i % g.C);
+        size_t t = i / g.C;
+        const int ix = (int)(t % g.W);
+        t /= g.W;
+        const int iy = (int)(t % g.H);
+        const int n = (int)(t / g.H);
+        float sum = 0.f;
+        for (int ky = 0; ky < g.kh; ++ky) {
+            const int ny = iy + g.pt - ky;
+            if (ny < 0 || ny % g.sh != 0 || ny / g.sh >= g.OH) continue;
+            for (int kx = 0; kx < g.kw; ++kx) {
+                const int nx = ix + g.pl - kx;
+                if (nx < 0 || nx % g.sw != 0 || nx / g.sw >= g.OW) continue;
+                const float *o = og + (((size_t)n * g.OH + ny / g.sh) * g.OW + nx / g.sw) * g.OC;
+                const float *f = filt + ((size_t)ky * g.kw + kx) * g.C + ci;
+                for (int co = 0; co < g.OC; ++co) sum += f[(size_t)co * g.K] * o[co];
+            }
+        }
+        ig[i] = sum;
+    }
+}
+
+// ---- filter gradient: B operand = im2col(input), gathered
+struct Im2colB {
+    const float *in;
+    unsigned bytes;
+    int H, W, C, OH, OW, kw, sh, sw, pt, pl, nimg;
+    int q32, r32;   // 32 / OW, 32 % OW: how a slice of 32 pixels moves (oy, ox)
+    struct Lane {
+        int img, oy, ox, ty, tx, cbase, krow;
+        bool ok;
+    };
+#if __HIP_DEVICE_COMPILE__
+    __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc() const {
+        return make_rsrc(reinterpret_cast<const char *>(in) - kImmSpan, bytes + kImmSpan);
+    }
+    // row krow of a slice is output pixel k_begin + krow (+32 per slice); column col is (ky, kx, ci)
+    __device__ __forceinline__ Lane init(int krow, int col, bool col_ok, int imm, int k_begin) const {
+        Lane s;
+        const int pix = k_begin + krow;
+        s.ox = pix % OW;
+        const int t = pix / OW;
+        s.oy = t % OH;
+        s.img = t / OH;
+        const int tap = col / C;
+        s.ty = tap / kw;
+        s.tx = tap - s.ty * kw;
+        s.cbase = (col - tap * C) * 4 + kImmSpan - imm;
+        s.krow = krow;
+        s.ok = col_ok;
+        return s;
+    }
+    __device__ __forceinline__ int voffset(const Lane &s, int k0, int k_end) const {
+        const int iy = s.oy * sh - pt + s.ty, ix = s.ox * sw - pl + s.tx;
+        const bool valid = s.ok && k0 + s.krow < k_end && s.img < nimg && (unsigned)iy < (unsigned)H &&
+                           (unsigned)ix < (unsigned)W;
+        return valid ? ((s.img * H + iy) * W + ix) * C * 4 + s.cbase : kOutOfRange;
+    }
+    __device__ __forceinline__ int soffset(int) const { return 0; }
+    __device__ __forceinline__ void advance(Lane &s) const {
+        s.ox += r32;
+        s.oy += q32;
+        if (s.ox >= OW) {
+            s.ox -= OW;
+            ++s.oy;
+        }
+        while (s.oy >= OH) {
+            s.oy -= OH;
+            ++s.img;
+        }
+    }
+#endif
+};
+
+template <int TM, int TN, int WM, int STAGES, bool MID, int NW>
+__global__ __launch_bounds__(64 * NW) void conv_wgrad(const float *__restrict__ ogT, unsigned a_bytes, int lda,
+                                                       Im2colB bsrc, float *__restrict__ part, size_t split_stride,
+                                                       int OC, int Kf, int M, int slices_per_split) {
+#if __HIP_DEVICE_COMPILE__
+    const int k_begin = blockIdx.y * slices_per_split * BK;
+    const int k_stop = k_begin + slices_per_split * BK;
+    const Epilogue ep{nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
+    dma2_tile_body<TM, TN, WM, STAGES, MID, NW>(ogT, a_bytes, lda, bsrc, part + blockIdx.y * split_stride, (size_t)Kf, OC,
+                                                Kf, k_begin, k_stop < M ? k_stop : M, ep);
+#endif
+}
+
+template <int TM, int TN, int WM, int STAGES, bool MID, int NW>
+int launch_wgrad(const float *ogT, size_t a_bytes, int lda, const Im2colB &bsrc, float *part, int OC, int Kf, int M,
+                 int splits, int sps) {
+    using T = Dma2Tile<TM, TN, WM, STAGES, NW>;
+    auto kern = conv_wgrad<TM, TN, WM, STAGES, MID, NW>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        SWC_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)T::kLdsBytes));
+        attr_set = true;
+    }
+    const unsigned tiles = (unsigned)(((OC + T::BM - 1) / T::BM) * ((Kf + T::BN - 1) / T::BN));
+    kern<<<dim3(tiles, splits), T::kThreadsWg, T::kLdsBytes, stream()>>>(ogT, (unsigned)a_bytes, lda, bsrc, part,
+                                                                         (size_t)OC * Kf, OC, Kf, M, sps);
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
+}
+
+// out[i] = part[0][i] + part[1][i] + ... in split order
+__global__ __launch_bounds__(256) void sum_splits(float *__restrict__ out, const float *__restrict__ part, size_t n,
+                                                  int splits) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        float s = part[i];
+        for (int k = 1; k < splits; ++k) s += part[(size_t)k * n + i];
+        out[i] = s;
+    }
+}
+
+// any shape: one workgroup per filter element, pixels strided over its threads
+__global__ __launch_bounds__(256) void wgrad_direct(float *__restrict__ fg, const float *__restrict__ og,
+                                                    const float *__restrict__ in, ConvGeom g) {
+    __shared__ float red[256];
+    const int e = blockIdx.x;   // (co, ky, kx, ci)
+    const int ci = e % g.C;
+    int t = e / g.C;
+    const int kx = t % g.kw;
+    t /= g.kw;
+    const int ky = t % g.kh;
+    const int co = t / g.kh;
+    float sum = 0.f;
+    for (int m = threadIdx.x; m < g.M; m += 256) {
+        const int ox = m % g.OW;
+        const int t2 = m / g.OW;
+        const int oy = t2 % g.OH;
+        const int n = t2 / g.OH;
+        const int iy = oy * g.sh - g.pt + ky, ix = ox * g.sw - g.pl + kx;
+        if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W)
+            sum += in[(((size_t)n * g.H + iy) * g.W + ix) * g.C + ci] * og[(size_t)m * g.OC + co];
+    }
+    red[threadIdx.x] = sum;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if (threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) fg[e] = red[0];
+}
+
+// ---- bias gradient: masked column sums of outputG [M, OC]
+constexpr int kBiasRows = 512;   // rows per partial sum
+__global__ __launch_bounds__(256) void bias_partials(float *__restrict__ part, const float *__restrict__ og, ConvGeom g) {
+    __shared__ float red[256];
+    const int co = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int sub = threadIdx.x >> 6;   // 4 row phases
+    const int m0 = blockIdx.y * kBiasRows;
+    const int m1 = m0 + kBiasRows < g.M ? m0 + kBiasRows : g.M;
+    float sum = 0.f;
+    if (co < g.OC)
+        for (int m = m0 + sub; m < m1; m += 4) {
+            const int ox = m % g.OW, oy = (m / g.OW) % g.OH;
+            const int iy = oy * g.sh - g.pt, ix = ox * g.sw - g.pl;
+            if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W) sum += og[(size_t)m * g.OC + co];
+        }
+    red[threadIdx.x] = sum;
+    __syncthreads();
+    if (sub == 0 && co < g.OC)
+        part[(size_t)blockIdx.y * g.OC + co] = (red[threadIdx.x] + red[threadIdx.x + 64]) + (red[threadIdx.x + 128] + red[threadIdx.x + 192]);
+}
+
+size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG, const float *input,
+              const float *filter, const size_t *odims, const size_t *idims, const size_t *fdims,
+              const size_t *kernels, const size_t *strides, const size_t *pads, size_t group) {
+    const char *who = "swc_hip_conv2dGrad_f";
+    if (!odims || !idims || !fdims || !kernels || !strides || !pads) return fail(SWC_HIP_EINVAL, "%s: null shape array", who);
+    if (group != 1) return fail(SWC_HIP_EUNSUPPORTED, "%s: group = %zu (only 1 is supported)", who, group);
+    for (int i = 0; i < 4; ++i)
+        if (odims[i] > 0x7fffffffu || idims[i] > 0x7fffffffu || fdims[i] > 0x7fffffffu)
+            return fail(SWC_HIP_EINVAL, "%s: dimension too large", who);
+    if (odims[0] != idims[0] || fdims[0] != odims[3] || fdims[3] != idims[3] || fdims[1] != kernels[0] ||
+        fdims[2] != kernels[1])
+        return fail(SWC_HIP_EINVAL, "%s: output, input and filter dims do not fit together", who);
+    if (strides[0] == 0 || strides[1] == 0 || strides[0] > 4096 || strides[1] > 4096 || pads[0] > 4096 ||
+        pads[1] > 4096 || kernels[0] == 0 || kernels[1] == 0)
+        return fail(SWC_HIP_EINVAL, "%s: bad kernel/stride/pad", who);
+    const size_t M = odims[0] * odims[1] * odims[2];
+    const size_t Kf = fdims[1] * fdims[2] * fdims[3];
+    const size_t in_elems = idims[0] * idims[1] * idims[2] * idims[3], f_elems = fdims[0] * Kf;
+    if (M > 0x7fffffffu || Kf > 0x7fffffffu || in_elems * 4 >= kMaxDmaBytes || M * odims[3] * 4 >= kMaxDmaBytes ||
+        f_elems * 4 >= kMaxDmaBytes)
+        return fail(SWC_HIP_EUNSUPPORTED, "%s: tensors of 2 GiB and more are not supported", who);
+    if (!inputG || !filterG || !biasG || !outputG || !input || !filter) return fail(SWC_HIP_EINVAL, "%s: null pointer", who);
+    ConvGeom g{(int)idims[0], (int)idims[1], (int)idims[2], (int)idims[3], (int)odims[1], (int)odims[2],
+               (int)odims[3], (int)kernels[0], (int)kernels[1], (int)strides[0], (int)strides[1], (int)pads[0],
+               (int)pads[1], (int)M, (int)Kf};
+    if (in_elems == 0 && f_elems == 0 && g.OC == 0) return SWC_HIP_OK;
+    if (M == 0 || g.OC == 0 || in_elems == 0 || f_elems == 0) {   // no products: the gradients are zero
+        int rc = SWC_HIP_OK;   // fill kernels, not memset nodes: this may be recorded into a graph
+        if (in_elems) rc = swc_hip_fill_f(inputG, 0.f, in_elems);
+        if (rc == SWC_HIP_OK && f_elems) rc = swc_hip_fill_f(filterG, 0.f, f_elems);
+        if (rc == SWC_HIP_OK && g.OC) rc = swc_hip_fill_f(biasG, 0.f, (size_t)g.OC);
+        return rc;
+    }
+
+    // ---- workspace layout
+    const bool dgrad_conv = g.sh == 1 && g.sw == 1 && g.pt <= g.kh - 1 && g.pl <= g.kw - 1;
+    const bool wgrad_mfma = g.C % 4 == 0 && aligned16(input) && aligned16(outputG) && aligned16(filterG);
+    const int lda = (int)((M + 3) & ~(size_t)3);   // row length of the transposed outputG
+    const int bias_chunks = (int)((M + kBiasRows - 1) / kBiasRows);
+    // filter-gradient tiles and splits: about three workgroups per CU
+    const bool narrow = g.OC <= 64;
+    const int bm = narrow ? 64 : 128, bn = narrow ? 256 : 128;
+    const int tiles = ((g.OC + bm - 1) / bm) * (int)((Kf + bn - 1) / bn);
+    const int nk = (int)((M + BK - 1) / BK);
+    int splits = (3 * num_cus() + tiles - 1) / tiles;
+    splits = splits < 1 ? 1 : (splits > nk ? nk : splits);
+    const int sps = (nk + splits - 1) / splits;
+    splits = (nk + sps - 1) / sps;
+    const size_t turned_b = dgrad_conv ? align256(f_elems * 4) : 0;
+    const size_t ogt_b = wgrad_mfma ? align256((size_t)g.OC * lda * 4) : 0;
+    const size_t part_b = wgrad_mfma && splits > 1 ? align256((size_t)splits * f_elems * 4) : 0;
+    const size_t bias_b = align256((size_t)bias_chunks * g.OC * 4);
+    char *ws = static_cast<char *>(workspace(turned_b + ogt_b + part_b + bias_b, who));
+    if (!ws) return SWC_HIP_ERUNTIME;
+    float *turned = reinterpret_cast<float *>(ws);
+    float *ogT = reinterpret_cast<float *>(ws + turned_b);
+    float *part = reinterpret_cast<float *>(ws + turned_b + ogt_b);
+    float *bias_part = reinterpret_cast<float *>(ws + turned_b + ogt_b + part_b);
+
+    // ---- bias gradient
+    bias_partials<<<dim3((g.OC + 63) / 64, bias_chunks), 256, 0, stream()>>>(bias_part, outputG, g);
+    SWC_LAUNCH_CHECK();
+    sum_splits<<<ceil_div(g.OC, 256), 256, 0, stream()>>>(biasG, bias_part, (size_t)g.OC, bias_chunks);
+    SWC_LAUNCH_CHECK();
+
+    // ---- input gradient
+    if (dgrad_conv) {
+        unsigned blocks = ceil_div(f_elems, 256);
+        turn_filter<<<blocks > 1024 ? 1024 : blocks, 256, 0, stream()>>>(filter, turned, g.OC, g.kh, g.kw, g.C);
+        SWC_LAUNCH_CHECK();
+        const size_t t_odims[4] = {idims[0], idims[1], idims[2], idims[3]};
+        const size_t t_idims[4] = {odims[0], odims[1], odims[2], odims[3]};
+        const size_t t_fdims[4] = {idims[3], kernels[0], kernels[1], odims[3]};
+        const size_t t_strides[2] = {1, 1};
+        const size_t t_pads[4] = {(size_t)(g.kh - 1 - g.pt), (size_t)(g.kw - 1 - g.pl), 0, 0};
+        const Epilogue ep{nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
+        const int rc = conv_dispatch(who, inputG, outputG, turned, nullptr, t_odims, t_idims, t_fdims, kernels, t_strides,
+                                     t_pads, 1, ep, /*bias_optional=*/true);
+        if (rc != SWC_HIP_OK) return rc;
+    } else {
+        unsigned blocks = ceil_div(in_elems, 256);
+        dgrad_direct<<<blocks > 65536 ? 65536 : blocks, 256, 0, stream()>>>(inputG, outputG, filter, g);
+        SWC_LAUNCH_CHECK();
+    }
+
+    // ---- filter gradient
+    if (wgrad_mfma) {
+        // the 128-bit loads of the last k chunk reach into the row padding: it must hold zeros, not stale bits
+        if ((size_t)lda != M) {
+            const int rc0 = swc_hip_fill_f(ogT, 0.f, (size_t)g.OC * lda);
+            if (rc0 != SWC_HIP_OK) return rc0;
+        }
+        const int rc = swc_hip_matrixTrans_f((int)M, g.OC, outputG, g.OC, ogT, lda);
+        if (rc != SWC_HIP_OK) return rc;
+        const Im2colB bsrc{input, (unsigned)(in_elems * 4), g.H, g.W, g.C, g.OH, g.OW, g.kw, g.sh, g.sw, g.pt, g.pl, g.N,
+                           BK / g.OW, BK % g.OW};
+        float *dst = splits > 1 ? part : filterG;
+        const size_t a_bytes = ((size_t)(g.OC - 1) * lda + M) * 4;
+        const int rc2 = narrow ? launch_wgrad<1, 4, 2, 2, false, 4>(ogT, a_bytes, lda, bsrc, dst, g.OC, (int)Kf, (int)M, splits, sps)
+                               : launch_wgrad<1, 4, 4, 2, false, 4>(ogT, a_bytes, lda, bsrc, dst, g.OC, (int)Kf, (int)M, splits, sps);
+        if (rc2 != SWC_HIP_OK) return rc2;
+        if (splits > 1) {
+            unsigned blocks = ceil_div(f_elems, 256);
+            sum_splits<<<blocks > 4096 ? 4096 : blocks, 256, 0, stream()>>>(filterG, part, f_elems, splits);
+            SWC_LAUNCH_CHECK();
+        }
+    } else {
+        wgrad_direct<<<(unsigned)f_elems, 256, 0, stream()>>>(filterG, outputG, input, g);
+        SWC_LAUNCH_CHECK();
+    }
+    return SWC_HIP_OK;
+}
+
 } // namespace
 
 extern "C" {
@@ -565,6 +890,15 @@ int swc_hip_conv2dFused_f(float *output, const float *input, const float *filter
     Epilogue ep{nullptr, bn_mean, bn_var, bn_scale, bn_bias, epsilon, relu};
     return conv_dispatch("swc_hip_conv2dFused_f", output, input, filter, bias, odims, idims, fdims, kernels, strides,
                          pads, group, ep);
+}
+
+int swc_hip_conv2dGrad_f(float *inputG, float *filterG, float *biasG, const float *outputG, const float *input,
+                         const float *filter, const size_t *odims, const size_t *idims, const size_t *fdims,
+                         const size_t *bdims, const size_t *kernels, const size_t *strides, const size_t *pads,
+                         size_t group) {
+    SWC_REQUIRE_INIT();
+    (void)bdims;
+    return conv_grad(inputG, filterG, biasG, outputG, input, filter, odims, idims, fdims, kernels, strides, pads, group);
 }
 
 } // extern "C"

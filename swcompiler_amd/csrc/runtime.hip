@@ -26,6 +26,10 @@ struct State {
     hipEvent_t slots[kEventSlots] = {};
     bool capturing = false;
     char arch[64] = "";
+    // workspace of the ops that need one (conv2dGrad_f, matrixSoftmaxWithLoss_f)
+    void *ws = nullptr;
+    size_t ws_bytes = 0;
+    bool ws_owned = false;
 } g;
 
 __global__ void fill_kernel(float *__restrict__ dst, float v, size_t n) {
@@ -47,6 +51,42 @@ void clear_error() { g_err[0] = 0; }
 hipStream_t stream() { return g.cur; }
 bool ready() { return g.ready; }
 int num_cus() { return g.cus; }
+
+// Device memory an op may use until it returns control to the stream's next op
+// (all ops run on one in-order stream, so one buffer serves them all).  The
+// caller's buffer (swc_hip_set_workspace) is used when it is large enough;
+// otherwise the library keeps one of its own and grows it on demand — never
+// while a graph is being recorded, where allocating is not allowed.
+void *workspace(size_t bytes, const char *who) {
+    if (bytes <= g.ws_bytes && g.ws) return g.ws;
+    if (g.capturing) {
+        fail(SWC_HIP_ERUNTIME, "%s: needs a %zu-byte workspace, which cannot be allocated while a graph is recorded; "
+             "run the op once eagerly first or provide one with swc_hip_set_workspace", who, bytes);
+        return nullptr;
+    }
+    if (g.ws && !g.ws_owned) {
+        fail(SWC_HIP_EINVAL, "%s: the workspace given to swc_hip_set_workspace has %zu bytes, %zu are needed", who,
+             g.ws_bytes, bytes);
+        return nullptr;
+    }
+    if (g.ws) {
+        (void)hipStreamSynchronize(g.cur);   // earlier ops may still be using it
+        (void)hipFree(g.ws);
+        g.ws = nullptr;
+        g.ws_bytes = 0;
+    }
+    const size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+    hipError_t e = hipMalloc(&g.ws, want);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        g.ws = nullptr;
+        fail(SWC_HIP_ERUNTIME, "%s: workspace of %zu bytes: %s", who, want, hipGetErrorString(e));
+        return nullptr;
+    }
+    g.ws_bytes = want;
+    g.ws_owned = true;
+    return g.ws;
+}
 
 } // namespace swc_hip
 
@@ -90,6 +130,10 @@ int swc_hip_shutdown(void) {
     std::lock_guard<std::mutex> lk(g.mu);
     if (!g.ready) return SWC_HIP_OK;
     (void)hipStreamSynchronize(g.cur);
+    if (g.ws && g.ws_owned) (void)hipFree(g.ws);
+    g.ws = nullptr;
+    g.ws_bytes = 0;
+    g.ws_owned = false;
     (void)hipEventDestroy(g.t0);
     (void)hipEventDestroy(g.t1);
     (void)hipStreamDestroy(g.own);
@@ -97,6 +141,21 @@ int swc_hip_shutdown(void) {
     g.t0 = g.t1 = nullptr;
     g.ready = false;
     g.device = -1;
+    return SWC_HIP_OK;
+}
+
+int swc_hip_set_workspace(void *dptr, size_t bytes) {
+    SWC_REQUIRE_INIT();
+    std::lock_guard<std::mutex> lk(g.mu);
+    SWC_ARG((dptr == nullptr) == (bytes == 0));
+    SWC_ARG(aligned16(dptr));
+    if (g.ws && g.ws_owned) {
+        SWC_HIP_TRY(hipStreamSynchronize(g.cur));
+        SWC_HIP_TRY(hipFree(g.ws));
+    }
+    g.ws = dptr;
+    g.ws_bytes = bytes;
+    g.ws_owned = false;
     return SWC_HIP_OK;
 }
 

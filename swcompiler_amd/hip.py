@@ -27,6 +27,9 @@ EXPORTS = [
     "swc_hip_matrixSoftmax_f", "swc_hip_matrixTanh_f", "swc_hip_argMax_i",
     "swc_hip_matrixMatrixFCBias_f", "swc_hip_vecAddRelu_f", "swc_hip_batchnormRelu_f",
     "swc_hip_batchnormReluMaxpool_f", "swc_hip_conv2dFused_f",
+    "swc_hip_set_workspace", "swc_hip_matrixTrans_f", "swc_hip_matrixTanhGrad_f", "swc_hip_matrixSoftmaxWithLoss_f",
+    "swc_hip_matrixSoftmaxGrad_f", "swc_hip_matrixSoftmaxWithLossGrad_f", "swc_hip_conv2dGrad_f",
+    "swc_hip_maxpoolGrad_f", "swc_hip_batchedreduceadd_f", "swc_hip_sgd_f", "swc_hip_reluGrad_f",
 ]
 
 
@@ -91,6 +94,17 @@ def load_library():
         "swc_hip_batchnormReluMaxpool_f": (i32, [vp, vp, vp, vp, vp, vp, szp, f32, szp, szp, szp, szp]),
         "swc_hip_conv2dFused_f": (i32, [vp, vp, vp, vp, szp, szp, szp, szp, szp, szp, szp, sz,
                                         vp, vp, vp, vp, f32, i32]),
+        "swc_hip_set_workspace": (i32, [vp, sz]),
+        "swc_hip_matrixTrans_f": (i32, [i32, i32, vp, i32, vp, i32]),
+        "swc_hip_matrixTanhGrad_f": (i32, [i32, i32, vp, i32, vp, i32, vp, i32]),
+        "swc_hip_matrixSoftmaxWithLoss_f": (i32, [i32, i32, vp, i32, vp, i32, vp, vp]),
+        "swc_hip_matrixSoftmaxGrad_f": (i32, [i32, i32, vp, i32, vp, i32, vp]),
+        "swc_hip_matrixSoftmaxWithLossGrad_f": (i32, [i32, i32, vp, i32, vp, i32, vp]),
+        "swc_hip_conv2dGrad_f": (i32, [vp, vp, vp, vp, vp, vp, szp, szp, szp, szp, szp, szp, szp, sz]),
+        "swc_hip_maxpoolGrad_f": (i32, [vp, vp, vp, szp, szp, szp, szp, szp]),
+        "swc_hip_batchedreduceadd_f": (i32, [vp, vp, sz, sz]),
+        "swc_hip_sgd_f": (i32, [sz, vp, vp, vp, vp, f32, f32, f32, sz]),
+        "swc_hip_reluGrad_f": (i32, [vp, vp, vp, sz]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -369,6 +383,74 @@ class SwcHip:
                                                             _dims(x.shape), eps, _dims(odims), _dims(kernels),
                                                             _dims(strides), _dims(pads)), "batchnormReluMaxpool_f")
         return out
+
+
+    # -- training kernels ------------------------------------------------
+    def matrixTrans(self, a):
+        m, n = a.shape
+        out = self.empty((n, m))
+        self._check(self.lib.swc_hip_matrixTrans_f(m, n, a.ptr, n, out.ptr, m), "matrixTrans_f")
+        return out
+
+    def matrixTanhGrad(self, out_, out_grad):
+        m, n = out_.shape
+        ig = self.empty(out_.shape)
+        self._check(self.lib.swc_hip_matrixTanhGrad_f(m, n, ig.ptr, n, out_.ptr, n, out_grad.ptr, n), "matrixTanhGrad_f")
+        return ig
+
+    def matrixSoftmaxWithLoss(self, a, selected):
+        """-> (probabilities DeviceArray, loss as a python float)"""
+        m, n = a.shape
+        out, loss = self.empty(a.shape), self.empty((1,))
+        self._check(self.lib.swc_hip_matrixSoftmaxWithLoss_f(m, n, a.ptr, n, out.ptr, n, selected.ptr, loss.ptr),
+                    "matrixSoftmaxWithLoss_f")
+        return out, float(loss.numpy()[0])
+
+    def matrixSoftmaxGrad(self, prob, selected, with_loss=False):
+        m, n = prob.shape
+        ig = self.empty(prob.shape)
+        fn = self.lib.swc_hip_matrixSoftmaxWithLossGrad_f if with_loss else self.lib.swc_hip_matrixSoftmaxGrad_f
+        self._check(fn(m, n, ig.ptr, n, prob.ptr, n, selected.ptr), "matrixSoftmaxGrad_f")
+        return ig
+
+    def conv2dGrad(self, x, filt, out_grad, kernels=None, strides=(1, 1), pads=(0, 0, 0, 0), group=1):
+        if kernels is None:
+            kernels = filt.shape[1:3]
+        ig, fg, bg = self.empty(x.shape), self.empty(filt.shape), self.empty((filt.shape[0],))
+        self._check(self.lib.swc_hip_conv2dGrad_f(ig.ptr, fg.ptr, bg.ptr, out_grad.ptr, x.ptr, filt.ptr,
+                                                  _dims(out_grad.shape), _dims(x.shape), _dims(filt.shape),
+                                                  _dims(bg.shape), _dims(kernels), _dims(strides), _dims(pads), group),
+                    "conv2dGrad_f")
+        return ig, fg, bg
+
+    def maxpoolGrad(self, x, out_grad, kernels, strides, pads=(0, 0, 0, 0)):
+        ig = self.empty(x.shape)
+        self._check(self.lib.swc_hip_maxpoolGrad_f(ig.ptr, out_grad.ptr, x.ptr, _dims(x.shape), _dims(out_grad.shape),
+                                                   _dims(kernels), _dims(strides), _dims(pads)), "maxpoolGrad_f")
+        return ig
+
+    def batchedreduceadd(self, batch):
+        ns, ss = batch.shape
+        out = self.empty((ns,))
+        self._check(self.lib.swc_hip_batchedreduceadd_f(out.ptr, batch.ptr, ns, ss), "batchedreduceadd_f")
+        return out
+
+    def sgd(self, w, dw, mom, lr, decay, momentum, batch):
+        """updates w and mom in place (out = w, as the generated call passes them)"""
+        self._check(self.lib.swc_hip_sgd_f(w.size, w.ptr, w.ptr, dw.ptr, mom.ptr, lr, decay, momentum, batch), "sgd_f")
+        return w, mom
+
+    def reluGrad(self, src, dest_grad):
+        out = self.empty(src.shape)
+        self._check(self.lib.swc_hip_reluGrad_f(out.ptr, src.ptr, dest_grad.ptr, src.size), "reluGrad_f")
+        return out
+
+    def set_workspace(self, arr):
+        """give the library a DeviceArray to use as scratch (None: its own buffer again)"""
+        if arr is None:
+            self._check(self.lib.swc_hip_set_workspace(None, 0), "swc_hip_set_workspace")
+        else:
+            self._check(self.lib.swc_hip_set_workspace(arr.ptr, arr.nbytes), "swc_hip_set_workspace")
 
 
 _RT = None
