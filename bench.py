@@ -22,6 +22,7 @@ Also in the line:
                 device, beside the datasheet peaks the fractions are computed from
   configs       the other synthetic configurations (samples/s and, per kernel,
                 TFLOP/s or GB/s with the fraction of the MI355X peak)
+                plus `training_kernels`: conv2dGrad, reluGrad, sgd, maxpoolGrad at those sizes
   cpu_baseline  the reference's own CPU kernels (oracle/_ref, g++ -std=c++11 -O2,
                 one thread) on the first rows of the same batch
 
@@ -217,6 +218,45 @@ def run_config(rt, graphs, cfg, steps, warmup):
                 graph_replay=dict(ms_per_step=graph_wall * 1e3 / steps, samples_per_s=batch * steps / graph_wall))
 
 
+def run_training(rt, iters=20):
+    """The training kernels at the sizes of the conv block and of the bandwidth configuration: gradients of the
+    four convolutions (2 x the forward flop: input and filter gradient; the bias gradient's adds are not
+    counted), ReLU gradient (12 B/elt), SGD step (20 B/elt) and 2x2 pooling gradient (9 B per input elt)."""
+    rng = np.random.default_rng(0x7EA1)
+    rows = []
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        rt.event_record(0)
+        for _ in range(iters):
+            fn()
+        rt.event_record(1)
+        return rt.event_elapsed_ms(0, 1) / iters
+
+    for xs, oc in [((32, 56, 56, 64), 64), ((32, 56, 56, 64), 128), ((32, 28, 28, 128), 128)]:
+        x = rt.upload(rng.standard_normal(xs).astype(np.float32))
+        f = rt.upload((rng.standard_normal((oc, 3, 3, xs[3])) / np.sqrt(9 * xs[3])).astype(np.float32))
+        og = rt.upload(rng.standard_normal(xs[:3] + (oc,)).astype(np.float32))
+        ig, fg, bg = rt.empty(xs), rt.empty(f.shape), rt.empty((oc,))
+        ms = timed(lambda: rt.conv2dGrad(x, f, og, (3, 3), (1, 1), (1, 1, 1, 1), out=(ig, fg, bg)))
+        flop = 2.0 * 2.0 * xs[0] * xs[1] * xs[2] * oc * 9 * xs[3]
+        rows.append(rate(dict(op="conv2dGrad", shape=f"{list(xs)}*{list(f.shape)}", ms=ms, flop=flop)))
+        for t in (x, f, og, ig, fg, bg):
+            t.free()
+    n = 256 * 32 * 32 * 256
+    a, b = rt.upload(rng.standard_normal(n).astype(np.float32)), rt.upload(rng.standard_normal(n).astype(np.float32))
+    c = rt.empty((n,))
+    rows.append(rate(dict(op="reluGrad", shape=f"[{n}]", ms=timed(lambda: rt.reluGrad(a, b, out=c)), bytes=12.0 * n)))
+    mom = rt.upload(np.zeros(n, np.float32))
+    rows.append(rate(dict(op="sgd", shape=f"[{n}]", ms=timed(lambda: rt.sgd(a, b, mom, 0.01, 0.001, 0.9, 32)), bytes=20.0 * n)))
+    x4 = a.reshape(256, 32, 32, 256)
+    og = rt.upload(rng.standard_normal((256, 16, 16, 256)).astype(np.float32))
+    rows.append(rate(dict(op="maxpoolGrad", shape="[256, 32, 32, 256] 2x2/2",
+                          ms=timed(lambda: rt.maxpoolGrad(x4, og, (2, 2), (2, 2), out=c)), bytes=9.0 * n)))
+    return rows
+
+
 def cpu_baseline(graphs, rows=64):
     """The reference's CPU kernels on the first `rows` rows of the headline batch."""
     from oracle import binding
@@ -299,6 +339,7 @@ def main():
             others[f"cfg{cfg}"] = dict(batch=r["batch"], samples_per_s=r["samples_per_s"], ms_per_step=r["ms_per_step"],
                                        gpu_ms_per_step=r["gpu_ms"] / steps, graph_replay=r["graph_replay"],
                                        kernels=r["kernels"])
+        others["training_kernels"] = dict(kernels=run_training(rt))
         out["configs"] = others
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(graphs, args.cpu_rows)

@@ -188,8 +188,8 @@ int swc_hip_matrixTanhGrad_f(int m, int n, float *a, int lda, const float *b, in
                              const float *c, int ldc);
 
 /* kernels.h:105-129; Codegen.cpp:2357-2370.  b = row softmax of a (as
- * matrixSoftmax_f); *loss = mean over rows of logf(sum*expf(max)) - a[row, selected[row]],
- * the rows added in order in fp32.  b may alias a. */
+ * matrixSoftmax_f); *loss = mean over rows of logf(sum*expf(max)) - a[row, selected[row]].
+ * b may alias a. */
 int swc_hip_matrixSoftmaxWithLoss_f(int m, int n, const float *a, int lda, float *b, int ldb,
                                     const int *selected, float *loss);
 

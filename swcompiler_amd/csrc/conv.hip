@@ -688,13 +688,26 @@ int launch_wgrad(const float *ogT, size_t a_bytes, int lda, const Im2colB &bsrc,
     return SWC_HIP_OK;
 }
 
-// out[i] = part[0][i] + part[1][i] + ... in split order
+// out[i] = sum over splits of part[split][i], in a fixed order: eight threads share an element, thread p adds
+// splits p, p+8, p+16, ... (eight independent chains instead of one long one), then the eight are added in order.
 __global__ __launch_bounds__(256) void sum_splits(float *__restrict__ out, const float *__restrict__ part, size_t n,
                                                   int splits) {
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
-        float s = part[i];
-        for (int k = 1; k < splits; ++k) s += part[(size_t)k * n + i];
-        out[i] = s;
+    __shared__ float red[8][33];
+    const int e = threadIdx.x & 31, p = threadIdx.x >> 5;
+    for (size_t base = (size_t)blockIdx.x * 32; base < n; base += (size_t)gridDim.x * 32) {
+        const size_t i = base + e;
+        float s = 0.f;
+        if (i < n)
+            for (int k = p; k < splits; k += 8) s += part[(size_t)k * n + i];
+        red[p][e] = s;
+        __syncthreads();
+        if (p == 0 && i < n) {
+            float t = red[0][e];
+#pragma unroll
+            for (int q = 1; q < 8; ++q) t += red[q][e];
+            out[i] = t;
+        }
+        __syncthreads();
     }
 }
 
@@ -729,24 +742,34 @@ __global__ __launch_bounds__(256) void wgrad_direct(float *__restrict__ fg, cons
 }
 
 // ---- bias gradient: masked column sums of outputG [M, OC]
-constexpr int kBiasRows = 512;   // rows per partial sum
-__global__ __launch_bounds__(256) void bias_partials(float *__restrict__ part, const float *__restrict__ og, ConvGeom g) {
+constexpr int kBiasRows = 128;   // rows per partial sum
+// A workgroup sums kBiasRows rows: thread = (column, row phase); the 256/cols... phases of a column are combined in
+// a fixed order.  cols = min(OC, 256) columns per workgroup in x, row chunks in y.
+__global__ __launch_bounds__(256) void bias_partials(float *__restrict__ part, const float *__restrict__ og, ConvGeom g,
+                                                     int cols, int phases) {
     __shared__ float red[256];
-    const int co = blockIdx.x * 64 + (threadIdx.x & 63);
-    const int sub = threadIdx.x >> 6;   // 4 row phases
+    const int c_local = threadIdx.x % cols, phase = threadIdx.x / cols;
+    const int co = blockIdx.x * cols + c_local;
     const int m0 = blockIdx.y * kBiasRows;
     const int m1 = m0 + kBiasRows < g.M ? m0 + kBiasRows : g.M;
-    float sum = 0.f;
-    if (co < g.OC)
-        for (int m = m0 + sub; m < m1; m += 4) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};   // four independent chains keep four loads in flight
+    if (co < g.OC && phase < phases) {
+        int u = 0;
+        for (int m = m0 + phase; m < m1; m += phases, u = (u + 1) & 3) {
             const int ox = m % g.OW, oy = (m / g.OW) % g.OH;
             const int iy = oy * g.sh - g.pt, ix = ox * g.sw - g.pl;
-            if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W) sum += og[(size_t)m * g.OC + co];
+            const float v = og[(size_t)m * g.OC + co];
+            if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W) acc[u] += v;
         }
+    }
+    const float sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
     red[threadIdx.x] = sum;
     __syncthreads();
-    if (sub == 0 && co < g.OC)
-        part[(size_t)blockIdx.y * g.OC + co] = (red[threadIdx.x] + red[threadIdx.x + 64]) + (red[threadIdx.x + 128] + red[threadIdx.x + 192]);
+    if (phase == 0 && co < g.OC) {
+        float t = red[c_local];
+        for (int q = 1; q < phases; ++q) t += red[q * cols + c_local];
+        part[(size_t)blockIdx.y * g.OC + co] = t;
+    }
 }
 
 size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
@@ -786,16 +809,17 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
     }
 
     // ---- workspace layout
-    const bool dgrad_conv = g.sh == 1 && g.sw == 1 && g.pt <= g.kh - 1 && g.pl <= g.kw - 1;
+    // (an input of very few channels leaves the GEMM form with a handful of columns: the gather is faster there)
+    const bool dgrad_conv = g.sh == 1 && g.sw == 1 && g.pt <= g.kh - 1 && g.pl <= g.kw - 1 && g.C >= 8;
     const bool wgrad_mfma = g.C % 4 == 0 && aligned16(input) && aligned16(outputG) && aligned16(filterG);
     const int lda = (int)((M + 3) & ~(size_t)3);   // row length of the transposed outputG
     const int bias_chunks = (int)((M + kBiasRows - 1) / kBiasRows);
-    // filter-gradient tiles and splits: about three workgroups per CU
+    // filter-gradient tiles and splits: about two workgroups per CU (what fits at once)
     const bool narrow = g.OC <= 64;
     const int bm = narrow ? 64 : 128, bn = narrow ? 256 : 128;
     const int tiles = ((g.OC + bm - 1) / bm) * (int)((Kf + bn - 1) / bn);
     const int nk = (int)((M + BK - 1) / BK);
-    int splits = (3 * num_cus() + tiles - 1) / tiles;
+    int splits = (2 * num_cus() + tiles - 1) / tiles;
     splits = splits < 1 ? 1 : (splits > nk ? nk : splits);
     const int sps = (nk + splits - 1) / splits;
     splits = (nk + sps - 1) / sps;
@@ -811,9 +835,14 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
     float *bias_part = reinterpret_cast<float *>(ws + turned_b + ogt_b + part_b);
 
     // ---- bias gradient
-    bias_partials<<<dim3((g.OC + 63) / 64, bias_chunks), 256, 0, stream()>>>(bias_part, outputG, g);
+    {
+        int cols = 1;
+        while (cols < g.OC && cols < 256) cols <<= 1;   // power of two, so that 256 % cols == 0
+        bias_partials<<<dim3((g.OC + cols - 1) / cols, bias_chunks), 256, 0, stream()>>>(bias_part, outputG, g, cols,
+                                                                                          256 / cols);
+    }
     SWC_LAUNCH_CHECK();
-    sum_splits<<<ceil_div(g.OC, 256), 256, 0, stream()>>>(biasG, bias_part, (size_t)g.OC, bias_chunks);
+    sum_splits<<<ceil_div(g.OC, 32), 256, 0, stream()>>>(biasG, bias_part, (size_t)g.OC, bias_chunks);
     SWC_LAUNCH_CHECK();
 
     // ---- input gradient
@@ -853,8 +882,8 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
                                : launch_wgrad<1, 4, 4, 2, false, 4>(ogT, a_bytes, lda, bsrc, dst, g.OC, (int)Kf, (int)M, splits, sps);
         if (rc2 != SWC_HIP_OK) return rc2;
         if (splits > 1) {
-            unsigned blocks = ceil_div(f_elems, 256);
-            sum_splits<<<blocks > 4096 ? 4096 : blocks, 256, 0, stream()>>>(filterG, part, f_elems, splits);
+            unsigned blocks = ceil_div(f_elems, 32);
+            sum_splits<<<blocks > 16384 ? 16384 : blocks, 256, 0, stream()>>>(filterG, part, f_elems, splits);
             SWC_LAUNCH_CHECK();
         }
     } else {

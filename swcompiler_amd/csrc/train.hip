@@ -1,5 +1,5 @@
 // The kernels a generated TRAINING program calls next to the inference ones,
-// except the convolution gradient (conv_grad.hip): matrixTrans_f,
+// except the convolution gradient (conv.hip): matrixTrans_f,
 // matrixTanhGrad_f, matrixSoftmaxWithLoss_f, matrixSoftmax[WithLoss]Grad_f,
 // maxpoolGrad_f, batchedreduceadd_f, sgd_f, reluGrad_f
 // (src/codegen/utils/kernels.h:68-86, 105-151, 380-442, 554-573, 586-590).
@@ -122,8 +122,16 @@ __global__ __launch_bounds__(kThreads) void row_sums(float *__restrict__ dest, c
         }
         __syncthreads();
         if (threadIdx.x < 64) {
-            const int lim = cols - c0 < 64 ? (int)(cols - c0) : 64;
-            for (int j = 0; j < lim; ++j) sum = sum + tile[threadIdx.x][j];
+            if (cols - c0 >= 64) {
+                float v[64];
+#pragma unroll
+                for (int j = 0; j < 64; ++j) v[j] = tile[threadIdx.x][j];   // independent reads first ...
+#pragma unroll
+                for (int j = 0; j < 64; ++j) sum = sum + v[j];              // ... then the adds, in order
+            } else {
+                const int lim = (int)(cols - c0);
+                for (int j = 0; j < lim; ++j) sum = sum + tile[threadIdx.x][j];
+            }
         }
         __syncthreads();
     }
@@ -149,22 +157,20 @@ __global__ __launch_bounds__(kThreads) void softmax_loss_terms(int m, int n, con
     if (lane == 0) terms[row] = logf(sum * expf(mx)) - ar[selected[row]];
 }
 
-// loss = (sum of the terms, row 0 first, in fp32) / m — one workgroup: chunks of
-// 1024 terms are fetched by all threads, added by thread 0 in order.
-__global__ __launch_bounds__(kThreads) void loss_mean(int m, const float *__restrict__ terms, float *__restrict__ loss) {
-#pragma clang fp contract(off)
-    __shared__ float chunk[1024];
+// loss = (sum of the terms) / m in fp32 — one workgroup, a fixed order: thread t adds terms t, t+1024, ...,
+// then the 1024 partial sums are halved ten times.  (The reference adds row after row; the terms already
+// differ from its in the last bits through expf/logf, so the loss is held to a relative tolerance.)
+__global__ __launch_bounds__(1024) void loss_mean(int m, const float *__restrict__ terms, float *__restrict__ loss) {
+    __shared__ float red[1024];
     float sum = 0.f;
-    for (int c0 = 0; c0 < m; c0 += 1024) {
-        for (int i = threadIdx.x; i < 1024; i += kThreads) chunk[i] = c0 + i < m ? terms[c0 + i] : 0.f;
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            const int lim = m - c0 < 1024 ? m - c0 : 1024;
-            for (int i = 0; i < lim; ++i) sum = sum + chunk[i];
-        }
+    for (int i = threadIdx.x; i < m; i += 1024) sum += terms[i];
+    red[threadIdx.x] = sum;
+    __syncthreads();
+    for (int s = 512; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
         __syncthreads();
     }
-    if (threadIdx.x == 0) *loss = sum / (float)m;
+    if (threadIdx.x == 0) *loss = red[0] / (float)m;
 }
 
 // ------------------------------------------------------ pooling gradient
@@ -172,51 +178,28 @@ struct PoolGeom {
     int N, H, W, C, OH, OW, kh, kw, sh, sw, pt, pl;
 };
 
-// Which input element window (oy, ox) of image n, channel c selects: the first
-// maximum in (ky, kx) scan order among the in-bounds taps; (0, 0) when no tap is
-// in bounds, as the reference's initial max_ix = max_iy = 0 (kernels.h:407-436).
-__device__ __forceinline__ void window_choice(const float *__restrict__ in, const PoolGeom &g, int n, int oy, int ox,
-                                              int c, int &cy, int &cx) {
-    bool uninit = true;
-    float mx = 0.f;
-    cy = 0;
-    cx = 0;
-    for (int ky = 0; ky < g.kh; ++ky) {
-        const int iy = oy * g.sh - g.pt + ky;
-        if ((unsigned)iy >= (unsigned)g.H) continue;
-        for (int kx = 0; kx < g.kw; ++kx) {
-            const int ix = ox * g.sw - g.pl + kx;
-            if ((unsigned)ix >= (unsigned)g.W) continue;
-            const float v = in[(((size_t)n * g.H + iy) * g.W + ix) * g.C + c];
-            if (uninit || v > mx) {
-                mx = v;
-                cy = iy;
-                cx = ix;
-                uninit = false;
-            }
-        }
-    }
-}
-
-// One thread per INPUT element: it visits, in the reference's (oy, ox) order,
-// the windows that can select it and adds their gradients — a gather, so the
-// sum is formed in the same order as the reference's scatter and needs no
-// atomics.  Element (0,0) of every image also collects the windows that have
-// no in-bounds tap when the geometry allows such windows (all_windows).
+// One thread per INPUT element (VEC = 1) or per four consecutive channels of an
+// input pixel (VEC = 4, 128-bit accesses): it visits, in the reference's
+// (oy, ox) order, the windows that can select it and adds their gradients — a
+// gather, so the sum is formed in the same order as the reference's scatter and
+// needs no atomics.  Element (0,0) of every image also collects the windows that
+// have no in-bounds tap when the geometry allows such windows (empty_windows).
+template <int VEC>
 __global__ __launch_bounds__(kThreads) void maxpool_grad(float *__restrict__ ig, const float *__restrict__ og,
-                                                         const float *__restrict__ in, PoolGeom g, int empty_windows) {
+                                                         const float *__restrict__ in, PoolGeom g, int empty_windows,
+                                                         int row_base) {
 #pragma clang fp contract(off)
-    const size_t total = (size_t)g.N * g.H * g.W * g.C;
-    size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
-    const size_t step = (size_t)gridDim.x * kThreads;
-    for (; i < total; i += step) {
-        const int c = (int)(i % g.C);
-        size_t t = i / g.C;
-        const int ix = (int)(t % g.W);
-        t /= g.W;
-        const int iy = (int)(t % g.H);
-        const int n = (int)(t / g.H);
-        float sum = 0.f;
+    // row_base + blockIdx.y = image row (n*H + iy); blockIdx.x, threadIdx.x walk the row's W * C/VEC items: 32-bit index arithmetic
+    const int cq = g.C / VEC;
+    const int row_items = g.W * cq;
+    const int image_row = row_base + blockIdx.y;
+    const int iy = image_row % g.H, n = image_row / g.H;
+    for (int item = blockIdx.x * kThreads + threadIdx.x; item < row_items; item += gridDim.x * kThreads) {
+        const int ix = item / cq;
+        const int c = (item - ix * cq) * VEC;
+        float sum[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) sum[v] = 0.f;
         int oy_lo, oy_hi, ox_lo, ox_hi;
         if (empty_windows && iy == 0 && ix == 0) {
             oy_lo = 0, oy_hi = g.OH - 1, ox_lo = 0, ox_hi = g.OW - 1;
@@ -230,11 +213,48 @@ __global__ __launch_bounds__(kThreads) void maxpool_grad(float *__restrict__ ig,
         }
         for (int oy = oy_lo; oy <= oy_hi; ++oy)
             for (int ox = ox_lo; ox <= ox_hi; ++ox) {
-                int cy, cx;
-                window_choice(in, g, n, oy, ox, c, cy, cx);
-                if (cy == iy && cx == ix) sum = sum + og[(((size_t)n * g.OH + oy) * g.OW + ox) * g.C + c];
+                // the window's choice per channel: first maximum in (ky, kx) scan order among the in-bounds
+                // taps; (0, 0) when no tap is in bounds, as the reference's initial max_ix = max_iy = 0
+                bool uninit = true;
+                float mx[VEC];
+                int cy[VEC], cx[VEC];
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) mx[v] = 0.f, cy[v] = 0, cx[v] = 0;
+                for (int ky = 0; ky < g.kh; ++ky) {
+                    const int wy = oy * g.sh - g.pt + ky;
+                    if ((unsigned)wy >= (unsigned)g.H) continue;
+                    for (int kx = 0; kx < g.kw; ++kx) {
+                        const int wx = ox * g.sw - g.pl + kx;
+                        if ((unsigned)wx >= (unsigned)g.W) continue;
+                        const float *p = in + (((size_t)n * g.H + wy) * g.W + wx) * g.C + c;
+                        float val[VEC];
+                        if (VEC == 4) {
+                            const float4 q = *reinterpret_cast<const float4 *>(p);
+                            val[0] = q.x, val[VEC > 1 ? 1 : 0] = q.y, val[VEC > 2 ? 2 : 0] = q.z, val[VEC > 3 ? 3 : 0] = q.w;
+                        } else {
+                            val[0] = *p;
+                        }
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v)
+                            if (uninit || val[v] > mx[v]) mx[v] = val[v], cy[v] = wy, cx[v] = wx;
+                        uninit = false;
+                    }
+                }
+                const float *gp = og + (((size_t)n * g.OH + oy) * g.OW + ox) * g.C + c;
+                float gv[VEC];
+                if (VEC == 4) {
+                    const float4 q = *reinterpret_cast<const float4 *>(gp);
+                    gv[0] = q.x, gv[VEC > 1 ? 1 : 0] = q.y, gv[VEC > 2 ? 2 : 0] = q.z, gv[VEC > 3 ? 3 : 0] = q.w;
+                } else {
+                    gv[0] = *gp;
+                }
+#pragma unroll
+                for (int v = 0; v < VEC; ++v)
+                    if (cy[v] == iy && cx[v] == ix) sum[v] = sum[v] + gv[v];
             }
-        ig[i] = sum;
+        float *op = ig + (((size_t)n * g.H + iy) * g.W + ix) * g.C + c;
+        if (VEC == 4) *reinterpret_cast<float4 *>(op) = make_float4(sum[0], sum[VEC > 1 ? 1 : 0], sum[VEC > 2 ? 2 : 0], sum[VEC > 3 ? 3 : 0]);
+        else *op = sum[0];
     }
 }
 
@@ -299,7 +319,7 @@ int swc_hip_matrixSoftmaxWithLoss_f(int m, int n, const float *a, int lda, float
     // the loss terms read a before the softmax may overwrite it (b may alias a)
     softmax_loss_terms<<<ceil_div(m, kThreads / 64), kThreads, 0, stream()>>>(m, n, a, lda, selected, terms);
     SWC_LAUNCH_CHECK();
-    loss_mean<<<1, kThreads, 0, stream()>>>(m, terms, loss);
+    loss_mean<<<1, 1024, 0, stream()>>>(m, terms, loss);
     SWC_LAUNCH_CHECK();
     return swc_hip_matrixSoftmax_f(m, n, a, lda, b, ldb);
 }
@@ -357,7 +377,18 @@ int swc_hip_maxpoolGrad_f(float *inputG, const float *outputG, const float *inpu
         const long last_y = (long)(g.OH - 1) * g.sh - g.pt, last_x = (long)(g.OW - 1) * g.sw - g.pl;
         empty = (g.kh - 1 - g.pt < 0) || (g.kw - 1 - g.pl < 0) || last_y >= g.H || last_x >= g.W;
     }
-    maxpool_grad<<<grid_for(total, kThreads), kThreads, 0, stream()>>>(inputG, outputG, input, g, empty);
+    const size_t image_rows = idims[0] * idims[1];
+    SWC_ARG(image_rows <= 0x7fffffffu);
+    const bool vec = g.C % 4 == 0 && aligned16(inputG) && aligned16(outputG) && aligned16(input);
+    const size_t row_items = (size_t)g.W * (vec ? g.C / 4 : g.C);
+    // grid.y is limited to 65535: rows beyond that are covered by launching in slabs of rows
+    for (size_t r0 = 0; r0 < image_rows; r0 += 65535) {
+        const unsigned rows = (unsigned)(image_rows - r0 < 65535 ? image_rows - r0 : 65535);
+        const dim3 grid(grid_for(row_items, kThreads, 1024), rows);
+        if (vec) maxpool_grad<4><<<grid, kThreads, 0, stream()>>>(inputG, outputG, input, g, empty, (int)r0);
+        else maxpool_grad<1><<<grid, kThreads, 0, stream()>>>(inputG, outputG, input, g, empty, (int)r0);
+        SWC_LAUNCH_CHECK();
+    }
     SWC_LAUNCH_CHECK();
     return SWC_HIP_OK;
 }

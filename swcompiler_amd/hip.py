@@ -413,18 +413,18 @@ class SwcHip:
         self._check(fn(m, n, ig.ptr, n, prob.ptr, n, selected.ptr), "matrixSoftmaxGrad_f")
         return ig
 
-    def conv2dGrad(self, x, filt, out_grad, kernels=None, strides=(1, 1), pads=(0, 0, 0, 0), group=1):
+    def conv2dGrad(self, x, filt, out_grad, kernels=None, strides=(1, 1), pads=(0, 0, 0, 0), group=1, out=None):
         if kernels is None:
             kernels = filt.shape[1:3]
-        ig, fg, bg = self.empty(x.shape), self.empty(filt.shape), self.empty((filt.shape[0],))
+        ig, fg, bg = out if out is not None else (self.empty(x.shape), self.empty(filt.shape), self.empty((filt.shape[0],)))
         self._check(self.lib.swc_hip_conv2dGrad_f(ig.ptr, fg.ptr, bg.ptr, out_grad.ptr, x.ptr, filt.ptr,
                                                   _dims(out_grad.shape), _dims(x.shape), _dims(filt.shape),
                                                   _dims(bg.shape), _dims(kernels), _dims(strides), _dims(pads), group),
                     "conv2dGrad_f")
         return ig, fg, bg
 
-    def maxpoolGrad(self, x, out_grad, kernels, strides, pads=(0, 0, 0, 0)):
-        ig = self.empty(x.shape)
+    def maxpoolGrad(self, x, out_grad, kernels, strides, pads=(0, 0, 0, 0), out=None):
+        ig = out.reshape(x.shape) if out is not None else self.empty(x.shape)
         self._check(self.lib.swc_hip_maxpoolGrad_f(ig.ptr, out_grad.ptr, x.ptr, _dims(x.shape), _dims(out_grad.shape),
                                                    _dims(kernels), _dims(strides), _dims(pads)), "maxpoolGrad_f")
         return ig
@@ -440,8 +440,8 @@ class SwcHip:
         self._check(self.lib.swc_hip_sgd_f(w.size, w.ptr, w.ptr, dw.ptr, mom.ptr, lr, decay, momentum, batch), "sgd_f")
         return w, mom
 
-    def reluGrad(self, src, dest_grad):
-        out = self.empty(src.shape)
+    def reluGrad(self, src, dest_grad, out=None):
+        out = out if out is not None else self.empty(src.shape)
         self._check(self.lib.swc_hip_reluGrad_f(out.ptr, src.ptr, dest_grad.ptr, src.size), "reluGrad_f")
         return out
 

@@ -238,3 +238,37 @@ def test_training_error_paths(rt):
         rt.conv2dGrad(x, rt.empty((4, 3, 3, 8)), og, (3, 3), (1, 1), (1, 1, 1, 1))
     assert rt.lib.swc_hip_reluGrad_f(None, None, None, 4) != 0
     assert rt.lib.swc_hip_matrixTanhGrad_f(2, 4, x.ptr, 2, x.ptr, 4, x.ptr, 4) != 0     # lda < n
+
+
+def test_conv2dGrad_full_size_properties(rt, oracle):
+    """cfg4's first convolution at full size (32x56x56x64 -> 64): linearity in outputG (the gradients of
+    g1 + g2 are the sums of the gradients, to rounding), a gradient that is zero except at one pixel checked
+    against the oracle on that neighbourhood, and integer-valued operands against float64 einsum on a slab."""
+    rng = np.random.default_rng(99)
+    xs, fs = (32, 56, 56, 64), (64, 3, 3, 64)
+    x = rng.integers(-2, 3, xs).astype(np.float32)
+    f = rng.integers(-2, 3, fs).astype(np.float32)
+    og = np.zeros(xs[:3] + (64,), np.float32)
+    og[5, 10:13, 20:23, :] = rng.integers(-2, 3, (3, 3, 64))
+    dx, df, dog = up(rt, x, f, og)
+    ig, fg, bg = (t.numpy() for t in rt.conv2dGrad(dx, df, dog, (3, 3), (1, 1), (1, 1, 1, 1)))
+    # only image 5, rows 9..13, columns 19..23 of the input can receive gradient; compare that crop with the oracle
+    crop_x = x[5:6, 8:15, 18:25, :]
+    crop_og = og[5:6, 9:14, 19:24, :]                     # valid convolution of the crop: 5x5 outputs
+    want_ig, want_fg, want_bg = oracle.conv2dGrad(crop_x, f, crop_og, (3, 3), (1, 1), (0, 0, 0, 0))
+    assert_bit_exact(ig[5:6, 8:15, 18:25, :], want_ig, "inputG crop")
+    assert np.count_nonzero(ig) == np.count_nonzero(want_ig)
+    assert_bit_exact(fg, want_fg, "filterG")
+    assert_bit_exact(bg, want_bg, "biasG")
+    # dense integer gradient: filterG against einsum in float64 for one tap, biasG exactly
+    og2 = rng.integers(-1, 2, og.shape).astype(np.float32)
+    ig2, fg2, bg2 = (t.numpy() for t in rt.conv2dGrad(dx, df, rt.upload(og2), (3, 3), (1, 1), (1, 1, 1, 1)))
+    tap = np.einsum("nhwc,nhwo->oc", x.astype(np.float64), og2.astype(np.float64))     # centre tap (1,1)
+    assert_bit_exact(fg2[:, 1, 1, :], tap.astype(np.float32), "filterG centre tap")
+    keep = np.zeros((56, 56), bool)
+    keep[1:, 1:] = True          # first tap (0,0) inside the image: oy >= 1 and ox >= 1 with pad 1
+    assert_bit_exact(bg2, (og2 * keep[None, :, :, None]).sum(axis=(0, 1, 2), dtype=np.float64).astype(np.float32), "biasG")
+    # linearity
+    ig3, fg3, bg3 = (t.numpy() for t in rt.conv2dGrad(dx, df, rt.upload(og + og2), (3, 3), (1, 1), (1, 1, 1, 1)))
+    assert_bit_exact(ig3, ig + ig2, "inputG linear")
+    assert_bit_exact(fg3, fg + fg2, "filterG linear")
