@@ -811,7 +811,9 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
     // ---- workspace layout
     // (an input of very few channels leaves the GEMM form with a handful of columns: the gather is faster there)
     const bool dgrad_conv = g.sh == 1 && g.sw == 1 && g.pt <= g.kh - 1 && g.pl <= g.kw - 1 && g.C >= 8;
-    const bool wgrad_mfma = g.C % 4 == 0 && aligned16(input) && aligned16(outputG) && aligned16(filterG);
+    // (the column-interleaved kernel body starts its descriptors 4 KiB early: operands stay below 2 GiB - 64 KiB)
+    const bool wgrad_mfma = g.C % 4 == 0 && aligned16(input) && aligned16(outputG) && aligned16(filterG) &&
+                            in_elems * 4 < 0x7fff0000u && (M + 4) * odims[3] * 4 < 0x7fff0000u;
     const int lda = (int)((M + 3) & ~(size_t)3);   // row length of the transposed outputG
     const int bias_chunks = (int)((M + kBiasRows - 1) / kBiasRows);
     // filter-gradient tiles and splits: about two workgroups per CU (what fits at once)
