@@ -245,6 +245,48 @@ __global__ __launch_bounds__(64 * NW) void gemm_dma2(const float *__restrict__ A
 #endif
 }
 
+// Split-K form for shapes with few output tiles (batch-8 MLP, LeNet's FC layers: a handful of tiles,
+// K of hundreds): blockIdx.y takes a range of K slices and writes its partial tile to the workspace;
+// splitk_finish adds the partial results in split order and applies bias and ReLU.
+template <int TM, int TN, int WM, int STAGES, bool MID, int NW>
+__global__ __launch_bounds__(64 * NW) void gemm_dma2_splitk(const float *__restrict__ A, const float *__restrict__ B,
+                                                             float *__restrict__ part, int M, int N, int K, int lda,
+                                                             int ldb, unsigned a_bytes, unsigned b_bytes,
+                                                             int slices_per_split) {
+#if __HIP_DEVICE_COMPILE__
+    const int k_begin = blockIdx.y * slices_per_split * BK;
+    const int k_stop = k_begin + slices_per_split * BK;
+    const Epilogue ep{nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
+    dma2_tile_body<TM, TN, WM, STAGES, MID, NW>(A, a_bytes, lda, DenseB{B, b_bytes, ldb},
+                                                part + (size_t)blockIdx.y * M * N, (size_t)N, M, N, k_begin,
+                                                k_stop < K ? k_stop : K, ep);
+#endif
+}
+
+// c[r][j] = f(sum over splits of part[split][r][j] + bias[j]); four threads share an element (four chains)
+__global__ __launch_bounds__(256) void splitk_finish(float *__restrict__ c, size_t ldc, const float *__restrict__ part,
+                                                     int M, int N, int splits, Epilogue ep) {
+    __shared__ float red[4][65];
+    const int e = threadIdx.x & 63, p = threadIdx.x >> 6;
+    const size_t n = (size_t)M * N;
+    for (size_t base = (size_t)blockIdx.x * 64; base < n; base += (size_t)gridDim.x * 64) {
+        const size_t i = base + e;
+        float s = 0.f;
+        if (i < n)
+            for (int k = p; k < splits; k += 4) s += part[(size_t)k * n + i];
+        red[p][e] = s;
+        __syncthreads();
+        if (p == 0 && i < n) {
+            const size_t r = i / N, j = i - r * N;
+            float x = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
+            if (ep.bias) x += ep.bias[j];
+            if (ep.relu) x = (x > 0.f) ? x : 0.f;
+            c[r * ldc + j] = x;
+        }
+        __syncthreads();
+    }
+}
+
 // --------------------------------------------------------------- skinny GEMM
 typedef float v4f __attribute__((ext_vector_type(4)));
 constexpr int kSkinnyMaxWaves = 16;
@@ -370,6 +412,30 @@ int launch_dma2(const float *a, const float *b, float *c, int m, int n, int k, i
     return SWC_HIP_OK;
 }
 
+int launch_splitk(const float *a, const float *b, float *c, int m, int n, int k, int lda, int ldb, int ldc,
+                  const Epilogue &ep, int splits, int sps) {
+    using T = Dma2Tile<1, 4, 4, 2, 4>;
+    float *part = static_cast<float *>(workspace((size_t)splits * m * n * sizeof(float), "gemm (split-K)"));
+    if (!part) return SWC_HIP_ERUNTIME;
+    auto kern = gemm_dma2_splitk<1, 4, 4, 2, false, 4>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        SWC_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)T::kLdsBytes));
+        attr_set = true;
+    }
+    const unsigned tiles = (unsigned)(((m + T::BM - 1) / T::BM) * ((n + T::BN - 1) / T::BN));
+    const unsigned a_bytes = (unsigned)(((size_t)(m - 1) * lda + k) * 4);
+    const unsigned b_bytes = (unsigned)(((size_t)(k - 1) * ldb + n) * 4);
+    kern<<<dim3(tiles, splits), T::kThreadsWg, T::kLdsBytes, stream()>>>(a, b, part, m, n, k, lda, ldb, a_bytes, b_bytes,
+                                                                         sps);
+    SWC_LAUNCH_CHECK();
+    unsigned blocks = ceil_div((size_t)m * n, 64);
+    splitk_finish<<<blocks > 8192 ? 8192 : blocks, 256, 0, stream()>>>(c, (size_t)ldc, part, m, n, splits, ep);
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
+}
+
 int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda, const float *b, int ldb,
                   const float *bias, float *c, int ldc, int relu) {
     if (m < 0 || n < 0 || k < 0) return fail(SWC_HIP_EINVAL, "%s: negative dimension", who);
@@ -397,8 +463,10 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
                          ((size_t)(k - 1) * ldb + n) * 4 < 0x7fff0000u;
     const long huge_tiles = (long)((m + 255) / 256) * ((n + 255) / 256);
     // Forces a kernel variant (tests, tuning).  reg: register-staged.  <TM><TN>_<STAGES>[m]: gemm_dma, m = ring
-    // hand-over in mid-slice.  <TM><TN>w<WM>_<STAGES>[m][x8]: gemm_dma2, x8 = eight wavefronts per workgroup.
+    // hand-over in mid-slice.  <TM><TN>w<WM>_<STAGES>[m][x8]: gemm_dma2, x8 = eight wavefronts per workgroup.  splitk: K split
+    // over blockIdx.y with partial tiles in the workspace.
     const char *force = getenv("SWC_HIP_GEMM");
+    const int nk = (k + BK - 1) / BK;
     if (dma_ok && !(force && !strcmp(force, "reg"))) {
         if (force) {
             if (!strcmp(force, "22_2")) return launch_dma<2, 2, 2>(a, b, c, m, n, k, lda, ldb, ldc, ep);
@@ -420,6 +488,17 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
         // 256x256 tiles with eight wavefronts once they fill the chip (least operand traffic per flop: 146
         // TFLOP/s at 4096^3 against 134 for 128x128 tiles of four wavefronts), 128x128 tiles next, and 64x64
         // tiles for everything smaller, where the number of workgroups matters more than their efficiency
+        // few tiles and a K of hundreds: split K over the chip (needs the workspace; not while recording a graph
+        // unless it is already large enough — an eager warm-up run sees to that)
+        const bool want_split = force ? !strcmp(force, "splitk") : (big_tiles * 4 <= num_cus() && nk >= 8);
+        if (dma2_ok && want_split && nk >= 2) {
+            int splits = (int)((2L * num_cus() + big_tiles - 1) / big_tiles);
+            splits = splits > nk ? nk : splits;
+            const int sps = (nk + splits - 1) / splits;
+            splits = (nk + sps - 1) / sps;
+            if (splits > 1 && (size_t)splits * m * n * 4 <= ((size_t)64 << 20))
+                return launch_splitk(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps);
+        }
         if (dma2_ok && huge_tiles >= num_cus()) return launch_dma2<2, 4, 4, 2, false, 8>(a, b, c, m, n, k, lda, ldb, ldc, ep);
         if (dma2_ok && big_tiles >= num_cus()) return launch_dma2<1, 4, 4, 2, false>(a, b, c, m, n, k, lda, ldb, ldc, ep);
         if (big_tiles >= num_cus()) return launch_dma<2, 2, 2>(a, b, c, m, n, k, lda, ldb, ldc, ep);

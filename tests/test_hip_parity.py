@@ -377,7 +377,7 @@ def test_error_paths(rt):
 # offsets), "TMTN_S[m]" = direct-to-LDS kernels with an S-stage ring (m: ring hand-over in
 # mid-slice), "TMTNwWM_S[m][x8]" = the column-interleaved kernels (x8: eight wavefronts).
 GEMM_VARIANTS = ["reg", "22_2", "22_3", "21_3", "12_3", "11_3", "11_4", "11_3m", "21_3m",
-                 "24w4_2x8", "14w4_2", "14w4_3m", "24w2_3m", "22w2_2"]
+                 "24w4_2x8", "14w4_2", "14w4_3m", "24w2_3m", "22w2_2", "splitk"]
 
 
 @pytest.mark.parametrize("variant", GEMM_VARIANTS)
