@@ -20,9 +20,9 @@
  *     src/codegen/Codegen.cpp:166-172); call swc_hip_sync() before reading
  *     results on the host.  swc_hip_d2h synchronises by itself.
  * Nothing here allocates device memory except swc_hip_malloc and, when no
- * workspace has been provided, the two ops that need scratch memory
- * (swc_hip_conv2dGrad_f, swc_hip_matrixSoftmaxWithLoss_f; see
- * swc_hip_set_workspace).
+ * workspace has been provided, the ops that need scratch memory
+ * (swc_hip_conv2dGrad_f, swc_hip_matrixSoftmaxWithLoss_f, and the FC/GEMM entry
+ * points for shapes they split over K; see swc_hip_set_workspace).
  * Layouts are the reference's: 4-D activations NHWC, conv filters
  * [oC, kH, kW, iC], matrices row-major.  All data is fp32.
  */
@@ -56,7 +56,8 @@ int swc_hip_d2h(void *dst_host, const void *src_dev, size_t bytes); /* ordered a
 int swc_hip_d2d(void *dst_dev, const void *src_dev, size_t bytes);  /* async on the stream */
 int swc_hip_fill_f(float *dst_dev, float value, size_t count);      /* initTensorConstant/Zero, kernels.h:23-29 */
 int swc_hip_sync(void);
-/* Scratch device memory for the ops that need some (conv2dGrad_f: the
+/* Scratch device memory for the ops that need some (FC/GEMM calls that are split
+ * over K: swc_hip_gemm_workspace_bytes; conv2dGrad_f: the
  * transposed gradient and operand copies, up to about twice the size of its
  * largest argument; matrixSoftmaxWithLoss_f: 4*m bytes).  A generated program
  * reserves a slot of its arena and passes it here once; without this call the
@@ -64,6 +65,11 @@ int swc_hip_sync(void);
  * (not possible while a graph is being recorded).  dptr NULL, bytes 0: back to
  * the library's own buffer.  The buffer is shared by all ops on the stream. */
 int swc_hip_set_workspace(void *dptr, size_t bytes);
+/* Workspace a matrixMatrixMul_f / matrixMatrixFCBias_f call of this shape uses on the
+ * initialised device (0 for most shapes: only products with few output tiles and a K
+ * of hundreds are split over K).  A generated program takes the maximum over its
+ * calls and provides that much with swc_hip_set_workspace. */
+size_t swc_hip_gemm_workspace_bytes(int m, int n, int k);
 const char *swc_hip_last_error(void);         /* message of the last failure on this thread ("" if none) */
 void *swc_hip_stream(void);                   /* the hipStream_t ops are launched on */
 int swc_hip_set_stream(void *hip_stream);     /* launch on a caller-owned stream (NULL: back to the library's own) */

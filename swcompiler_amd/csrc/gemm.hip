@@ -436,6 +436,19 @@ int launch_splitk(const float *a, const float *b, float *c, int m, int n, int k,
     return SWC_HIP_OK;
 }
 
+// Split-K plan of an m x n x k product on this device: true with the number of splits and the K slices per
+// split when the shape has too few output tiles to fill the chip.
+bool splitk_plan(int m, int n, int k, int &splits, int &sps, bool forced = false) {
+    const long big_tiles = (long)((m + 127) / 128) * ((n + 127) / 128);
+    const int nk = (k + BK - 1) / BK;
+    if (n <= 16 || nk < 2 || (!forced && (big_tiles * 4 > num_cus() || nk < 8))) return false;
+    splits = (int)((2L * num_cus() + big_tiles - 1) / big_tiles);
+    splits = splits > nk ? nk : splits;
+    sps = (nk + splits - 1) / splits;
+    splits = (nk + sps - 1) / sps;
+    return splits > 1 && (size_t)splits * m * n * 4 <= ((size_t)64 << 20);
+}
+
 int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda, const float *b, int ldb,
                   const float *bias, float *c, int ldc, int relu) {
     if (m < 0 || n < 0 || k < 0) return fail(SWC_HIP_EINVAL, "%s: negative dimension", who);
@@ -490,15 +503,9 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
         // tiles for everything smaller, where the number of workgroups matters more than their efficiency
         // few tiles and a K of hundreds: split K over the chip (needs the workspace; not while recording a graph
         // unless it is already large enough — an eager warm-up run sees to that)
-        const bool want_split = force ? !strcmp(force, "splitk") : (big_tiles * 4 <= num_cus() && nk >= 8);
-        if (dma2_ok && want_split && nk >= 2) {
-            int splits = (int)((2L * num_cus() + big_tiles - 1) / big_tiles);
-            splits = splits > nk ? nk : splits;
-            const int sps = (nk + splits - 1) / splits;
-            splits = (nk + sps - 1) / sps;
-            if (splits > 1 && (size_t)splits * m * n * 4 <= ((size_t)64 << 20))
-                return launch_splitk(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps);
-        }
+        int splits = 0, sps = 0;
+        if (dma2_ok && (!force || !strcmp(force, "splitk")) && splitk_plan(m, n, k, splits, sps, force != nullptr))
+            return launch_splitk(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps);
         if (dma2_ok && huge_tiles >= num_cus()) return launch_dma2<2, 4, 4, 2, false, 8>(a, b, c, m, n, k, lda, ldb, ldc, ep);
         if (dma2_ok && big_tiles >= num_cus()) return launch_dma2<1, 4, 4, 2, false>(a, b, c, m, n, k, lda, ldb, ldc, ep);
         if (big_tiles >= num_cus()) return launch_dma<2, 2, 2>(a, b, c, m, n, k, lda, ldb, ldc, ep);
@@ -516,6 +523,12 @@ int swc_hip_matrixMatrixMul_f(int m, int n, int k, const float *a, int lda, cons
                               int ldc) {
     SWC_REQUIRE_INIT();
     return gemm_dispatch("swc_hip_matrixMatrixMul_f", m, n, k, a, lda, b, ldb, nullptr, c, ldc, 0);
+}
+
+size_t swc_hip_gemm_workspace_bytes(int m, int n, int k) {
+    if (!ready() || m <= 0 || n <= 0 || k <= 0) return 0;
+    int splits = 0, sps = 0;
+    return splitk_plan(m, n, k, splits, sps) ? (size_t)splits * m * n * sizeof(float) : 0;
 }
 
 int swc_hip_matrixMatrixFCBias_f(int m, int n, int k, const float *a, int lda, const float *b, int ldb,

@@ -155,6 +155,7 @@ class Codegen {
 
 class HipCodegen : public Codegen {
     devices::HipDevice device_;
+    bool has_workspace_ = false;   // the program holds a workspace for its FC calls
 
   public:
     HipCodegen(IRGraph *graph, Config &config) : Codegen(graph, config) {}
@@ -164,6 +165,7 @@ class HipCodegen : public Codegen {
     void emitEnvFinalize() override;
     void allocateMemAddr() override;
     void emitMemAllocations() override;
+    void emitWorkspace();
     void emitTensorInitializations() override;
     void emitExecute() override;
     void emitMemFree() override;

@@ -6,6 +6,7 @@
 // tensor on a 256-byte boundary) — uploads parameters once, then per iteration
 // issues one asynchronous swc_hip_* call per op node on the library's single
 // stream and synchronises only where a Gather brings a result back.
+#include <array>
 #include <cassert>
 #include <cstdlib>
 #include <iomanip>
@@ -38,7 +39,7 @@ void HipCodegen::initMakefileBuilder() {
 void HipCodegen::emitHeader() {
     headerWriter_ << "// Graph.cpp -- generated from an IRGraph with " << graph_->tensorNodeNum() << " tensor nodes and "
                   << graph_->opNodeNum() << " op nodes (HIP target, " << device_.arch << ")\n";
-    headerWriter_ << "#include <iostream>\n#include <random>\n#include <cstdlib>\n#include <cstdio>\n#include <cmath>\n"
+    headerWriter_ << "#include <algorithm>\n#include <iostream>\n#include <random>\n#include <cstdlib>\n#include <cstdio>\n#include <cmath>\n"
                   << "#include <sys/time.h>\n"
                   << "#include \"swc_host_utils.h\"\n#include \"swc_hip.h\"\n";
     headerWriter_ << "#define SWC_HIP_CHECK(call) do { if ((call) != 0) { std::fprintf(stderr, \"%s:%d: %s\\n  %s\\n\", "
@@ -63,7 +64,32 @@ void HipCodegen::allocateMemAddr() {
     }
 }
 
+// The FC entry points split small-output products over K and keep the partial results in a workspace:
+// the program asks the library how much its calls need and provides it, so that no op allocates.
+void HipCodegen::emitWorkspace() {
+    std::vector<std::array<size_t, 3>> shapes;
+    for (int i = 0; i < graph_->opNodeNum(); ++i) {
+        OpNode *op = graph_->getOpNode(i);
+        if (op->getLabel()->getDeviceLabel().type != DeviceType::GPU) continue;   // (runable() counts its calls: not asked here)
+        const std::string type = op->getOp()->getOpName();
+        if (type != "MatrixMatrixMul" && type != "MatrixMatrixFCBias" && type != "MatrixMatrixFCBiasRelu") continue;
+        Tensor *x = static_cast<TensorNode *>(op->getParentNode(0))->getTensor();
+        Tensor *w = static_cast<TensorNode *>(op->getParentNode(1))->getTensor();
+        shapes.push_back({x->size() / w->getDim(0), w->getDim(1), w->getDim(0)});
+    }
+    has_workspace_ = !shapes.empty();
+    if (shapes.empty()) return;
+    writer_ << "size_t gpu0_ws_bytes = 0;\n";
+    for (auto &s : shapes)
+        writer_ << "gpu0_ws_bytes = std::max(gpu0_ws_bytes, swc_hip_gemm_workspace_bytes(" << s[0] << ", " << s[1] << ", "
+                << s[2] << "));\n";
+    writer_ << "void *gpu0_ws = gpu0_ws_bytes ? swc_hip_malloc(gpu0_ws_bytes) : nullptr;\n"
+            << "if (gpu0_ws_bytes && !gpu0_ws) { std::fprintf(stderr, \"%s\\n\", swc_hip_last_error()); return 1; }\n"
+            << "if (gpu0_ws) SWC_HIP_CHECK(swc_hip_set_workspace(gpu0_ws, gpu0_ws_bytes));\n";
+}
+
 void HipCodegen::emitMemAllocations() {
+    emitWorkspace();
     for (auto &a : mem_allocators_) {
         if (!a->getMemAllocated()) continue;
         if (a->getDevice().type == DeviceType::CPU) {
@@ -192,6 +218,9 @@ void HipCodegen::emitDeviceOpsOnly() {
 }
 
 void HipCodegen::emitMemFree() {
+    if (has_workspace_)
+        writer_ << "SWC_HIP_CHECK(swc_hip_set_workspace(nullptr, 0));\n"
+                << "if (gpu0_ws) SWC_HIP_CHECK(swc_hip_free(gpu0_ws));\n";
     for (auto &a : mem_allocators_) {
         if (!a->getMemAllocated()) continue;
         if (a->getDevice().type == DeviceType::CPU) writer_ << "free(" << a->getBasePtrName() << ");\n";

@@ -146,6 +146,12 @@ def test_hip_program_structure_and_build(gen, tmp_path):
     mlp = generate(gen, "cfg2", "hip", tmp_path, 64)
     assert mlp.count("swc_hip_matrixMatrixFCBias_f(") == 3 and "swc_hip_batchedadd_f" not in mlp
     assert re.search(r"swc_hip_matrixMatrixFCBias_f\(64, 4096, 784, .*, 1\)\);", mlp)
+    # the program sizes and owns the scratch memory of its FC calls: one query per call, one buffer, given
+    # to the library before the first op and taken back before it is freed
+    assert mlp.count("swc_hip_gemm_workspace_bytes(") == 3 and "swc_hip_gemm_workspace_bytes(64, 4096, 784)" in mlp
+    assert mlp.index("swc_hip_set_workspace(gpu0_ws, gpu0_ws_bytes)") < mlp.index("// call op routine functions")
+    assert mlp.index("swc_hip_set_workspace(nullptr, 0)") < mlp.index("swc_hip_free(gpu0_ws)")
+    assert "workspace" not in code   # no FC in the conv block: no workspace code
     lenet = generate(gen, "cfg3", "hip", tmp_path, 4)
     assert lenet.count("swc_hip_conv2dFused_f(") == 2 and "swc_hip_matrixMatrixFCBias_f(4, 500, 800" in lenet
     timed = generate(gen, "cfg5b", "hip", tmp_path, 1, iters=10)

@@ -404,6 +404,29 @@ def test_gemm_every_variant(rt, oracle, variant, monkeypatch):
     assert_bit_exact(rt.fcbias(*up(rt, a, b, bias), relu=False).numpy(), want, f"integer gemm {m}x{k}x{n} variant {variant}")
 
 
+def test_gemm_split_over_k_uses_exactly_the_size_it_reports(rt, oracle):
+    from swcompiler_amd.hip import SwcHipError
+    assert rt.gemm_workspace_bytes(4096, 4096, 784) == 0 and rt.gemm_workspace_bytes(8, 10, 512) == 0
+    m, n, k = 8, 512, 784
+    need = rt.gemm_workspace_bytes(m, n, k)
+    assert need > 0 and need % (m * n * 4) == 0
+    rng = np.random.default_rng(21)
+    a = rng.integers(-8, 9, (m, k)).astype(np.float32)
+    b = rng.integers(-8, 9, (k, n)).astype(np.float32)
+    bias = rng.integers(-8, 9, n).astype(np.float32)
+    want = np.maximum(a.astype(np.int64) @ b.astype(np.int64) + bias.astype(np.int64), 0).astype(np.float32)
+    exact, short = rt.empty((need // 4,)), rt.empty((need // 4 - 4,))
+    try:
+        rt.set_workspace(exact)
+        assert_bit_exact(rt.fcbias(*up(rt, a, b, bias), relu=True).numpy(), want, "split-K in a caller workspace")
+        rt.set_workspace(short)
+        with pytest.raises(SwcHipError, match="workspace"):
+            rt.fcbias(*up(rt, a, b, bias), relu=True)
+    finally:
+        rt.sync()
+        rt.set_workspace(None)
+
+
 @pytest.mark.parametrize("variant", ["reg22", "reg21", "reg12", "reg11", "22_2", "21_3", "12_3", "11_3", "11_4", "11_3m", "21_3m", "12_3m", "22_3m"])
 def test_conv_every_variant(rt, oracle, variant, monkeypatch):
     print("case conv variant", variant, flush=True)
