@@ -21,8 +21,8 @@
  *     results on the host.  swc_hip_d2h synchronises by itself.
  * Nothing here allocates device memory except swc_hip_malloc and, when no
  * workspace has been provided, the ops that need scratch memory
- * (swc_hip_conv2dGrad_f, swc_hip_matrixSoftmaxWithLoss_f, and the FC/GEMM entry
- * points for shapes they split over K; see swc_hip_set_workspace).
+ * (swc_hip_conv2dGrad_f, swc_hip_matrixSoftmaxWithLoss_f, and the FC/GEMM and
+ * convolution entry points for shapes they cut along K; see swc_hip_set_workspace).
  * Layouts are the reference's: 4-D activations NHWC, conv filters
  * [oC, kH, kW, iC], matrices row-major.  All data is fp32.
  */
@@ -56,8 +56,9 @@ int swc_hip_d2h(void *dst_host, const void *src_dev, size_t bytes); /* ordered a
 int swc_hip_d2d(void *dst_dev, const void *src_dev, size_t bytes);  /* async on the stream */
 int swc_hip_fill_f(float *dst_dev, float value, size_t count);      /* initTensorConstant/Zero, kernels.h:23-29 */
 int swc_hip_sync(void);
-/* Scratch device memory for the ops that need some (FC/GEMM calls that are split
- * over K: swc_hip_gemm_workspace_bytes; conv2dGrad_f: the
+/* Scratch device memory for the ops that need some (FC/GEMM and convolution calls
+ * that are cut along K: swc_hip_gemm_workspace_bytes, swc_hip_conv2d_workspace_bytes;
+ * conv2dGrad_f: the
  * transposed gradient and operand copies, up to about twice the size of its
  * largest argument; matrixSoftmaxWithLoss_f: 4*m bytes).  A generated program
  * reserves a slot of its arena and passes it here once; without this call the
@@ -70,6 +71,13 @@ int swc_hip_set_workspace(void *dptr, size_t bytes);
  * of hundreds are split over K).  A generated program takes the maximum over its
  * calls and provides that much with swc_hip_set_workspace. */
 size_t swc_hip_gemm_workspace_bytes(int m, int n, int k);
+/* The same for a conv2d_f / conv2dFused_f call of these shapes (arguments as in
+ * swc_hip_conv2d_f, tensors assumed 16-byte aligned): the output tiles that are
+ * left over after every CU has had its share of whole tiles are cut along K and
+ * their partial sums kept here.  Without a workspace large enough the library
+ * allocates its own at the first such call. */
+size_t swc_hip_conv2d_workspace_bytes(const size_t *odims, const size_t *idims, const size_t *fdims,
+                                      const size_t *kernels, const size_t *strides, const size_t *pads);
 const char *swc_hip_last_error(void);         /* message of the last failure on this thread ("" if none) */
 void *swc_hip_stream(void);                   /* the hipStream_t ops are launched on */
 int swc_hip_set_stream(void *hip_stream);     /* launch on a caller-owned stream (NULL: back to the library's own) */

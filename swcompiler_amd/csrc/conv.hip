@@ -187,148 +187,312 @@ __global__ __launch_bounds__(kThreads) void conv_igemm(const float *__restrict__
 // 32-bit byte offset per lane per load — out-of-image taps and rows past M get
 // the out-of-range offset and arrive in LDS as zeros.  Needs iC % 4 == 0,
 // 16-byte-aligned tensors and input/filter below 2 GiB.
+//
+// Work is counted in units of one K slice of one tile.  The first `dp_tiles`
+// workgroups each take a whole tile.  The tiles that are left — fewer than the
+// chip holds workgroups at a time, so that handing them out whole would leave
+// most CUs idle while a few finish — are cut along K: their units form one
+// sequence that `sk_wgs` further workgroups share evenly (the first `r` take
+// q + 1 units, the others q).  A workgroup whose share covers a whole tile
+// stores it as usual; otherwise it stores the raw partial sums of its piece in
+// slot 2s (the piece its share begins with) or 2s + 1 (the piece it ends with)
+// of `part`, and conv_sk_finish adds the pieces of each tile in K order.
+struct SkPlan {
+    int dp_tiles;   // tiles computed whole, one workgroup each
+    int sk_wgs;     // workgroups sharing the remaining tiles (0: none remain)
+    int q, r;       // units per sharing workgroup: q, and one more for the first r
+};
+
+// Tile number -> tile coordinates (see tile_coords): the whole tiles are renumbered for the 8 XCDs, the
+// shared ones are taken in order.
+__device__ __forceinline__ void sk_tile_coords(int pid, int dp_tiles, int tiles_m, int tiles_n, int &tile_m, int &tile_n) {
+    constexpr int kXcd = 8;
+    if (pid < dp_tiles && dp_tiles % kXcd == 0) pid = (pid % kXcd) * (dp_tiles / kXcd) + pid / kXcd;
+    constexpr int kGroup = 8;
+    const int per_group = kGroup * tiles_n;
+    const int group = pid / per_group;
+    const int first_m = group * kGroup;
+    const int rows = (tiles_m - first_m < kGroup) ? (tiles_m - first_m) : kGroup;
+    const int in_group = pid - group * per_group;
+    tile_m = first_m + in_group % rows;
+    tile_n = in_group / rows;
+}
+
 template <int TM, int TN, int STAGES, bool MID = false>
 __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ in, const float *__restrict__ filt,
                                                      float *__restrict__ out, ConvGeom g, unsigned in_bytes,
-                                                     unsigned filt_bytes, Epilogue ep) {
+                                                     unsigned filt_bytes, Epilogue ep, SkPlan sk,
+                                                     float *__restrict__ part) {
 #if __HIP_DEVICE_COMPILE__   // the host pass only needs the launch stub
     using T = DmaTile<TM, TN, true, STAGES>;
     extern __shared__ __align__(16) float lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int M = g.M, N = g.OC, K = g.K;
-
-    int tile_m, tile_n;
-    tile_coords((M + T::BM - 1) / T::BM, (N + T::BN - 1) / T::BN, tile_m, tile_n);
-    const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
+    const int tiles_m = (M + T::BM - 1) / T::BM, tiles_n = (N + T::BN - 1) / T::BN;
+    const int nk = (K + BK - 1) / BK;
 
     const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(in, in_bytes);
     const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(filt, filt_bytes);
 
-    // Per load, the output pixel this lane gathers for: element offset of its
-    // window's top-left tap (may be negative) and that tap's coordinates; rows
-    // past M get coordinates no tap can bring back inside the image.
-    int row_off[T::kALoads], iy0[T::kALoads], ix0[T::kALoads], f_base[T::kBLoads];
-#pragma unroll
-    for (int j = 0; j < T::kALoads; ++j) {
-        const int m = m0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
-        if (m < M) {
-            const int ox = m % g.OW;
-            const int t = m / g.OW;
-            const int oy = t % g.OH;
-            const int img = t / g.OH;
-            iy0[j] = oy * g.sh - g.pt;
-            ix0[j] = ox * g.sw - g.pl;
-            row_off[j] = ((img * g.H + iy0[j]) * g.W + ix0[j]) * g.C;
-        } else {
-            iy0[j] = ix0[j] = -(1 << 20);
-            row_off[j] = 0;
-        }
+    // this workgroup's units [u0, u1) of the sequence (tile 0: units 0..nk-1, tile 1: nk..2nk-1, ...)
+    int u0, u1, share = -1;
+    if ((int)blockIdx.x < sk.dp_tiles) {
+        u0 = blockIdx.x * nk;
+        u1 = u0 + nk;
+    } else {
+        share = blockIdx.x - sk.dp_tiles;
+        u0 = sk.dp_tiles * nk + share * sk.q + (share < sk.r ? share : sk.r);
+        u1 = u0 + sk.q + (share < sk.r ? 1 : 0);
     }
-#pragma unroll
-    for (int j = 0; j < T::kBLoads; ++j) {
-        const int n = n0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
-        f_base[j] = n < N ? n * K * 4 : kOutOfRange;
-    }
-    // k position of this lane's chunk, as (ky, kx, ci), stepped by BK per slice
-    int kpos = kc_chunk(lane) * 4;
-    int ky, kx, ci;
-    {
-        const int tap = kpos / g.C;
-        ci = kpos - tap * g.C;
-        ky = tap / g.kw;
-        kx = tap - ky * g.kw;
-    }
-    int va[T::kALoads], vb[T::kBLoads];
-    auto next_offsets = [&]() {   // offsets of the next slice in order
-        const bool k_ok = kpos < K;
-        const int tap_off = (ky * g.W + kx) * g.C + ci;
+    for (int piece = 0; u0 < u1; ++piece) {
+        const int pid = u0 / nk;
+        const int kt_begin = u0 - pid * nk;
+        const int kt_end = (u1 - u0 < nk - kt_begin) ? kt_begin + (u1 - u0) : nk;
+        const bool whole = kt_begin == 0 && kt_end == nk;
+        u0 += kt_end - kt_begin;
+        if (piece) __builtin_amdgcn_s_barrier();   // every wavefront is done reading the ring of the previous piece
+
+        int tile_m, tile_n;
+        sk_tile_coords(pid, sk.dp_tiles, tiles_m, tiles_n, tile_m, tile_n);
+        const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
+        const int k_limit = (kt_end * BK < K) ? kt_end * BK : K;
+
+        // Per load, the output pixel this lane gathers for: element offset of its
+        // window's top-left tap (may be negative) and that tap's coordinates; rows
+        // past M get coordinates no tap can bring back inside the image.
+        int row_off[T::kALoads], iy0[T::kALoads], ix0[T::kALoads], f_base[T::kBLoads];
 #pragma unroll
         for (int j = 0; j < T::kALoads; ++j) {
-            const bool ok = k_ok && (unsigned)(iy0[j] + ky) < (unsigned)g.H && (unsigned)(ix0[j] + kx) < (unsigned)g.W;
-            va[j] = ok ? (row_off[j] + tap_off) * 4 : kOutOfRange;
-        }
-#pragma unroll
-        for (int j = 0; j < T::kBLoads; ++j)
-            vb[j] = (k_ok && f_base[j] != kOutOfRange) ? f_base[j] + kpos * 4 : kOutOfRange;
-        kpos += BK;
-        ci += BK;
-        while (ci >= g.C) {
-            ci -= g.C;
-            if (++kx == g.kw) {
-                kx = 0;
-                ++ky;
+            const int m = m0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
+            if (m < M) {
+                const int ox = m % g.OW;
+                const int t = m / g.OW;
+                const int oy = t % g.OH;
+                const int img = t / g.OH;
+                iy0[j] = oy * g.sh - g.pt;
+                ix0[j] = ox * g.sw - g.pl;
+                row_off[j] = ((img * g.H + iy0[j]) * g.W + ix0[j]) * g.C;
+            } else {
+                iy0[j] = ix0[j] = -(1 << 20);
+                row_off[j] = 0;
             }
         }
-    };
-
-    v16f acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
-#pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s) {
-        next_offsets();
-        float *wr = lds + s * T::kStageFloats;
-#pragma unroll
-        for (int j = 0; j < T::kALoads; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t *)(wr + (4 * j + wave) * 256), 16, va[j], 0, 0, 0);
-#pragma unroll
-        for (int j = 0; j < T::kBLoads; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_t *)(wr + T::kAFloats + (4 * j + wave) * 256), 16,
-                                                     vb[j], 0, 0, 0);
-    }
-    const int nk = (K + BK - 1) / BK;
-    int rd_stage = 0, wr_stage = STAGES - 1;
-    if constexpr (MID) {   // ring hand-over after the first MFMA group of a slice (dma_step_mid)
-        ring_sync<(STAGES - 2) * T::kLoads>();   // slice 0 has landed
-        Frag<TM, TN> frag[2];
-        load_frag_swz<TM, TN, true>(frag[0], lds, lds + T::kAFloats, 0, wave >> 1, wave & 1, lane & 31, lane >> 5);
-        for (int kt = 0; kt < nk; ++kt) {
-            next_offsets();
-            const int nx_stage = rd_stage + 1 == STAGES ? 0 : rd_stage + 1;
-            dma_step_mid<TM, TN, true, STAGES>(lds + wr_stage * T::kStageFloats, lds + rd_stage * T::kStageFloats,
-                                               lds + nx_stage * T::kStageFloats, rsrc_a, rsrc_b, va, vb, acc, frag,
-                                               wave, lane);
-            rd_stage = nx_stage;
-            wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
+        for (int j = 0; j < T::kBLoads; ++j) {
+            const int n = n0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
+            f_base[j] = n < N ? n * K * 4 : kOutOfRange;
         }
-    } else {
-        for (int kt = 0; kt < nk; ++kt) {
-            ring_sync<(STAGES - 2) * T::kLoads>();
+        // k position of this lane's chunk, as (ky, kx, ci), stepped by BK per slice
+        int kpos = kt_begin * BK + kc_chunk(lane) * 4;
+        int ky, kx, ci;
+        {
+            const int tap = kpos / g.C;
+            ci = kpos - tap * g.C;
+            ky = tap / g.kw;
+            kx = tap - ky * g.kw;
+        }
+        int va[T::kALoads], vb[T::kBLoads];
+        auto next_offsets = [&]() {   // offsets of the next slice in order
+            const bool k_ok = kpos < k_limit;
+            const int tap_off = (ky * g.W + kx) * g.C + ci;
+#pragma unroll
+            for (int j = 0; j < T::kALoads; ++j) {
+                const bool ok = k_ok && (unsigned)(iy0[j] + ky) < (unsigned)g.H && (unsigned)(ix0[j] + kx) < (unsigned)g.W;
+                va[j] = ok ? (row_off[j] + tap_off) * 4 : kOutOfRange;
+            }
+#pragma unroll
+            for (int j = 0; j < T::kBLoads; ++j)
+                vb[j] = (k_ok && f_base[j] != kOutOfRange) ? f_base[j] + kpos * 4 : kOutOfRange;
+            kpos += BK;
+            ci += BK;
+            while (ci >= g.C) {
+                ci -= g.C;
+                if (++kx == g.kw) {
+                    kx = 0;
+                    ++ky;
+                }
+            }
+        };
+
+        v16f acc[TM][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+#pragma unroll
+        for (int s = 0; s < STAGES - 1; ++s) {
             next_offsets();
-            dma_step<TM, TN, true, STAGES>(lds + wr_stage * T::kStageFloats, lds + rd_stage * T::kStageFloats, rsrc_a,
-                                           rsrc_b, va, vb, acc, wave, lane);
-            rd_stage = rd_stage + 1 == STAGES ? 0 : rd_stage + 1;
-            wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
+            float *wr = lds + s * T::kStageFloats;
+#pragma unroll
+            for (int j = 0; j < T::kALoads; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t *)(wr + (4 * j + wave) * 256), 16, va[j], 0, 0,
+                                                         0);
+#pragma unroll
+            for (int j = 0; j < T::kBLoads; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_t *)(wr + T::kAFloats + (4 * j + wave) * 256),
+                                                         16, vb[j], 0, 0, 0);
+        }
+        int rd_stage = 0, wr_stage = STAGES - 1;
+        if constexpr (MID) {   // ring hand-over after the first MFMA group of a slice (dma_step_mid)
+            ring_sync<(STAGES - 2) * T::kLoads>();   // the first slice has landed
+            Frag<TM, TN> frag[2];
+            load_frag_swz<TM, TN, true>(frag[0], lds, lds + T::kAFloats, 0, wave >> 1, wave & 1, lane & 31, lane >> 5);
+            for (int kt = kt_begin; kt < kt_end; ++kt) {
+                next_offsets();
+                const int nx_stage = rd_stage + 1 == STAGES ? 0 : rd_stage + 1;
+                dma_step_mid<TM, TN, true, STAGES>(lds + wr_stage * T::kStageFloats, lds + rd_stage * T::kStageFloats,
+                                                   lds + nx_stage * T::kStageFloats, rsrc_a, rsrc_b, va, vb, acc, frag,
+                                                   wave, lane);
+                rd_stage = nx_stage;
+                wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
+            }
+        } else {
+            for (int kt = kt_begin; kt < kt_end; ++kt) {
+                ring_sync<(STAGES - 2) * T::kLoads>();
+                next_offsets();
+                dma_step<TM, TN, true, STAGES>(lds + wr_stage * T::kStageFloats, lds + rd_stage * T::kStageFloats, rsrc_a,
+                                               rsrc_b, va, vb, acc, wave, lane);
+                rd_stage = rd_stage + 1 == STAGES ? 0 : rd_stage + 1;
+                wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
+            }
+        }
+        wait_vmcnt<0>();   // the trailing dummy loads still target this workgroup's LDS
+        acc_settle(acc);
+        if (whole) {
+            store_tile<TM, TN>(acc, out, (size_t)N, M, N, m0 + (wave >> 1) * 32 * TM, n0 + (wave & 1) * 32 * TN, lane, ep);
+        } else {
+            float *slot = part + (size_t)(2 * share + (piece ? 1 : 0)) * (T::BM * T::BN);
+            store_tile_impl<TM, TN, false>(acc, slot, (size_t)T::BN, T::BM, T::BN, (wave >> 1) * 32 * TM,
+                                           (wave & 1) * 32 * TN, lane, Epilogue{});
         }
     }
-    wait_vmcnt<0>();   // the trailing dummy loads still target this workgroup's LDS
-    acc_settle(acc);
-    store_tile<TM, TN>(acc, out, (size_t)N, M, N, m0 + (wave >> 1) * 32 * TM, n0 + (wave & 1) * 32 * TN, lane, ep);
 #endif
 }
 
-template <int TM, int TN, int STAGES, bool MID = false>
-int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGeom &g, size_t in_bytes,
-                    size_t filt_bytes, const Epilogue &ep) {
+// Adds the pieces of every shared tile that more than one workgroup worked on (see conv_dma) in K order and
+// applies the epilogue.  blockIdx.x = shared tile, blockIdx.y = block of 16 rows of it.
+template <int BM, int BN>
+__global__ __launch_bounds__(256) void conv_sk_finish(float *__restrict__ out, const float *__restrict__ part, int M,
+                                                      int N, int nk, SkPlan sk, Epilogue ep, int vec_ok) {
+    const int t = blockIdx.x;
+    const int first = t * nk, last = first + nk - 1;   // this tile's units, counted from the first shared unit
+    const int big = sk.r * (sk.q + 1);                 // units held by the shares of q + 1
+    auto share_of = [&](int u) { return u < big ? u / (sk.q + 1) : sk.r + (u - big) / sk.q; };
+    const int s_lo = share_of(first), s_hi = share_of(last);
+    if (s_lo == s_hi) return;   // one workgroup had the whole tile and stored it
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    int tile_m, tile_n;
+    sk_tile_coords(sk.dp_tiles + t, sk.dp_tiles, tiles_m, tiles_n, tile_m, tile_n);
+    constexpr int kQuads = 16 * BN / 4;   // float4s in a block of 16 rows
+    for (int i = threadIdx.x; i < kQuads; i += 256) {
+        const int r = blockIdx.y * 16 + i / (BN / 4), c = (i % (BN / 4)) * 4;
+        const int row = tile_m * BM + r, col = tile_n * BN + c;
+        if (row >= M || col >= N) continue;
+        float4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int s = s_lo; s <= s_hi; ++s) {
+            const int begin = s * sk.q + (s < sk.r ? s : sk.r);
+            const float *slot = part + (size_t)(2 * s + (begin < first ? 1 : 0)) * (BM * BN);
+            const float4 v = *reinterpret_cast<const float4 *>(slot + r * BN + c);
+            sum.x += v.x, sum.y += v.y, sum.z += v.z, sum.w += v.w;
+        }
+        float x[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (col + e >= N) break;   // same arithmetic as store_tile_impl
+            float y = x[e] + (ep.bias ? ep.bias[col + e] : 0.f);
+            if (ep.bn_mean) {
+                const float ve = ep.bn_var[col + e] + ep.eps;
+                const float slope = (float)((double)ep.bn_scale[col + e] / sqrt((double)ve));
+                y = fmaf(y - ep.bn_mean[col + e], slope, ep.bn_bias[col + e]);
+            }
+            if (ep.relu) y = (y > 0.f) ? y : 0.f;
+            x[e] = y;
+        }
+        float *dst = out + (size_t)row * N + col;
+        if (vec_ok && col + 3 < N) {
+            *reinterpret_cast<float4 *>(dst) = make_float4(x[0], x[1], x[2], x[3]);
+        } else {
+            for (int e = 0; e < 4 && col + e < N; ++e) dst[e] = x[e];
+        }
+    }
+}
+
+// How the tiles of an M x OC output are handed out (see conv_dma): whole tiles while they fill every
+// workgroup slot of the chip (`slots` = CUs x workgroups resident per CU), the rest cut along K — when at
+// least one full round of whole tiles precedes them and they would fill less than half of the last round;
+// otherwise (small layers, nearly full last rounds) the pieces and the second kernel cost more than the idle
+// CUs (LeNet's 12x12x20 -> 50 layer: 20 us whole, 28 us cut).
+SkPlan sk_plan(long tiles, int nk, int slots, bool allow_shared) {
+    SkPlan p{(int)tiles, 0, 0, 0};
+    const long rest = tiles % slots;
+    if (!allow_shared || rest == 0 || tiles < slots || 2 * rest > slots) return p;
+    const long units = rest * nk;
+    long wgs = slots;
+    if (units < 4 * wgs) wgs = units / 4;   // at least four slices per share: a piece costs a ring start and a tile store
+    if (wgs <= rest) return p;              // shares of a tile or more each: nothing to gain
+    p.dp_tiles = (int)(tiles - rest);
+    p.sk_wgs = (int)wgs;
+    p.q = (int)(units / wgs);
+    p.r = (int)(units % wgs);
+    return p;
+}
+
+// Workgroups of one kernel variant that the chip holds at a time (its LDS and registers decide).
+template <int TM, int TN, int STAGES, bool MID>
+int conv_dma_slots() {
+    if (const char *e = getenv("SWC_HIP_CONV_SLOTS"))   // tests: pretend the chip holds this many workgroups
+        if (atoi(e) > 0) return atoi(e);
+    static int per_cu = 0;
+    if (!per_cu) {
+        using T = DmaTile<TM, TN, true, STAGES>;
+        auto kern = conv_dma<TM, TN, STAGES, MID>;
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)T::kLdsBytes);
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, kThreads, T::kLdsBytes) != hipSuccess || n < 1) {
+            (void)hipGetLastError();
+            n = 1;
+        }
+        per_cu = n;
+    }
+    return per_cu * num_cus();
+}
+
+template <int TM, int TN, int STAGES, bool MID>
+SkPlan conv_dma_plan(const ConvGeom &g, bool allow_shared) {
     using T = DmaTile<TM, TN, true, STAGES>;
     const long tiles = (long)((g.M + T::BM - 1) / T::BM) * ((g.OC + T::BN - 1) / T::BN);
+    return sk_plan(tiles, (g.K + BK - 1) / BK, conv_dma_slots<TM, TN, STAGES, MID>(), allow_shared);
+}
+
+template <int TM, int TN, int STAGES, bool MID>
+size_t conv_dma_scratch_bytes(const ConvGeom &g) {
+    using T = DmaTile<TM, TN, true, STAGES>;
+    return (size_t)2 * conv_dma_plan<TM, TN, STAGES, MID>(g, true).sk_wgs * T::BM * T::BN * sizeof(float);
+}
+
+// `scratch` (may be null) receives the pieces of shared tiles; without it every tile is computed whole.
+template <int TM, int TN, int STAGES, bool MID = false>
+int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGeom &g, size_t in_bytes,
+                    size_t filt_bytes, const Epilogue &ep, float *scratch = nullptr) {
+    using T = DmaTile<TM, TN, true, STAGES>;
+    const long tiles = (long)((g.M + T::BM - 1) / T::BM) * ((g.OC + T::BN - 1) / T::BN);
+    const int nk = (g.K + BK - 1) / BK;
+    const SkPlan p = conv_dma_plan<TM, TN, STAGES, MID>(g, scratch != nullptr);
     auto kern = conv_dma<TM, TN, STAGES, MID>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        SWC_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)T::kLdsBytes));
-        attr_set = true;
-    }
-    kern<<<(unsigned)tiles, kThreads, T::kLdsBytes, stream()>>>(in, filt, out, g, (unsigned)in_bytes,
-                                                                 (unsigned)filt_bytes, ep);
+    kern<<<(unsigned)(p.dp_tiles + p.sk_wgs), kThreads, T::kLdsBytes, stream()>>>(in, filt, out, g, (unsigned)in_bytes,
+                                                                                  (unsigned)filt_bytes, ep, p, scratch);
     SWC_LAUNCH_CHECK();
+    if (p.sk_wgs) {
+        conv_sk_finish<T::BM, T::BN><<<dim3((unsigned)(tiles - p.dp_tiles), T::BM / 16), 256, 0, stream()>>>(
+            out, scratch, g.M, g.OC, nk, p, ep, (g.OC % 4 == 0 && aligned16(out)) ? 1 : 0);
+        SWC_LAUNCH_CHECK();
+    }
     return SWC_HIP_OK;
 }
 
@@ -472,10 +636,74 @@ int launch_conv(bool vec, const float *in, const float *filt, float *out, const 
     return SWC_HIP_OK;
 }
 
-int conv_dispatch(const char *who, float *output, const float *input, const float *filter, const float *bias,
-                  const size_t *odims, const size_t *idims, const size_t *fdims, const size_t *kernels,
-                  const size_t *strides, const size_t *pads, size_t group, const Epilogue &ep_in,
-                  bool bias_optional = false) {
+// The direct-to-LDS variants by name ("TMTN_S", m = ring hand-over in mid-slice).
+enum DmaVariant { kV22_2, kV21_3, kV12_3, kV11_3, kV11_4, kV11_3m, kV21_3m, kV12_3m, kV22_3m, kVariants };
+const char *const kDmaVariantName[kVariants] = {"22_2", "21_3", "12_3", "11_3", "11_4", "11_3m", "21_3m", "12_3m", "22_3m"};
+
+// Calls f.template operator()<TM, TN, STAGES, MID>() for the variant.
+template <class F> auto with_dma_variant(int v, F &&f) {
+    switch (v) {
+    case kV22_2: return f.template operator()<2, 2, 2, false>();
+    case kV21_3: return f.template operator()<2, 1, 3, false>();
+    case kV12_3: return f.template operator()<1, 2, 3, false>();
+    case kV11_3: return f.template operator()<1, 1, 3, false>();
+    case kV11_4: return f.template operator()<1, 1, 4, false>();
+    case kV21_3m: return f.template operator()<2, 1, 3, true>();
+    case kV12_3m: return f.template operator()<1, 2, 3, true>();
+    case kV22_3m: return f.template operator()<2, 2, 3, true>();
+    default: return f.template operator()<1, 1, 3, true>();
+    }
+}
+
+// Whether the leftover tiles are cut along K (SWC_HIP_CONV_SHARE=0 turns it off; read per call).
+bool share_tiles() {
+    const char *e = getenv("SWC_HIP_CONV_SHARE");
+    return !(e && e[0] == '0');
+}
+
+// Variant for a geometry the direct-to-LDS kernels can take; `forced` = SWC_HIP_CONV.
+int pick_dma_variant(const ConvGeom &g, const char *forced, bool shared) {
+    if (forced)
+        for (int v = 0; v < kVariants; ++v)
+            if (!strcmp(forced, kDmaVariantName[v])) return v;
+    // These layers last 80-160 us: how evenly the work divides over the 256 CUs matters as much as the
+    // tile's own efficiency.  With the leftover tiles cut along K, 64x64 tiles (ring hand-over in
+    // mid-slice, three workgroups per CU) were the fastest or within 1 % of it for every layer shape
+    // measured (56x56x64->64: 88 TFLOP/s against 84 for 128x64 tiles; 28x28x128->128: 98 against 92-95).
+    if (shared) return kV11_3m;
+    // All tiles whole: 64x64 tiles while there are at least eight of them per CU; below that 64x128 tiles
+    // for wide layers, which halve the count but keep two workgroups per CU busy to the end.
+    const size_t M = (size_t)g.M;
+    const size_t tiles64 = ((M + 63) / 64) * ((g.OC + 63) / 64);
+    if (tiles64 < 8 * (size_t)num_cus() && g.OC > 64 && ((M + 63) / 64) * ((g.OC + 127) / 128) >= (size_t)num_cus())
+        return kV12_3;
+    return kV11_3m;
+}
+
+struct ConvScratch {   // where a convolution may keep the pieces of shared tiles
+    float *ptr;        // null: take the library's workspace
+    size_t bytes;
+};
+
+bool conv_uses_dma(const ConvGeom &g, const void *input, const void *filter, const char *force) {
+    const size_t in_bytes = (size_t)g.N * g.H * g.W * g.C * 4, filt_bytes = (size_t)g.OC * g.K * 4;
+    if (!(g.C % 4 == 0 && aligned16(input) && aligned16(filter) && in_bytes < kMaxDmaBytes && filt_bytes < kMaxDmaBytes))
+        return false;
+    if (force && !strncmp(force, "reg", 3)) return false;
+    return true;
+}
+
+// Scratch bytes the forward convolution of this geometry uses (0: none).
+size_t conv_scratch_bytes(const ConvGeom &g, const void *input, const void *filter) {
+    const char *force = getenv("SWC_HIP_CONV");
+    if (!share_tiles() || !conv_uses_dma(g, input, filter, force)) return 0;
+    return with_dma_variant(pick_dma_variant(g, force, true), [&]<int TM, int TN, int STAGES, bool MID>() {
+        return conv_dma_scratch_bytes<TM, TN, STAGES, MID>(g);
+    });
+}
+
+int check_conv_dims(const char *who, const size_t *odims, const size_t *idims, const size_t *fdims,
+                    const size_t *kernels, const size_t *strides, const size_t *pads, size_t group) {
     if (!odims || !idims || !fdims || !kernels || !strides || !pads)
         return fail(SWC_HIP_EINVAL, "%s: null shape array", who);
     if (group != 1) return fail(SWC_HIP_EUNSUPPORTED, "%s: group = %zu (only 1 is supported)", who, group);
@@ -493,46 +721,61 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
     const size_t K = fdims[1] * fdims[2] * fdims[3];
     if (M > 0x7fffffffu || K > 0x7fffffffu || M * odims[3] > (size_t)1 << 40)
         return fail(SWC_HIP_EINVAL, "%s: problem too large", who);
+    return SWC_HIP_OK;
+}
+
+ConvGeom make_geom(const size_t *odims, const size_t *idims, const size_t *fdims, const size_t *kernels,
+                   const size_t *strides, const size_t *pads) {
+    return ConvGeom{(int)idims[0],   (int)idims[1],   (int)idims[2],   (int)idims[3], (int)odims[1],
+                    (int)odims[2],   (int)odims[3],   (int)kernels[0], (int)kernels[1], (int)strides[0],
+                    (int)strides[1], (int)pads[0],    (int)pads[1],    (int)(odims[0] * odims[1] * odims[2]),
+                    (int)(fdims[1] * fdims[2] * fdims[3])};
+}
+
+int conv_dispatch(const char *who, float *output, const float *input, const float *filter, const float *bias,
+                  const size_t *odims, const size_t *idims, const size_t *fdims, const size_t *kernels,
+                  const size_t *strides, const size_t *pads, size_t group, const Epilogue &ep_in,
+                  bool bias_optional = false, ConvScratch scratch = {nullptr, 0}) {
+    if (int rc = check_conv_dims(who, odims, idims, fdims, kernels, strides, pads, group)) return rc;
+    const ConvGeom g = make_geom(odims, idims, fdims, kernels, strides, pads);
+    const size_t M = (size_t)g.M;
     if (M == 0 || odims[3] == 0) return SWC_HIP_OK;
     if (!output || !input || !filter || (!bias && !bias_optional)) return fail(SWC_HIP_EINVAL, "%s: null pointer", who);
-    ConvGeom g{(int)idims[0], (int)idims[1], (int)idims[2], (int)idims[3], (int)odims[1], (int)odims[2],
-               (int)odims[3], (int)kernels[0], (int)kernels[1], (int)strides[0], (int)strides[1], (int)pads[0],
-               (int)pads[1], (int)M, (int)K};
     Epilogue ep = ep_in;
     ep.bias = bias;
     const bool vec = (g.C % 4 == 0) && aligned16(input) && aligned16(filter);
-    const size_t in_bytes = idims[0] * idims[1] * idims[2] * idims[3] * 4, filt_bytes = odims[3] * K * 4;
-    const bool dma_ok = vec && in_bytes < kMaxDmaBytes && filt_bytes < kMaxDmaBytes;
+    const size_t in_bytes = idims[0] * idims[1] * idims[2] * idims[3] * 4, filt_bytes = odims[3] * (size_t)g.K * 4;
     const char *force = getenv("SWC_HIP_CONV");   // forces a kernel variant (tests, tuning): reg22 reg21 reg12 reg11 | 22_2 21_3 12_3 11_3 11_4 | 11_3m 21_3m 12_3m 22_3m (m: ring hand-over in mid-slice)
     if (force) {
         if (!strcmp(force, "reg22")) return launch_conv<2, 2>(vec, input, filter, output, g, ep);
         if (!strcmp(force, "reg21")) return launch_conv<2, 1>(vec, input, filter, output, g, ep);
         if (!strcmp(force, "reg12")) return launch_conv<1, 2>(vec, input, filter, output, g, ep);
         if (!strcmp(force, "reg11")) return launch_conv<1, 1>(vec, input, filter, output, g, ep);
-        if (dma_ok) {
-            if (!strcmp(force, "22_2")) return launch_conv_dma<2, 2, 2>(input, filter, output, g, in_bytes, filt_bytes, ep);
-            if (!strcmp(force, "21_3")) return launch_conv_dma<2, 1, 3>(input, filter, output, g, in_bytes, filt_bytes, ep);
-            if (!strcmp(force, "12_3")) return launch_conv_dma<1, 2, 3>(input, filter, output, g, in_bytes, filt_bytes, ep);
-            if (!strcmp(force, "11_3")) return launch_conv_dma<1, 1, 3>(input, filter, output, g, in_bytes, filt_bytes, ep);
-            if (!strcmp(force, "11_4")) return launch_conv_dma<1, 1, 4>(input, filter, output, g, in_bytes, filt_bytes, ep);
-            if (!strcmp(force, "11_3m")) return launch_conv_dma<1, 1, 3, true>(input, filter, output, g, in_bytes, filt_bytes, ep);
-            if (!strcmp(force, "21_3m")) return launch_conv_dma<2, 1, 3, true>(input, filter, output, g, in_bytes, filt_bytes, ep);
-            if (!strcmp(force, "12_3m")) return launch_conv_dma<1, 2, 3, true>(input, filter, output, g, in_bytes, filt_bytes, ep);
-            if (!strcmp(force, "22_3m")) return launch_conv_dma<2, 2, 3, true>(input, filter, output, g, in_bytes, filt_bytes, ep);
-        }
     }
-    if (!(force && !strncmp(force, "reg", 3)) && g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0)
+    bool forced_dma = false;
+    if (force)
+        for (int v = 0; v < kVariants; ++v) forced_dma |= !strcmp(force, kDmaVariantName[v]);
+    if (!forced_dma && !(force && !strncmp(force, "reg", 3)) && g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0)
         return launch_conv_direct(input, filter, bias, output, g, ep);
-    if (dma_ok) {
-        // These layers last 80-160 us: how evenly the tiles divide over the 256 CUs matters as much as
-        // the tile's own efficiency.  64x64 tiles (ring hand-over in mid-slice) while there are at least
-        // eight of them per CU; below that 64x128 tiles for wide layers, which halve the count but keep
-        // two workgroups per CU busy to the end (measured: 105 vs 100 TFLOP/s for 56x56x64->128,
-        // 85 vs 90 for 28x28x128->128).
-        const size_t tiles64 = ((M + 63) / 64) * ((g.OC + 63) / 64);
-        if (tiles64 < 8 * (size_t)num_cus() && g.OC > 64 && ((M + 63) / 64) * ((g.OC + 127) / 128) >= (size_t)num_cus())
-            return launch_conv_dma<1, 2, 3>(input, filter, output, g, in_bytes, filt_bytes, ep);
-        return launch_conv_dma<1, 1, 3, true>(input, filter, output, g, in_bytes, filt_bytes, ep);
+    if (conv_uses_dma(g, input, filter, force)) {
+        // the pieces of shared tiles go into the caller's region when it gave one (and none are made if that
+        // is too small), else into the library workspace
+        float *pieces = nullptr;
+        bool shared = share_tiles();
+        if (shared) {
+            const size_t need = conv_scratch_bytes(g, input, filter);
+            if (!need || (scratch.ptr && scratch.bytes < need)) {
+                shared = false;
+            } else if (scratch.ptr) {
+                pieces = scratch.ptr;
+            } else {
+                pieces = static_cast<float *>(workspace(need, who));
+                if (!pieces) return SWC_HIP_ERUNTIME;
+            }
+        }
+        return with_dma_variant(pick_dma_variant(g, force, shared), [&]<int TM, int TN, int STAGES, bool MID>() {
+            return launch_conv_dma<TM, TN, STAGES, MID>(input, filter, output, g, in_bytes, filt_bytes, ep, pieces);
+        });
     }
     const long tiles_m128 = (M + 127) / 128;
     if (g.OC > 64 && tiles_m128 * ((g.OC + 127) / 128) >= num_cus())
@@ -825,16 +1068,27 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
     splits = splits < 1 ? 1 : (splits > nk ? nk : splits);
     const int sps = (nk + splits - 1) / splits;
     splits = (nk + sps - 1) / sps;
+    // the input gradient as a convolution of outputG with the turned filter
+    const size_t t_odims[4] = {idims[0], idims[1], idims[2], idims[3]};
+    const size_t t_idims[4] = {odims[0], odims[1], odims[2], odims[3]};
+    const size_t t_fdims[4] = {idims[3], kernels[0], kernels[1], odims[3]};
+    const size_t t_strides[2] = {1, 1};
+    const size_t t_pads[4] = {(size_t)(g.kh - 1 - g.pt), (size_t)(g.kw - 1 - g.pl), 0, 0};
     const size_t turned_b = dgrad_conv ? align256(f_elems * 4) : 0;
+    // (the turned filter lies at the start of the workspace, which is 256-byte aligned like outputG must be)
+    const size_t dgrad_b =
+        dgrad_conv ? align256(conv_scratch_bytes(make_geom(t_odims, t_idims, t_fdims, kernels, t_strides, t_pads), outputG,
+                                                 nullptr)) : 0;
     const size_t ogt_b = wgrad_mfma ? align256((size_t)g.OC * lda * 4) : 0;
     const size_t part_b = wgrad_mfma && splits > 1 ? align256((size_t)splits * f_elems * 4) : 0;
     const size_t bias_b = align256((size_t)bias_chunks * g.OC * 4);
-    char *ws = static_cast<char *>(workspace(turned_b + ogt_b + part_b + bias_b, who));
+    char *ws = static_cast<char *>(workspace(turned_b + ogt_b + part_b + bias_b + dgrad_b, who));
     if (!ws) return SWC_HIP_ERUNTIME;
     float *turned = reinterpret_cast<float *>(ws);
     float *ogT = reinterpret_cast<float *>(ws + turned_b);
     float *part = reinterpret_cast<float *>(ws + turned_b + ogt_b);
     float *bias_part = reinterpret_cast<float *>(ws + turned_b + ogt_b + part_b);
+    float *dgrad_pieces = reinterpret_cast<float *>(ws + turned_b + ogt_b + part_b + bias_b);
 
     // ---- bias gradient
     {
@@ -852,14 +1106,10 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
         unsigned blocks = ceil_div(f_elems, 256);
         turn_filter<<<blocks > 1024 ? 1024 : blocks, 256, 0, stream()>>>(filter, turned, g.OC, g.kh, g.kw, g.C);
         SWC_LAUNCH_CHECK();
-        const size_t t_odims[4] = {idims[0], idims[1], idims[2], idims[3]};
-        const size_t t_idims[4] = {odims[0], odims[1], odims[2], odims[3]};
-        const size_t t_fdims[4] = {idims[3], kernels[0], kernels[1], odims[3]};
-        const size_t t_strides[2] = {1, 1};
-        const size_t t_pads[4] = {(size_t)(g.kh - 1 - g.pt), (size_t)(g.kw - 1 - g.pl), 0, 0};
         const Epilogue ep{nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
+        // its shared-tile pieces go into this call's own region: the library workspace is in use here
         const int rc = conv_dispatch(who, inputG, outputG, turned, nullptr, t_odims, t_idims, t_fdims, kernels, t_strides,
-                                     t_pads, 1, ep, /*bias_optional=*/true);
+                                     t_pads, 1, ep, /*bias_optional=*/true, ConvScratch{dgrad_pieces, dgrad_b});
         if (rc != SWC_HIP_OK) return rc;
     } else {
         unsigned blocks = ceil_div(in_elems, 256);
@@ -921,6 +1171,16 @@ int swc_hip_conv2dFused_f(float *output, const float *input, const float *filter
     Epilogue ep{nullptr, bn_mean, bn_var, bn_scale, bn_bias, epsilon, relu};
     return conv_dispatch("swc_hip_conv2dFused_f", output, input, filter, bias, odims, idims, fdims, kernels, strides,
                          pads, group, ep);
+}
+
+size_t swc_hip_conv2d_workspace_bytes(const size_t *odims, const size_t *idims, const size_t *fdims,
+                                      const size_t *kernels, const size_t *strides, const size_t *pads) {
+    if (!ready() || check_conv_dims("swc_hip_conv2d_workspace_bytes", odims, idims, fdims, kernels, strides, pads, 1))
+        return 0;
+    const ConvGeom g = make_geom(odims, idims, fdims, kernels, strides, pads);
+    if (g.M == 0 || g.OC == 0) return 0;
+    if (g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0) return 0;
+    return conv_scratch_bytes(g, nullptr, nullptr);   // (tensors of a generated program are 256-byte aligned)
 }
 
 int swc_hip_conv2dGrad_f(float *inputG, float *filterG, float *biasG, const float *outputG, const float *input,

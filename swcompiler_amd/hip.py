@@ -27,7 +27,7 @@ EXPORTS = [
     "swc_hip_matrixSoftmax_f", "swc_hip_matrixTanh_f", "swc_hip_argMax_i",
     "swc_hip_matrixMatrixFCBias_f", "swc_hip_vecAddRelu_f", "swc_hip_batchnormRelu_f",
     "swc_hip_batchnormReluMaxpool_f", "swc_hip_conv2dFused_f",
-    "swc_hip_set_workspace", "swc_hip_gemm_workspace_bytes", "swc_hip_matrixTrans_f", "swc_hip_matrixTanhGrad_f", "swc_hip_matrixSoftmaxWithLoss_f",
+    "swc_hip_set_workspace", "swc_hip_gemm_workspace_bytes", "swc_hip_conv2d_workspace_bytes", "swc_hip_matrixTrans_f", "swc_hip_matrixTanhGrad_f", "swc_hip_matrixSoftmaxWithLoss_f",
     "swc_hip_matrixSoftmaxGrad_f", "swc_hip_matrixSoftmaxWithLossGrad_f", "swc_hip_conv2dGrad_f",
     "swc_hip_maxpoolGrad_f", "swc_hip_batchedreduceadd_f", "swc_hip_sgd_f", "swc_hip_reluGrad_f",
 ]
@@ -96,6 +96,7 @@ def load_library():
                                         vp, vp, vp, vp, f32, i32]),
         "swc_hip_set_workspace": (i32, [vp, sz]),
         "swc_hip_gemm_workspace_bytes": (sz, [i32, i32, i32]),
+        "swc_hip_conv2d_workspace_bytes": (sz, [szp] * 6),
         "swc_hip_matrixTrans_f": (i32, [i32, i32, vp, i32, vp, i32]),
         "swc_hip_matrixTanhGrad_f": (i32, [i32, i32, vp, i32, vp, i32, vp, i32]),
         "swc_hip_matrixSoftmaxWithLoss_f": (i32, [i32, i32, vp, i32, vp, i32, vp, vp]),
@@ -449,6 +450,12 @@ class SwcHip:
     def gemm_workspace_bytes(self, m, n, k):
         """scratch bytes an m x n x k FC/GEMM call uses on this device (0 unless it is split over K)"""
         return int(self.lib.swc_hip_gemm_workspace_bytes(m, n, k))
+
+    def conv2d_workspace_bytes(self, xshape, fshape, strides=(1, 1), pads=(0, 0, 0, 0)):
+        """scratch bytes a conv2d call of these shapes uses on this device (0 if every tile is computed whole)"""
+        odims = pool_out_dims(xshape, fshape[1:3], strides, pads)[:3] + (fshape[0],)
+        return int(self.lib.swc_hip_conv2d_workspace_bytes(_dims(odims), _dims(xshape), _dims(fshape), _dims(fshape[1:3]),
+                                                           _dims(strides), _dims(pads)))
 
     def set_workspace(self, arr):
         """give the library a DeviceArray to use as scratch (None: its own buffer again)"""

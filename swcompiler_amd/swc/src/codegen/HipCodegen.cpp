@@ -10,6 +10,7 @@
 #include <cassert>
 #include <cstdlib>
 #include <iomanip>
+#include <sstream>
 
 #include "../graphIR/IRGraph.h"
 #include "../graphIR/OpNode.h"
@@ -64,25 +65,36 @@ void HipCodegen::allocateMemAddr() {
     }
 }
 
-// The FC entry points split small-output products over K and keep the partial results in a workspace:
-// the program asks the library how much its calls need and provides it, so that no op allocates.
+// Some FC and convolution calls cut their work along K and keep partial results in a workspace: the program
+// asks the library how much each of its calls needs and provides the maximum, so that no op allocates.
 void HipCodegen::emitWorkspace() {
-    std::vector<std::array<size_t, 3>> shapes;
+    std::vector<std::string> queries;
     for (int i = 0; i < graph_->opNodeNum(); ++i) {
         OpNode *op = graph_->getOpNode(i);
         if (op->getLabel()->getDeviceLabel().type != DeviceType::GPU) continue;   // (runable() counts its calls: not asked here)
         const std::string type = op->getOp()->getOpName();
-        if (type != "MatrixMatrixMul" && type != "MatrixMatrixFCBias" && type != "MatrixMatrixFCBiasRelu") continue;
-        Tensor *x = static_cast<TensorNode *>(op->getParentNode(0))->getTensor();
-        Tensor *w = static_cast<TensorNode *>(op->getParentNode(1))->getTensor();
-        shapes.push_back({x->size() / w->getDim(0), w->getDim(1), w->getDim(0)});
+        auto T = [&](int j) { return static_cast<TensorNode *>(op->getParentNode(j))->getTensor(); };
+        std::ostringstream q;
+        if (type == "MatrixMatrixMul" || type == "MatrixMatrixFCBias" || type == "MatrixMatrixFCBiasRelu") {
+            Tensor *x = T(0), *w = T(1);
+            q << "gpu0_ws_bytes = std::max(gpu0_ws_bytes, swc_hip_gemm_workspace_bytes(" << x->size() / w->getDim(0) << ", "
+              << w->getDim(1) << ", " << w->getDim(0) << "));\n";
+        } else if (type == "Conv2d" || type == "Conv2dWithActivation" || type == "Conv2dBatchNorm") {
+            auto *conv = static_cast<Conv2dOp *>(op->getOp());
+            Tensor *y = static_cast<TensorNode *>(op->getChildNode(0))->getTensor();
+            q << "{\n"
+              << arrayDef("o", y->getDims()) << arrayDef("i", T(0)->getDims()) << arrayDef("f", T(1)->getDims())
+              << arrayDef("k", conv->getKernels()) << arrayDef("s", conv->getStrides()) << arrayDef("p", conv->getPads())
+              << "gpu0_ws_bytes = std::max(gpu0_ws_bytes, swc_hip_conv2d_workspace_bytes(o, i, f, k, s, p));\n}\n";
+        } else {
+            continue;
+        }
+        queries.push_back(q.str());
     }
-    has_workspace_ = !shapes.empty();
-    if (shapes.empty()) return;
+    has_workspace_ = !queries.empty();
+    if (queries.empty()) return;
     writer_ << "size_t gpu0_ws_bytes = 0;\n";
-    for (auto &s : shapes)
-        writer_ << "gpu0_ws_bytes = std::max(gpu0_ws_bytes, swc_hip_gemm_workspace_bytes(" << s[0] << ", " << s[1] << ", "
-                << s[2] << "));\n";
+    for (auto &q : queries) writer_ << q;
     writer_ << "void *gpu0_ws = gpu0_ws_bytes ? swc_hip_malloc(gpu0_ws_bytes) : nullptr;\n"
             << "if (gpu0_ws_bytes && !gpu0_ws) { std::fprintf(stderr, \"%s\\n\", swc_hip_last_error()); return 1; }\n"
             << "if (gpu0_ws) SWC_HIP_CHECK(swc_hip_set_workspace(gpu0_ws, gpu0_ws_bytes));\n";

@@ -151,7 +151,10 @@ def test_hip_program_structure_and_build(gen, tmp_path):
     assert mlp.count("swc_hip_gemm_workspace_bytes(") == 3 and "swc_hip_gemm_workspace_bytes(64, 4096, 784)" in mlp
     assert mlp.index("swc_hip_set_workspace(gpu0_ws, gpu0_ws_bytes)") < mlp.index("// call op routine functions")
     assert mlp.index("swc_hip_set_workspace(nullptr, 0)") < mlp.index("swc_hip_free(gpu0_ws)")
-    assert "workspace" not in code   # no FC in the conv block: no workspace code
+    # ... and of its convolutions: one query per conv, with the conv's own shape arrays
+    assert code.count("swc_hip_conv2d_workspace_bytes(o, i, f, k, s, p)") == 4
+    assert "const size_t o[] = {2, 56, 56, 64};" in code and "const size_t f[] = {128, 3, 3, 64};" in code
+    assert code.index("swc_hip_set_workspace(gpu0_ws, gpu0_ws_bytes)") < code.index("// call op routine functions")
     lenet = generate(gen, "cfg3", "hip", tmp_path, 4)
     assert lenet.count("swc_hip_conv2dFused_f(") == 2 and "swc_hip_matrixMatrixFCBias_f(4, 500, 800" in lenet
     timed = generate(gen, "cfg5b", "hip", tmp_path, 1, iters=10)

@@ -443,6 +443,82 @@ def test_conv_every_variant(rt, oracle, variant, monkeypatch):
         assert_bit_exact(got, want, f"integer conv {idims} variant {variant}")
 
 
+# Leftover output tiles (those beyond the last full round over the chip's workgroup slots) are cut along K and
+# their partial sums added by a second kernel.  SWC_HIP_CONV_SLOTS makes a small chip of the real one so that
+# small shapes have full rounds and leftovers.
+SHARED_CONV_CASES = [((2, 20, 20, 32), (70, 3, 3, 32), (1, 1), (1, 1, 1, 1)),     # oC % 4 != 0: scalar stores
+                     ((3, 17, 23, 32), (136, 3, 3, 32), (1, 1), (1, 1, 1, 1)),    # ragged rows and columns
+                     ((1, 50, 50, 16), (64, 5, 5, 16), (2, 2), (2, 2, 2, 2))]
+
+
+@pytest.mark.parametrize("variant", [None, "11_3m", "11_4", "21_3", "12_3m", "22_2", "22_3m"])
+def test_conv_tiles_shared_along_k(rt, oracle, variant, monkeypatch):
+    print("case conv shared tiles, variant", variant, flush=True)
+    if variant:
+        monkeypatch.setenv("SWC_HIP_CONV", variant)
+    rng = np.random.default_rng(31)
+    for idims, fdims, strides, pads in SHARED_CONV_CASES:
+        oc = fdims[0]
+        x = rng.integers(-4, 5, idims).astype(np.float32)
+        f = rng.integers(-4, 5, fdims).astype(np.float32)
+        b = rng.integers(-4, 5, oc).astype(np.float32)
+        mean, beta = (rng.integers(-4, 5, oc).astype(np.float32) for _ in range(2))
+        var = rng.uniform(0.5, 2.0, oc).astype(np.float32)
+        gamma = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+        dx, df, db = up(rt, x, f, b)
+        bn = up(rt, mean, var, gamma, beta)
+        want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
+        monkeypatch.setenv("SWC_HIP_CONV_SHARE", "0")
+        assert rt.conv2d_workspace_bytes(idims, fdims, strides, pads) == 0
+        whole = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, bn=bn, eps=1e-5, relu=True).numpy()
+        monkeypatch.setenv("SWC_HIP_CONV_SHARE", "1")
+        shared = 0
+        for slots in (3, 4, 5, 6, 7):
+            monkeypatch.setenv("SWC_HIP_CONV_SLOTS", str(slots))
+            shared += rt.conv2d_workspace_bytes(idims, fdims, strides, pads) > 0
+            plain = rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy()
+            fused = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, bn=bn, eps=1e-5, relu=True).numpy()
+            # integer-valued operands: every summation order is exact, so the sums agree bit for bit with the
+            # reference's, and the fused epilogue sees the same sums whether a tile was cut or not
+            assert_bit_exact(plain, want, f"shared tiles {idims} {variant} slots {slots}")
+            assert_bit_exact(fused, whole, f"shared tiles, fused epilogue {idims} {variant} slots {slots}")
+        monkeypatch.delenv("SWC_HIP_CONV_SLOTS")
+        assert shared, f"{idims} {variant}: no slot count made this case share tiles"
+    # real-valued operands: the usual tolerance
+    idims, fdims, strides, pads = SHARED_CONV_CASES[1]
+    monkeypatch.setenv("SWC_HIP_CONV_SLOTS", "4")
+    x = rng.standard_normal(idims).astype(np.float32)
+    f = rng.standard_normal(fdims).astype(np.float32)
+    b = rng.standard_normal(fdims[0]).astype(np.float32)
+    got = rt.conv2d(*up(rt, x, f, b), fdims[1:3], strides, pads).numpy()
+    want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
+    scale = oracle.conv2d(np.abs(x), np.abs(f), np.abs(b), fdims[1:3], strides, pads)
+    assert np.max(np.abs(got - want) / scale) < TOL
+
+
+def test_conv_shared_tiles_in_a_caller_workspace(rt, oracle, monkeypatch):
+    from swcompiler_amd.hip import SwcHipError
+    idims, fdims, strides, pads = SHARED_CONV_CASES[0]
+    monkeypatch.setenv("SWC_HIP_CONV_SLOTS", "4")
+    need = rt.conv2d_workspace_bytes(idims, fdims, strides, pads)
+    assert need > 0
+    rng = np.random.default_rng(32)
+    x = rng.integers(-4, 5, idims).astype(np.float32)
+    f = rng.integers(-4, 5, fdims).astype(np.float32)
+    b = rng.integers(-4, 5, fdims[0]).astype(np.float32)
+    want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
+    exact, short = rt.empty((need // 4,)), rt.empty((need // 4 - 4,))
+    try:
+        rt.set_workspace(exact)
+        assert_bit_exact(rt.conv2d(*up(rt, x, f, b), fdims[1:3], strides, pads).numpy(), want, "caller workspace")
+        rt.set_workspace(short)
+        with pytest.raises(SwcHipError, match="workspace"):
+            rt.conv2d(*up(rt, x, f, b), fdims[1:3], strides, pads)
+    finally:
+        rt.sync()
+        rt.set_workspace(None)
+
+
 @pytest.mark.parametrize("idims,fdims,strides,pads", [((4, 28, 28, 1), (20, 5, 5, 1), (1, 1), (0, 0, 0, 0)),
                                                       ((2, 9, 9, 3), (4, 3, 3, 3), (1, 1), (1, 1, 1, 1)),
                                                       ((1, 17, 13, 3), (32, 5, 3, 3), (2, 1), (2, 1, 2, 1)),
