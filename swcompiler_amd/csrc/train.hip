@@ -83,6 +83,31 @@ __global__ __launch_bounds__(kThreads) void sgd_step(size_t n, float *out, const
     }
 }
 
+// The same four elements at a time; out == w (the generated call) is read once.
+template <bool NT, bool IN_PLACE>
+__global__ __launch_bounds__(kThreads) void sgd_step4(size_t n4, float4 *out, const float4 *w, const float4 *dw,
+                                                      float4 *mom, float neglr, float decay, float momentum) {
+#pragma clang fp contract(off)
+    const size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    if (i >= n4) return;
+    const float4 wv = ld4<NT>(w + i), gv = ld4<NT>(dw + i), mv = ld4<NT>(mom + i);
+    const float4 ov = IN_PLACE ? wv : ld4<NT>(out + i);
+    const float wa[4] = {wv.x, wv.y, wv.z, wv.w}, ga[4] = {gv.x, gv.y, gv.z, gv.w}, ma[4] = {mv.x, mv.y, mv.z, mv.w};
+    const float oa[4] = {ov.x, ov.y, ov.z, ov.w};
+    float nm[4], no[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float wd = wa[e] * decay;
+        const float g = wd + ga[e];
+        const float t0 = g * neglr;
+        const float t1 = ma[e] * momentum;
+        nm[e] = t0 + t1;
+        no[e] = oa[e] + nm[e];
+    }
+    st4<NT>(mom + i, make_float4(nm[0], nm[1], nm[2], nm[3]));
+    st4<NT>(out + i, make_float4(no[0], no[1], no[2], no[3]));
+}
+
 // kernels.h:68-76: B[n,m] = A[m,n]^T through a 32x33 LDS tile (coalesced on both sides)
 __global__ __launch_bounds__(256) void matrix_trans(int m, int n, const float *__restrict__ a, size_t lda,
                                                     float *__restrict__ b, size_t ldb) {
@@ -258,6 +283,65 @@ __global__ __launch_bounds__(kThreads) void maxpool_grad(float *__restrict__ ig,
     }
 }
 
+// Windows that tile the image exactly (stride = kernel, no padding, H = OH*kh, W = OW*kw): every input
+// element lies in exactly one window, so one thread per window and channel quad reads its taps once, finds
+// the first maximum in the reference's scan order and writes the whole window of the gradient — outputG at
+// the chosen tap, zeros at the others.  item = (image row of windows, ox, channel quad).
+// KH, KW > 0: the window size as a constant (all taps are loaded before the first comparison); 0: g.kh, g.kw.
+template <bool NT, int KH, int KW>
+__global__ __launch_bounds__(kThreads) void maxpool_grad_tiled(float *__restrict__ ig, const float *__restrict__ og,
+                                                               const float *__restrict__ in, PoolGeom g, int row_base) {
+    const int cq = g.C / 4;
+    const int row_items = g.OW * cq;
+    const int item = blockIdx.x * kThreads + threadIdx.x;
+    if (item >= row_items) return;
+    const int window_row = row_base + blockIdx.y;   // n*OH + oy
+    const int oy = window_row % g.OH, n = window_row / g.OH;
+    const int ox = item / cq;
+    const int c = (item - ox * cq) * 4;
+    const size_t first = (((size_t)n * g.H + (size_t)oy * g.kh) * g.W + (size_t)ox * g.kw) * g.C + c;   // tap (0,0)
+    const size_t row_pitch = (size_t)g.W * g.C;
+    const int kh = KH ? KH : g.kh, kw = KW ? KW : g.kw;
+    const float4 gq = ld4<NT>(reinterpret_cast<const float4 *>(og + ((size_t)window_row * g.OW + ox) * g.C + c));
+    float mx[4];
+    int chosen[4] = {0, 0, 0, 0};
+    if (KH) {
+        float4 q[KH ? KH * KW : 1];
+#pragma unroll
+        for (int tap = 0; tap < KH * KW; ++tap)
+            q[tap] = ld4<NT>(reinterpret_cast<const float4 *>(in + first + (tap / (KW ? KW : 1)) * row_pitch +
+                                                              (size_t)(tap % (KW ? KW : 1)) * g.C));
+#pragma unroll
+        for (int tap = 0; tap < KH * KW; ++tap) {
+            const float val[4] = {q[tap].x, q[tap].y, q[tap].z, q[tap].w};
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (tap == 0 || val[v] > mx[v]) mx[v] = val[v], chosen[v] = tap;
+        }
+    } else {
+        for (int ky = 0; ky < kh; ++ky)
+            for (int kx = 0; kx < kw; ++kx) {
+                const float4 q = ld4<NT>(reinterpret_cast<const float4 *>(in + first + ky * row_pitch + (size_t)kx * g.C));
+                const float val[4] = {q.x, q.y, q.z, q.w};
+                const int tap = ky * kw + kx;
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (tap == 0 || val[v] > mx[v]) mx[v] = val[v], chosen[v] = tap;
+            }
+    }
+    const float gv[4] = {gq.x, gq.y, gq.z, gq.w};
+#pragma unroll
+    for (int ky = 0; ky < kh; ++ky)
+#pragma unroll
+        for (int kx = 0; kx < kw; ++kx) {
+            const int tap = ky * kw + kx;
+            // 0.f + outputG as the reference's "+=" into a zeroed gradient forms it (a -0 becomes +0)
+            st4<NT>(reinterpret_cast<float4 *>(ig + first + ky * row_pitch + (size_t)kx * g.C),
+                    make_float4(chosen[0] == tap ? 0.f + gv[0] : 0.f, chosen[1] == tap ? 0.f + gv[1] : 0.f,
+                                chosen[2] == tap ? 0.f + gv[2] : 0.f, chosen[3] == tap ? 0.f + gv[3] : 0.f));
+        }
+}
+
 } // namespace
 
 extern "C" {
@@ -352,7 +436,22 @@ int swc_hip_sgd_f(size_t size, float *out, float *w, float *dw, float *dw_mom, f
     if (size == 0) return SWC_HIP_OK;
     SWC_ARG(out && w && dw && dw_mom);
     const float neglr = -lr / (float)batch;   // float / size_t in the reference: the divisor converts to float
-    sgd_step<<<grid_for(size, kThreads), kThreads, 0, stream()>>>(size, out, w, dw, dw_mom, neglr, decay, momentum);
+    const size_t n4 = size / 4;
+    if (n4 && aligned16(out) && aligned16(w) && aligned16(dw) && aligned16(dw_mom) && n4 / kThreads < 0x7fffffffu) {
+        const unsigned blocks = (unsigned)((n4 + kThreads - 1) / kThreads);
+        const bool nt = size * sizeof(float) >= kStreamingBytes, in_place = out == w;
+        auto kern = nt ? (in_place ? sgd_step4<true, true> : sgd_step4<true, false>)
+                       : (in_place ? sgd_step4<false, true> : sgd_step4<false, false>);
+        kern<<<blocks, kThreads, 0, stream()>>>(n4, (float4 *)out, (const float4 *)w, (const float4 *)dw, (float4 *)dw_mom,
+                                               neglr, decay, momentum);
+        SWC_LAUNCH_CHECK();
+        const size_t done = n4 * 4;
+        if (done == size) return SWC_HIP_OK;
+        sgd_step<<<1, kThreads, 0, stream()>>>(size - done, out + done, w + done, dw + done, dw_mom + done, neglr, decay,
+                                               momentum);
+    } else {
+        sgd_step<<<grid_for(size, kThreads), kThreads, 0, stream()>>>(size, out, w, dw, dw_mom, neglr, decay, momentum);
+    }
     SWC_LAUNCH_CHECK();
     return SWC_HIP_OK;
 }
@@ -380,6 +479,21 @@ int swc_hip_maxpoolGrad_f(float *inputG, const float *outputG, const float *inpu
     const size_t image_rows = idims[0] * idims[1];
     SWC_ARG(image_rows <= 0x7fffffffu);
     const bool vec = g.C % 4 == 0 && aligned16(inputG) && aligned16(outputG) && aligned16(input);
+    if (vec && g.sh == g.kh && g.sw == g.kw && g.pt == 0 && g.pl == 0 && (long)g.OH * g.kh == g.H &&
+        (long)g.OW * g.kw == g.W && g.kh * g.kw <= 64) {
+        const size_t window_rows = idims[0] * (size_t)g.OH;
+        const unsigned blocks = ceil_div((size_t)g.OW * (g.C / 4), kThreads);
+        const bool nt = total * sizeof(float) >= kStreamingBytes;
+        auto kern = g.kh == 2 && g.kw == 2   ? (nt ? maxpool_grad_tiled<true, 2, 2> : maxpool_grad_tiled<false, 2, 2>)
+                    : g.kh == 3 && g.kw == 3 ? (nt ? maxpool_grad_tiled<true, 3, 3> : maxpool_grad_tiled<false, 3, 3>)
+                                             : (nt ? maxpool_grad_tiled<true, 0, 0> : maxpool_grad_tiled<false, 0, 0>);
+        for (size_t r0 = 0; r0 < window_rows; r0 += 65535) {
+            const unsigned rows = (unsigned)(window_rows - r0 < 65535 ? window_rows - r0 : 65535);
+            kern<<<dim3(blocks, rows), kThreads, 0, stream()>>>(inputG, outputG, input, g, (int)r0);
+            SWC_LAUNCH_CHECK();
+        }
+        return SWC_HIP_OK;
+    }
     const size_t row_items = (size_t)g.W * (vec ? g.C / 4 : g.C);
     // grid.y is limited to 65535: rows beyond that are covered by launching in slabs of rows
     for (size_t r0 = 0; r0 < image_rows; r0 += 65535) {

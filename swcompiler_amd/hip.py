@@ -437,10 +437,11 @@ class SwcHip:
         self._check(self.lib.swc_hip_batchedreduceadd_f(out.ptr, batch.ptr, ns, ss), "batchedreduceadd_f")
         return out
 
-    def sgd(self, w, dw, mom, lr, decay, momentum, batch):
-        """updates w and mom in place (out = w, as the generated call passes them)"""
-        self._check(self.lib.swc_hip_sgd_f(w.size, w.ptr, w.ptr, dw.ptr, mom.ptr, lr, decay, momentum, batch), "sgd_f")
-        return w, mom
+    def sgd(self, w, dw, mom, lr, decay, momentum, batch, out=None):
+        """updates out (default: w itself, as the generated call passes it) and mom in place"""
+        out = w if out is None else out
+        self._check(self.lib.swc_hip_sgd_f(w.size, out.ptr, w.ptr, dw.ptr, mom.ptr, lr, decay, momentum, batch), "sgd_f")
+        return out, mom
 
     def reluGrad(self, src, dest_grad, out=None):
         out = out if out is not None else self.empty(src.shape)

@@ -93,7 +93,22 @@ def test_sgd_bit_exact(rt, oracle, n):
     assert_bit_exact(gm2.numpy(), om2, "sgd momentum, step 2")
 
 
-POOLS = [((2, 8, 8, 5), (2, 2), (2, 2), (0, 0, 0, 0)), ((2, 7, 9, 4), (3, 3), (2, 2), (1, 1, 1, 1)),
+@pytest.mark.parametrize("n", [3, 4096, 100003])
+def test_sgd_into_another_tensor(rt, oracle, n):
+    """out != w: out receives out + the step computed from w (kernels.h:565-573)"""
+    rng = np.random.default_rng(n + 1)
+    w, dw, mom, out = (rng.standard_normal(n).astype(np.float32) for _ in range(4))
+    _, om = oracle.sgd(w, dw, mom, 0.05, 0.001, 0.9, 32)
+    dwv, ddw, dmom, dout = up(rt, w, dw, mom, out)
+    gout, gm = rt.sgd(dwv, ddw, dmom, 0.05, 0.001, 0.9, 32, out=dout)
+    assert_bit_exact(gm.numpy(), om, "sgd momentum")
+    assert_bit_exact(gout.numpy(), out + om, "sgd out")
+    assert_bit_exact(dwv.numpy(), w, "w untouched")
+
+
+POOLS = [((2, 8, 8, 8), (2, 2), (2, 2), (0, 0, 0, 0)), ((2, 9, 12, 8), (3, 3), (3, 3), (0, 0, 0, 0)),
+         ((1, 10, 9, 4), (2, 2), (2, 2), (0, 0, 0, 0)), ((2, 6, 8, 12), (3, 2), (3, 2), (0, 0, 0, 0)),
+         ((2, 8, 8, 5), (2, 2), (2, 2), (0, 0, 0, 0)), ((2, 7, 9, 4), (3, 3), (2, 2), (1, 1, 1, 1)),
          ((1, 6, 6, 3), (3, 3), (1, 1), (1, 1, 1, 1)), ((3, 24, 24, 20), (2, 2), (2, 2), (0, 0, 0, 0)),
          ((2, 9, 11, 7), (3, 2), (2, 3), (1, 0, 0, 1)), ((2, 5, 5, 2), (2, 2), (1, 1), (2, 2, 2, 2))]
 
