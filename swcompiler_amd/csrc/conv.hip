@@ -499,15 +499,17 @@ int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGe
 // ------------------------------------------------------------ small direct conv
 // First layers (iC = 1 or 3, a handful of output channels) have K = kH*kW*iC of
 // a few dozen: far too short for the MFMA pipeline, and iC % 4 != 0 rules out
-// 128-bit gathers.  One thread per output pixel keeps all oC accumulators in
-// registers, walks the taps in the reference's (ky, kx, ci) order and adds
-// fl(x*w) with separate fp32 multiply and add starting from the bias — the very
-// operation sequence of conv2d_f, so this path is bit-exact.  The filter is
-// staged in LDS as [k][oC] and read as wavefront-uniform broadcasts.
+// 128-bit gathers.  A thread computes P output pixels with all their oC
+// accumulators in registers, walks the taps in the reference's (ky, kx, ci)
+// order and adds fl(x*w) with separate fp32 multiply and add starting from the
+// bias — the very operation sequence of conv2d_f, so this path is bit-exact.
+// The filter is staged in LDS as [k][oC] and read as wavefront-uniform 128-bit
+// broadcasts; each such read feeds 8*P VALU operations (with P = 1 the kernel
+// needed the whole LDS bandwidth and ran at half the VALU rate).
 constexpr int kDirectMaxK = 128;
 constexpr int kDirectMaxOC = 32;
 
-template <int OCQ>   // output channels rounded up to 4*OCQ
+template <int OCQ, int P>   // output channels rounded up to 4*OCQ; pixels per thread
 __global__ __launch_bounds__(256) void conv_direct(const float *__restrict__ in, const float *__restrict__ filt,
                                                    const float *__restrict__ bias, float *__restrict__ out,
                                                    ConvGeom g, Epilogue ep) {
@@ -515,7 +517,7 @@ __global__ __launch_bounds__(256) void conv_direct(const float *__restrict__ in,
     constexpr int OCP = 4 * OCQ;
     __shared__ __align__(16) float w[kDirectMaxK * OCP];
     __shared__ float bsh[OCP], mean_sh[OCP], slope_sh[OCP], beta_sh[OCP];
-    __shared__ float stage[256 * OCP];
+    __shared__ float stage[256 * (OCP + 1)];
     const int K = g.K, OC = g.OC;
     for (int i = threadIdx.x; i < K * OCP; i += 256) {
         const int k = i / OCP, oc = i - k * OCP;
@@ -532,89 +534,151 @@ __global__ __launch_bounds__(256) void conv_direct(const float *__restrict__ in,
         }
     }
     __syncthreads();
-    const int m = blockIdx.x * 256 + threadIdx.x;
-    const bool active = m < g.M;
-    const int mm = active ? m : 0;
-    const int ox = mm % g.OW;
-    const int t = mm / g.OW;
-    const int oy = t % g.OH;
-    const int img = t / g.OH;
-    float acc[OCP];
+    // pixel p of this thread: first + p*256 + threadIdx.x (consecutive lanes, consecutive pixels)
+    const int first = blockIdx.x * (256 * P);
+    int iy0[P], ix0[P];
+    long img_base[P];
 #pragma unroll
-    for (int oc = 0; oc < OCP; ++oc) acc[oc] = bsh[oc];
+    for (int p = 0; p < P; ++p) {
+        const int m = first + p * 256 + threadIdx.x;
+        const int mm = m < g.M ? m : 0;
+        const int ox = mm % g.OW;
+        const int t = mm / g.OW;
+        const int oy = t % g.OH;
+        iy0[p] = m < g.M ? oy * g.sh - g.pt : -(1 << 20);   // pixels past M: no tap in bounds
+        ix0[p] = ox * g.sw - g.pl;
+        img_base[p] = (long)(t / g.OH) * g.H;
+    }
+    float acc[P][OCP];
+#pragma unroll
+    for (int p = 0; p < P; ++p)
+#pragma unroll
+        for (int oc = 0; oc < OCP; ++oc) acc[p][oc] = bsh[oc];
     // For a fixed ky the taps (kx, ci) are L = kw*C consecutive floats of one input
     // row (NHWC).  They are fetched eight at a time — all loads of a group issued
-    // before the first multiply — so the pixel's ~K dependent load latencies
-    // shrink to K/8.
+    // before the first multiply.
     const int L = g.kw * g.C;
-    const int ix0 = ox * g.sw - g.pl;
     for (int ky = 0; ky < g.kh; ++ky) {
-        const int iy = oy * g.sh - g.pt + ky;
-        if ((unsigned)iy >= (unsigned)g.H) continue;   // whole kernel row outside: skipped, as in the reference
-        const float *row = in + (((long)img * g.H + iy) * g.W + ix0) * g.C;
-        const int kbase = ky * L;
         for (int j0 = 0; j0 < L; j0 += 8) {
-            float xv[8];
-            bool ok[8];
-            int kx = j0 / g.C, ci = j0 - kx * g.C;
+            float xv[P][8];
+            unsigned ok[P];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                ok[u] = j0 + u < L && (unsigned)(ix0 + kx) < (unsigned)g.W;
-                xv[u] = ok[u] ? row[j0 + u] : 0.f;
-                if (++ci == g.C) {
-                    ci = 0;
-                    ++kx;
+            for (int p = 0; p < P; ++p) {
+                const int iy = iy0[p] + ky;
+                const bool row_ok = (unsigned)iy < (unsigned)g.H;   // whole kernel row outside: skipped, as in the reference
+                const float *row = in + ((img_base[p] + iy) * g.W + ix0[p]) * g.C;
+                int kx = j0 / g.C, ci = j0 - kx * g.C;
+                ok[p] = 0;
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const bool tap_ok = row_ok && j0 + u < L && (unsigned)(ix0[p] + kx) < (unsigned)g.W;
+                    xv[p][u] = tap_ok ? row[j0 + u] : 0.f;
+                    ok[p] |= tap_ok ? 1u << u : 0u;
+                    if (++ci == g.C) {
+                        ci = 0;
+                        ++kx;
+                    }
                 }
             }
+            const int taps = L - j0 < 8 ? L - j0 : 8;            // uniform
+            const unsigned in_group = (1u << taps) - 1u;
+            bool skips = false;
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                if (!ok[u]) continue;
-                const float x = xv[u];
-                const float4 *wk = reinterpret_cast<const float4 *>(&w[(kbase + j0 + u) * OCP]);
+            for (int p = 0; p < P; ++p) skips |= ok[p] != in_group;
+            const float *wk0 = &w[(ky * L + j0) * OCP];
+            if (__builtin_amdgcn_ballot_w64(skips) == 0) {       // no lane of the wavefront skips a tap
 #pragma unroll
-                for (int q = 0; q < OCQ; ++q) {
-                    const float4 wv = wk[q];
-                    acc[4 * q + 0] += x * wv.x;
-                    acc[4 * q + 1] += x * wv.y;
-                    acc[4 * q + 2] += x * wv.z;
-                    acc[4 * q + 3] += x * wv.w;
+                for (int u = 0; u < 8; ++u) {
+                    if (u >= taps) break;
+#pragma unroll
+                    for (int q = 0; q < OCQ; ++q) {
+                        const float4 wv = *reinterpret_cast<const float4 *>(wk0 + u * OCP + 4 * q);
+#pragma unroll
+                        for (int p = 0; p < P; ++p) {
+                            const float x = xv[p][u];
+                            acc[p][4 * q + 0] += x * wv.x;
+                            acc[p][4 * q + 1] += x * wv.y;
+                            acc[p][4 * q + 2] += x * wv.z;
+                            acc[p][4 * q + 3] += x * wv.w;
+                        }
+                    }
+                }
+            } else {   // padding taps are skipped, not added as zeros (a skipped tap leaves -0 and NaN cases alone)
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    if (u >= taps) break;
+#pragma unroll
+                    for (int q = 0; q < OCQ; ++q) {
+                        const float4 wv = *reinterpret_cast<const float4 *>(wk0 + u * OCP + 4 * q);
+#pragma unroll
+                        for (int p = 0; p < P; ++p) {
+                            const bool use = ok[p] >> u & 1;
+                            const float x = xv[p][u];
+                            acc[p][4 * q + 0] = use ? acc[p][4 * q + 0] + x * wv.x : acc[p][4 * q + 0];
+                            acc[p][4 * q + 1] = use ? acc[p][4 * q + 1] + x * wv.y : acc[p][4 * q + 1];
+                            acc[p][4 * q + 2] = use ? acc[p][4 * q + 2] + x * wv.z : acc[p][4 * q + 2];
+                            acc[p][4 * q + 3] = use ? acc[p][4 * q + 3] + x * wv.w : acc[p][4 * q + 3];
+                        }
+                    }
                 }
             }
         }
     }
-    // Results go through LDS as the [pixel][oC] block they form in the output, so
-    // that the global stores are contiguous across the workgroup (a thread's own
-    // oC values are only 4*oC bytes apart from its neighbour's).
-    if (active) {
+    // Results go through LDS so that the global stores are contiguous across the workgroup (a thread's own oC
+    // values are only 4*oC bytes apart from its neighbour's).  Rows of the staging block have an odd stride: the
+    // threads of a wavefront, each writing its own row, then hit distinct banks.  On the way out a wavefront
+    // moves 64/oC whole pixels per step, lane = (pixel in step, channel).
+    const int stride = OC | 1;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int per_step = 64 / OC;   // OC <= kDirectMaxOC: at least two
+    const int lane_px = lane / OC, lane_oc = lane - lane_px * OC;
 #pragma unroll
-        for (int oc = 0; oc < OCP; ++oc) {
-            if (oc >= OC) break;
-            float v = acc[oc];
-            if (bn) v = fmaf(v - mean_sh[oc], slope_sh[oc], beta_sh[oc]);
-            if (ep.relu) v = (v > 0.f) ? v : 0.f;
-            stage[threadIdx.x * OC + oc] = v;
+    for (int p = 0; p < P; ++p) {
+        const int base = first + p * 256;   // (past M: nothing is staged or stored; the barriers are still met)
+        if (p) __syncthreads();
+        if (base + (int)threadIdx.x < g.M) {
+#pragma unroll
+            for (int oc = 0; oc < OCP; ++oc) {
+                if (oc >= OC) continue;   // (not "break": an early exit keeps the compiler from unrolling the pixel loop)
+                float v = acc[p][oc];
+                if (bn) v = fmaf(v - mean_sh[oc], slope_sh[oc], beta_sh[oc]);
+                if (ep.relu) v = (v > 0.f) ? v : 0.f;
+                stage[threadIdx.x * stride + oc] = v;
+            }
         }
+        __syncthreads();
+        const int pixels = (g.M - base < 256) ? (g.M - base) : 256;   // may be <= 0
+        float *o = out + (size_t)base * OC;
+        if (lane_px < per_step)
+            for (int px = wave * per_step + lane_px; px < pixels; px += 4 * per_step)
+                o[px * OC + lane_oc] = stage[px * stride + lane_oc];
     }
-    __syncthreads();
-    const int first = blockIdx.x * 256;
-    const int pixels = (g.M - first < 256) ? (g.M - first) : 256;
-    float *o = out + (size_t)first * OC;
-    for (int i = threadIdx.x; i < pixels * OC; i += 256) o[i] = stage[i];
 }
 
 int launch_conv_direct(const float *in, const float *filt, const float *bias, float *out, const ConvGeom &g,
                        const Epilogue &ep) {
-    const unsigned blocks = ceil_div((size_t)g.M, 256);
     const int ocq = (g.OC + 3) / 4;
+    // four (two) pixels per thread while that leaves at least two workgroups per CU; four only while the
+    // accumulators leave room for two wavefronts per SIMD
+    const bool four = ocq <= 5 && (size_t)g.M >= (size_t)2048 * num_cus();
+    const bool two = !four && (size_t)g.M >= (size_t)1024 * num_cus();
+    const int pixels = four ? 4 : two ? 2 : 1;
+    const unsigned blocks = ceil_div((size_t)g.M, (size_t)256 * pixels);
+    auto launch = [&]<int OCQ>() {
+        if constexpr (OCQ <= 5)
+            if (four) return conv_direct<OCQ, 4><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep);
+        if (two) return conv_direct<OCQ, 2><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep);
+        return conv_direct<OCQ, 1><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep);
+    };
     switch (ocq) {
-    case 1: conv_direct<1><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
-    case 2: conv_direct<2><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
-    case 3: conv_direct<3><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
-    case 4: conv_direct<4><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
-    case 5: conv_direct<5><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
-    case 6: conv_direct<6><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
-    case 7: conv_direct<7><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
-    default: conv_direct<8><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep); break;
+    case 1: launch.template operator()<1>(); break;
+    case 2: launch.template operator()<2>(); break;
+    case 3: launch.template operator()<3>(); break;
+    case 4: launch.template operator()<4>(); break;
+    case 5: launch.template operator()<5>(); break;
+    case 6: launch.template operator()<6>(); break;
+    case 7: launch.template operator()<7>(); break;
+    default: launch.template operator()<8>(); break;
     }
     SWC_LAUNCH_CHECK();
     return SWC_HIP_OK;

@@ -492,10 +492,6 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
             if (!strcmp(force, "21_3m")) return launch_dma<2, 1, 3, true>(a, b, c, m, n, k, lda, ldb, ldc, ep);
             if (dma2_ok) {
                 if (!strcmp(force, "24w4_2x8")) return launch_dma2<2, 4, 4, 2, false, 8>(a, b, c, m, n, k, lda, ldb, ldc, ep);
-                if (!strcmp(force, "22w4_2")) return launch_dma2<2, 2, 4, 2, false>(a, b, c, m, n, k, lda, ldb, ldc, ep);
-                if (!strcmp(force, "22w4_3")) return launch_dma2<2, 2, 4, 3, false>(a, b, c, m, n, k, lda, ldb, ldc, ep);
-                if (!strcmp(force, "24w4_2")) return launch_dma2<2, 4, 4, 2, false>(a, b, c, m, n, k, lda, ldb, ldc, ep);
-                if (!strcmp(force, "24w4_3")) return launch_dma2<2, 4, 4, 3, false>(a, b, c, m, n, k, lda, ldb, ldc, ep);
                 if (!strcmp(force, "14w4_2")) return launch_dma2<1, 4, 4, 2, false>(a, b, c, m, n, k, lda, ldb, ldc, ep);
                 if (!strcmp(force, "14w4_3m")) return launch_dma2<1, 4, 4, 3, true>(a, b, c, m, n, k, lda, ldb, ldc, ep);
                 if (!strcmp(force, "24w2_3m")) return launch_dma2<2, 4, 2, 3, true>(a, b, c, m, n, k, lda, ldb, ldc, ep);

@@ -330,9 +330,7 @@ __global__ __launch_bounds__(kThreads) void maxpool_grad_tiled(float *__restrict
             }
     }
     const float gv[4] = {gq.x, gq.y, gq.z, gq.w};
-#pragma unroll
     for (int ky = 0; ky < kh; ++ky)
-#pragma unroll
         for (int kx = 0; kx < kw; ++kx) {
             const int tap = ky * kw + kx;
             // 0.f + outputG as the reference's "+=" into a zeroed gradient forms it (a -0 becomes +0)
