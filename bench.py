@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--headline-only] [--no-cpu]
 
 Headline workload (the configuration the metric is quoted on): the wide MLP,
-batch 4096 x 784 -> FC 4096 + ReLU -> FC 4096 + ReLU -> FC 10 -> softmax, fp32,
+batch 4096 x 784 -> FC 4096 + ReLU -> FC 4096 + ReLU -> FC 10 + softmax (one call), fp32,
 as the HIP target emits it (bias and ReLU in the GEMM epilogue).  One step = one
 pass of that graph over one batch already resident in HBM.  Prints ONE JSON
 line; `value` is samples/s over exactly K timed steps.

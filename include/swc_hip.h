@@ -256,6 +256,15 @@ int swc_hip_matrixMatrixFCBias_f(int m, int n, int k, const float *a, int lda,
                                  const float *b, int ldb, const float *bias,
                                  float *c, int ldc, int relu);
 
+/* MatrixMatrixFCBias followed by MatrixSoftmax (the classifier head of every
+ * MLP/LeNet graph): c = softmax over each row of A*B + bias, i.e. the result of
+ * matrixMatrixMul_f + batchedadd_f + matrixSoftmax_f (kernels.h:41-56, 542-552,
+ * 88-103).  One launch when n <= 16 (the workgroup that computes 16 rows also
+ * normalises them); otherwise the two kernels in sequence. */
+int swc_hip_matrixMatrixFCBiasSoftmax_f(int m, int n, int k, const float *a, int lda,
+                                        const float *b, int ldb, const float *bias,
+                                        float *c, int ldc);
+
 /* vecAdd_f followed by relu_f. */
 int swc_hip_vecAddRelu_f(int size, const float *a, const float *b, float *c);
 

@@ -300,7 +300,8 @@ template <bool VEC>
 __global__ __launch_bounds__(64 * kSkinnyMaxWaves) void gemm_skinny(const float *__restrict__ A,
                                                                     const float *__restrict__ B,
                                                                     float *__restrict__ C, int M, int N, int K,
-                                                                    size_t lda, size_t ldb, size_t ldc, Epilogue ep) {
+                                                                    size_t lda, size_t ldb, size_t ldc, Epilogue ep,
+                                                                    int softmax) {
     __shared__ float part[kSkinnyMaxWaves][16][17];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
@@ -346,7 +347,22 @@ __global__ __launch_bounds__(64 * kSkinnyMaxWaves) void gemm_skinny(const float 
         if (grow < M && c < N) {
             float x = s + (ep.bias ? ep.bias[c] : 0.f);
             if (ep.relu) x = (x > 0.f) ? x : 0.f;
-            C[(size_t)grow * ldc + c] = x;
+            if (softmax) part[0][r][c] = x;   // (this thread alone read part[.][r][c])
+            else C[(size_t)grow * ldc + c] = x;
+        }
+    }
+    if (softmax) {   // the workgroup holds whole rows: the row softmax of matrixSoftmax_f, one lane per row,
+        __syncthreads();   // with the arithmetic of the stand-alone kernel for short rows
+        const int grow = blockIdx.x * 16 + tid;
+        if (tid < 16 && grow < M) {
+            const float *src = part[0][tid];
+            float *dst = C + (size_t)grow * ldc;
+            float mx = src[0];
+            for (int j = 1; j < N; ++j) mx = fmaxf(mx, src[j]);
+            float sum = 0.f;
+            for (int j = 0; j < N; ++j) sum += fast_exp(src[j] - mx);
+            const float inv = 1.f / sum;
+            for (int j = 0; j < N; ++j) dst[j] = fast_exp(src[j] - mx) * inv;
         }
     }
 }
@@ -449,8 +465,9 @@ bool splitk_plan(int m, int n, int k, int &splits, int &sps, bool forced = false
     return splits > 1 && (size_t)splits * m * n * 4 <= ((size_t)64 << 20);
 }
 
+// softmax != 0: the row softmax of the result is stored instead of the result (n <= 16 only: the caller checks)
 int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda, const float *b, int ldb,
-                  const float *bias, float *c, int ldc, int relu) {
+                  const float *bias, float *c, int ldc, int relu, int softmax = 0) {
     if (m < 0 || n < 0 || k < 0) return fail(SWC_HIP_EINVAL, "%s: negative dimension", who);
     if (m == 0 || n == 0) return SWC_HIP_OK;
     if (!a || !b || !c) return fail(SWC_HIP_EINVAL, "%s: null pointer", who);
@@ -462,8 +479,8 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
         waves = waves < 1 ? 1 : (waves > kSkinnyMaxWaves ? kSkinnyMaxWaves : waves);
         if (waves < 4) waves = 4;   // the reduction step needs 256 threads
         const unsigned blocks = ceil_div(m, 16);
-        if (vec) gemm_skinny<true><<<blocks, 64 * waves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep);
-        else gemm_skinny<false><<<blocks, 64 * waves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep);
+        if (vec) gemm_skinny<true><<<blocks, 64 * waves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep, softmax);
+        else gemm_skinny<false><<<blocks, 64 * waves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep, softmax);
         SWC_LAUNCH_CHECK();
         return SWC_HIP_OK;
     }
@@ -535,6 +552,16 @@ int swc_hip_matrixMatrixFCBias_f(int m, int n, int k, const float *a, int lda, c
                                  const float *bias, float *c, int ldc, int relu) {
     SWC_REQUIRE_INIT();
     return gemm_dispatch("swc_hip_matrixMatrixFCBias_f", m, n, k, a, lda, b, ldb, bias, c, ldc, relu);
+}
+
+int swc_hip_matrixMatrixFCBiasSoftmax_f(int m, int n, int k, const float *a, int lda, const float *b, int ldb,
+                                        const float *bias, float *c, int ldc) {
+    SWC_REQUIRE_INIT();
+    const char *who = "swc_hip_matrixMatrixFCBiasSoftmax_f";
+    if (n > 0 && n <= 16) return gemm_dispatch(who, m, n, k, a, lda, b, ldb, bias, c, ldc, 0, 1);
+    // wider rows: the two kernels in sequence (every softmax kernel reads an element before it overwrites it)
+    if (int rc = gemm_dispatch(who, m, n, k, a, lda, b, ldb, bias, c, ldc, 0)) return rc;
+    return swc_hip_matrixSoftmax_f(m, n, c, ldc, c, ldc);
 }
 
 } // extern "C"

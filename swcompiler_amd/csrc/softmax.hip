@@ -26,10 +26,6 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// exp(x) for x <= 0 through the hardware exp2; relative error ~2e-6 at x = -30,
-// far inside the 1e-4 contract.
-__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
-
 // VEC = float4s per lane; row length n = 4*n4 with n4 <= 64*VEC.
 template <int VEC, bool NT>
 __global__ __launch_bounds__(kWave *kRowsPerBlock) void softmax_rows_reg(const float *a, float *b, int m, int n4,

@@ -96,11 +96,14 @@ class _Ws:
         return res
 
 
-def _fc(be, ws, key, x, w, b, relu, fused):
+def _fc(be, ws, key, x, w, b, relu, fused, softmax=False):
+    """FC + bias, then ReLU or the row softmax; fused: as the single calls the HIP target emits"""
     if fused:
-        return ws(key, be.fcbias, x, w, b, relu=relu)
+        return ws(key, be.fcbias, x, w, b, softmax=True) if softmax else ws(key, be.fcbias, x, w, b, relu=relu)
     y = ws(key + ".mm", be.matrixMatrixMul, x, w)
     y = ws(key + ".add", be.batchedadd, y, b)
+    if softmax:
+        return ws("sm", be.matrixSoftmax, y)
     return ws(key + ".relu", be.relu, y) if relu else y
 
 
@@ -115,11 +118,11 @@ def run(cfg, be, t, fused=False, ws=None):
     w = _Ws(ws)
     if cfg == 1:
         h = _fc(be, w, "fc1", t["x"], t["w1"], t["b1"], True, fused)
-        return w("sm", be.matrixSoftmax, _fc(be, w, "fc2", h, t["w2"], t["b2"], False, fused))
+        return _fc(be, w, "fc2", h, t["w2"], t["b2"], False, fused, softmax=True)
     if cfg == 2:
         h = _fc(be, w, "fc1", t["x"], t["w1"], t["b1"], True, fused)
         h = _fc(be, w, "fc2", h, t["w2"], t["b2"], True, fused)
-        return w("sm", be.matrixSoftmax, _fc(be, w, "fc3", h, t["w3"], t["b3"], False, fused))
+        return _fc(be, w, "fc3", h, t["w3"], t["b3"], False, fused, softmax=True)
     if cfg == 3:
         h = t["x"]
         for i in (1, 2):
@@ -131,7 +134,7 @@ def run(cfg, be, t, fused=False, ws=None):
             h = w(f"p{i}", be.maxpool, h, (2, 2), (2, 2))
         h = h.reshape(h.shape[0], -1)  # ReshapeOp alias, (h,w,c) order
         h = _fc(be, w, "fc1", h, t["w1"], t["b1"], True, fused)
-        return w("sm", be.matrixSoftmax, _fc(be, w, "fc2", h, t["w2"], t["b2"], False, fused))
+        return _fc(be, w, "fc2", h, t["w2"], t["b2"], False, fused, softmax=True)
     if cfg == 4:
         h = t["x"]
         for i in (1, 2, 3, 4):

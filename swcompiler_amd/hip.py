@@ -27,7 +27,7 @@ EXPORTS = [
     "swc_hip_matrixSoftmax_f", "swc_hip_matrixTanh_f", "swc_hip_argMax_i",
     "swc_hip_matrixMatrixFCBias_f", "swc_hip_vecAddRelu_f", "swc_hip_batchnormRelu_f",
     "swc_hip_batchnormReluMaxpool_f", "swc_hip_conv2dFused_f",
-    "swc_hip_set_workspace", "swc_hip_gemm_workspace_bytes", "swc_hip_conv2d_workspace_bytes", "swc_hip_matrixTrans_f", "swc_hip_matrixTanhGrad_f", "swc_hip_matrixSoftmaxWithLoss_f",
+    "swc_hip_set_workspace", "swc_hip_matrixMatrixFCBiasSoftmax_f", "swc_hip_gemm_workspace_bytes", "swc_hip_conv2d_workspace_bytes", "swc_hip_matrixTrans_f", "swc_hip_matrixTanhGrad_f", "swc_hip_matrixSoftmaxWithLoss_f",
     "swc_hip_matrixSoftmaxGrad_f", "swc_hip_matrixSoftmaxWithLossGrad_f", "swc_hip_conv2dGrad_f",
     "swc_hip_maxpoolGrad_f", "swc_hip_batchedreduceadd_f", "swc_hip_sgd_f", "swc_hip_reluGrad_f",
 ]
@@ -89,6 +89,7 @@ def load_library():
         "swc_hip_matrixTanh_f": (i32, [i32, i32, vp, i32, vp, i32]),
         "swc_hip_argMax_i": (i32, [vp, vp, i32, i32, i32]),
         "swc_hip_matrixMatrixFCBias_f": (i32, [i32, i32, i32, vp, i32, vp, i32, vp, vp, i32, i32]),
+        "swc_hip_matrixMatrixFCBiasSoftmax_f": (i32, [i32, i32, i32, vp, i32, vp, i32, vp, vp, i32]),
         "swc_hip_vecAddRelu_f": (i32, [i32, vp, vp, vp]),
         "swc_hip_batchnormRelu_f": (i32, [vp, vp, vp, vp, vp, vp, szp, f32]),
         "swc_hip_batchnormReluMaxpool_f": (i32, [vp, vp, vp, vp, vp, vp, szp, f32, szp, szp, szp, szp]),
@@ -282,14 +283,19 @@ class SwcHip:
         self._check(self.lib.swc_hip_batchedadd_f(out.ptr, batch.ptr, slice_.ptr, rows, cols), "batchedadd_f")
         return out
 
-    def fcbias(self, a, w, bias, relu=False, out=None):
+    def fcbias(self, a, w, bias, relu=False, softmax=False, out=None):
+        """a @ w + bias, then ReLU or the row softmax (the fused calls of the HIP target)"""
         m, k = a.shape
         k2, n = w.shape
-        assert k == k2
+        assert k == k2 and not (relu and softmax)
         out = out if out is not None else self.empty((m, n))
-        self._check(self.lib.swc_hip_matrixMatrixFCBias_f(m, n, k, a.ptr, k, w.ptr, n,
-                                                          bias.ptr if bias is not None else None,
-                                                          out.ptr, n, int(relu)), "matrixMatrixFCBias_f")
+        bptr = bias.ptr if bias is not None else None
+        if softmax:
+            self._check(self.lib.swc_hip_matrixMatrixFCBiasSoftmax_f(m, n, k, a.ptr, k, w.ptr, n, bptr, out.ptr, n),
+                        "matrixMatrixFCBiasSoftmax_f")
+        else:
+            self._check(self.lib.swc_hip_matrixMatrixFCBias_f(m, n, k, a.ptr, k, w.ptr, n, bptr, out.ptr, n, int(relu)),
+                        "matrixMatrixFCBias_f")
         return out
 
     def relu(self, x, out=None):

@@ -75,7 +75,8 @@ void HipCodegen::emitWorkspace() {
         const std::string type = op->getOp()->getOpName();
         auto T = [&](int j) { return static_cast<TensorNode *>(op->getParentNode(j))->getTensor(); };
         std::ostringstream q;
-        if (type == "MatrixMatrixMul" || type == "MatrixMatrixFCBias" || type == "MatrixMatrixFCBiasRelu") {
+        if (type == "MatrixMatrixMul" || type == "MatrixMatrixFCBias" || type == "MatrixMatrixFCBiasRelu" ||
+            type == "MatrixMatrixFCBiasSoftmax") {
             Tensor *x = T(0), *w = T(1);
             q << "gpu0_ws_bytes = std::max(gpu0_ws_bytes, swc_hip_gemm_workspace_bytes(" << x->size() / w->getDim(0) << ", "
               << w->getDim(1) << ", " << w->getDim(0) << "));\n";
@@ -301,6 +302,13 @@ void HipCodegen::emitHipCall(OpNode *op) {
         writer_ << "SWC_HIP_CHECK(swc_hip_matrixMatrixFCBias_f(" << rc.first << ", " << n << ", " << k << ", "
                 << nameOf(in(0)) << ", " << k << ", " << nameOf(in(1)) << ", " << n << ", " << nameOf(in(2)) << ", "
                 << nameOf(out(0)) << ", " << n << ", " << (type == "MatrixMatrixFCBiasRelu" ? 1 : 0) << "));\n";
+    } else if (type == "MatrixMatrixFCBiasSoftmax") {
+        auto rc = rowsCols(T(in(0)));
+        const size_t k = T(in(1))->getDim(0), n = T(in(1))->getDim(1);
+        assert(rc.second == k && "FC: flattened input width != weight rows");
+        writer_ << "SWC_HIP_CHECK(swc_hip_matrixMatrixFCBiasSoftmax_f(" << rc.first << ", " << n << ", " << k << ", "
+                << nameOf(in(0)) << ", " << k << ", " << nameOf(in(1)) << ", " << n << ", " << nameOf(in(2)) << ", "
+                << nameOf(out(0)) << ", " << n << "));\n";
     } else if (type == "MatrixVectorAdd" || type == "BatchedAdd") {
         auto rc = rowsCols(T(in(0)));
         writer_ << "SWC_HIP_CHECK(swc_hip_batchedadd_f(" << nameOf(out(0)) << ", " << nameOf(in(0)) << ", "

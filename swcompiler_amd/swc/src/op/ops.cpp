@@ -58,6 +58,7 @@ void MatrixMatrixMulOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *sha
 void MatrixMatrixFCOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *shape) { fcShape(node, shape); }
 void MatrixMatrixFCBiasOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *shape) { fcShape(node, shape); }
 void MatrixMatrixFCBiasReluOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *shape) { fcShape(node, shape); }
+void MatrixMatrixFCBiasSoftmaxOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *shape) { fcShape(node, shape); }
 
 void ReshapeOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *shape) {
     if (!oshape_.empty()) shape->setShape(oshape_);

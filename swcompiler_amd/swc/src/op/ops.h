@@ -209,6 +209,12 @@ class MatrixMatrixFCBiasReluOp : public Op {
     MatrixMatrixFCBiasReluOp() : Op(DL_OP, 3, 1, "MatrixMatrixFCBiasRelu") {}
     void outTensorShapeGen(OpNode *node, size_t index, TensorShape *shape) override;
 };
+// MatrixMatrixFCBias followed by MatrixSoftmax: swc_hip_matrixMatrixFCBiasSoftmax_f
+class MatrixMatrixFCBiasSoftmaxOp : public Op {
+  public:
+    MatrixMatrixFCBiasSoftmaxOp() : Op(DL_OP, 3, 1, "MatrixMatrixFCBiasSoftmax") {}
+    void outTensorShapeGen(OpNode *node, size_t index, TensorShape *shape) override;
+};
 // ElementAdd followed by Relu: swc_hip_vecAddRelu_f
 class ElementAddReluOp : public Op {
   public:

@@ -211,6 +211,9 @@ void HipFusionPass::run() {
                 if (OpNode *r = soleConsumer(o, "Relu", _graph)) {
                     splice(_graph, o, r, new MatrixMatrixFCBiasReluOp());
                     changed = true;
+                } else if (OpNode *sm = soleConsumer(o, "MatrixSoftmax", _graph)) {
+                    splice(_graph, o, sm, new MatrixMatrixFCBiasSoftmaxOp());
+                    changed = true;
                 }
             } else if (type == "Conv2d") {
                 auto *conv = static_cast<Conv2dOp *>(o->getOp());
@@ -255,7 +258,7 @@ void HipFusionPass::run() {
 bool DeviceMemoryLoweringPass::runsOnGpu(const std::string &t) {
     static const std::set<std::string> gpu = {
         "MatrixMatrixMul", "MatrixVectorAdd", "BatchedAdd", "MatrixMatrixFCBias", "MatrixMatrixFCBiasRelu",
-        "Reshape", "MatrixTanh", "MatrixSoftmax", "ElementAdd", "ElementAddRelu", "Relu", "Dropout",
+        "MatrixMatrixFCBiasSoftmax", "Reshape", "MatrixTanh", "MatrixSoftmax", "ElementAdd", "ElementAddRelu", "Relu", "Dropout",
         "Conv2d", "Conv2dWithActivation", "Conv2dBatchNorm", "MaxPool", "AveragePool", "Transpose",
         "BatchNormalization",
         "BatchNormalizationRelu", "ArgMax"};

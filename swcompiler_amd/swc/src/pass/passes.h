@@ -73,6 +73,7 @@ class ElimTransposePass : public OptimizePass {
 // Rewrites, wherever the intermediate tensor has a single consumer and is not a
 // graph output:
 //   MatrixMatrixFCBias -> Relu                    => MatrixMatrixFCBiasRelu
+//   MatrixMatrixFCBias -> MatrixSoftmax           => MatrixMatrixFCBiasSoftmax
 //   Conv2d -> BatchNormalization [-> Relu]        => Conv2dBatchNorm(relu)
 //   Conv2d -> Relu                                => Conv2dWithActivation(RELU)
 //   BatchNormalization -> Relu                    => BatchNormalizationRelu

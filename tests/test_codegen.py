@@ -144,7 +144,11 @@ def test_hip_program_structure_and_build(gen, tmp_path):
     assert unfused.count("swc_hip_relu_f(") == 4
 
     mlp = generate(gen, "cfg2", "hip", tmp_path, 64)
-    assert mlp.count("swc_hip_matrixMatrixFCBias_f(") == 3 and "swc_hip_batchedadd_f" not in mlp
+    assert mlp.count("swc_hip_matrixMatrixFCBias_f(") == 2 and "swc_hip_batchedadd_f" not in mlp
+    # the classifier head and its softmax are one call
+    assert re.search(r"swc_hip_matrixMatrixFCBiasSoftmax_f\(64, 10, 4096, ", mlp) and "swc_hip_matrixSoftmax_f" not in mlp
+    unfused_mlp = generate(gen, "cfg2", "hip", tmp_path, 64, nofuse=True)
+    assert unfused_mlp.count("swc_hip_matrixMatrixFCBias_f(") == 3 and unfused_mlp.count("swc_hip_matrixSoftmax_f(") == 1
     assert re.search(r"swc_hip_matrixMatrixFCBias_f\(64, 4096, 784, .*, 1\)\);", mlp)
     # the program sizes and owns the scratch memory of its FC calls: one query per call, one buffer, given
     # to the library before the first op and taken back before it is freed

@@ -404,6 +404,28 @@ def test_gemm_every_variant(rt, oracle, variant, monkeypatch):
     assert_bit_exact(rt.fcbias(*up(rt, a, b, bias), relu=False).numpy(), want, f"integer gemm {m}x{k}x{n} variant {variant}")
 
 
+@pytest.mark.parametrize("m,k,n", [(8, 512, 10), (256, 500, 10), (1000, 4096, 10), (33, 70, 16), (5, 12, 1), (17, 36, 3),
+                                   (40, 64, 100), (17, 33, 1000), (300, 128, 17)])
+def test_fcbias_softmax_fused(rt, oracle, m, k, n):
+    """FC + bias + row softmax in one call: the reference's matrixMatrixMul_f, batchedadd_f, matrixSoftmax_f"""
+    print("case fcbias+softmax", m, k, n, flush=True)
+    rng = np.random.default_rng(m + k + n)
+    a = rng.uniform(0, 1, (m, k)).astype(np.float32)
+    w = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32)
+    b = rng.uniform(-0.01, 0.01, n).astype(np.float32)
+    da, dw, db = up(rt, a, w, b)
+    got = rt.fcbias(da, dw, db, softmax=True).numpy()
+    want = oracle.matrixSoftmax(oracle.fcbias(a, w, b))
+    nz = want > 1e-30
+    assert strict_rel_err(got[nz], want[nz]) < 5 * TOL
+    assert np.allclose(got.sum(axis=1), 1.0, atol=1e-5)
+    # the same bits as the two calls in sequence on the device
+    assert_bit_exact(got, rt.matrixSoftmax(rt.fcbias(da, dw, db)).numpy(), "fused vs sequence")
+    # no bias
+    assert_bit_exact(rt.fcbias(da, dw, None, softmax=True).numpy(), rt.matrixSoftmax(rt.fcbias(da, dw, None)).numpy(),
+                     "fused vs sequence, no bias")
+
+
 def test_gemm_split_over_k_uses_exactly_the_size_it_reports(rt, oracle):
     from swcompiler_amd.hip import SwcHipError
     assert rt.gemm_workspace_bytes(4096, 4096, 784) == 0 and rt.gemm_workspace_bytes(8, 10, 512) == 0
