@@ -257,6 +257,29 @@ def run_training(rt, iters=20):
     return rows
 
 
+def run_bn_pool_separately(rt, graphs, iters=20):
+    """BN+ReLU and max-pool of the bandwidth configuration as two launches (the target emits one fused call,
+    which is what that configuration's step times): the two kernels' own rates against the HBM roofline."""
+    t = graphs.make_inputs(5)
+    x = rt.upload(t["p"])
+    bn = [rt.upload(t[f"bn_{k}"]) for k in ("mean", "var", "scale", "bias")]
+    h, y = rt.empty(x.shape), rt.empty((x.shape[0], x.shape[1] // 2, x.shape[2] // 2, x.shape[3]))
+    rows = []
+    for op, fn, nbytes in (("batchnormalization", lambda: rt.batchnormalization(x, *bn, graphs.EPS, relu=True, out=h),
+                            8.0 * x.size),
+                           ("maxpool", lambda: rt.maxpool(h, (2, 2), (2, 2), out=y), 4.0 * x.size + 4.0 * y.size)):
+        for _ in range(3):
+            fn()
+        rt.event_record(0)
+        for _ in range(iters):
+            fn()
+        rt.event_record(1)
+        rows.append(rate(dict(op=op, shape=str(list(x.shape)), ms=rt.event_elapsed_ms(0, 1) / iters, bytes=nbytes)))
+    for a in [x, h, y] + bn:
+        a.free()
+    return rows
+
+
 def cpu_baseline(graphs, rows=64):
     """The reference's CPU kernels on the first `rows` rows of the headline batch."""
     from oracle import binding
@@ -339,6 +362,7 @@ def main():
             others[f"cfg{cfg}"] = dict(batch=r["batch"], samples_per_s=r["samples_per_s"], ms_per_step=r["ms_per_step"],
                                        gpu_ms_per_step=r["gpu_ms"] / steps, graph_replay=r["graph_replay"],
                                        kernels=r["kernels"])
+        others["cfg5"]["kernels_unfused"] = run_bn_pool_separately(rt, graphs)
         others["training_kernels"] = dict(kernels=run_training(rt))
         out["configs"] = others
     if not args.no_cpu:

@@ -153,7 +153,8 @@ def run(cfg, be, t, fused=False, ws=None):
         bn = _bn(t, "bn")
         if fused:
             out["b"] = w("b", be.vecAdd, t["p"], t["q"], relu=True)
-            h = w("c.bn", be.batchnormalization, t["p"], *bn, EPS, relu=True)
+            out["c"] = w("c", be.batchnormReluMaxpool, t["p"], *bn, EPS, (2, 2), (2, 2))
+            return out
         else:
             out["b"] = w("b.relu", be.relu, w("b.add", be.vecAdd, t["p"], t["q"]))
             h = w("c.relu", be.relu, w("c.bn", be.batchnormalization, t["p"], *bn, EPS))

@@ -353,6 +353,15 @@ void HipCodegen::emitHipCall(OpNode *op) {
         writer_ << "SWC_HIP_CHECK(swc_hip_" << (relu ? "batchnormRelu_f(" : "batchnormalization_f(") << nameOf(out(0))
                 << ", " << nameOf(in(0)) << ", " << nameOf(in(3)) << ", " << nameOf(in(4)) << ", " << nameOf(in(1))
                 << ", " << nameOf(in(2)) << ", " << nm << "_inDims, " << std::setprecision(12) << eps << "));\n";
+    } else if (type == "BatchNormReluMaxPool") {   // parents as BatchNormalization: in, scale, bias, mean, var
+        auto *bp = static_cast<BatchNormReluMaxPoolOp *>(op->getOp());
+        writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims()) << arrayDef(nm + "_outDims", T(out(0))->getDims())
+                << arrayDef(nm + "_filterSizes", bp->getKernels()) << arrayDef(nm + "_strides", bp->getStrides())
+                << arrayDef(nm + "_pads", bp->getPads());
+        writer_ << "SWC_HIP_CHECK(swc_hip_batchnormReluMaxpool_f(" << nameOf(out(0)) << ", " << nameOf(in(0)) << ", "
+                << nameOf(in(3)) << ", " << nameOf(in(4)) << ", " << nameOf(in(1)) << ", " << nameOf(in(2)) << ", " << nm
+                << "_inDims, " << std::setprecision(12) << bp->getEpsilon() << ", " << nm << "_outDims, " << nm
+                << "_filterSizes, " << nm << "_strides, " << nm << "_pads));\n";
     } else if (type == "MaxPool") {
         auto *pool = static_cast<MaxPoolOp *>(op->getOp());
         writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims()) << arrayDef(nm + "_outDims", T(out(0))->getDims())

@@ -72,6 +72,10 @@ void MaxPoolOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *shape) {
     const auto idims = dimsOfParent(node, 0);
     shape->setShape(windowedShape(idims, kernels_, strides_, pads_, idims[3]));
 }
+void BatchNormReluMaxPoolOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *shape) {
+    const auto idims = dimsOfParent(node, 0);
+    shape->setShape(windowedShape(idims, kernels_, strides_, pads_, idims[3]));
+}
 void AvgPoolOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *shape) {
     const auto idims = dimsOfParent(node, 0);
     shape->setShape(windowedShape(idims, kernels_, strides_, pads_, idims[3]));

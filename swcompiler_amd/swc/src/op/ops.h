@@ -228,6 +228,21 @@ class BatchNormalizationReluOp : public Op {
     explicit BatchNormalizationReluOp(float eps) : Op(DL_OP, 5, 1, "BatchNormalizationRelu"), epsilon_(eps) {}
     float getEpsilon() const { return epsilon_; }
 };
+// BatchNormalization, Relu, then MaxPool over the result: swc_hip_batchnormReluMaxpool_f
+class BatchNormReluMaxPoolOp : public Op {
+    float epsilon_;
+    std::vector<size_t> kernels_, strides_, pads_;
+
+  public:
+    BatchNormReluMaxPoolOp(float eps, std::vector<size_t> kernels, std::vector<size_t> strides, std::vector<size_t> pads)
+        : Op(DL_OP, 5, 1, "BatchNormReluMaxPool"), epsilon_(eps), kernels_(std::move(kernels)),
+          strides_(std::move(strides)), pads_(std::move(pads)) {}
+    float getEpsilon() const { return epsilon_; }
+    std::vector<size_t> getPads() const { return pads_; }
+    std::vector<size_t> getKernels() const { return kernels_; }
+    std::vector<size_t> getStrides() const { return strides_; }
+    void outTensorShapeGen(OpNode *node, size_t index, TensorShape *shape) override;
+};
 // Conv2d followed by an activation: the class the reference declares
 // (src/op/dlOp/dlOp.h:655-700) but never emits code for.  Only ReLU here.
 class Conv2dWithActivationOp : public Conv2dOp {

@@ -241,6 +241,13 @@ void HipFusionPass::run() {
                     splice(_graph, o, r, new BatchNormalizationReluOp(eps));
                     changed = true;
                 }
+            } else if (type == "BatchNormalizationRelu") {
+                if (OpNode *pool = soleConsumer(o, "MaxPool", _graph)) {
+                    auto *mp = static_cast<MaxPoolOp *>(pool->getOp());
+                    const float eps = static_cast<BatchNormalizationReluOp *>(o->getOp())->getEpsilon();
+                    splice(_graph, o, pool, new BatchNormReluMaxPoolOp(eps, mp->getKernels(), mp->getStrides(), mp->getPads()));
+                    changed = true;
+                }
             } else if (type == "ElementAdd") {
                 if (OpNode *r = soleConsumer(o, "Relu", _graph)) {
                     splice(_graph, o, r, new ElementAddReluOp());
@@ -261,7 +268,7 @@ bool DeviceMemoryLoweringPass::runsOnGpu(const std::string &t) {
         "MatrixMatrixFCBiasSoftmax", "Reshape", "MatrixTanh", "MatrixSoftmax", "ElementAdd", "ElementAddRelu", "Relu", "Dropout",
         "Conv2d", "Conv2dWithActivation", "Conv2dBatchNorm", "MaxPool", "AveragePool", "Transpose",
         "BatchNormalization",
-        "BatchNormalizationRelu", "ArgMax"};
+        "BatchNormalizationRelu", "BatchNormReluMaxPool", "ArgMax"};
     return gpu.count(t) != 0;
 }
 

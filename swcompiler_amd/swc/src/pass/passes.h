@@ -77,6 +77,7 @@ class ElimTransposePass : public OptimizePass {
 //   Conv2d -> BatchNormalization [-> Relu]        => Conv2dBatchNorm(relu)
 //   Conv2d -> Relu                                => Conv2dWithActivation(RELU)
 //   BatchNormalization -> Relu                    => BatchNormalizationRelu
+//   BatchNormalizationRelu -> MaxPool             => BatchNormReluMaxPool
 //   ElementAdd -> Relu                            => ElementAddRelu
 // Each right-hand side is one kernel launch of libswc_hip whose result equals
 // the left-hand sequence of reference kernels.

@@ -161,6 +161,11 @@ def test_hip_program_structure_and_build(gen, tmp_path):
     assert code.index("swc_hip_set_workspace(gpu0_ws, gpu0_ws_bytes)") < code.index("// call op routine functions")
     lenet = generate(gen, "cfg3", "hip", tmp_path, 4)
     assert lenet.count("swc_hip_conv2dFused_f(") == 2 and "swc_hip_matrixMatrixFCBias_f(4, 500, 800" in lenet
+    bnpool = generate(gen, "cfg5c", "hip", tmp_path, 1)
+    assert bnpool.count("swc_hip_batchnormReluMaxpool_f(") == 1 and "swc_hip_maxpool_f" not in bnpool
+    assert "swc_hip_batchnormRelu_f" not in bnpool and "swc_hip_batchnormalization_f" not in bnpool
+    bnpool = generate(gen, "cfg5c", "hip", tmp_path, 1, nofuse=True)
+    assert bnpool.count("swc_hip_batchnormalization_f(") == 1 and bnpool.count("swc_hip_maxpool_f(") == 1
     timed = generate(gen, "cfg5b", "hip", tmp_path, 1, iters=10)
     assert "swc_hip_vecAddRelu_f(" in timed and "swc_time_ms_per_iter" in timed and "swc_iter < 10" in timed
 
