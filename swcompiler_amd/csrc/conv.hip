@@ -394,11 +394,18 @@ __global__ __launch_bounds__(256) void conv_sk_finish(float *__restrict__ out, c
         const int row = tile_m * BM + r, col = tile_n * BN + c;
         if (row >= M || col >= N) continue;
         float4 sum = {0.f, 0.f, 0.f, 0.f};
-        for (int s = s_lo; s <= s_hi; ++s) {
-            const int begin = s * sk.q + (s < sk.r ? s : sk.r);
-            const float *slot = part + (size_t)(2 * s + (begin < first ? 1 : 0)) * (BM * BN);
-            const float4 v = *reinterpret_cast<const float4 *>(slot + r * BN + c);
-            sum.x += v.x, sum.y += v.y, sum.z += v.z, sum.w += v.w;
+        for (int s0 = s_lo; s0 <= s_hi; s0 += 4) {   // four pieces' loads in flight, added in K order
+            float4 v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int s = s0 + i;
+                const int begin = s * sk.q + (s < sk.r ? s : sk.r);
+                const float *slot = part + (size_t)(2 * s + (begin < first ? 1 : 0)) * (BM * BN);
+                v[i] = s <= s_hi ? *reinterpret_cast<const float4 *>(slot + r * BN + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (s0 + i <= s_hi) sum.x += v[i].x, sum.y += v[i].y, sum.z += v[i].z, sum.w += v[i].w;
         }
         float x[4] = {sum.x, sum.y, sum.z, sum.w};
 #pragma unroll
