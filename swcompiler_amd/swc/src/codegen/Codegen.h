@@ -166,6 +166,8 @@ class HipCodegen : public Codegen {
     void allocateMemAddr() override;
     void emitMemAllocations() override;
     void emitWorkspace();
+    bool isDeviceComputeOp(OpNode *op) const;
+    bool deviceOpsAreContiguous() const;
     void emitTensorInitializations() override;
     void emitExecute() override;
     void emitMemFree() override;

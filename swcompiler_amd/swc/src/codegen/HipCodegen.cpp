@@ -164,6 +164,48 @@ void HipCodegen::emitTensorInitializations() {
 }
 
 void HipCodegen::emitExecute() {
+    if (config_.use_dataloader && config_.hip_graph && deviceOpsAreContiguous()) {
+        // The batch loop with the device ops of an iteration as one HIP graph: a pass over whatever the arena
+        // holds (kernels configure themselves), the ops recorded once, and per batch the upload, one graph
+        // launch, the download and the host ops.
+        writer_ << "// warm-up pass and recording of the device ops\n{\n";
+        writer_.indentInc();
+        emitDeviceOpsOnly();
+        writer_.indentDec();
+        writer_ << "}\nSWC_HIP_CHECK(swc_hip_sync());\n";
+        writer_ << "void *swc_graph = NULL;\n";
+        writer_ << "SWC_HIP_CHECK(swc_hip_graph_begin());\n{\n";
+        writer_.indentInc();
+        emitDeviceOpsOnly();
+        writer_.indentDec();
+        writer_ << "}\nSWC_HIP_CHECK(swc_hip_graph_end(&swc_graph));\n";
+        writer_ << "while(loader.next(" << nameOf(graph_->getInferLabelNode()) << ", "
+                << nameOf(graph_->getInferDataNode()) << ")) {\n";
+        writer_.indentInc();
+        bool launched = false;
+        for (int i = 0; i < graph_->topologyNum(); ++i)
+            for (int j = 0; j < graph_->getNumInTopoLevel(i); ++j) {
+                IRNode *node = graph_->getNodeInTopo(i, j);
+                if (node->nodeType() != OP_NODE) continue;
+                auto *op = static_cast<OpNode *>(node);
+                if (op->isRunOnce()) continue;
+                if (isDeviceComputeOp(op)) {
+                    if (!launched) writer_ << "SWC_HIP_CHECK(swc_hip_graph_launch(swc_graph));\n";
+                    launched = true;
+                    continue;
+                }
+                writer_ << "// topology(" << i << ", " << j << "): " << op->name() << " : " << op->getOp()->getOpName()
+                        << "\n";
+                dispatchOpNode(op);
+            }
+        writer_ << "\niter++;\n";
+        if (config_.display > 0) emitPrintGraphOutputs();
+        writer_.indentDec();
+        writer_ << "} //while\n";
+        writer_ << "SWC_HIP_CHECK(swc_hip_sync());\n";
+        writer_ << "SWC_HIP_CHECK(swc_hip_graph_destroy(swc_graph));\n";
+        return;
+    }
     if (config_.use_dataloader) {
         // the batch loop of the CPU target; the per-iteration Scatter of the data
         // tensor and the Gather in front of each host op are ordinary op nodes
@@ -216,17 +258,40 @@ void HipCodegen::emitExecute() {
     writer_ << "SWC_HIP_CHECK(swc_hip_sync());\n";
 }
 
+// an op of the per-iteration part that runs on the device (not a transfer, not a host op)
+bool HipCodegen::isDeviceComputeOp(OpNode *op) const {
+    const std::string type = op->getOp()->getOpName();
+    return !op->isRunOnce() && type != "Scatter" && type != "Gather" &&
+           op->getLabel()->getDeviceLabel().type == DeviceType::GPU;
+}
+
+// In emission order, do all uploads come before the first device op and all downloads and host ops after the
+// last?  Only then can the device ops of an iteration be replayed as one recorded graph.
+bool HipCodegen::deviceOpsAreContiguous() const {
+    int phase = 0;   // 0: before the device ops, 1: among them, 2: after
+    for (int i = 0; i < graph_->topologyNum(); ++i)
+        for (int j = 0; j < graph_->getNumInTopoLevel(i); ++j) {
+            IRNode *node = graph_->getNodeInTopo(i, j);
+            if (node->nodeType() != OP_NODE) continue;
+            auto *op = static_cast<OpNode *>(node);
+            if (op->isRunOnce()) continue;
+            if (isDeviceComputeOp(op)) {
+                if (phase == 2) return false;
+                phase = 1;
+            } else if (phase == 1) {
+                phase = 2;
+            }
+        }
+    return phase != 0;
+}
+
 void HipCodegen::emitDeviceOpsOnly() {
     for (int i = 0; i < graph_->topologyNum(); ++i)
         for (int j = 0; j < graph_->getNumInTopoLevel(i); ++j) {
             IRNode *node = graph_->getNodeInTopo(i, j);
             if (node->nodeType() != OP_NODE) continue;
             auto *op = static_cast<OpNode *>(node);
-            const std::string type = op->getOp()->getOpName();
-            if (op->isRunOnce() || type == "Scatter" || type == "Gather" ||
-                op->getLabel()->getDeviceLabel().type != DeviceType::GPU)
-                continue;
-            emitHipCall(op);
+            if (isDeviceComputeOp(op)) emitHipCall(op);
         }
 }
 

@@ -273,12 +273,25 @@ def test_batch_loop_hip_program_structure(gen, tmp_path):
     # before the loop: the four parameter uploads
     assert code[:code.index("while(loader")].count("swc_hip_h2d(") == 4
     build_hip(tmp_path)
+    # with hip_graph: the device ops of an iteration are recorded once before the loop (after an eager pass) and
+    # each batch is upload, one graph launch, download, host ops
+    code = generate(gen, "mnist_loader", "hip", tmp_path, 44, graph=True)
+    head, body = code.split("while(loader.next(selected, data0))")
+    assert head.count("swc_hip_graph_begin()") == 1 and head.count("swc_hip_matrixMatrixFCBiasSoftmax_f(") == 2
+    assert head.index("swc_hip_sync()", head.index("warm-up pass")) < head.index("swc_hip_graph_begin()")
+    loop = body[:body.index("} //while")]
+    assert loop.count("swc_hip_graph_launch(swc_graph)") == 1 and "swc_hip_matrixMatrixFCBias" not in loop
+    assert loop.index("swc_hip_h2d(data0_dev") < loop.index("swc_hip_graph_launch") < loop.index("swc_hip_d2h(top1_host")
+    assert "swc_hip_graph_destroy(swc_graph)" in body
+    build_hip(tmp_path)
 
 
 @pytest.mark.gpu
-def test_batch_loop_hip_program(gen, oracle, tmp_path):
+@pytest.mark.parametrize("graph", [False, True])
+def test_batch_loop_hip_program(gen, oracle, tmp_path, graph):
+    print("case batch loop, graph =", graph, flush=True)
     images, labels = write_record_file(tmp_path, 44)
-    generate(gen, "mnist_loader", "hip", tmp_path, 44)
+    generate(gen, "mnist_loader", "hip", tmp_path, 44, graph=graph)
     exe = build_hip(tmp_path)
     out = subprocess.run([exe], cwd=tmp_path, check=True, capture_output=True, text=True, timeout=120).stdout
     assert parse_counters(out) == expected_counters(oracle, images, labels)
