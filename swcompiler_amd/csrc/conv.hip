@@ -1049,7 +1049,7 @@ __global__ __launch_bounds__(256) void wgrad_direct(float *__restrict__ fg, cons
     red[threadIdx.x] = sum;
     __syncthreads();
     for (int s = 128; s > 0; s >>= 1) {
-        if (threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+        if ((int)threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
         __syncthreads();
     }
     if (threadIdx.x == 0) fg[e] = red[0];

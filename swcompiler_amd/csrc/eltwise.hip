@@ -11,7 +11,6 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kUnroll = 1;                            // float4 per thread per operand
-constexpr size_t kBlockElems = (size_t)kThreads * kUnroll * 4;
 
 // (x > 0) ? x : 0 of kernels.h:578, kept as a compare+select: a max() would
 // keep -0.0 and is not what the reference computes.

@@ -497,7 +497,6 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
     // hand-over in mid-slice.  <TM><TN>w<WM>_<STAGES>[m][x8]: gemm_dma2, x8 = eight wavefronts per workgroup.  splitk: K split
     // over blockIdx.y with partial tiles in the workspace.
     const char *force = getenv("SWC_HIP_GEMM");
-    const int nk = (k + BK - 1) / BK;
     if (dma_ok && !(force && !strcmp(force, "reg"))) {
         if (force) {
             if (!strcmp(force, "22_2")) return launch_dma<2, 2, 2>(a, b, c, m, n, k, lda, ldb, ldc, ep);
@@ -516,11 +515,12 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
                 if (!strcmp(force, "22w2_2")) return launch_dma2<2, 2, 2, 2, false>(a, b, c, m, n, k, lda, ldb, ldc, ep);
             }
         }
-        // 256x256 tiles with eight wavefronts once they fill the chip (least operand traffic per flop: 146
-        // TFLOP/s at 4096^3 against 134 for 128x128 tiles of four wavefronts), 128x128 tiles next, and 64x64
-        // tiles for everything smaller, where the number of workgroups matters more than their efficiency
-        // few tiles and a K of hundreds: split K over the chip (needs the workspace; not while recording a graph
-        // unless it is already large enough — an eager warm-up run sees to that)
+        // Few output tiles and a K of hundreds: K is split over the chip (needs the workspace; while a graph is
+        // being recorded only if that is already large enough — an eager warm-up run or swc_hip_set_workspace
+        // sees to it).  Otherwise 256x256 tiles with eight wavefronts once they fill the chip (least operand
+        // traffic per flop: 146 TFLOP/s at 4096^3 against 134 for 128x128 tiles of four wavefronts), 128x128
+        // tiles next, and 64x64 tiles for everything smaller, where the number of workgroups matters more than
+        // their efficiency.
         int splits = 0, sps = 0;
         if (dma2_ok && (!force || !strcmp(force, "splitk")) && splitk_plan(m, n, k, splits, sps, force != nullptr))
             return launch_splitk(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps);
