@@ -367,6 +367,59 @@ __global__ __launch_bounds__(64 * kSkinnyMaxWaves) void gemm_skinny(const float 
     }
 }
 
+// ------------------------------------------------------------ few-rows GEMM
+// M <= 16 (single-sample and small-batch inference) with a B of a few MB: the product is bound by the latency
+// of one pass over B.  A workgroup owns 16 columns of C; its sixteen wavefronts split K into contiguous ranges
+// and feed v_mfma_f32_16x16x4_f32 straight from global memory (A is a few KB and stays in cache), all operands
+// of a trip requested before its first MFMA — for K up to 1024 a single trip, i.e. one memory latency.  The
+// sixteen partial 16x16 tiles are summed through LDS in wavefront order.  One launch where the tiled kernels
+// need a split-K pair.
+constexpr int kFewRowsWaves = 16;
+constexpr int kFewRowsUnroll = 16;
+
+__global__ __launch_bounds__(64 * kFewRowsWaves) void gemm_fewrows(const float *__restrict__ A,
+                                                                   const float *__restrict__ B, float *__restrict__ C,
+                                                                   int M, int N, int K, size_t lda, size_t ldb,
+                                                                   size_t ldc, Epilogue ep) {
+    __shared__ float part[kFewRowsWaves][16][17];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 15, kk = lane >> 4;   // as operand A the lane's row is j, as operand B its column
+    const int col = blockIdx.x * 16 + j;
+    const bool col_ok = col < N, row_ok = j < M;
+    const float *arow = A + (size_t)(row_ok ? j : 0) * lda;
+    // this wavefront's range of K, a multiple of 4 long
+    const int chunk = ((K + kFewRowsWaves - 1) / kFewRowsWaves + 3) & ~3;
+    const int k_begin = wave * chunk, k_end = (k_begin + chunk < K) ? k_begin + chunk : K;
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    for (int kb = k_begin; kb < k_end; kb += 4 * kFewRowsUnroll) {
+        float a[kFewRowsUnroll], b[kFewRowsUnroll];
+#pragma unroll
+        for (int u = 0; u < kFewRowsUnroll; ++u) {
+            const int k = kb + 4 * u + kk;
+            const bool k_ok = k < k_end;
+            b[u] = (k_ok && col_ok) ? B[(size_t)k * ldb + col] : 0.f;
+            a[u] = (k_ok && row_ok) ? arow[k] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < kFewRowsUnroll; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u], b[u], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v) part[wave][4 * kk + v][j] = acc[v];   // D[i][j]: i = 4*(l/16) + v
+    __syncthreads();
+    if (tid < 256) {
+        const int r = tid >> 4, c = tid & 15;
+        float s = 0.f;
+        for (int w = 0; w < kFewRowsWaves; ++w) s += part[w][r][c];
+        const int gc = blockIdx.x * 16 + c;
+        if (r < M && gc < N) {
+            float x = s + (ep.bias ? ep.bias[gc] : 0.f);
+            if (ep.relu) x = (x > 0.f) ? x : 0.f;
+            C[(size_t)r * ldc + gc] = x;
+        }
+    }
+}
+
 template <int TM, int TN>
 int launch_tiled(bool vec, const float *a, const float *b, float *c, int m, int n, int k, int lda, int ldb, int ldc,
                  const Epilogue &ep) {
@@ -454,7 +507,10 @@ int launch_splitk(const float *a, const float *b, float *c, int m, int n, int k,
 
 // Split-K plan of an m x n x k product on this device: true with the number of splits and the K slices per
 // split when the shape has too few output tiles to fill the chip.
+bool takes_fewrows(int m, int n, int k) { return m <= 16 && k > 0 && (size_t)k * n <= ((size_t)2 << 20); }
+
 bool splitk_plan(int m, int n, int k, int &splits, int &sps, bool forced = false) {
+    if (!forced && takes_fewrows(m, n, k)) return false;
     const long big_tiles = (long)((m + 127) / 128) * ((n + 127) / 128);
     const int nk = (k + BK - 1) / BK;
     if (n <= 16 || nk < 2 || (!forced && (big_tiles * 4 > num_cus() || nk < 8))) return false;
@@ -485,6 +541,13 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
         SWC_LAUNCH_CHECK();
         return SWC_HIP_OK;
     }
+    const char *force = getenv("SWC_HIP_GEMM");
+    // a handful of rows and a B of a few MB: one latency-bound pass over B (see gemm_fewrows)
+    if (takes_fewrows(m, n, k) && (!force || !strcmp(force, "fewrows"))) {
+        gemm_fewrows<<<ceil_div(n, 16), 64 * kFewRowsWaves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep);
+        SWC_LAUNCH_CHECK();
+        return SWC_HIP_OK;
+    }
     const bool vec = (k % 4 == 0) && (n % 4 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) && aligned16(a) && aligned16(b);
     const long big_tiles = (long)((m + 127) / 128) * ((n + 127) / 128);
     const bool dma_ok = vec && k > 0 && ((size_t)(m - 1) * lda + k) * 4 < kMaxDmaBytes &&
@@ -495,8 +558,7 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
     const long huge_tiles = (long)((m + 255) / 256) * ((n + 255) / 256);
     // Forces a kernel variant (tests, tuning).  reg: register-staged.  <TM><TN>_<STAGES>[m]: gemm_dma, m = ring
     // hand-over in mid-slice.  <TM><TN>w<WM>_<STAGES>[m][x8]: gemm_dma2, x8 = eight wavefronts per workgroup.  splitk: K split
-    // over blockIdx.y with partial tiles in the workspace.
-    const char *force = getenv("SWC_HIP_GEMM");
+    // over blockIdx.y with partial tiles in the workspace.  fewrows: gemm_fewrows where it applies.
     if (dma_ok && !(force && !strcmp(force, "reg"))) {
         if (force) {
             if (!strcmp(force, "22_2")) return launch_dma<2, 2, 2>(a, b, c, m, n, k, lda, ldb, ldc, ep);

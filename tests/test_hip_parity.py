@@ -426,10 +426,33 @@ def test_fcbias_softmax_fused(rt, oracle, m, k, n):
                      "fused vs sequence, no bias")
 
 
+@pytest.mark.parametrize("m,k,n", [(8, 784, 512), (1, 784, 512), (16, 1000, 100), (3, 5, 17), (16, 1, 33), (7, 64, 520),
+                                   (8, 4096, 512), (2, 130, 4099)])
+def test_gemm_of_a_few_rows(rt, oracle, m, k, n):
+    """M <= 16 with a small B: one launch, A in LDS, K split over the wavefronts of a workgroup"""
+    print("case few-rows gemm", m, k, n, flush=True)
+    rng = np.random.default_rng(m * 7 + k + n)
+    a = rng.integers(-8, 9, (m, k)).astype(np.float32)
+    b = rng.integers(-8, 9, (k, n)).astype(np.float32)
+    bias = rng.integers(-8, 9, n).astype(np.float32)
+    exact = a.astype(np.int64) @ b.astype(np.int64)
+    assert_bit_exact(rt.matrixMatrixMul(*up(rt, a, b)).numpy(), exact.astype(np.float32), "integer product")
+    assert_bit_exact(rt.fcbias(*up(rt, a, b, bias), relu=True).numpy(),
+                     np.maximum(exact + bias.astype(np.int64), 0).astype(np.float32), "integer product + bias + relu")
+    a = rng.uniform(0, 1, (m, k)).astype(np.float32)
+    b = rng.uniform(0, 1, (k, n)).astype(np.float32)
+    assert strict_rel_err(rt.matrixMatrixMul(*up(rt, a, b)).numpy(), oracle.matrixMatrixMul(a, b)) < TOL
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    b = rng.standard_normal((k, n)).astype(np.float32)
+    assert scaled_err(rt.matrixMatrixMul(*up(rt, a, b)).numpy(), oracle.matrixMatrixMul(a, b),
+                      np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)) < TOL
+
+
 def test_gemm_split_over_k_uses_exactly_the_size_it_reports(rt, oracle):
     from swcompiler_amd.hip import SwcHipError
     assert rt.gemm_workspace_bytes(4096, 4096, 784) == 0 and rt.gemm_workspace_bytes(8, 10, 512) == 0
-    m, n, k = 8, 512, 784
+    assert rt.gemm_workspace_bytes(8, 512, 784) == 0   # a handful of rows: the one-pass kernel, no scratch
+    m, n, k = 32, 512, 784
     need = rt.gemm_workspace_bytes(m, n, k)
     assert need > 0 and need % (m * n * 4) == 0
     rng = np.random.default_rng(21)
