@@ -151,6 +151,44 @@ __global__ __launch_bounds__(kThreads) void maxpool_vec4(const float *__restrict
     }
 }
 
+// Windows that tile the image exactly (stride = kernel, no padding, H = OH*KH, W = OW*KW: the 2x2/2 pools of
+// the configurations): every tap of every window is in bounds, so a thread — four channels of one window —
+// requests all its taps at once and only then normalises and compares them.  blockIdx.y + row_base = n*OH + oy;
+// blockIdx.x, threadIdx.x walk OW * C/4: 32-bit index arithmetic throughout.  The values and the first-maximum
+// rule are those of maxpool_vec4.
+template <int KH, int KW, bool BN, bool NT>
+__global__ __launch_bounds__(kThreads) void maxpool_tiled(const float *__restrict__ in, float *__restrict__ out,
+                                                          PoolGeom g, int row_base, const float *__restrict__ mean,
+                                                          const float *__restrict__ var,
+                                                          const float *__restrict__ scale,
+                                                          const float *__restrict__ bias, float eps) {
+    const int quads = g.C / 4;
+    const int item = blockIdx.x * kThreads + threadIdx.x;
+    if (item >= g.OW * quads) return;
+    const int ox = item / quads, cq = item - ox * quads;
+    const int window_row = row_base + blockIdx.y;
+    const int oy = window_row % g.OH, n = window_row / g.OH;
+    BnQuad q;
+    if (BN) load_bn_quad(q, mean, var, scale, bias, (size_t)cq * 4, eps);
+    const size_t row_pitch = (size_t)g.W * quads;   // in float4s
+    const float4 *tap0 = reinterpret_cast<const float4 *>(in) + ((size_t)n * g.H + (size_t)oy * KH) * row_pitch +
+                         (size_t)ox * KW * quads + cq;
+    float4 t[KH * KW];
+#pragma unroll
+    for (int i = 0; i < KH * KW; ++i) t[i] = ld4<NT>(tap0 + (i / KW) * row_pitch + (size_t)(i % KW) * quads);
+    float best[4];
+#pragma unroll
+    for (int i = 0; i < KH * KW; ++i) {
+        const float4 v4 = BN ? bn4<true>(t[i], q) : t[i];
+        const float v[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            if (i == 0 || v[c] > best[c]) best[c] = v[c];
+    }
+    st4<NT>(reinterpret_cast<float4 *>(out) + ((size_t)window_row * g.OW + ox) * quads + cq,
+            make_float4(best[0], best[1], best[2], best[3]));
+}
+
 template <bool ARGMAX, bool BN>
 __global__ __launch_bounds__(kThreads) void maxpool_scalar(const float *__restrict__ in, float *__restrict__ out,
                                                            int32_t *__restrict__ arg, PoolGeom g, size_t total,
@@ -324,7 +362,21 @@ int launch_pool(const char *who, const float *input, float *output, int32_t *arg
     PoolGeom g{(int)idims[0], (int)idims[1], (int)idims[2], (int)idims[3], (int)odims[1], (int)odims[2],
                (int)kernels[0], (int)kernels[1], (int)strides[0], (int)strides[1], (int)pads[0], (int)pads[1]};
     const size_t C = idims[3];
-    if (C % 4 == 0 && aligned16(input) && aligned16(output) && (!ARGMAX || aligned16(argmax))) {
+    const bool vec = C % 4 == 0 && aligned16(input) && aligned16(output) && (!ARGMAX || aligned16(argmax));
+    const bool tiles_exactly = g.sh == g.kh && g.sw == g.kw && g.pt == 0 && g.pl == 0 && (size_t)g.OH * g.kh == idims[1] &&
+                               (size_t)g.OW * g.kw == idims[2];
+    // (without batchnorm the strided kernel below is as fast or faster: 53 against 56 us on [256,32,32,256])
+    if (BN && !ARGMAX && vec && tiles_exactly && g.kh == g.kw && (g.kh == 2 || g.kh == 3) && odims[0] * odims[1] <= 0x7fffffffu) {
+        const size_t window_rows = odims[0] * odims[1];
+        const unsigned blocks = (unsigned)(((size_t)g.OW * (C / 4) + kThreads - 1) / kThreads);
+        const bool nt = in_total * sizeof(float) >= kStreamingBytes;
+        auto kern = g.kh == 2 ? (nt ? maxpool_tiled<2, 2, BN, true> : maxpool_tiled<2, 2, BN, false>)
+                              : (nt ? maxpool_tiled<3, 3, BN, true> : maxpool_tiled<3, 3, BN, false>);
+        for (size_t r0 = 0; r0 < window_rows; r0 += 65535) {   // grid.y is limited to 65535
+            const unsigned rows = (unsigned)(window_rows - r0 < 65535 ? window_rows - r0 : 65535);
+            kern<<<dim3(blocks, rows), kThreads, 0, stream()>>>(input, output, g, (int)r0, mean, var, scale, bias, eps);
+        }
+    } else if (vec) {
         const size_t total4 = total / 4;
         const unsigned blocks = quad_stable_blocks(total4, (unsigned)(C / 4), (unsigned)num_cus() * 128u);
         if (in_total * sizeof(float) >= kStreamingBytes)

@@ -243,7 +243,8 @@ def test_batchnorm(rt, oracle, idims):
 POOLS = [((2, 8, 8, 5), (2, 2), (2, 2), (0, 0, 0, 0)), ((1, 9, 9, 3), (3, 3), (3, 3), (0, 0, 0, 0)),
          ((2, 7, 9, 4), (3, 3), (2, 2), (1, 1, 1, 1)), ((1, 7, 7, 2), (2, 2), (2, 2), (0, 0, 0, 0)),
          ((3, 24, 24, 20), (2, 2), (2, 2), (0, 0, 0, 0)), ((2, 8, 8, 50), (2, 2), (2, 2), (0, 0, 0, 0)),
-         ((2, 28, 28, 128), (2, 2), (2, 2), (0, 0, 0, 0)), ((1, 9, 9, 8), (3, 2), (1, 3), (0, 1, 0, 1))]
+         ((2, 28, 28, 128), (2, 2), (2, 2), (0, 0, 0, 0)), ((1, 9, 9, 8), (3, 2), (1, 3), (0, 1, 0, 1)),
+         ((2, 9, 12, 8), (3, 3), (3, 3), (0, 0, 0, 0)), ((1, 10, 9, 4), (2, 2), (2, 2), (0, 0, 0, 0))]
 
 
 @pytest.mark.parametrize("idims,k,s,p", POOLS)
@@ -303,17 +304,19 @@ def test_transpose_golden(rt, golden):
         assert_bit_exact(got, golden[f"avg_{tag}_y"], "avgpool golden " + tag)
 
 
-def test_bn_relu_maxpool_fused_equals_sequence(rt, oracle):
+@pytest.mark.parametrize("idims,k", [((2, 16, 16, 64), (2, 2)), ((1, 9, 12, 8), (3, 3)), ((2, 7, 9, 12), (2, 2)),
+                                     ((1, 6, 6, 5), (2, 2))])
+def test_bn_relu_maxpool_fused_equals_sequence(rt, oracle, idims, k):
     rng = np.random.default_rng(77)
-    x = rng.standard_normal((2, 16, 16, 64)).astype(np.float32)
-    c = 64
+    x = rng.standard_normal(idims).astype(np.float32)
+    c = idims[3]
     mean, beta = (rng.standard_normal(c) * 0.1).astype(np.float32), (rng.standard_normal(c) * 0.1).astype(np.float32)
     var, gamma = rng.uniform(0.5, 2, c).astype(np.float32), rng.uniform(0.5, 1.5, c).astype(np.float32)
     dx, dm, dv, dg, db = up(rt, x, mean, var, gamma, beta)
-    seq = rt.maxpool(rt.batchnormalization(dx, dm, dv, dg, db, 1e-5, relu=True), (2, 2), (2, 2)).numpy()
-    fused = rt.batchnormReluMaxpool(dx, dm, dv, dg, db, 1e-5, (2, 2), (2, 2)).numpy()
+    seq = rt.maxpool(rt.batchnormalization(dx, dm, dv, dg, db, 1e-5, relu=True), k, k).numpy()
+    fused = rt.batchnormReluMaxpool(dx, dm, dv, dg, db, 1e-5, k, k).numpy()
     assert_bit_exact(fused, seq, "bn+relu+pool fused vs sequence")
-    want = oracle.maxpool(oracle.relu(oracle.batchnormalization(x, mean, var, gamma, beta, 1e-5)), (2, 2), (2, 2))
+    want = oracle.maxpool(oracle.relu(oracle.batchnormalization(x, mean, var, gamma, beta, 1e-5)), k, k)
     assert rel_err(fused, want) < TOL
 
 
