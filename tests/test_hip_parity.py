@@ -491,9 +491,9 @@ def test_conv_every_variant(rt, oracle, variant, monkeypatch):
         assert_bit_exact(got, want, f"integer conv {idims} variant {variant}")
 
 
-# Leftover output tiles (those beyond the last full round over the chip's workgroup slots) are cut along K and
+# Leftover output tiles (those beyond one full round over the chip's workgroup slots) are cut along K and
 # their partial sums added by a second kernel.  SWC_HIP_CONV_SLOTS makes a small chip of the real one so that
-# small shapes have full rounds and leftovers.
+# small shapes have a full round and leftovers.
 SHARED_CONV_CASES = [((2, 20, 20, 32), (70, 3, 3, 32), (1, 1), (1, 1, 1, 1)),     # oC % 4 != 0: scalar stores
                      ((3, 17, 23, 32), (136, 3, 3, 32), (1, 1), (1, 1, 1, 1)),    # ragged rows and columns
                      ((1, 50, 50, 16), (64, 5, 5, 16), (2, 2), (2, 2, 2, 2))]
@@ -521,7 +521,7 @@ def test_conv_tiles_shared_along_k(rt, oracle, variant, monkeypatch):
         whole = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, bn=bn, eps=1e-5, relu=True).numpy()
         monkeypatch.setenv("SWC_HIP_CONV_SHARE", "1")
         shared = 0
-        for slots in (3, 4, 5, 6, 7):
+        for slots in (3, 4, 5, 6, 7, 9, 11, 13, 17, 19, 23, 29, 37, 47):
             monkeypatch.setenv("SWC_HIP_CONV_SLOTS", str(slots))
             shared += rt.conv2d_workspace_bytes(idims, fdims, strides, pads) > 0
             plain = rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy()
@@ -547,7 +547,7 @@ def test_conv_tiles_shared_along_k(rt, oracle, variant, monkeypatch):
 def test_conv_shared_tiles_in_a_caller_workspace(rt, oracle, monkeypatch):
     from swcompiler_amd.hip import SwcHipError
     idims, fdims, strides, pads = SHARED_CONV_CASES[0]
-    monkeypatch.setenv("SWC_HIP_CONV_SLOTS", "4")
+    monkeypatch.setenv("SWC_HIP_CONV_SLOTS", "19")
     need = rt.conv2d_workspace_bytes(idims, fdims, strides, pads)
     assert need > 0
     rng = np.random.default_rng(32)
