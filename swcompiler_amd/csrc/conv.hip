@@ -285,7 +285,7 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
             f_base[j] = n < N ? n * K * 4 : kOutOfRange;
         }
         // k position of this lane's chunk, as (ky, kx, ci), stepped by BK per slice
-        int kpos = kt_begin * BK + kc_chunk(lane) * 4;
+        int kpos = kt_begin * BK + kc_chunk(lane, wave) * 4;
         int ky, kx, ci;
         {
             const int tap = kpos / g.C;

@@ -155,7 +155,7 @@ __global__ __launch_bounds__(kThreads) void gemm_dma(const float *__restrict__ A
     const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(B, b_bytes);
 
     // byte offsets of this lane's 16 bytes in slice 0, per load
-    const int a_k = kc_chunk(lane) * 4;           // k of the lane's chunk inside a slice
+    const int a_k = kc_chunk(lane, wave) * 4;           // k of the lane's chunk inside a slice
     int a_base[T::kALoads], b_base[T::kBLoads], b_k[T::kBLoads];
 #pragma unroll
     for (int j = 0; j < T::kALoads; ++j) {

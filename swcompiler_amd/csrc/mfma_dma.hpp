@@ -17,8 +17,10 @@
 // LDS layout of one stage (no padding is possible: the hardware places lanes
 // contiguously), conflict-free by XOR swizzles chosen on the GLOBAL-address side:
 //   k-contiguous operand (A; B given as [n][k]): row r = 32 floats = 8 chunks of
-//     16 B; logical chunk q is stored at position q ^ (r & 7).  A fragment read
-//     (32 consecutive rows, same q) then touches 8 distinct positions per 8 rows.
+//     16 B; logical chunk q is stored at position q ^ ((r >> 1) & 7).  A 128-bit fragment read is served
+//     sixteen lanes at a time (16 x 16 B = all 64 banks once): the sixteen consecutive rows of such a group,
+//     same q, then touch 8 distinct positions in their even rows (the lower 32 banks) and 8 in their odd rows
+//     (the upper 32).  (A key of r & 7 repeats after 8 rows: two-way conflicts on every read.)
 //   n-contiguous B ([k][n]): row k = BN floats; column c of a row with
 //     (k >> 2) & 1 == 1 is stored at c ^ 32, so the two half-waves of a fragment
 //     read (rows 4 apart) use opposite halves of the banks.
@@ -75,16 +77,17 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 
 // Position of a lane inside one 1-KiB load of a k-contiguous tile: the load
 // covers 8 rows; lane l writes row (l >> 3), chunk position (l & 7), which holds
-// logical chunk (l & 7) ^ (l >> 3).
+// logical chunk (l & 7) ^ key of its row, key = (row >> 1) & 7.
 __device__ __forceinline__ int kc_row_in_load(int lane) { return lane >> 3; }
-__device__ __forceinline__ int kc_chunk(int lane) { return (lane & 7) ^ (lane >> 3); }
+// `block` = which 8-row block of the tile the load fills (its parity is all that matters)
+__device__ __forceinline__ int kc_chunk(int lane, int block) { return (lane & 7) ^ (((block & 1) << 2) | (lane >> 4)); }
 
 template <int TM, int TN, bool B_NT>
 __device__ __forceinline__ void load_frag_swz(Frag<TM, TN> &f, const float *__restrict__ As,
                                               const float *__restrict__ Bs, int g, int wave_m, int wave_n, int l32,
                                               int h) {
     constexpr int BN = 64 * TN;
-    const int swz = l32 & 7;
+    const int swz = (l32 >> 1) & 7;
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
         const int row = wave_m * 32 * TM + tm * 32 + l32;

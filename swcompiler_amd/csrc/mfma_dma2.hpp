@@ -54,7 +54,7 @@ __device__ __forceinline__ void load_frag2_piece(Frag2<TM, TN> &f, const float *
                                                  int l32, int h) {
     if (piece < TM) {
         const int row = row0 + piece * 32 + l32;
-        const float4 v = *reinterpret_cast<const float4 *>(&As[row * BK + (((2 * g + h) ^ (l32 & 7)) << 2)]);
+        const float4 v = *reinterpret_cast<const float4 *>(&As[row * BK + (((2 * g + h) ^ ((l32 >> 1) & 7)) << 2)]);
         f.a[piece][0] = v.x; f.a[piece][1] = v.y; f.a[piece][2] = v.z; f.a[piece][3] = v.w;
     } else {
         const int s = piece - TM;
@@ -181,13 +181,14 @@ __device__ __forceinline__ void dma2_tile_body(const float *__restrict__ A, unsi
     // Per-lane byte offsets of slice 0 (out-of-range for rows/columns outside the
     // matrix); a slice adds a scalar: k0*4 bytes for A, k0*ldb*4 for B.  Only a
     // slice that reaches past K needs the per-lane k check.
-    const int a_k = kc_chunk(lane) * 4;
+    int a_k[T::kALoads];   // k of the lane's chunk inside a slice, per load (the swizzle key depends on the row block)
     int a_base[T::kALoads];
     typename BSrc::Lane bl[T::kBLoads];
 #pragma unroll
     for (int j = 0; j < T::kALoads; ++j) {
         const int row = m0 + (wave * T::kALoads + j) * 8 + kc_row_in_load(lane);
-        a_base[j] = row < M ? (row * lda + a_k) * 4 + kImmSpan - (j & 3) * 1024 : kOutOfRange;
+        a_k[j] = kc_chunk(lane, wave * T::kALoads + j) * 4;
+        a_base[j] = row < M ? (row * lda + a_k[j]) * 4 + kImmSpan - (j & 3) * 1024 : kOutOfRange;
     }
 #pragma unroll
     for (int j = 0; j < T::kBLoads; ++j) {
@@ -199,7 +200,7 @@ __device__ __forceinline__ void dma2_tile_body(const float *__restrict__ A, unsi
     auto issue = [&](float *__restrict__ wr, int j) {
         const bool whole = k0 + BK <= k_end;   // scalar
         if (j < T::kALoads) {
-            const int v = whole ? a_base[j] : ((a_base[j] != kOutOfRange && k0 + a_k < k_end) ? a_base[j] : kOutOfRange);
+            const int v = whole ? a_base[j] : ((a_base[j] != kOutOfRange && k0 + a_k[j] < k_end) ? a_base[j] : kOutOfRange);
             lds_void_t *dst = (lds_void_t *)(wr + (wave * T::kALoads + (j & ~3)) * 256);
             switch (j & 3) {   // the immediate must be a compile-time constant
             case 0: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, dst, 16, v, k0 * 4, 0, 0); break;
