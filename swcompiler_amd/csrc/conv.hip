@@ -1056,33 +1056,54 @@ __global__ __launch_bounds__(256) void wgrad_direct(float *__restrict__ fg, cons
 }
 
 // ---- bias gradient: masked column sums of outputG [M, OC]
-constexpr int kBiasRows = 128;   // rows per partial sum
-// A workgroup sums kBiasRows rows: thread = (column, row phase); the 256/cols... phases of a column are combined in
-// a fixed order.  cols = min(OC, 256) columns per workgroup in x, row chunks in y.
+constexpr int kBiasRows = 256;   // rows per partial sum (enough workgroups to fill the chip at the sizes of interest)
+// A workgroup sums kBiasRows rows: thread = (VEC columns, row phase), the pixel coordinates of its rows kept
+// incrementally (no division in the loop); the 256/colsq phases of a column are combined in a fixed order.
+// colsq * VEC columns per workgroup in x (colsq a power of two), row chunks in y.
+template <int VEC>
 __global__ __launch_bounds__(256) void bias_partials(float *__restrict__ part, const float *__restrict__ og, ConvGeom g,
-                                                     int cols, int phases) {
-    __shared__ float red[256];
-    const int c_local = threadIdx.x % cols, phase = threadIdx.x / cols;
-    const int co = blockIdx.x * cols + c_local;
+                                                     int colsq, int phases) {
+    __shared__ float red[256 * VEC];
+    const int c_local = threadIdx.x % colsq, phase = threadIdx.x / colsq;
+    const int co = (blockIdx.x * colsq + c_local) * VEC;
     const int m0 = blockIdx.y * kBiasRows;
     const int m1 = m0 + kBiasRows < g.M ? m0 + kBiasRows : g.M;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};   // four independent chains keep four loads in flight
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
     if (co < g.OC && phase < phases) {
-        int u = 0;
-        for (int m = m0 + phase; m < m1; m += phases, u = (u + 1) & 3) {
-            const int ox = m % g.OW, oy = (m / g.OW) % g.OH;
-            const int iy = oy * g.sh - g.pt, ix = ox * g.sw - g.pl;
-            const float v = og[(size_t)m * g.OC + co];
-            if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W) acc[u] += v;
+        int m = m0 + phase;
+        int ox = m % g.OW, oy = (m / g.OW) % g.OH;
+        const int step_y = phases / g.OW, step_x = phases - step_y * g.OW;   // phases rows further on
+#pragma unroll 4
+        for (; m < m1; m += phases) {
+            // the reference adds outputG at tap (0,0) after that tap's bounds test: pixels whose first tap lies
+            // in the padding do not contribute
+            const bool counts = (unsigned)(oy * g.sh - g.pt) < (unsigned)g.H && (unsigned)(ox * g.sw - g.pl) < (unsigned)g.W;
+            const float *p = og + (size_t)m * g.OC + co;
+            if (VEC == 4) {
+                const float4 q = *reinterpret_cast<const float4 *>(p);
+                if (counts) acc[0] += q.x, acc[VEC > 1 ? 1 : 0] += q.y, acc[VEC > 2 ? 2 : 0] += q.z, acc[VEC > 3 ? 3 : 0] += q.w;
+            } else {
+                const float q = *p;
+                if (counts) acc[0] += q;
+            }
+            ox += step_x;
+            oy += step_y;
+            if (ox >= g.OW) ox -= g.OW, ++oy;
+            while (oy >= g.OH) oy -= g.OH;
         }
     }
-    const float sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
-    red[threadIdx.x] = sum;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) red[threadIdx.x * VEC + v] = acc[v];
     __syncthreads();
     if (phase == 0 && co < g.OC) {
-        float t = red[c_local];
-        for (int q = 1; q < phases; ++q) t += red[q * cols + c_local];
-        part[(size_t)blockIdx.y * g.OC + co] = t;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+            float t = red[c_local * VEC + v];
+            for (int q = 1; q < phases; ++q) t += red[(q * colsq + c_local) * VEC + v];
+            if (co + v < g.OC) part[(size_t)blockIdx.y * g.OC + co + v] = t;
+        }
     }
 }
 
@@ -1163,10 +1184,13 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
 
     // ---- bias gradient
     {
-        int cols = 1;
-        while (cols < g.OC && cols < 256) cols <<= 1;   // power of two, so that 256 % cols == 0
-        bias_partials<<<dim3((g.OC + cols - 1) / cols, bias_chunks), 256, 0, stream()>>>(bias_part, outputG, g, cols,
-                                                                                          256 / cols);
+        const bool vec4 = g.OC % 4 == 0 && aligned16(outputG);
+        const int quads = vec4 ? g.OC / 4 : g.OC;
+        int colsq = 1;
+        while (colsq < quads && colsq < 256) colsq <<= 1;   // power of two, so that 256 % colsq == 0
+        const dim3 grid((quads + colsq - 1) / colsq, bias_chunks);
+        if (vec4) bias_partials<4><<<grid, 256, 0, stream()>>>(bias_part, outputG, g, colsq, 256 / colsq);
+        else bias_partials<1><<<grid, 256, 0, stream()>>>(bias_part, outputG, g, colsq, 256 / colsq);
     }
     SWC_LAUNCH_CHECK();
     sum_splits<<<ceil_div(g.OC, 32), 256, 0, stream()>>>(biasG, bias_part, (size_t)g.OC, bias_chunks);
