@@ -877,18 +877,29 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
 // inputG and filterG are sums of the same fp32 products as the reference's, in
 // a different order.
 
-// turned[ci][ky][kx][co] = filter[co][kh-1-ky][kw-1-kx][ci]
+// turned[ci][ky][kx][co] = filter[co][kh-1-ky][kw-1-kx][ci]; rows of OCP >= OC floats, the tail zero
 __global__ __launch_bounds__(256) void turn_filter(const float *__restrict__ filt, float *__restrict__ turned, int OC,
-                                                   int kh, int kw, int C) {
-    const int total = OC * kh * kw * C;
+                                                   int OCP, int kh, int kw, int C) {
+    const int total = OCP * kh * kw * C;
     for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
-        const int co = i % OC;
-        int t = i / OC;
+        const int co = i % OCP;
+        int t = i / OCP;
         const int kx = t % kw;
         t /= kw;
         const int ky = t % kh;
         const int ci = t / kh;
-        turned[i] = filt[((co * kh + (kh - 1 - ky)) * kw + (kw - 1 - kx)) * C + ci];
+        turned[i] = co < OC ? filt[((co * kh + (kh - 1 - ky)) * kw + (kw - 1 - kx)) * C + ci] : 0.f;
+    }
+}
+
+// dst[m][0..OCP) = src[m][0..OC), zeros behind: rows of a channel count the 128-bit gathers can take
+__global__ __launch_bounds__(256) void pad_channels(float *__restrict__ dst, const float *__restrict__ src, size_t rows,
+                                                    int OC, int OCP) {
+    const size_t total = rows * OCP;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const size_t m = i / OCP;
+        const int co = (int)(i - m * OCP);
+        dst[i] = co < OC ? src[m * OC + co] : 0.f;
     }
 }
 
@@ -916,6 +927,64 @@ __global__ __launch_bounds__(256) void dgrad_direct(float *__restrict__ ig, cons
             }
         }
         ig[i] = sum;
+    }
+}
+
+// Up to four input channels (first layers), any stride: one thread per input pixel gathers the taps that reach
+// it for all its channels.  The filter sits in LDS as [ky][kx][ci][co] (rows of OCP floats, a multiple of 4), read
+// as wavefront-uniform 128-bit broadcasts; outputG is read four output channels at a time where it can be.
+template <int CI, bool VEC>
+__global__ __launch_bounds__(256) void dgrad_few_channels(float *__restrict__ ig, const float *__restrict__ og,
+                                                          const float *__restrict__ filt, ConvGeom g, int OCP) {
+    extern __shared__ __align__(16) float f_s[];   // [kh][kw][CI][OCP]
+    const int taps = g.kh * g.kw;
+    for (int i = threadIdx.x; i < taps * CI * OCP; i += 256) {
+        const int co = i % OCP;
+        int t = i / OCP;
+        const int ci = t % CI;
+        t /= CI;   // ky*kw + kx
+        f_s[i] = co < g.OC ? filt[((size_t)co * taps + t) * CI + ci] : 0.f;
+    }
+    __syncthreads();
+    const size_t pixels = (size_t)g.N * g.H * g.W;
+    for (size_t p = (size_t)blockIdx.x * 256 + threadIdx.x; p < pixels; p += (size_t)gridDim.x * 256) {
+        const int ix = (int)(p % g.W);
+        const size_t t = p / g.W;
+        const int iy = (int)(t % g.H), n = (int)(t / g.H);
+        float sum[CI];
+#pragma unroll
+        for (int c = 0; c < CI; ++c) sum[c] = 0.f;
+        for (int ky = 0; ky < g.kh; ++ky) {
+            const int ny = iy + g.pt - ky;
+            if (ny < 0 || ny % g.sh != 0 || ny / g.sh >= g.OH) continue;
+            for (int kx = 0; kx < g.kw; ++kx) {
+                const int nx = ix + g.pl - kx;
+                if (nx < 0 || nx % g.sw != 0 || nx / g.sw >= g.OW) continue;
+                const float *o = og + (((size_t)n * g.OH + ny / g.sh) * g.OW + nx / g.sw) * g.OC;
+                const float *f = f_s + (ky * g.kw + kx) * CI * OCP;
+                if (VEC) {   // OC % 4 == 0, outputG 16-byte aligned
+                    for (int co = 0; co < g.OC; co += 4) {
+                        const float4 ov = *reinterpret_cast<const float4 *>(o + co);
+#pragma unroll
+                        for (int c = 0; c < CI; ++c) {
+                            const float4 fv = *reinterpret_cast<const float4 *>(f + c * OCP + co);
+                            sum[c] += fv.x * ov.x;
+                            sum[c] += fv.y * ov.y;
+                            sum[c] += fv.z * ov.z;
+                            sum[c] += fv.w * ov.w;
+                        }
+                    }
+                } else {
+                    for (int co = 0; co < g.OC; ++co) {
+                        const float ov = o[co];
+#pragma unroll
+                        for (int c = 0; c < CI; ++c) sum[c] += f[c * OCP + co] * ov;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CI; ++c) ig[p * CI + c] = sum[c];
     }
 }
 
@@ -1002,27 +1071,46 @@ int launch_wgrad(const float *ogT, size_t a_bytes, int lda, const Im2colB &bsrc,
     return SWC_HIP_OK;
 }
 
-// out[i] = sum over splits of part[split][i], in a fixed order: eight threads share an element, thread p adds
-// splits p, p+8, p+16, ... (eight independent chains instead of one long one), then the eight are added in order.
-__global__ __launch_bounds__(256) void sum_splits(float *__restrict__ out, const float *__restrict__ part, size_t n,
-                                                  int splits) {
-    __shared__ float red[8][33];
+// out[i] = sum over splits of part[split][i], in a fixed order: PH threads share an element, thread p adds
+// splits p, p+PH, p+2PH, ... four loads at a time (PH independent chains instead of one long one), then the PH
+// partial sums are added in order.  PH = 8 for a few splits of many elements, 32 for hundreds of splits.
+template <int PH>
+__global__ __launch_bounds__(32 * PH) void sum_splits(float *__restrict__ out, const float *__restrict__ part, size_t n,
+                                                      int splits) {
+    __shared__ float red[PH][33];
     const int e = threadIdx.x & 31, p = threadIdx.x >> 5;
     for (size_t base = (size_t)blockIdx.x * 32; base < n; base += (size_t)gridDim.x * 32) {
         const size_t i = base + e;
         float s = 0.f;
-        if (i < n)
-            for (int k = p; k < splits; k += 8) s += part[(size_t)k * n + i];
+        if (i < n) {
+            int k = p;
+            for (; k + 3 * PH < splits; k += 4 * PH) {
+                const float v0 = part[(size_t)k * n + i], v1 = part[(size_t)(k + PH) * n + i];
+                const float v2 = part[(size_t)(k + 2 * PH) * n + i], v3 = part[(size_t)(k + 3 * PH) * n + i];
+                s += v0, s += v1, s += v2, s += v3;
+            }
+            for (; k < splits; k += PH) s += part[(size_t)k * n + i];
+        }
         red[p][e] = s;
         __syncthreads();
         if (p == 0 && i < n) {
             float t = red[0][e];
 #pragma unroll
-            for (int q = 1; q < 8; ++q) t += red[q][e];
+            for (int q = 1; q < PH; ++q) t += red[q][e];
             out[i] = t;
         }
         __syncthreads();
     }
+}
+
+// launches sum_splits with the number of chains that suits `splits`
+int launch_sum_splits(float *out, const float *part, size_t n, int splits) {
+    unsigned blocks = ceil_div(n, 32);
+    blocks = blocks > 16384 ? 16384 : blocks;
+    if (splits >= 128) sum_splits<32><<<blocks, 1024, 0, stream()>>>(out, part, n, splits);
+    else sum_splits<8><<<blocks, 256, 0, stream()>>>(out, part, n, splits);
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
 }
 
 // any shape: one workgroup per filter element, pixels strided over its threads
@@ -1053,6 +1141,54 @@ __global__ __launch_bounds__(256) void wgrad_direct(float *__restrict__ fg, cons
         __syncthreads();
     }
     if (threadIdx.x == 0) fg[e] = red[0];
+}
+
+// Small filters that the MFMA path cannot take (first layers: iC = 1 or 3): one thread per filter element
+// (co, ky, kx, ci), a workgroup per block of `rows` output rows of one image.  The block's outputG rows and
+// the input rows under them are staged in LDS, where the many threads that need the same value read it as a
+// broadcast; partial sums per block go to `part`, sum_splits adds them.  blockIdx.x = image, blockIdx.y = row block.
+__global__ __launch_bounds__(1024) void wgrad_small(float *__restrict__ part, const float *__restrict__ og,
+                                                    const float *__restrict__ in, ConvGeom g, int rows) {
+    extern __shared__ float wg_lds[];
+    const int n = blockIdx.x, oy0 = blockIdx.y * rows;
+    const int oy1 = oy0 + rows < g.OH ? oy0 + rows : g.OH;
+    const int iy_first = oy0 * g.sh - g.pt;                           // input row under tap row 0 of the first output row
+    const int in_rows = (oy1 - 1 - oy0) * g.sh + g.kh;
+    float *og_s = wg_lds;                                             // [oy1-oy0][OW][OC]
+    float *in_s = wg_lds + (size_t)rows * g.OW * g.OC;                // [in_rows][W][C], rows outside the image zero
+    const int og_count = (oy1 - oy0) * g.OW * g.OC, row_len = g.W * g.C;
+    const float *og_src = og + ((size_t)n * g.OH + oy0) * g.OW * g.OC;
+    for (int i = threadIdx.x; i < og_count; i += blockDim.x) og_s[i] = og_src[i];
+    for (int i = threadIdx.x; i < in_rows * row_len; i += blockDim.x) {
+        const int r = i / row_len, iy = iy_first + r;
+        in_s[i] = (unsigned)iy < (unsigned)g.H ? in[((size_t)n * g.H + iy) * row_len + (i - r * row_len)] : 0.f;
+    }
+    __syncthreads();
+    const int e = threadIdx.x;
+    const int elems = g.OC * g.K;
+    if (e >= elems) return;
+    const int ci = e % g.C;
+    int t = e / g.C;
+    const int kx = t % g.kw;
+    t /= g.kw;
+    const int ky = t % g.kh;
+    const int co = t / g.kh;
+    // output columns whose tap kx lies inside the image
+    int ox_lo = 0, ox_hi = g.OW;
+    while (ox_lo < ox_hi && ox_lo * g.sw - g.pl + kx < 0) ++ox_lo;
+    while (ox_hi > ox_lo && (ox_hi - 1) * g.sw - g.pl + kx >= g.W) --ox_hi;
+    float acc[2] = {0.f, 0.f};
+    for (int oy = oy0; oy < oy1; ++oy) {
+        const float *o = og_s + ((oy - oy0) * g.OW) * g.OC + co;
+        const float *x = in_s + ((oy - oy0) * g.sh + ky) * row_len + (kx - g.pl) * g.C + ci;   // rows outside hold zeros
+        int ox = ox_lo;
+        for (; ox + 1 < ox_hi; ox += 2) {
+            acc[0] += x[ox * g.sw * g.C] * o[ox * g.OC];
+            acc[1] += x[(ox + 1) * g.sw * g.C] * o[(ox + 1) * g.OC];
+        }
+        if (ox < ox_hi) acc[0] += x[ox * g.sw * g.C] * o[ox * g.OC];
+    }
+    part[((size_t)n * gridDim.y + blockIdx.y) * elems + e] = acc[0] + acc[1];
 }
 
 // ---- bias gradient: masked column sums of outputG [M, OC]
@@ -1109,6 +1245,10 @@ __global__ __launch_bounds__(256) void bias_partials(float *__restrict__ part, c
 
 size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
 
+size_t wgrad_small_lds(const ConvGeom &g, int rows) {
+    return ((size_t)rows * g.OW * g.OC + ((size_t)(rows - 1) * g.sh + g.kh) * g.W * g.C) * sizeof(float);
+}
+
 int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG, const float *input,
               const float *filter, const size_t *odims, const size_t *idims, const size_t *fdims,
               const size_t *kernels, const size_t *strides, const size_t *pads, size_t group) {
@@ -1162,25 +1302,40 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
     splits = (nk + sps - 1) / sps;
     // the input gradient as a convolution of outputG with the turned filter
     const size_t t_odims[4] = {idims[0], idims[1], idims[2], idims[3]};
-    const size_t t_idims[4] = {odims[0], odims[1], odims[2], odims[3]};
-    const size_t t_fdims[4] = {idims[3], kernels[0], kernels[1], odims[3]};
+    // (its channel count is OC: padded to a multiple of 4 with zeros where needed, so that the 128-bit gathers
+    // of the MFMA kernels apply — 50 channels: 230 us on the scalar path, 30 with two small copies)
+    const size_t ocp = (odims[3] + 3) & ~(size_t)3;
+    const size_t t_idims[4] = {odims[0], odims[1], odims[2], ocp};
+    const size_t t_fdims[4] = {idims[3], kernels[0], kernels[1], ocp};
     const size_t t_strides[2] = {1, 1};
     const size_t t_pads[4] = {(size_t)(g.kh - 1 - g.pt), (size_t)(g.kw - 1 - g.pl), 0, 0};
-    const size_t turned_b = dgrad_conv ? align256(f_elems * 4) : 0;
+    const size_t turned_b = dgrad_conv ? align256(idims[3] * fdims[1] * fdims[2] * ocp * 4) : 0;
+    const size_t ogp_b = dgrad_conv && ocp != odims[3] ? align256(M * ocp * 4) : 0;   // outputG with padded channels
     // (the turned filter lies at the start of the workspace, which is 256-byte aligned like outputG must be)
     const size_t dgrad_b =
         dgrad_conv ? align256(conv_scratch_bytes(make_geom(t_odims, t_idims, t_fdims, kernels, t_strides, t_pads), outputG,
                                                  nullptr)) : 0;
     const size_t ogt_b = wgrad_mfma ? align256((size_t)g.OC * lda * 4) : 0;
-    const size_t part_b = wgrad_mfma && splits > 1 ? align256((size_t)splits * f_elems * 4) : 0;
+    // small filters off the MFMA path: row blocks of about three workgroups per CU, as LDS allows
+    int wgrad_rows = 0;
+    if (!wgrad_mfma && f_elems <= 1024 && g.OH > 0 && g.N <= 65535) {
+        int rows = (int)((size_t)g.N * g.OH / (3 * (size_t)num_cus()));
+        rows = rows < 1 ? 1 : (rows > g.OH ? g.OH : rows);
+        while (rows > 1 && wgrad_small_lds(g, rows) > 64 * 1024) --rows;
+        if (wgrad_small_lds(g, rows) <= 64 * 1024 && (g.OH + rows - 1) / rows <= 65535) wgrad_rows = rows;
+    }
+    const size_t wgrad_blocks = wgrad_rows ? (size_t)g.N * ((g.OH + wgrad_rows - 1) / wgrad_rows) : 0;
+    const size_t part_b = wgrad_mfma && splits > 1 ? align256((size_t)splits * f_elems * 4)
+                                                   : align256(wgrad_blocks * f_elems * 4);
     const size_t bias_b = align256((size_t)bias_chunks * g.OC * 4);
-    char *ws = static_cast<char *>(workspace(turned_b + ogt_b + part_b + bias_b + dgrad_b, who));
+    char *ws = static_cast<char *>(workspace(turned_b + ogt_b + part_b + bias_b + dgrad_b + ogp_b, who));
     if (!ws) return SWC_HIP_ERUNTIME;
     float *turned = reinterpret_cast<float *>(ws);
     float *ogT = reinterpret_cast<float *>(ws + turned_b);
     float *part = reinterpret_cast<float *>(ws + turned_b + ogt_b);
     float *bias_part = reinterpret_cast<float *>(ws + turned_b + ogt_b + part_b);
     float *dgrad_pieces = reinterpret_cast<float *>(ws + turned_b + ogt_b + part_b + bias_b);
+    float *og_padded = reinterpret_cast<float *>(ws + turned_b + ogt_b + part_b + bias_b + dgrad_b);
 
     // ---- bias gradient
     {
@@ -1193,19 +1348,41 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
         else bias_partials<1><<<grid, 256, 0, stream()>>>(bias_part, outputG, g, colsq, 256 / colsq);
     }
     SWC_LAUNCH_CHECK();
-    sum_splits<<<ceil_div(g.OC, 32), 256, 0, stream()>>>(biasG, bias_part, (size_t)g.OC, bias_chunks);
-    SWC_LAUNCH_CHECK();
+    if (int rc = launch_sum_splits(biasG, bias_part, (size_t)g.OC, bias_chunks)) return rc;
 
     // ---- input gradient
     if (dgrad_conv) {
-        unsigned blocks = ceil_div(f_elems, 256);
-        turn_filter<<<blocks > 1024 ? 1024 : blocks, 256, 0, stream()>>>(filter, turned, g.OC, g.kh, g.kw, g.C);
+        unsigned blocks = ceil_div(idims[3] * fdims[1] * fdims[2] * ocp, 256);
+        turn_filter<<<blocks > 1024 ? 1024 : blocks, 256, 0, stream()>>>(filter, turned, g.OC, (int)ocp, g.kh, g.kw, g.C);
         SWC_LAUNCH_CHECK();
+        const float *og_in = outputG;
+        if (ogp_b) {
+            blocks = ceil_div(M * ocp, 256);
+            pad_channels<<<blocks > 16384 ? 16384 : blocks, 256, 0, stream()>>>(og_padded, outputG, M, g.OC, (int)ocp);
+            SWC_LAUNCH_CHECK();
+            og_in = og_padded;
+        }
         const Epilogue ep{nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
         // its shared-tile pieces go into this call's own region: the library workspace is in use here
-        const int rc = conv_dispatch(who, inputG, outputG, turned, nullptr, t_odims, t_idims, t_fdims, kernels, t_strides,
+        const int rc = conv_dispatch(who, inputG, og_in, turned, nullptr, t_odims, t_idims, t_fdims, kernels, t_strides,
                                      t_pads, 1, ep, /*bias_optional=*/true, ConvScratch{dgrad_pieces, dgrad_b});
         if (rc != SWC_HIP_OK) return rc;
+    } else if (g.C <= 4 && (size_t)g.kh * g.kw * g.C * ocp * 4 <= 48 * 1024) {
+        unsigned blocks = ceil_div(in_elems / g.C, 256);
+        blocks = blocks > 65536 ? 65536 : blocks;
+        const size_t lds = (size_t)g.kh * g.kw * g.C * ocp * 4;
+        const bool vec = g.OC % 4 == 0 && aligned16(outputG);
+        auto launch = [&]<int CI>() {
+            if (vec) dgrad_few_channels<CI, true><<<blocks, 256, lds, stream()>>>(inputG, outputG, filter, g, (int)ocp);
+            else dgrad_few_channels<CI, false><<<blocks, 256, lds, stream()>>>(inputG, outputG, filter, g, (int)ocp);
+        };
+        switch (g.C) {
+        case 1: launch.template operator()<1>(); break;
+        case 2: launch.template operator()<2>(); break;
+        case 3: launch.template operator()<3>(); break;
+        default: launch.template operator()<4>(); break;
+        }
+        SWC_LAUNCH_CHECK();
     } else {
         unsigned blocks = ceil_div(in_elems, 256);
         dgrad_direct<<<blocks > 65536 ? 65536 : blocks, 256, 0, stream()>>>(inputG, outputG, filter, g);
@@ -1229,10 +1406,14 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
                                : launch_wgrad<1, 4, 4, 2, false, 4>(ogT, a_bytes, lda, bsrc, dst, g.OC, (int)Kf, (int)M, splits, sps);
         if (rc2 != SWC_HIP_OK) return rc2;
         if (splits > 1) {
-            unsigned blocks = ceil_div(f_elems, 32);
-            sum_splits<<<blocks > 16384 ? 16384 : blocks, 256, 0, stream()>>>(filterG, part, f_elems, splits);
-            SWC_LAUNCH_CHECK();
+            if (int rc3 = launch_sum_splits(filterG, part, f_elems, splits)) return rc3;
         }
+    } else if (wgrad_rows) {
+        const dim3 grid((unsigned)g.N, (unsigned)((g.OH + wgrad_rows - 1) / wgrad_rows));
+        wgrad_small<<<grid, (unsigned)((f_elems + 63) / 64 * 64), wgrad_small_lds(g, wgrad_rows), stream()>>>(
+            part, outputG, input, g, wgrad_rows);
+        SWC_LAUNCH_CHECK();
+        if (int rc3 = launch_sum_splits(filterG, part, f_elems, (int)(grid.x * grid.y))) return rc3;
     } else {
         wgrad_direct<<<(unsigned)f_elems, 256, 0, stream()>>>(filterG, outputG, input, g);
         SWC_LAUNCH_CHECK();
