@@ -74,7 +74,9 @@ size_t swc_hip_gemm_workspace_bytes(int m, int n, int k);
 /* The same for a conv2d_f / conv2dFused_f call of these shapes (arguments as in
  * swc_hip_conv2d_f, tensors assumed 16-byte aligned): the output tiles that are
  * left over after every CU has had its share of whole tiles are cut along K and
- * their partial sums kept here.  Without a workspace large enough the library
+ * their partial sums kept here; a layer whose input-channel count is no multiple
+ * of 4 (and that is too large for the direct first-layer kernel) is computed on
+ * zero-padded copies of input and filter, which live here too.  Without a workspace large enough the library
  * allocates its own at the first such call. */
 size_t swc_hip_conv2d_workspace_bytes(const size_t *odims, const size_t *idims, const size_t *fdims,
                                       const size_t *kernels, const size_t *strides, const size_t *pads);

@@ -764,6 +764,17 @@ bool conv_uses_dma(const ConvGeom &g, const void *input, const void *filter, con
     return true;
 }
 
+// dst[m][0..OCP) = src[m][0..OC), zeros behind: rows of a channel count the 128-bit gathers can take
+__global__ __launch_bounds__(256) void pad_channels(float *__restrict__ dst, const float *__restrict__ src, size_t rows,
+                                                    int OC, int OCP) {
+    const size_t total = rows * OCP;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const size_t m = i / OCP;
+        const int co = (int)(i - m * OCP);
+        dst[i] = co < OC ? src[m * OC + co] : 0.f;
+    }
+}
+
 // Scratch bytes the forward convolution of this geometry uses (0: none).
 size_t conv_scratch_bytes(const ConvGeom &g, const void *input, const void *filter) {
     const char *force = getenv("SWC_HIP_CONV");
@@ -771,6 +782,33 @@ size_t conv_scratch_bytes(const ConvGeom &g, const void *input, const void *filt
     return with_dma_variant(pick_dma_variant(g, force, true), [&]<int TM, int TN, int STAGES, bool MID>() {
         return conv_dma_scratch_bytes<TM, TN, STAGES, MID>(g);
     });
+}
+
+size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+// An input-channel count that is no multiple of 4 keeps a layer off the 128-bit gathers of the MFMA kernels
+// (the register-staged fallback reaches a tenth of their rate).  Such a layer — unless it is one for the direct
+// kernel — is computed on zero-padded copies of input and filter instead: this returns the padded count, or 0.
+int padded_channels(const ConvGeom &g, const char *force) {
+    if (g.C % 4 == 0 || (force && !strncmp(force, "reg", 3))) return 0;
+    if (g.K <= kDirectMaxK && g.OC <= kDirectMaxOC) return 0;   // the direct kernel's
+    const int cp = (g.C + 3) & ~3;
+    const size_t in_bytes = (size_t)g.N * g.H * g.W * cp * 4, filt_bytes = (size_t)g.OC * g.kh * g.kw * cp * 4;
+    return in_bytes < kMaxDmaBytes && filt_bytes < kMaxDmaBytes ? cp : 0;
+}
+
+ConvGeom with_channels(ConvGeom g, int c) {
+    g.C = c;
+    g.K = g.kh * g.kw * c;
+    return g;
+}
+
+// Scratch bytes a forward convolution uses in all: padded copies (if any) and the pieces of shared tiles.
+size_t conv_total_scratch(const ConvGeom &g, const void *input, const void *filter) {
+    const int cp = padded_channels(g, getenv("SWC_HIP_CONV"));
+    if (!cp) return conv_scratch_bytes(g, input, filter);
+    return align256((size_t)g.N * g.H * g.W * cp * 4) + align256((size_t)g.OC * g.kh * g.kw * cp * 4) +
+           conv_scratch_bytes(with_channels(g, cp), nullptr, nullptr);
 }
 
 int check_conv_dims(const char *who, const size_t *odims, const size_t *idims, const size_t *fdims,
@@ -815,7 +853,8 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
     Epilogue ep = ep_in;
     ep.bias = bias;
     const bool vec = (g.C % 4 == 0) && aligned16(input) && aligned16(filter);
-    const size_t in_bytes = idims[0] * idims[1] * idims[2] * idims[3] * 4, filt_bytes = odims[3] * (size_t)g.K * 4;
+    const size_t M_in = idims[0] * idims[1] * idims[2];
+    const size_t in_bytes = M_in * idims[3] * 4, filt_bytes = odims[3] * (size_t)g.K * 4;
     const char *force = getenv("SWC_HIP_CONV");   // forces a kernel variant (tests, tuning): reg22 reg21 reg12 reg11 | 22_2 21_3 12_3 11_3 11_4 | 11_3m 21_3m 12_3m 22_3m (m: ring hand-over in mid-slice)
     if (force) {
         if (!strcmp(force, "reg22")) return launch_conv<2, 2>(vec, input, filter, output, g, ep);
@@ -828,6 +867,29 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
         for (int v = 0; v < kVariants; ++v) forced_dma |= !strcmp(force, kDmaVariantName[v]);
     if (!forced_dma && !(force && !strncmp(force, "reg", 3)) && g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0)
         return launch_conv_direct(input, filter, bias, output, g, ep);
+    if (const int cp = forced_dma || !(force && !strncmp(force, "reg", 3)) ? padded_channels(g, force) : 0) {
+        // zero-padded copies of input and filter, then the same convolution with a channel count of cp
+        const size_t in_b = align256(M_in * cp * 4), f_b = align256((size_t)g.OC * g.kh * g.kw * cp * 4);
+        const ConvGeom gp = with_channels(g, cp);
+        const size_t need = in_b + f_b + conv_scratch_bytes(gp, nullptr, nullptr);
+        char *base = nullptr;
+        if (scratch.ptr && scratch.bytes >= need) base = reinterpret_cast<char *>(scratch.ptr);
+        else if (!scratch.ptr) base = static_cast<char *>(workspace(need, who));
+        if (!base && !scratch.ptr) return SWC_HIP_ERUNTIME;
+        if (base) {
+            float *in_p = reinterpret_cast<float *>(base), *f_p = reinterpret_cast<float *>(base + in_b);
+            unsigned blocks = ceil_div(M_in * cp, 256);
+            pad_channels<<<blocks > 16384 ? 16384 : blocks, 256, 0, stream()>>>(in_p, input, M_in, g.C, cp);
+            SWC_LAUNCH_CHECK();
+            blocks = ceil_div((size_t)g.OC * g.kh * g.kw * cp, 256);
+            pad_channels<<<blocks > 16384 ? 16384 : blocks, 256, 0, stream()>>>(f_p, filter, (size_t)g.OC * g.kh * g.kw, g.C, cp);
+            SWC_LAUNCH_CHECK();
+            const size_t p_idims[4] = {idims[0], idims[1], idims[2], (size_t)cp};
+            const size_t p_fdims[4] = {fdims[0], fdims[1], fdims[2], (size_t)cp};
+            return conv_dispatch(who, output, in_p, f_p, bias, odims, p_idims, p_fdims, kernels, strides, pads, group, ep_in,
+                                 bias_optional, ConvScratch{reinterpret_cast<float *>(base + in_b + f_b), need - in_b - f_b});
+        }
+    }
     if (conv_uses_dma(g, input, filter, force)) {
         // the pieces of shared tiles go into the caller's region when it gave one (and none are made if that
         // is too small), else into the library workspace
@@ -889,17 +951,6 @@ __global__ __launch_bounds__(256) void turn_filter(const float *__restrict__ fil
         const int ky = t % kh;
         const int ci = t / kh;
         turned[i] = co < OC ? filt[((co * kh + (kh - 1 - ky)) * kw + (kw - 1 - kx)) * C + ci] : 0.f;
-    }
-}
-
-// dst[m][0..OCP) = src[m][0..OC), zeros behind: rows of a channel count the 128-bit gathers can take
-__global__ __launch_bounds__(256) void pad_channels(float *__restrict__ dst, const float *__restrict__ src, size_t rows,
-                                                    int OC, int OCP) {
-    const size_t total = rows * OCP;
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
-        const size_t m = i / OCP;
-        const int co = (int)(i - m * OCP);
-        dst[i] = co < OC ? src[m * OC + co] : 0.f;
     }
 }
 
@@ -1243,8 +1294,6 @@ __global__ __launch_bounds__(256) void bias_partials(float *__restrict__ part, c
     }
 }
 
-size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
-
 size_t wgrad_small_lds(const ConvGeom &g, int rows) {
     return ((size_t)rows * g.OW * g.OC + ((size_t)(rows - 1) * g.sh + g.kh) * g.W * g.C) * sizeof(float);
 }
@@ -1456,7 +1505,7 @@ size_t swc_hip_conv2d_workspace_bytes(const size_t *odims, const size_t *idims, 
     const ConvGeom g = make_geom(odims, idims, fdims, kernels, strides, pads);
     if (g.M == 0 || g.OC == 0) return 0;
     if (g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0) return 0;
-    return conv_scratch_bytes(g, nullptr, nullptr);   // (tensors of a generated program are 256-byte aligned)
+    return conv_total_scratch(g, nullptr, nullptr);   // (tensors of a generated program are 256-byte aligned)
 }
 
 int swc_hip_conv2dGrad_f(float *inputG, float *filterG, float *biasG, const float *outputG, const float *input,

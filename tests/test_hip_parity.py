@@ -544,6 +544,41 @@ def test_conv_tiles_shared_along_k(rt, oracle, variant, monkeypatch):
     assert np.max(np.abs(got - want) / scale) < TOL
 
 
+@pytest.mark.parametrize("idims,fdims,strides,pads", [((2, 9, 10, 6), (40, 3, 3, 6), (1, 1), (1, 1, 1, 1)),
+                                                      ((1, 13, 11, 50), (20, 5, 5, 50), (1, 1), (0, 0, 0, 0)),
+                                                      ((2, 15, 15, 3), (64, 7, 7, 3), (2, 2), (3, 3, 3, 3)),
+                                                      ((3, 8, 8, 10), (33, 3, 3, 10), (1, 1), (1, 1, 1, 1))])
+def test_conv_with_a_channel_count_that_is_no_multiple_of_4(rt, oracle, idims, fdims, strides, pads):
+    """Too large for the direct kernel: computed on zero-padded copies of input and filter in the workspace."""
+    from swcompiler_amd.hip import SwcHipError
+    print("case conv, padded channels", idims, fdims, flush=True)
+    rng = np.random.default_rng(sum(idims) + sum(fdims))
+    x = rng.integers(-4, 5, idims).astype(np.float32)
+    f = rng.integers(-4, 5, fdims).astype(np.float32)
+    b = rng.integers(-4, 5, fdims[0]).astype(np.float32)
+    want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
+    need = rt.conv2d_workspace_bytes(idims, fdims, strides, pads)
+    cp = (idims[3] + 3) // 4 * 4
+    assert need >= 4 * (idims[0] * idims[1] * idims[2] * cp + fdims[0] * fdims[1] * fdims[2] * cp)
+    assert_bit_exact(rt.conv2d(*up(rt, x, f, b), fdims[1:3], strides, pads).numpy(), want, "padded channels")
+    exact, short = rt.empty((need // 4,)), rt.empty((need // 4 - 4,))
+    try:
+        rt.set_workspace(exact)
+        assert_bit_exact(rt.conv2d(*up(rt, x, f, b), fdims[1:3], strides, pads, relu=True).numpy(), oracle.relu(want),
+                         "padded channels, caller workspace")
+        rt.set_workspace(short)
+        with pytest.raises(SwcHipError, match="workspace"):
+            rt.conv2d(*up(rt, x, f, b), fdims[1:3], strides, pads)
+    finally:
+        rt.sync()
+        rt.set_workspace(None)
+    xr = rng.standard_normal(idims).astype(np.float32)
+    fr = rng.standard_normal(fdims).astype(np.float32)
+    got = rt.conv2d(*up(rt, xr, fr, b), fdims[1:3], strides, pads).numpy()
+    scale = oracle.conv2d(np.abs(xr), np.abs(fr), np.abs(b), fdims[1:3], strides, pads)
+    assert np.max(np.abs(got - oracle.conv2d(xr, fr, b, fdims[1:3], strides, pads)) / scale) < TOL
+
+
 def test_conv_shared_tiles_in_a_caller_workspace(rt, oracle, monkeypatch):
     from swcompiler_amd.hip import SwcHipError
     idims, fdims, strides, pads = SHARED_CONV_CASES[0]
