@@ -137,22 +137,27 @@ def merge_rows(all_rows):
 
 def with_transfers(rt, graphs, cfg, steps):
     """The same step with the input batch uploaded and the result downloaded every step
-    (pageable host memory, synchronous copies: what a generated program's batch loop does)."""
+    (page-locked host memory, synchronous copies: what a generated program's batch loop does)."""
     t = graphs.make_inputs(cfg)
     dt = {k: rt.upload(v) for k, v in t.items()}
     batch = graphs.batch_of(cfg, t)
     ws = {}
     out = graphs.run(cfg, rt, dt, fused=True, ws=ws)
-    host_out = np.empty(out.shape, np.float32)
+    # page-locked host buffers, as the host arena of a generated program is
+    host_x, host_out = rt.pinned_empty(t["x"].shape), rt.pinned_empty(out.shape)
+    host_x[...] = t["x"]
     rt.sync()
     t0 = time.perf_counter()
     for _ in range(steps):
-        rt.upload_into(dt["x"], t["x"])
+        rt.upload_into(dt["x"], host_x)
         out = graphs.run(cfg, rt, dt, fused=True, ws=ws)
         rt.download_into(host_out, out)
     wall = time.perf_counter() - t0
-    return dict(samples_per_s=batch * steps / wall, ms_per_step=wall * 1e3 / steps,
-                h2d_bytes=int(t["x"].nbytes), d2h_bytes=int(host_out.nbytes))
+    res = dict(samples_per_s=batch * steps / wall, ms_per_step=wall * 1e3 / steps,
+               h2d_bytes=int(host_x.nbytes), d2h_bytes=int(host_out.nbytes), host_memory="page-locked")
+    rt.free_pinned(host_x)
+    rt.free_pinned(host_out)
+    return res
 
 
 def measured_peaks(rt):

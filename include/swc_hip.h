@@ -51,6 +51,11 @@ int swc_hip_init(int device);                 /* idempotent; selects device, cre
 int swc_hip_shutdown(void);                   /* destroys the stream; outstanding allocations stay valid */
 void *swc_hip_malloc(size_t bytes);           /* 256-byte aligned device memory, NULL on failure */
 int swc_hip_free(void *dptr);
+/* Page-locked host memory for buffers that are uploaded or downloaded every
+ * iteration (the host arena of a generated program): copies from and to it run
+ * at the full rate of the link, without the staging copy pageable memory costs. */
+void *swc_hip_host_malloc(size_t bytes);      /* NULL on failure */
+int swc_hip_host_free(void *hptr);
 int swc_hip_h2d(void *dst_dev, const void *src_host, size_t bytes); /* ordered after prior ops, returns when done */
 int swc_hip_d2h(void *dst_host, const void *src_dev, size_t bytes); /* ordered after prior ops, returns when done */
 int swc_hip_d2d(void *dst_dev, const void *src_dev, size_t bytes);  /* async on the stream */

@@ -182,6 +182,28 @@ int swc_hip_free(void *dptr) {
     return SWC_HIP_OK;
 }
 
+void *swc_hip_host_malloc(size_t bytes) {
+    if (!ready()) {
+        fail(SWC_HIP_ENOTINIT, "swc_hip_host_malloc: swc_hip_init has not been called");
+        return nullptr;
+    }
+    void *p = nullptr;
+    hipError_t e = hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        fail(SWC_HIP_ERUNTIME, "swc_hip_host_malloc(%zu): %s", bytes, hipGetErrorString(e));
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return p;
+}
+
+int swc_hip_host_free(void *p) {
+    SWC_REQUIRE_INIT();
+    if (!p) return SWC_HIP_OK;
+    SWC_HIP_TRY(hipHostFree(p));
+    return SWC_HIP_OK;
+}
+
 int swc_hip_h2d(void *dst, const void *src, size_t bytes) {
     SWC_REQUIRE_INIT();
     SWC_ARG(bytes == 0 || (dst && src));

@@ -27,7 +27,7 @@ EXPORTS = [
     "swc_hip_matrixSoftmax_f", "swc_hip_matrixTanh_f", "swc_hip_argMax_i",
     "swc_hip_matrixMatrixFCBias_f", "swc_hip_vecAddRelu_f", "swc_hip_batchnormRelu_f",
     "swc_hip_batchnormReluMaxpool_f", "swc_hip_conv2dFused_f",
-    "swc_hip_set_workspace", "swc_hip_matrixMatrixFCBiasSoftmax_f", "swc_hip_gemm_workspace_bytes", "swc_hip_conv2d_workspace_bytes", "swc_hip_matrixTrans_f", "swc_hip_matrixTanhGrad_f", "swc_hip_matrixSoftmaxWithLoss_f",
+    "swc_hip_set_workspace", "swc_hip_matrixMatrixFCBiasSoftmax_f", "swc_hip_gemm_workspace_bytes", "swc_hip_conv2d_workspace_bytes", "swc_hip_host_malloc", "swc_hip_host_free", "swc_hip_matrixTrans_f", "swc_hip_matrixTanhGrad_f", "swc_hip_matrixSoftmaxWithLoss_f",
     "swc_hip_matrixSoftmaxGrad_f", "swc_hip_matrixSoftmaxWithLossGrad_f", "swc_hip_conv2dGrad_f",
     "swc_hip_maxpoolGrad_f", "swc_hip_batchedreduceadd_f", "swc_hip_sgd_f", "swc_hip_reluGrad_f",
 ]
@@ -96,6 +96,8 @@ def load_library():
         "swc_hip_conv2dFused_f": (i32, [vp, vp, vp, vp, szp, szp, szp, szp, szp, szp, szp, sz,
                                         vp, vp, vp, vp, f32, i32]),
         "swc_hip_set_workspace": (i32, [vp, sz]),
+        "swc_hip_host_malloc": (vp, [sz]),
+        "swc_hip_host_free": (i32, [vp]),
         "swc_hip_gemm_workspace_bytes": (sz, [i32, i32, i32]),
         "swc_hip_conv2d_workspace_bytes": (sz, [szp] * 6),
         "swc_hip_matrixTrans_f": (i32, [i32, i32, vp, i32, vp, i32]),
@@ -180,6 +182,7 @@ class SwcHip:
     def __init__(self, device=0):
         self.lib = load_library()
         self._check(self.lib.swc_hip_init(device), "swc_hip_init")
+        self._pinned = {}   # address of a pinned numpy array -> the pointer to free
 
     # -- plumbing --------------------------------------------------------
     def _check(self, rc, what):
@@ -453,6 +456,20 @@ class SwcHip:
         out = out if out is not None else self.empty(src.shape)
         self._check(self.lib.swc_hip_reluGrad_f(out.ptr, src.ptr, dest_grad.ptr, src.size), "reluGrad_f")
         return out
+
+    def pinned_empty(self, shape, dtype=np.float32):
+        """a numpy array in page-locked host memory (kept alive by the returned array; freed with free_pinned)"""
+        n = int(np.prod(shape)) * np.dtype(dtype).itemsize
+        ptr = self.lib.swc_hip_host_malloc(max(n, 1))
+        if not ptr:
+            raise SwcHipError("swc_hip_host_malloc: " + self.lib.swc_hip_last_error().decode())
+        buf = (C.c_char * max(n, 1)).from_address(ptr)
+        arr = np.frombuffer(buf, dtype=dtype, count=int(np.prod(shape))).reshape(shape)
+        self._pinned[arr.ctypes.data] = ptr
+        return arr
+
+    def free_pinned(self, arr):
+        self._check(self.lib.swc_hip_host_free(self._pinned.pop(arr.ctypes.data)), "swc_hip_host_free")
 
     def gemm_workspace_bytes(self, m, n, k):
         """scratch bytes an m x n x k FC/GEMM call uses on this device (0 unless it is split over K)"""

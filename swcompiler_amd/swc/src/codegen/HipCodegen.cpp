@@ -106,7 +106,10 @@ void HipCodegen::emitMemAllocations() {
     for (auto &a : mem_allocators_) {
         if (!a->getMemAllocated()) continue;
         if (a->getDevice().type == DeviceType::CPU) {
-            writer_ << a->getBasePtrName() << " = (char*)malloc(" << a->getMemAllocated() << ");\n";
+            // page-locked: the per-iteration uploads and downloads run at the rate of the link
+            writer_ << a->getBasePtrName() << " = (char*)swc_hip_host_malloc(" << a->getMemAllocated() << ");\n";
+            writer_ << "if (!" << a->getBasePtrName() << ") { std::fprintf(stderr, \"%s\\n\", swc_hip_last_error()); "
+                    << "return 1; }\n";
         } else {
             writer_ << a->getBasePtrName() << " = (char*)swc_hip_malloc(" << a->getMemAllocated() << ");\n";
             writer_ << "if (!" << a->getBasePtrName() << ") { std::fprintf(stderr, \"%s\\n\", swc_hip_last_error()); "
@@ -301,7 +304,7 @@ void HipCodegen::emitMemFree() {
                 << "if (gpu0_ws) SWC_HIP_CHECK(swc_hip_free(gpu0_ws));\n";
     for (auto &a : mem_allocators_) {
         if (!a->getMemAllocated()) continue;
-        if (a->getDevice().type == DeviceType::CPU) writer_ << "free(" << a->getBasePtrName() << ");\n";
+        if (a->getDevice().type == DeviceType::CPU) writer_ << "SWC_HIP_CHECK(swc_hip_host_free(" << a->getBasePtrName() << "));\n";
         else writer_ << "SWC_HIP_CHECK(swc_hip_free(" << a->getBasePtrName() << "));\n";
     }
 }

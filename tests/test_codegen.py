@@ -133,6 +133,9 @@ def test_hip_program_structure_and_build(gen, tmp_path):
     # every device tensor sits on a 256-byte boundary of the arena
     offs = [int(v) for v in re.findall(r"gpu0_baseptr \+ (\d+)\)", code)]
     assert offs and all(o % 256 == 0 for o in offs)
+    # the host arena is page-locked memory of the library's, the device arena one allocation
+    assert "cpu0_baseptr = (char*)swc_hip_host_malloc(" in code and "swc_hip_host_free(cpu0_baseptr)" in code
+    assert code.count("swc_hip_malloc(") == 2   # workspace and arena
     # parameters are uploaded once, before the op calls; the result comes back once, after them
     body = code[code.index("// call op routine functions"):]
     assert "swc_hip_h2d" not in body and body.count("swc_hip_d2h(") == 1
