@@ -52,8 +52,10 @@ int swc_hip_shutdown(void);                   /* destroys the stream; outstandin
 void *swc_hip_malloc(size_t bytes);           /* 256-byte aligned device memory, NULL on failure */
 int swc_hip_free(void *dptr);
 /* Page-locked host memory for buffers that are uploaded or downloaded every
- * iteration (the host arena of a generated program): copies from and to it run
- * at the full rate of the link, without the staging copy pageable memory costs. */
+ * iteration (the host arena of a generated program, where the reference's
+ * generated code calls malloc, src/codegen/Codegen.cpp:504-511): copies from
+ * and to it run at the full rate of the link, without the staging copy pageable
+ * memory costs. */
 void *swc_hip_host_malloc(size_t bytes);      /* NULL on failure */
 int swc_hip_host_free(void *hptr);
 int swc_hip_h2d(void *dst_dev, const void *src_host, size_t bytes); /* ordered after prior ops, returns when done */
@@ -61,18 +63,19 @@ int swc_hip_d2h(void *dst_host, const void *src_dev, size_t bytes); /* ordered a
 int swc_hip_d2d(void *dst_dev, const void *src_dev, size_t bytes);  /* async on the stream */
 int swc_hip_fill_f(float *dst_dev, float value, size_t count);      /* initTensorConstant/Zero, kernels.h:23-29 */
 int swc_hip_sync(void);
-/* Scratch device memory for the ops that need some (FC/GEMM and convolution calls
- * that are cut along K: swc_hip_gemm_workspace_bytes, swc_hip_conv2d_workspace_bytes;
- * conv2dGrad_f: the
- * transposed gradient and operand copies, up to about twice the size of its
- * largest argument; matrixSoftmaxWithLoss_f: 4*m bytes).  A generated program
- * reserves a slot of its arena and passes it here once; without this call the
+/* No counterpart in the reference (its kernels need no scratch memory).
+ * Scratch device memory for the ops that need some (FC/GEMM and convolution
+ * calls that are cut along K or run on padded copies: swc_hip_gemm_workspace_bytes,
+ * swc_hip_conv2d_workspace_bytes; conv2dGrad_f: the transposed gradient and
+ * operand copies, up to about twice the size of its largest argument;
+ * matrixSoftmaxWithLoss_f: 4*m bytes).  A generated program allocates the
+ * maximum over its calls once and passes it here; without this call the
  * library allocates a buffer of its own on first need and grows it on demand
  * (not possible while a graph is being recorded).  dptr NULL, bytes 0: back to
  * the library's own buffer.  The buffer is shared by all ops on the stream. */
 int swc_hip_set_workspace(void *dptr, size_t bytes);
-/* Workspace a matrixMatrixMul_f / matrixMatrixFCBias_f call of this shape uses on the
- * initialised device (0 for most shapes: only products with few output tiles and a K
+/* No counterpart in the reference.  Workspace a matrixMatrixMul_f /
+ * matrixMatrixFCBias_f call of this shape uses on the initialised device (0 for most shapes: only products with few output tiles and a K
  * of hundreds are split over K).  A generated program takes the maximum over its
  * calls and provides that much with swc_hip_set_workspace. */
 size_t swc_hip_gemm_workspace_bytes(int m, int n, int k);
@@ -81,8 +84,8 @@ size_t swc_hip_gemm_workspace_bytes(int m, int n, int k);
  * left over after every CU has had its share of whole tiles are cut along K and
  * their partial sums kept here; a layer whose input-channel count is no multiple
  * of 4 (and that is too large for the direct first-layer kernel) is computed on
- * zero-padded copies of input and filter, which live here too.  Without a workspace large enough the library
- * allocates its own at the first such call. */
+ * zero-padded copies of input and filter, which live here too.  Without a
+ * workspace large enough the library allocates its own at the first such call. */
 size_t swc_hip_conv2d_workspace_bytes(const size_t *odims, const size_t *idims, const size_t *fdims,
                                       const size_t *kernels, const size_t *strides, const size_t *pads);
 const char *swc_hip_last_error(void);         /* message of the last failure on this thread ("" if none) */
