@@ -289,7 +289,7 @@ __global__ __launch_bounds__(256) void splitk_finish(float *__restrict__ c, size
 
 // --------------------------------------------------------------- skinny GEMM
 typedef float v4f __attribute__((ext_vector_type(4)));
-constexpr int kSkinnyMaxWaves = 8;
+constexpr int kSkinnyMaxWaves = 16;
 constexpr int kSkinnyUnroll = 4;
 
 // v_mfma_f32_16x16x4_f32: A[i][kk] i = l%16, kk = l/16; B[kk][j] j = l%16, kk = l/16;
@@ -532,9 +532,10 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
     if (n <= 16) {
         const bool vec = (k % 4 == 0) && (lda % 4 == 0) && aligned16(a);
         // K is split over the wavefronts of a workgroup: four (the reduction step needs 256 threads) take K up
-        // to 1024 in one or two trips each; eight beyond that.  More wavefronts only lengthen the reduction
-        // (8x512x10: 6.0 us with sixteen, 4.5 with four; 65536x1024x16: 116 against 79 us).
-        const int waves = k <= 1024 ? 4 : 8;
+        // to 1024 in one or two trips each — more only lengthen the reduction (8x512x10: 6.0 us with sixteen,
+        // 4.5 with four; 65536x1024x16: 116 against 79 us); sixteen for longer K (4096x4096x10 inside the MLP:
+        // 19.6 us against 22.0 with eight).
+        const int waves = k <= 1024 ? 4 : kSkinnyMaxWaves;
         const unsigned blocks = ceil_div(m, 16);
         if (vec) gemm_skinny<true><<<blocks, 64 * waves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep, softmax);
         else gemm_skinny<false><<<blocks, 64 * waves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep, softmax);
