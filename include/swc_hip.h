@@ -62,6 +62,7 @@ int swc_hip_h2d(void *dst_dev, const void *src_host, size_t bytes); /* ordered a
 int swc_hip_d2h(void *dst_host, const void *src_dev, size_t bytes); /* ordered after prior ops, returns when done */
 int swc_hip_d2d(void *dst_dev, const void *src_dev, size_t bytes);  /* async on the stream */
 int swc_hip_fill_f(float *dst_dev, float value, size_t count);      /* initTensorConstant/Zero, kernels.h:23-29 */
+int swc_hip_fill_i(int *dst_dev, int value, size_t count);          /* the same for an Int32 tensor (counters) */
 int swc_hip_sync(void);
 /* No counterpart in the reference (its kernels need no scratch memory).
  * Scratch device memory for the ops that need some (FC/GEMM and convolution
@@ -198,6 +199,11 @@ int swc_hip_matrixTanh_f(int m, int n, const float *a, int lda, float *b,
 /* kernels.h:601-613; Codegen.cpp:2372-2385 (ArgMax op).  idx[m,top_k] = columns of the top_k largest
  * values of each row, ties listing the larger column first. top_k <= 8. */
 int swc_hip_argMax_i(const float *input, int *idx, int m, int n, int top_k);
+
+/* kernels.h:615-627; Codegen.cpp:2387-2398 (Accuracy op).  For each of the m rows: accum_cnt[1] += 1, and
+ * accum_cnt[0] += 1 when label[row] is among the row's n predictions pred[row, 0..n).  The counters
+ * accumulate over calls; all three pointers are device memory. */
+int swc_hip_accuracy_i(const int *pred, const int *label, int *accum_cnt, int m, int n);
 
 /* ---- training kernels: same arguments as the reference's; `selected` and `loss`
  * are device pointers like every other data pointer ---- */

@@ -188,6 +188,16 @@ class CpuKernels:
                              C.c_int(n), C.c_int(top_k))
         return idx
 
+    def accuracy(self, pred, label, counters):
+        """adds this batch to counters = [hits, rows] (int32[2]) in place and returns it"""
+        pred = np.ascontiguousarray(pred, np.int32)
+        label = np.ascontiguousarray(label, np.int32)
+        m, n = pred.shape
+        assert counters.dtype == np.int32 and counters.size == 2 and counters.flags.c_contiguous
+        self._fn("accuracy_i")(pred.ctypes.data_as(_i32p), label.ctypes.data_as(_i32p),
+                               counters.ctypes.data_as(_i32p), C.c_int(m), C.c_int(n))
+        return counters
+
     # ---- training kernels ---------------------------------------------
     def matrixTrans(self, a):
         a = np.ascontiguousarray(a, np.float32)

@@ -69,6 +69,7 @@ void ref_vecAdd_f(int n, float *a, float *b, float *c) { vecAdd_f(n, a, b, c); }
 void ref_argMax_i(const float *in, int *idx, int m, int n, int k) {
     argMax_i(in, idx, m, n, k);
 }
+void ref_accuracy_i(const int *pred, const int *label, int *accum, int m, int n) { accuracy_i(pred, label, accum, m, n); }
 void ref_matrixTrans_f(int m, int n, const float *a, int lda, float *b, int ldb) { matrixTrans_f(m, n, a, lda, b, ldb); }
 void ref_matrixTanhGrad_f(int m, int n, float *a, int lda, const float *b, int ldb, const float *c, int ldc) {
     matrixTanhGrad_f(m, n, a, lda, b, ldb, c, ldc);

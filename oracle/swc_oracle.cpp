@@ -294,6 +294,16 @@ void oracle_argMax_i(const float *input, int *idx, int m, int n, int top_k) {
     }
 }
 
+// kernels.h:615-627.  Each of the m rows adds one to accum_cnt[1], and one to accum_cnt[0] when its
+// label is among its n predictions (first match ends the search of the row).
+void oracle_accuracy_i(const int *pred, const int *label, int *accum_cnt, int m, int n) {
+    for (int row = 0; row < m; ++row) {
+        accum_cnt[1] += 1;
+        const int *p = pred + (size_t)row * n;
+        if (std::find(p, p + n, label[row]) != p + n) accum_cnt[0] += 1;
+    }
+}
+
 // image.h:13-33: raw little-endian fp32 file, `offset` counted in elements.
 // Returns the number of elements copied, or -1 if the file cannot be read.
 long oracle_load_f(float *data, size_t size, size_t offset, const char *path);

@@ -32,7 +32,7 @@ struct State {
     bool ws_owned = false;
 } g;
 
-__global__ void fill_kernel(float *__restrict__ dst, float v, size_t n) {
+template <typename T> __global__ void fill_kernel(T *__restrict__ dst, T v, size_t n) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t step = (size_t)gridDim.x * blockDim.x;
     for (; i < n; i += step) dst[i] = v;
@@ -231,6 +231,17 @@ int swc_hip_d2d(void *dst, const void *src, size_t bytes) {
 }
 
 int swc_hip_fill_f(float *dst, float value, size_t count) {
+    SWC_REQUIRE_INIT();
+    SWC_ARG(count == 0 || dst);
+    if (!count) return SWC_HIP_OK;
+    unsigned blocks = ceil_div(count, 256);
+    if (blocks > 4096u) blocks = 4096u;
+    fill_kernel<<<blocks, 256, 0, stream()>>>(dst, value, count);
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
+}
+
+int swc_hip_fill_i(int *dst, int value, size_t count) {
     SWC_REQUIRE_INIT();
     SWC_ARG(count == 0 || dst);
     if (!count) return SWC_HIP_OK;

@@ -1,4 +1,4 @@
-// matrixSoftmax_f (kernels.h:88-103) and argMax_i (kernels.h:601-613).
+// matrixSoftmax_f (kernels.h:88-103), argMax_i (kernels.h:601-613) and accuracy_i (kernels.h:615-627).
 //
 // Softmax is one read and one write of the matrix (8 B/element): a 64-lane
 // wavefront owns a row, keeps it in registers as float4s, and reduces the row
@@ -131,6 +131,24 @@ __global__ __launch_bounds__(256) void argmax_rows(const float *in, int *idx, in
     for (int t = 0; t < top_k; ++t) idx[(size_t)row * top_k + t] = (t < have) ? bi[t] : 0;
 }
 
+// accuracy_i: one lane per row looks for its label among the row's n predictions; the workgroup's count of
+// hits and its row count go to the two counters with one integer atomic each, so repeated calls accumulate
+// exactly as the host loop does, in any order.
+__global__ __launch_bounds__(256) void accuracy_rows(const int *pred, const int *label, int *accum, int m, int n) {
+    const int row = blockIdx.x * 256 + threadIdx.x;
+    int hit = 0;
+    if (row < m) {
+        const int want = label[row];
+        for (int j = 0; j < n; ++j) hit |= pred[(size_t)row * n + j] == want;
+    }
+    const int hits = __syncthreads_count(hit);
+    if (threadIdx.x == 0) {
+        const int rows = min(256, m - (int)blockIdx.x * 256);
+        if (hits) atomicAdd(accum, hits);
+        atomicAdd(accum + 1, rows);
+    }
+}
+
 } // namespace
 
 extern "C" {
@@ -174,6 +192,16 @@ int swc_hip_argMax_i(const float *input, int *idx, int m, int n, int top_k) {
     if (top_k > kMaxTopK)
         return fail(SWC_HIP_EUNSUPPORTED, "swc_hip_argMax_i: top_k %d exceeds %d", top_k, kMaxTopK);
     argmax_rows<<<ceil_div(m, 256), 256, 0, stream()>>>(input, idx, m, n, top_k);
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
+}
+
+int swc_hip_accuracy_i(const int *pred, const int *label, int *accum_cnt, int m, int n) {
+    SWC_REQUIRE_INIT();
+    SWC_ARG(m >= 0 && n >= 0);
+    if (m == 0) return SWC_HIP_OK;
+    SWC_ARG(label && accum_cnt && (n == 0 || pred));
+    accuracy_rows<<<ceil_div(m, 256), 256, 0, stream()>>>(pred, label, accum_cnt, m, n);
     SWC_LAUNCH_CHECK();
     return SWC_HIP_OK;
 }

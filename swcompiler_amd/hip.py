@@ -24,7 +24,7 @@ EXPORTS = [
     "swc_hip_matrixMatrixMul_f", "swc_hip_batchedadd_f", "swc_hip_relu_f",
     "swc_hip_vecAdd_f", "swc_hip_conv2d_f", "swc_hip_batchnormalization_f", "swc_hip_maxpool_f",
     "swc_hip_maxpool_argmax_f", "swc_hip_avgpool_f", "swc_hip_transpose4d_f", "swc_hip_transpose2d_f",
-    "swc_hip_matrixSoftmax_f", "swc_hip_matrixTanh_f", "swc_hip_argMax_i",
+    "swc_hip_matrixSoftmax_f", "swc_hip_matrixTanh_f", "swc_hip_argMax_i", "swc_hip_accuracy_i", "swc_hip_fill_i",
     "swc_hip_matrixMatrixFCBias_f", "swc_hip_vecAddRelu_f", "swc_hip_batchnormRelu_f",
     "swc_hip_batchnormReluMaxpool_f", "swc_hip_conv2dFused_f",
     "swc_hip_set_workspace", "swc_hip_matrixMatrixFCBiasSoftmax_f", "swc_hip_gemm_workspace_bytes", "swc_hip_conv2d_workspace_bytes", "swc_hip_host_malloc", "swc_hip_host_free", "swc_hip_matrixTrans_f", "swc_hip_matrixTanhGrad_f", "swc_hip_matrixSoftmaxWithLoss_f",
@@ -88,6 +88,8 @@ def load_library():
         "swc_hip_matrixSoftmax_f": (i32, [i32, i32, vp, i32, vp, i32]),
         "swc_hip_matrixTanh_f": (i32, [i32, i32, vp, i32, vp, i32]),
         "swc_hip_argMax_i": (i32, [vp, vp, i32, i32, i32]),
+        "swc_hip_accuracy_i": (i32, [vp, vp, vp, i32, i32]),
+        "swc_hip_fill_i": (i32, [vp, i32, sz]),
         "swc_hip_matrixMatrixFCBias_f": (i32, [i32, i32, i32, vp, i32, vp, i32, vp, vp, i32, i32]),
         "swc_hip_matrixMatrixFCBiasSoftmax_f": (i32, [i32, i32, i32, vp, i32, vp, i32, vp, vp, i32]),
         "swc_hip_vecAddRelu_f": (i32, [i32, vp, vp, vp]),
@@ -330,6 +332,16 @@ class SwcHip:
         out = self.empty((m, top_k), np.int32)
         self._check(self.lib.swc_hip_argMax_i(x.ptr, out.ptr, m, n, top_k), "argMax_i")
         return out
+
+    def accuracy(self, pred, label, counters):
+        """adds this batch to the device counters [hits, rows] (int32[2]) and returns them"""
+        m, n = pred.shape
+        self._check(self.lib.swc_hip_accuracy_i(pred.ptr, label.ptr, counters.ptr, m, n), "accuracy_i")
+        return counters
+
+    def fill_i(self, t, value):
+        self._check(self.lib.swc_hip_fill_i(t.ptr, int(value), t.size), "fill_i")
+        return t
 
     def conv2d(self, x, filt, bias, kernels=None, strides=(1, 1), pads=(0, 0, 0, 0), group=1, bn=None,
                eps=1e-5, relu=False, out=None):

@@ -126,7 +126,7 @@ class Codegen {
     virtual void emitMemFree();
     virtual void emitDataLoaderInit() {}          // training loader: not part of the inference build
     virtual void emitInferDataLoaderInit();        // `DataLoader loader(...)` + iteration counter
-    void emitPrintGraphOutputs();                  // every Config::display iterations: the display tensors
+    virtual void emitPrintGraphOutputs();          // every Config::display iterations: the display tensors
 
     void codeGenInit();
     void emitMemAllocs();
@@ -156,6 +156,11 @@ class Codegen {
 class HipCodegen : public Codegen {
     devices::HipDevice device_;
     bool has_workspace_ = false;   // the program holds a workspace for its FC calls
+    // Inside the batch loop a download nobody on the host reads (a graph output, a counter that is only
+    // displayed) is not emitted per iteration: it is held here and emitted where it is shown and once after
+    // the loop, so the device runs one batch while the loader reads the next.
+    bool defer_output_gathers_ = false;
+    std::vector<OpNode *> deferred_gathers_;
 
   public:
     HipCodegen(IRGraph *graph, Config &config) : Codegen(graph, config) {}
@@ -171,8 +176,11 @@ class HipCodegen : public Codegen {
     void emitTensorInitializations() override;
     void emitExecute() override;
     void emitMemFree() override;
+    void emitPrintGraphOutputs() override;
 
   protected:
+    void emitDeviceFills();        // constant initialisers of device tensors that have no host twin
+    void emitDeferredGathers();
     void dispatchOpNode(OpNode *op) override;
     void emitHipCall(OpNode *op);
     void emitTransfer(OpNode *op, bool toDevice);

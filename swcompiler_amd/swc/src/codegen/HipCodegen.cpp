@@ -133,14 +133,12 @@ void HipCodegen::emitTensorInitializations() {
         case TensorInitType::PARENTOP:   // filled by its run-once producer, below
             break;
         case TensorInitType::CONSTANT:
-        case TensorInitType::ZERO: {
-            const float v = t->getTensorInitType() == TensorInitType::ZERO ? 0.f : info.getConstant();
-            if (onGpu && t->getDataType() == DataType::Float_t)
-                writer_ << "SWC_HIP_CHECK(swc_hip_fill_f(" << name << ", " << v << ", " << t->size() << "));\n";
-            else if (!onGpu)
+        case TensorInitType::ZERO:
+            if (!onGpu) {
+                const float v = t->getTensorInitType() == TensorInitType::ZERO ? 0.f : info.getConstant();
                 writer_ << "initTensorConstant(" << name << ", " << t->size() << ", " << v << ");\n";
-            break;
-        }
+            }
+            break;   // device tensors: emitDeviceFills()
         case TensorInitType::XAVIER:
             assert(!onGpu);
             writer_ << "initTensorXavier(" << name << ", " << t->size() << ", " << info.getFilterSize() << ");\n";
@@ -154,6 +152,7 @@ void HipCodegen::emitTensorInitializations() {
             break;
         }
     }
+    emitDeviceFills();
     // every run-once op (parameter uploads), in topological order; runable() lets each through once
     for (int i = 0; i < graph_->topologyNum(); ++i)
         for (int j = 0; j < graph_->getNumInTopoLevel(i); ++j) {
@@ -166,6 +165,60 @@ void HipCodegen::emitTensorInitializations() {
     writer_ << "\n";
 }
 
+// A device tensor with a constant initialiser of its own is filled on the device (the counters of an
+// Accuracy node are the usual case).
+void HipCodegen::emitDeviceFills() {
+    for (TensorNode *tn : decl_order_) {
+        Tensor *t = tn->getTensor();
+        if (tn->getLabel()->getDeviceLabel().type != DeviceType::GPU) continue;
+        const TensorInitType init = t->getTensorInitType();
+        if (init != TensorInitType::CONSTANT && init != TensorInitType::ZERO) continue;
+        const float v = init == TensorInitType::ZERO ? 0.f : t->getTensorInitInfo().getConstant();
+        const std::string name = tensors_name_map_.at(t);
+        if (t->getDataType() == DataType::Float_t)
+            writer_ << "SWC_HIP_CHECK(swc_hip_fill_f(" << name << ", " << v << ", " << t->size() << "));\n";
+        else if (t->getDataType() == DataType::Int32_t)
+            writer_ << "SWC_HIP_CHECK(swc_hip_fill_i(" << name << ", " << static_cast<int>(v) << ", " << t->size()
+                    << "));\n";
+    }
+}
+
+void HipCodegen::emitDeferredGathers() {
+    defer_output_gathers_ = false;
+    if (!deferred_gathers_.empty()) writer_ << "// what the last batch left on the device\n";
+    for (OpNode *g : deferred_gathers_) emitTransfer(g, false);
+    deferred_gathers_.clear();
+}
+
+// The display tensors every Config::display iterations (reference: src/codegen/Codegen.cpp:815-854); one
+// that lives on the device is downloaded there, into its host twin, and the twin is printed.
+void HipCodegen::emitPrintGraphOutputs() {
+    writer_ << "\nif (iter % " << config_.display << " == 0) {\n";
+    writer_.indentInc();
+    writer_ << "std::cout << \"iterations \" << iter << \"\\n\";\n";
+    for (TensorNode *tn : graph_->getDisplayTensorNodes()) {
+        TensorNode *shown = tn;
+        if (tn->getLabel()->getDeviceLabel().type == DeviceType::GPU) {
+            OpNode *gather = nullptr;
+            for (IRNode *c : tn->getChildNodes())
+                if (c->nodeType() == OP_NODE && static_cast<OpNode *>(c)->getOp()->getOpName() == "Gather")
+                    gather = static_cast<OpNode *>(c);
+            if (!gather) {
+                SWLOG_ERROR << "display tensor " << tn->name() << " lives on the device and has no Gather" << std::endl;
+                std::abort();
+            }
+            emitTransfer(gather, false);
+            shown = static_cast<TensorNode *>(gather->getChildNode(0));
+        }
+        Tensor *t = shown->getTensor();
+        writer_ << "// " << tn->name() << "\n";
+        writer_ << "printMatrix(" << tensors_name_map_.at(t) << ", " << t->getDim(0) << ", "
+                << (t->getNDim() == 2 ? t->getDim(1) : 1) << ");\n";
+    }
+    writer_.indentDec();
+    writer_ << "}\n";
+}
+
 void HipCodegen::emitExecute() {
     if (config_.use_dataloader && config_.hip_graph && deviceOpsAreContiguous()) {
         // The batch loop with the device ops of an iteration as one HIP graph: a pass over whatever the arena
@@ -175,13 +228,16 @@ void HipCodegen::emitExecute() {
         writer_.indentInc();
         emitDeviceOpsOnly();
         writer_.indentDec();
-        writer_ << "}\nSWC_HIP_CHECK(swc_hip_sync());\n";
+        writer_ << "}\n";
+        emitDeviceFills();   // counters the warm-up pass has touched start again
+        writer_ << "SWC_HIP_CHECK(swc_hip_sync());\n";
         writer_ << "void *swc_graph = NULL;\n";
         writer_ << "SWC_HIP_CHECK(swc_hip_graph_begin());\n{\n";
         writer_.indentInc();
         emitDeviceOpsOnly();
         writer_.indentDec();
         writer_ << "}\nSWC_HIP_CHECK(swc_hip_graph_end(&swc_graph));\n";
+        defer_output_gathers_ = true;
         writer_ << "while(loader.next(" << nameOf(graph_->getInferLabelNode()) << ", "
                 << nameOf(graph_->getInferDataNode()) << ")) {\n";
         writer_.indentInc();
@@ -205,6 +261,7 @@ void HipCodegen::emitExecute() {
         if (config_.display > 0) emitPrintGraphOutputs();
         writer_.indentDec();
         writer_ << "} //while\n";
+        emitDeferredGathers();
         writer_ << "SWC_HIP_CHECK(swc_hip_sync());\n";
         writer_ << "SWC_HIP_CHECK(swc_hip_graph_destroy(swc_graph));\n";
         return;
@@ -212,7 +269,9 @@ void HipCodegen::emitExecute() {
     if (config_.use_dataloader) {
         // the batch loop of the CPU target; the per-iteration Scatter of the data
         // tensor and the Gather in front of each host op are ordinary op nodes
+        defer_output_gathers_ = true;
         Codegen::emitExecute();
+        emitDeferredGathers();
         writer_ << "SWC_HIP_CHECK(swc_hip_sync());\n";
         return;
     }
@@ -313,9 +372,17 @@ void HipCodegen::dispatchOpNode(OpNode *op) {
     if (!op->runable()) return;
     const std::string type = op->getOp()->getOpName();
     if (type == "Scatter") return emitTransfer(op, true);
-    if (type == "Gather") return emitTransfer(op, false);
+    if (type == "Gather") {
+        if (defer_output_gathers_ && op->getChildNode(0)->childNum() == 0) {
+            if (std::find(deferred_gathers_.begin(), deferred_gathers_.end(), op) == deferred_gathers_.end())
+                deferred_gathers_.push_back(op);
+            writer_ << "// (no host op reads it: downloaded where it is displayed and after the loop)\n";
+            return;
+        }
+        return emitTransfer(op, false);
+    }
     if (op->getLabel()->getDeviceLabel().type == DeviceType::GPU) return emitHipCall(op);
-    emitFuncCall(op);   // host-side ops: Debug, Accuracy
+    emitFuncCall(op);   // host-side ops: Debug
 }
 
 void HipCodegen::emitTransfer(OpNode *op, bool toDevice) {
@@ -461,6 +528,9 @@ void HipCodegen::emitHipCall(OpNode *op) {
         const int topK = static_cast<ArgMaxOp *>(op->getOp())->getTopK();
         writer_ << "SWC_HIP_CHECK(swc_hip_argMax_i(" << nameOf(in(0)) << ", " << nameOf(out(0)) << ", "
                 << T(in(0))->getDim(0) << ", " << T(in(0))->getDim(1) << ", " << topK << "));\n";
+    } else if (type == "Accuracy") {
+        writer_ << "SWC_HIP_CHECK(swc_hip_accuracy_i(" << nameOf(in(0)) << ", " << nameOf(in(1)) << ", " << nameOf(out(0))
+                << ", " << T(in(0))->getDim(0) << ", " << T(in(0))->getDim(1) << "));\n";
     } else {
         SWLOG_ERROR << "no HIP emitter for op type " << type << " (node " << nm << ")" << std::endl;
         std::abort();

@@ -268,7 +268,7 @@ bool DeviceMemoryLoweringPass::runsOnGpu(const std::string &t) {
         "MatrixMatrixFCBiasSoftmax", "Reshape", "MatrixTanh", "MatrixSoftmax", "ElementAdd", "ElementAddRelu", "Relu", "Dropout",
         "Conv2d", "Conv2dWithActivation", "Conv2dBatchNorm", "MaxPool", "AveragePool", "Transpose",
         "BatchNormalization",
-        "BatchNormalizationRelu", "BatchNormReluMaxPool", "ArgMax"};
+        "BatchNormalizationRelu", "BatchNormReluMaxPool", "ArgMax", "Accuracy"};
     return gpu.count(t) != 0;
 }
 

@@ -270,9 +270,18 @@ def test_batch_loop_cpu_program(gen, oracle, tmp_path, compat):
 def test_batch_loop_hip_program_structure(gen, tmp_path):
     code = generate(gen, "mnist_loader", "hip", tmp_path, 44)
     body = code[code.index("while(loader.next(selected, data0))"):]
-    # inside the loop: the data batch goes up, the top-1 table comes back, accuracy runs on the host
-    assert body.count("swc_hip_h2d(") == 1 and "swc_hip_h2d(data0_dev, data0" in body
-    assert body.count("swc_hip_d2h(") == 1 and "accuracy_i(top1_host, selected, accur" in body
+    loop, tail = body[:body.index("} //while")], body[body.index("} //while"):]
+    # inside the loop: the data batch and its labels go up, ArgMax and Accuracy run on the device, and the
+    # counters come back only where they are displayed
+    assert loop.count("swc_hip_h2d(") == 2 and "swc_hip_h2d(data0_dev, data0" in loop
+    assert "swc_hip_h2d(selected_dev, selected, 32)" in loop
+    assert "swc_hip_accuracy_i(top1, selected_dev, accur, 8, 1)" in loop and "accuracy_i(top1_host" not in code
+    shown = loop[loop.index("if (iter % "):]
+    assert loop.count("swc_hip_d2h(") == 1 and shown.index("swc_hip_d2h(accur_host, accur, 8)") < shown.index("printMatrix(accur_host, 1, 2)")
+    # after the loop: the counters of the last batch reach the host once more (for the output dump)
+    assert tail.count("swc_hip_d2h(accur_host, accur, 8)") == 1
+    # the counters start at zero on the device
+    assert "swc_hip_fill_i(accur, 0, 2)" in code[:code.index("while(loader")]
     # before the loop: the four parameter uploads
     assert code[:code.index("while(loader")].count("swc_hip_h2d(") == 4
     build_hip(tmp_path)
@@ -284,7 +293,11 @@ def test_batch_loop_hip_program_structure(gen, tmp_path):
     assert head.index("swc_hip_sync()", head.index("warm-up pass")) < head.index("swc_hip_graph_begin()")
     loop = body[:body.index("} //while")]
     assert loop.count("swc_hip_graph_launch(swc_graph)") == 1 and "swc_hip_matrixMatrixFCBias" not in loop
-    assert loop.index("swc_hip_h2d(data0_dev") < loop.index("swc_hip_graph_launch") < loop.index("swc_hip_d2h(top1_host")
+    assert loop.index("swc_hip_h2d(data0_dev") < loop.index("swc_hip_h2d(selected_dev") < loop.index("swc_hip_graph_launch")
+    assert loop.index("swc_hip_graph_launch") < loop.index("swc_hip_d2h(accur_host") and "swc_hip_accuracy_i" not in loop
+    # the warm-up pass has counted a batch of whatever the arena held: the counters are cleared again before recording
+    warm = head[head.index("warm-up pass"):head.index("swc_hip_graph_begin()")]
+    assert warm.index("swc_hip_accuracy_i(") < warm.index("swc_hip_fill_i(accur, 0, 2)")
     assert "swc_hip_graph_destroy(swc_graph)" in body
     build_hip(tmp_path)
 

@@ -347,6 +347,26 @@ def test_softmax_golden_and_argmax(rt, oracle, golden):
         assert_bit_exact(rt.argMax(rt.upload(z), k).numpy(), oracle.argMax(z, k), f"argMax top{k}")
 
 
+@pytest.mark.parametrize("m,n", [(8, 1), (300, 3), (4097, 5), (256, 8), (1, 1)])
+def test_accuracy_counters(rt, oracle, m, n):
+    """accuracy_i: the two counters accumulate over calls exactly as the host loop's."""
+    rng = np.random.default_rng(m + n)
+    want = np.array([5, 7], np.int32)
+    counters = rt.upload(want.copy())
+    for call in range(3):
+        pred = rng.integers(0, 10, (m, n)).astype(np.int32)
+        label = rng.integers(0, 10, m).astype(np.int32)
+        rt.accuracy(rt.upload(pred), rt.upload(label), counters)
+        oracle.accuracy(pred, label, want)
+        assert_bit_exact(counters.numpy(), want, f"accuracy call {call}")
+    assert want[1] == 7 + 3 * m
+    # no rows: nothing changes; fill_i sets the counters
+    rt._check(rt.lib.swc_hip_accuracy_i(None, None, counters.ptr, 0, n), "accuracy_i of no rows")
+    assert_bit_exact(counters.numpy(), want, "accuracy of no rows")
+    assert rt.fill_i(counters, 0).numpy().tolist() == [0, 0]
+    assert rt.fill_i(counters, -3).numpy().tolist() == [-3, -3]
+
+
 def test_mnist8_known_answer(rt, golden):
     """test/input of the reference: FCBias -> Tanh -> FCBias -> Softmax -> ArgMax = 5 0 4 1 9 2 1 3."""
     d = os.path.join(HERE, "golden", "mnist8")

@@ -120,6 +120,19 @@ def test_relu_add_bias_specials(oracle):
     assert_bit_exact(oracle.batchedadd(m, np.array([1, 2, 3, 4], np.float32)), m + np.array([1, 2, 3, 4], np.float32), "batchedadd")
 
 
+def test_accuracy_counts(oracle):
+    """kernels.h:615-627: hits and rows accumulate over calls; a label listed twice in a row counts once."""
+    pred = np.array([[3, 1], [2, 2], [0, 4], [7, 7]], np.int32)
+    label = np.array([1, 2, 5, 7], np.int32)
+    cnt = np.array([10, 100], np.int32)
+    assert oracle.accuracy(pred, label, cnt).tolist() == [13, 104]
+    assert oracle.accuracy(pred[:, :1], label, cnt).tolist() == [15, 108]   # first column only: rows 1 and 3 hit
+    rng = np.random.default_rng(3)
+    pred, label = rng.integers(0, 10, (500, 3)).astype(np.int32), rng.integers(0, 10, 500).astype(np.int32)
+    want = int((pred == label[:, None]).any(axis=1).sum())
+    assert oracle.accuracy(pred, label, np.zeros(2, np.int32)).tolist() == [want, 500]
+
+
 def test_argmax_order(oracle):
     x = np.array([[1, 3, 3, 2, 0]], np.float32)
     assert oracle.argMax(x, 3).tolist() == [[2, 1, 3]]

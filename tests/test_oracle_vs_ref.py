@@ -72,3 +72,7 @@ def test_bn_softmax_tanh_elt(oracle, ref):
     assert_bit_exact(oracle.relu(v), ref.relu(v), "relu")
     assert_bit_exact(oracle.vecAdd(v, v[::-1].copy()), ref.vecAdd(v, v[::-1].copy()), "vecAdd")
     assert_bit_exact(oracle.argMax(np.round(z), 5), ref.argMax(np.round(z), 5), "argMax")
+    pred = oracle.argMax(np.round(z), 2)
+    label = np.random.default_rng(9).integers(0, z.shape[1], z.shape[0]).astype(np.int32)
+    assert_bit_exact(oracle.accuracy(pred, label, np.array([3, 4], np.int32)),
+                     ref.accuracy(pred, label, np.array([3, 4], np.int32)), "accuracy")
