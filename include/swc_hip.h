@@ -85,10 +85,12 @@ size_t swc_hip_gemm_workspace_bytes(int m, int n, int k);
  * left over after every CU has had its share of whole tiles are cut along K and
  * their partial sums kept here; a layer whose input-channel count is no multiple
  * of 4 (and that is too large for the direct first-layer kernel) is computed on
- * zero-padded copies of input and filter, which live here too.  Without a
- * workspace large enough the library allocates its own at the first such call. */
+ * zero-padded copies of input and filter, which live here too, and so does the
+ * filter copy of a call with more than one group.  Without a workspace large
+ * enough the library allocates its own at the first such call. */
 size_t swc_hip_conv2d_workspace_bytes(const size_t *odims, const size_t *idims, const size_t *fdims,
-                                      const size_t *kernels, const size_t *strides, const size_t *pads);
+                                      const size_t *kernels, const size_t *strides, const size_t *pads,
+                                      size_t group);
 const char *swc_hip_last_error(void);         /* message of the last failure on this thread ("" if none) */
 void *swc_hip_stream(void);                   /* the hipStream_t ops are launched on */
 int swc_hip_set_stream(void *hip_stream);     /* launch on a caller-owned stream (NULL: back to the library's own) */
@@ -145,8 +147,13 @@ int swc_hip_vecAdd_f(int size, const float *a, const float *b, float *c);
 
 /* kernels.h:177-243; Codegen.cpp:1777-1782.  NHWC input idims[4], filter
  * fdims = {oC,kH,kW,iC}, bias bdims = {oC}, output odims[4]; pads = {t,l,b,r} of
- * which only t and l enter the index arithmetic (as in the reference); group
- * must be 1.  out = bias + sum over in-bounds taps. */
+ * which only t and l enter the index arithmetic (as in the reference).
+ * out = bias + sum over in-bounds taps.  group > 1 as the reference indexes it:
+ * the filter keeps all iC channels per tap, and output channel co of group g
+ * reads channels [g*iC/group, (g+1)*iC/group) of input and filter only (computed
+ * as one group over a filter copy with the other channels zeroed, so a non-finite
+ * input value in another group's channels reaches the output as NaN).  The
+ * gradient entry point takes group 1 only. */
 int swc_hip_conv2d_f(float *output, const float *input, const float *filter,
                      const float *bias, const size_t *odims, const size_t *idims,
                      const size_t *fdims, const size_t *bdims,

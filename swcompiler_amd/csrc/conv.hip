@@ -775,6 +775,21 @@ __global__ __launch_bounds__(256) void pad_channels(float *__restrict__ dst, con
     }
 }
 
+// Grouped convolution as the reference indexes it (kernels.h:177-243: the filter keeps all iC channels per tap and
+// output channel co of group g reads only channels [g*iC/group, (g+1)*iC/group) of input and filter): a copy of
+// the filter with every other channel set to zero makes it an ordinary convolution over all channels, whose
+// extra terms are products with zero.
+__global__ __launch_bounds__(256) void mask_filter_groups(float *__restrict__ dst, const float *__restrict__ src, int OC,
+                                                          int taps, int C, int group) {
+    const size_t total = (size_t)OC * taps * C;
+    const int ocg = OC / group, cg = C / group;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const int ci = (int)(i % C);
+        const int co = (int)(i / ((size_t)taps * C));
+        dst[i] = ci / cg == co / ocg ? src[i] : 0.f;
+    }
+}
+
 // Scratch bytes the forward convolution of this geometry uses (0: none).
 size_t conv_scratch_bytes(const ConvGeom &g, const void *input, const void *filter) {
     const char *force = getenv("SWC_HIP_CONV");
@@ -812,10 +827,13 @@ size_t conv_total_scratch(const ConvGeom &g, const void *input, const void *filt
 }
 
 int check_conv_dims(const char *who, const size_t *odims, const size_t *idims, const size_t *fdims,
-                    const size_t *kernels, const size_t *strides, const size_t *pads, size_t group) {
+                    const size_t *kernels, const size_t *strides, const size_t *pads, size_t group,
+                    bool groups_ok = false) {
     if (!odims || !idims || !fdims || !kernels || !strides || !pads)
         return fail(SWC_HIP_EINVAL, "%s: null shape array", who);
-    if (group != 1) return fail(SWC_HIP_EUNSUPPORTED, "%s: group = %zu (only 1 is supported)", who, group);
+    if (group != 1 && !groups_ok) return fail(SWC_HIP_EUNSUPPORTED, "%s: group = %zu (only 1 is supported)", who, group);
+    if (group == 0 || odims[3] % group || idims[3] % group)
+        return fail(SWC_HIP_EINVAL, "%s: group = %zu does not divide oC = %zu and iC = %zu", who, group, odims[3], idims[3]);
     for (int i = 0; i < 4; ++i)
         if (odims[i] > 0x7fffffffu || idims[i] > 0x7fffffffu || fdims[i] > 0x7fffffffu)
             return fail(SWC_HIP_EINVAL, "%s: dimension too large", who);
@@ -845,11 +863,28 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
                   const size_t *odims, const size_t *idims, const size_t *fdims, const size_t *kernels,
                   const size_t *strides, const size_t *pads, size_t group, const Epilogue &ep_in,
                   bool bias_optional = false, ConvScratch scratch = {nullptr, 0}) {
-    if (int rc = check_conv_dims(who, odims, idims, fdims, kernels, strides, pads, group)) return rc;
+    if (int rc = check_conv_dims(who, odims, idims, fdims, kernels, strides, pads, group, true)) return rc;
     const ConvGeom g = make_geom(odims, idims, fdims, kernels, strides, pads);
     const size_t M = (size_t)g.M;
     if (M == 0 || odims[3] == 0) return SWC_HIP_OK;
     if (!output || !input || !filter || (!bias && !bias_optional)) return fail(SWC_HIP_EINVAL, "%s: null pointer", who);
+    if (group > 1) {
+        // the filter with the channels of other groups zeroed, then the layer as one group
+        const size_t f_b = align256((size_t)g.OC * g.K * 4);
+        const size_t need = f_b + conv_total_scratch(g, input, nullptr);
+        char *base = nullptr;
+        if (scratch.ptr && scratch.bytes >= need) base = reinterpret_cast<char *>(scratch.ptr);
+        else if (!scratch.ptr) base = static_cast<char *>(workspace(need, who));
+        if (!base) return scratch.ptr ? fail(SWC_HIP_EINVAL, "%s: scratch region too small for %zu groups", who, group)
+                                      : SWC_HIP_ERUNTIME;
+        float *masked = reinterpret_cast<float *>(base);
+        const unsigned blocks = ceil_div((size_t)g.OC * g.K, 256);
+        mask_filter_groups<<<blocks > 16384 ? 16384 : blocks, 256, 0, stream()>>>(masked, filter, g.OC, g.kh * g.kw, g.C,
+                                                                                 (int)group);
+        SWC_LAUNCH_CHECK();
+        return conv_dispatch(who, output, input, masked, bias, odims, idims, fdims, kernels, strides, pads, 1, ep_in,
+                             bias_optional, ConvScratch{reinterpret_cast<float *>(base + f_b), need - f_b});
+    }
     Epilogue ep = ep_in;
     ep.bias = bias;
     const bool vec = (g.C % 4 == 0) && aligned16(input) && aligned16(filter);
@@ -1499,13 +1534,15 @@ int swc_hip_conv2dFused_f(float *output, const float *input, const float *filter
 }
 
 size_t swc_hip_conv2d_workspace_bytes(const size_t *odims, const size_t *idims, const size_t *fdims,
-                                      const size_t *kernels, const size_t *strides, const size_t *pads) {
-    if (!ready() || check_conv_dims("swc_hip_conv2d_workspace_bytes", odims, idims, fdims, kernels, strides, pads, 1))
+                                      const size_t *kernels, const size_t *strides, const size_t *pads, size_t group) {
+    if (!ready() ||
+        check_conv_dims("swc_hip_conv2d_workspace_bytes", odims, idims, fdims, kernels, strides, pads, group, true))
         return 0;
     const ConvGeom g = make_geom(odims, idims, fdims, kernels, strides, pads);
     if (g.M == 0 || g.OC == 0) return 0;
-    if (g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0) return 0;
-    return conv_total_scratch(g, nullptr, nullptr);   // (tensors of a generated program are 256-byte aligned)
+    const size_t masked = group > 1 ? align256((size_t)g.OC * g.K * 4) : 0;
+    if (g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0) return masked;
+    return masked + conv_total_scratch(g, nullptr, nullptr);   // (tensors of a generated program are 256-byte aligned)
 }
 
 int swc_hip_conv2dGrad_f(float *inputG, float *filterG, float *biasG, const float *outputG, const float *input,

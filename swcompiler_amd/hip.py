@@ -101,7 +101,7 @@ def load_library():
         "swc_hip_host_malloc": (vp, [sz]),
         "swc_hip_host_free": (i32, [vp]),
         "swc_hip_gemm_workspace_bytes": (sz, [i32, i32, i32]),
-        "swc_hip_conv2d_workspace_bytes": (sz, [szp] * 6),
+        "swc_hip_conv2d_workspace_bytes": (sz, [szp] * 6 + [sz]),
         "swc_hip_matrixTrans_f": (i32, [i32, i32, vp, i32, vp, i32]),
         "swc_hip_matrixTanhGrad_f": (i32, [i32, i32, vp, i32, vp, i32, vp, i32]),
         "swc_hip_matrixSoftmaxWithLoss_f": (i32, [i32, i32, vp, i32, vp, i32, vp, vp]),
@@ -487,11 +487,11 @@ class SwcHip:
         """scratch bytes an m x n x k FC/GEMM call uses on this device (0 unless it is split over K)"""
         return int(self.lib.swc_hip_gemm_workspace_bytes(m, n, k))
 
-    def conv2d_workspace_bytes(self, xshape, fshape, strides=(1, 1), pads=(0, 0, 0, 0)):
+    def conv2d_workspace_bytes(self, xshape, fshape, strides=(1, 1), pads=(0, 0, 0, 0), group=1):
         """scratch bytes a conv2d call of these shapes uses on this device (0 if every tile is computed whole)"""
         odims = pool_out_dims(xshape, fshape[1:3], strides, pads)[:3] + (fshape[0],)
         return int(self.lib.swc_hip_conv2d_workspace_bytes(_dims(odims), _dims(xshape), _dims(fshape), _dims(fshape[1:3]),
-                                                           _dims(strides), _dims(pads)))
+                                                           _dims(strides), _dims(pads), group))
 
     def set_workspace(self, arr):
         """give the library a DeviceArray to use as scratch (None: its own buffer again)"""

@@ -86,7 +86,8 @@ void HipCodegen::emitWorkspace() {
             q << "{\n"
               << arrayDef("o", y->getDims()) << arrayDef("i", T(0)->getDims()) << arrayDef("f", T(1)->getDims())
               << arrayDef("k", conv->getKernels()) << arrayDef("s", conv->getStrides()) << arrayDef("p", conv->getPads())
-              << "gpu0_ws_bytes = std::max(gpu0_ws_bytes, swc_hip_conv2d_workspace_bytes(o, i, f, k, s, p));\n}\n";
+              << "gpu0_ws_bytes = std::max(gpu0_ws_bytes, swc_hip_conv2d_workspace_bytes(o, i, f, k, s, p, "
+              << conv->getGroup() << "));\n}\n";
         } else {
             continue;
         }

@@ -159,7 +159,7 @@ def test_hip_program_structure_and_build(gen, tmp_path):
     assert mlp.index("swc_hip_set_workspace(gpu0_ws, gpu0_ws_bytes)") < mlp.index("// call op routine functions")
     assert mlp.index("swc_hip_set_workspace(nullptr, 0)") < mlp.index("swc_hip_free(gpu0_ws)")
     # ... and of its convolutions: one query per conv, with the conv's own shape arrays
-    assert code.count("swc_hip_conv2d_workspace_bytes(o, i, f, k, s, p)") == 4
+    assert code.count("swc_hip_conv2d_workspace_bytes(o, i, f, k, s, p, 1)") == 4
     assert "const size_t o[] = {2, 56, 56, 64};" in code and "const size_t f[] = {128, 3, 3, 64};" in code
     assert code.index("swc_hip_set_workspace(gpu0_ws, gpu0_ws_bytes)") < code.index("// call op routine functions")
     lenet = generate(gen, "cfg3", "hip", tmp_path, 4)

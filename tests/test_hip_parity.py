@@ -215,11 +215,62 @@ def test_conv_golden(rt, golden, tag):
     assert scaled_err(got, golden[f"conv_{tag}_y"], mag) < TOL
 
 
-def test_conv_rejects_groups(rt):
+GROUPED_CONV_CASES = [((2, 9, 9, 8), (8, 3, 3, 8), (1, 1), (1, 1, 1, 1), 2),          # few channels, MFMA path
+                      ((3, 14, 14, 64), (96, 3, 3, 64), (1, 1), (1, 1, 1, 1), 4),     # direct-to-LDS path
+                      ((2, 7, 7, 16), (16, 3, 3, 16), (2, 2), (1, 1, 1, 1), 16),      # one channel per group
+                      ((2, 10, 10, 6), (9, 3, 3, 6), (1, 1), (0, 0, 0, 0), 3),        # padded-channel path
+                      ((4, 12, 12, 2), (4, 5, 5, 2), (1, 1), (2, 2, 2, 2), 2)]        # the direct kernel
+
+
+@pytest.mark.parametrize("idims,fdims,strides,pads,group", GROUPED_CONV_CASES)
+def test_conv_with_groups(rt, oracle, idims, fdims, strides, pads, group):
+    """group > 1 as conv2d_f indexes it (kernels.h:196-238): the filter keeps all iC channels per tap and output
+    channel co reads the channels of its group only."""
+    rng = np.random.default_rng(sum(idims) + sum(fdims) + group)
+    b = rng.integers(-4, 5, fdims[0]).astype(np.float32)
+    x = rng.integers(-4, 5, idims).astype(np.float32)
+    f = rng.integers(-4, 5, fdims).astype(np.float32)
+    got = rt.conv2d(*up(rt, x, f, b), fdims[1:3], strides, pads, group=group).numpy()
+    assert_bit_exact(got, oracle.conv2d(x, f, b, fdims[1:3], strides, pads, group), "grouped conv, integer-valued")
+    xr = rng.standard_normal(idims).astype(np.float32)
+    fr = rng.standard_normal(fdims).astype(np.float32)
+    got = rt.conv2d(*up(rt, xr, fr, b), fdims[1:3], strides, pads, group=group, relu=True).numpy()
+    want = oracle.relu(oracle.conv2d(xr, fr, b, fdims[1:3], strides, pads, group))
+    scale = oracle.conv2d(np.abs(xr), np.abs(fr), np.abs(b), fdims[1:3], strides, pads, group)
+    assert np.max(np.abs(got - want) / scale) < TOL
+    # the result does not depend on the filter channels outside the group
+    f2 = f.copy()
+    cg, ocg = idims[3] // group, fdims[0] // group
+    for co in range(fdims[0]):
+        g = co // ocg
+        f2[co, :, :, :g * cg] = 99
+        f2[co, :, :, (g + 1) * cg:] = -99
+    assert_bit_exact(rt.conv2d(*up(rt, x, f2, b), fdims[1:3], strides, pads, group=group).numpy(),
+                     oracle.conv2d(x, f, b, fdims[1:3], strides, pads, group), "channels outside the group")
+
+
+def test_conv_groups_in_a_caller_workspace_and_error_paths(rt, oracle):
     from swcompiler_amd.hip import SwcHipError
-    x, f, b = up(rt, np.zeros((1, 4, 4, 4), np.float32), np.zeros((4, 1, 1, 4), np.float32), np.zeros(4, np.float32))
+    idims, fdims, strides, pads, group = GROUPED_CONV_CASES[1]
+    need = rt.conv2d_workspace_bytes(idims, fdims, strides, pads, group)
+    assert need >= int(np.prod(fdims)) * 4 and need >= rt.conv2d_workspace_bytes(idims, fdims, strides, pads)
+    rng = np.random.default_rng(77)
+    x = rng.integers(-4, 5, idims).astype(np.float32)
+    f = rng.integers(-4, 5, fdims).astype(np.float32)
+    b = rng.integers(-4, 5, fdims[0]).astype(np.float32)
+    ws = rt.empty((need // 4,))
+    try:
+        rt.set_workspace(ws)
+        assert_bit_exact(rt.conv2d(*up(rt, x, f, b), fdims[1:3], strides, pads, group=group).numpy(),
+                         oracle.conv2d(x, f, b, fdims[1:3], strides, pads, group), "groups, caller workspace")
+    finally:
+        rt.sync()
+        rt.set_workspace(None)
+    z = up(rt, np.zeros((1, 4, 4, 4), np.float32), np.zeros((4, 1, 1, 4), np.float32), np.zeros(4, np.float32))
     with pytest.raises(SwcHipError, match="group"):
-        rt.conv2d(x, f, b, group=2)
+        rt.conv2d(*z, group=3)          # divides neither channel count
+    with pytest.raises(SwcHipError, match="group"):
+        rt.conv2dGrad(z[0], z[1], rt.upload(np.zeros((1, 4, 4, 4), np.float32)), group=2)   # gradients: one group only
 
 
 # ------------------------------------------------------- batchnorm / pool

@@ -120,6 +120,22 @@ def test_relu_add_bias_specials(oracle):
     assert_bit_exact(oracle.batchedadd(m, np.array([1, 2, 3, 4], np.float32)), m + np.array([1, 2, 3, 4], np.float32), "batchedadd")
 
 
+def test_conv_groups_are_independent_convolutions(oracle):
+    """A convolution in G groups equals G separate one-group convolutions over the channel slices, each with the
+    filter's slice of the same channels (the filter keeps all iC channels per tap: kernels.h:208-211)."""
+    rng = np.random.default_rng(12)
+    idims, fdims, group = (2, 7, 6, 6), (4, 3, 3, 6), 2
+    x = rng.standard_normal(idims).astype(np.float32)
+    f = rng.standard_normal(fdims).astype(np.float32)
+    b = rng.standard_normal(fdims[0]).astype(np.float32)
+    got = oracle.conv2d(x, f, b, (3, 3), (1, 1), (1, 1, 1, 1), group)
+    cg, ocg = idims[3] // group, fdims[0] // group
+    for g in range(group):
+        cs, os_ = slice(g * cg, (g + 1) * cg), slice(g * ocg, (g + 1) * ocg)
+        part = oracle.conv2d(x[..., cs], f[os_][..., cs], b[os_], (3, 3), (1, 1), (1, 1, 1, 1))
+        assert_bit_exact(got[..., os_], part, f"group {g}")
+
+
 def test_accuracy_counts(oracle):
     """kernels.h:615-627: hits and rows accumulate over calls; a label listed twice in a row counts once."""
     pred = np.array([[3, 1], [2, 2], [0, 4], [7, 7]], np.int32)

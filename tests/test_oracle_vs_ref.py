@@ -36,6 +36,15 @@ def test_conv(oracle, ref):
         b = rng.standard_normal(fdims[0]).astype(np.float32)
         assert_bit_exact(oracle.conv2d(x, f, b, fdims[1:3], s, p),
                          ref.conv2d(x, f, b, fdims[1:3], s, p), f"conv {idims} {fdims}")
+    # more than one group: the filter keeps all iC channels per tap, each output channel reads its group's
+    for idims, fdims, s, p, group in [((2, 9, 9, 8), (6, 3, 3, 8), (1, 1), (1, 1, 1, 1), 2),
+                                      ((1, 7, 8, 12), (12, 3, 2, 12), (2, 1), (0, 1, 0, 1), 12),
+                                      ((2, 6, 6, 6), (9, 1, 1, 6), (1, 1), (0, 0, 0, 0), 3)]:
+        x = rng.standard_normal(idims).astype(np.float32)
+        f = rng.standard_normal(fdims).astype(np.float32)
+        b = rng.standard_normal(fdims[0]).astype(np.float32)
+        assert_bit_exact(oracle.conv2d(x, f, b, fdims[1:3], s, p, group),
+                         ref.conv2d(x, f, b, fdims[1:3], s, p, group), f"conv {idims} {fdims} in {group} groups")
 
 
 def test_maxpool(oracle, ref):
