@@ -26,7 +26,8 @@ struct State {
     hipEvent_t slots[kEventSlots] = {};
     bool capturing = false;
     char arch[64] = "";
-    // workspace of the ops that need one (conv2dGrad_f, matrixSoftmaxWithLoss_f)
+    // scratch memory of the ops that need some (products and convolutions cut along K, padded or masked operand
+    // copies, conv2dGrad_f, matrixSoftmaxWithLoss_f): the caller's (swc_hip_set_workspace) or the library's own
     void *ws = nullptr;
     size_t ws_bytes = 0;
     bool ws_owned = false;
@@ -136,6 +137,13 @@ int swc_hip_shutdown(void) {
     g.ws_owned = false;
     (void)hipEventDestroy(g.t0);
     (void)hipEventDestroy(g.t1);
+    for (hipEvent_t &e : g.slots)
+        if (e) {
+            (void)hipEventDestroy(e);
+            e = nullptr;
+        }
+    g.capturing = false;
+    g.last_ms = -1.f;
     (void)hipStreamDestroy(g.own);
     g.own = g.cur = nullptr;
     g.t0 = g.t1 = nullptr;

@@ -28,6 +28,7 @@
 
 #include "../src/devices/HipDevice.h"
 #include "../src/codegen/Codegen.h"
+#include "../src/importer/Caffe2Importer.h"
 #include "../src/engine/Engine.h"
 
 #endif

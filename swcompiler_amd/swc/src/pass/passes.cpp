@@ -294,9 +294,14 @@ void DeviceMemoryLoweringPass::run() {
         if (!onGpu(t)) {
             // 2. host tensor read by GPU ops: device twin + Scatter
             std::vector<IRNode *> gpuReaders;
-            for (IRNode *c : t->getChildNodes())
+            for (IRNode *c : t->getChildNodes()) {
+                // the mask operand of a Dropout node is not read at inference: it needs no device copy
+                if (c->nodeType() == OP_NODE && static_cast<OpNode *>(c)->getOp()->getOpName() == "Dropout" &&
+                    c->parentNum() > 1 && c->getParentNode(1) == t && c->getParentNode(0) != t)
+                    continue;
                 if (onGpu(c) && std::find(gpuReaders.begin(), gpuReaders.end(), c) == gpuReaders.end())
                     gpuReaders.push_back(c);
+            }
             if (gpuReaders.empty()) continue;
             auto *twin = new TensorNode(t->name() + "_dev", t->getTensor()->clone());
             twin->getTensor()->setTensorInit(TensorInitType::NONE);
@@ -347,6 +352,34 @@ void DeviceMemoryLoweringPass::run() {
     }
     _graph->findInOut();
     _graph->updateTopology();
+
+    // 4. a device op that reads nothing but uploaded parameters (the layout change of an imported weight) has
+    //    the same result in every iteration: it runs once, after the uploads, like them
+    for (int i = 0; i < _graph->topologyNum(); ++i)
+        for (int j = 0; j < _graph->getNumInTopoLevel(i); ++j) {
+            IRNode *node = _graph->getNodeInTopo(i, j);
+            if (node->nodeType() != OP_NODE || !onGpu(node)) continue;
+            auto *op = static_cast<OpNode *>(node);
+            const std::string type = op->getOp()->getOpName();
+            if (op->isRunOnce() || type == "Scatter" || type == "Gather" || type == "Accuracy" || op->parentNum() == 0) continue;
+            bool constant = true;
+            for (IRNode *p : op->getParentNodes()) {
+                auto *pt = static_cast<TensorNode *>(p);
+                const bool fromRunOnce = pt->parentNum() == 1 && static_cast<OpNode *>(pt->getParentNode(0))->isRunOnce() &&
+                                         pt->getTensor()->getTensorInitType() == TensorInitType::PARENTOP;
+                constant = constant && fromRunOnce && pt->childNum() >= 1;
+            }
+            if (!constant) continue;
+            bool plainResults = true;   // results that are graph outputs or shared with another node stay per-iteration
+            for (IRNode *c : op->getChildNodes())
+                plainResults = plainResults && !c->getLabel()->getIsOut() &&
+                               static_cast<TensorNode *>(c)->getTensor()->getTensorInitType() == TensorInitType::NONE;
+            if (!plainResults) continue;
+            op->setRunOnce();
+            for (IRNode *c : op->getChildNodes())
+                static_cast<TensorNode *>(c)->getTensor()->setTensorInit(TensorInitType::PARENTOP);
+            ++hoisted_;
+        }
 }
 
 } // namespace pass

@@ -4,7 +4,7 @@
 // the reference's test/engine/testEngineMLPInfer.cpp.
 //
 //   genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse|graph]
-//   model: mnist8 | mnist_loader | nchw | manual | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
+//   model: mnist8 | mnist_loader | nchw | manual | caffe2 | caffe2txt | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
 //   mnist_loader: [batch] is the number of records in mnist_labels_images.bin
 //
 // Every parameter/input tensor is initialised from "<name>.bin" in the
@@ -348,6 +348,30 @@ int main(int argc, char **argv) {
             out = pool(graph, "pool", h);
             graph->initTensorNodes();
         }
+    } else if (model == "caffe2" || model == "caffe2txt") {
+        // the reference's test/importer/testResnetImport.cpp: the caller defines the data tensor in NHWC, the
+        // network and its weights come from a Caffe2 predict_net / init_net pair in the current directory
+        // (binary .pb, or .pbtxt for "caffe2txt"), ArgMax(3) + a Debug print follow the softmax
+        const size_t b = batch ? batch : 2;
+        vector<TensorNode *> udef;
+        auto *data = new TensorNode("gpu_0/data", new Tensor({b, 12, 12, 3}));
+        data->getTensor()->setTensorInit(TensorInitType::FILE, "data.bin");
+        udef.push_back(data);
+        const string ext = model == "caffe2" ? ".pb" : ".pbtxt";
+        Caffe2Importer importer(graph, "predict_net" + ext, "init_net" + ext, udef, "weights");
+        auto *softmax_t = static_cast<TensorNode *>(graph->getNodeByName("gpu_0/softmax"));
+        if (!softmax_t) {
+            cerr << "gpu_0/softmax not found\n";
+            return 2;
+        }
+        auto *argmax_o = new OpNode("argmax", new ArgMaxOp(3));
+        argmax_o->exlinkUpperNode(softmax_t);
+        auto *top3_t = new TensorNode("top3", new Tensor({b, 3}, DataType::Int32_t), argmax_o);
+        auto *print_o = new OpNode("print", new DebugOp());
+        print_o->exlinkUpperNode(top3_t);
+        graph->pushOpNode(argmax_o, print_o);
+        graph->pushTensorNode(top3_t);
+        graph->addLogicalOutNodes(softmax_t, top3_t);
     } else {
         cerr << "unknown model " << model << "\n";
         return 2;

@@ -1,0 +1,266 @@
+"""Caffe2 import (reference: src/importer/Caffe2Importer.cpp, test/importer/testResnetImport.cpp).
+
+The reference's own tests import ResNet50 / VGG19 / LeNet files that it downloads; none is in the reference
+tree.  Here a small residual network is written in the Caffe2 file format by the encoder below (binary wire
+format as protobuf serialises proto2 messages, and the text format), imported through the SWC API, compiled
+for the CPU and the HIP target, and checked against the same network computed with the oracle's kernels.
+"""
+import os
+import struct
+import subprocess
+
+import numpy as np
+import pytest
+
+from tests.test_codegen import GEN, SWC, TOL, build_cpu, build_hip, generate
+from tests.util import assert_bit_exact, rel_err
+
+
+@pytest.fixture(scope="module")
+def gen():
+    if not os.path.exists(GEN):
+        subprocess.check_call(["make", "-C", SWC, "-j8"], stdout=subprocess.DEVNULL)
+    return GEN
+
+
+# ------------------------------------------------ the Caffe2 file format, written by hand
+def varint(n):
+    n &= (1 << 64) - 1          # negative int64 values take ten bytes
+    out = bytearray()
+    while True:
+        out.append((n & 0x7f) | (0x80 if n > 0x7f else 0))
+        n >>= 7
+        if not n:
+            return bytes(out)
+
+
+def tag(field, wire_type):
+    return varint(field << 3 | wire_type)
+
+
+def delimited(field, payload):
+    return tag(field, 2) + varint(len(payload)) + payload
+
+
+def enc_arg(name, value, packed=False):
+    """Argument (caffe2.proto:152-166): name=1, f=2, i=3, s=4, floats=5, ints=6"""
+    out = delimited(1, name.encode())
+    if isinstance(value, float):
+        out += tag(2, 5) + struct.pack("<f", value)
+    elif isinstance(value, int):
+        out += tag(3, 0) + varint(value)
+    elif isinstance(value, str):
+        out += delimited(4, value.encode())
+    elif isinstance(value, np.ndarray) and value.dtype == np.float32:
+        if packed:
+            out += delimited(5, value.astype("<f4").tobytes())
+        else:
+            out += b"".join(tag(5, 5) + struct.pack("<f", v) for v in value.ravel())
+    else:                                                  # list of ints
+        if packed:
+            out += delimited(6, b"".join(varint(int(v)) for v in value))
+        else:
+            out += b"".join(tag(6, 0) + varint(int(v)) for v in value)
+    return out
+
+
+def enc_op(op, packed=False):
+    """OperatorDef (caffe2.proto:208-268): input=1, output=2, name=3, type=4, arg=5 (+ engine=7, skipped by the importer)"""
+    out = b"".join(delimited(1, s.encode()) for s in op["input"])
+    out += b"".join(delimited(2, s.encode()) for s in op["output"])
+    out += delimited(3, b"") + delimited(4, op["type"].encode())
+    out += b"".join(delimited(5, enc_arg(k, v, packed)) for k, v in op.get("arg", {}).items())
+    return out + delimited(7, b"CUDNN") + tag(9, 0) + varint(0)
+
+
+def enc_net(name, ops, packed=False):
+    """NetDef (caffe2.proto:270-309): name=1, op=2, external_input=7"""
+    return delimited(1, name.encode()) + b"".join(delimited(2, enc_op(o, packed)) for o in ops) + delimited(7, b"gpu_0/data")
+
+
+def text_net(name, ops):
+    def q(s):
+        return '"' + s.replace("\\", "\\\\").replace('"', '\\"') + '"'
+    lines = [f"name: {q(name)}  # written by the test"]
+    for o in ops:
+        lines.append("op {")
+        lines += [f"  input: {q(s)}" for s in o["input"]] + [f"  output: {q(s)}" for s in o["output"]]
+        lines += ['  name: ""', f"  type: {q(o['type'])}"]
+        for k, v in o.get("arg", {}).items():
+            lines.append("  arg {")
+            lines.append(f"    name: {q(k)}")
+            if isinstance(v, float):
+                lines.append(f"    f: {v!r}")
+            elif isinstance(v, int):
+                lines.append(f"    i: {v}")
+            elif isinstance(v, str):
+                lines.append(f"    s: {q(v)}")
+            elif isinstance(v, np.ndarray):
+                lines += [f"    floats: {float(x)!r}" for x in v.ravel()]   # repr of the float32 value as a double: exact
+            else:
+                lines += [f"    ints: {int(x)}" for x in v]
+            lines.append("  }")
+        lines += ['  engine: "CUDNN"', "  device_option { device_type: 1 cuda_gpu_id: 0 }", "}"]
+    lines.append('external_input: "gpu_0/data"')
+    return "\n".join(lines) + "\n"
+
+
+# ------------------------------------------------ the network
+def make_weights():
+    rng = np.random.default_rng(2019)
+    f32 = lambda a: np.asarray(a, np.float32)
+    w = {
+        "gpu_0/conv1_w": f32(rng.standard_normal((8, 3, 3, 3)) / 5),      # OIHW, as Caffe2 stores them
+        "gpu_0/conv1_b": f32(rng.standard_normal(8) / 10),
+        "gpu_0/res_w": f32(rng.standard_normal((8, 8, 3, 3)) / 8),
+        "gpu_0/pred_w": f32(rng.standard_normal((10, 72)) / 8),            # [out, in], in = (c, h, w) flattened
+        "gpu_0/pred_b": f32(rng.standard_normal(10) / 10),
+    }
+    for bn in ("gpu_0/conv1_bn", "gpu_0/res_bn"):
+        w[bn + "_s"] = f32(rng.uniform(0.5, 1.5, 8))
+        w[bn + "_b"] = f32(rng.standard_normal(8) / 10)
+        w[bn + "_rm"] = f32(rng.standard_normal(8) / 10)
+        w[bn + "_riv"] = f32(rng.uniform(0.5, 2.0, 8))
+    return w
+
+
+def make_nets(weights):
+    init = [dict(type="GivenTensorFill", input=[], output=[k], arg=dict(shape=list(v.shape), values=v))
+            for k, v in weights.items()]
+    init.append(dict(type="ConstantFill", input=[], output=["gpu_0/data"], arg=dict(shape=[1], value=0.0)))   # the caller's wins
+    g = "gpu_0/"
+    bn = lambda x: [g + x + s for s in ("_s", "_b", "_rm", "_riv")]
+    predict = [
+        dict(type="Conv", input=[g + "data", g + "conv1_w", g + "conv1_b"], output=[g + "conv1"],
+             arg=dict(kernel=3, pad=1, stride=1, order="NCHW", exhaustive_search=0)),
+        dict(type="SpatialBN", input=[g + "conv1"] + bn("conv1_bn"), output=[g + "conv1_bn"],
+             arg=dict(epsilon=float(np.float32(1e-5)), is_test=1, order="NCHW")),
+        dict(type="Relu", input=[g + "conv1_bn"], output=[g + "conv1_bn"]),                      # in place
+        dict(type="MaxPool", input=[g + "conv1_bn"], output=[g + "pool1"], arg=dict(kernel=2, stride=2, order="NCHW")),
+        dict(type="Conv", input=[g + "pool1", g + "res_w"], output=[g + "res"],                    # no bias blob
+             arg=dict(kernels=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1])),
+        dict(type="SpatialBN", input=[g + "res"] + bn("res_bn"), output=[g + "res_bn"], arg=dict(is_test=1)),
+        dict(type="Sum", input=[g + "res_bn", g + "pool1"], output=[g + "res_bn"]),                # in place
+        dict(type="Relu", input=[g + "res_bn"], output=[g + "res_bn"]),
+        dict(type="AveragePool", input=[g + "res_bn"], output=[g + "pool2"], arg=dict(kernel_h=2, kernel_w=2, stride_h=2, stride_w=2)),
+        dict(type="Dropout", input=[g + "pool2"], output=[g + "drop"], arg=dict(ratio=0.5, is_test=1)),
+        dict(type="FC", input=[g + "drop", g + "pred_w", g + "pred_b"], output=[g + "pred"]),
+        dict(type="Softmax", input=[g + "pred"], output=[g + "softmax"]),
+    ]
+    return predict, init
+
+
+def expected(oracle, data, w):
+    g = "gpu_0/"
+    ohwi = lambda f: oracle.transpose(f, (0, 2, 3, 1))
+    bn = lambda x, p: oracle.batchnormalization(x, w[g + p + "_rm"], w[g + p + "_riv"], w[g + p + "_s"], w[g + p + "_b"],
+                                                float(np.float32(1e-5)))
+    y = oracle.conv2d(data, ohwi(w[g + "conv1_w"]), w[g + "conv1_b"], (3, 3), (1, 1), (1, 1, 1, 1))
+    pool1 = oracle.maxpool(oracle.relu(bn(y, "conv1_bn")), (2, 2), (2, 2))
+    r = oracle.conv2d(pool1, ohwi(w[g + "res_w"]), np.zeros(8, np.float32), (3, 3), (1, 1), (1, 1, 1, 1))
+    r = oracle.relu(oracle.vecAdd(bn(r, "res_bn").ravel(), pool1.ravel()).reshape(pool1.shape))
+    pool2 = oracle.avgpool(r, (2, 2), (2, 2))
+    flat = oracle.transpose(pool2, (0, 3, 1, 2)).reshape(data.shape[0], -1)      # (c, h, w) order, as trained
+    pred = oracle.fcbias(flat, oracle.transpose(w[g + "pred_w"], (1, 0)), w[g + "pred_b"])
+    prob = oracle.matrixSoftmax(pred)
+    return prob, oracle.argMax(prob, 3)
+
+
+def write_model(tmp_path, binary, packed=False):
+    w = make_weights()
+    predict, init = make_nets(w)
+    if binary:
+        open(os.path.join(tmp_path, "predict_net.pb"), "wb").write(enc_net("mini_resnet", predict, packed))
+        open(os.path.join(tmp_path, "init_net.pb"), "wb").write(enc_net("mini_resnet_init", init, packed))
+    else:
+        open(os.path.join(tmp_path, "predict_net.pbtxt"), "w").write(text_net("mini_resnet", predict))
+        open(os.path.join(tmp_path, "init_net.pbtxt"), "w").write(text_net("mini_resnet_init", init))
+    data = np.random.default_rng(7).standard_normal((2, 12, 12, 3)).astype(np.float32)
+    data.tofile(os.path.join(tmp_path, "data.bin"))
+    return w, data
+
+
+def read_outputs(tmp_path, suffix):
+    prob = np.fromfile(os.path.join(tmp_path, f"gpu_0_softmax{suffix}.bin"), np.float32).reshape(2, 10)
+    top3 = np.fromfile(os.path.join(tmp_path, f"top3{suffix}.bin"), np.int32).reshape(2, 3)
+    return prob, top3
+
+
+# ------------------------------------------------ tests
+@pytest.mark.parametrize("binary,packed", [(True, False), (True, True), (False, False)])
+def test_import_cpu_program(gen, oracle, tmp_path, binary, packed):
+    w, data = write_model(tmp_path, binary, packed)
+    code = generate(gen, "caffe2" if binary else "caffe2txt", "cpu", tmp_path, 2)
+    # the graph the reference's importer builds: a transpose per Conv / FC weight and one in front of the FC
+    assert code.count("transpose4d_f(") == 3 and code.count("transpose2d_f(") == 1
+    assert code.count("conv2d_f(") == 2 and code.count("batchnormalization_f(") == 2 and code.count("relu_f(") == 2
+    assert "vecAdd_f(" in code and "maxpool_f(" in code and "avgpool_f(" in code and "matrixSoftmax_f(" in code
+    # every weight blob became a raw fp32 file the program loads
+    for name, v in w.items():
+        path = os.path.join(tmp_path, "weights", name.replace("/", "_") + ".bin")
+        assert_bit_exact(np.fromfile(path, np.float32).reshape(v.shape), v, name)
+        assert f'"weights/{name.replace("/", "_")}.bin"' in code
+    out = subprocess.run([build_cpu(tmp_path)], cwd=tmp_path, check=True, capture_output=True, text=True).stdout
+    prob, top3 = read_outputs(tmp_path, "")
+    want_prob, want_top3 = expected(oracle, data, w)
+    assert_bit_exact(prob, want_prob, "probabilities")
+    assert_bit_exact(top3, want_top3, "top-3")
+    assert [int(v) for v in out.split()[-6:]] == want_top3.ravel().tolist()      # the Debug print
+
+
+def test_text_and_binary_files_give_the_same_program(gen, tmp_path):
+    a, b = os.path.join(tmp_path, "a"), os.path.join(tmp_path, "b")
+    os.mkdir(a), os.mkdir(b)
+    write_model(a, True)
+    write_model(b, False)
+    assert generate(gen, "caffe2", "cpu", a, 2) == generate(gen, "caffe2txt", "cpu", b, 2)
+    assert generate(gen, "caffe2", "hip", a, 2) == generate(gen, "caffe2txt", "hip", b, 2)
+
+
+def test_import_hip_program_structure(gen, tmp_path):
+    write_model(tmp_path, True)
+    code = generate(gen, "caffe2", "hip", tmp_path, 2)
+    # conv+BN+ReLU and add+ReLU fuse; the weight transposes run once, before the op sequence
+    assert code.count("swc_hip_conv2dFused_f(") == 2 and "swc_hip_vecAddRelu_f(" in code
+    head, body = code.split("// call op routine functions")
+    assert head.count("swc_hip_transpose4d_f(") == 2 and head.count("swc_hip_transpose2d_f(") == 1
+    assert body.count("swc_hip_transpose4d_f(") == 1 and "swc_hip_transpose2d_f(" not in body
+    assert "swc_hip_matrixMatrixFCBiasSoftmax_f(2, 10, 72" in body
+    build_hip(tmp_path)
+
+
+@pytest.mark.parametrize("damage", ["unsupported op", "truncated", "missing blob", "value count"])
+def test_import_errors(gen, tmp_path, damage):
+    w = make_weights()
+    predict, init = make_nets(w)
+    if damage == "unsupported op":
+        predict.insert(3, dict(type="LRN", input=["gpu_0/conv1_bn"], output=["gpu_0/conv1_bn"]))
+        message = "unsupported Caffe2 operator LRN"
+    elif damage == "missing blob":
+        init = [o for o in init if o["output"] != ["gpu_0/res_w"]]
+        message = "blob gpu_0/res_w"
+    elif damage == "value count":
+        init[0]["arg"]["shape"] = [8, 3, 3, 4]
+        message = "216 values for a shape of 288 elements"
+    else:
+        message = "not a serialized NetDef"
+    pred_bytes = enc_net("mini", predict)
+    if damage == "truncated":
+        pred_bytes = pred_bytes[:len(pred_bytes) // 2 + 1]
+    open(os.path.join(tmp_path, "predict_net.pb"), "wb").write(pred_bytes)
+    open(os.path.join(tmp_path, "init_net.pb"), "wb").write(enc_net("mini_init", init))
+    r = subprocess.run([gen, "caffe2", "cpu", "2"], cwd=tmp_path, capture_output=True, text=True)
+    assert r.returncode != 0 and message in r.stderr + r.stdout
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("graph", [False, True])
+def test_import_hip_program(gen, oracle, tmp_path, graph):
+    print("case caffe2 import, graph =", graph, flush=True)
+    w, data = write_model(tmp_path, True)
+    generate(gen, "caffe2", "hip", tmp_path, 2, iters=3 if graph else 0, graph=graph)
+    subprocess.run([build_hip(tmp_path)], cwd=tmp_path, check=True, timeout=120, stdout=subprocess.DEVNULL)
+    prob, top3 = read_outputs(tmp_path, "_host")
+    want_prob, want_top3 = expected(oracle, data, w)
+    assert rel_err(prob, want_prob) < TOL
+    assert_bit_exact(top3, want_top3, "top-3")
