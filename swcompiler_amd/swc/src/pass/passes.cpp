@@ -353,31 +353,31 @@ void DeviceMemoryLoweringPass::run() {
     _graph->findInOut();
     _graph->updateTopology();
 
-    // 4. a device op that reads nothing but uploaded parameters (the layout change of an imported weight) has
-    //    the same result in every iteration: it runs once, after the uploads, like them
+    // 4. the layout change of a weight (the Transpose an importer puts behind a Conv or FC weight stored in
+    //    another order) has the same result in every iteration: it runs once, after the uploads, like them.
+    //    A weight is recognised by its use: an uploaded parameter whose transposed copy is read only as a
+    //    second or later operand (operand 0 carries the data).
     for (int i = 0; i < _graph->topologyNum(); ++i)
         for (int j = 0; j < _graph->getNumInTopoLevel(i); ++j) {
             IRNode *node = _graph->getNodeInTopo(i, j);
             if (node->nodeType() != OP_NODE || !onGpu(node)) continue;
             auto *op = static_cast<OpNode *>(node);
-            const std::string type = op->getOp()->getOpName();
-            if (op->isRunOnce() || type == "Scatter" || type == "Gather" || type == "Accuracy" || op->parentNum() == 0) continue;
-            bool constant = true;
-            for (IRNode *p : op->getParentNodes()) {
-                auto *pt = static_cast<TensorNode *>(p);
-                const bool fromRunOnce = pt->parentNum() == 1 && static_cast<OpNode *>(pt->getParentNode(0))->isRunOnce() &&
-                                         pt->getTensor()->getTensorInitType() == TensorInitType::PARENTOP;
-                constant = constant && fromRunOnce && pt->childNum() >= 1;
-            }
-            if (!constant) continue;
-            bool plainResults = true;   // results that are graph outputs or shared with another node stay per-iteration
-            for (IRNode *c : op->getChildNodes())
-                plainResults = plainResults && !c->getLabel()->getIsOut() &&
-                               static_cast<TensorNode *>(c)->getTensor()->getTensorInitType() == TensorInitType::NONE;
-            if (!plainResults) continue;
+            if (op->isRunOnce() || op->getOp()->getOpName() != "Transpose" || op->parentNum() != 1 || op->childNum() != 1)
+                continue;
+            auto *src = static_cast<TensorNode *>(op->getParentNode(0));
+            auto *dst = static_cast<TensorNode *>(op->getChildNode(0));
+            const bool uploaded = src->parentNum() == 1 && static_cast<OpNode *>(src->getParentNode(0))->isRunOnce() &&
+                                  src->getTensor()->getTensorInitType() == TensorInitType::PARENTOP;
+            if (!uploaded || dst->getLabel()->getIsOut() || dst->childNum() == 0 ||
+                dst->getTensor()->getTensorInitType() != TensorInitType::NONE)
+                continue;
+            bool weightOnly = true;
+            for (IRNode *reader : dst->getChildNodes())
+                weightOnly = weightOnly && reader->nodeType() == OP_NODE && onGpu(reader) && reader->parentNum() > 1 &&
+                             reader->getParentNode(0) != dst;
+            if (!weightOnly) continue;
             op->setRunOnce();
-            for (IRNode *c : op->getChildNodes())
-                static_cast<TensorNode *>(c)->getTensor()->setTensorInit(TensorInitType::PARENTOP);
+            dst->getTensor()->setTensorInit(TensorInitType::PARENTOP);
             ++hoisted_;
         }
 }

@@ -96,8 +96,8 @@ class HipFusionPass : public OptimizePass {
 // when the tensor is a parameter, i.e. has an initialiser and is not the
 // per-iteration data/label input); every GPU tensor that is a graph output or
 // is read by a host op (Debug, Accuracy) gets a host twin fed by a GatherOp.
-// A device op all of whose operands are uploaded parameters (the Transpose an
-// importer puts behind a weight) becomes run-once itself.
+// The Transpose an importer puts behind a weight (an uploaded parameter whose
+// transposed copy is read only as a second or later operand) becomes run-once itself.
 // After the pass the graph itself says where each buffer lives and where each
 // transfer happens; the code generator only walks it.
 class DeviceMemoryLoweringPass : public OptimizePass {
@@ -110,7 +110,7 @@ class DeviceMemoryLoweringPass : public OptimizePass {
     static bool runsOnGpu(const std::string &typeName);
     int scatterCount() const { return scatters_; }
     int gatherCount() const { return gathers_; }
-    int hoistedCount() const { return hoisted_; }   // device ops of parameters only, made run-once
+    int hoistedCount() const { return hoisted_; }   // weight transposes made run-once
 };
 
 } // namespace pass

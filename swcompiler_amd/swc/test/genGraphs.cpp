@@ -4,7 +4,7 @@
 // the reference's test/engine/testEngineMLPInfer.cpp.
 //
 //   genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse|graph]
-//   model: mnist8 | mnist_loader | nchw | manual | caffe2 | caffe2txt | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
+//   model: mnist8 | mnist_loader | nchw | manual | caffe2[txt][@image size] | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
 //   mnist_loader: [batch] is the number of records in mnist_labels_images.bin
 //
 // Every parameter/input tensor is initialised from "<name>.bin" in the
@@ -107,7 +107,8 @@ int main(int argc, char **argv) {
         cerr << "usage: genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse|graph]\n";
         return 2;
     }
-    const string model = argv[1], target = argv[2];
+    string model = argv[1];
+    const string target = argv[2];
     const size_t batch = argc > 3 ? strtoul(argv[3], nullptr, 10) : 0;
     const size_t iters = argc > 4 ? strtoul(argv[4], nullptr, 10) : 0;
     const bool nofuse = argc > 5 && string(argv[5]) == "nofuse";
@@ -348,13 +349,23 @@ int main(int argc, char **argv) {
             out = pool(graph, "pool", h);
             graph->initTensorNodes();
         }
-    } else if (model == "caffe2" || model == "caffe2txt") {
+    } else if (model.rfind("caffe2", 0) == 0) {
         // the reference's test/importer/testResnetImport.cpp: the caller defines the data tensor in NHWC, the
         // network and its weights come from a Caffe2 predict_net / init_net pair in the current directory
-        // (binary .pb, or .pbtxt for "caffe2txt"), ArgMax(3) + a Debug print follow the softmax
+        // (binary .pb, or .pbtxt for "caffe2txt"), ArgMax(3) + a Debug print follow the softmax.
+        // "caffe2@64": images of 64 x 64 (default 12 x 12), always 3 channels.
         const size_t b = batch ? batch : 2;
+        size_t hw = 12;
+        if (model.find('@') != string::npos) {
+            hw = stoul(model.substr(model.find('@') + 1));
+            model = model.substr(0, model.find('@'));
+        }
+        if (model != "caffe2" && model != "caffe2txt") {
+            cerr << "unknown model " << model << "\n";
+            return 2;
+        }
         vector<TensorNode *> udef;
-        auto *data = new TensorNode("gpu_0/data", new Tensor({b, 12, 12, 3}));
+        auto *data = new TensorNode("gpu_0/data", new Tensor({b, hw, hw, 3}));
         data->getTensor()->setTensorInit(TensorInitType::FILE, "data.bin");
         udef.push_back(data);
         const string ext = model == "caffe2" ? ".pb" : ".pbtxt";

@@ -166,6 +166,104 @@ def expected(oracle, data, w):
     return prob, oracle.argMax(prob, 3)
 
 
+def run_net(oracle, predict, w, data):
+    """The operators of a predict_net executed with the oracle's kernels: activations NHWC, weights as stored
+    (Conv OIHW, FC [out, in] over an NCHW-flattened input) — what the imported graph must compute."""
+    blobs = dict(w)
+    blobs["gpu_0/data"] = data
+    pair = lambda a, one, h, wd, lst, default: ((a[one],) * 2 if one in a else (a[h], a[wd]) if h in a else
+                                                tuple(a[lst]) if lst in a else default)
+    for op in predict:
+        a, x = op.get("arg", {}), [blobs[n] for n in op["input"]]
+        pads = (a["pad"],) * 4 if "pad" in a else tuple(a.get("pads", (0, 0, 0, 0)))
+        if op["type"] == "Conv":
+            f = oracle.transpose(x[1], (0, 2, 3, 1))
+            bias = x[2] if len(x) > 2 else np.zeros(f.shape[0], np.float32)
+            y = oracle.conv2d(x[0], f, bias, pair(a, "kernel", "kernel_h", "kernel_w", "kernels", f.shape[1:3]),
+                              pair(a, "stride", "stride_h", "stride_w", "strides", (1, 1)), pads)
+        elif op["type"] == "SpatialBN":
+            y = oracle.batchnormalization(x[0], x[3], x[4], x[1], x[2], a.get("epsilon", float(np.float32(1e-5))))
+        elif op["type"] == "Relu":
+            y = oracle.relu(x[0].ravel()).reshape(x[0].shape)
+        elif op["type"] == "Sum":
+            y = oracle.vecAdd(x[0].ravel(), x[1].ravel()).reshape(x[0].shape)
+        elif op["type"] in ("MaxPool", "AveragePool"):
+            k = pair(a, "kernel", "kernel_h", "kernel_w", "kernels", None)
+            if a.get("global_pooling"):
+                k = x[0].shape[1:3]
+            fn = oracle.maxpool if op["type"] == "MaxPool" else oracle.avgpool
+            y = fn(x[0], k, pair(a, "stride", "stride_h", "stride_w", "strides", (1, 1)), pads)
+        elif op["type"] == "Dropout":
+            y = x[0]
+        elif op["type"] == "FC":
+            flat = oracle.transpose(x[0], (0, 3, 1, 2)) if x[0].ndim == 4 else x[0]
+            y = oracle.fcbias(flat.reshape(flat.shape[0], -1), oracle.transpose(x[1], (1, 0)), x[2])
+        elif op["type"] == "Softmax":
+            y = oracle.matrixSoftmax(x[0])
+        else:
+            raise ValueError(op["type"])
+        blobs[op["output"][0]] = y
+    return blobs
+
+
+def make_resnet50(width=64, blocks=(3, 4, 6, 3), classes=1000, image=224, seed=50):
+    """ResNet-50 as the Caffe2 model zoo stores it (bias-free convolutions each followed by SpatialBN, in-place
+    Relu and Sum, stride on the first 1x1 of a stage, 3x3/2 max pooling with pad 1, average pooling over the last
+    map, FC, Softmax) with random weights; `width` = channels of the first stage's 3x3 (64 in the real model)."""
+    rng = np.random.default_rng(seed)
+    w, ops, g = {}, [], "gpu_0/"
+
+    def conv_bn(name, src, cin, cout, k, stride, relu):
+        w[g + name + "_w"] = (rng.standard_normal((cout, cin, k, k)) * np.sqrt(2.0 / (cin * k * k))).astype(np.float32)
+        ops.append(dict(type="Conv", input=[g + src, g + name + "_w"], output=[g + name],
+                        arg=dict(kernel=k, stride=stride, pad=k // 2, order="NCHW")))
+        bn = name + "_bn"
+        w[g + bn + "_s"] = rng.uniform(0.5, 1.0, cout).astype(np.float32)
+        w[g + bn + "_b"] = (rng.standard_normal(cout) * 0.1).astype(np.float32)
+        w[g + bn + "_rm"] = (rng.standard_normal(cout) * 0.1).astype(np.float32)
+        w[g + bn + "_riv"] = rng.uniform(0.5, 2.0, cout).astype(np.float32)
+        ops.append(dict(type="SpatialBN", input=[g + name] + [g + bn + s for s in ("_s", "_b", "_rm", "_riv")],
+                        output=[g + bn], arg=dict(epsilon=float(np.float32(1e-5)), is_test=1, order="NCHW")))
+        if relu:
+            ops.append(dict(type="Relu", input=[g + bn], output=[g + bn]))
+        return bn
+
+    x = conv_bn("conv1", "data", 3, width, 7, 2, True)
+    ops.append(dict(type="MaxPool", input=[g + x], output=[g + "pool1"], arg=dict(kernel=3, stride=2, pad=1)))
+    x, cin, hw = "pool1", width, (image + 6 - 7) // 2 + 1
+    hw = (hw + 2 - 3) // 2 + 1
+    for stage, n in enumerate(blocks):
+        mid, cout = width << stage, (width << stage) * 4
+        for b in range(n):
+            name = f"res{stage + 2}_{b}"
+            stride = 2 if stage > 0 and b == 0 else 1
+            short = x if (cin == cout and stride == 1) else conv_bn(name + "_branch1", x, cin, cout, 1, stride, False)
+            y = conv_bn(name + "_branch2a", x, cin, mid, 1, stride, True)
+            y = conv_bn(name + "_branch2b", y, mid, mid, 3, 1, True)
+            y = conv_bn(name + "_branch2c", y, mid, cout, 1, 1, False)
+            ops.append(dict(type="Sum", input=[g + y, g + short], output=[g + y]))
+            ops.append(dict(type="Relu", input=[g + y], output=[g + y]))
+            x, cin = y, cout
+            hw = (hw - 1) // stride + 1
+    ops.append(dict(type="AveragePool", input=[g + x], output=[g + "pool5"], arg=dict(kernel=hw, stride=1)))
+    w[g + "pred_w"] = (rng.standard_normal((classes, cin)) / np.sqrt(cin)).astype(np.float32)
+    w[g + "pred_b"] = (rng.standard_normal(classes) * 0.1).astype(np.float32)
+    ops.append(dict(type="FC", input=[g + "pool5", g + "pred_w", g + "pred_b"], output=[g + "pred"]))
+    ops.append(dict(type="Softmax", input=[g + "pred"], output=[g + "softmax"]))
+    init = [dict(type="GivenTensorFill", input=[], output=[k], arg=dict(shape=list(v.shape), values=v)) for k, v in w.items()]
+    return ops, init, w
+
+
+def write_resnet50(tmp_path, batch, **kw):
+    predict, init, w = make_resnet50(**kw)
+    open(os.path.join(tmp_path, "predict_net.pb"), "wb").write(enc_net("resnet50", predict, packed=True))
+    open(os.path.join(tmp_path, "init_net.pb"), "wb").write(enc_net("resnet50_init", init, packed=True))
+    image = kw.get("image", 224)
+    data = np.random.default_rng(11).standard_normal((batch, image, image, 3)).astype(np.float32)
+    data.tofile(os.path.join(tmp_path, "data.bin"))
+    return predict, w, data
+
+
 def write_model(tmp_path, binary, packed=False):
     w = make_weights()
     predict, init = make_nets(w)
@@ -180,9 +278,9 @@ def write_model(tmp_path, binary, packed=False):
     return w, data
 
 
-def read_outputs(tmp_path, suffix):
-    prob = np.fromfile(os.path.join(tmp_path, f"gpu_0_softmax{suffix}.bin"), np.float32).reshape(2, 10)
-    top3 = np.fromfile(os.path.join(tmp_path, f"top3{suffix}.bin"), np.int32).reshape(2, 3)
+def read_outputs(tmp_path, suffix, batch=2, classes=10):
+    prob = np.fromfile(os.path.join(tmp_path, f"gpu_0_softmax{suffix}.bin"), np.float32).reshape(batch, classes)
+    top3 = np.fromfile(os.path.join(tmp_path, f"top3{suffix}.bin"), np.int32).reshape(batch, 3)
     return prob, top3
 
 
@@ -203,6 +301,7 @@ def test_import_cpu_program(gen, oracle, tmp_path, binary, packed):
     out = subprocess.run([build_cpu(tmp_path)], cwd=tmp_path, check=True, capture_output=True, text=True).stdout
     prob, top3 = read_outputs(tmp_path, "")
     want_prob, want_top3 = expected(oracle, data, w)
+    assert_bit_exact(run_net(oracle, make_nets(w)[0], w, data)["gpu_0/softmax"], want_prob, "the two statements of the network")
     assert_bit_exact(prob, want_prob, "probabilities")
     assert_bit_exact(top3, want_top3, "top-3")
     assert [int(v) for v in out.split()[-6:]] == want_top3.ravel().tolist()      # the Debug print
@@ -264,3 +363,51 @@ def test_import_hip_program(gen, oracle, tmp_path, graph):
     want_prob, want_top3 = expected(oracle, data, w)
     assert rel_err(prob, want_prob) < TOL
     assert_bit_exact(top3, want_top3, "top-3")
+
+
+# A ResNet-50 of reduced width and resolution (all 16 bottleneck blocks, every layer type and stride of the real
+# one): 1/4 of the channels, 64 x 64 images.
+SMALL_RESNET = dict(width=16, classes=100, image=64)
+
+
+def test_resnet50_import_cpu_program(gen, oracle, tmp_path):
+    predict, w, data = write_resnet50(tmp_path, 1, **SMALL_RESNET)
+    code = generate(gen, "caffe2@64", "cpu", tmp_path, 1)
+    assert code.count("conv2d_f(") == 53 and code.count("batchnormalization_f(") == 53 and code.count("vecAdd_f(") == 16
+    subprocess.run([build_cpu(tmp_path)], cwd=tmp_path, check=True, stdout=subprocess.DEVNULL)
+    prob, top3 = read_outputs(tmp_path, "", 1, 100)
+    want = run_net(oracle, predict, w, data)["gpu_0/softmax"]
+    assert_bit_exact(prob, want, "probabilities")
+    assert_bit_exact(top3, oracle.argMax(want, 3), "top-3")
+
+
+@pytest.mark.gpu
+def test_resnet50_import_hip_program(gen, oracle, tmp_path):
+    print("case resnet50 import", flush=True)
+    predict, w, data = write_resnet50(tmp_path, 4, **SMALL_RESNET)
+    code = generate(gen, "caffe2@64", "hip", tmp_path, 4)
+    head, body = code.split("// call op routine functions")
+    # the 53 filter transposes and the FC weight's run once; in the op sequence only pool5 is reordered for the FC
+    assert head.count("swc_hip_transpose4d_f(") == 53 and head.count("swc_hip_transpose2d_f(") == 1
+    assert body.count("swc_hip_transpose4d_f(") == 1 and "swc_hip_conv2dFused_f(" not in head
+    assert body.count("swc_hip_conv2dFused_f(") == 53 and body.count("swc_hip_vecAddRelu_f(") == 16
+    subprocess.run([build_hip(tmp_path)], cwd=tmp_path, check=True, timeout=120, stdout=subprocess.DEVNULL)
+    prob, top3 = read_outputs(tmp_path, "_host", 4, 100)
+    want = run_net(oracle, predict, w, data)["gpu_0/softmax"]
+    assert rel_err(prob, want) < TOL
+    assert (top3[:, 0] == oracle.argMax(want, 1)[:, 0]).all()
+
+
+@pytest.mark.gpu
+def test_resnet50_full_size_hip_program(gen, oracle, tmp_path):
+    """All of ResNet-50 at its real size (25.6 M parameters, 224 x 224 images, 1000 classes), one image: the 7x7/2
+    first layer on padded channels, 1x1 and strided 1x1 convolutions, 3x3/2 pooling with padding, 7x7 average
+    pooling and a 2048 -> 1000 FC, against the oracle's run of the same network."""
+    print("case resnet50 full size", flush=True)
+    predict, w, data = write_resnet50(tmp_path, 1)
+    generate(gen, "caffe2@224", "hip", tmp_path, 1)
+    subprocess.run([build_hip(tmp_path)], cwd=tmp_path, check=True, timeout=120, stdout=subprocess.DEVNULL)
+    prob, top3 = read_outputs(tmp_path, "_host", 1, 1000)
+    want = run_net(oracle, predict, w, data)["gpu_0/softmax"]
+    assert rel_err(prob, want) < TOL
+    assert top3[0, 0] == int(np.argmax(want))
