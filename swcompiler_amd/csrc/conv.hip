@@ -434,10 +434,26 @@ __global__ __launch_bounds__(256) void conv_sk_finish(float *__restrict__ out, c
 // least one full round of whole tiles precedes them and they would fill less than half of the last round;
 // otherwise (small layers, nearly full last rounds) the pieces and the second kernel cost more than the idle
 // CUs (LeNet's 12x12x20 -> 50 layer: 20 us whole, 28 us cut).
+// A layer with fewer tiles than slots and a long K (the late stages of a residual network at a moderate
+// batch: 32 x 7 x 7 x 512 -> 512 has 200 tiles of 144 slices each) would leave CUs idle for its whole
+// duration: all of its tiles are cut, into as many shares as there are slots.
+constexpr int kShareAllMinSlices = 64;   // K >= 2048: below that the pieces and the second kernel cost what the idle CUs do
+int share_all_min_slices() {
+    if (const char *e = getenv("SWC_HIP_CONV_SHARE_ALL"))   // tuning: slices per tile from which a short layer is cut (0: never)
+        return atoi(e) > 0 ? atoi(e) : 1 << 30;
+    return kShareAllMinSlices;
+}
+
 SkPlan sk_plan(long tiles, int nk, int slots, bool allow_shared) {
     SkPlan p{(int)tiles, 0, 0, 0};
-    const long rest = tiles % slots;
-    if (!allow_shared || rest == 0 || tiles < slots || 2 * rest > slots) return p;
+    if (!allow_shared || tiles == 0) return p;
+    long rest = tiles % slots;
+    if (tiles < slots) {
+        if (nk < share_all_min_slices() || 4 * tiles > 3 * slots) return p;   // (a nearly full round: leave it)
+        rest = tiles;
+    } else if (rest == 0 || 2 * rest > slots) {
+        return p;
+    }
     const long units = rest * nk;
     long wgs = slots;
     if (units < 4 * wgs) wgs = units / 4;   // at least four slices per share: a piece costs a ring start and a tile store

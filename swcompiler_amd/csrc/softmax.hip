@@ -131,6 +131,60 @@ __global__ __launch_bounds__(256) void argmax_rows(const float *in, int *idx, in
     for (int t = 0; t < top_k; ++t) idx[(size_t)row * top_k + t] = (t < have) ? bi[t] : 0;
 }
 
+// The same for long rows (a thousand classes): a wavefront per row.  Lane l keeps the top_k of columns l, l+64,
+// ... as above; then top_k rounds pick the best head among the 64 lanes (descending (value, column)) and the
+// lane that held it moves on to its next entry.
+__device__ __forceinline__ bool goes_first(float v, int j, bool valid, float w, int i, bool wvalid) {
+    if (!wvalid) return valid;
+    if (!valid) return false;
+    return v > w || (v == w && j > i);
+}
+
+__global__ __launch_bounds__(256) void argmax_rows_wave(const float *in, int *idx, int m, int n, int top_k) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= m) return;   // whole wavefronts leave together
+    const float *src = in + (size_t)row * n;
+    float bv[kMaxTopK];
+    int bi[kMaxTopK];
+#pragma unroll
+    for (int t = 0; t < kMaxTopK; ++t) bv[t] = 0.f, bi[t] = 0;
+    int have = 0;
+    for (int j = lane; j < n; j += 64) {
+        const float v = src[j];
+        // position among the kept ones; (v, j) precedes an equal value (j is the larger column)
+        int pos = 0;
+#pragma unroll
+        for (int t = 0; t < kMaxTopK; ++t) pos += (t < have && !(v > bv[t] || v == bv[t])) ? 1 : 0;
+        if (pos >= top_k) continue;
+#pragma unroll
+        for (int t = kMaxTopK - 1; t > 0; --t)
+            if (t > pos) bv[t] = bv[t - 1], bi[t] = bi[t - 1];
+#pragma unroll
+        for (int t = 0; t < kMaxTopK; ++t)
+            if (t == pos) bv[t] = v, bi[t] = j;
+        if (have < top_k) ++have;
+    }
+    for (int t = 0; t < top_k; ++t) {
+        float v = bv[0];
+        int j = bi[0];
+        bool valid = have > 0;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float w = __shfl_xor(v, off);
+            const int i = __shfl_xor(j, off);
+            const bool wvalid = __shfl_xor((int)valid, off) != 0;
+            if (goes_first(w, i, wvalid, v, j, valid)) v = w, j = i, valid = wvalid;
+        }
+        if (lane == 0) idx[(size_t)row * top_k + t] = valid ? j : 0;
+        if (have > 0 && bi[0] == j) {   // this lane held the winner (columns are distinct across lanes): next entry
+#pragma unroll
+            for (int u = 0; u < kMaxTopK - 1; ++u) bv[u] = bv[u + 1], bi[u] = bi[u + 1];
+            --have;
+        }
+    }
+}
+
 // accuracy_i: one lane per row looks for its label among the row's n predictions; the workgroup's count of
 // hits and its row count go to the two counters with one integer atomic each, so repeated calls accumulate
 // exactly as the host loop does, in any order.
@@ -191,7 +245,8 @@ int swc_hip_argMax_i(const float *input, int *idx, int m, int n, int top_k) {
     SWC_ARG(input && idx && top_k <= n);
     if (top_k > kMaxTopK)
         return fail(SWC_HIP_EUNSUPPORTED, "swc_hip_argMax_i: top_k %d exceeds %d", top_k, kMaxTopK);
-    argmax_rows<<<ceil_div(m, 256), 256, 0, stream()>>>(input, idx, m, n, top_k);
+    if (n >= 128) argmax_rows_wave<<<ceil_div(m, 4), 256, 0, stream()>>>(input, idx, m, n, top_k);
+    else argmax_rows<<<ceil_div(m, 256), 256, 0, stream()>>>(input, idx, m, n, top_k);
     SWC_LAUNCH_CHECK();
     return SWC_HIP_OK;
 }

@@ -398,6 +398,22 @@ def test_softmax_golden_and_argmax(rt, oracle, golden):
         assert_bit_exact(rt.argMax(rt.upload(z), k).numpy(), oracle.argMax(z, k), f"argMax top{k}")
 
 
+@pytest.mark.parametrize("m,n", [(32, 1000), (7, 128), (5, 129), (3, 4099), (130, 200)])
+def test_argmax_of_long_rows(rt, oracle, m, n):
+    """Rows of 128 columns and more take a wavefront each; same order as argMax_i (ties: the larger column first)."""
+    rng = np.random.default_rng(m * n)
+    z = np.round(rng.standard_normal((m, n)) * 1.5).astype(np.float32)     # many ties
+    z[0, :] = 2.0                                                           # a constant row: the last columns win
+    if m > 2:
+        z[2, :] = -np.inf
+        z[2, n // 2] = -1e30
+    dz = rt.upload(z)
+    for k in (1, 3, 5, 8):
+        assert_bit_exact(rt.argMax(dz, k).numpy(), oracle.argMax(z, k), f"argMax top{k} of {m}x{n}")
+    x = rng.standard_normal((m, n)).astype(np.float32)
+    assert_bit_exact(rt.argMax(rt.upload(x), 5).numpy(), oracle.argMax(x, 5), "argMax top5, distinct values")
+
+
 @pytest.mark.parametrize("m,n", [(8, 1), (300, 3), (4097, 5), (256, 8), (1, 1)])
 def test_accuracy_counters(rt, oracle, m, n):
     """accuracy_i: the two counters accumulate over calls exactly as the host loop's."""
@@ -613,6 +629,39 @@ def test_conv_tiles_shared_along_k(rt, oracle, variant, monkeypatch):
     want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
     scale = oracle.conv2d(np.abs(x), np.abs(f), np.abs(b), fdims[1:3], strides, pads)
     assert np.max(np.abs(got - want) / scale) < TOL
+
+
+@pytest.mark.parametrize("idims,fdims,strides,pads", [((2, 7, 7, 256), (130, 3, 3, 256), (1, 1), (1, 1, 1, 1)),    # 6 tiles of 72 slices
+                                                      ((1, 9, 9, 2048), (64, 1, 1, 2048), (1, 1), (0, 0, 0, 0)),   # 1x1, 2 tiles of 64 slices
+                                                      ((3, 14, 14, 96), (72, 3, 3, 96), (2, 2), (1, 1, 1, 1))])     # 27 slices: below the limit
+def test_conv_layers_of_few_tiles_and_a_long_k_are_cut_throughout(rt, oracle, idims, fdims, strides, pads, monkeypatch):
+    """Fewer tiles than the chip holds workgroups and K >= 2048: every tile is cut along K (no whole tiles at all)."""
+    print("case conv, all tiles shared", idims, fdims, flush=True)
+    rng = np.random.default_rng(sum(idims) + sum(fdims))
+    x = rng.integers(-4, 5, idims).astype(np.float32)
+    f = rng.integers(-4, 5, fdims).astype(np.float32)
+    b = rng.integers(-4, 5, fdims[0]).astype(np.float32)
+    want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
+    long_k = int(np.prod(fdims[1:])) >= 2048
+    assert (rt.conv2d_workspace_bytes(idims, fdims, strides, pads) > 0) == long_k
+    dx, df, db = up(rt, x, f, b)
+    for slots in (None, 5, 9, 37, 100):
+        if slots:
+            monkeypatch.setenv("SWC_HIP_CONV_SLOTS", str(slots))
+        assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy(), want, f"all tiles shared, slots {slots}")
+        assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True).numpy(), oracle.relu(want),
+                         f"all tiles shared + relu, slots {slots}")
+    monkeypatch.delenv("SWC_HIP_CONV_SLOTS")
+    monkeypatch.setenv("SWC_HIP_CONV_SHARE_ALL", "0")
+    assert rt.conv2d_workspace_bytes(idims, fdims, strides, pads) == 0
+    assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy(), want, "whole tiles")
+    monkeypatch.setenv("SWC_HIP_CONV_SHARE_ALL", "8")
+    assert rt.conv2d_workspace_bytes(idims, fdims, strides, pads) > 0
+    xr = rng.standard_normal(idims).astype(np.float32)
+    fr = rng.standard_normal(fdims).astype(np.float32)
+    got = rt.conv2d(*up(rt, xr, fr, b), fdims[1:3], strides, pads).numpy()
+    scale = oracle.conv2d(np.abs(xr), np.abs(fr), np.abs(b), fdims[1:3], strides, pads)
+    assert np.max(np.abs(got - oracle.conv2d(xr, fr, b, fdims[1:3], strides, pads)) / scale) < TOL
 
 
 @pytest.mark.parametrize("idims,fdims,strides,pads", [((2, 9, 10, 6), (40, 3, 3, 6), (1, 1), (1, 1, 1, 1)),
