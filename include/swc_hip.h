@@ -317,6 +317,20 @@ int swc_hip_conv2dFused_f(float *output, const float *input, const float *filter
                           const float *bn_var, const float *bn_scale,
                           const float *bn_bias, float epsilon, int relu);
 
+/* The same with a second summand before the ReLU: conv2d_f, optionally
+ * batchnormalization_f, then vecAdd_f with `residual` (a tensor of the output's
+ * shape: the other branch of a residual block; NULL: none; it may be the output
+ * itself), then optionally relu_f. */
+int swc_hip_conv2dFusedAdd_f(float *output, const float *input, const float *filter,
+                             const float *bias, const size_t *odims,
+                             const size_t *idims, const size_t *fdims,
+                             const size_t *bdims, const size_t *kernels,
+                             const size_t *strides, const size_t *pads,
+                             size_t group, const float *bn_mean,
+                             const float *bn_var, const float *bn_scale,
+                             const float *bn_bias, float epsilon,
+                             const float *residual, int relu);
+
 #ifdef __cplusplus
 }
 #endif

@@ -367,7 +367,7 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
             store_tile<TM, TN>(acc, out, (size_t)N, M, N, m0 + (wave >> 1) * 32 * TM, n0 + (wave & 1) * 32 * TN, lane, ep);
         } else {
             float *slot = part + (size_t)(2 * share + (piece ? 1 : 0)) * (T::BM * T::BN);
-            store_tile_impl<TM, TN, false>(acc, slot, (size_t)T::BN, T::BM, T::BN, (wave >> 1) * 32 * TM,
+            store_tile_impl<TM, TN, false, false>(acc, slot, (size_t)T::BN, T::BM, T::BN, (wave >> 1) * 32 * TM,
                                            (wave & 1) * 32 * TN, lane, Epilogue{});
         }
     }
@@ -417,6 +417,7 @@ __global__ __launch_bounds__(256) void conv_sk_finish(float *__restrict__ out, c
                 const float slope = (float)((double)ep.bn_scale[col + e] / sqrt((double)ve));
                 y = fmaf(y - ep.bn_mean[col + e], slope, ep.bn_bias[col + e]);
             }
+            if (ep.residual) y += ep.residual[(size_t)row * N + col + e];
             if (ep.relu) y = (y > 0.f) ? y : 0.f;
             x[e] = y;
         }
@@ -665,16 +666,23 @@ __global__ __launch_bounds__(256) void conv_direct(const float *__restrict__ in,
                 if (oc >= OC) continue;   // (not "break": an early exit keeps the compiler from unrolling the pixel loop)
                 float v = acc[p][oc];
                 if (bn) v = fmaf(v - mean_sh[oc], slope_sh[oc], beta_sh[oc]);
-                if (ep.relu) v = (v > 0.f) ? v : 0.f;
+                if (ep.relu && !ep.residual) v = (v > 0.f) ? v : 0.f;
                 stage[threadIdx.x * stride + oc] = v;
             }
         }
         __syncthreads();
         const int pixels = (g.M - base < 256) ? (g.M - base) : 256;   // may be <= 0
         float *o = out + (size_t)base * OC;
+        const float *res = ep.residual ? ep.residual + (size_t)base * OC : nullptr;
         if (lane_px < per_step)
-            for (int px = wave * per_step + lane_px; px < pixels; px += 4 * per_step)
-                o[px * OC + lane_oc] = stage[px * stride + lane_oc];
+            for (int px = wave * per_step + lane_px; px < pixels; px += 4 * per_step) {
+                float v = stage[px * stride + lane_oc];
+                if (res) {
+                    v += res[px * OC + lane_oc];
+                    if (ep.relu) v = (v > 0.f) ? v : 0.f;
+                }
+                o[px * OC + lane_oc] = v;
+            }
     }
 }
 
@@ -1546,6 +1554,20 @@ int swc_hip_conv2dFused_f(float *output, const float *input, const float *filter
         SWC_ARG(bn_mean && bn_var && bn_scale && bn_bias);
     Epilogue ep{nullptr, bn_mean, bn_var, bn_scale, bn_bias, epsilon, relu};
     return conv_dispatch("swc_hip_conv2dFused_f", output, input, filter, bias, odims, idims, fdims, kernels, strides,
+                         pads, group, ep);
+}
+
+int swc_hip_conv2dFusedAdd_f(float *output, const float *input, const float *filter, const float *bias,
+                             const size_t *odims, const size_t *idims, const size_t *fdims, const size_t *bdims,
+                             const size_t *kernels, const size_t *strides, const size_t *pads, size_t group,
+                             const float *bn_mean, const float *bn_var, const float *bn_scale, const float *bn_bias,
+                             float epsilon, const float *residual, int relu) {
+    SWC_REQUIRE_INIT();
+    (void)bdims;
+    if (bn_mean || bn_var || bn_scale || bn_bias)
+        SWC_ARG(bn_mean && bn_var && bn_scale && bn_bias);
+    Epilogue ep{nullptr, bn_mean, bn_var, bn_scale, bn_bias, epsilon, relu, residual};
+    return conv_dispatch("swc_hip_conv2dFusedAdd_f", output, input, filter, bias, odims, idims, fdims, kernels, strides,
                          pads, group, ep);
 }
 

@@ -132,7 +132,9 @@ __device__ __forceinline__ void compute_slice(const float *__restrict__ As, cons
 }
 
 // Per-column epilogue constants: out = f(acc + bias[col]) with optional
-// inference batchnorm and optional ReLU.
+// inference batchnorm, an optional second summand of the output's shape (the
+// other branch of a residual block; read by the tile kernels of this header and
+// by the convolution's own kernels) and optional ReLU, in that order.
 struct Epilogue {
     const float *bias;      // may be null
     const float *bn_mean;   // null: no batchnorm
@@ -141,6 +143,7 @@ struct Epilogue {
     const float *bn_bias;
     float eps;
     int relu;
+    const float *residual = nullptr;   // [M, ldc] like the output, or null; may be the output itself
 };
 
 // Writes this wavefront's accumulators to C (row-major, leading dimension ldc).
@@ -152,7 +155,7 @@ struct Epilogue {
 // the previous store to be acknowledged — before every store.)  The guarded
 // path first waits for the per-column parameters explicitly, after which its
 // row blocks have no load to wait for either.
-template <int TM, int TN, bool GUARD>
+template <int TM, int TN, bool GUARD, bool RES>
 __device__ __forceinline__ void store_tile_impl(const v16f (&acc)[TM][TN], float *__restrict__ C, size_t ldc, int M,
                                                 int N, int row0, int col0, int lane, const Epilogue &ep) {
     const int l32 = lane & 31;
@@ -183,14 +186,24 @@ __device__ __forceinline__ void store_tile_impl(const v16f (&acc)[TM][TN], float
         const int col = col0 + tn * 32 + l32;
         if (GUARD && col >= N) continue;
         float *__restrict__ p = C + (size_t)(row0 + 4 * h) * ldc + col;
+        const float *res = RES ? ep.residual + (size_t)(row0 + 4 * h) * ldc + col : nullptr;
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
+            float add[16];   // the second summand of these 16 rows, all loads issued before the first store
+            if (RES) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int r = tm * 32 + 8 * (v / 4) + (v % 4);   // row relative to row0 + 4*h
+                    add[v] = (GUARD && row0 + 4 * h + r >= M) ? 0.f : res[(size_t)r * ldc];
+                }
+            }
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int r = tm * 32 + 8 * (v / 4) + (v % 4);   // row relative to row0 + 4*h
+                const int r = tm * 32 + 8 * (v / 4) + (v % 4);
                 if (GUARD && row0 + 4 * h + r >= M) continue;
                 float x = acc[tm][tn][v] + bias[tn];
                 if (bn) x = fmaf(x - mean[tn], slope[tn], beta[tn]);
+                if (RES) x += add[v];
                 if (ep.relu) x = (x > 0.f) ? x : 0.f;
                 p[(size_t)r * ldc] = x;
             }
@@ -201,10 +214,14 @@ __device__ __forceinline__ void store_tile_impl(const v16f (&acc)[TM][TN], float
 template <int TM, int TN>
 __device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], float *__restrict__ C, size_t ldc, int M, int N,
                                            int row0, int col0, int lane, const Epilogue &ep) {
-    if (row0 + 32 * TM <= M && col0 + 32 * TN <= N)   // wavefront-uniform
-        store_tile_impl<TM, TN, false>(acc, C, ldc, M, N, row0, col0, lane, ep);
-    else
-        store_tile_impl<TM, TN, true>(acc, C, ldc, M, N, row0, col0, lane, ep);
+    const bool inside = row0 + 32 * TM <= M && col0 + 32 * TN <= N;   // all four choices are wavefront-uniform
+    if (ep.residual) {
+        if (inside) store_tile_impl<TM, TN, false, true>(acc, C, ldc, M, N, row0, col0, lane, ep);
+        else store_tile_impl<TM, TN, true, true>(acc, C, ldc, M, N, row0, col0, lane, ep);
+    } else {
+        if (inside) store_tile_impl<TM, TN, false, false>(acc, C, ldc, M, N, row0, col0, lane, ep);
+        else store_tile_impl<TM, TN, true, false>(acc, C, ldc, M, N, row0, col0, lane, ep);
+    }
 }
 
 // Workgroup id -> tile coordinates.  Workgroups are dealt round-robin to the 8

@@ -26,7 +26,7 @@ EXPORTS = [
     "swc_hip_maxpool_argmax_f", "swc_hip_avgpool_f", "swc_hip_transpose4d_f", "swc_hip_transpose2d_f",
     "swc_hip_matrixSoftmax_f", "swc_hip_matrixTanh_f", "swc_hip_argMax_i", "swc_hip_accuracy_i", "swc_hip_fill_i",
     "swc_hip_matrixMatrixFCBias_f", "swc_hip_vecAddRelu_f", "swc_hip_batchnormRelu_f",
-    "swc_hip_batchnormReluMaxpool_f", "swc_hip_conv2dFused_f",
+    "swc_hip_batchnormReluMaxpool_f", "swc_hip_conv2dFused_f", "swc_hip_conv2dFusedAdd_f",
     "swc_hip_set_workspace", "swc_hip_matrixMatrixFCBiasSoftmax_f", "swc_hip_gemm_workspace_bytes", "swc_hip_conv2d_workspace_bytes", "swc_hip_host_malloc", "swc_hip_host_free", "swc_hip_matrixTrans_f", "swc_hip_matrixTanhGrad_f", "swc_hip_matrixSoftmaxWithLoss_f",
     "swc_hip_matrixSoftmaxGrad_f", "swc_hip_matrixSoftmaxWithLossGrad_f", "swc_hip_conv2dGrad_f",
     "swc_hip_maxpoolGrad_f", "swc_hip_batchedreduceadd_f", "swc_hip_sgd_f", "swc_hip_reluGrad_f",
@@ -97,6 +97,8 @@ def load_library():
         "swc_hip_batchnormReluMaxpool_f": (i32, [vp, vp, vp, vp, vp, vp, szp, f32, szp, szp, szp, szp]),
         "swc_hip_conv2dFused_f": (i32, [vp, vp, vp, vp, szp, szp, szp, szp, szp, szp, szp, sz,
                                         vp, vp, vp, vp, f32, i32]),
+        "swc_hip_conv2dFusedAdd_f": (i32, [vp, vp, vp, vp, szp, szp, szp, szp, szp, szp, szp, sz,
+                                        vp, vp, vp, vp, f32, vp, i32]),
         "swc_hip_set_workspace": (i32, [vp, sz]),
         "swc_hip_host_malloc": (vp, [sz]),
         "swc_hip_host_free": (i32, [vp]),
@@ -344,7 +346,7 @@ class SwcHip:
         return t
 
     def conv2d(self, x, filt, bias, kernels=None, strides=(1, 1), pads=(0, 0, 0, 0), group=1, bn=None,
-               eps=1e-5, relu=False, out=None):
+               eps=1e-5, relu=False, out=None, residual=None):
         """bn = (mean, var, scale, bias) DeviceArrays to fuse inference batchnorm."""
         if kernels is None:
             kernels = filt.shape[1:3]
@@ -353,7 +355,12 @@ class SwcHip:
         out = out if out is not None else self.empty(odims)
         shp = (_dims(odims), _dims(x.shape), _dims(filt.shape), _dims(bias.shape), _dims(kernels),
                _dims(strides), _dims(pads))
-        if bn is None and not relu:
+        if residual is not None:
+            assert tuple(residual.shape) == tuple(odims)
+            ptrs = [p.ptr for p in bn] if bn is not None else [None] * 4
+            rc = self.lib.swc_hip_conv2dFusedAdd_f(out.ptr, x.ptr, filt.ptr, bias.ptr, *shp, group, *ptrs,
+                                                   eps, residual.ptr, int(relu))
+        elif bn is None and not relu:
             rc = self.lib.swc_hip_conv2d_f(out.ptr, x.ptr, filt.ptr, bias.ptr, *shp, group)
         else:
             ptrs = [p.ptr for p in bn] if bn is not None else [None] * 4

@@ -80,7 +80,7 @@ void HipCodegen::emitWorkspace() {
             Tensor *x = T(0), *w = T(1);
             q << "gpu0_ws_bytes = std::max(gpu0_ws_bytes, swc_hip_gemm_workspace_bytes(" << x->size() / w->getDim(0) << ", "
               << w->getDim(1) << ", " << w->getDim(0) << "));\n";
-        } else if (type == "Conv2d" || type == "Conv2dWithActivation" || type == "Conv2dBatchNorm") {
+        } else if (type == "Conv2d" || type == "Conv2dWithActivation" || type == "Conv2dBatchNorm" || type == "Conv2dAdd") {
             auto *conv = static_cast<Conv2dOp *>(op->getOp());
             Tensor *y = static_cast<TensorNode *>(op->getChildNode(0))->getTensor();
             q << "{\n"
@@ -481,6 +481,17 @@ void HipCodegen::emitHipCall(OpNode *op) {
         writer_ << "SWC_HIP_CHECK(swc_hip_conv2dFused_f(" << convArgs(conv) << ", " << nameOf(in(5)) << ", "
                 << nameOf(in(6)) << ", " << nameOf(in(3)) << ", " << nameOf(in(4)) << ", " << std::setprecision(12)
                 << conv->getEpsilon() << ", " << (conv->hasRelu() ? 1 : 0) << "));\n";
+    } else if (type == "Conv2dAdd") {
+        // parents: input, filter, bias, [bn scale, bn bias, bn mean, bn var,] the other summand
+        auto *conv = static_cast<Conv2dAddOp *>(op->getOp());
+        convArrays(conv);
+        writer_ << "SWC_HIP_CHECK(swc_hip_conv2dFusedAdd_f(" << convArgs(conv) << ", ";
+        if (conv->hasBatchNorm())
+            writer_ << nameOf(in(5)) << ", " << nameOf(in(6)) << ", " << nameOf(in(3)) << ", " << nameOf(in(4)) << ", "
+                    << std::setprecision(12) << conv->getEpsilon() << ", " << nameOf(in(7));
+        else
+            writer_ << "NULL, NULL, NULL, NULL, 0.f, " << nameOf(in(3));
+        writer_ << ", " << (conv->hasRelu() ? 1 : 0) << "));\n";
     } else if (type == "BatchNormalization" || type == "BatchNormalizationRelu") {
         const bool relu = type == "BatchNormalizationRelu";
         const float eps = relu ? static_cast<BatchNormalizationReluOp *>(op->getOp())->getEpsilon()

@@ -267,6 +267,21 @@ class Conv2dBatchNormOp : public Conv2dOp {
     float getEpsilon() const { return epsilon_; }
     bool hasRelu() const { return relu_; }
 };
+// Conv2d (+ BatchNormalization) + ElementAdd (+ Relu): the last convolution of a residual block with the sum
+// and the activation that follow it.  Parents: input, filter, bias, [bn scale, bias, mean, var,] the other
+// summand.  swc_hip_conv2dFusedAdd_f
+class Conv2dAddOp : public Conv2dOp {
+    float epsilon_;
+    bool bn_, relu_;
+
+  public:
+    Conv2dAddOp(std::vector<size_t> &kernels, std::vector<size_t> &strides, std::vector<size_t> &pads, bool bn, float eps,
+                bool relu)
+        : Conv2dOp("Conv2dAdd", bn ? 8 : 4, kernels, strides, pads), epsilon_(eps), bn_(bn), relu_(relu) {}
+    float getEpsilon() const { return epsilon_; }
+    bool hasBatchNorm() const { return bn_; }
+    bool hasRelu() const { return relu_; }
+};
 
 } // namespace op
 } // namespace swc

@@ -198,6 +198,45 @@ void splice(IRGraph *g, OpNode *producer, OpNode *consumer, Op *fusedOp) {
     g->pushOpNode(fused);
 }
 
+// The ElementAdd / ElementAddRelu node that is the only reader of `producer`'s result (which is no graph output)
+// and whose other operand is a different tensor; null if there is none, or while a Relu behind a plain
+// ElementAdd is still to be merged into it.
+OpNode *soleAddConsumer(OpNode *producer, IRGraph *g, IRNode *&other) {
+    if (producer->childNum() != 1) return nullptr;
+    IRNode *t = producer->getChildNode(0);
+    if (t->childNum() != 1 || t->getLabel()->getIsOut()) return nullptr;
+    for (IRNode *lo : g->getLogicalOutNodes())
+        if (lo == t) return nullptr;
+    IRNode *c = t->getChildNode(0);
+    if (!(isType(c, "ElementAdd") || isType(c, "ElementAddRelu")) || c->parentNum() != 2) return nullptr;
+    auto *add = static_cast<OpNode *>(c);
+    other = add->getParentNode(0) == t ? add->getParentNode(1) : add->getParentNode(0);
+    if (other == t) return nullptr;
+    if (isType(c, "ElementAdd") && soleConsumer(add, "Relu", g)) return nullptr;
+    return add;
+}
+
+// producer -> mid -> add(mid, other) -> out  becomes  fused(producer's operands..., other) -> out
+void spliceAdd(IRGraph *g, OpNode *producer, OpNode *add, IRNode *other, Op *fusedOp) {
+    auto *mid = static_cast<TensorNode *>(producer->getChildNode(0));
+    auto *out = static_cast<TensorNode *>(add->getChildNode(0));
+    auto *fused = new OpNode(producer->name(), fusedOp);
+    *fused->getLabel() = *producer->getLabel();
+    fused->getLabel()->setTypeNameLabel(fusedOp->getOpName());
+    std::vector<IRNode *> operands(producer->getParentNodes());
+    operands.push_back(other);
+    while (producer->parentNum()) producer->destroyUpperNode(producer->getParentNode(0));
+    mid->destroyUpperNode(producer);
+    while (add->parentNum()) add->destroyUpperNode(add->getParentNode(0));
+    out->destroyUpperNode(add);
+    for (IRNode *p : operands) fused->exlinkUpperNode(p);
+    out->exlinkUpperNode(fused);
+    g->delOpNode(producer);
+    g->delOpNode(add);
+    g->delTensorNode(mid);
+    g->pushOpNode(fused);
+}
+
 } // namespace
 
 void HipFusionPass::run() {
@@ -226,13 +265,20 @@ void HipFusionPass::run() {
                 } else if (OpNode *r = soleConsumer(o, "Relu", _graph)) {
                     splice(_graph, o, r, new Conv2dWithActivationOp(k, s, p, SWC_ACTIVATION_RELU));
                     changed = true;
+                } else if (IRNode *other = nullptr; OpNode *add = soleAddConsumer(o, _graph, other)) {
+                    spliceAdd(_graph, o, add, other, new Conv2dAddOp(k, s, p, false, 0.f, isType(add, "ElementAddRelu")));
+                    changed = true;
                 }
             } else if (type == "Conv2dBatchNorm") {
                 auto *cb = static_cast<Conv2dBatchNormOp *>(o->getOp());
                 if (cb->hasRelu()) continue;
+                auto k = cb->getKernels(), s = cb->getStrides(), p = cb->getPads();
                 if (OpNode *r = soleConsumer(o, "Relu", _graph)) {
-                    auto k = cb->getKernels(), s = cb->getStrides(), p = cb->getPads();
                     splice(_graph, o, r, new Conv2dBatchNormOp(k, s, p, cb->getEpsilon(), true));
+                    changed = true;
+                } else if (IRNode *other = nullptr; OpNode *add = soleAddConsumer(o, _graph, other)) {
+                    spliceAdd(_graph, o, add, other,
+                              new Conv2dAddOp(k, s, p, true, cb->getEpsilon(), isType(add, "ElementAddRelu")));
                     changed = true;
                 }
             } else if (type == "BatchNormalization") {
@@ -266,7 +312,7 @@ bool DeviceMemoryLoweringPass::runsOnGpu(const std::string &t) {
     static const std::set<std::string> gpu = {
         "MatrixMatrixMul", "MatrixVectorAdd", "BatchedAdd", "MatrixMatrixFCBias", "MatrixMatrixFCBiasRelu",
         "MatrixMatrixFCBiasSoftmax", "Reshape", "MatrixTanh", "MatrixSoftmax", "ElementAdd", "ElementAddRelu", "Relu", "Dropout",
-        "Conv2d", "Conv2dWithActivation", "Conv2dBatchNorm", "MaxPool", "AveragePool", "Transpose",
+        "Conv2d", "Conv2dWithActivation", "Conv2dBatchNorm", "Conv2dAdd", "MaxPool", "AveragePool", "Transpose",
         "BatchNormalization",
         "BatchNormalizationRelu", "BatchNormReluMaxPool", "ArgMax", "Accuracy"};
     return gpu.count(t) != 0;

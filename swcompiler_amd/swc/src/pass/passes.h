@@ -79,6 +79,7 @@ class ElimTransposePass : public OptimizePass {
 //   BatchNormalization -> Relu                    => BatchNormalizationRelu
 //   BatchNormalizationRelu -> MaxPool             => BatchNormReluMaxPool
 //   ElementAdd -> Relu                            => ElementAddRelu
+//   Conv2d | Conv2dBatchNorm -> ElementAdd[Relu]  => Conv2dAdd (the other summand becomes its last operand)
 // Each right-hand side is one kernel launch of libswc_hip whose result equals
 // the left-hand sequence of reference kernels.
 class HipFusionPass : public OptimizePass {

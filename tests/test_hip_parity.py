@@ -699,6 +699,55 @@ def test_conv_with_a_channel_count_that_is_no_multiple_of_4(rt, oracle, idims, f
     assert np.max(np.abs(got - oracle.conv2d(xr, fr, b, fdims[1:3], strides, pads)) / scale) < TOL
 
 
+RESIDUAL_CONV_CASES = [((2, 14, 14, 64), (256, 1, 1, 64), (1, 1), (0, 0, 0, 0)),      # 1x1, whole tiles
+                       ((3, 17, 23, 32), (136, 3, 3, 32), (1, 1), (1, 1, 1, 1)),     # ragged rows and columns
+                       ((2, 7, 7, 256), (130, 3, 3, 256), (1, 1), (1, 1, 1, 1)),     # every tile cut along K
+                       ((2, 9, 10, 6), (40, 3, 3, 6), (1, 1), (1, 1, 1, 1)),         # padded channels
+                       ((4, 12, 12, 3), (16, 3, 3, 3), (1, 1), (1, 1, 1, 1))]        # the direct kernel
+
+
+@pytest.mark.parametrize("idims,fdims,strides,pads", RESIDUAL_CONV_CASES)
+@pytest.mark.parametrize("variant", [None, "reg11", "22_3m"])
+def test_conv_with_a_second_summand(rt, oracle, idims, fdims, strides, pads, variant, monkeypatch):
+    """conv2dFusedAdd_f = conv2d_f, batchnormalization_f, vecAdd_f with the other branch, relu_f."""
+    print("case conv + residual", idims, fdims, variant, flush=True)
+    if variant:
+        monkeypatch.setenv("SWC_HIP_CONV", variant)
+    rng = np.random.default_rng(sum(idims) + sum(fdims))
+    oc = fdims[0]
+    x = rng.integers(-4, 5, idims).astype(np.float32)
+    f = rng.integers(-4, 5, fdims).astype(np.float32)
+    b = rng.integers(-4, 5, oc).astype(np.float32)
+    conv = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
+    res = rng.integers(-40, 41, conv.shape).astype(np.float32)
+    dx, df, db, dres = up(rt, x, f, b, res)
+    add = lambda a, c: oracle.vecAdd(a.ravel(), c.ravel()).reshape(a.shape)
+    # integer-valued, no batchnorm: exact
+    assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads, residual=dres).numpy(), add(conv, res), "conv + residual")
+    assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads, residual=dres, relu=True).numpy(),
+                     oracle.relu(add(conv, res)), "conv + residual + relu")
+    # the summand may be the output itself (a Sum that writes one of its operands)
+    inplace = rt.upload(res)
+    rt.conv2d(dx, df, db, fdims[1:3], strides, pads, residual=inplace, relu=True, out=inplace)
+    assert_bit_exact(inplace.numpy(), oracle.relu(add(conv, res)), "conv + residual in place")
+    # with batchnorm: the fused call equals the library's own conv+BN call followed by add and relu, bit for bit
+    mean, beta = (rng.integers(-4, 5, oc).astype(np.float32) for _ in range(2))
+    var = rng.uniform(0.5, 2.0, oc).astype(np.float32)
+    gamma = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    bn = up(rt, mean, var, gamma, beta)
+    xr = rng.standard_normal(idims).astype(np.float32)
+    fr = (rng.standard_normal(fdims) / np.sqrt(np.prod(fdims[1:]))).astype(np.float32)
+    resr = rng.standard_normal(conv.shape).astype(np.float32)
+    dxr, dfr, dresr = up(rt, xr, fr, resr)
+    fused = rt.conv2d(dxr, dfr, db, fdims[1:3], strides, pads, bn=bn, eps=1e-5, relu=True, residual=dresr).numpy()
+    steps = rt.vecAdd(rt.conv2d(dxr, dfr, db, fdims[1:3], strides, pads, bn=bn, eps=1e-5).reshape((-1,)), dresr.reshape((-1,)), relu=True)
+    assert_bit_exact(fused.ravel(), steps.numpy(), "conv + bn + residual + relu against the separate calls")
+    want = oracle.relu(add(oracle.batchnormalization(oracle.conv2d(xr, fr, b, fdims[1:3], strides, pads), mean, var, gamma, beta, 1e-5), resr))
+    mag = np.abs(oracle.batchnormalization(oracle.conv2d(np.abs(xr), np.abs(fr), np.abs(b), fdims[1:3], strides, pads),
+                                           -np.abs(mean), var, gamma, np.abs(beta), 1e-5)) + np.abs(resr)
+    assert np.max(np.abs(fused - want) / mag) < TOL
+
+
 def test_conv_shared_tiles_in_a_caller_workspace(rt, oracle, monkeypatch):
     from swcompiler_amd.hip import SwcHipError
     idims, fdims, strides, pads = SHARED_CONV_CASES[0]

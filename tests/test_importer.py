@@ -319,8 +319,10 @@ def test_text_and_binary_files_give_the_same_program(gen, tmp_path):
 def test_import_hip_program_structure(gen, tmp_path):
     write_model(tmp_path, True)
     code = generate(gen, "caffe2", "hip", tmp_path, 2)
-    # conv+BN+ReLU and add+ReLU fuse; the weight transposes run once, before the op sequence
-    assert code.count("swc_hip_conv2dFused_f(") == 2 and "swc_hip_vecAddRelu_f(" in code
+    # conv+BN+ReLU is one call, and so is conv+BN+Sum+ReLU (the other summand, pool1, is the call's `residual`);
+    # the weight transposes run once, before the op sequence
+    assert code.count("swc_hip_conv2dFused_f(") == 1 and "swc_hip_vecAdd" not in code
+    assert code.count("swc_hip_conv2dFusedAdd_f(") == 1 and "1e-05, gpu_0_pool1, 1));" in code
     head, body = code.split("// call op routine functions")
     assert head.count("swc_hip_transpose4d_f(") == 2 and head.count("swc_hip_transpose2d_f(") == 1
     assert body.count("swc_hip_transpose4d_f(") == 1 and "swc_hip_transpose2d_f(" not in body
@@ -390,7 +392,9 @@ def test_resnet50_import_hip_program(gen, oracle, tmp_path):
     # the 53 filter transposes and the FC weight's run once; in the op sequence only pool5 is reordered for the FC
     assert head.count("swc_hip_transpose4d_f(") == 53 and head.count("swc_hip_transpose2d_f(") == 1
     assert body.count("swc_hip_transpose4d_f(") == 1 and "swc_hip_conv2dFused_f(" not in head
-    assert body.count("swc_hip_conv2dFused_f(") == 53 and body.count("swc_hip_vecAddRelu_f(") == 16
+    # the last convolution of each of the 16 blocks takes the block's sum and ReLU along
+    assert body.count("swc_hip_conv2dFused_f(") == 37 and body.count("swc_hip_conv2dFusedAdd_f(") == 16
+    assert "swc_hip_vecAdd" not in body
     subprocess.run([build_hip(tmp_path)], cwd=tmp_path, check=True, timeout=120, stdout=subprocess.DEVNULL)
     prob, top3 = read_outputs(tmp_path, "_host", 4, 100)
     want = run_net(oracle, predict, w, data)["gpu_0/softmax"]
