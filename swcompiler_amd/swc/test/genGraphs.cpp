@@ -4,7 +4,7 @@
 // the reference's test/engine/testEngineMLPInfer.cpp.
 //
 //   genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse|graph]
-//   model: mnist8 | mnist_loader | nchw | manual | caffe2[txt][@image size] | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
+//   model: mnist8 | mnist_loader | nchw | manual | caffe2[txt][@size[xchannels]] | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
 //   mnist_loader: [batch] is the number of records in mnist_labels_images.bin
 //
 // Every parameter/input tensor is initialised from "<name>.bin" in the
@@ -353,11 +353,13 @@ int main(int argc, char **argv) {
         // the reference's test/importer/testResnetImport.cpp: the caller defines the data tensor in NHWC, the
         // network and its weights come from a Caffe2 predict_net / init_net pair in the current directory
         // (binary .pb, or .pbtxt for "caffe2txt"), ArgMax(3) + a Debug print follow the softmax.
-        // "caffe2@64": images of 64 x 64 (default 12 x 12), always 3 channels.
+        // "caffe2@64": images of 64 x 64 (default 12 x 12) with 3 channels; "caffe2@28x1": 28 x 28 with one.
         const size_t b = batch ? batch : 2;
-        size_t hw = 12;
+        size_t hw = 12, channels = 3;
         if (model.find('@') != string::npos) {
-            hw = stoul(model.substr(model.find('@') + 1));
+            const string size = model.substr(model.find('@') + 1);
+            hw = stoul(size);
+            if (size.find('x') != string::npos) channels = stoul(size.substr(size.find('x') + 1));
             model = model.substr(0, model.find('@'));
         }
         if (model != "caffe2" && model != "caffe2txt") {
@@ -365,7 +367,7 @@ int main(int argc, char **argv) {
             return 2;
         }
         vector<TensorNode *> udef;
-        auto *data = new TensorNode("gpu_0/data", new Tensor({b, hw, hw, 3}));
+        auto *data = new TensorNode("gpu_0/data", new Tensor({b, hw, hw, channels}));
         data->getTensor()->setTensorInit(TensorInitType::FILE, "data.bin");
         udef.push_back(data);
         const string ext = model == "caffe2" ? ".pb" : ".pbtxt";

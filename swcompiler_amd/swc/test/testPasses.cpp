@@ -189,11 +189,85 @@ static void testElimination() {
     CHECK(et2.cancelledCount() == 0 && r2->getParentNode(0) == ab);
 }
 
+// A residual block as an importer builds it: weights stored [oC,iC,kh,kw] behind a Transpose, conv -> BN ->
+// Sum with the block's input -> Relu; then ArgMax and Accuracy.
+static void testResidualBlockAndCounters() {
+    TENSOR(x, 2, 6, 6, 8);
+    auto *w = new TensorNode("w", new Tensor({8, 8, 3, 3}, DataType::Float_t, layout_nchw));
+    w->getTensor()->setTensorInit(TensorInitType::FILE, "w.bin");
+    auto *tw = new OpNode("w_T_op", new TransposeOp(NCHW2NHWC));
+    tw->exlinkUpperNode(w);
+    auto *wT = new TensorNode("w_T", new Tensor({8, 3, 3, 8}), tw);
+    TENSOR(cb, 8);
+    TENSOR(scale, 8);
+    TENSOR(beta, 8);
+    TENSOR(mean, 8);
+    TENSOR(var, 8);
+    vector<size_t> k{3, 3}, st{1, 1}, p{1, 1, 1, 1};
+    DYOP(conv, Conv2dOp, k, st, p);
+    LINKUPPER(conv, x, wT, cb);
+    TENSOR(y, 2, 6, 6, 8);
+    LINKUPPER(y, conv);
+    auto *bn = new OpNode("bn", new BatchNormalizationOp(1e-5f));
+    bn->exlinkUpperNode(y, scale, beta, mean, var);
+    TENSOR(z, 2, 6, 6, 8);
+    LINKUPPER(z, bn);
+    OP(sum, ElementAddOp);
+    LINKUPPER(sum, x, z);   // the convolution's result is the SECOND summand here
+    auto *s1 = new TensorNode("z", z->getTensor(), sum);   // written in place, as Caffe2's Sum does
+    OP(relu, ReluOp);
+    LINKUPPER(relu, s1);
+    auto *r = new TensorNode("z", z->getTensor(), relu);
+    TENSOR(fw, 288, 10);
+    TENSOR(fb, 10);
+    OP(fc, MatrixMatrixFCBiasOp);
+    LINKUPPER(fc, r, fw, fb);
+    TENSOR(logits, 2, 10);
+    LINKUPPER(logits, fc);
+    auto *am = new OpNode("argmax", new ArgMaxOp(1));
+    am->exlinkUpperNode(logits);
+    auto *top1 = new TensorNode("top1", new Tensor({2, 1}, DataType::Int32_t), am);
+    auto *label = new TensorNode("label", new Tensor({2}, DataType::Int32_t));
+    OP(acc, AccuracyOp);
+    LINKUPPER(acc, top1, label);
+    auto *counters = new TensorNode("counters", new Tensor({1, 2}, DataType::Int32_t), acc);
+    counters->getTensor()->setTensorInit(TensorInitType::CONSTANT, 0);
+    G(g);
+    GpT(g, x, w, wT, cb, scale, beta, mean, var, y, z, s1, r, fw, fb, logits, top1, label, counters);
+    GpO(g, tw, conv, bn, sum, relu, fc, am, acc);
+    g->findInOut();
+    g->updateTopology();
+    Config hip;
+    hip.hip = true;
+    g->setConfig(hip);
+    Engine e(g);
+    e.compile();
+    CHECK(countOps(g, "Conv2dAdd") == 1 && countOps(g, "ElementAdd") + countOps(g, "ElementAddRelu") + countOps(g, "Relu") == 0);
+    OpNode *fused = nullptr, *trans = nullptr, *accuracy = nullptr;
+    for (int i = 0; i < g->opNodeNum(); ++i) {
+        const string t = g->getOpNode(i)->getOp()->getOpName();
+        if (t == "Conv2dAdd") fused = g->getOpNode(i);
+        if (t == "Transpose") trans = g->getOpNode(i);
+        if (t == "Accuracy") accuracy = g->getOpNode(i);
+    }
+    CHECK(fused && fused->parentNum() == 8 && fused->getParentNode(7)->name() == "x_dev");
+    auto *fop = static_cast<Conv2dAddOp *>(fused->getOp());
+    CHECK(fop->hasBatchNorm() && fop->hasRelu() && fused->getChildNode(0) == r);
+    // the weight's layout change runs once, after its upload; the data tensor's consumers stay per-iteration
+    CHECK(trans && trans->isRunOnce() && wT->getTensor()->getTensorInitType() == TensorInitType::PARENTOP);
+    CHECK(!fused->isRunOnce());
+    // Accuracy runs on the device: labels get a device twin, the counters live there and have a host twin
+    CHECK(accuracy && accuracy->getLabel()->getDeviceLabel().type == DeviceType::GPU);
+    CHECK(accuracy->getParentNode(1)->name() == "label_dev" && counters->getLabel()->getDeviceLabel().type == DeviceType::GPU);
+    CHECK(g->getNodeByName("counters_host") != nullptr && g->getNodeByName("top1_host") == nullptr);
+}
+
 int main() {
     testTopologyAndShapes();
     testLoweringAndRenaming();
     testFusionAndPlacement();
     testElimination();
+    testResidualBlockAndCounters();
     if (failures) {
         cerr << failures << " check(s) failed" << endl;
         return 1;

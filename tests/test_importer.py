@@ -415,3 +415,96 @@ def test_resnet50_full_size_hip_program(gen, oracle, tmp_path):
     want = run_net(oracle, predict, w, data)["gpu_0/softmax"]
     assert rel_err(prob, want) < TOL
     assert top3[0, 0] == int(np.argmax(want))
+
+
+# ------------------------------------------------ the other two networks the reference's tests import
+def conv_relu(ops, w, rng, name, src, cin, cout, k, pad, relu=True):
+    g = "gpu_0/"
+    w[g + name + "_w"] = (rng.standard_normal((cout, cin, k, k)) / np.sqrt(cin * k * k)).astype(np.float32)
+    w[g + name + "_b"] = (rng.standard_normal(cout) * 0.1).astype(np.float32)
+    ops.append(dict(type="Conv", input=[g + src, g + name + "_w", g + name + "_b"], output=[g + name],
+                    arg=dict(kernel=k, pad=pad, stride=1)))
+    if relu:
+        ops.append(dict(type="Relu", input=[g + name], output=[g + name]))
+    return name
+
+
+def fc(ops, w, rng, name, src, cin, cout, relu=False, dropout=False):
+    g = "gpu_0/"
+    w[g + name + "_w"] = (rng.standard_normal((cout, cin)) / np.sqrt(cin)).astype(np.float32)
+    w[g + name + "_b"] = (rng.standard_normal(cout) * 0.1).astype(np.float32)
+    ops.append(dict(type="FC", input=[g + src, g + name + "_w", g + name + "_b"], output=[g + name]))
+    if relu:
+        ops.append(dict(type="Relu", input=[g + name], output=[g + name]))
+    if dropout:
+        ops.append(dict(type="Dropout", input=[g + name], output=[g + name + "_drop"], arg=dict(ratio=0.5, is_test=1)))
+        return name + "_drop"
+    return name
+
+
+def make_lenet():
+    """Caffe2's lenet_mnist (test/importer/testLeNetImport.cpp): conv 5x5 -> pool -> conv 5x5 -> pool -> FC 500 ->
+    ReLU -> FC 10 -> softmax on 28 x 28 x 1 images."""
+    rng, w, ops, g = np.random.default_rng(1998), {}, [], "gpu_0/"
+    x = conv_relu(ops, w, rng, "conv1", "data", 1, 20, 5, 0, relu=False)
+    ops.append(dict(type="MaxPool", input=[g + x], output=[g + "pool1"], arg=dict(kernel=2, stride=2)))
+    x = conv_relu(ops, w, rng, "conv2", "pool1", 20, 50, 5, 0, relu=False)
+    ops.append(dict(type="MaxPool", input=[g + x], output=[g + "pool2"], arg=dict(kernel=2, stride=2)))
+    x = fc(ops, w, rng, "fc3", "pool2", 800, 500, relu=True)
+    x = fc(ops, w, rng, "pred", x, 500, 10)
+    ops.append(dict(type="Softmax", input=[g + x], output=[g + "softmax"]))
+    return ops, w, (28, 1, 10)
+
+
+def make_vgg(width=8, image=32, classes=20):
+    """VGG-19's layer sequence (test/importer/testVGG19Import.cpp) at 1/8 of its width on 32 x 32 images: 2-2-4-4-4
+    convolutions 3x3 + ReLU with 2x2 pooling between the groups, FC + ReLU + Dropout twice, FC, softmax."""
+    rng, w, ops, g = np.random.default_rng(2014), {}, [], "gpu_0/"
+    x, cin, hw = "data", 3, image
+    for group, (n, mult) in enumerate(((2, 1), (2, 2), (4, 4), (4, 8), (4, 8))):
+        for i in range(n):
+            x = conv_relu(ops, w, rng, f"conv{group + 1}_{i + 1}", x, cin, width * mult, 3, 1)
+            cin = width * mult
+        ops.append(dict(type="MaxPool", input=[g + x], output=[g + f"pool{group + 1}"], arg=dict(kernel=2, stride=2)))
+        x, hw = f"pool{group + 1}", hw // 2
+    x = fc(ops, w, rng, "fc6", x, cin * hw * hw, 64 * width, relu=True, dropout=True)
+    x = fc(ops, w, rng, "fc7", x, 64 * width, 64 * width, relu=True, dropout=True)
+    x = fc(ops, w, rng, "fc8", x, 64 * width, classes)
+    ops.append(dict(type="Softmax", input=[g + x], output=[g + "softmax"]))
+    return ops, w, (image, 3, classes)
+
+
+def write_net(tmp_path, batch, predict, w, image, channels):
+    init = [dict(type="GivenTensorFill", input=[], output=[k], arg=dict(shape=list(v.shape), values=v)) for k, v in w.items()]
+    open(os.path.join(tmp_path, "predict_net.pb"), "wb").write(enc_net("net", predict, packed=True))
+    open(os.path.join(tmp_path, "init_net.pb"), "wb").write(enc_net("net_init", init, packed=True))
+    data = np.random.default_rng(13).uniform(0, 1, (batch, image, image, channels)).astype(np.float32)
+    data.tofile(os.path.join(tmp_path, "data.bin"))
+    return data
+
+
+@pytest.mark.parametrize("make", [make_lenet, make_vgg])
+def test_lenet_and_vgg_import_cpu_program(gen, oracle, tmp_path, make):
+    predict, w, (image, channels, classes) = make()
+    data = write_net(tmp_path, 2, predict, w, image, channels)
+    generate(gen, f"caffe2@{image}x{channels}", "cpu", tmp_path, 2)
+    subprocess.run([build_cpu(tmp_path)], cwd=tmp_path, check=True, stdout=subprocess.DEVNULL)
+    prob, top3 = read_outputs(tmp_path, "", 2, classes)
+    want = run_net(oracle, predict, w, data)["gpu_0/softmax"]
+    assert_bit_exact(prob, want, "probabilities")
+    assert_bit_exact(top3, oracle.argMax(want, 3), "top-3")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("make", [make_lenet, make_vgg])
+def test_lenet_and_vgg_import_hip_program(gen, oracle, tmp_path, make):
+    print("case import", make.__name__, flush=True)
+    predict, w, (image, channels, classes) = make()
+    data = write_net(tmp_path, 8, predict, w, image, channels)
+    code = generate(gen, f"caffe2@{image}x{channels}", "hip", tmp_path, 8)
+    assert "swc_hip_relu_f(" not in code.split("// call op routine functions")[1] or make is make_lenet   # VGG: every ReLU fused
+    subprocess.run([build_hip(tmp_path)], cwd=tmp_path, check=True, timeout=120, stdout=subprocess.DEVNULL)
+    prob, top3 = read_outputs(tmp_path, "_host", 8, classes)
+    want = run_net(oracle, predict, w, data)["gpu_0/softmax"]
+    assert rel_err(prob, want) < TOL
+    assert (top3[:, 0] == oracle.argMax(want, 1)[:, 0]).all()
