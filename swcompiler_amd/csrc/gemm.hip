@@ -481,12 +481,13 @@ int launch_dma2(const float *a, const float *b, float *c, int m, int n, int k, i
     return SWC_HIP_OK;
 }
 
+template <int TM, int TN, int WM, int STAGES>
 int launch_splitk(const float *a, const float *b, float *c, int m, int n, int k, int lda, int ldb, int ldc,
                   const Epilogue &ep, int splits, int sps) {
-    using T = Dma2Tile<1, 4, 4, 2, 4>;
+    using T = Dma2Tile<TM, TN, WM, STAGES, 4>;
     float *part = static_cast<float *>(workspace((size_t)splits * m * n * sizeof(float), "gemm (split-K)"));
     if (!part) return SWC_HIP_ERUNTIME;
-    auto kern = gemm_dma2_splitk<1, 4, 4, 2, false, 4>;
+    auto kern = gemm_dma2_splitk<TM, TN, WM, STAGES, false, 4>;
     static bool attr_set = false;
     if (!attr_set) {
         SWC_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -509,15 +510,32 @@ int launch_splitk(const float *a, const float *b, float *c, int m, int n, int k,
 // split when the shape has too few output tiles to fill the chip.
 bool takes_fewrows(int m, int n, int k) { return m <= 16 && k > 0 && (size_t)k * n <= ((size_t)2 << 20); }
 
+// Up to 64 rows (small-batch inference: the product streams B once and is bound by that): tiles of 32 x 256
+// or 64 x 256 instead of 128 x 128, so that no matrix-core work goes into rows that do not exist — with
+// 128-row tiles the MFMAs of the empty rows hold a 25088 x 4096 layer at 2.1 TB/s of B (32 rows: 5.1 TB/s
+// with the thin tiles).  Always cut along K so that at least two workgroups per CU stream.
+constexpr int kThinRows = 64;
+constexpr int kThinCols = 256;   // Dma2Tile<1, 2, 1, ...>::BN
+bool takes_thin(int m, int n, int k) {
+    return m <= kThinRows && n > 16 && (size_t)k * n >= ((size_t)1 << 20) && !takes_fewrows(m, n, k);
+}
+
 bool splitk_plan(int m, int n, int k, int &splits, int &sps, bool forced = false) {
     if (!forced && takes_fewrows(m, n, k)) return false;
-    const long big_tiles = (long)((m + 127) / 128) * ((n + 127) / 128);
     const int nk = (k + BK - 1) / BK;
-    if (n <= 16 || nk < 2 || (!forced && (big_tiles * 4 > num_cus() || nk < 8))) return false;
-    splits = (int)((2L * num_cus() + big_tiles - 1) / big_tiles);
+    long tiles;
+    if (takes_thin(m, n, k)) {
+        tiles = (n + kThinCols - 1) / kThinCols;
+    } else {
+        tiles = (long)((m + 127) / 128) * ((n + 127) / 128);
+        if (n <= 16 || nk < 2 || (!forced && (tiles * 4 > num_cus() || nk < 8))) return false;
+    }
+    splits = (int)((2L * num_cus() + tiles - 1) / tiles);
     splits = splits > nk ? nk : splits;
+    if (takes_thin(m, n, k) && splits > 1 && nk / splits < 4) splits = nk / 4 > 0 ? nk / 4 : 1;   // four slices a share at least
     sps = (nk + splits - 1) / splits;
     splits = (nk + sps - 1) / sps;
+    if (takes_thin(m, n, k)) return (size_t)splits * m * n * 4 <= ((size_t)64 << 20);   // (one split: the finish adds the bias)
     return splits > 1 && (size_t)splits * m * n * 4 <= ((size_t)64 << 20);
 }
 
@@ -586,7 +604,9 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
         // their efficiency.
         int splits = 0, sps = 0;
         if (dma2_ok && (!force || !strcmp(force, "splitk")) && splitk_plan(m, n, k, splits, sps, force != nullptr))
-            return launch_splitk(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps);
+            return !takes_thin(m, n, k) ? launch_splitk<1, 4, 4, 2>(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps)
+                   : m <= 32            ? launch_splitk<1, 2, 1, 3>(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps)
+                                        : launch_splitk<2, 2, 1, 3>(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps);
         if (dma2_ok && huge_tiles >= num_cus()) return launch_dma2<2, 4, 4, 2, false, 8>(a, b, c, m, n, k, lda, ldb, ldc, ep);
         if (dma2_ok && big_tiles >= num_cus()) return launch_dma2<1, 4, 4, 2, false>(a, b, c, m, n, k, lda, ldb, ldc, ep);
         if (big_tiles >= num_cus()) return launch_dma<2, 2, 2>(a, b, c, m, n, k, lda, ldb, ldc, ep);

@@ -516,6 +516,30 @@ def test_fcbias_softmax_fused(rt, oracle, m, k, n):
                      "fused vs sequence, no bias")
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 4100, 600), (7, 4096, 1000), (32, 2048, 1000), (32, 1030, 1028), (17, 3000, 404),
+                                   (8, 25088, 512), (33, 2048, 1000), (64, 4100, 300), (50, 1111, 1000)])
+def test_gemm_of_up_to_64_rows_and_a_large_b(rt, oracle, m, k, n):
+    """Small-batch FC layers stream B once: 32 x 256 or 64 x 256 tiles cut along K, partial sums in the workspace."""
+    print("case thin gemm", m, k, n, flush=True)
+    assert rt.gemm_workspace_bytes(m, n, k) >= 4 * m * n
+    rng = np.random.default_rng(m * 7 + k + n)
+    a = rng.integers(-8, 9, (m, k)).astype(np.float32)
+    b = rng.integers(-8, 9, (k, n)).astype(np.float32)
+    bias = rng.integers(-8, 9, n).astype(np.float32)
+    exact = a.astype(np.int64) @ b.astype(np.int64)
+    assert_bit_exact(rt.matrixMatrixMul(*up(rt, a, b)).numpy(), exact.astype(np.float32), "integer product")
+    assert_bit_exact(rt.fcbias(*up(rt, a, b, bias), relu=True).numpy(),
+                     np.maximum(exact + bias.astype(np.int64), 0).astype(np.float32), "integer product + bias + relu")
+    ar = rng.standard_normal((m, k)).astype(np.float32)
+    br = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32)
+    got = rt.fcbias(*up(rt, ar, br, bias)).numpy()
+    want = ar.astype(np.float64) @ br.astype(np.float64) + bias
+    mag = np.abs(ar).astype(np.float64) @ np.abs(br).astype(np.float64) + np.abs(bias)
+    assert np.max(np.abs(got - want) / mag) < TOL
+    if m * k * n <= 32 * 2048 * 1000:
+        assert np.max(np.abs(got - oracle.fcbias(ar, br, bias)) / mag) < TOL
+
+
 @pytest.mark.parametrize("m,k,n", [(8, 784, 512), (1, 784, 512), (16, 1000, 100), (3, 5, 17), (16, 1, 33), (7, 64, 520),
                                    (8, 4096, 512), (2, 130, 4099)])
 def test_gemm_of_a_few_rows(rt, oracle, m, k, n):
