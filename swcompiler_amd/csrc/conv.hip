@@ -437,7 +437,8 @@ __global__ __launch_bounds__(256) void conv_sk_finish(float *__restrict__ out, c
 // CUs (LeNet's 12x12x20 -> 50 layer: 20 us whole, 28 us cut).
 // A layer with fewer tiles than slots and a long K (the late stages of a residual network at a moderate
 // batch: 32 x 7 x 7 x 512 -> 512 has 200 tiles of 144 slices each) would leave CUs idle for its whole
-// duration: all of its tiles are cut, into as many shares as there are slots.
+// duration: all of its tiles are cut, into as many shares as there are slots.  With a twelfth of a round or
+// less (one image: 16 tiles of 32 slices for 14 x 14 x 1024 -> 256, 24 us as whole tiles) K = 512 is long enough.
 constexpr int kShareAllMinSlices = 64;   // K >= 2048: below that the pieces and the second kernel cost what the idle CUs do
 int share_all_min_slices() {
     if (const char *e = getenv("SWC_HIP_CONV_SHARE_ALL"))   // tuning: slices per tile from which a short layer is cut (0: never)
@@ -450,7 +451,10 @@ SkPlan sk_plan(long tiles, int nk, int slots, bool allow_shared) {
     if (!allow_shared || tiles == 0) return p;
     long rest = tiles % slots;
     if (tiles < slots) {
-        if (nk < share_all_min_slices() || 4 * tiles > 3 * slots) return p;   // (a nearly full round: leave it)
+        // (a nearly full round: leave it; a twelfth of a round or less — single images — is cut from K = 512 on)
+        const int min_slices = share_all_min_slices();
+        const bool long_k = nk >= min_slices || (min_slices == kShareAllMinSlices && 12 * tiles <= slots && nk >= 16);
+        if (!long_k || 4 * tiles > 3 * slots) return p;
         rest = tiles;
     } else if (rest == 0 || 2 * rest > slots) {
         return p;

@@ -657,16 +657,18 @@ def test_conv_tiles_shared_along_k(rt, oracle, variant, monkeypatch):
 
 @pytest.mark.parametrize("idims,fdims,strides,pads", [((2, 7, 7, 256), (130, 3, 3, 256), (1, 1), (1, 1, 1, 1)),    # 6 tiles of 72 slices
                                                       ((1, 9, 9, 2048), (64, 1, 1, 2048), (1, 1), (0, 0, 0, 0)),   # 1x1, 2 tiles of 64 slices
-                                                      ((3, 14, 14, 96), (72, 3, 3, 96), (2, 2), (1, 1, 1, 1))])     # 27 slices: below the limit
+                                                      ((3, 14, 14, 96), (72, 3, 3, 96), (2, 2), (1, 1, 1, 1)),      # 6 tiles of 27 slices: few enough tiles
+                                                      ((3, 14, 14, 32), (72, 3, 3, 32), (2, 2), (1, 1, 1, 1))])     # 9 slices: below the limit
 def test_conv_layers_of_few_tiles_and_a_long_k_are_cut_throughout(rt, oracle, idims, fdims, strides, pads, monkeypatch):
-    """Fewer tiles than the chip holds workgroups and K >= 2048: every tile is cut along K (no whole tiles at all)."""
+    """Fewer tiles than the chip holds workgroups and K >= 2048 (K >= 512 for a twelfth of a round or less): every
+    tile is cut along K (no whole tiles at all)."""
     print("case conv, all tiles shared", idims, fdims, flush=True)
     rng = np.random.default_rng(sum(idims) + sum(fdims))
     x = rng.integers(-4, 5, idims).astype(np.float32)
     f = rng.integers(-4, 5, fdims).astype(np.float32)
     b = rng.integers(-4, 5, fdims[0]).astype(np.float32)
     want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
-    long_k = int(np.prod(fdims[1:])) >= 2048
+    long_k = int(np.prod(fdims[1:])) >= 512
     assert (rt.conv2d_workspace_bytes(idims, fdims, strides, pads) > 0) == long_k
     dx, df, db = up(rt, x, f, b)
     for slots in (None, 5, 9, 37, 100):
