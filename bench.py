@@ -17,7 +17,8 @@ Also in the line:
   graph_replay  the same K steps replayed as one HIP graph per step (no per-kernel
                 events in the loop): what a launch-bound small graph gains
   incl_transfers  the step with the input batch uploaded and the result downloaded
-                each time (never the headline value)
+                each time (never the headline value); `overlapped_uploads`: the same with
+                the next batch's upload on a second stream while this batch is computed
   peaks_measured  fp32 MFMA rate of a register-only loop and a streaming copy on this
                 device, beside the datasheet peaks the fractions are computed from
   configs       the other synthetic configurations (samples/s and, per kernel,
@@ -155,6 +156,23 @@ def with_transfers(rt, graphs, cfg, steps):
     wall = time.perf_counter() - t0
     res = dict(samples_per_s=batch * steps / wall, ms_per_step=wall * 1e3 / steps,
                h2d_bytes=int(host_x.nbytes), d2h_bytes=int(host_out.nbytes), host_memory="page-locked")
+    # the same with the upload of the next batch on the library's copy stream while this one is computed:
+    # the batch lands in a staging buffer, a device-to-device copy hands it to the graph's input
+    stage = rt.empty(t["x"].shape)
+    rt.copy_h2d_async(stage, host_x)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        rt.copy_sync()            # the batch has arrived (and host_x may be refilled)
+        rt.ops_wait_copies()
+        rt.d2d(dt["x"], stage)
+        rt.copy_wait_ops()        # the next upload starts when the staging buffer has been read
+        out = graphs.run(cfg, rt, dt, fused=True, ws=ws)
+        rt.copy_h2d_async(stage, host_x)
+        rt.download_into(host_out, out)
+    rt.copy_sync()
+    wall = time.perf_counter() - t0
+    res["overlapped_uploads"] = dict(samples_per_s=batch * steps / wall, ms_per_step=wall * 1e3 / steps)
+    stage.free()
     rt.free_pinned(host_x)
     rt.free_pinned(host_out)
     return res

@@ -61,6 +61,23 @@ int swc_hip_host_free(void *hptr);
 int swc_hip_h2d(void *dst_dev, const void *src_host, size_t bytes); /* ordered after prior ops, returns when done */
 int swc_hip_d2h(void *dst_host, const void *src_dev, size_t bytes); /* ordered after prior ops, returns when done */
 int swc_hip_d2d(void *dst_dev, const void *src_dev, size_t bytes);  /* async on the stream */
+/* No counterpart in the reference (its one stream per GPU carries copies and
+ * kernels alike, src/codegen/Codegen.cpp:166-172, 1142-1168).  Uploads on a second
+ * stream of the library, so that the next batch travels while the ops work on
+ * this one:
+ *   swc_hip_copy_h2d_async  enqueues a copy from page-locked host memory
+ *                           (swc_hip_host_malloc) on the copy stream and returns;
+ *   swc_hip_copy_wait_ops   copies enqueued from now on start only after every op
+ *                           issued so far (the buffer they overwrite is free then);
+ *   swc_hip_ops_wait_copies ops issued from now on start only after every copy
+ *                           enqueued so far (on the device; the host does not wait);
+ *   swc_hip_copy_sync       the host waits for the copy stream (the host buffer of
+ *                           a copy may be written again).
+ * Both streams have the default priority. */
+int swc_hip_copy_h2d_async(void *dst_dev, const void *src_host, size_t bytes);
+int swc_hip_copy_wait_ops(void);
+int swc_hip_ops_wait_copies(void);
+int swc_hip_copy_sync(void);
 int swc_hip_fill_f(float *dst_dev, float value, size_t count);      /* initTensorConstant/Zero, kernels.h:23-29 */
 int swc_hip_fill_i(int *dst_dev, int value, size_t count);          /* the same for an Int32 tensor (counters) */
 int swc_hip_sync(void);

@@ -21,6 +21,8 @@ struct State {
     hipStream_t own = nullptr;   // created by init
     hipStream_t cur = nullptr;   // where ops launch (own or caller's)
     bool cur_is_own = true;
+    hipStream_t copy = nullptr;  // uploads that overlap the ops (created on first use)
+    hipEvent_t ev_ops = nullptr, ev_copy = nullptr;
     hipEvent_t t0 = nullptr, t1 = nullptr;
     float last_ms = -1.f;
     hipEvent_t slots[kEventSlots] = {};
@@ -137,6 +139,14 @@ int swc_hip_shutdown(void) {
     g.ws_owned = false;
     (void)hipEventDestroy(g.t0);
     (void)hipEventDestroy(g.t1);
+    if (g.copy) {
+        (void)hipStreamSynchronize(g.copy);
+        (void)hipStreamDestroy(g.copy);
+        (void)hipEventDestroy(g.ev_ops);
+        (void)hipEventDestroy(g.ev_copy);
+        g.copy = nullptr;
+        g.ev_ops = g.ev_copy = nullptr;
+    }
     for (hipEvent_t &e : g.slots)
         if (e) {
             (void)hipEventDestroy(e);
@@ -235,6 +245,54 @@ int swc_hip_d2d(void *dst, const void *src, size_t bytes) {
     SWC_ARG(bytes == 0 || (dst && src));
     if (!bytes) return SWC_HIP_OK;
     SWC_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, stream()));
+    return SWC_HIP_OK;
+}
+
+// ---- uploads on a second stream, so that the next batch arrives while the ops work on this one ----
+namespace {
+int copy_stream_ready() {
+    if (g.copy) return SWC_HIP_OK;
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (g.copy) return SWC_HIP_OK;
+    hipStream_t s = nullptr;
+    SWC_HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));   // default priority, like the op stream
+    SWC_HIP_TRY(hipEventCreateWithFlags(&g.ev_ops, hipEventDisableTiming));
+    SWC_HIP_TRY(hipEventCreateWithFlags(&g.ev_copy, hipEventDisableTiming));
+    g.copy = s;
+    return SWC_HIP_OK;
+}
+} // namespace
+
+int swc_hip_copy_h2d_async(void *dst, const void *src, size_t bytes) {
+    SWC_REQUIRE_INIT();
+    SWC_ARG(bytes == 0 || (dst && src));
+    if (int rc = copy_stream_ready()) return rc;
+    if (!bytes) return SWC_HIP_OK;
+    SWC_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g.copy));
+    return SWC_HIP_OK;
+}
+
+int swc_hip_copy_wait_ops(void) {
+    SWC_REQUIRE_INIT();
+    if (g.capturing) return fail(SWC_HIP_EINVAL, "swc_hip_copy_wait_ops: not while a graph is being recorded");
+    if (int rc = copy_stream_ready()) return rc;
+    SWC_HIP_TRY(hipEventRecord(g.ev_ops, stream()));
+    SWC_HIP_TRY(hipStreamWaitEvent(g.copy, g.ev_ops, 0));
+    return SWC_HIP_OK;
+}
+
+int swc_hip_ops_wait_copies(void) {
+    SWC_REQUIRE_INIT();
+    if (g.capturing) return fail(SWC_HIP_EINVAL, "swc_hip_ops_wait_copies: not while a graph is being recorded");
+    if (int rc = copy_stream_ready()) return rc;
+    SWC_HIP_TRY(hipEventRecord(g.ev_copy, g.copy));
+    SWC_HIP_TRY(hipStreamWaitEvent(stream(), g.ev_copy, 0));
+    return SWC_HIP_OK;
+}
+
+int swc_hip_copy_sync(void) {
+    SWC_REQUIRE_INIT();
+    if (g.copy) SWC_HIP_TRY(hipStreamSynchronize(g.copy));
     return SWC_HIP_OK;
 }
 

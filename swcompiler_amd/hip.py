@@ -17,7 +17,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 
 EXPORTS = [
     "swc_hip_init", "swc_hip_shutdown", "swc_hip_malloc", "swc_hip_free", "swc_hip_h2d", "swc_hip_d2h",
-    "swc_hip_d2d", "swc_hip_fill_f", "swc_hip_sync", "swc_hip_last_error", "swc_hip_stream",
+    "swc_hip_d2d", "swc_hip_copy_h2d_async", "swc_hip_copy_wait_ops", "swc_hip_ops_wait_copies", "swc_hip_copy_sync", "swc_hip_fill_f", "swc_hip_sync", "swc_hip_last_error", "swc_hip_stream",
     "swc_hip_set_stream", "swc_hip_device_name", "swc_hip_timer_begin", "swc_hip_timer_end",
     "swc_hip_timer_elapsed_ms", "swc_hip_event_record", "swc_hip_event_elapsed_ms", "swc_hip_graph_begin",
     "swc_hip_graph_end", "swc_hip_graph_launch", "swc_hip_graph_destroy", "swc_hip_probe_mfma_f32",
@@ -59,6 +59,10 @@ def load_library():
         "swc_hip_d2h": (i32, [vp, vp, sz]),
         "swc_hip_d2d": (i32, [vp, vp, sz]),
         "swc_hip_fill_f": (i32, [vp, f32, sz]),
+        "swc_hip_copy_h2d_async": (i32, [vp, vp, sz]),
+        "swc_hip_copy_wait_ops": (i32, []),
+        "swc_hip_ops_wait_copies": (i32, []),
+        "swc_hip_copy_sync": (i32, []),
         "swc_hip_sync": (i32, []),
         "swc_hip_last_error": (C.c_char_p, []),
         "swc_hip_stream": (vp, []),
@@ -229,6 +233,25 @@ class SwcHip:
     def download_into(self, host, d):
         assert host.nbytes == d.nbytes and host.flags.c_contiguous
         self._check(self.lib.swc_hip_d2h(host.ctypes.data, d.ptr, d.nbytes), "swc_hip_d2h")
+
+    def d2d(self, dst, src):
+        """device-to-device copy on the op stream (asynchronous)"""
+        assert dst.nbytes == src.nbytes
+        self._check(self.lib.swc_hip_d2d(dst.ptr, src.ptr, src.nbytes), "swc_hip_d2d")
+
+    # uploads on the library's second stream (see include/swc_hip.h)
+    def copy_h2d_async(self, d, pinned_host):
+        assert pinned_host.nbytes == d.nbytes
+        self._check(self.lib.swc_hip_copy_h2d_async(d.ptr, pinned_host.ctypes.data, d.nbytes), "swc_hip_copy_h2d_async")
+
+    def copy_wait_ops(self):
+        self._check(self.lib.swc_hip_copy_wait_ops(), "swc_hip_copy_wait_ops")
+
+    def ops_wait_copies(self):
+        self._check(self.lib.swc_hip_ops_wait_copies(), "swc_hip_ops_wait_copies")
+
+    def copy_sync(self):
+        self._check(self.lib.swc_hip_copy_sync(), "swc_hip_copy_sync")
 
     def probe_mfma_tflops(self, iters=2000):
         """fp32 MFMA rate a register-only loop sustains (TFLOP/s) and its duration in ms"""

@@ -239,9 +239,54 @@ void HipCodegen::emitExecute() {
         writer_.indentDec();
         writer_ << "}\nSWC_HIP_CHECK(swc_hip_graph_end(&swc_graph));\n";
         defer_output_gathers_ = true;
-        writer_ << "while(loader.next(" << nameOf(graph_->getInferLabelNode()) << ", "
-                << nameOf(graph_->getInferDataNode()) << ")) {\n";
-        writer_.indentInc();
+        // per-batch uploads (the Scatter nodes that are not run-once), in emission order
+        std::vector<OpNode *> uploads;
+        for (int i = 0; i < graph_->topologyNum(); ++i)
+            for (int j = 0; j < graph_->getNumInTopoLevel(i); ++j) {
+                IRNode *node = graph_->getNodeInTopo(i, j);
+                if (node->nodeType() != OP_NODE) continue;
+                auto *op = static_cast<OpNode *>(node);
+                if (!op->isRunOnce() && op->getOp()->getOpName() == "Scatter") uploads.push_back(op);
+            }
+        const bool prefetch = config_.hip_prefetch && !uploads.empty();
+        const std::string next = "loader.next(" + nameOf(graph_->getInferLabelNode()) + ", " +
+                                 nameOf(graph_->getInferDataNode()) + ")";
+        auto stageName = [&](OpNode *u) { return nameOf(u->getChildNode(0)) + "_stage"; };
+        auto bytesOf = [&](OpNode *u) {
+            return std::min(T(u->getParentNode(0))->getSizeInBytes(), T(u->getChildNode(0))->getSizeInBytes());
+        };
+        auto emitPrefetch = [&]() {   // the batch the loader has just produced starts its way to the staging buffers
+            for (OpNode *u : uploads) {
+                std::string src = nameOf(u->getParentNode(0));
+                if (const size_t off = static_cast<ScatterOp *>(u->getOp())->getOffset()) src += " + " + std::to_string(off);
+                writer_ << "SWC_HIP_CHECK(swc_hip_copy_h2d_async(" << stageName(u) << ", " << src << ", " << bytesOf(u)
+                        << "));\n";
+            }
+        };
+        if (prefetch) {
+            // The loader reads batch i+1 and the copy stream uploads it into staging buffers while the device
+            // computes batch i; a device-to-device copy hands a staged batch to the tensors the graph reads.
+            writer_ << "// staging buffers: the next batch is uploaded while this one is computed\n";
+            for (OpNode *u : uploads)
+                writer_ << "void *" << stageName(u) << " = swc_hip_malloc(" << bytesOf(u) << ");\n"
+                        << "if (!" << stageName(u) << ") { std::fprintf(stderr, \"%s\\n\", swc_hip_last_error()); return 1; }\n";
+            writer_ << "bool swc_more = " << next << ";\n";
+            writer_ << "if (swc_more) {\n";
+            writer_.indentInc();
+            emitPrefetch();
+            writer_.indentDec();
+            writer_ << "}\nwhile (swc_more) {\n";
+            writer_.indentInc();
+            writer_ << "SWC_HIP_CHECK(swc_hip_copy_sync());          // the batch has arrived; the host buffers are free\n";
+            writer_ << "SWC_HIP_CHECK(swc_hip_ops_wait_copies());\n";
+            for (OpNode *u : uploads)
+                writer_ << "SWC_HIP_CHECK(swc_hip_d2d(" << nameOf(u->getChildNode(0)) << ", " << stageName(u) << ", "
+                        << bytesOf(u) << "));\n";
+            writer_ << "SWC_HIP_CHECK(swc_hip_copy_wait_ops());      // the next upload may overwrite the staging buffers after this\n";
+        } else {
+            writer_ << "while(" << next << ") {\n";
+            writer_.indentInc();
+        }
         bool launched = false;
         for (int i = 0; i < graph_->topologyNum(); ++i)
             for (int j = 0; j < graph_->getNumInTopoLevel(i); ++j) {
@@ -250,10 +295,21 @@ void HipCodegen::emitExecute() {
                 auto *op = static_cast<OpNode *>(node);
                 if (op->isRunOnce()) continue;
                 if (isDeviceComputeOp(op)) {
-                    if (!launched) writer_ << "SWC_HIP_CHECK(swc_hip_graph_launch(swc_graph));\n";
+                    if (!launched) {
+                        writer_ << "SWC_HIP_CHECK(swc_hip_graph_launch(swc_graph));\n";
+                        if (prefetch) {
+                            writer_ << "swc_more = " << next << ";   // the next batch, while the device works on this one\n";
+                            writer_ << "if (swc_more) {\n";
+                            writer_.indentInc();
+                            emitPrefetch();
+                            writer_.indentDec();
+                            writer_ << "}\n";
+                        }
+                    }
                     launched = true;
                     continue;
                 }
+                if (prefetch && op->getOp()->getOpName() == "Scatter") continue;   // done above
                 writer_ << "// topology(" << i << ", " << j << "): " << op->name() << " : " << op->getOp()->getOpName()
                         << "\n";
                 dispatchOpNode(op);
@@ -264,6 +320,8 @@ void HipCodegen::emitExecute() {
         writer_ << "} //while\n";
         emitDeferredGathers();
         writer_ << "SWC_HIP_CHECK(swc_hip_sync());\n";
+        if (prefetch)
+            for (OpNode *u : uploads) writer_ << "SWC_HIP_CHECK(swc_hip_free(" << stageName(u) << "));\n";
         writer_ << "SWC_HIP_CHECK(swc_hip_graph_destroy(swc_graph));\n";
         return;
     }

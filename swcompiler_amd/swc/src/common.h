@@ -69,6 +69,7 @@ struct Config {
     int hip_device{0};          // device ordinal passed to swc_hip_init
     bool hip_fusion{true};      // fold bias/BN/ReLU into GEMM/conv epilogues, BN+ReLU(+pool) into one pass
     size_t time_iters{0};       // > 0: generated program repeats the op sequence and prints ms/iteration
+    bool hip_prefetch{false};   // with use_dataloader and hip_graph: the next batch is read and uploaded (second stream) while this one is computed
     bool hip_graph{false};      // with time_iters or use_dataloader: record the device ops of an iteration into one HIP graph and replay that
     bool dump_outputs{false};   // generated program writes every graph output to <name>.bin (raw fp32/int32)
 };

@@ -3,7 +3,7 @@
 // directory.  User-level code: only `SWC.h` and the DSL macros, in the style of
 // the reference's test/engine/testEngineMLPInfer.cpp.
 //
-//   genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse|graph]
+//   genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse|graph|prefetch]
 //   model: mnist8 | mnist_loader | nchw | manual | caffe2[txt][@size[xchannels]] | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
 //   mnist_loader: [batch] is the number of records in mnist_labels_images.bin
 //
@@ -104,7 +104,7 @@ static TensorNode *lazyUnary(IRGraph *g, const string &name, Op *op, TensorNode 
 
 int main(int argc, char **argv) {
     if (argc < 3) {
-        cerr << "usage: genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse|graph]\n";
+        cerr << "usage: genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse|graph|prefetch]\n";
         return 2;
     }
     string model = argv[1];
@@ -112,7 +112,8 @@ int main(int argc, char **argv) {
     const size_t batch = argc > 3 ? strtoul(argv[3], nullptr, 10) : 0;
     const size_t iters = argc > 4 ? strtoul(argv[4], nullptr, 10) : 0;
     const bool nofuse = argc > 5 && string(argv[5]) == "nofuse";
-    const bool useGraph = argc > 5 && string(argv[5]) == "graph";
+    const bool prefetch = argc > 5 && string(argv[5]) == "prefetch";   // (implies graph)
+    const bool useGraph = prefetch || (argc > 5 && string(argv[5]) == "graph");
 
     G(graph);
     TensorNode *out = nullptr;
@@ -400,6 +401,7 @@ int main(int argc, char **argv) {
     config.hip_fusion = !nofuse;
     config.time_iters = iters;
     config.hip_graph = useGraph;
+    config.hip_prefetch = prefetch;
     config.dump_outputs = true;
     if (model == "mnist_loader") {
         config.use_dataloader = true;

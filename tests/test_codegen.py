@@ -57,8 +57,9 @@ def write_inputs(cfg, t, workdir):
         t[k].tofile(os.path.join(workdir, stem + ".bin"))
 
 
-def generate(gen, model, target, workdir, batch=0, iters=0, nofuse=False, graph=False):
-    args = [gen, model, target, str(batch), str(iters)] + (["nofuse"] if nofuse else []) + (["graph"] if graph else [])
+def generate(gen, model, target, workdir, batch=0, iters=0, nofuse=False, graph=False, prefetch=False):
+    args = [gen, model, target, str(batch), str(iters)] + (["nofuse"] if nofuse else []) + (["graph"] if graph else []) + \
+           (["prefetch"] if prefetch else [])
     code = subprocess.run(args, cwd=workdir, check=True, capture_output=True, text=True).stdout
     assert open(os.path.join(workdir, "Graph.cpp")).read() == code
     return code
@@ -302,12 +303,31 @@ def test_batch_loop_hip_program_structure(gen, tmp_path):
     build_hip(tmp_path)
 
 
+def test_prefetching_batch_loop_structure(gen, tmp_path):
+    """Config::hip_prefetch: the loader reads and the copy stream uploads batch i+1 while the graph of batch i runs."""
+    code = generate(gen, "mnist_loader", "hip", tmp_path, 44, prefetch=True)
+    head, body = code.split("while (swc_more) {")
+    assert "while(loader.next(" not in code
+    assert head.count("loader.next(selected, data0)") == 1 and head.count("swc_hip_copy_h2d_async(") == 2
+    assert "void *data0_dev_stage = swc_hip_malloc(25088);" in head and "void *selected_dev_stage = swc_hip_malloc(32);" in head
+    loop = body[:body.index("} //while")]
+    order = ["swc_hip_copy_sync()", "swc_hip_ops_wait_copies()", "swc_hip_d2d(data0_dev, data0_dev_stage, 25088)",
+             "swc_hip_d2d(selected_dev, selected_dev_stage, 32)", "swc_hip_copy_wait_ops()", "swc_hip_graph_launch(swc_graph)",
+             "swc_more = loader.next(selected, data0)", "swc_hip_copy_h2d_async(data0_dev_stage, data0, 25088)",
+             "swc_hip_copy_h2d_async(selected_dev_stage, selected, 32)", "iter++"]
+    positions = [loop.index(s) for s in order]
+    assert positions == sorted(positions)
+    assert "swc_hip_h2d(" not in loop      # no synchronous upload is left in the loop
+    assert body.count("swc_hip_free(data0_dev_stage)") == 1
+    build_hip(tmp_path)
+
+
 @pytest.mark.gpu
-@pytest.mark.parametrize("graph", [False, True])
-def test_batch_loop_hip_program(gen, oracle, tmp_path, graph):
-    print("case batch loop, graph =", graph, flush=True)
+@pytest.mark.parametrize("graph,prefetch", [(False, False), (True, False), (True, True)])
+def test_batch_loop_hip_program(gen, oracle, tmp_path, graph, prefetch):
+    print("case batch loop, graph =", graph, "prefetch =", prefetch, flush=True)
     images, labels = write_record_file(tmp_path, 44)
-    generate(gen, "mnist_loader", "hip", tmp_path, 44, graph=graph)
+    generate(gen, "mnist_loader", "hip", tmp_path, 44, graph=graph and not prefetch, prefetch=prefetch)
     exe = build_hip(tmp_path)
     out = subprocess.run([exe], cwd=tmp_path, check=True, capture_output=True, text=True, timeout=120).stdout
     assert parse_counters(out) == expected_counters(oracle, images, labels)
