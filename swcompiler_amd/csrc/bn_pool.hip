@@ -255,11 +255,19 @@ __global__ __launch_bounds__(kThreads) void avgpool_vec4(const float *__restrict
         for (int ky = 0; ky < g.kh; ++ky) {
             const int iy = oy * g.sh - g.pt + ky;
             if (iy < 0 || iy >= g.H) continue;
-            for (int kx = 0; kx < g.kw; ++kx) {
-                const int ix = ox * g.sw - g.pl + kx;
-                if (ix < 0 || ix >= g.W) continue;
-                const float4 v = ld4<NT>(i4 + (((size_t)n * g.H + iy) * g.W + ix) * quads + cq);
-                sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+            // eight taps' loads in flight, then their adds in tap order; a tap outside the image adds +0, which
+            // leaves the sum (never -0: it starts from +0) as skipping the tap does
+            const float4 *row = i4 + ((size_t)n * g.H + iy) * g.W * quads + cq;
+            for (int kx0 = 0; kx0 < g.kw; kx0 += 8) {
+                float4 v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int ix = ox * g.sw - g.pl + kx0 + u;
+                    const bool ok = kx0 + u < g.kw && ix >= 0 && ix < g.W;
+                    v[u] = ok ? ld4<NT>(row + (size_t)ix * quads) : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) sum.x += v[u].x, sum.y += v[u].y, sum.z += v[u].z, sum.w += v[u].w;
             }
         }
         st4<NT>(reinterpret_cast<float4 *>(out) + o,

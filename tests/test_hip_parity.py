@@ -325,10 +325,15 @@ def test_maxpool_golden(rt, golden, tag):
     assert_bit_exact(scat.reshape(x.shape), golden[f"pool_{tag}_scatter"], "chosen tap golden")
 
 
-@pytest.mark.parametrize("idims,k,s,p", POOLS)
+@pytest.mark.parametrize("idims,k,s,p", POOLS + [((2, 7, 7, 2048), (7, 7), (1, 1), (0, 0, 0, 0)),        # global pooling
+                                                 ((1, 13, 19, 8), (11, 9), (3, 2), (5, 4, 5, 4)),           # windows wider than 8
+                                                 ((2, 9, 9, 6), (9, 9), (1, 1), (4, 4, 4, 4))])
 def test_avgpool_bit_exact(rt, oracle, idims, k, s, p):
     x = np.random.default_rng(sum(idims)).standard_normal(idims).astype(np.float32)
+    x.flat[::7] = -0.0
     assert_bit_exact(rt.avgpool(rt.upload(x), k, s, p).numpy(), oracle.avgpool(x, k, s, p), "avgpool")
+    z = np.full(idims, -0.0, np.float32)      # all taps -0: the sum starts from +0 either way
+    assert_bit_exact(rt.avgpool(rt.upload(z), k, s, p).numpy(), oracle.avgpool(z, k, s, p), "avgpool of -0")
 
 
 @pytest.mark.parametrize("shape,shuffle", [((2, 3, 5, 7), (0, 2, 3, 1)), ((2, 3, 5, 7), (0, 3, 1, 2)),
