@@ -5,6 +5,7 @@
 #include <cstdlib>
 #include <fstream>
 #include <iomanip>
+#include <set>
 
 #include "../graphIR/IRGraph.h"
 #include "../graphIR/OpNode.h"
@@ -94,8 +95,30 @@ std::string Codegen::UniqueName(std::string name) {
 }
 
 // ------------------------------------------------------------------- set-up
-Codegen::Codegen(IRGraph *graph) : graph_(graph) { config_ = graph->getConfig(); }
-Codegen::Codegen(IRGraph *graph, Config &config) : graph_(graph), config_(config) {}
+Codegen::Codegen(IRGraph *graph) : graph_(graph) {
+    config_ = graph->getConfig();
+    trainAsBatchLoop();
+}
+Codegen::Codegen(IRGraph *graph, Config &config) : graph_(graph), config_(config) { trainAsBatchLoop(); }
+
+// A training program is the batch loop of the inference generator over the training records (reference:
+// src/codegen/Codegen.cpp:952-1019: the same `while(loader.next(label, data))` with the gradient and optimizer
+// calls inside): the training settings are carried over into the fields that loop reads.
+void Codegen::trainAsBatchLoop() {
+    if (!config_.train_mode) return;
+    config_.use_dataloader = true;
+    config_.dataloader_src = config_.train_config.train_data_file;
+    config_.label_bytes = config_.train_config.label_bytes;
+    config_.data_bytes = config_.train_config.data_bytes;
+    config_.dataloader_samples = config_.train_config.train_data_samples;
+    config_.display = config_.train_config.display;
+}
+TensorNode *Codegen::loaderLabelNode() const {
+    return config_.train_mode ? graph_->getTrainLabelNode() : graph_->getInferLabelNode();
+}
+TensorNode *Codegen::loaderDataNode() const {
+    return config_.train_mode ? graph_->getTrainDataNode() : graph_->getInferDataNode();
+}
 
 void Codegen::codeGenInit() {
     mem_allocators_.clear();
@@ -196,18 +219,26 @@ static std::string bracedDims(const std::vector<size_t> &dims) {
 // Config::dataloader_samples records of Config::dataloader_src, mini-batch =
 // dim 0 of the label tensor.
 void Codegen::emitInferDataLoaderInit() {
-    TensorNode *label = graph_->getInferLabelNode();
-    TensorNode *data = graph_->getInferDataNode();
+    TensorNode *label = loaderLabelNode();
+    TensorNode *data = loaderDataNode();
     if (!label || !data) {
-        SWLOG_ERROR << "Config::use_dataloader needs IRGraph::setInferDataNodes(label, data)" << std::endl;
+        SWLOG_ERROR << "the batch loop needs IRGraph::setInferDataNodes(label, data) (training: setTrainDataNodes)" << std::endl;
         std::abort();
     }
     auto proto = [](BytesProto p) { return p == ONE_BYTE_AS_INT ? "ONE_BYTE_AS_INT" : "FOUR_BYTES_AS_FLOAT"; };
     writer_ << "std::string dataloader_infer_source = \"" << config_.dataloader_src << "\";\n";
     writer_ << "DataLoader loader(dataloader_infer_source, " << proto(config_.label_bytes) << ", "
-            << proto(config_.data_bytes) << ", 1, " << config_.dataloader_samples << ", " << bracedDims(label->getDims())
+            << proto(config_.data_bytes) << ", " << (config_.train_mode ? config_.train_config.max_epoch : 1) << ", "
+            << config_.dataloader_samples << ", " << bracedDims(label->getDims())
             << ", " << bracedDims(data->getDims()) << ");\n";
     writer_ << "size_t iter = 0;\n\n";
+}
+
+// TrainingConfig::max_iters > 0 ends the loop early (the reference's ParallelCodegen does the same,
+// src/codegen/ParallelCodegen.cpp:156-157; its single-process loop runs until the epochs are used up).
+void Codegen::emitMaxItersBreak() {
+    if (config_.train_mode && config_.train_config.max_iters > 0)
+        writer_ << "if (iter >= " << config_.train_config.max_iters << ") break;\n";
 }
 
 // Reference: src/codegen/Codegen.cpp:815-854.
@@ -274,7 +305,9 @@ void Codegen::emitMemAllocations() {
             SWLOG_ERROR << "the CPU generator met a GPU-labelled tensor; use HipCodegen (Config::hip)" << std::endl;
             std::abort();
         }
-        writer_ << a->getBasePtrName() << " = (char*)malloc(" << a->getMemAllocated() << ");\n";
+        // (training: zeroed, as the fresh pages of the reference's malloc are — part of a bias gradient is never written)
+        if (config_.train_mode) writer_ << a->getBasePtrName() << " = (char*)calloc(" << a->getMemAllocated() << ", 1);\n";
+        else writer_ << a->getBasePtrName() << " = (char*)malloc(" << a->getMemAllocated() << ");\n";
     }
     writer_ << "\n";
 }
@@ -320,12 +353,12 @@ void Codegen::emitTensorInitializations() {
 
 void Codegen::emitExecute() {
     if (config_.use_dataloader) {   // reference: src/codegen/Codegen.cpp:979-993, 1020-1030
-        writer_ << "while(loader.next(" << nameOf(graph_->getInferLabelNode()) << ", "
-                << nameOf(graph_->getInferDataNode()) << ")) {\n";
+        writer_ << "while(loader.next(" << nameOf(loaderLabelNode()) << ", " << nameOf(loaderDataNode()) << ")) {\n";
         writer_.indentInc();
         emitFuncCalls();
         writer_ << "\niter++;\n";
         if (config_.display > 0) emitPrintGraphOutputs();
+        emitMaxItersBreak();
         writer_.indentDec();
         writer_ << "} //while\n";
         return;
@@ -373,13 +406,19 @@ void Codegen::emitMemFree() {
             writer_ << "free(" << a->getBasePtrName() << ");\n";
 }
 
-// Writes every output-marked tensor that lives on the host to "<name>.bin".
+// Writes every output-marked tensor that lives on the host to "<name>.bin" (a Tensor named by several nodes —
+// a parameter and its updated self — is an output if any of them is marked).
 void Codegen::emitOutputDump() {
     if (!config_.dump_outputs) return;
     writer_ << "\n// dump graph outputs\n";
+    std::set<Tensor *> marked;
+    for (int i = 0; i < graph_->tensorNodeNum(); ++i) {
+        TensorNode *tn = graph_->getTensorNode(i);
+        if (tn->getLabel()->getIsOut() && tn->getLabel()->getDeviceLabel().type == DeviceType::CPU) marked.insert(tn->getTensor());
+    }
     for (TensorNode *tn : decl_order_) {
-        if (!tn->getLabel()->getIsOut() || tn->getLabel()->getDeviceLabel().type != DeviceType::CPU) continue;
         Tensor *t = tn->getTensor();
+        if (!marked.count(t)) continue;
         writer_ << "store(" << tensors_name_map_.at(t) << ", " << t->size() << ", \"" << tensors_name_map_.at(t)
                 << ".bin\");\n";
     }
@@ -466,6 +505,52 @@ void Codegen::emitFuncCall(OpNode *op) {
     } else if (type == "Accuracy") {   // Codegen.cpp:2387-2398
         writer_ << "accuracy_i(" << nameOf(in(0)) << ", " << nameOf(in(1)) << ", " << nameOf(out(0)) << ", "
                 << T(in(0))->getDim(0) << ", " << T(in(0))->getDim(1) << ");\n";
+    } else if (type == "BatchedReduceAdd") {   // Codegen.cpp:1517-1531
+        const auto rc = T(in(0))->viewAs2D(T(in(0))->getNDim() - 1);
+        if (rc.first > T(out(0))->size()) {   // one sum per ROW goes into the result (kernels.h:554-563): it must hold them
+            SWLOG_ERROR << "BatchedReduceAdd " << nm << ": " << rc.first << " rows into a result of " << T(out(0))->size()
+                        << " elements — the reference's kernel would write past it (mini-batch larger than the layer)" << std::endl;
+            std::abort();
+        }
+        writer_ << "batchedreduceadd_f(" << nameOf(out(0)) << ", " << nameOf(in(0)) << ", " << rc.first << ", " << rc.second
+                << ");\n";
+    } else if (type == "ReluGrad") {   // Codegen.cpp:2138-2148: parents input, outputGrad
+        writer_ << "reluGrad_f(" << nameOf(out(0)) << ", " << nameOf(in(0)) << ", " << nameOf(in(1)) << ", "
+                << T(in(0))->size() << ");\n";
+    } else if (type == "MatrixTanhGrad") {   // Codegen.cpp:2414-2427: parents input, output, outputGrad
+        const size_t m = T(in(0))->getDim(0), n = T(in(0))->getDim(1);
+        writer_ << "matrixTanhGrad_f(" << m << ", " << n << ", " << nameOf(out(0)) << ", " << n << ", " << nameOf(in(1))
+                << ", " << n << ", " << nameOf(in(2)) << ", " << n << ");\n";
+    } else if (type == "MaxPoolGrad") {   // Codegen.cpp:2047-2079: parents input, output, outputGrad
+        auto *pool = static_cast<MaxPoolGradOp *>(op->getOp());
+        writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims()) << arrayDef(nm + "_outDims", T(in(1))->getDims())
+                << arrayDef(nm + "_filterSizes", pool->getKernels()) << arrayDef(nm + "_strides", pool->getStrides())
+                << arrayDef(nm + "_pads", pool->getPads());
+        writer_ << "maxpoolGrad_f(" << nameOf(out(0)) << ", " << nameOf(in(2)) << ", " << nameOf(in(0)) << ", " << nm
+                << "_inDims, " << nm << "_outDims, " << nm << "_filterSizes, " << nm << "_strides, " << nm << "_pads);\n";
+    } else if (type == "Conv2dGrad") {   // Codegen.cpp:1785-1830: parents input, filter, outputGrad
+        auto *conv = static_cast<Conv2dGradOp *>(op->getOp());
+        writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims()) << arrayDef(nm + "_outDims", T(in(2))->getDims())
+                << arrayDef(nm + "_filterDims", T(in(1))->getDims()) << arrayDef(nm + "_biasDims", T(out(2))->getDims())
+                << arrayDef(nm + "_filterSizes", conv->getKernels()) << arrayDef(nm + "_strides", conv->getStrides())
+                << arrayDef(nm + "_pads", conv->getPads());
+        writer_ << "conv2dGrad_f(" << nameOf(out(0)) << ", " << nameOf(out(1)) << ", " << nameOf(out(2)) << ", "
+                << nameOf(in(2)) << ", " << nameOf(in(0)) << ", " << nameOf(in(1)) << ", " << nm << "_outDims, " << nm
+                << "_inDims, " << nm << "_filterDims, " << nm << "_biasDims, " << nm << "_filterSizes, " << nm
+                << "_strides, " << nm << "_pads, " << conv->getGroup() << ");\n";
+    } else if (type == "MatrixSoftmaxWithLoss") {   // Codegen.cpp:2357-2370: parents logits, label -> prob, loss
+        const size_t m = T(in(0))->getDim(0), n = T(in(0))->getDim(1);
+        writer_ << "matrixSoftmaxWithLoss_f(" << m << ", " << n << ", " << nameOf(in(0)) << ", " << n << ", "
+                << nameOf(out(0)) << ", " << n << ", " << nameOf(in(1)) << ", " << nameOf(out(1)) << ");\n";
+    } else if (type == "MatrixSoftmaxWithLossGrad") {   // Codegen.cpp:2446-2465: parents label, prob
+        const size_t m = T(in(1))->getDim(0), n = T(in(1))->getDim(1);
+        writer_ << "matrixSoftmaxWithLossGrad_f(" << m << ", " << n << ", " << nameOf(out(0)) << ", " << n << ", "
+                << nameOf(in(1)) << ", " << n << ", " << nameOf(in(0)) << ");\n";
+    } else if (type == "SGD") {   // Codegen.cpp:2468-2489: parents parameter, gradient, momentum; in place
+        auto *sgd = static_cast<SGDOp *>(op->getOp());
+        writer_ << "sgd_f(" << T(in(0))->size() << ", " << nameOf(in(0)) << ", " << nameOf(in(0)) << ", " << nameOf(in(1))
+                << ", " << nameOf(in(2)) << ", " << sgd->getLR() << ", " << sgd->getDecay() << ", " << sgd->getMomentum()
+                << ", " << sgd->getBatch() << ");\n";
     } else if (type == "Debug") {   // Codegen.cpp:2401-2412
         Tensor *a = T(in(0));
         writer_ << "printMatrix(" << nameOf(in(0)) << ", " << a->getDim(0) << ", "

@@ -124,7 +124,11 @@ class Codegen {
     virtual void emitExecute();
     virtual void emitFuncCalls();
     virtual void emitMemFree();
-    virtual void emitDataLoaderInit() {}          // training loader: not part of the inference build
+    virtual void emitDataLoaderInit() {}          // (the training loader is emitInferDataLoaderInit over the training records)
+    void emitMaxItersBreak();
+    void trainAsBatchLoop();                       // Config::train_mode: the training settings become the batch loop's
+    TensorNode *loaderLabelNode() const;           // what loader.next fills: the training or the inference pair
+    TensorNode *loaderDataNode() const;
     virtual void emitInferDataLoaderInit();        // `DataLoader loader(...)` + iteration counter
     virtual void emitPrintGraphOutputs();          // every Config::display iterations: the display tensors
 

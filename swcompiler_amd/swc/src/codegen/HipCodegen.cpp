@@ -40,7 +40,7 @@ void HipCodegen::initMakefileBuilder() {
 void HipCodegen::emitHeader() {
     headerWriter_ << "// Graph.cpp -- generated from an IRGraph with " << graph_->tensorNodeNum() << " tensor nodes and "
                   << graph_->opNodeNum() << " op nodes (HIP target, " << device_.arch << ")\n";
-    headerWriter_ << "#include <algorithm>\n#include <iostream>\n#include <random>\n#include <cstdlib>\n#include <cstdio>\n#include <cmath>\n"
+    headerWriter_ << "#include <algorithm>\n#include <iostream>\n#include <random>\n#include <cstdlib>\n#include <cstdio>\n#include <cstring>\n#include <cmath>\n"
                   << "#include <sys/time.h>\n"
                   << "#include \"swc_host_utils.h\"\n#include \"swc_hip.h\"\n";
     headerWriter_ << "#define SWC_HIP_CHECK(call) do { if ((call) != 0) { std::fprintf(stderr, \"%s:%d: %s\\n  %s\\n\", "
@@ -103,7 +103,8 @@ void HipCodegen::emitWorkspace() {
 }
 
 void HipCodegen::emitMemAllocations() {
-    emitWorkspace();
+    // (a training program leaves the scratch memory to the library: the gradient kernels size their own)
+    if (!config_.train_mode) emitWorkspace();
     for (auto &a : mem_allocators_) {
         if (!a->getMemAllocated()) continue;
         if (a->getDevice().type == DeviceType::CPU) {
@@ -115,6 +116,15 @@ void HipCodegen::emitMemAllocations() {
             writer_ << a->getBasePtrName() << " = (char*)swc_hip_malloc(" << a->getMemAllocated() << ");\n";
             writer_ << "if (!" << a->getBasePtrName() << ") { std::fprintf(stderr, \"%s\\n\", swc_hip_last_error()); "
                     << "return 1; }\n";
+        }
+        // training: gradients start from zeros wherever a kernel leaves part of one unwritten (the bias
+        // gradient of an FC layer, see BatchedReduceAdd) — what fresh pages give the CPU program
+        if (config_.train_mode) {
+            if (a->getDevice().type == DeviceType::CPU)
+                writer_ << "std::memset(" << a->getBasePtrName() << ", 0, " << a->getMemAllocated() << ");\n";
+            else
+                writer_ << "SWC_HIP_CHECK(swc_hip_fill_f(reinterpret_cast<float*>(" << a->getBasePtrName() << "), 0.f, "
+                        << a->getMemAllocated() / 4 << "));\n";
         }
     }
     writer_ << "\n";
@@ -230,6 +240,18 @@ void HipCodegen::emitExecute() {
         emitDeviceOpsOnly();
         writer_.indentDec();
         writer_ << "}\n";
+        if (config_.train_mode) {
+            // the warm-up pass has taken an optimizer step on whatever the arena held: parameters and momenta
+            // are uploaded again
+            writer_ << "// parameters and momenta as they were before the warm-up pass\n";
+            for (int i = 0; i < graph_->topologyNum(); ++i)
+                for (int j = 0; j < graph_->getNumInTopoLevel(i); ++j) {
+                    IRNode *node = graph_->getNodeInTopo(i, j);
+                    if (node->nodeType() != OP_NODE) continue;
+                    auto *op = static_cast<OpNode *>(node);
+                    if (op->isRunOnce() && op->getOp()->getOpName() == "Scatter") emitTransfer(op, true);
+                }
+        }
         emitDeviceFills();   // counters the warm-up pass has touched start again
         writer_ << "SWC_HIP_CHECK(swc_hip_sync());\n";
         writer_ << "void *swc_graph = NULL;\n";
@@ -249,8 +271,7 @@ void HipCodegen::emitExecute() {
                 if (!op->isRunOnce() && op->getOp()->getOpName() == "Scatter") uploads.push_back(op);
             }
         const bool prefetch = config_.hip_prefetch && !uploads.empty();
-        const std::string next = "loader.next(" + nameOf(graph_->getInferLabelNode()) + ", " +
-                                 nameOf(graph_->getInferDataNode()) + ")";
+        const std::string next = "loader.next(" + nameOf(loaderLabelNode()) + ", " + nameOf(loaderDataNode()) + ")";
         auto stageName = [&](OpNode *u) { return nameOf(u->getChildNode(0)) + "_stage"; };
         auto bytesOf = [&](OpNode *u) {
             return std::min(T(u->getParentNode(0))->getSizeInBytes(), T(u->getChildNode(0))->getSizeInBytes());
@@ -396,6 +417,10 @@ bool HipCodegen::deviceOpsAreContiguous() const {
             if (node->nodeType() != OP_NODE) continue;
             auto *op = static_cast<OpNode *>(node);
             if (op->isRunOnce()) continue;
+            // (a download nobody on the host reads is not part of the batch loop's body: it is emitted where its
+            // tensor is displayed and after the loop)
+            if (config_.use_dataloader && op->getOp()->getOpName() == "Gather" && op->getChildNode(0)->childNum() == 0)
+                continue;
             if (isDeviceComputeOp(op)) {
                 if (phase == 2) return false;
                 phase = 1;
@@ -598,6 +623,53 @@ void HipCodegen::emitHipCall(OpNode *op) {
         const int topK = static_cast<ArgMaxOp *>(op->getOp())->getTopK();
         writer_ << "SWC_HIP_CHECK(swc_hip_argMax_i(" << nameOf(in(0)) << ", " << nameOf(out(0)) << ", "
                 << T(in(0))->getDim(0) << ", " << T(in(0))->getDim(1) << ", " << topK << "));\n";
+    } else if (type == "BatchedReduceAdd") {
+        const auto rc = T(in(0))->viewAs2D(T(in(0))->getNDim() - 1);
+        if (rc.first > T(out(0))->size()) {   // one sum per ROW goes into the result (kernels.h:554-563): it must hold them
+            SWLOG_ERROR << "BatchedReduceAdd " << nm << ": " << rc.first << " rows into a result of " << T(out(0))->size()
+                        << " elements — the reference's kernel would write past it (mini-batch larger than the layer)" << std::endl;
+            std::abort();
+        }
+        writer_ << "SWC_HIP_CHECK(swc_hip_batchedreduceadd_f(" << nameOf(out(0)) << ", " << nameOf(in(0)) << ", " << rc.first
+                << ", " << rc.second << "));\n";
+    } else if (type == "ReluGrad") {
+        writer_ << "SWC_HIP_CHECK(swc_hip_reluGrad_f(" << nameOf(out(0)) << ", " << nameOf(in(0)) << ", " << nameOf(in(1))
+                << ", " << T(in(0))->size() << "));\n";
+    } else if (type == "MatrixTanhGrad") {
+        const size_t m = T(in(0))->getDim(0), n = T(in(0))->getDim(1);
+        writer_ << "SWC_HIP_CHECK(swc_hip_matrixTanhGrad_f(" << m << ", " << n << ", " << nameOf(out(0)) << ", " << n << ", "
+                << nameOf(in(1)) << ", " << n << ", " << nameOf(in(2)) << ", " << n << "));\n";
+    } else if (type == "MaxPoolGrad") {
+        auto *pool = static_cast<MaxPoolGradOp *>(op->getOp());
+        writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims()) << arrayDef(nm + "_outDims", T(in(1))->getDims())
+                << arrayDef(nm + "_filterSizes", pool->getKernels()) << arrayDef(nm + "_strides", pool->getStrides())
+                << arrayDef(nm + "_pads", pool->getPads());
+        writer_ << "SWC_HIP_CHECK(swc_hip_maxpoolGrad_f(" << nameOf(out(0)) << ", " << nameOf(in(2)) << ", " << nameOf(in(0))
+                << ", " << nm << "_inDims, " << nm << "_outDims, " << nm << "_filterSizes, " << nm << "_strides, " << nm
+                << "_pads));\n";
+    } else if (type == "Conv2dGrad") {
+        auto *conv = static_cast<Conv2dGradOp *>(op->getOp());
+        writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims()) << arrayDef(nm + "_outDims", T(in(2))->getDims())
+                << arrayDef(nm + "_filterDims", T(in(1))->getDims()) << arrayDef(nm + "_biasDims", T(out(2))->getDims())
+                << arrayDef(nm + "_filterSizes", conv->getKernels()) << arrayDef(nm + "_strides", conv->getStrides())
+                << arrayDef(nm + "_pads", conv->getPads());
+        writer_ << "SWC_HIP_CHECK(swc_hip_conv2dGrad_f(" << nameOf(out(0)) << ", " << nameOf(out(1)) << ", " << nameOf(out(2))
+                << ", " << nameOf(in(2)) << ", " << nameOf(in(0)) << ", " << nameOf(in(1)) << ", " << nm << "_outDims, "
+                << nm << "_inDims, " << nm << "_filterDims, " << nm << "_biasDims, " << nm << "_filterSizes, " << nm
+                << "_strides, " << nm << "_pads, " << conv->getGroup() << "));\n";
+    } else if (type == "MatrixSoftmaxWithLoss") {
+        const size_t m = T(in(0))->getDim(0), n = T(in(0))->getDim(1);
+        writer_ << "SWC_HIP_CHECK(swc_hip_matrixSoftmaxWithLoss_f(" << m << ", " << n << ", " << nameOf(in(0)) << ", " << n
+                << ", " << nameOf(out(0)) << ", " << n << ", " << nameOf(in(1)) << ", " << nameOf(out(1)) << "));\n";
+    } else if (type == "MatrixSoftmaxWithLossGrad") {
+        const size_t m = T(in(1))->getDim(0), n = T(in(1))->getDim(1);
+        writer_ << "SWC_HIP_CHECK(swc_hip_matrixSoftmaxWithLossGrad_f(" << m << ", " << n << ", " << nameOf(out(0)) << ", " << n
+                << ", " << nameOf(in(1)) << ", " << n << ", " << nameOf(in(0)) << "));\n";
+    } else if (type == "SGD") {
+        auto *sgd = static_cast<SGDOp *>(op->getOp());
+        writer_ << "SWC_HIP_CHECK(swc_hip_sgd_f(" << T(in(0))->size() << ", " << nameOf(in(0)) << ", " << nameOf(in(0)) << ", "
+                << nameOf(in(1)) << ", " << nameOf(in(2)) << ", " << sgd->getLR() << ", " << sgd->getDecay() << ", "
+                << sgd->getMomentum() << ", " << sgd->getBatch() << "));\n";
     } else if (type == "Accuracy") {
         writer_ << "SWC_HIP_CHECK(swc_hip_accuracy_i(" << nameOf(in(0)) << ", " << nameOf(in(1)) << ", " << nameOf(out(0))
                 << ", " << T(in(0))->getDim(0) << ", " << T(in(0))->getDim(1) << "));\n";

@@ -14,12 +14,40 @@ using namespace pass;
 
 void Engine::compile() {
     const Config cfg = graph_->getConfig();
-    if (cfg.train_mode || cfg.mpi || cfg.mkldnn || cfg.cuda) {
-        SWLOG_ERROR << "Engine: only the inference pipeline (CPU or Config::hip) is part of this build" << std::endl;
+    if (cfg.mpi || cfg.mkldnn || cfg.cuda) {
+        SWLOG_ERROR << "Engine: only the single-device pipelines (CPU or Config::hip) are part of this build" << std::endl;
         std::abort();
     }
-    runInferPasses();
+    if (cfg.train_mode) runTrainPasses();
+    else runInferPasses();
     if (cfg.hip) transformForHIP();
+}
+
+// autodiff on the graph itself, then labeling -> lowering -> labeling -> renaming -> elimination
+// (reference order: src/engine/Engine.cpp:88-126).  The updated parameters are the graph's outputs; what
+// leads to none of them or to a displayed tensor (the loss) is removed.
+void Engine::runTrainPasses() {
+    const Config cfg = graph_->getConfig();
+    AutodiffPass autodiff(graph_);
+    autodiff.getMethods(cfg.train_config.optimizer, cfg.train_config.lr, cfg.train_config.decay, cfg.train_config.momentum,
+                        cfg.train_config.batch);
+    autodiff.run();
+    LabelingPass labeling(graph_);
+    LoweringPass lowering(graph_);
+    RenamingNodePass renaming(graph_);
+    PassManager pm;
+    pm.add(&labeling);
+    pm.add(&lowering);
+    pm.add(&labeling);
+    pm.add(&renaming);
+    pm.run();
+    graph_->findInOut();
+    graph_->updateTopology();
+    graph_->clearOutMark();
+    graph_->setLogicalOutMark();
+    for (TensorNode *t : graph_->getDisplayTensorNodes()) t->getLabel()->setIsOut(1);
+    EliminationPass elimination(graph_);
+    elimination.run();
 }
 
 // labeling -> lowering -> labeling (new nodes) -> renaming, then refresh the

@@ -27,6 +27,7 @@ class Engine {
     IRGraph *getGraph() { return graph_; }
     virtual void compile();
     void runInferPasses();
+    void runTrainPasses();
     // HIP target only: fusion (if enabled) + device placement + renaming
     virtual void transformForHIP();
     std::string genCode();

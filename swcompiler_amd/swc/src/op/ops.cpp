@@ -155,6 +155,64 @@ static void lowerFC(IRGraph *graph, IRNode *node, bool withBias) {
     graph->updateTopology();
 }
 
+// prob has the logits' shape, loss is one number
+void MatrixSoftmaxWithLossOp::outTensorShapeGen(OpNode *node, size_t index, TensorShape *shape) {
+    if (index == 0) shape->setShape(static_cast<TensorNode *>(node->getParentNode(0))->getDims());
+    else shape->setShape({1});
+}
+
+// Y = X W + b (reference: src/op/dlOp/dlOpEinsum.cpp:239-318):
+//   dX = dY * W^T      dW = X^T * dY      db = column sums of dY
+// X of rank > 2 is read as [dim0, rest] through a Reshape alias; dX keeps X's shape (same storage size).
+void MatrixMatrixFCBiasGradOp::lowering(IRGraph *graph, IRNode *node) {
+    auto *input = static_cast<TensorNode *>(node->getParentNode(0));
+    auto *weight = static_cast<TensorNode *>(node->getParentNode(1));
+    auto *bias = static_cast<TensorNode *>(node->getParentNode(2));
+    auto *outputG = static_cast<TensorNode *>(node->getParentNode(3));
+    auto *inputG = static_cast<TensorNode *>(node->getChildNode(0));
+    auto *weightG = static_cast<TensorNode *>(node->getChildNode(1));
+    auto *biasG = static_cast<TensorNode *>(node->getChildNode(2));
+
+    auto *wT_op = new OpNode("op_" + weight->name() + "_T", new TransposeOp({1, 0}));
+    wT_op->exlinkUpperNode(weight);
+    auto *wT = new TensorNode(weight->name() + "_T", new Tensor(weight->getTensor()->getShuffledTensorShape({1, 0})), wT_op);
+    auto *dx = new OpNode(node->name() + "_dx_mm", new MatrixMatrixMulOp());
+    dx->exlinkUpperNode(outputG, wT);
+
+    TensorNode *x2d = input;
+    if (input->getTensor()->getNDim() > 2) {
+        const auto rc = input->getTensor()->viewAs2D(1);
+        std::vector<size_t> flat{rc.first, rc.second};
+        auto *reshape = new OpNode(input->name() + "_reshape_op", new ReshapeOp(flat));
+        reshape->exlinkUpperNode(input);
+        x2d = new TensorNode(input->name() + "_reshape", new Tensor({rc.first, rc.second}), reshape);
+        graph->pushOpNode(reshape);
+        graph->pushTensorNode(x2d);
+    }
+    auto *xT_op = new OpNode("op_" + x2d->name() + "_T", new TransposeOp({1, 0}));
+    xT_op->exlinkUpperNode(x2d);
+    auto *xT = new TensorNode(x2d->name() + "_T", new Tensor(x2d->getTensor()->getShuffledTensorShape({1, 0})), xT_op);
+    auto *dw = new OpNode(node->name() + "_dw_mm", new MatrixMatrixMulOp());
+    dw->exlinkUpperNode(xT, outputG);
+    auto *db = new OpNode(node->name() + "_db_bra", new BatchedReduceAddOp());
+    db->exlinkUpperNode(outputG);
+
+    node->destroyUpperNode(input);
+    node->destroyUpperNode(weight);
+    node->destroyUpperNode(bias);
+    node->destroyUpperNode(outputG);
+    inputG->destroyUpperNode(node);
+    weightG->destroyUpperNode(node);
+    biasG->destroyUpperNode(node);
+    inputG->exlinkUpperNode(dx);
+    weightG->exlinkUpperNode(dw);
+    biasG->exlinkUpperNode(db);
+    graph->delOpNode(static_cast<OpNode *>(node));
+    graph->pushOpNode(wT_op, xT_op, dx, dw, db);
+    graph->pushTensorNode(wT, xT);
+    graph->updateTopology();
+}
+
 void MatrixMatrixFCOp::lowering(IRGraph *graph, IRNode *node) { lowerFC(graph, node, false); }
 void MatrixMatrixFCBiasOp::lowering(IRGraph *graph, IRNode *node) { lowerFC(graph, node, true); }
 

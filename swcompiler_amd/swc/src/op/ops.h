@@ -267,6 +267,75 @@ class Conv2dBatchNormOp : public Conv2dOp {
     float getEpsilon() const { return epsilon_; }
     bool hasRelu() const { return relu_; }
 };
+// ---- training: the loss, the gradient ops the autodiff pass creates, the optimizer step ----
+// (reference: src/op/dlOp/dlOp.h:61-75, 121-141, 182-193, 213-222, 243-256, 290-336, 600-640, 715-770)
+// parents: logits [m,n], label [m] int32 -> prob [m,n], loss [1]
+class MatrixSoftmaxWithLossOp : public Op {
+  public:
+    MatrixSoftmaxWithLossOp() : Op(DL_OP, 2, 2, "MatrixSoftmaxWithLoss") {}
+    void outTensorShapeGen(OpNode *node, size_t index, TensorShape *shape) override;
+};
+// parents: label, prob -> gradient of the logits
+class MatrixSoftmaxWithLossGradOp : public Op {
+  public:
+    MatrixSoftmaxWithLossGradOp() : Op(DL_OP, 2, 1, "MatrixSoftmaxWithLossGrad") {}
+};
+// parents: input, weight, bias, outputGrad -> inputGrad, weightGrad, biasGrad; always lowered to
+// Transpose + MatrixMatrixMul (twice) + BatchedReduceAdd
+class MatrixMatrixFCBiasGradOp : public Op {
+  public:
+    MatrixMatrixFCBiasGradOp() : Op(DL_OP, 4, 3, "MatrixMatrixFCBiasGrad") {}
+    void lowering(IRGraph *graph, IRNode *node) override;
+};
+class BatchedReduceAddOp : public Op {    // out[j] = sum over rows of in[r, j]
+  public:
+    BatchedReduceAddOp() : Op(DL_OP, 1, 1, "BatchedReduceAdd") {}
+};
+class MatrixTanhGradOp : public Op {      // parents: input, output, outputGrad
+  public:
+    MatrixTanhGradOp() : Op(DL_OP, 3, 1, "MatrixTanhGrad") {}
+};
+class ReluGradOp : public Op {            // parents: input, outputGrad
+  public:
+    ReluGradOp() : Op(DL_OP, 2, 1, "ReluGrad") {}
+};
+class MaxPoolGradOp : public Op {         // parents: input, output, outputGrad
+    std::vector<size_t> kernels_, strides_, pads_;
+
+  public:
+    MaxPoolGradOp(const std::vector<size_t> &kernels, const std::vector<size_t> &strides, const std::vector<size_t> &pads)
+        : Op(DL_OP, 3, 1, "MaxPoolGrad"), kernels_(kernels), strides_(strides), pads_(pads) {}
+    std::vector<size_t> getPads() const { return pads_; }
+    std::vector<size_t> getKernels() const { return kernels_; }
+    std::vector<size_t> getStrides() const { return strides_; }
+};
+class Conv2dGradOp : public Op {          // parents: input, filter, outputGrad -> inputGrad, filterGrad, biasGrad
+    std::vector<size_t> kernels_, strides_, pads_;
+    int group_;
+
+  public:
+    Conv2dGradOp(const std::vector<size_t> &kernels, const std::vector<size_t> &strides, const std::vector<size_t> &pads,
+                 int group)
+        : Op(DL_OP, 3, 3, "Conv2dGrad"), kernels_(kernels), strides_(strides), pads_(pads), group_(group) {}
+    std::vector<size_t> getPads() const { return pads_; }
+    std::vector<size_t> getKernels() const { return kernels_; }
+    std::vector<size_t> getStrides() const { return strides_; }
+    size_t getGroup() const { return (size_t)group_; }
+};
+// parents: parameter, its gradient, its momentum -> the parameter again (same Tensor: updated in place)
+class SGDOp : public Op {
+    float lr_, decay_, momentum_;
+    size_t batch_;
+
+  public:
+    SGDOp(float lr, float decay, float momentum, size_t batch)
+        : Op(DL_OP, 3, 1, "SGD"), lr_(lr), decay_(decay), momentum_(momentum), batch_(batch) {}
+    float getLR() const { return lr_; }
+    float getDecay() const { return decay_; }
+    float getMomentum() const { return momentum_; }
+    size_t getBatch() const { return batch_; }
+};
+
 // Conv2d (+ BatchNormalization) + ElementAdd (+ Relu): the last convolution of a residual block with the sum
 // and the activation that follow it.  Parents: input, filter, bias, [bn scale, bias, mean, var,] the other
 // summand.  swc_hip_conv2dFusedAdd_f

@@ -1,7 +1,10 @@
 #include "passes.h"
 
 #include <cassert>
+#include <cctype>
+#include <cstdlib>
 #include <set>
+#include <unordered_map>
 #include <unordered_set>
 
 #include "../graphIR/OpNode.h"
@@ -46,7 +49,7 @@ void LabelingPass::run() {
         // FC without bias always becomes a plain GEMM.  FC with bias is split
         // into GEMM + bias-add only for targets without a fused kernel: the CPU
         // generator; MKL-DNN and the HIP target keep it whole.
-        if (type == "MatrixMatrixFC") l->setLowerMark();
+        if (type == "MatrixMatrixFC" || type == "MatrixMatrixFCBiasGrad") l->setLowerMark();   // (no target has a kernel for the latter)
         else if (type == "MatrixMatrixFCBias" && !cfg.mkldnn && !cfg.hip) l->setLowerMark();
     }
 }
@@ -105,6 +108,10 @@ void EliminationPass::run() {
         for (IRNode *p : n->getParentNodes())
             if (live.insert(p).second) work.push_back(p);
     }
+    // every result of a live op stays, read or not: the op's emitter addresses its results by position
+    for (int i = 0; i < _graph->opNodeNum(); ++i)
+        if (live.count(_graph->getOpNode(i)))
+            for (IRNode *c : _graph->getOpNode(i)->getChildNodes()) live.insert(c);
     std::vector<TensorNode *> deadT;
     std::vector<OpNode *> deadO;
     for (int i = 0; i < _graph->tensorNodeNum(); ++i)
@@ -122,6 +129,96 @@ void EliminationPass::run() {
     for (auto *o : deadO) {
         detach(o);
         _graph->delOpNode(o);
+    }
+    _graph->findInOut();
+    _graph->updateTopology();
+}
+
+// ------------------------------------------------------------------ autodiff
+void AutodiffPass::getMethods(const std::string &method, float lr, float decay, float momentum, size_t batch) {
+    std::string m = method;
+    for (char &c : m) c = (char)std::tolower((unsigned char)c);
+    if (m != "sgd") {
+        SWLOG_ERROR << "AutodiffPass: optimizer \"" << method << "\" is not implemented (sgd)" << std::endl;
+        std::abort();
+    }
+    lr_ = lr, decay_ = decay, momentum_ = momentum, batch_ = batch;
+}
+
+void AutodiffPass::run() {
+    std::vector<IRNode *> order;
+    for (int i = 0; i < _graph->topologyNum(); ++i)
+        for (int j = 0; j < _graph->getNumInTopoLevel(i); ++j) order.push_back(_graph->getNodeInTopo(i, j));
+    std::unordered_map<IRNode *, TensorNode *> gradOf;
+
+    // gradient op with the given operands; one gradient tensor per operand of the forward op, in operand order
+    auto addGrad = [&](OpNode *fwd, Op *gradOp, const std::vector<IRNode *> &operands) {
+        auto *g = new OpNode(fwd->name() + "_grad", gradOp);
+        for (IRNode *p : operands) g->exlinkUpperNode(p);
+        _graph->pushOpNode(g);
+        for (int i = 0; i < fwd->parentNum(); ++i) {
+            auto *t = static_cast<TensorNode *>(fwd->getParentNode(i));
+            auto *gt = new TensorNode(t->name() + "_grad", new Tensor(new TensorShape(t->getDims())), g);
+            gradOf[t] = gt;
+            _graph->pushTensorNode(gt);
+        }
+        ++gradOps_;
+    };
+
+    for (auto it = order.rbegin(); it != order.rend(); ++it) {
+        IRNode *node = *it;
+        if (node->nodeType() == TENSOR_NODE) {
+            auto *t = static_cast<TensorNode *>(node);
+            if (gradOf.count(t)) {
+                if (!t->getTraining()) continue;
+                auto *momT = new Tensor(new TensorShape(t->getDims()));
+                momT->setTensorInit(TensorInitType::CONSTANT, 0.f);
+                auto *mom = new TensorNode(t->name() + "_momentum", momT);
+                auto *sgd = new OpNode(t->name() + "_sgd", new SGDOp(lr_, decay_, momentum_, batch_));
+                sgd->exlinkUpperNode(t, gradOf[t], mom);
+                auto *updated = new TensorNode(t->name(), t->getTensor(), sgd);   // the same Tensor: in place
+                updated->setTraining(t->getTraining());
+                _graph->pushOpNode(sgd);
+                _graph->pushTensorNode(mom, updated);
+                _graph->addLogicalOutNodes(updated);
+                ++sgdOps_;
+            } else if (t->childNum() == 0) {
+                // an end point (loss, probabilities): its gradient exists by name only, no op computes or reads it
+                gradOf[t] = new TensorNode(t->name() + "_grad", new Tensor(new TensorShape(t->getDims())));
+            }
+            continue;
+        }
+        auto *op = static_cast<OpNode *>(node);
+        const std::string type = op->getOp()->getOpName();
+        auto in = [&](int i) { return op->getParentNode(i); };
+        auto outGrad = [&]() -> IRNode * {
+            auto *out = static_cast<TensorNode *>(op->getChildNode(0));
+            if (!gradOf.count(out)) {
+                SWLOG_ERROR << "AutodiffPass: no gradient reaches the output of " << op->name() << std::endl;
+                std::abort();
+            }
+            return gradOf[out];
+        };
+        if (type == "MatrixMatrixFCBias") {
+            addGrad(op, new MatrixMatrixFCBiasGradOp(), {in(0), in(1), in(2), outGrad()});
+        } else if (type == "MatrixTanh") {
+            addGrad(op, new MatrixTanhGradOp(), {in(0), op->getChildNode(0), outGrad()});
+        } else if (type == "Relu") {
+            addGrad(op, new ReluGradOp(), {in(0), outGrad()});
+        } else if (type == "MaxPool") {
+            auto *mp = static_cast<MaxPoolOp *>(op->getOp());
+            addGrad(op, new MaxPoolGradOp(mp->getKernels(), mp->getStrides(), mp->getPads()),
+                    {in(0), op->getChildNode(0), outGrad()});
+        } else if (type == "Conv2d") {
+            auto *cv = static_cast<Conv2dOp *>(op->getOp());
+            addGrad(op, new Conv2dGradOp(cv->getKernels(), cv->getStrides(), cv->getPads(), (int)cv->getGroup()),
+                    {in(0), in(1), outGrad()});
+        } else if (type == "MatrixSoftmaxWithLoss") {
+            addGrad(op, new MatrixSoftmaxWithLossGradOp(), {in(1), op->getChildNode(0)});   // label, prob
+        } else {
+            SWLOG_ERROR << "AutodiffPass: no gradient for op type " << type << " (node " << op->name() << ")" << std::endl;
+            std::abort();
+        }
     }
     _graph->findInOut();
     _graph->updateTopology();
@@ -314,7 +411,9 @@ bool DeviceMemoryLoweringPass::runsOnGpu(const std::string &t) {
         "MatrixMatrixFCBiasSoftmax", "Reshape", "MatrixTanh", "MatrixSoftmax", "ElementAdd", "ElementAddRelu", "Relu", "Dropout",
         "Conv2d", "Conv2dWithActivation", "Conv2dBatchNorm", "Conv2dAdd", "MaxPool", "AveragePool", "Transpose",
         "BatchNormalization",
-        "BatchNormalizationRelu", "BatchNormReluMaxPool", "ArgMax", "Accuracy"};
+        "BatchNormalizationRelu", "BatchNormReluMaxPool", "ArgMax", "Accuracy",
+        "MatrixSoftmaxWithLoss", "MatrixSoftmaxWithLossGrad", "BatchedReduceAdd", "MatrixTanhGrad", "ReluGrad",
+        "MaxPoolGrad", "Conv2dGrad", "SGD"};
     return gpu.count(t) != 0;
 }
 
@@ -355,14 +454,19 @@ void DeviceMemoryLoweringPass::run() {
             auto *scatter = new OpNode(t->name() + "_h2d", new ScatterOp());
             scatter->getLabel()->setDeviceLabel(gpu);
             scatter->getLabel()->setTypeNameLabel("Scatter");
-            const bool perIteration = cfg.use_dataloader &&
-                                      (t == _graph->getInferDataNode() || t == _graph->getInferLabelNode());
+            const bool perIteration =
+                cfg.train_mode ? (t == _graph->getTrainDataNode() || t == _graph->getTrainLabelNode())
+                               : cfg.use_dataloader && (t == _graph->getInferDataNode() || t == _graph->getInferLabelNode());
             const bool parameter = t->parentNum() == 0 && !perIteration;
             if (parameter) {
                 scatter->setRunOnce();
                 twin->getTensor()->setTensorInit(TensorInitType::PARENTOP);
             }
             for (IRNode *reader : gpuReaders) t->replaceUseKeepOrder(reader, twin);
+            // a device node that names the same Tensor (the parameter as an SGD node rewrites it in place) means
+            // the device copy from now on
+            for (TensorNode *other : tensors)
+                if (other != t && other->getTensor() == t->getTensor() && onGpu(other)) other->setTensor(twin->getTensor());
             scatter->exlinkUpperNode(t);
             twin->exlinkUpperNode(scatter);
             _graph->pushOpNode(scatter);
@@ -374,7 +478,9 @@ void DeviceMemoryLoweringPass::run() {
             for (IRNode *c : t->getChildNodes())
                 if (!onGpu(c) && std::find(hostReaders.begin(), hostReaders.end(), c) == hostReaders.end())
                     hostReaders.push_back(c);
-            bool isOutput = t->getLabel()->getIsOut() != 0 || t->childNum() == 0;
+            // (a training graph marks its outputs — the updated parameters, the displayed loss; a gradient nobody
+            // reads, such as the one a conv2dGrad computes for the data, is not one)
+            bool isOutput = t->getLabel()->getIsOut() != 0 || (!cfg.train_mode && t->childNum() == 0);
             for (IRNode *lo : _graph->getLogicalOutNodes())
                 if (lo == t) isOutput = true;
             if (hostReaders.empty() && !isOutput) continue;
@@ -412,8 +518,10 @@ void DeviceMemoryLoweringPass::run() {
                 continue;
             auto *src = static_cast<TensorNode *>(op->getParentNode(0));
             auto *dst = static_cast<TensorNode *>(op->getChildNode(0));
-            const bool uploaded = src->parentNum() == 1 && static_cast<OpNode *>(src->getParentNode(0))->isRunOnce() &&
-                                  src->getTensor()->getTensorInitType() == TensorInitType::PARENTOP;
+            bool uploaded = src->parentNum() == 1 && static_cast<OpNode *>(src->getParentNode(0))->isRunOnce() &&
+                            src->getTensor()->getTensorInitType() == TensorInitType::PARENTOP && !cfg.train_mode;
+            for (TensorNode *other : tensors)   // a parameter that an op rewrites in place is no constant
+                if (other != src && other->getTensor() == src->getTensor()) uploaded = false;
             if (!uploaded || dst->getLabel()->getIsOut() || dst->childNum() == 0 ||
                 dst->getTensor()->getTensorInitType() != TensorInitType::NONE)
                 continue;

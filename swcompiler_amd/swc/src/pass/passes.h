@@ -58,6 +58,26 @@ class EliminationPass : public OptimizePass {
     void run() override;
 };
 
+// Turns an inference graph that ends in a loss into a training graph (reference:
+// src/pass/AutodiffPass.cpp:69-117, src/op/dlOp/dlOpAD.cpp, src/graphIR/TensorNode.cpp:66-134).  Nodes are
+// visited in reverse topological order: a tensor without readers seeds a gradient; an op gets its gradient op
+// (operands as the reference links them) and a gradient tensor per operand; a tensor marked for training gets
+// an SGD node reading (parameter, gradient, momentum) whose result is a second node of the SAME Tensor — the
+// parameter is updated in place — registered as a logical graph output.  As in the reference a tensor read by
+// several ops keeps the gradient of the reader visited last (no summation), and only "sgd" is implemented.
+class AutodiffPass : public OptimizePass {
+    float lr_{0.001f}, decay_{0.001f}, momentum_{0.9f};
+    size_t batch_{1};
+    int gradOps_{0}, sgdOps_{0};
+
+  public:
+    explicit AutodiffPass(IRGraph *graph) : OptimizePass(graph) {}
+    void getMethods(const std::string &method, float lr, float decay, float momentum, size_t batch);
+    void run() override;
+    int gradOpCount() const { return gradOps_; }
+    int sgdCount() const { return sgdOps_; }
+};
+
 // Transpose(a) followed by Transpose(b) with a[b[i]] == i is the identity: the
 // readers of the second result are rewired to the first operand (the pair itself
 // is left for EliminationPass).  Reference: src/pass/ElimTransposePass.h:23-88.

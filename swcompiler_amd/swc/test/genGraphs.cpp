@@ -4,7 +4,7 @@
 // the reference's test/engine/testEngineMLPInfer.cpp.
 //
 //   genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse|graph|prefetch]
-//   model: mnist8 | mnist_loader | nchw | manual | caffe2[txt][@size[xchannels]] | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
+//   model: mnist8 | mnist_loader | mlp_train | lenet_train | nchw | manual | caffe2[txt][@size[xchannels]] | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
 //   mnist_loader: [batch] is the number of records in mnist_labels_images.bin
 //
 // Every parameter/input tensor is initialised from "<name>.bin" in the
@@ -195,6 +195,56 @@ int main(int argc, char **argv) {
         GpO(graph, fc0, tanh0, fc1, softmax, argmax_o, accuracy_o);
         graph->setInferDataNodes(label, data0);
         graph->addDisplayTensorNodes(accuracy_t);
+    } else if (model == "mlp_train" || model == "lenet_train") {
+        // Training programs in the style of the reference's test/engine/testEngineLenetDistTrain.cpp (one process,
+        // no MPI): the inference graph ends in MatrixSoftmaxWithLoss, the parameters are marked for training, and
+        // Config::train_mode lets Engine::compile add the gradient ops and the SGD updates.  [batch] = records in
+        // mnist_labels_images.bin; mini-batches of 8; every parameter starts from "<name>.bin".
+        const size_t mb = 8;
+        auto param = [&](const string &name, Tensor *t) {
+            auto *n = new TensorNode(name, t);
+            fromFile(t, name);
+            n->setTraining(1);
+            graph->pushTensorNode(n);
+            return n;
+        };
+        auto apply = [&](const string &name, Op *o, std::initializer_list<TensorNode *> ins) {
+            auto *opn = new OpNode(name, o);
+            for (TensorNode *i : ins) opn->exlinkUpperNode(i);
+            auto *y = new TensorNode(name + "_out", new Tensor({0}), opn);
+            graph->pushOpNode(opn);
+            graph->pushTensorNode(y);
+            return y;
+        };
+        TensorNode *data, *h;
+        if (model == "mlp_train") {
+            data = new TensorNode("data0", new Tensor({mb, 784}));
+            graph->pushTensorNode(data);
+            h = apply("fc0", new MatrixMatrixFCBiasOp(), {data, param("fc0_w", new Tensor({784, 64})), param("fc0_b", new Tensor({64}))});
+            h = apply("tanh0", new MatrixTanhOp(), {h});
+            h = apply("fc1", new MatrixMatrixFCBiasOp(), {h, param("fc1_w", new Tensor({64, 10})), param("fc1_b", new Tensor({10}))});
+        } else {
+            data = new TensorNode("data0", new Tensor({mb, 28, 28, 1}));
+            graph->pushTensorNode(data);
+            vector<size_t> ck{5, 5}, cs{1, 1}, cp{2, 2, 2, 2}, pk{3, 3}, ps{3, 3}, pp{0, 0, 0, 0};
+            h = apply("conv0", new Conv2dOp(ck, cs, cp), {data, param("conv0_w", new Tensor({16, 5, 5, 1})), param("conv0_b", new Tensor({16}))});
+            h = apply("pool0", new MaxPoolOp(pk, ps, pp), {h});
+            h = apply("relu0", new ReluOp(), {h});
+            h = apply("conv1", new Conv2dOp(ck, cs, cp), {h, param("conv1_w", new Tensor({16, 5, 5, 16})), param("conv1_b", new Tensor({16}))});
+            h = apply("pool1", new MaxPoolOp(pk, ps, pp), {h});
+            h = apply("relu1", new ReluOp(), {h});
+            h = apply("fc0", new MatrixMatrixFCBiasOp(), {h, param("fc0_w", new Tensor({144, 10})), param("fc0_b", new Tensor({10}))});
+        }
+        auto *label = new TensorNode("selected", new Tensor({mb}, DataType::Int32_t));
+        auto *loss_op = new OpNode("softmax", new MatrixSoftmaxWithLossOp());
+        loss_op->exlinkUpperNode(h, label);
+        auto *prob = new TensorNode("prob", new Tensor({0}), loss_op);
+        auto *loss = new TensorNode("loss", new Tensor({1}), loss_op);
+        graph->pushOpNode(loss_op);
+        graph->pushTensorNode(label, prob, loss);
+        graph->initTensorNodes();
+        graph->setTrainDataNodes(label, data);
+        graph->addDisplayTensorNodes(loss);
     } else if (model == "manual") {
         // placement written out by hand, the way the reference's test/cuda/testGPUInfer.cpp does it:
         // device twins, ScatterOp / GatherOp nodes, Label::setDeviceLabel, run-once parameter uploads,
@@ -403,6 +453,20 @@ int main(int argc, char **argv) {
     config.hip_graph = useGraph;
     config.hip_prefetch = prefetch;
     config.dump_outputs = true;
+    if (model == "mlp_train" || model == "lenet_train") {
+        config.train_mode = true;
+        config.train_config.optimizer = "sgd";
+        config.train_config.lr = 0.01f;
+        config.train_config.decay = 0.001f;
+        config.train_config.momentum = 0.9f;
+        config.train_config.batch = 8;
+        config.train_config.train_data_file = "mnist_labels_images.bin";
+        config.train_config.label_bytes = BytesProto::ONE_BYTE_AS_INT;
+        config.train_config.data_bytes = BytesProto::FOUR_BYTES_AS_FLOAT;
+        config.train_config.train_data_samples = batch;
+        config.train_config.max_epoch = 2;
+        config.train_config.display = 4;
+    }
     if (model == "mnist_loader") {
         config.use_dataloader = true;
         config.dataloader_src = "mnist_labels_images.bin";
