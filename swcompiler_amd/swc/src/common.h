@@ -20,8 +20,8 @@ enum ParallelStrategy { SLICE, TILING, MEM_SAVING, COMM_SAVING };
 enum BytesProto { ONE_BYTE_AS_INT, FOUR_BYTES_AS_FLOAT };
 enum NetTopology { FC_MESH_NET, STAR_NET, RING_NET, TREE_NET };
 
-// Carried for source compatibility with programs that fill it in; the HIP
-// target is inference-only and reads none of it.
+// Settings of a training program (Config::train_mode; reference: src/common.h:40-58).  `snapshot` is carried
+// for source compatibility only.
 struct TrainingConfig {
     std::string optimizer;
     float lr{0.001f};
