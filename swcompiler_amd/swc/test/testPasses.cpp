@@ -262,12 +262,70 @@ static void testResidualBlockAndCounters() {
     CHECK(g->getNodeByName("counters_host") != nullptr && g->getNodeByName("top1_host") == nullptr);
 }
 
+// Config::train_mode: FCBias -> Tanh -> FCBias -> SoftmaxWithLoss grows gradient ops, SGD nodes that rewrite
+// their parameter in place, and (after lowering and elimination) no gradient for the data.
+static void testAutodiff() {
+    TENSOR(x, 8, 20);
+    TENSOR(w0, 20, 16);
+    TENSOR(b0, 16);
+    TENSOR(w1, 16, 10);
+    TENSOR(b1, 10);
+    for (TensorNode *p : {w0, b0, w1, b1}) p->setTraining(1);
+    OP(fc0, MatrixMatrixFCBiasOp);
+    LINKUPPER(fc0, x, w0, b0);
+    TENSOR(h0, 8, 16);
+    LINKUPPER(h0, fc0);
+    OP(act, MatrixTanhOp);
+    LINKUPPER(act, h0);
+    TENSOR(h1, 8, 16);
+    LINKUPPER(h1, act);
+    OP(fc1, MatrixMatrixFCBiasOp);
+    LINKUPPER(fc1, h1, w1, b1);
+    TENSOR(logits, 8, 10);
+    LINKUPPER(logits, fc1);
+    auto *label = new TensorNode("label", new Tensor({8}, DataType::Int32_t));
+    OP(lossop, MatrixSoftmaxWithLossOp);
+    LINKUPPER(lossop, logits, label);
+    TENSOR(prob, 8, 10);
+    LINKUPPER(prob, lossop);
+    TENSOR(loss, 1);
+    LINKUPPER(loss, lossop);
+    G(g);
+    GpT(g, x, w0, b0, w1, b1, h0, h1, logits, label, prob, loss);
+    GpO(g, fc0, act, fc1, lossop);
+    g->findInOut();
+    g->updateTopology();
+    g->setTrainDataNodes(label, x);
+    g->addDisplayTensorNodes(loss);
+    Config cfg;
+    cfg.train_mode = true;
+    cfg.train_config.optimizer = "sgd";
+    cfg.train_config.batch = 8;
+    g->setConfig(cfg);
+    Engine e(g);
+    e.compile();
+    CHECK(countOps(g, "SGD") == 4 && countOps(g, "MatrixSoftmaxWithLossGrad") == 1 && countOps(g, "MatrixTanhGrad") == 1);
+    CHECK(countOps(g, "MatrixMatrixFCBiasGrad") == 0 && countOps(g, "BatchedReduceAdd") == 2);
+    // forward: 2 products (FCBias is lowered on the CPU target); backward: dW twice, dX once (the data needs none)
+    CHECK(countOps(g, "MatrixMatrixMul") == 5 && countOps(g, "Transpose") == 3);
+    CHECK(g->getNodeByName("x_grad") == nullptr && g->getNodeByName("w0_grad") != nullptr);
+    auto *sgd = static_cast<OpNode *>(g->getNodeByName("w0_sgd"));
+    CHECK(sgd && sgd->parentNum() == 3 && sgd->getParentNode(0) == w0 && sgd->getParentNode(1)->name() == "w0_grad");
+    auto *updated = static_cast<TensorNode *>(sgd->getChildNode(0));
+    CHECK(updated != w0 && updated->getTensor() == w0->getTensor() && updated->getLabel()->getIsOut());
+    auto *step = static_cast<SGDOp *>(sgd->getOp());
+    CHECK(step->getLR() == 0.001f && step->getDecay() == 0.001f && step->getMomentum() == 0.9f && step->getBatch() == 8);
+    // every SGD node comes after every reader of its parameter
+    CHECK(sgd->topologyId() > static_cast<OpNode *>(g->getNodeByName("fc0_mm"))->topologyId());
+}
+
 int main() {
     testTopologyAndShapes();
     testLoweringAndRenaming();
     testFusionAndPlacement();
     testElimination();
     testResidualBlockAndCounters();
+    testAutodiff();
     if (failures) {
         cerr << failures << " check(s) failed" << endl;
         return 1;
