@@ -79,9 +79,12 @@ inline void accuracy_i(const int *pred, const int *label, int *accum, int m, int
 // <label><data>, where a label is one byte (ONE_BYTE_AS_INT) or a 4-byte float
 // read as an integer class (FOUR_BYTES_AS_FLOAT), and data elements are bytes or
 // 4-byte floats likewise.  next() fills one mini-batch (label_shape[0] records)
-// and returns false once `epochs` passes over the file are done; a trailing
-// partial batch is dropped.  Same constructor and next()/shift() as the
-// reference's src/codegen/utils/DataLoader.h:56-63.
+// and returns false once `epochs` passes over the file are done; a mini-batch
+// that reaches the end of the file goes on with the first records of the next
+// pass, and what is left of the last pass is dropped.  A byte is read as the
+// reference reads it, through `char` (values above 127 come out negative).
+// Same constructor and next()/shift() as the reference's
+// src/codegen/utils/DataLoader.h:56-63 (DataLoader.cpp:98-168).
 #ifndef SWC_BYTES_PROTO_DEFINED
 #define SWC_BYTES_PROTO_DEFINED
 enum BytesProto { ONE_BYTE_AS_INT, FOUR_BYTES_AS_FLOAT };
@@ -103,7 +106,7 @@ class DataLoader {
     template <typename T> static void decode(const unsigned char *src, BytesProto p, size_t n, T *dst) {
         for (size_t i = 0; i < n; ++i) {
             if (p == ONE_BYTE_AS_INT) {
-                dst[i] = (T)src[i];
+                dst[i] = (T)(signed char)src[i];
             } else {
                 float f;
                 std::memcpy(&f, src + 4 * i, 4);
@@ -135,25 +138,29 @@ class DataLoader {
     DataLoader &operator=(const DataLoader &) = delete;
 
     bool next(int *label_batch, float *data_batch) {
-        if (cursor_ + batch_ > samples_) {
-            if (++epoch_ >= epochs_) return false;
-            rewindFile();
-            if (batch_ > samples_) return false;
-        }
         if (epoch_ >= epochs_) return false;
         for (size_t s = 0; s < batch_; ++s) {
+            if (cursor_ == samples_) {   // the mini-batch goes on with the first records of the next epoch
+                ++epoch_;
+                rewindFile();
+                if (epoch_ >= epochs_ || samples_ == 0) return false;
+            }
             if (std::fread(raw_.data(), 1, raw_.size(), file_) != raw_.size()) return false;
             decode(raw_.data(), labelProto_, 1, label_batch + s);
             decode(raw_.data() + width(labelProto_), dataProto_, dataPerSample_, data_batch + s * dataPerSample_);
+            ++cursor_;
         }
-        cursor_ += batch_;
         return true;
     }
-    // skip n mini-batches
+    // continue as if n mini-batches had been read since the start (a run restored from a snapshot): epoch and
+    // position follow from n, as in the reference's DataLoader.cpp:161-168.  (There the file is opened by the
+    // first next(), so a shift before it — where the generated program has it — leaves the file position at the
+    // start while the counters move; here both move.)
     void shift(size_t n) {
-        const size_t skip = n * batch_;
-        std::fseek(file_, (long)(skip * raw_.size()), SEEK_CUR);
-        cursor_ += skip;
+        const size_t seen = n * batch_;
+        epoch_ = samples_ ? seen / samples_ : 0;
+        cursor_ = samples_ ? seen % samples_ : 0;
+        std::fseek(file_, (long)(cursor_ * raw_.size()), SEEK_SET);
     }
 };
 

@@ -159,6 +159,7 @@ void Codegen::emitHeader() {
                   << "#include <sys/time.h>\n#include <sys/types.h>\n"
                   << "#include \"utils/image.h\"\n#include \"utils/kernels.h\"\n";
     if (config_.use_dataloader) headerWriter_ << "#include \"utils/DataLoader.h\"\n";
+    if (config_.train_mode) headerWriter_ << "#include \"swc_snapshot.h\"\n";
 }
 
 void Codegen::emitEnvInit() {
@@ -178,6 +179,8 @@ std::string Codegen::generate() {
     writer_ << "\nint main(int argc, char** argv) {\n";
     writer_.indentInc();
     writer_ << "struct timeval ts,te;\n(void)ts; (void)te; (void)argc; (void)argv;\n";
+    if (config_.train_mode)   // (the reference defines the same flag with gflags, src/codegen/Codegen.h:44-48)
+        writer_ << "const std::string FLAGS_snapshot = swcFlagString(argc, argv, \"snapshot\");\n";
     emitEnvInit();
     writer_ << "\n// variable declaration and initiation\n";
     emitMemAllocs();
@@ -323,10 +326,12 @@ void Codegen::emitTensorAddresses() {
 }
 
 void Codegen::emitTensorInitializations() {
+    emitSnapshotRestoreBegin();
     for (TensorNode *tn : decl_order_) {
         Tensor *t = tn->getTensor();
         const std::string name = tensors_name_map_.at(t);
         const TensorInitInfo info = t->getTensorInitInfo();
+        writer_ << restoreGuard(t);
         switch (t->getTensorInitType()) {
         case TensorInitType::XAVIER:
             writer_ << "initTensorXavier(" << name << ", " << t->size() << ", " << info.getFilterSize() << ");\n";
@@ -348,7 +353,63 @@ void Codegen::emitTensorInitializations() {
             break;
         }
     }
+    emitSnapshotRestoreEnd();
     writer_ << "\n";
+}
+
+bool Codegen::inSnapshot(Tensor *t) const {
+    if (!config_.train_mode || t->getDataType() != DataType::Float_t) return false;
+    const TensorInitType init = t->getTensorInitType();
+    return init == TensorInitType::XAVIER || init == TensorInitType::CONSTANT || init == TensorInitType::ZERO;
+}
+
+std::string Codegen::restoreGuard(Tensor *t) const {
+    if (!inSnapshot(t)) return "";
+    const std::string name = tensors_name_map_.at(t);
+    return "if (!swc_restored || !loadFromSnapShot(swc_snapshot, \"" + name + "\", " + name + ", " +
+           std::to_string(t->size()) + ")) ";
+}
+
+void Codegen::emitSnapshotRestoreBegin() {
+    if (!config_.train_mode) return;
+    writer_ << "SnapshotNet swc_snapshot;\nconst bool swc_restored = FLAGS_snapshot.size() > 0;\n";
+    writer_ << "if (swc_restored) {\n";
+    writer_.indentInc();
+    writer_ << "std::cout << \"restoring from snapshot \" << FLAGS_snapshot << std::endl;\n";
+    writer_ << "if (!swc_snapshot.parse(FLAGS_snapshot)) { std::cout << \"Error loading \" << FLAGS_snapshot << \"\\n\"; "
+            << "return 1; }\n";
+    writer_.indentDec();
+    writer_ << "}\n";
+}
+
+void Codegen::emitSnapshotRestoreEnd() {
+    if (!config_.train_mode) return;
+    writer_ << "if (swc_restored) {\n";
+    writer_.indentInc();
+    writer_ << "size_t snap_iter = getIterFromSnapShot(swc_snapshot);\nloader.shift(snap_iter);\niter = snap_iter;\n";
+    writer_ << "std::cout << \"snapshot iter= \" << snap_iter << std::endl;\n";
+    writer_.indentDec();
+    writer_ << "}\n";
+}
+
+void Codegen::emitSaveSnapshot() {
+    if (!config_.train_mode || !config_.train_config.snapshot) return;
+    writer_ << "\nif (iter % " << config_.train_config.snapshot << " == 0) {\n";
+    writer_.indentInc();
+    writer_ << "std::cout << \"iter = \" << iter << \", snapshot\\n\";\n";
+    writer_ << "SnapshotNet net;\nnet.setIter(iter);\n";
+    std::set<Tensor *> seen;
+    for (TensorNode *tn : decl_order_) {
+        Tensor *t = tn->getTensor();
+        if (!inSnapshot(t) || !seen.insert(t).second) continue;
+        const std::string name = tensors_name_map_.at(t);
+        writer_ << "addOp(net, \"" << name << "\", " << name << ", " << t->size() << ");\n";
+    }
+    writer_ << "std::string snapfile = \"snapshot_iter\" + std::to_string(iter) + \".model\";\n";
+    writer_ << "if (!net.save(snapfile)) { std::cout << \"Error opening \" << snapfile << \"\\n\"; return 1; }\n";
+    writer_ << "std::cout << \"save snapshot to \" << snapfile << \"\\n\";\n";
+    writer_.indentDec();
+    writer_ << "}\n";
 }
 
 void Codegen::emitExecute() {
@@ -357,6 +418,7 @@ void Codegen::emitExecute() {
         writer_.indentInc();
         emitFuncCalls();
         writer_ << "\niter++;\n";
+        emitSaveSnapshot();
         if (config_.display > 0) emitPrintGraphOutputs();
         emitMaxItersBreak();
         writer_.indentDec();

@@ -131,6 +131,15 @@ class Codegen {
     TensorNode *loaderDataNode() const;
     virtual void emitInferDataLoaderInit();        // `DataLoader loader(...)` + iteration counter
     virtual void emitPrintGraphOutputs();          // every Config::display iterations: the display tensors
+    // Snapshots of a training program (reference: src/codegen/Codegen.cpp:659-812).  Every
+    // TrainingConfig::snapshot iterations the tensors that start from an initialiser (Xavier, constant, zero:
+    // parameters and momenta) and the iteration count go to snapshot_iter<N>.model; a program started with
+    // --snapshot=<file> takes those tensors and the count from the file and moves the loader on accordingly.
+    virtual void emitSaveSnapshot();
+    void emitSnapshotRestoreBegin();               // parses the file named by the flag, if any
+    void emitSnapshotRestoreEnd();                 // iteration count and loader position
+    bool inSnapshot(Tensor *t) const;              // float tensor with an initialiser of its own, training program
+    std::string restoreGuard(Tensor *t) const;     // prefix of such a tensor's initialiser call: restore, else initialise
 
     void codeGenInit();
     void emitMemAllocs();
@@ -181,6 +190,7 @@ class HipCodegen : public Codegen {
     void emitExecute() override;
     void emitMemFree() override;
     void emitPrintGraphOutputs() override;
+    void emitSaveSnapshot() override;   // the trained copies live on the device: they are downloaded into their host tensors first
 
   protected:
     void emitDeviceFills();        // constant initialisers of device tensors that have no host twin

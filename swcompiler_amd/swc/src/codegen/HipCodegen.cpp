@@ -10,6 +10,7 @@
 #include <cassert>
 #include <cstdlib>
 #include <iomanip>
+#include <set>
 #include <sstream>
 
 #include "../graphIR/IRGraph.h"
@@ -43,6 +44,7 @@ void HipCodegen::emitHeader() {
     headerWriter_ << "#include <algorithm>\n#include <iostream>\n#include <random>\n#include <cstdlib>\n#include <cstdio>\n#include <cstring>\n#include <cmath>\n"
                   << "#include <sys/time.h>\n"
                   << "#include \"swc_host_utils.h\"\n#include \"swc_hip.h\"\n";
+    if (config_.train_mode) headerWriter_ << "#include \"swc_snapshot.h\"\n";
     headerWriter_ << "#define SWC_HIP_CHECK(call) do { if ((call) != 0) { std::fprintf(stderr, \"%s:%d: %s\\n  %s\\n\", "
                      "__FILE__, __LINE__, #call, swc_hip_last_error()); std::exit(1); } } while (0)\n";
 }
@@ -135,11 +137,13 @@ void HipCodegen::emitMemAllocations() {
 // uploads (run-once Scatter nodes) follow in graph order.
 void HipCodegen::emitTensorInitializations() {
     std::vector<OpNode *> uploads;
+    emitSnapshotRestoreBegin();
     for (TensorNode *tn : decl_order_) {
         Tensor *t = tn->getTensor();
         const std::string name = tensors_name_map_.at(t);
         const bool onGpu = tn->getLabel()->getDeviceLabel().type == DeviceType::GPU;
         const TensorInitInfo info = t->getTensorInitInfo();
+        if (!onGpu) writer_ << restoreGuard(t);
         switch (t->getTensorInitType()) {
         case TensorInitType::PARENTOP:   // filled by its run-once producer, below
             break;
@@ -163,6 +167,7 @@ void HipCodegen::emitTensorInitializations() {
             break;
         }
     }
+    emitSnapshotRestoreEnd();
     emitDeviceFills();
     // every run-once op (parameter uploads), in topological order; runable() lets each through once
     for (int i = 0; i < graph_->topologyNum(); ++i)
@@ -192,6 +197,36 @@ void HipCodegen::emitDeviceFills() {
             writer_ << "SWC_HIP_CHECK(swc_hip_fill_i(" << name << ", " << static_cast<int>(v) << ", " << t->size()
                     << "));\n";
     }
+}
+
+// The host tensors a snapshot holds are the ones the CPU program would write, under the same names, so a
+// snapshot of either program restores the other.  What the device has trained is downloaded into them first.
+void HipCodegen::emitSaveSnapshot() {
+    if (!config_.train_mode || !config_.train_config.snapshot) return;
+    writer_ << "\nif (iter % " << config_.train_config.snapshot << " == 0) {\n";
+    writer_.indentInc();
+    writer_ << "std::cout << \"iter = \" << iter << \", snapshot\\n\";\n";
+    writer_ << "SnapshotNet net;\nnet.setIter(iter);\n";
+    std::set<Tensor *> seen;
+    for (TensorNode *tn : decl_order_) {
+        Tensor *t = tn->getTensor();
+        if (tn->getLabel()->getDeviceLabel().type != DeviceType::CPU || !inSnapshot(t) || !seen.insert(t).second) continue;
+        const std::string name = tensors_name_map_.at(t);
+        for (IRNode *c : tn->getChildNodes()) {
+            if (c->nodeType() != OP_NODE) continue;
+            auto *up = static_cast<OpNode *>(c);
+            if (up->getOp()->getOpName() != "Scatter" || !up->isRunOnce() || up->childNum() != 1) continue;
+            writer_ << "SWC_HIP_CHECK(swc_hip_d2h(" << name << ", " << nameOf(up->getChildNode(0)) << ", "
+                    << t->getSizeInBytes() << "));\n";
+            break;
+        }
+        writer_ << "addOp(net, \"" << name << "\", " << name << ", " << t->size() << ");\n";
+    }
+    writer_ << "std::string snapfile = \"snapshot_iter\" + std::to_string(iter) + \".model\";\n";
+    writer_ << "if (!net.save(snapfile)) { std::cout << \"Error opening \" << snapfile << \"\\n\"; return 1; }\n";
+    writer_ << "std::cout << \"save snapshot to \" << snapfile << \"\\n\";\n";
+    writer_.indentDec();
+    writer_ << "}\n";
 }
 
 void HipCodegen::emitDeferredGathers() {
@@ -336,7 +371,9 @@ void HipCodegen::emitExecute() {
                 dispatchOpNode(op);
             }
         writer_ << "\niter++;\n";
+        emitSaveSnapshot();
         if (config_.display > 0) emitPrintGraphOutputs();
+        emitMaxItersBreak();
         writer_.indentDec();
         writer_ << "} //while\n";
         emitDeferredGathers();

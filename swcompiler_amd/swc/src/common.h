@@ -20,8 +20,8 @@ enum ParallelStrategy { SLICE, TILING, MEM_SAVING, COMM_SAVING };
 enum BytesProto { ONE_BYTE_AS_INT, FOUR_BYTES_AS_FLOAT };
 enum NetTopology { FC_MESH_NET, STAR_NET, RING_NET, TREE_NET };
 
-// Settings of a training program (Config::train_mode; reference: src/common.h:40-58).  `snapshot` is carried
-// for source compatibility only.
+// Settings of a training program (Config::train_mode; reference: src/common.h:40-58).  snapshot: every that many
+// iterations the parameters, momenta and the iteration count are written to snapshot_iter<N>.model (0: never).
 struct TrainingConfig {
     std::string optimizer;
     float lr{0.001f};

@@ -3,9 +3,11 @@
 // directory.  User-level code: only `SWC.h` and the DSL macros, in the style of
 // the reference's test/engine/testEngineMLPInfer.cpp.
 //
-//   genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse|graph|prefetch]
+//   genGraphs <model> <cpu|hip> [batch] [time_iters] [nofuse|graph|prefetch|-] [snapshot]
 //   model: mnist8 | mnist_loader | mlp_train | lenet_train | nchw | manual | caffe2[txt][@size[xchannels]] | cfg1 | cfg2 | cfg3 | cfg4 | cfg5a | cfg5b | cfg5c
 //   mnist_loader: [batch] is the number of records in mnist_labels_images.bin
+//   [snapshot] (training models): TrainingConfig::snapshot; the parameters then start from Xavier / zero
+//   initialisers instead of files
 //
 // Every parameter/input tensor is initialised from "<name>.bin" in the
 // directory the generated program runs in; outputs are dumped to "<name>.bin".
@@ -114,6 +116,7 @@ int main(int argc, char **argv) {
     const bool nofuse = argc > 5 && string(argv[5]) == "nofuse";
     const bool prefetch = argc > 5 && string(argv[5]) == "prefetch";   // (implies graph)
     const bool useGraph = prefetch || (argc > 5 && string(argv[5]) == "graph");
+    const size_t snapshot = argc > 6 ? strtoul(argv[6], nullptr, 10) : 0;   // training models: TrainingConfig::snapshot
 
     G(graph);
     TensorNode *out = nullptr;
@@ -203,7 +206,10 @@ int main(int argc, char **argv) {
         const size_t mb = 8;
         auto param = [&](const string &name, Tensor *t) {
             auto *n = new TensorNode(name, t);
-            fromFile(t, name);
+            // (only tensors that start from an initialiser are part of a snapshot, as in the reference)
+            if (!snapshot) fromFile(t, name);
+            else if (t->getNDim() == 1) t->setTensorInit(TensorInitType::ZERO);
+            else t->setTensorInit(TensorInitType::XAVIER, (float)(t->size() / t->getDim(t->getNDim() == 2 ? 1 : 0)));
             n->setTraining(1);
             graph->pushTensorNode(n);
             return n;
@@ -466,6 +472,7 @@ int main(int argc, char **argv) {
         config.train_config.train_data_samples = batch;
         config.train_config.max_epoch = 2;
         config.train_config.display = 4;
+        config.train_config.snapshot = snapshot;
     }
     if (model == "mnist_loader") {
         config.use_dataloader = true;

@@ -57,9 +57,11 @@ def write_inputs(cfg, t, workdir):
         t[k].tofile(os.path.join(workdir, stem + ".bin"))
 
 
-def generate(gen, model, target, workdir, batch=0, iters=0, nofuse=False, graph=False, prefetch=False):
+def generate(gen, model, target, workdir, batch=0, iters=0, nofuse=False, graph=False, prefetch=False, snapshot=0):
     args = [gen, model, target, str(batch), str(iters)] + (["nofuse"] if nofuse else []) + (["graph"] if graph else []) + \
            (["prefetch"] if prefetch else [])
+    if snapshot:
+        args += ["-"] * (6 - len(args)) + [str(snapshot)]
     code = subprocess.run(args, cwd=workdir, check=True, capture_output=True, text=True).stdout
     assert open(os.path.join(workdir, "Graph.cpp")).read() == code
     return code
@@ -67,7 +69,7 @@ def generate(gen, model, target, workdir, batch=0, iters=0, nofuse=False, graph=
 
 def build_cpu(workdir, with_loader=False, force_compat=False):
     if os.path.isdir(REF_UTILS) and not force_compat:   # the reference's own image.h / kernels.h (/ DataLoader)
-        cmd = ["g++", "-std=c++11", "-O2", "-w", "-I", REF_UTILS, "Graph.cpp"]
+        cmd = ["g++", "-std=c++11", "-O2", "-w", "-I", REF_UTILS, "-I", os.path.join(ROOT, "include"), "Graph.cpp"]
         if with_loader:
             cmd.append(os.path.join(REF_UTILS, "utils", "DataLoader.cpp"))
         cmd += ["-o", "net_cpu.bin"]
