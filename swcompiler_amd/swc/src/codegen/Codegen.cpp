@@ -608,6 +608,10 @@ void Codegen::emitFuncCall(OpNode *op) {
         const size_t m = T(in(1))->getDim(0), n = T(in(1))->getDim(1);
         writer_ << "matrixSoftmaxWithLossGrad_f(" << m << ", " << n << ", " << nameOf(out(0)) << ", " << n << ", "
                 << nameOf(in(1)) << ", " << n << ", " << nameOf(in(0)) << ");\n";
+    } else if (type == "MatrixSoftmaxGrad") {   // Codegen.cpp:2429-2444: parents input, label, output(, outputGrad)
+        const size_t m = T(in(0))->getDim(0), n = T(in(0))->getDim(1);
+        writer_ << "matrixSoftmaxGrad_f(" << m << ", " << n << ", " << nameOf(out(0)) << ", " << n << ", "
+                << nameOf(in(2)) << ", " << n << ", " << nameOf(in(1)) << ");\n";
     } else if (type == "SGD") {   // Codegen.cpp:2468-2489: parents parameter, gradient, momentum; in place
         auto *sgd = static_cast<SGDOp *>(op->getOp());
         writer_ << "sgd_f(" << T(in(0))->size() << ", " << nameOf(in(0)) << ", " << nameOf(in(0)) << ", " << nameOf(in(1))

@@ -702,6 +702,10 @@ void HipCodegen::emitHipCall(OpNode *op) {
         const size_t m = T(in(1))->getDim(0), n = T(in(1))->getDim(1);
         writer_ << "SWC_HIP_CHECK(swc_hip_matrixSoftmaxWithLossGrad_f(" << m << ", " << n << ", " << nameOf(out(0)) << ", " << n
                 << ", " << nameOf(in(1)) << ", " << n << ", " << nameOf(in(0)) << "));\n";
+    } else if (type == "MatrixSoftmaxGrad") {
+        const size_t m = T(in(0))->getDim(0), n = T(in(0))->getDim(1);
+        writer_ << "SWC_HIP_CHECK(swc_hip_matrixSoftmaxGrad_f(" << m << ", " << n << ", " << nameOf(out(0)) << ", " << n
+                << ", " << nameOf(in(2)) << ", " << n << ", " << nameOf(in(1)) << "));\n";
     } else if (type == "SGD") {
         auto *sgd = static_cast<SGDOp *>(op->getOp());
         writer_ << "SWC_HIP_CHECK(swc_hip_sgd_f(" << T(in(0))->size() << ", " << nameOf(in(0)) << ", " << nameOf(in(0)) << ", "

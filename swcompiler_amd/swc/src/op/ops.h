@@ -276,6 +276,12 @@ class MatrixSoftmaxWithLossOp : public Op {
     void outTensorShapeGen(OpNode *node, size_t index, TensorShape *shape) override;
 };
 // parents: label, prob -> gradient of the logits
+// the older way to train: a label linked to MatrixSoftmax as its second operand (reference:
+// src/op/dlOp/dlOpAD.cpp:213-247); parents input, label, output, outputGrad -> inputGrad (, labelGrad: by name only)
+class MatrixSoftmaxGradOp : public Op {
+  public:
+    MatrixSoftmaxGradOp() : Op(DL_OP, 4, 1, "MatrixSoftmaxGrad") {}
+};
 class MatrixSoftmaxWithLossGradOp : public Op {
   public:
     MatrixSoftmaxWithLossGradOp() : Op(DL_OP, 2, 1, "MatrixSoftmaxWithLossGrad") {}

@@ -215,6 +215,8 @@ void AutodiffPass::run() {
                     {in(0), in(1), outGrad()});
         } else if (type == "MatrixSoftmaxWithLoss") {
             addGrad(op, new MatrixSoftmaxWithLossGradOp(), {in(1), op->getChildNode(0)});   // label, prob
+        } else if (type == "MatrixSoftmax" && op->parentNum() == 2) {   // a label as second operand: the network's end
+            addGrad(op, new MatrixSoftmaxGradOp(), {in(0), in(1), op->getChildNode(0), outGrad()});
         } else {
             SWLOG_ERROR << "AutodiffPass: no gradient for op type " << type << " (node " << op->name() << ")" << std::endl;
             std::abort();
@@ -223,6 +225,20 @@ void AutodiffPass::run() {
     _graph->findInOut();
     _graph->updateTopology();
 }
+
+} // namespace pass
+
+IRGraph *getTrainNet(IRGraph *graph, TrainingConfig &profile) {
+    IRGraph *net = graph->clone();
+    net->findInOut();
+    net->updateTopology();
+    pass::AutodiffPass autodiff(net);
+    autodiff.getMethods("sgd", profile.lr, profile.decay, profile.momentum, profile.batch);
+    autodiff.run();
+    return net;
+}
+
+namespace pass {
 
 // -------------------------------------------------------- transpose cancelling
 void ElimTransposePass::run() {
@@ -412,7 +428,7 @@ bool DeviceMemoryLoweringPass::runsOnGpu(const std::string &t) {
         "Conv2d", "Conv2dWithActivation", "Conv2dBatchNorm", "Conv2dAdd", "MaxPool", "AveragePool", "Transpose",
         "BatchNormalization",
         "BatchNormalizationRelu", "BatchNormReluMaxPool", "ArgMax", "Accuracy",
-        "MatrixSoftmaxWithLoss", "MatrixSoftmaxWithLossGrad", "BatchedReduceAdd", "MatrixTanhGrad", "ReluGrad",
+        "MatrixSoftmaxWithLoss", "MatrixSoftmaxWithLossGrad", "MatrixSoftmaxGrad", "BatchedReduceAdd", "MatrixTanhGrad", "ReluGrad",
         "MaxPoolGrad", "Conv2dGrad", "SGD"};
     return gpu.count(t) != 0;
 }

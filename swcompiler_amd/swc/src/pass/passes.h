@@ -78,6 +78,16 @@ class AutodiffPass : public OptimizePass {
     int sgdCount() const { return sgdOps_; }
 };
 
+} // namespace pass
+
+// The training graph of `graph` as a new graph: a copy with the gradient ops and the SGD updates of the trained
+// parameters added (AutodiffPass on the copy, SGD with the profile's lr / decay / momentum / batch).  The
+// reference's free function of the same name (src/diff/AutoDiff.h:21, AutoDiff.cpp:27-184), which programs
+// written before Engine::compile use; nodes keep their names, so getNodeByName finds them in the copy.
+IRGraph *getTrainNet(IRGraph *graph, TrainingConfig &profile);
+
+namespace pass {
+
 // Transpose(a) followed by Transpose(b) with a[b[i]] == i is the identity: the
 // readers of the second result are rewired to the first operand (the pair itself
 // is left for EliminationPass).  Reference: src/pass/ElimTransposePass.h:23-88.

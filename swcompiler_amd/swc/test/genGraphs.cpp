@@ -118,6 +118,12 @@ int main(int argc, char **argv) {
     const bool useGraph = prefetch || (argc > 5 && string(argv[5]) == "graph");
     const size_t snapshot = argc > 6 ? strtoul(argv[6], nullptr, 10) : 0;   // training models: TrainingConfig::snapshot
 
+    // mlp_train_label: the MLP with the label linked to a MatrixSoftmax node (the older way to end a training graph);
+    // mlp_train_getnet: the same graph taken through getTrainNet and hand-run passes to codegen::Codegen, in the
+    // style of the reference's test/testSnapshot.cpp (no Engine)
+    const bool labelled = model == "mlp_train_label" || model == "mlp_train_getnet";
+    const bool training = model == "mlp_train" || model == "lenet_train" || labelled;
+
     G(graph);
     TensorNode *out = nullptr;
 
@@ -198,7 +204,7 @@ int main(int argc, char **argv) {
         GpO(graph, fc0, tanh0, fc1, softmax, argmax_o, accuracy_o);
         graph->setInferDataNodes(label, data0);
         graph->addDisplayTensorNodes(accuracy_t);
-    } else if (model == "mlp_train" || model == "lenet_train") {
+    } else if (training) {
         // Training programs in the style of the reference's test/engine/testEngineLenetDistTrain.cpp (one process,
         // no MPI): the inference graph ends in MatrixSoftmaxWithLoss, the parameters are marked for training, and
         // Config::train_mode lets Engine::compile add the gradient ops and the SGD updates.  [batch] = records in
@@ -223,7 +229,7 @@ int main(int argc, char **argv) {
             return y;
         };
         TensorNode *data, *h;
-        if (model == "mlp_train") {
+        if (model == "mlp_train" || labelled) {
             data = new TensorNode("data0", new Tensor({mb, 784}));
             graph->pushTensorNode(data);
             h = apply("fc0", new MatrixMatrixFCBiasOp(), {data, param("fc0_w", new Tensor({784, 64})), param("fc0_b", new Tensor({64}))});
@@ -242,15 +248,22 @@ int main(int argc, char **argv) {
             h = apply("fc0", new MatrixMatrixFCBiasOp(), {h, param("fc0_w", new Tensor({144, 10})), param("fc0_b", new Tensor({10}))});
         }
         auto *label = new TensorNode("selected", new Tensor({mb}, DataType::Int32_t));
-        auto *loss_op = new OpNode("softmax", new MatrixSoftmaxWithLossOp());
+        auto *loss_op = new OpNode("softmax", labelled ? static_cast<Op *>(new MatrixSoftmaxOp()) : new MatrixSoftmaxWithLossOp());
         loss_op->exlinkUpperNode(h, label);
         auto *prob = new TensorNode("prob", new Tensor({0}), loss_op);
-        auto *loss = new TensorNode("loss", new Tensor({1}), loss_op);
         graph->pushOpNode(loss_op);
-        graph->pushTensorNode(label, prob, loss);
-        graph->initTensorNodes();
-        graph->setTrainDataNodes(label, data);
-        graph->addDisplayTensorNodes(loss);
+        graph->pushTensorNode(label, prob);
+        if (labelled) {
+            graph->initTensorNodes();
+            graph->setTrainDataNodes(label, data);
+            graph->addDisplayTensorNodes(prob);
+        } else {
+            auto *loss = new TensorNode("loss", new Tensor({1}), loss_op);
+            graph->pushTensorNode(loss);
+            graph->initTensorNodes();
+            graph->setTrainDataNodes(label, data);
+            graph->addDisplayTensorNodes(loss);
+        }
     } else if (model == "manual") {
         // placement written out by hand, the way the reference's test/cuda/testGPUInfer.cpp does it:
         // device twins, ScatterOp / GatherOp nodes, Label::setDeviceLabel, run-once parameter uploads,
@@ -459,7 +472,7 @@ int main(int argc, char **argv) {
     config.hip_graph = useGraph;
     config.hip_prefetch = prefetch;
     config.dump_outputs = true;
-    if (model == "mlp_train" || model == "lenet_train") {
+    if (training) {
         config.train_mode = true;
         config.train_config.optimizer = "sgd";
         config.train_config.lr = 0.01f;
@@ -483,6 +496,28 @@ int main(int argc, char **argv) {
         config.display = batch / 8;   // print once, after the last mini-batch
     }
     graph->setConfig(config);
+
+    if (model == "mlp_train_getnet") {
+        IRGraph *net = getTrainNet(graph, config.train_config);
+        net->setTrainDataNodes(static_cast<TensorNode *>(net->getNodeByName("selected")),
+                               static_cast<TensorNode *>(net->getNodeByName("data0")));
+        net->addDisplayTensorNodes(static_cast<TensorNode *>(net->getNodeByName("prob")));
+        net->updateTopology();
+        pass::RenamingNodePass renaming(net);
+        pass::LabelingPass labeling(net);
+        pass::LoweringPass lowering(net);
+        pass::PassManager manager;
+        manager.add(&renaming);
+        manager.add(&labeling);
+        manager.add(&lowering);
+        manager.add(&labeling);
+        manager.run();
+        for (int i = 0; i < net->tensorNodeNum(); ++i)   // what the program leaves behind: the trained parameters
+            if (net->getTensorNode(i)->getTraining()) net->getTensorNode(i)->getLabel()->setIsOut(1);
+        codegen::Codegen generator(net, config);
+        cout << generator.generate();
+        return 0;
+    }
 
     Engine engine(graph);
     engine.compile();

@@ -165,3 +165,40 @@ def test_training_hip_program(gen, oracle, tmp_path, model, mode):
         change = np.abs(want[name] - params[name]).max()
         assert change > 0 and np.abs(got - want[name]).max() < 1e-3 * change + 1e-6, name
     assert np.allclose(printed_losses(out), losses[3::4], atol=2e-3)
+
+
+@pytest.mark.parametrize("model", ["mlp_train_label", "mlp_train_getnet"])
+def test_training_through_a_labelled_softmax_cpu(gen, oracle, tmp_path, model):
+    """The older way to end a training graph: the label is the second operand of MatrixSoftmax, whose gradient op
+    is MatrixSoftmaxGrad (reference: src/op/dlOp/dlOpAD.cpp:213-247, Codegen.cpp:2429-2444); once through
+    Engine::compile, once through getTrainNet and hand-run passes as the reference's test/testSnapshot.cpp does.
+    matrixSoftmaxGrad_f is the arithmetic of matrixSoftmaxWithLossGrad_f, so the parameters end where the
+    MatrixSoftmaxWithLoss network's end."""
+    images, labels = write_record_file(tmp_path, SAMPLES)
+    params = make_params("mlp_train", tmp_path)
+    code = generate(gen, model, "cpu", tmp_path, SAMPLES)
+    assert "matrixSoftmaxGrad_f(8, 10, fc1_out_grad, 10, prob, 10, selected);" in code and "WithLoss" not in code
+    assert code.count("sgd_f(") == len(params)
+    exe = build_cpu(tmp_path, with_loader=True)
+    subprocess.run([exe], cwd=tmp_path, check=True, capture_output=True, text=True)
+    want, _ = train_reference(oracle, "mlp_train", params, images, labels)
+    for name in params:
+        got = np.fromfile(os.path.join(tmp_path, name + ".bin"), np.float32).reshape(params[name].shape)
+        assert_bit_exact(got, want[name], name)
+
+
+@pytest.mark.gpu
+def test_training_through_a_labelled_softmax_hip(gen, oracle, tmp_path):
+    print("case training mlp_train_label graph", flush=True)
+    images, labels = write_record_file(tmp_path, SAMPLES)
+    params = make_params("mlp_train", tmp_path)
+    code = generate(gen, "mlp_train_label", "hip", tmp_path, SAMPLES, graph=True)
+    assert "swc_hip_matrixSoftmaxGrad_f(8, 10, fc1_out_grad, 10, prob, 10, selected_dev)" in code
+    subprocess.run([build_hip(tmp_path)], cwd=tmp_path, check=True, capture_output=True, text=True, timeout=120)
+    want, _ = train_reference(oracle, "mlp_train", params, images, labels)
+    for name in params:
+        files = [f for f in os.listdir(tmp_path) if f.startswith(name) and f.endswith("_host.bin")]
+        assert len(files) == 1, (name, files)
+        got = np.fromfile(os.path.join(tmp_path, files[0]), np.float32).reshape(params[name].shape)
+        change = np.abs(want[name] - params[name]).max()
+        assert change > 0 and np.abs(got - want[name]).max() < 1e-3 * change + 1e-6, name
