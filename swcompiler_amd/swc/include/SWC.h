@@ -26,6 +26,8 @@
 #include "../src/pass/OptimizePass.h"
 #include "../src/pass/passes.h"
 
+#include "../src/diff/AutoDiff.h"
+#include "../src/tool/dotGen.h"
 #include "../src/devices/HipDevice.h"
 #include "../src/codegen/Codegen.h"
 #include "../src/importer/Caffe2Importer.h"

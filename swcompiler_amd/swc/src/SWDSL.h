@@ -48,6 +48,15 @@ template <typename OpT, typename... A> inline OpNode *makeOpNode(const char *nam
 
 #define CHECKT(t) SWLOG_INFO << (t)->toString() << " topo " << (t)->topologyId() << std::endl
 #define CHECKO(o) SWLOG_INFO << (o)->toString() << " topo " << (o)->topologyId() << std::endl
+// TRAIN(net, "sgd", lr, decay, momentum, batch): declares the graph `net_train`, a copy of `net` with the gradient
+// ops and the optimizer updates added (reference: src/SWDSL.h:106-111)
+#define TRAIN(graph, parameters...)                                                                \
+    swc::pass::AutodiffPass auto_diff_path(graph);                                                 \
+    auto_diff_path.getMethods(parameters);                                                         \
+    auto_diff_path.show();                                                                         \
+    G(graph##_train);                                                                              \
+    auto_diff_path.run(graph##_train)
+
 #define CHECKG(g)                                                                                  \
     for (int i_ = 0; i_ < (g)->tensorNodeNum(); i_++) CHECKT((g)->getTensorNode(i_));              \
     for (int i_ = 0; i_ < (g)->opNodeNum(); i_++) CHECKO((g)->getOpNode(i_))

@@ -279,7 +279,8 @@ void Codegen::allocateMemAddr() {
             MemoryAllocator *arena = it->second;
             uint64_t off;
             IRNode *producer = tn->parentNum() ? tn->getParentNode(0) : nullptr;
-            if (producer && static_cast<OpNode *>(producer)->getOp()->getOpName() == "Reshape" &&
+            const std::string made = producer ? static_cast<OpNode *>(producer)->getOp()->getOpName() : "";
+            if ((made == "Reshape" || made == "TensorDescend" || made == "TensorAscend") &&
                 tensors_offset_map_.count(T(producer->getParentNode(0))) &&
                 producer->getParentNode(0)->getLabel()->getDeviceLabel() == dev) {
                 off = tensors_offset_map_.at(T(producer->getParentNode(0))).second;
@@ -504,7 +505,7 @@ void Codegen::emitFuncCall(OpNode *op) {
         assert(rc.second == T(in(1))->size() && "bias length != row length");
         writer_ << "batchedadd_f(" << nameOf(out(0)) << ", " << nameOf(in(0)) << ", " << nameOf(in(1)) << ", "
                 << rc.first << ", " << rc.second << ");\n";
-    } else if (type == "Reshape" || type == "Dropout") {   // Codegen.cpp:1480-1485 (pointer alias)
+    } else if (type == "Reshape" || type == "TensorDescend" || type == "TensorAscend" || type == "Dropout") {   // Codegen.cpp:1480-1485 (pointer alias)
         writer_ << nameOf(out(0)) << " = " << nameOf(in(0)) << ";\n";
     } else if (type == "MatrixTanh") {   // Codegen.cpp:2293-2295
         const size_t m = T(in(0))->getDim(0), n = T(in(0))->getDim(1);

@@ -569,7 +569,7 @@ void HipCodegen::emitHipCall(OpNode *op) {
         auto rc = rowsCols(T(in(0)));
         writer_ << "SWC_HIP_CHECK(swc_hip_batchedadd_f(" << nameOf(out(0)) << ", " << nameOf(in(0)) << ", "
                 << nameOf(in(1)) << ", " << rc.first << ", " << rc.second << "));\n";
-    } else if (type == "Reshape" || type == "Dropout") {
+    } else if (type == "Reshape" || type == "TensorDescend" || type == "TensorAscend" || type == "Dropout") {
         writer_ << nameOf(out(0)) << " = " << nameOf(in(0)) << ";\n";
     } else if (type == "MatrixTanh" || type == "MatrixSoftmax") {
         const size_t m = T(in(0))->getDim(0), n = T(in(0))->getDim(1);

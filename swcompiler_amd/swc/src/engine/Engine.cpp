@@ -13,6 +13,15 @@ namespace swc {
 using namespace pass;
 
 void Engine::compile() {
+    // SWC_TARGET=hip in the environment retargets a program that was written for the CPU target without touching
+    // its source: the same as Config::hip = true in it
+    if (const char *target = std::getenv("SWC_TARGET")) {
+        if (std::string(target) == "hip") {
+            Config retargeted = graph_->getConfig();
+            retargeted.hip = true;
+            graph_->setConfig(retargeted);
+        }
+    }
     const Config cfg = graph_->getConfig();
     if (cfg.mpi || cfg.mkldnn || cfg.cuda) {
         SWLOG_ERROR << "Engine: only the single-device pipelines (CPU or Config::hip) are part of this build" << std::endl;

@@ -103,6 +103,11 @@ void IRGraph::setDeviceLabel(Device dev) {
 
 IRGraph *IRGraph::clone() const {
     auto *g = new IRGraph();
+    copyTo(g);
+    return g;
+}
+
+void IRGraph::copyTo(IRGraph *g) const {
     std::unordered_map<const IRNode *, IRNode *> twin;
     for (auto *t : tensors_) {
         auto *c = t->deepClone();
@@ -138,7 +143,6 @@ IRGraph *IRGraph::clone() const {
     for (auto *l : logicalOutNodes_) g->logicalOutNodes_.push_back(twin[l]);
     g->findInOut();
     g->updateTopology();
-    return g;
 }
 
 } // namespace swc

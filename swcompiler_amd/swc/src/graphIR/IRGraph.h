@@ -91,7 +91,12 @@ class IRGraph {
 
     // Structural copy: every node cloned (tensor metadata deep-copied), links,
     // in/out lists, config and device preserved.
+    // Traffic between the ranks of a parallel program (reference: src/graphIR/IRGraph.h:165-170).  A program for one
+    // device exchanges nothing.
+    size_t getCommCost() const { return 0; }
+    std::string getCommTrace() const { return ""; }
     IRGraph *clone() const;
+    void copyTo(IRGraph *empty) const;   // the same copy into a graph the caller has made
 };
 
 template <typename V, typename N> void IRGraph::eraseNode(V &vec, N *node, const char *what) {

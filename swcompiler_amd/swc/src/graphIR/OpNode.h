@@ -41,4 +41,8 @@ class OpNode : public IRNode {
     void outTensorShapeGen(size_t index, TensorShape *shape) { op_->outTensorShapeGen(this, index, shape); }
 };
 } // namespace swc
+// The reference's header of the same name has this directive at file scope (src/graphIR/OpNode.h:16), and its
+// user programs — the importer examples, for one — name ops without `swc::op::` because of it.
+using namespace swc::op;
+
 #endif

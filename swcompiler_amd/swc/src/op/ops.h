@@ -55,6 +55,34 @@ class ReshapeOp : public Op {           // alias of the input buffer with a new 
     void outTensorShapeGen(OpNode *node, size_t index, TensorShape *shape) override;
 };
 
+// Dimensions start..end of an nDim tensor folded into one (TensorDescend) and unfolded again (TensorAscend): a view
+// of the same buffer, like Reshape (reference: src/op/tensorOp/tensorOps.h:18-70; emitted as a pointer alias,
+// src/codegen/Codegen.cpp:1487-1499).  Each is the other's gradient op.
+class TensorDescendOp : public Op {
+    int nDim_, start_, end_;
+
+  public:
+    TensorDescendOp(int nDim, int start, int end) : Op(TENSOR_OP, 1, 1, "TensorDescend"), nDim_(nDim), start_(start), end_(end) {}
+    int getNDim() const { return nDim_; }
+    int getStart() const { return start_; }
+    int getEnd() const { return end_; }
+};
+class TensorAscendOp : public Op {
+    int nDim_, start_, end_;
+
+  public:
+    TensorAscendOp(int nDim, int start, int end) : Op(TENSOR_OP, 1, 1, "TensorAscend"), nDim_(nDim), start_(start), end_(end) {}
+    int getNDim() const { return nDim_; }
+    int getStart() const { return start_; }
+    int getEnd() const { return end_; }
+};
+// Local response normalisation: declared so that programs naming it compile (reference: src/op/dlOp/dlOp.h:765-784);
+// like the reference's generators, this build's emit no code for it.
+class LRNOp : public Op {
+  public:
+    LRNOp() : Op(DL_OP, 1, 1, "LRN") {}
+};
+
 // ---- element-wise / row-wise ----------------------------------------------
 class MatrixTanhOp : public Op {
   public:

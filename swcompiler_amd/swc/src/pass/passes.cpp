@@ -145,6 +145,19 @@ void AutodiffPass::getMethods(const std::string &method, float lr, float decay, 
     lr_ = lr, decay_ = decay, momentum_ = momentum, batch_ = batch;
 }
 
+void AutodiffPass::show() const {
+    SWLOG_INFO << "AutodiffPass: sgd, lr " << lr_ << ", decay " << decay_ << ", momentum " << momentum_ << ", batch "
+               << batch_ << std::endl;
+}
+
+void AutodiffPass::run(IRGraph *graph_train) {
+    if (graph_train) {
+        _graph->copyTo(graph_train);
+        _graph = graph_train;
+    }
+    run();
+}
+
 void AutodiffPass::run() {
     std::vector<IRNode *> order;
     for (int i = 0; i < _graph->topologyNum(); ++i)
@@ -213,6 +226,12 @@ void AutodiffPass::run() {
             auto *cv = static_cast<Conv2dOp *>(op->getOp());
             addGrad(op, new Conv2dGradOp(cv->getKernels(), cv->getStrides(), cv->getPads(), (int)cv->getGroup()),
                     {in(0), in(1), outGrad()});
+        } else if (type == "TensorDescend") {   // tensorOps.cpp:25-85: the gradient is unfolded the way the input was folded
+            auto *d = static_cast<TensorDescendOp *>(op->getOp());
+            addGrad(op, new TensorAscendOp(d->getNDim(), d->getStart(), d->getEnd()), {outGrad()});
+        } else if (type == "TensorAscend") {
+            auto *a = static_cast<TensorAscendOp *>(op->getOp());
+            addGrad(op, new TensorDescendOp(a->getNDim(), a->getStart(), a->getEnd()), {outGrad()});
         } else if (type == "MatrixSoftmaxWithLoss") {
             addGrad(op, new MatrixSoftmaxWithLossGradOp(), {in(1), op->getChildNode(0)});   // label, prob
         } else if (type == "MatrixSoftmax" && op->parentNum() == 2) {   // a label as second operand: the network's end
@@ -424,7 +443,7 @@ void HipFusionPass::run() {
 bool DeviceMemoryLoweringPass::runsOnGpu(const std::string &t) {
     static const std::set<std::string> gpu = {
         "MatrixMatrixMul", "MatrixVectorAdd", "BatchedAdd", "MatrixMatrixFCBias", "MatrixMatrixFCBiasRelu",
-        "MatrixMatrixFCBiasSoftmax", "Reshape", "MatrixTanh", "MatrixSoftmax", "ElementAdd", "ElementAddRelu", "Relu", "Dropout",
+        "MatrixMatrixFCBiasSoftmax", "Reshape", "TensorDescend", "TensorAscend", "MatrixTanh", "MatrixSoftmax", "ElementAdd", "ElementAddRelu", "Relu", "Dropout",
         "Conv2d", "Conv2dWithActivation", "Conv2dBatchNorm", "Conv2dAdd", "MaxPool", "AveragePool", "Transpose",
         "BatchNormalization",
         "BatchNormalizationRelu", "BatchNormReluMaxPool", "ArgMax", "Accuracy",

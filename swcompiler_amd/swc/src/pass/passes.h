@@ -12,6 +12,7 @@
 #include <string>
 #include <unordered_map>
 
+#include "../diff/AutoDiff.h"
 #include "OptimizePass.h"
 
 namespace swc {
@@ -73,20 +74,16 @@ class AutodiffPass : public OptimizePass {
   public:
     explicit AutodiffPass(IRGraph *graph) : OptimizePass(graph) {}
     void getMethods(const std::string &method, float lr, float decay, float momentum, size_t batch);
+    void getMethods() {}   // the settings this object already has
+    void show() const;     // logs the optimizer and its settings
     void run() override;
+    // copies the graph into `graph_train` (a graph the caller has made, empty) and differentiates the copy; with
+    // nullptr the pass's own graph is differentiated (reference: src/pass/AutodiffPass.h:100-105; the TRAIN macro)
+    void run(IRGraph *graph_train);
     int gradOpCount() const { return gradOps_; }
     int sgdCount() const { return sgdOps_; }
 };
 
-} // namespace pass
-
-// The training graph of `graph` as a new graph: a copy with the gradient ops and the SGD updates of the trained
-// parameters added (AutodiffPass on the copy, SGD with the profile's lr / decay / momentum / batch).  The
-// reference's free function of the same name (src/diff/AutoDiff.h:21, AutoDiff.cpp:27-184), which programs
-// written before Engine::compile use; nodes keep their names, so getNodeByName finds them in the copy.
-IRGraph *getTrainNet(IRGraph *graph, TrainingConfig &profile);
-
-namespace pass {
 
 // Transpose(a) followed by Transpose(b) with a[b[i]] == i is the identity: the
 // readers of the second result are rewired to the first operand (the pair itself
