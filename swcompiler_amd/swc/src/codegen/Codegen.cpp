@@ -147,6 +147,7 @@ void Codegen::initMakefileBuilder() {
     makefile_builder_.addCXXFlag("-std=c++11");
     makefile_builder_.addCXXFlag("-O2");
     makefile_builder_.addIncDir("/usr/local/include");
+    if (config_.train_mode) makefile_builder_.addIncDir("$(SWC_HIP_ROOT)/include");   // swc_snapshot.h (header-only)
     makefile_builder_.addCXXSrc("Graph.cpp");
     swmakefile_builder_.setCXXCompiler("mpiCC");
     swmakefile_builder_.addCXXFlag("-O2");
@@ -246,6 +247,10 @@ void Codegen::emitMaxItersBreak() {
 
 // Reference: src/codegen/Codegen.cpp:815-854.
 void Codegen::emitPrintGraphOutputs() {
+    if (config_.train_mode && config_.benchmark) {   // reference: src/codegen/Codegen.cpp:1009-1015
+        writer_ << "// emitPrintGraphOutputs() disabled in benchmark mode\n";
+        return;
+    }
     writer_ << "\nif (iter % " << config_.display << " == 0) {\n";
     writer_.indentInc();
     writer_ << "std::cout << \"iterations \" << iter << \"\\n\";\n";
@@ -395,6 +400,10 @@ void Codegen::emitSnapshotRestoreEnd() {
 
 void Codegen::emitSaveSnapshot() {
     if (!config_.train_mode || !config_.train_config.snapshot) return;
+    if (config_.benchmark) {   // reference: src/codegen/Codegen.cpp:1001-1007
+        writer_ << "// emitSaveSnapshot() disabled in benchmark mode\n";
+        return;
+    }
     writer_ << "\nif (iter % " << config_.train_config.snapshot << " == 0) {\n";
     writer_.indentInc();
     writer_ << "std::cout << \"iter = \" << iter << \", snapshot\\n\";\n";

@@ -203,6 +203,10 @@ void HipCodegen::emitDeviceFills() {
 // snapshot of either program restores the other.  What the device has trained is downloaded into them first.
 void HipCodegen::emitSaveSnapshot() {
     if (!config_.train_mode || !config_.train_config.snapshot) return;
+    if (config_.benchmark) {
+        writer_ << "// emitSaveSnapshot() disabled in benchmark mode\n";
+        return;
+    }
     writer_ << "\nif (iter % " << config_.train_config.snapshot << " == 0) {\n";
     writer_.indentInc();
     writer_ << "std::cout << \"iter = \" << iter << \", snapshot\\n\";\n";
@@ -239,6 +243,10 @@ void HipCodegen::emitDeferredGathers() {
 // The display tensors every Config::display iterations (reference: src/codegen/Codegen.cpp:815-854); one
 // that lives on the device is downloaded there, into its host twin, and the twin is printed.
 void HipCodegen::emitPrintGraphOutputs() {
+    if (config_.train_mode && config_.benchmark) {
+        writer_ << "// emitPrintGraphOutputs() disabled in benchmark mode\n";
+        return;
+    }
     writer_ << "\nif (iter % " << config_.display << " == 0) {\n";
     writer_.indentInc();
     writer_ << "std::cout << \"iterations \" << iter << \"\\n\";\n";

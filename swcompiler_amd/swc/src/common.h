@@ -60,7 +60,7 @@ struct Config {
     bool enable_lowering{true};
     bool compute_op_annotation{false};
     bool comm_op_annotation{false};
-    bool benchmark{false};
+    bool benchmark{false};   // training programs: no snapshots, no display output
     NetTopology net_topo{FC_MESH_NET};
     bool decentralized_optimizer{false};
 
