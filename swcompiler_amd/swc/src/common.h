@@ -39,7 +39,8 @@ struct TrainingConfig {
 };
 
 struct Config {
-    bool train_mode{false};
+    bool train_mode{false};     // Engine::compile adds gradient ops and optimizer updates; the program loops over train_config's records
+    // targets of the reference that this build does not have: setting one makes Engine::compile / Codegen stop with a message
     bool mkldnn{false};
     bool cuda{false};
     bool cublas{false};
@@ -47,20 +48,22 @@ struct Config {
     bool mpi{false};
     int mpi_size{1};
     TrainingConfig train_config;
+    // inference over a file of records: `while (loader.next(label, data))` around the op sequence
     bool use_dataloader{false};
-    std::string dataloader_src;
-    BytesProto label_bytes{ONE_BYTE_AS_INT};
-    BytesProto data_bytes{FOUR_BYTES_AS_FLOAT};
-    size_t dataloader_samples{0};
-    size_t display{0};
+    std::string dataloader_src;                  // the record file
+    BytesProto label_bytes{ONE_BYTE_AS_INT};     // how a record stores its label ...
+    BytesProto data_bytes{FOUR_BYTES_AS_FLOAT};  // ... and its data elements
+    size_t dataloader_samples{0};                // records in the file
+    size_t display{0};                           // > 0: the display tensors are printed every that many iterations
+    bool enable_lowering{true};                  // LoweringPass rewrites FC ops into MatrixMatrixMul + bias add (false: left whole)
+    bool benchmark{false};                       // training programs: no snapshots, no display output
+    // settings of the reference's multi-rank generators: carried for source compatibility, read by nothing here
     ParallelStrategy parallel_preference{MEM_SAVING};
     bool force_data_parallel{false};
     bool handcraft_parallel{false};
     bool geneticalgo_opt_parallel{false};
-    bool enable_lowering{true};
     bool compute_op_annotation{false};
     bool comm_op_annotation{false};
-    bool benchmark{false};   // training programs: no snapshots, no display output
     NetTopology net_topo{FC_MESH_NET};
     bool decentralized_optimizer{false};
 
