@@ -1404,8 +1404,13 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
     const int lda = (int)((M + 3) & ~(size_t)3);   // row length of the transposed outputG
     const int bias_chunks = (int)((M + kBiasRows - 1) / kBiasRows);
     // filter-gradient tiles and splits: about two workgroups per CU (what fits at once)
+    // (up to 64 output channels: tiles of 64 rows, 256 columns wide — or 128 where that covers the kh*kw*iC columns
+    // with over a tenth fewer: 576 columns are 768 on three wide tiles, 640 on five narrow ones)
     const bool narrow = g.OC <= 64;
-    const int bm = narrow ? 64 : 128, bn = narrow ? 256 : 128;
+    bool narrow128 = narrow && ((Kf + 127) / 128 * 128) * 11 < ((Kf + 255) / 256 * 256) * 10;
+    if (const char *e = getenv("SWC_HIP_WGRAD_BN"))   // tuning: 128 or 256 forces the width for narrow layers
+        narrow128 = narrow && atoi(e) == 128;
+    const int bm = narrow ? 64 : 128, bn = narrow && !narrow128 ? 256 : 128;
     const int tiles = ((g.OC + bm - 1) / bm) * (int)((Kf + bn - 1) / bn);
     const int nk = (int)((M + BK - 1) / BK);
     int splits = (2 * num_cus() + tiles - 1) / tiles;
@@ -1514,8 +1519,9 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
                            BK / g.OW, BK % g.OW};
         float *dst = splits > 1 ? part : filterG;
         const size_t a_bytes = ((size_t)(g.OC - 1) * lda + M) * 4;
-        const int rc2 = narrow ? launch_wgrad<1, 4, 2, 2, false, 4>(ogT, a_bytes, lda, bsrc, dst, g.OC, (int)Kf, (int)M, splits, sps)
-                               : launch_wgrad<1, 4, 4, 2, false, 4>(ogT, a_bytes, lda, bsrc, dst, g.OC, (int)Kf, (int)M, splits, sps);
+        const int rc2 = narrow128 ? launch_wgrad<1, 2, 2, 2, false, 4>(ogT, a_bytes, lda, bsrc, dst, g.OC, (int)Kf, (int)M, splits, sps)
+                        : narrow  ? launch_wgrad<1, 4, 2, 2, false, 4>(ogT, a_bytes, lda, bsrc, dst, g.OC, (int)Kf, (int)M, splits, sps)
+                                  : launch_wgrad<1, 4, 4, 2, false, 4>(ogT, a_bytes, lda, bsrc, dst, g.OC, (int)Kf, (int)M, splits, sps);
         if (rc2 != SWC_HIP_OK) return rc2;
         if (splits > 1) {
             if (int rc3 = launch_sum_splits(filterG, part, f_elems, splits)) return rc3;
