@@ -219,6 +219,32 @@ def test_conv2dGrad_many_pixels_split_k(rt, oracle):
         assert_bit_exact(g, w, name)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("width", ["128", "256", None])
+@pytest.mark.parametrize("fdims", [(24, 3, 3, 32), (40, 1, 1, 128)])
+def test_conv2dGrad_narrow_layer_tile_widths(rt, oracle, monkeypatch, width, fdims):
+    """up to 64 output channels: the filter gradient runs on 64 x 128 or 64 x 256 tiles (SWC_HIP_WGRAD_BN forces one;
+    unset, the layer's column count decides: 288 columns take the narrow tiles, 128 the wide one).  Integer-valued
+    operands: the gradients equal the oracle's bit for bit on either."""
+    print("case conv2dGrad tile width", width, fdims, flush=True)
+    if width is None:
+        monkeypatch.delenv("SWC_HIP_WGRAD_BN", raising=False)
+    else:
+        monkeypatch.setenv("SWC_HIP_WGRAD_BN", width)
+    rng = np.random.default_rng(fdims[0])
+    k = fdims[1]
+    pads = (k // 2,) * 4
+    idims = (3, 21, 19, fdims[3])
+    odims = idims[:3] + (fdims[0],)
+    x = rng.integers(-2, 3, idims).astype(np.float32)
+    f = rng.integers(-2, 3, fdims).astype(np.float32)
+    og = rng.integers(-2, 3, odims).astype(np.float32)
+    want = oracle.conv2dGrad(x, f, og, (k, k), (1, 1), pads)
+    got = [t.numpy() for t in rt.conv2dGrad(*up(rt, x, f, og), (k, k), (1, 1), pads)]
+    for g, w, name in zip(got, want, ("inputG", "filterG", "biasG")):
+        assert_bit_exact(g, w, name)
+
+
 def test_workspace_given_by_the_caller(rt, oracle):
     rng = np.random.default_rng(8)
     idims, fdims = (2, 12, 12, 8), (8, 3, 3, 8)
