@@ -19,10 +19,13 @@
  *     reference's CUDA path uses one stream per GPU,
  *     src/codegen/Codegen.cpp:166-172); call swc_hip_sync() before reading
  *     results on the host.  swc_hip_d2h synchronises by itself.
- * Nothing here allocates device memory except swc_hip_malloc and, when no
- * workspace has been provided, the ops that need scratch memory
- * (swc_hip_conv2dGrad_f, swc_hip_matrixSoftmaxWithLoss_f, and the FC/GEMM and
- * convolution entry points for shapes they cut along K; see swc_hip_set_workspace).
+ * Nothing here allocates device memory except swc_hip_malloc: an op that needs
+ * scratch memory (swc_hip_conv2dGrad_f, swc_hip_matrixSoftmaxWithLoss_f, and the
+ * FC/GEMM and convolution entry points for shapes they cut along K) takes it
+ * from the workspace the caller sized with the swc_hip_*_workspace_bytes queries
+ * and handed over with swc_hip_set_workspace, and fails with SWC_HIP_EINVAL when
+ * there is none or it is too small.  (A harness may opt in to a buffer the
+ * library allocates and grows by itself: swc_hip_enable_auto_workspace.)
  * Layouts are the reference's: 4-D activations NHWC, conv filters
  * [oC, kH, kW, iC], matrices row-major.  All data is fp32.
  */
@@ -84,14 +87,22 @@ int swc_hip_sync(void);
 /* No counterpart in the reference (its kernels need no scratch memory).
  * Scratch device memory for the ops that need some (FC/GEMM and convolution
  * calls that are cut along K or run on padded copies: swc_hip_gemm_workspace_bytes,
- * swc_hip_conv2d_workspace_bytes; conv2dGrad_f: the transposed gradient and
- * operand copies, up to about twice the size of its largest argument;
- * matrixSoftmaxWithLoss_f: 4*m bytes).  A generated program allocates the
- * maximum over its calls once and passes it here; without this call the
- * library allocates a buffer of its own on first need and grows it on demand
- * (not possible while a graph is being recorded).  dptr NULL, bytes 0: back to
- * the library's own buffer.  The buffer is shared by all ops on the stream. */
+ * swc_hip_conv2d_workspace_bytes; conv2dGrad_f: swc_hip_conv2dGrad_workspace_bytes;
+ * matrixSoftmaxWithLoss_f: swc_hip_matrixSoftmaxWithLoss_workspace_bytes).  A
+ * generated program allocates the maximum over its calls once and passes it
+ * here; an op that finds no workspace, or one too small, fails with
+ * SWC_HIP_EINVAL and a message naming the query.  dptr NULL, bytes 0: no
+ * workspace.  The buffer is shared by all ops on the stream.  Not while a graph
+ * is being recorded. */
 int swc_hip_set_workspace(void *dptr, size_t bytes);
+/* No counterpart in the reference.  enable != 0: an op that needs more scratch
+ * memory than the current workspace holds lets the library allocate (and later
+ * grow) a buffer of its own instead of failing — for test and bench harnesses
+ * that call ops of many shapes; a generated program never needs it.  The
+ * library's buffer is not replaced while a graph is being recorded, nor while an
+ * executable graph recorded on it is still alive (the call that would need it
+ * fails instead, and so does swc_hip_set_workspace). */
+int swc_hip_enable_auto_workspace(int enable);
 /* No counterpart in the reference.  Workspace a matrixMatrixMul_f /
  * matrixMatrixFCBias_f call of this shape uses on the initialised device (0 for most shapes: only products with few output tiles and a K
  * of hundreds are split over K).  A generated program takes the maximum over its
@@ -108,10 +119,19 @@ size_t swc_hip_gemm_workspace_bytes(int m, int n, int k);
 size_t swc_hip_conv2d_workspace_bytes(const size_t *odims, const size_t *idims, const size_t *fdims,
                                       const size_t *kernels, const size_t *strides, const size_t *pads,
                                       size_t group);
+/* The same for a conv2dGrad_f call (arguments as there): the turned filter, the
+ * transposed output gradient, padded operand copies and the partial sums of the
+ * filter and bias gradients. */
+size_t swc_hip_conv2dGrad_workspace_bytes(const size_t *odims, const size_t *idims, const size_t *fdims,
+                                          const size_t *kernels, const size_t *strides, const size_t *pads,
+                                          size_t group);
+/* The same for a matrixSoftmaxWithLoss_f call over m rows of n (the rows' loss terms). */
+size_t swc_hip_matrixSoftmaxWithLoss_workspace_bytes(int m, int n);
 const char *swc_hip_last_error(void);         /* message of the last failure on this thread ("" if none) */
 void *swc_hip_stream(void);                   /* the hipStream_t ops are launched on */
 int swc_hip_set_stream(void *hip_stream);     /* launch on a caller-owned stream (NULL: back to the library's own) */
 const char *swc_hip_device_name(void);        /* gcnArchName of the selected device */
+int swc_hip_device_cus(void);                 /* its compute units (what the split plans divide work over); 0 before init */
 
 /* Event timing on the library's stream, for harnesses: begin/end bracket a
  * region; elapsed returns milliseconds of the last closed region. */
@@ -123,14 +143,6 @@ float swc_hip_timer_elapsed_ms(void);
  * `second` and returns milliseconds, or a negative value on error. */
 int swc_hip_event_record(int slot);
 float swc_hip_event_elapsed_ms(int first, int second);
-
-/* Diagnostic without a counterpart in the reference: runs `iters` rounds of 16
- * independent v_mfma_f32_32x32x2_f32 per wavefront on two workgroups per CU and
- * returns the elapsed milliseconds and the flop executed, so a harness can print
- * the fp32 matrix rate the device sustains beside the datasheet figure.
- * scratch_dev: device buffer of at least 512 * (number of CUs) floats. */
-int swc_hip_probe_mfma_f32(float *scratch_dev, size_t scratch_floats, int iters,
-                           float *ms_out, double *flop_out);
 
 /* HIP graphs: the ops issued between begin and end are recorded instead of run;
  * launch replays them with a single submission (the launch-bound small graphs —

@@ -15,6 +15,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 LIB = os.path.join(HERE, "libswc_hip.so")
+BENCH_LIB = os.path.join(HERE, "libswc_hip_bench.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -29,7 +30,8 @@ def build_lib(verbose=True, jobs=8):
     """Compile each .hip to an object (in parallel), then link the shared library."""
     objdir = os.path.join(HERE, "csrc", "build")
     os.makedirs(objdir, exist_ok=True)
-    inc = ["-I", os.path.join(ROOT, "include"), "-I", os.path.join(HERE, "csrc")]
+    inc = ["-I", os.path.join(ROOT, "include"), "-I", os.path.join(HERE, "csrc"),
+           "-I", os.path.join(HERE, "swc", "src")]   # devices/HipDevice.h: the device description shared with the code generator
     procs, objs = [], []
     for src in sources():
         obj = os.path.join(objdir, os.path.basename(src)[:-4] + ".o")
@@ -55,6 +57,15 @@ def build_lib(verbose=True, jobs=8):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
+    # the bench-only helper library (include/swc_hip_bench.h): not part of the product ABI
+    cmd = [HIPCC] + FLAGS + ["-I", os.path.join(ROOT, "include"), "-shared", "-o", BENCH_LIB] + \
+        sorted(glob.glob(os.path.join(HERE, "csrc", "bench", "*.hip")))
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if out.returncode != 0:
+        print(out.stdout, file=sys.stderr)
+        raise RuntimeError("hipcc failed (bench library)")
     return LIB
 
 

@@ -7,18 +7,23 @@
 #include <cstdint>
 #include <cstdio>
 
+#include "devices/HipDevice.h"
 #include "swc_hip.h"
 
 namespace swc_hip {
 
+// The device the kernels are written for (shared with the code generator).
+using Device = swc::devices::HipDevice;
+
 // Records a printf-style message for swc_hip_last_error() and returns `code`.
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 void clear_error();
+int fail_code();   // the code of this thread's last fail() (for callers of helpers that return null on failure)
 
 // The stream every op launches on; nullptr until swc_hip_init succeeded.
 hipStream_t stream();
 bool ready();
-int num_cus();
+int num_cus();   // of the initialised device (Device::computeUnits on a whole MI355X)
 // Scratch device memory for the current op (see runtime.hip); nullptr with the error recorded on failure.
 void *workspace(size_t bytes, const char *who);
 

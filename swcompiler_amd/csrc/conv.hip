@@ -206,7 +206,7 @@ struct SkPlan {
 // Tile number -> tile coordinates (see tile_coords): the whole tiles are renumbered for the 8 XCDs, the
 // shared ones are taken in order.
 __device__ __forceinline__ void sk_tile_coords(int pid, int dp_tiles, int tiles_m, int tiles_n, int &tile_m, int &tile_n) {
-    constexpr int kXcd = 8;
+    constexpr int kXcd = Device::xcds;
     if (pid < dp_tiles && dp_tiles % kXcd == 0) pid = (pid % kXcd) * (dp_tiles / kXcd) + pid / kXcd;
     constexpr int kGroup = 8;
     const int per_group = kGroup * tiles_n;
@@ -807,8 +807,8 @@ __global__ __launch_bounds__(256) void pad_channels(float *__restrict__ dst, con
 // output channel co of group g reads only channels [g*iC/group, (g+1)*iC/group) of input and filter): a copy of
 // the filter with every other channel set to zero makes it an ordinary convolution over all channels, whose
 // extra terms are products with zero.
-__global__ __launch_bounds__(256) void mask_filter_groups(float *__restrict__ dst, const float *__restrict__ src, int OC,
-                                                          int taps, int C, int group) {
+__global__ __launch_bounds__(256) void mask_filter_groups(float *dst, const float *src, int OC, int taps, int C,
+                                                          int group) {   // dst may be src
     const size_t total = (size_t)OC * taps * C;
     const int ocg = OC / group, cg = C / group;
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
@@ -904,7 +904,7 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
         if (scratch.ptr && scratch.bytes >= need) base = reinterpret_cast<char *>(scratch.ptr);
         else if (!scratch.ptr) base = static_cast<char *>(workspace(need, who));
         if (!base) return scratch.ptr ? fail(SWC_HIP_EINVAL, "%s: scratch region too small for %zu groups", who, group)
-                                      : SWC_HIP_ERUNTIME;
+                                      : fail_code();
         float *masked = reinterpret_cast<float *>(base);
         const unsigned blocks = ceil_div((size_t)g.OC * g.K, 256);
         mask_filter_groups<<<blocks > 16384 ? 16384 : blocks, 256, 0, stream()>>>(masked, filter, g.OC, g.kh * g.kw, g.C,
@@ -938,7 +938,7 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
         char *base = nullptr;
         if (scratch.ptr && scratch.bytes >= need) base = reinterpret_cast<char *>(scratch.ptr);
         else if (!scratch.ptr) base = static_cast<char *>(workspace(need, who));
-        if (!base && !scratch.ptr) return SWC_HIP_ERUNTIME;
+        if (!base && !scratch.ptr) return fail_code();
         if (base) {
             float *in_p = reinterpret_cast<float *>(base), *f_p = reinterpret_cast<float *>(base + in_b);
             unsigned blocks = ceil_div(M_in * cp, 256);
@@ -966,7 +966,7 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
                 pieces = scratch.ptr;
             } else {
                 pieces = static_cast<float *>(workspace(need, who));
-                if (!pieces) return SWC_HIP_ERUNTIME;
+                if (!pieces) return fail_code();
             }
         }
         return with_dma_variant(pick_dma_variant(g, force, shared), [&]<int TM, int TN, int STAGES, bool MID>() {
@@ -1361,12 +1361,80 @@ size_t wgrad_small_lds(const ConvGeom &g, int rows) {
     return ((size_t)rows * g.OW * g.OC + ((size_t)(rows - 1) * g.sh + g.kh) * g.W * g.C) * sizeof(float);
 }
 
+// Where conv_grad keeps its intermediate results in the workspace, and the kernel choices that decide their
+// sizes; a pure function of the shapes, the device and the operands' alignment, shared by the call and by
+// swc_hip_conv2dGrad_workspace_bytes.
+struct GradLayout {
+    bool dgrad_conv, wgrad_mfma, narrow, narrow128;
+    int lda, bias_chunks, splits, sps, wgrad_rows;
+    size_t ocp, turned_b, ogp_b, dgrad_b, ogt_b, part_b, bias_b;
+    size_t t_odims[4], t_idims[4], t_fdims[4], t_strides[2], t_pads[4];
+    size_t total() const { return turned_b + ogt_b + part_b + bias_b + dgrad_b + ogp_b; }
+};
+
+GradLayout grad_layout(const ConvGeom &g, const size_t *odims, const size_t *idims, const size_t *fdims,
+                       const size_t *kernels, bool input_aligned, bool og_aligned, bool fg_aligned) {
+    GradLayout L{};
+    const size_t M = (size_t)g.M, Kf = (size_t)g.K;
+    const size_t in_elems = idims[0] * idims[1] * idims[2] * idims[3], f_elems = fdims[0] * Kf;
+    // (an input of very few channels leaves the GEMM form with a handful of columns: the gather is faster there)
+    L.dgrad_conv = g.sh == 1 && g.sw == 1 && g.pt <= g.kh - 1 && g.pl <= g.kw - 1 && g.C >= 8;
+    // (the column-interleaved kernel body starts its descriptors 4 KiB early: operands stay below 2 GiB - 64 KiB)
+    L.wgrad_mfma = g.C % 4 == 0 && input_aligned && og_aligned && fg_aligned && in_elems * 4 < 0x7fff0000u &&
+                   (M + 4) * odims[3] * 4 < 0x7fff0000u;
+    L.lda = (int)((M + 3) & ~(size_t)3);   // row length of the transposed outputG
+    L.bias_chunks = (int)((M + kBiasRows - 1) / kBiasRows);
+    // filter-gradient tiles and splits: about two workgroups per CU (what fits at once)
+    // (up to 64 output channels: tiles of 64 rows, 256 columns wide — or 128 where that covers the kh*kw*iC columns
+    // with over a tenth fewer: 576 columns are 768 on three wide tiles, 640 on five narrow ones)
+    L.narrow = g.OC <= 64;
+    L.narrow128 = L.narrow && ((Kf + 127) / 128 * 128) * 11 < ((Kf + 255) / 256 * 256) * 10;
+    if (const char *e = getenv("SWC_HIP_WGRAD_BN"))   // test-only: 128 or 256 forces the width for narrow layers
+        L.narrow128 = L.narrow && atoi(e) == 128;
+    const int bm = L.narrow ? 64 : 128, bn = L.narrow && !L.narrow128 ? 256 : 128;
+    const int tiles = ((g.OC + bm - 1) / bm) * (int)((Kf + bn - 1) / bn);
+    const int nk = (int)((M + BK - 1) / BK);
+    int splits = (2 * num_cus() + tiles - 1) / tiles;
+    splits = splits < 1 ? 1 : (splits > nk ? nk : splits);
+    L.sps = (nk + splits - 1) / splits;
+    L.splits = (nk + L.sps - 1) / L.sps;
+    // the input gradient as a convolution of outputG with the turned filter
+    // (its channel count is OC: padded to a multiple of 4 with zeros where needed, so that the 128-bit gathers
+    // of the MFMA kernels apply — 50 channels: 230 us on the scalar path, 30 with two small copies)
+    L.ocp = (odims[3] + 3) & ~(size_t)3;
+    const size_t t_odims[4] = {idims[0], idims[1], idims[2], idims[3]};
+    const size_t t_idims[4] = {odims[0], odims[1], odims[2], L.ocp};
+    const size_t t_fdims[4] = {idims[3], kernels[0], kernels[1], L.ocp};
+    const size_t t_pads[4] = {(size_t)(g.kh - 1 - g.pt), (size_t)(g.kw - 1 - g.pl), 0, 0};
+    for (int i = 0; i < 4; ++i) L.t_odims[i] = t_odims[i], L.t_idims[i] = t_idims[i], L.t_fdims[i] = t_fdims[i], L.t_pads[i] = t_pads[i];
+    L.t_strides[0] = L.t_strides[1] = 1;
+    L.turned_b = L.dgrad_conv ? align256(idims[3] * fdims[1] * fdims[2] * L.ocp * 4) : 0;
+    L.ogp_b = L.dgrad_conv && L.ocp != odims[3] ? align256(M * L.ocp * 4) : 0;   // outputG with padded channels
+    // (the turned filter lies at the start of the workspace, which is 256-byte aligned like outputG must be)
+    L.dgrad_b = L.dgrad_conv ? align256(conv_scratch_bytes(make_geom(t_odims, t_idims, t_fdims, kernels, L.t_strides, t_pads),
+                                                           og_aligned ? nullptr : reinterpret_cast<const void *>(4), nullptr))
+                             : 0;
+    L.ogt_b = L.wgrad_mfma ? align256((size_t)g.OC * L.lda * 4) : 0;
+    // small filters off the MFMA path: row blocks of about three workgroups per CU, as LDS allows
+    if (!L.wgrad_mfma && f_elems <= 1024 && g.OH > 0 && g.N <= 65535) {
+        int rows = (int)((size_t)g.N * g.OH / (3 * (size_t)num_cus()));
+        rows = rows < 1 ? 1 : (rows > g.OH ? g.OH : rows);
+        while (rows > 1 && wgrad_small_lds(g, rows) > 64 * 1024) --rows;
+        if (wgrad_small_lds(g, rows) <= 64 * 1024 && (g.OH + rows - 1) / rows <= 65535) L.wgrad_rows = rows;
+    }
+    const size_t wgrad_blocks = L.wgrad_rows ? (size_t)g.N * ((g.OH + L.wgrad_rows - 1) / L.wgrad_rows) : 0;
+    L.part_b = L.wgrad_mfma && L.splits > 1 ? align256((size_t)L.splits * f_elems * 4) : align256(wgrad_blocks * f_elems * 4);
+    L.bias_b = align256((size_t)L.bias_chunks * g.OC * 4);
+    return L;
+}
+
 int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG, const float *input,
               const float *filter, const size_t *odims, const size_t *idims, const size_t *fdims,
               const size_t *kernels, const size_t *strides, const size_t *pads, size_t group) {
     const char *who = "swc_hip_conv2dGrad_f";
     if (!odims || !idims || !fdims || !kernels || !strides || !pads) return fail(SWC_HIP_EINVAL, "%s: null shape array", who);
-    if (group != 1) return fail(SWC_HIP_EUNSUPPORTED, "%s: group = %zu (only 1 is supported)", who, group);
+    if (group == 0 || odims[3] % group || idims[3] % group)
+        return fail(SWC_HIP_EINVAL, "%s: group = %zu does not divide oC = %zu and iC = %zu", who, group, odims[3], idims[3]);
     for (int i = 0; i < 4; ++i)
         if (odims[i] > 0x7fffffffu || idims[i] > 0x7fffffffu || fdims[i] > 0x7fffffffu)
             return fail(SWC_HIP_EINVAL, "%s: dimension too large", who);
@@ -1395,58 +1463,29 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
         return rc;
     }
 
-    // ---- workspace layout
-    // (an input of very few channels leaves the GEMM form with a handful of columns: the gather is faster there)
-    const bool dgrad_conv = g.sh == 1 && g.sw == 1 && g.pt <= g.kh - 1 && g.pl <= g.kw - 1 && g.C >= 8;
-    // (the column-interleaved kernel body starts its descriptors 4 KiB early: operands stay below 2 GiB - 64 KiB)
-    const bool wgrad_mfma = g.C % 4 == 0 && aligned16(input) && aligned16(outputG) && aligned16(filterG) &&
-                            in_elems * 4 < 0x7fff0000u && (M + 4) * odims[3] * 4 < 0x7fff0000u;
-    const int lda = (int)((M + 3) & ~(size_t)3);   // row length of the transposed outputG
-    const int bias_chunks = (int)((M + kBiasRows - 1) / kBiasRows);
-    // filter-gradient tiles and splits: about two workgroups per CU (what fits at once)
-    // (up to 64 output channels: tiles of 64 rows, 256 columns wide — or 128 where that covers the kh*kw*iC columns
-    // with over a tenth fewer: 576 columns are 768 on three wide tiles, 640 on five narrow ones)
-    const bool narrow = g.OC <= 64;
-    bool narrow128 = narrow && ((Kf + 127) / 128 * 128) * 11 < ((Kf + 255) / 256 * 256) * 10;
-    if (const char *e = getenv("SWC_HIP_WGRAD_BN"))   // tuning: 128 or 256 forces the width for narrow layers
-        narrow128 = narrow && atoi(e) == 128;
-    const int bm = narrow ? 64 : 128, bn = narrow && !narrow128 ? 256 : 128;
-    const int tiles = ((g.OC + bm - 1) / bm) * (int)((Kf + bn - 1) / bn);
-    const int nk = (int)((M + BK - 1) / BK);
-    int splits = (2 * num_cus() + tiles - 1) / tiles;
-    splits = splits < 1 ? 1 : (splits > nk ? nk : splits);
-    const int sps = (nk + splits - 1) / splits;
-    splits = (nk + sps - 1) / sps;
-    // the input gradient as a convolution of outputG with the turned filter
-    const size_t t_odims[4] = {idims[0], idims[1], idims[2], idims[3]};
-    // (its channel count is OC: padded to a multiple of 4 with zeros where needed, so that the 128-bit gathers
-    // of the MFMA kernels apply — 50 channels: 230 us on the scalar path, 30 with two small copies)
-    const size_t ocp = (odims[3] + 3) & ~(size_t)3;
-    const size_t t_idims[4] = {odims[0], odims[1], odims[2], ocp};
-    const size_t t_fdims[4] = {idims[3], kernels[0], kernels[1], ocp};
-    const size_t t_strides[2] = {1, 1};
-    const size_t t_pads[4] = {(size_t)(g.kh - 1 - g.pt), (size_t)(g.kw - 1 - g.pl), 0, 0};
-    const size_t turned_b = dgrad_conv ? align256(idims[3] * fdims[1] * fdims[2] * ocp * 4) : 0;
-    const size_t ogp_b = dgrad_conv && ocp != odims[3] ? align256(M * ocp * 4) : 0;   // outputG with padded channels
-    // (the turned filter lies at the start of the workspace, which is 256-byte aligned like outputG must be)
-    const size_t dgrad_b =
-        dgrad_conv ? align256(conv_scratch_bytes(make_geom(t_odims, t_idims, t_fdims, kernels, t_strides, t_pads), outputG,
-                                                 nullptr)) : 0;
-    const size_t ogt_b = wgrad_mfma ? align256((size_t)g.OC * lda * 4) : 0;
-    // small filters off the MFMA path: row blocks of about three workgroups per CU, as LDS allows
-    int wgrad_rows = 0;
-    if (!wgrad_mfma && f_elems <= 1024 && g.OH > 0 && g.N <= 65535) {
-        int rows = (int)((size_t)g.N * g.OH / (3 * (size_t)num_cus()));
-        rows = rows < 1 ? 1 : (rows > g.OH ? g.OH : rows);
-        while (rows > 1 && wgrad_small_lds(g, rows) > 64 * 1024) --rows;
-        if (wgrad_small_lds(g, rows) <= 64 * 1024 && (g.OH + rows - 1) / rows <= 65535) wgrad_rows = rows;
+    const GradLayout L = grad_layout(g, odims, idims, fdims, kernels, aligned16(input), aligned16(outputG), aligned16(filterG));
+    const bool dgrad_conv = L.dgrad_conv, wgrad_mfma = L.wgrad_mfma, narrow = L.narrow, narrow128 = L.narrow128;
+    const int lda = L.lda, bias_chunks = L.bias_chunks, splits = L.splits, sps = L.sps, wgrad_rows = L.wgrad_rows;
+    const size_t ocp = L.ocp, turned_b = L.turned_b, ogp_b = L.ogp_b, dgrad_b = L.dgrad_b, ogt_b = L.ogt_b,
+                 part_b = L.part_b, bias_b = L.bias_b;
+    const size_t *t_odims = L.t_odims, *t_idims = L.t_idims, *t_fdims = L.t_fdims, *t_strides = L.t_strides,
+                 *t_pads = L.t_pads;
+    // More than one group, as the reference indexes it (kernels.h:245-319: output channel co of group gr pairs
+    // with channels [gr*iC/group, (gr+1)*iC/group) only): the gradients of the one-group layer whose filter has the
+    // other channels zeroed — inputG then holds exactly the group's terms (plus products with zero), biasG does not
+    // depend on groups, and filterG is right inside the groups and gets its cross-group elements zeroed at the end,
+    // which is what the reference's zero fill leaves there.
+    const size_t mask_b = group > 1 ? align256(f_elems * 4) : 0;
+    char *ws0 = static_cast<char *>(workspace(mask_b + L.total(), who));
+    if (!ws0) return fail_code();
+    char *ws = ws0 + mask_b;
+    const unsigned mask_blocks = ceil_div(f_elems, 256) > 16384 ? 16384 : ceil_div(f_elems, 256);
+    if (group > 1) {
+        float *masked = reinterpret_cast<float *>(ws0);
+        mask_filter_groups<<<mask_blocks, 256, 0, stream()>>>(masked, filter, g.OC, g.kh * g.kw, g.C, (int)group);
+        SWC_LAUNCH_CHECK();
+        filter = masked;
     }
-    const size_t wgrad_blocks = wgrad_rows ? (size_t)g.N * ((g.OH + wgrad_rows - 1) / wgrad_rows) : 0;
-    const size_t part_b = wgrad_mfma && splits > 1 ? align256((size_t)splits * f_elems * 4)
-                                                   : align256(wgrad_blocks * f_elems * 4);
-    const size_t bias_b = align256((size_t)bias_chunks * g.OC * 4);
-    char *ws = static_cast<char *>(workspace(turned_b + ogt_b + part_b + bias_b + dgrad_b + ogp_b, who));
-    if (!ws) return SWC_HIP_ERUNTIME;
     float *turned = reinterpret_cast<float *>(ws);
     float *ogT = reinterpret_cast<float *>(ws + turned_b);
     float *part = reinterpret_cast<float *>(ws + turned_b + ogt_b);
@@ -1536,6 +1575,10 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
         wgrad_direct<<<(unsigned)f_elems, 256, 0, stream()>>>(filterG, outputG, input, g);
         SWC_LAUNCH_CHECK();
     }
+    if (group > 1) {   // element-wise, in place
+        mask_filter_groups<<<mask_blocks, 256, 0, stream()>>>(filterG, filterG, g.OC, g.kh * g.kw, g.C, (int)group);
+        SWC_LAUNCH_CHECK();
+    }
     return SWC_HIP_OK;
 }
 
@@ -1591,6 +1634,20 @@ size_t swc_hip_conv2d_workspace_bytes(const size_t *odims, const size_t *idims, 
     const size_t masked = group > 1 ? align256((size_t)g.OC * g.K * 4) : 0;
     if (g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0) return masked;
     return masked + conv_total_scratch(g, nullptr, nullptr);   // (tensors of a generated program are 256-byte aligned)
+}
+
+size_t swc_hip_conv2dGrad_workspace_bytes(const size_t *odims, const size_t *idims, const size_t *fdims,
+                                          const size_t *kernels, const size_t *strides, const size_t *pads, size_t group) {
+    if (!ready() ||
+        check_conv_dims("swc_hip_conv2dGrad_workspace_bytes", odims, idims, fdims, kernels, strides, pads, group, true))
+        return 0;
+    const ConvGeom g = make_geom(odims, idims, fdims, kernels, strides, pads);
+    const size_t f_elems = fdims[0] * fdims[1] * fdims[2] * fdims[3];
+    if (g.M == 0 || g.OC == 0 || f_elems == 0 || idims[0] * idims[1] * idims[2] * idims[3] == 0) return 0;
+    // operands on 16-byte boundaries (every tensor of a generated program) or not: the larger of the two layouts
+    const size_t a = grad_layout(g, odims, idims, fdims, kernels, true, true, true).total();
+    const size_t u = grad_layout(g, odims, idims, fdims, kernels, false, false, false).total();
+    return (group > 1 ? align256(f_elems * 4) : 0) + (a > u ? a : u);
 }
 
 int swc_hip_conv2dGrad_f(float *inputG, float *filterG, float *biasG, const float *outputG, const float *input,

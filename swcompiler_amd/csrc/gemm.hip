@@ -21,6 +21,13 @@ using namespace swc_hip::mfma;
 
 namespace {
 
+// Where a product cut along K keeps its partial tiles: a fixed region (the call fails if it is too small), or,
+// with ptr == nullptr, the workspace.
+struct PartialStore {
+    float *ptr = nullptr;
+    size_t bytes = 0;
+};
+
 // ---------------------------------------------------------------- tiled GEMM
 // VEC: A and B rows may be read with aligned 128-bit loads (lda, ldb, K, N
 // multiples of 4 and 16-byte aligned bases).  Otherwise 32-bit loads.
@@ -483,10 +490,18 @@ int launch_dma2(const float *a, const float *b, float *c, int m, int n, int k, i
 
 template <int TM, int TN, int WM, int STAGES>
 int launch_splitk(const float *a, const float *b, float *c, int m, int n, int k, int lda, int ldb, int ldc,
-                  const Epilogue &ep, int splits, int sps) {
+                  const Epilogue &ep, int splits, int sps, const PartialStore &fixed) {
     using T = Dma2Tile<TM, TN, WM, STAGES, 4>;
-    float *part = static_cast<float *>(workspace((size_t)splits * m * n * sizeof(float), "gemm (split-K)"));
-    if (!part) return SWC_HIP_ERUNTIME;
+    const size_t need = (size_t)splits * m * n * sizeof(float);
+    float *part = fixed.ptr;
+    if (part) {
+        if (need > fixed.bytes)
+            return fail(SWC_HIP_EINVAL, "gemm (split-K): the partial tiles take %zu bytes, the fixed scratch holds %zu",
+                        need, fixed.bytes);
+    } else {
+        part = static_cast<float *>(workspace(need, "gemm (split-K)"));
+        if (!part) return fail_code();   // (no workspace, one too small, or the allocation failed)
+    }
     auto kern = gemm_dma2_splitk<TM, TN, WM, STAGES, false, 4>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -539,9 +554,19 @@ bool splitk_plan(int m, int n, int k, int &splits, int &sps, bool forced = false
     return splits > 1 && (size_t)splits * m * n * 4 <= ((size_t)64 << 20);
 }
 
+// The one decision function for "is this product cut along K, and how": the dispatch, swc_hip_gemm_workspace_bytes
+// and the entry point with fixed scratch all ask it, so a size query always matches what the call then does.
+// SWC_HIP_GEMM is a test-only variable (it forces a kernel variant; read per call so that one test process can run
+// every variant): "splitk" forces the cut for shapes the plan would leave whole, any other value rules it out.
+bool splitk_decision(int m, int n, int k, int &splits, int &sps) {
+    const char *force = getenv("SWC_HIP_GEMM");
+    if (force && strcmp(force, "splitk")) return false;
+    return splitk_plan(m, n, k, splits, sps, force != nullptr);
+}
+
 // softmax != 0: the row softmax of the result is stored instead of the result (n <= 16 only: the caller checks)
 int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda, const float *b, int ldb,
-                  const float *bias, float *c, int ldc, int relu, int softmax = 0) {
+                  const float *bias, float *c, int ldc, int relu, int softmax = 0, const PartialStore &fixed = {}) {
     if (m < 0 || n < 0 || k < 0) return fail(SWC_HIP_EINVAL, "%s: negative dimension", who);
     if (m == 0 || n == 0) return SWC_HIP_OK;
     if (!a || !b || !c) return fail(SWC_HIP_EINVAL, "%s: null pointer", who);
@@ -603,10 +628,10 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
         // tiles next, and 64x64 tiles for everything smaller, where the number of workgroups matters more than
         // their efficiency.
         int splits = 0, sps = 0;
-        if (dma2_ok && (!force || !strcmp(force, "splitk")) && splitk_plan(m, n, k, splits, sps, force != nullptr))
-            return !takes_thin(m, n, k) ? launch_splitk<1, 4, 4, 2>(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps)
-                   : m <= 32            ? launch_splitk<1, 2, 1, 3>(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps)
-                                        : launch_splitk<2, 2, 1, 3>(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps);
+        if (dma2_ok && splitk_decision(m, n, k, splits, sps))
+            return !takes_thin(m, n, k) ? launch_splitk<1, 4, 4, 2>(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps, fixed)
+                   : m <= 32            ? launch_splitk<1, 2, 1, 3>(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps, fixed)
+                                        : launch_splitk<2, 2, 1, 3>(a, b, c, m, n, k, lda, ldb, ldc, ep, splits, sps, fixed);
         if (dma2_ok && huge_tiles >= num_cus()) return launch_dma2<2, 4, 4, 2, false, 8>(a, b, c, m, n, k, lda, ldb, ldc, ep);
         if (dma2_ok && big_tiles >= num_cus()) return launch_dma2<1, 4, 4, 2, false>(a, b, c, m, n, k, lda, ldb, ldc, ep);
         if (big_tiles >= num_cus()) return launch_dma<2, 2, 2>(a, b, c, m, n, k, lda, ldb, ldc, ep);
@@ -629,7 +654,7 @@ int swc_hip_matrixMatrixMul_f(int m, int n, int k, const float *a, int lda, cons
 size_t swc_hip_gemm_workspace_bytes(int m, int n, int k) {
     if (!ready() || m <= 0 || n <= 0 || k <= 0) return 0;
     int splits = 0, sps = 0;
-    return splitk_plan(m, n, k, splits, sps) ? (size_t)splits * m * n * sizeof(float) : 0;
+    return splitk_decision(m, n, k, splits, sps) ? (size_t)splits * m * n * sizeof(float) : 0;
 }
 
 int swc_hip_matrixMatrixFCBias_f(int m, int n, int k, const float *a, int lda, const float *b, int ldb,

@@ -58,6 +58,7 @@ struct DmaTile {
     static constexpr int kBLoads = BN / 32;
     static constexpr int kLoads = kALoads + kBLoads;
     static_assert(STAGES >= 2 && (STAGES - 2) * kLoads < 64, "pending loads must fit the vmcnt field");
+    static_assert(kLdsBytes <= swc::devices::HipDevice::ldsBytesPerCU, "the ring must fit one CU's LDS");
 };
 
 #if __HIP_DEVICE_COMPILE__   // buffer-resource types and LDS-DMA builtins exist in the device pass only

@@ -39,6 +39,7 @@ struct Dma2Tile {
     static_assert(kALoads >= 1 && kBLoads >= 1 && kALoads * 8 * NW == BM && kBLoads * 8 * NW == BN, "");
     static_assert(TN == 2 || TN == 4, "a lane reads TN consecutive floats");
     static_assert(STAGES >= 2 && (STAGES - 1) * kLoads < 64, "pending loads must fit the vmcnt field");
+    static_assert(kLdsBytes <= swc::devices::HipDevice::ldsBytesPerCU, "the ring must fit one CU's LDS");
 };
 
 #if __HIP_DEVICE_COMPILE__

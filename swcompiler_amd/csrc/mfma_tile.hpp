@@ -23,6 +23,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include "devices/HipDevice.h"
+
 namespace swc_hip {
 namespace mfma {
 
@@ -231,7 +233,7 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], float *__r
 __device__ __forceinline__ void tile_coords(int tiles_m, int tiles_n, int &tile_m, int &tile_n) {
     const int total = tiles_m * tiles_n;
     int pid = blockIdx.x;
-    constexpr int kXcd = 8;
+    constexpr int kXcd = swc::devices::HipDevice::xcds;
     if (total % kXcd == 0) pid = (pid % kXcd) * (total / kXcd) + pid / kXcd;
     constexpr int kGroup = 8;
     const int per_group = kGroup * tiles_n;

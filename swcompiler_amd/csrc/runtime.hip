@@ -10,8 +10,10 @@
 namespace swc_hip {
 namespace {
 
-thread_local char g_err[512] = "";
+thread_local char g_err[768] = "";
+thread_local int g_err_code = SWC_HIP_OK;
 constexpr int kEventSlots = 4096;
+constexpr int kGraphSlots = 256;
 
 struct State {
     std::mutex mu;
@@ -33,6 +35,11 @@ struct State {
     void *ws = nullptr;
     size_t ws_bytes = 0;
     bool ws_owned = false;
+    bool ws_auto = false;   // the library may allocate and grow a buffer of its own (swc_hip_enable_auto_workspace)
+    // executable graphs recorded while the library's own buffer was the workspace: their kernels keep its
+    // address, so it is neither freed nor replaced before the last of them is destroyed
+    void *graphs_on_own_ws[kGraphSlots] = {};
+    int n_graphs_on_own_ws = 0;
 } g;
 
 template <typename T> __global__ void fill_kernel(T *__restrict__ dst, T v, size_t n) {
@@ -48,28 +55,46 @@ int fail(int code, const char *fmt, ...) {
     va_start(ap, fmt);
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
+    g_err_code = code;
     return code;
 }
-void clear_error() { g_err[0] = 0; }
+void clear_error() { g_err[0] = 0, g_err_code = SWC_HIP_OK; }
+int fail_code() { return g_err_code != SWC_HIP_OK ? g_err_code : SWC_HIP_ERUNTIME; }
 hipStream_t stream() { return g.cur; }
 bool ready() { return g.ready; }
 int num_cus() { return g.cus; }
 
 // Device memory an op may use until it returns control to the stream's next op
-// (all ops run on one in-order stream, so one buffer serves them all).  The
-// caller's buffer (swc_hip_set_workspace) is used when it is large enough;
-// otherwise the library keeps one of its own and grows it on demand — never
-// while a graph is being recorded, where allocating is not allowed.
+// (all ops run on one in-order stream, so one buffer serves them all).  Ops never
+// allocate: the buffer is the caller's (swc_hip_set_workspace), sized with the
+// swc_hip_*_workspace_bytes queries.  Only a caller that opted in with
+// swc_hip_enable_auto_workspace lets the library keep one of its own, grown on
+// demand — never while a graph is being recorded, where allocating is not
+// allowed, and never while a recorded graph still holds the old buffer's address.
 void *workspace(size_t bytes, const char *who) {
     if (bytes <= g.ws_bytes && g.ws) return g.ws;
+    if (g.ws && !g.ws_owned) {
+        fail(SWC_HIP_EINVAL, "%s: the workspace given to swc_hip_set_workspace has %zu bytes, %zu are needed", who,
+             g.ws_bytes, bytes);
+        return nullptr;
+    }
+    if (!g.ws_auto) {
+        fail(SWC_HIP_EINVAL, "%s: needs %zu bytes of scratch memory and no workspace is set: size one with "
+             "swc_hip_gemm_workspace_bytes / swc_hip_conv2d_workspace_bytes / swc_hip_conv2dGrad_workspace_bytes / "
+             "swc_hip_matrixSoftmaxWithLoss_workspace_bytes and pass it to swc_hip_set_workspace (ops do not allocate; "
+             "swc_hip_enable_auto_workspace lets the library keep a buffer of its own)", who, bytes);
+        return nullptr;
+    }
     if (g.capturing) {
         fail(SWC_HIP_ERUNTIME, "%s: needs a %zu-byte workspace, which cannot be allocated while a graph is recorded; "
              "run the op once eagerly first or provide one with swc_hip_set_workspace", who, bytes);
         return nullptr;
     }
-    if (g.ws && !g.ws_owned) {
-        fail(SWC_HIP_EINVAL, "%s: the workspace given to swc_hip_set_workspace has %zu bytes, %zu are needed", who,
-             g.ws_bytes, bytes);
+    if (g.ws && g.n_graphs_on_own_ws > 0) {
+        fail(SWC_HIP_ERUNTIME, "%s: needs a %zu-byte workspace, but %d recorded graph(s) still use the library's "
+             "%zu-byte buffer, which therefore cannot be replaced: destroy them first, or provide a workspace large "
+             "enough for every op with swc_hip_set_workspace before recording", who, bytes, g.n_graphs_on_own_ws,
+             g.ws_bytes);
         return nullptr;
     }
     if (g.ws) {
@@ -115,9 +140,9 @@ int swc_hip_init(int device) {
     hipDeviceProp_t prop;
     SWC_HIP_TRY(hipGetDeviceProperties(&prop, device));
     snprintf(g.arch, sizeof(g.arch), "%s", prop.gcnArchName);
-    if (std::strncmp(g.arch, "gfx950", 6) != 0)
-        return fail(SWC_HIP_EUNSUPPORTED, "swc_hip_init: kernels are built for gfx950 only, device is %s", g.arch);
-    g.cus = prop.multiProcessorCount;
+    if (std::strncmp(g.arch, Device::arch, std::strlen(Device::arch)) != 0)
+        return fail(SWC_HIP_EUNSUPPORTED, "swc_hip_init: kernels are built for %s only, device is %s", Device::arch, g.arch);
+    g.cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : Device::computeUnits;
     SWC_HIP_TRY(hipStreamCreateWithFlags(&g.own, hipStreamNonBlocking));
     SWC_HIP_TRY(hipEventCreate(&g.t0));
     SWC_HIP_TRY(hipEventCreate(&g.t1));
@@ -137,6 +162,9 @@ int swc_hip_shutdown(void) {
     g.ws = nullptr;
     g.ws_bytes = 0;
     g.ws_owned = false;
+    g.ws_auto = false;
+    g.n_graphs_on_own_ws = 0;
+    for (void *&h : g.graphs_on_own_ws) h = nullptr;
     (void)hipEventDestroy(g.t0);
     (void)hipEventDestroy(g.t1);
     if (g.copy) {
@@ -167,13 +195,24 @@ int swc_hip_set_workspace(void *dptr, size_t bytes) {
     std::lock_guard<std::mutex> lk(g.mu);
     SWC_ARG((dptr == nullptr) == (bytes == 0));
     SWC_ARG(aligned16(dptr));
+    if (g.capturing) return fail(SWC_HIP_EINVAL, "swc_hip_set_workspace: not while a graph is being recorded");
     if (g.ws && g.ws_owned) {
+        if (g.n_graphs_on_own_ws > 0)
+            return fail(SWC_HIP_ERUNTIME, "swc_hip_set_workspace: %d recorded graph(s) still use the library's own "
+                        "buffer; destroy them before replacing it", g.n_graphs_on_own_ws);
         SWC_HIP_TRY(hipStreamSynchronize(g.cur));
         SWC_HIP_TRY(hipFree(g.ws));
     }
     g.ws = dptr;
     g.ws_bytes = bytes;
     g.ws_owned = false;
+    return SWC_HIP_OK;
+}
+
+int swc_hip_enable_auto_workspace(int enable) {
+    SWC_REQUIRE_INIT();
+    std::lock_guard<std::mutex> lk(g.mu);
+    g.ws_auto = enable != 0;
     return SWC_HIP_OK;
 }
 
@@ -318,6 +357,8 @@ int swc_hip_fill_i(int *dst, int value, size_t count) {
     return SWC_HIP_OK;
 }
 
+int swc_hip_device_cus(void) { return ready() ? g.cus : 0; }
+
 int swc_hip_sync(void) {
     SWC_REQUIRE_INIT();
     SWC_HIP_TRY(hipStreamSynchronize(stream()));
@@ -381,6 +422,17 @@ int swc_hip_graph_end(void **graph_out) {
     hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);
     if (e != hipSuccess) return fail(SWC_HIP_ERUNTIME, "swc_hip_graph_end: hipGraphInstantiate -> %s", hipGetErrorString(e));
+    if (g.ws && g.ws_owned) {   // its kernels may hold the address of the library's own buffer
+        int slot = 0;
+        while (slot < kGraphSlots && g.graphs_on_own_ws[slot]) ++slot;
+        if (slot == kGraphSlots) {
+            (void)hipGraphExecDestroy(exec);
+            return fail(SWC_HIP_ERUNTIME, "swc_hip_graph_end: more than %d graphs alive on the library's own workspace; "
+                        "provide one with swc_hip_set_workspace", kGraphSlots);
+        }
+        g.graphs_on_own_ws[slot] = (void *)exec;
+        ++g.n_graphs_on_own_ws;
+    }
     *graph_out = (void *)exec;
     return SWC_HIP_OK;
 }
@@ -397,6 +449,11 @@ int swc_hip_graph_destroy(void *graph) {
     if (!graph) return SWC_HIP_OK;
     SWC_HIP_TRY(hipStreamSynchronize(stream()));
     SWC_HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph));
+    for (void *&h : g.graphs_on_own_ws)
+        if (h == graph) {
+            h = nullptr;
+            --g.n_graphs_on_own_ws;
+        }
     return SWC_HIP_OK;
 }
 

@@ -397,13 +397,17 @@ int swc_hip_matrixSoftmaxWithLoss_f(int m, int n, const float *a, int lda, float
     if (m == 0 || n == 0) return swc_hip_fill_f(loss, 0.f, 1);   // the reference would divide 0 by m
     SWC_ARG(a && b && selected);
     float *terms = static_cast<float *>(workspace((size_t)m * sizeof(float), "swc_hip_matrixSoftmaxWithLoss_f"));
-    if (!terms) return SWC_HIP_ERUNTIME;
+    if (!terms) return fail_code();
     // the loss terms read a before the softmax may overwrite it (b may alias a)
     softmax_loss_terms<<<ceil_div(m, kThreads / 64), kThreads, 0, stream()>>>(m, n, a, lda, selected, terms);
     SWC_LAUNCH_CHECK();
     loss_mean<<<1, 1024, 0, stream()>>>(m, terms, loss);
     SWC_LAUNCH_CHECK();
     return swc_hip_matrixSoftmax_f(m, n, a, lda, b, ldb);
+}
+
+size_t swc_hip_matrixSoftmaxWithLoss_workspace_bytes(int m, int n) {
+    return (m > 0 && n > 0) ? (size_t)m * sizeof(float) : 0;
 }
 
 int swc_hip_matrixTrans_f(int m, int n, const float *a, int lda, float *b, int ldb) {

@@ -20,7 +20,8 @@ EXPORTS = [
     "swc_hip_d2d", "swc_hip_copy_h2d_async", "swc_hip_copy_wait_ops", "swc_hip_ops_wait_copies", "swc_hip_copy_sync", "swc_hip_fill_f", "swc_hip_sync", "swc_hip_last_error", "swc_hip_stream",
     "swc_hip_set_stream", "swc_hip_device_name", "swc_hip_timer_begin", "swc_hip_timer_end",
     "swc_hip_timer_elapsed_ms", "swc_hip_event_record", "swc_hip_event_elapsed_ms", "swc_hip_graph_begin",
-    "swc_hip_graph_end", "swc_hip_graph_launch", "swc_hip_graph_destroy", "swc_hip_probe_mfma_f32",
+    "swc_hip_graph_end", "swc_hip_graph_launch", "swc_hip_graph_destroy", "swc_hip_device_cus",
+    "swc_hip_enable_auto_workspace", "swc_hip_conv2dGrad_workspace_bytes", "swc_hip_matrixSoftmaxWithLoss_workspace_bytes",
     "swc_hip_matrixMatrixMul_f", "swc_hip_batchedadd_f", "swc_hip_relu_f",
     "swc_hip_vecAdd_f", "swc_hip_conv2d_f", "swc_hip_batchnormalization_f", "swc_hip_maxpool_f",
     "swc_hip_maxpool_argmax_f", "swc_hip_avgpool_f", "swc_hip_transpose4d_f", "swc_hip_transpose2d_f",
@@ -77,7 +78,10 @@ def load_library():
         "swc_hip_graph_end": (i32, [C.POINTER(vp)]),
         "swc_hip_graph_launch": (i32, [vp]),
         "swc_hip_graph_destroy": (i32, [vp]),
-        "swc_hip_probe_mfma_f32": (i32, [vp, sz, i32, C.POINTER(f32), C.POINTER(C.c_double)]),
+        "swc_hip_device_cus": (i32, []),
+        "swc_hip_enable_auto_workspace": (i32, [i32]),
+        "swc_hip_conv2dGrad_workspace_bytes": (sz, [szp] * 6 + [sz]),
+        "swc_hip_matrixSoftmaxWithLoss_workspace_bytes": (sz, [i32, i32]),
         "swc_hip_matrixMatrixMul_f": (i32, [i32, i32, i32, vp, i32, vp, i32, vp, i32]),
         "swc_hip_batchedadd_f": (i32, [vp, vp, vp, sz, sz]),
         "swc_hip_relu_f": (i32, [vp, vp, sz]),
@@ -187,10 +191,21 @@ class DeviceArray:
 class SwcHip:
     """One process-wide runtime: device 0 unless told otherwise."""
 
-    def __init__(self, device=0):
+    def __init__(self, device=0, auto_workspace=True):
+        """auto_workspace: let the library keep (and grow) a scratch buffer of its own, as a harness that calls
+        ops of many shapes wants; False: ops that need scratch fail until set_workspace() provides it, as in a
+        generated program."""
         self.lib = load_library()
         self._check(self.lib.swc_hip_init(device), "swc_hip_init")
+        self._check(self.lib.swc_hip_enable_auto_workspace(int(auto_workspace)), "swc_hip_enable_auto_workspace")
         self._pinned = {}   # address of a pinned numpy array -> the pointer to free
+        self._bench_lib = None
+
+    def enable_auto_workspace(self, on):
+        self._check(self.lib.swc_hip_enable_auto_workspace(int(on)), "swc_hip_enable_auto_workspace")
+
+    def device_cus(self):
+        return int(self.lib.swc_hip_device_cus())
 
     # -- plumbing --------------------------------------------------------
     def _check(self, rc, what):
@@ -254,11 +269,23 @@ class SwcHip:
         self._check(self.lib.swc_hip_copy_sync(), "swc_hip_copy_sync")
 
     def probe_mfma_tflops(self, iters=2000):
-        """fp32 MFMA rate a register-only loop sustains (TFLOP/s) and its duration in ms"""
+        """fp32 MFMA rate a register-only loop sustains (TFLOP/s) and its duration in ms; runs the bench-only
+        helper library (include/swc_hip_bench.h) on the library's stream"""
+        if self._bench_lib is None:
+            path = os.path.join(_HERE, "libswc_hip_bench.so")
+            if not os.path.exists(path):
+                raise SwcHipError(f"{path} is missing: build it with `python -m swcompiler_amd.build`")
+            self._bench_lib = C.CDLL(path)
+            self._bench_lib.swc_hip_bench_probe_mfma_f32.restype = C.c_int
+            self._bench_lib.swc_hip_bench_probe_mfma_f32.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_size_t, C.c_int,
+                                                                     C.POINTER(C.c_float), C.POINTER(C.c_double)]
+        self.sync()
         scratch = self.empty((512 * 512,))
         ms, flop = C.c_float(), C.c_double()
-        self._check(self.lib.swc_hip_probe_mfma_f32(scratch.ptr, scratch.size, iters, C.byref(ms), C.byref(flop)),
-                    "swc_hip_probe_mfma_f32")
+        rc = self._bench_lib.swc_hip_bench_probe_mfma_f32(self.lib.swc_hip_stream(), self.device_cus(), scratch.ptr,
+                                                          scratch.size, iters, C.byref(ms), C.byref(flop))
+        if rc != 0:
+            raise SwcHipError(f"swc_hip_bench_probe_mfma_f32 failed (hipError {rc})")
         scratch.free()
         return flop.value / (ms.value * 1e-3) / 1e12, ms.value
 
@@ -522,6 +549,11 @@ class SwcHip:
         odims = pool_out_dims(xshape, fshape[1:3], strides, pads)[:3] + (fshape[0],)
         return int(self.lib.swc_hip_conv2d_workspace_bytes(_dims(odims), _dims(xshape), _dims(fshape), _dims(fshape[1:3]),
                                                            _dims(strides), _dims(pads), group))
+
+    def conv2dGrad_workspace_bytes(self, xshape, fshape, strides=(1, 1), pads=(0, 0, 0, 0), group=1):
+        odims = pool_out_dims(xshape, fshape[1:3], strides, pads)[:3] + (fshape[0],)
+        return int(self.lib.swc_hip_conv2dGrad_workspace_bytes(_dims(odims), _dims(xshape), _dims(fshape),
+                                                               _dims(fshape[1:3]), _dims(strides), _dims(pads), group))
 
     def set_workspace(self, arr):
         """give the library a DeviceArray to use as scratch (None: its own buffer again)"""

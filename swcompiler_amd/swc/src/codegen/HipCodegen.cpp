@@ -90,6 +90,16 @@ void HipCodegen::emitWorkspace() {
               << arrayDef("k", conv->getKernels()) << arrayDef("s", conv->getStrides()) << arrayDef("p", conv->getPads())
               << "gpu0_ws_bytes = std::max(gpu0_ws_bytes, swc_hip_conv2d_workspace_bytes(o, i, f, k, s, p, "
               << conv->getGroup() << "));\n}\n";
+        } else if (type == "Conv2dGrad") {   // parents: input, filter, outputGrad
+            auto *conv = static_cast<Conv2dGradOp *>(op->getOp());
+            q << "{\n"
+              << arrayDef("o", T(2)->getDims()) << arrayDef("i", T(0)->getDims()) << arrayDef("f", T(1)->getDims())
+              << arrayDef("k", conv->getKernels()) << arrayDef("s", conv->getStrides()) << arrayDef("p", conv->getPads())
+              << "gpu0_ws_bytes = std::max(gpu0_ws_bytes, swc_hip_conv2dGrad_workspace_bytes(o, i, f, k, s, p, "
+              << conv->getGroup() << "));\n}\n";
+        } else if (type == "MatrixSoftmaxWithLoss") {
+            q << "gpu0_ws_bytes = std::max(gpu0_ws_bytes, swc_hip_matrixSoftmaxWithLoss_workspace_bytes(" << T(0)->getDim(0)
+              << ", " << T(0)->getDim(1) << "));\n";
         } else {
             continue;
         }
@@ -105,8 +115,7 @@ void HipCodegen::emitWorkspace() {
 }
 
 void HipCodegen::emitMemAllocations() {
-    // (a training program leaves the scratch memory to the library: the gradient kernels size their own)
-    if (!config_.train_mode) emitWorkspace();
+    emitWorkspace();   // ops never allocate: the program sizes the scratch memory of all its calls, gradients included
     for (auto &a : mem_allocators_) {
         if (!a->getMemAllocated()) continue;
         if (a->getDevice().type == DeviceType::CPU) {

@@ -162,3 +162,35 @@ def test_hip_graph_replay_equals_eager(rt, cfg, batch):
     assert_bit_exact(replay2, eager2, "replay on new input")
     assert not np.array_equal(replay2, eager)
     rt.graph_destroy(handle)
+
+
+def test_library_workspace_is_not_replaced_under_a_recorded_graph(rt):
+    """A graph recorded while the library's own scratch buffer (swc_hip_enable_auto_workspace) served a
+    split-K product keeps that buffer's address in its kernel arguments: until the graph is destroyed an op that
+    needs a larger buffer fails instead of freeing it, and so does swc_hip_set_workspace; the graph still replays."""
+    from swcompiler_amd.hip import SwcHipError
+    rng = np.random.default_rng(3)
+    rt.sync()
+    rt.set_workspace(None)                      # drop whatever earlier tests grew
+    a = rt.upload(rng.standard_normal((96, 512)).astype(np.float32))
+    w = rt.upload(rng.standard_normal((512, 200)).astype(np.float32))
+    out = rt.empty((96, 200))
+    small, big = rt.gemm_workspace_bytes(96, 200, 512), rt.gemm_workspace_bytes(256, 500, 800)
+    assert 0 < small < big - (1 << 20)          # (the library rounds its buffer up to 1 MiB)
+    rt.fcbias(a, w, None, out=out)              # eager: the library allocates `small`
+    eager = out.numpy().copy()
+    handle = rt.capture(lambda: rt.fcbias(a, w, None, out=out))
+    a2, w2 = rt.empty((256, 800)), rt.empty((800, 500))
+    try:
+        with pytest.raises(SwcHipError, match="recorded graph"):
+            rt.fcbias(a2, w2, None)             # would need `big`
+        ws = rt.empty((big // 4,))
+        with pytest.raises(SwcHipError, match="recorded graph"):
+            rt.set_workspace(ws)
+        rt.lib.swc_hip_fill_f(out.ptr, 0.0, out.size)
+        rt.graph_launch(handle)
+        assert_bit_exact(out.numpy(), eager, "replay after the refused growth")
+    finally:
+        rt.graph_destroy(handle)
+    rt.fcbias(a2, w2, None)                     # the graph is gone: the buffer may grow now
+    rt.sync()

@@ -270,7 +270,7 @@ def test_conv_groups_in_a_caller_workspace_and_error_paths(rt, oracle):
     with pytest.raises(SwcHipError, match="group"):
         rt.conv2d(*z, group=3)          # divides neither channel count
     with pytest.raises(SwcHipError, match="group"):
-        rt.conv2dGrad(z[0], z[1], rt.upload(np.zeros((1, 4, 4, 4), np.float32)), group=2)   # gradients: one group only
+        rt.conv2dGrad(z[0], z[1], rt.upload(np.zeros((1, 4, 4, 4), np.float32)), group=3)   # the gradients likewise
 
 
 # ------------------------------------------------------- batchnorm / pool

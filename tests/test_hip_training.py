@@ -221,11 +221,13 @@ def test_conv2dGrad_many_pixels_split_k(rt, oracle):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("width", ["128", "256", None])
-@pytest.mark.parametrize("fdims", [(24, 3, 3, 32), (40, 1, 1, 128)])
+@pytest.mark.parametrize("fdims", [(24, 3, 3, 32), (40, 1, 1, 128), (24, 1, 1, 256), (24, 3, 3, 128), (24, 1, 1, 1408)])
 def test_conv2dGrad_narrow_layer_tile_widths(rt, oracle, monkeypatch, width, fdims):
     """up to 64 output channels: the filter gradient runs on 64 x 128 or 64 x 256 tiles (SWC_HIP_WGRAD_BN forces one;
-    unset, the layer's column count decides: 288 columns take the narrow tiles, 128 the wide one).  Integer-valued
-    operands: the gradients equal the oracle's bit for bit on either."""
+    unset, the narrow tiles are taken where they cover the kh*kw*iC columns with over a tenth fewer: 288 and 128
+    columns take them; 256 columns fill one wide tile exactly and keep it; 1152 columns (nine narrow tiles against
+    1280 covered by five wide ones, a ratio of 0.9) sit just on the narrow side of the rule and 1408 (against 1536:
+    0.917) just on the wide side).  Integer-valued operands: the gradients equal the oracle's bit for bit on either."""
     print("case conv2dGrad tile width", width, fdims, flush=True)
     if width is None:
         monkeypatch.delenv("SWC_HIP_WGRAD_BN", raising=False)
@@ -245,6 +247,36 @@ def test_conv2dGrad_narrow_layer_tile_widths(rt, oracle, monkeypatch, width, fdi
         assert_bit_exact(g, w, name)
 
 
+@pytest.mark.parametrize("case", [
+    # (idims, fdims, strides, pads, group)
+    ((2, 9, 11, 8), (8, 3, 3, 8), (1, 1), (1, 1, 1, 1), 2),
+    ((3, 12, 12, 16), (32, 3, 3, 16), (1, 1), (1, 1, 1, 1), 4),
+    ((2, 13, 10, 6), (4, 3, 3, 6), (2, 2), (1, 1, 1, 1), 2),     # strided: the gather form of the input gradient
+    ((2, 8, 8, 3), (6, 5, 5, 3), (1, 1), (2, 2, 2, 2), 3),      # three channels: the small-filter kernels
+])
+def test_conv2dGrad_groups(rt, oracle, case):
+    """group > 1 as kernels.h:245-319 indexes it: computed as one group over a filter with the other groups'
+    channels zeroed, the cross-group part of filterG zeroed afterwards.  Integer-valued operands: bit-exact."""
+    idims, fdims, strides, pads, group = case
+    print("case conv2dGrad groups", case, flush=True)
+    rng = np.random.default_rng(group * 100 + fdims[0])
+    k = fdims[1:3]
+    odims = pool_out_dims(idims, k, strides, pads)[:3] + (fdims[0],)
+    x = rng.integers(-2, 3, idims).astype(np.float32)
+    f = rng.integers(-2, 3, fdims).astype(np.float32)
+    og = rng.integers(-2, 3, odims).astype(np.float32)
+    want = oracle.conv2dGrad(x, f, og, k, strides, pads, group)
+    got = [t.numpy() for t in rt.conv2dGrad(*up(rt, x, f, og), k, strides, pads, group=group)]
+    for g, w, name in zip(got, want, ("inputG", "filterG", "biasG")):
+        assert_bit_exact(g, w, name)
+    # the elements of filterG that pair an output channel with another group's input channel stay zero
+    ocg, cg = fdims[0] // group, fdims[3] // group
+    cross = (np.arange(fdims[0])[:, None] // ocg) != (np.arange(fdims[3])[None, :] // cg)
+    assert not got[1].transpose(0, 3, 1, 2)[cross].any()
+    assert rt.conv2dGrad_workspace_bytes(idims, fdims, strides, pads, group) > 0
+
+
+@pytest.mark.gpu
 def test_workspace_given_by_the_caller(rt, oracle):
     rng = np.random.default_rng(8)
     idims, fdims = (2, 12, 12, 8), (8, 3, 3, 8)
@@ -274,7 +306,7 @@ def test_training_error_paths(rt):
     f = rt.empty((4, 3, 3, 4))
     og = rt.empty((1, 4, 4, 4))
     with pytest.raises(SwcHipError, match="group"):
-        rt.conv2dGrad(x, f, og, (3, 3), (1, 1), (1, 1, 1, 1), group=2)
+        rt.conv2dGrad(x, f, og, (3, 3), (1, 1), (1, 1, 1, 1), group=3)   # divides neither channel count
     with pytest.raises(SwcHipError):
         rt.conv2dGrad(x, rt.empty((4, 3, 3, 8)), og, (3, 3), (1, 1), (1, 1, 1, 1))
     assert rt.lib.swc_hip_reluGrad_f(None, None, None, 4) != 0
