@@ -308,6 +308,25 @@ int swc_hip_matrixMatrixFCBias_f(int m, int n, int k, const float *a, int lda,
                                  const float *b, int ldb, const float *bias,
                                  float *c, int ldc, int relu);
 
+/* No counterpart in the reference, whose kernels need no scratch memory at all.
+ * For callers that cannot allocate device memory or have it allocated on their
+ * behalf — code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc: swc_hip_matrixMatrixFCBias_f (same arguments, same kernels,
+ * bit-identical result) with the partial tiles of a product cut along K kept in
+ * a fixed array of SWC_HIP_NOALLOC_SCRATCH_BYTES inside the library's device
+ * code instead of the workspace.  It never calls hipMalloc/hipFree and ignores
+ * swc_hip_set_workspace.  A product whose partial tiles
+ * (swc_hip_gemm_workspace_bytes) exceed the array is refused with
+ * SWC_HIP_EINVAL before anything is launched.  All calls on one GPU share the
+ * one array (nothing in it needs to start at zero: every partial tile is
+ * written in full before it is read), so calls that overlap on one GPU — two
+ * streams, two host threads — race; calls on the library's single in-order
+ * stream do not. */
+#define SWC_HIP_NOALLOC_SCRATCH_BYTES (16u << 20)
+int swc_hip_matrixMatrixFCBias_noalloc_f(int m, int n, int k, const float *a, int lda,
+                                         const float *b, int ldb, const float *bias,
+                                         float *c, int ldc, int relu);
+
 /* MatrixMatrixFCBias followed by MatrixSoftmax (the classifier head of every
  * MLP/LeNet graph): c = softmax over each row of A*B + bias, i.e. the result of
  * matrixMatrixMul_f + batchedadd_f + matrixSoftmax_f (kernels.h:41-56, 542-552,

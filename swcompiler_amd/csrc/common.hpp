@@ -26,6 +26,9 @@ bool ready();
 int num_cus();   // of the initialised device (Device::computeUnits on a whole MI355X)
 // Scratch device memory for the current op (see runtime.hip); nullptr with the error recorded on failure.
 void *workspace(size_t bytes, const char *who);
+// Looks up, for `device` (which must be current), the address of the fixed scratch array of the entry point
+// that allocates nothing (gemm.hip); called once per device by swc_hip_init.
+int gemm_noalloc_setup(int device);
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -19,7 +19,17 @@
 using namespace swc_hip;
 using namespace swc_hip::mfma;
 
+// Scratch memory of swc_hip_matrixMatrixFCBias_noalloc_f, the one entry point that never allocates: the partial
+// tiles of a product cut along K live in this fixed array instead of the workspace.  Every GPU the library runs
+// on holds its own copy at its own address until the process ends.  In host code the array's name is only a
+// handle for hipGetSymbolAddress, never a device address: kernels are given g_scratch_ptr[device].
+static __device__ __align__(256) float scratch[SWC_HIP_NOALLOC_SCRATCH_BYTES / sizeof(float)];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+float *g_scratch_ptr[kMaxDevices] = {};   // per device: address of `scratch` there (swc_hip::gemm_noalloc_setup)
+int g_scratch_device = -1;                // the device swc_hip_init selected
 
 // Where a product cut along K keeps its partial tiles: a fixed region (the call fails if it is too small), or,
 // with ptr == nullptr, the workspace.
@@ -643,6 +653,24 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
 
 } // namespace
 
+// Once per device, with that device current (swc_hip_init calls this): the address `scratch` has there.
+int swc_hip::gemm_noalloc_setup(int device) {
+    if (device < 0 || device >= kMaxDevices)
+        return fail(SWC_HIP_EINVAL, "swc_hip_init: device %d is beyond the %d devices the library keeps scratch for", device,
+                    kMaxDevices);
+    g_scratch_device = device;
+    if (g_scratch_ptr[device]) return SWC_HIP_OK;
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+        (void)hipGetLastError();
+        return fail(SWC_HIP_ERUNTIME, "swc_hip_init: hipGetSymbolAddress(scratch) on device %d -> %s", device,
+                    hipGetErrorString(e));
+    }
+    g_scratch_ptr[device] = static_cast<float *>(p);
+    return SWC_HIP_OK;
+}
+
 extern "C" {
 
 int swc_hip_matrixMatrixMul_f(int m, int n, int k, const float *a, int lda, const float *b, int ldb, float *c,
@@ -661,6 +689,24 @@ int swc_hip_matrixMatrixFCBias_f(int m, int n, int k, const float *a, int lda, c
                                  const float *bias, float *c, int ldc, int relu) {
     SWC_REQUIRE_INIT();
     return gemm_dispatch("swc_hip_matrixMatrixFCBias_f", m, n, k, a, lda, b, ldb, bias, c, ldc, relu);
+}
+
+int swc_hip_matrixMatrixFCBias_noalloc_f(int m, int n, int k, const float *a, int lda, const float *b, int ldb,
+                                         const float *bias, float *c, int ldc, int relu) {
+    SWC_REQUIRE_INIT();
+    const char *who = "swc_hip_matrixMatrixFCBias_noalloc_f";
+    float *fixed = (g_scratch_device >= 0 && g_scratch_device < kMaxDevices) ? g_scratch_ptr[g_scratch_device] : nullptr;
+    if (!fixed) return fail(SWC_HIP_ERUNTIME, "%s: the fixed scratch array was not located at swc_hip_init", who);
+    if (m > 0 && n > 0 && k > 0) {   // refused before anything is launched
+        int splits = 0, sps = 0;
+        if (splitk_decision(m, n, k, splits, sps) && (size_t)splits * m * n * sizeof(float) > SWC_HIP_NOALLOC_SCRATCH_BYTES)
+            return fail(SWC_HIP_EINVAL, "%s: a %d x %d x %d product is cut into %d ranges of K whose partial tiles take %zu "
+                        "bytes, more than the %zu bytes of fixed scratch (SWC_HIP_NOALLOC_SCRATCH_BYTES); use "
+                        "swc_hip_matrixMatrixFCBias_f with a workspace", who, m, n, k, splits,
+                        (size_t)splits * m * n * sizeof(float), (size_t)SWC_HIP_NOALLOC_SCRATCH_BYTES);
+    }
+    return gemm_dispatch(who, m, n, k, a, lda, b, ldb, bias, c, ldc, relu, 0,
+                         PartialStore{fixed, (size_t)SWC_HIP_NOALLOC_SCRATCH_BYTES});
 }
 
 int swc_hip_matrixMatrixFCBiasSoftmax_f(int m, int n, int k, const float *a, int lda, const float *b, int ldb,

@@ -143,6 +143,7 @@ int swc_hip_init(int device) {
     if (std::strncmp(g.arch, Device::arch, std::strlen(Device::arch)) != 0)
         return fail(SWC_HIP_EUNSUPPORTED, "swc_hip_init: kernels are built for %s only, device is %s", Device::arch, g.arch);
     g.cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : Device::computeUnits;
+    if (int rc = gemm_noalloc_setup(device)) return rc;   // (the device is current here)
     SWC_HIP_TRY(hipStreamCreateWithFlags(&g.own, hipStreamNonBlocking));
     SWC_HIP_TRY(hipEventCreate(&g.t0));
     SWC_HIP_TRY(hipEventCreate(&g.t1));

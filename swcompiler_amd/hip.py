@@ -22,6 +22,7 @@ EXPORTS = [
     "swc_hip_timer_elapsed_ms", "swc_hip_event_record", "swc_hip_event_elapsed_ms", "swc_hip_graph_begin",
     "swc_hip_graph_end", "swc_hip_graph_launch", "swc_hip_graph_destroy", "swc_hip_device_cus",
     "swc_hip_enable_auto_workspace", "swc_hip_conv2dGrad_workspace_bytes", "swc_hip_matrixSoftmaxWithLoss_workspace_bytes",
+    "swc_hip_matrixMatrixFCBias_noalloc_f",
     "swc_hip_matrixMatrixMul_f", "swc_hip_batchedadd_f", "swc_hip_relu_f",
     "swc_hip_vecAdd_f", "swc_hip_conv2d_f", "swc_hip_batchnormalization_f", "swc_hip_maxpool_f",
     "swc_hip_maxpool_argmax_f", "swc_hip_avgpool_f", "swc_hip_transpose4d_f", "swc_hip_transpose2d_f",
@@ -82,6 +83,7 @@ def load_library():
         "swc_hip_enable_auto_workspace": (i32, [i32]),
         "swc_hip_conv2dGrad_workspace_bytes": (sz, [szp] * 6 + [sz]),
         "swc_hip_matrixSoftmaxWithLoss_workspace_bytes": (sz, [i32, i32]),
+        "swc_hip_matrixMatrixFCBias_noalloc_f": (i32, [i32, i32, i32, vp, i32, vp, i32, vp, vp, i32, i32]),
         "swc_hip_matrixMatrixMul_f": (i32, [i32, i32, i32, vp, i32, vp, i32, vp, i32]),
         "swc_hip_batchedadd_f": (i32, [vp, vp, vp, sz, sz]),
         "swc_hip_relu_f": (i32, [vp, vp, sz]),
@@ -353,6 +355,17 @@ class SwcHip:
         else:
             self._check(self.lib.swc_hip_matrixMatrixFCBias_f(m, n, k, a.ptr, k, w.ptr, n, bptr, out.ptr, n, int(relu)),
                         "matrixMatrixFCBias_f")
+        return out
+
+    def fcbias_noalloc(self, a, w, bias, relu=False, out=None):
+        """fcbias through the entry point that allocates nothing (fixed scratch inside the library)"""
+        m, k = a.shape
+        k2, n = w.shape
+        assert k == k2
+        out = out if out is not None else self.empty((m, n))
+        bptr = bias.ptr if bias is not None else None
+        self._check(self.lib.swc_hip_matrixMatrixFCBias_noalloc_f(m, n, k, a.ptr, k, w.ptr, n, bptr, out.ptr, n, int(relu)),
+                    "matrixMatrixFCBias_noalloc_f")
         return out
 
     def relu(self, x, out=None):
