@@ -11,6 +11,7 @@
 // from the FC GEMM.  When iC % 4 == 0 four consecutive k's lie in one tap, so
 // the gather uses 128-bit loads; otherwise (first layer, iC = 1 or 3) 32-bit.
 #include "common.hpp"
+#include "conv_strip.hpp"
 #include "mfma_dma.hpp"
 #include "mfma_dma2.hpp"
 #include "mfma_tile.hpp"
@@ -21,13 +22,6 @@ using namespace swc_hip;
 using namespace swc_hip::mfma;
 
 namespace {
-
-struct ConvGeom {
-    int N, H, W, C;      // input NHWC
-    int OH, OW, OC;      // output
-    int kh, kw, sh, sw, pt, pl;
-    int M, K;            // GEMM view
-};
 
 template <int TM, int TN, bool VEC>
 __global__ __launch_bounds__(kThreads) void conv_igemm(const float *__restrict__ in, const float *__restrict__ filt,
@@ -524,6 +518,66 @@ int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGe
     return SWC_HIP_OK;
 }
 
+// ------------------------------------------------------------ row-strip kernel (conv_strip.hpp)
+// Layers whose rows divide evenly over the compute units: whole output rows per workgroup, the input patch
+// resident in LDS, no scratch memory and no second kernel.  `min_eff`: the planner's estimate of useful matrix
+// time below which the tile kernels above, which balance by cutting tiles along K, are the better choice.
+constexpr float kStripMinEff = 0.80f;
+
+// Whether a call with these operands runs on the row-strip kernel, and its plan.  SWC_HIP_CONV (test-only, read
+// per call) = "strip" takes it wherever a plan exists; any other value rules it out.
+bool takes_strip(const ConvGeom &g, const void *input, const void *filter, const void *output, const void *residual,
+                 strip::Plan &p) {
+    const char *force = getenv("SWC_HIP_CONV");
+    if (force && strcmp(force, "strip")) return false;
+    const size_t in_bytes = (size_t)g.N * g.H * g.W * g.C * 4, filt_bytes = (size_t)g.OC * g.K * 4;
+    if (!(aligned16(input) && aligned16(filter) && aligned16(output) && aligned16(residual) && in_bytes < kMaxDmaBytes &&
+          filt_bytes < kMaxDmaBytes))
+        return false;
+    if (const char *e = getenv("SWC_HIP_STRIP_PLAN")) {   // test-only: "R,BN,WM" takes that tiling if the kernel can
+        int R = 0, BN = 0, WM = 0;
+        if (sscanf(e, "%d,%d,%d", &R, &BN, &WM) == 3 && g.C % strip::kChunk == 0 && g.OC % 16 == 0 &&
+            strip::make_plan(g, num_cus(), R, BN, WM, p))
+            return true;
+    }
+    return strip::plan(g, num_cus(), p) && (force || p.eff >= kStripMinEff);
+}
+
+template <int TMW, int TNW, int LP>
+int launch_conv_strip_as(const float *in, const float *filt, float *out, const ConvGeom &g, const strip::Plan &p,
+                         const Epilogue &ep) {
+    auto kern = strip::conv_strip<TMW, TNW, LP>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        SWC_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        strip::kMaxLds));
+        attr_set = true;
+    }
+    const unsigned in_bytes = (unsigned)((size_t)g.N * g.H * g.W * g.C * 4), filt_bytes = (unsigned)((size_t)g.OC * g.K * 4);
+    kern<<<(unsigned)(p.tiles_m * p.tiles_n), strip::kThreads, (size_t)p.lds_bytes, stream()>>>(in, filt, out, g, p, in_bytes,
+                                                                                                  filt_bytes, ep);
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
+}
+
+int launch_conv_strip(const float *in, const float *filt, float *out, const ConvGeom &g, const strip::Plan &p,
+                      const Epilogue &ep) {
+    const int key = p.TMW * 100 + p.TNW * 10 + p.LP;
+    switch (key) {
+    case 711: return launch_conv_strip_as<7, 1, 1>(in, filt, out, g, p, ep);
+    case 712: return launch_conv_strip_as<7, 1, 2>(in, filt, out, g, p, ep);
+    case 721: return launch_conv_strip_as<7, 2, 1>(in, filt, out, g, p, ep);
+    case 722: return launch_conv_strip_as<7, 2, 2>(in, filt, out, g, p, ep);
+    case 741: return launch_conv_strip_as<7, 4, 1>(in, filt, out, g, p, ep);
+    case 742: return launch_conv_strip_as<7, 4, 2>(in, filt, out, g, p, ep);
+    case 1311: return launch_conv_strip_as<13, 1, 1>(in, filt, out, g, p, ep);
+    case 1312: return launch_conv_strip_as<13, 1, 2>(in, filt, out, g, p, ep);
+    case 1321: return launch_conv_strip_as<13, 2, 1>(in, filt, out, g, p, ep);
+    case 1322: return launch_conv_strip_as<13, 2, 2>(in, filt, out, g, p, ep);
+    default: return fail(SWC_HIP_ERUNTIME, "conv (row strips): no kernel for %d x %d blocks, %d loads", p.TMW, p.TNW, p.LP);
+    }
+}
+
 // ------------------------------------------------------------ small direct conv
 // First layers (iC = 1 or 3, a handful of output channels) have K = kH*kW*iC of
 // a few dozen: far too short for the MFMA pipeline, and iC % 4 != 0 rules out
@@ -821,6 +875,9 @@ __global__ __launch_bounds__(256) void mask_filter_groups(float *dst, const floa
 // Scratch bytes the forward convolution of this geometry uses (0: none).
 size_t conv_scratch_bytes(const ConvGeom &g, const void *input, const void *filter) {
     const char *force = getenv("SWC_HIP_CONV");
+    strip::Plan sp;
+    if (takes_strip(g, input, filter, nullptr, nullptr, sp)) return 0;   // (output taken as 16-byte aligned: a call whose
+                                                                        // output is not computes every tile whole)
     if (!share_tiles() || !conv_uses_dma(g, input, filter, force)) return 0;
     return with_dma_variant(pick_dma_variant(g, force, true), [&]<int TM, int TN, int STAGES, bool MID>() {
         return conv_dma_scratch_bytes<TM, TN, STAGES, MID>(g);
@@ -952,6 +1009,12 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
             return conv_dispatch(who, output, in_p, f_p, bias, odims, p_idims, p_fdims, kernels, strides, pads, group, ep_in,
                                  bias_optional, ConvScratch{reinterpret_cast<float *>(base + in_b + f_b), need - in_b - f_b});
         }
+    }
+    // Whole rows per workgroup where the planner finds an even division ("strip" forces it wherever a plan exists,
+    // any other forced variant rules it out)
+    {
+        strip::Plan sp;
+        if (takes_strip(g, input, filter, output, ep.residual, sp)) return launch_conv_strip(input, filter, output, g, sp, ep);
     }
     if (conv_uses_dma(g, input, filter, force)) {
         // the pieces of shared tiles go into the caller's region when it gave one (and none are made if that

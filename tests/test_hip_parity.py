@@ -817,3 +817,81 @@ def test_small_direct_conv_is_bit_exact(rt, oracle, idims, fdims, strides, pads)
     dx, df, db = up(rt, x, f, b)
     assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy(), want, "direct conv")
     assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True).numpy(), oracle.relu(want), "direct conv + relu")
+
+
+# ---------------------------------------------------------------- row-strip convolution kernel
+# Layers with channel counts that are multiples of 16 whose rows divide evenly over the compute units run on
+# a kernel that gives every workgroup whole output rows (the planner decides; SWC_HIP_CONV=strip takes it
+# wherever a plan exists, so small shapes can exercise it).
+STRIP_CONV_CASES = [((2, 8, 8, 16), (16, 3, 3, 16), (1, 1), (1, 1, 1, 1)),
+                    ((3, 14, 14, 32), (32, 3, 3, 32), (1, 1), (1, 1, 1, 1)),      # 196 pixels per image: 12.25 blocks of 16
+                    ((1, 12, 10, 16), (48, 3, 3, 16), (1, 1), (0, 0, 0, 0)),      # no padding, 48 output channels
+                    ((2, 9, 9, 16), (32, 5, 5, 16), (1, 1), (2, 2, 2, 2)),        # 5 x 5 taps
+                    ((2, 13, 11, 16), (16, 3, 3, 16), (2, 2), (1, 1, 1, 1)),      # stride 2
+                    ((5, 14, 14, 64), (128, 3, 3, 64), (1, 1), (1, 1, 1, 1)),     # four channel chunks, eight column blocks
+                    ((2, 28, 28, 128), (64, 3, 3, 128), (1, 1), (1, 1, 1, 1))]
+
+
+@pytest.mark.parametrize("idims,fdims,strides,pads", STRIP_CONV_CASES)
+def test_conv_row_strips(rt, oracle, idims, fdims, strides, pads, monkeypatch):
+    print("case conv row strips", idims, fdims, strides, flush=True)
+    monkeypatch.setenv("SWC_HIP_CONV", "strip")
+    assert rt.conv2d_workspace_bytes(idims, fdims, strides, pads) == 0    # no scratch memory, no second kernel
+    rng = np.random.default_rng(sum(idims) + sum(fdims))
+    oc = fdims[0]
+    x = rng.integers(-4, 5, idims).astype(np.float32)
+    f = rng.integers(-4, 5, fdims).astype(np.float32)
+    b = rng.integers(-4, 5, oc).astype(np.float32)
+    dx, df, db = up(rt, x, f, b)
+    want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
+    assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy(), want, "integer-valued")
+    assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True).numpy(), oracle.relu(want), "+ relu")
+    res = rng.integers(-40, 41, want.shape).astype(np.float32)
+    assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads, residual=rt.upload(res), relu=True).numpy(),
+                     oracle.relu(oracle.vecAdd(want.ravel(), res.ravel()).reshape(want.shape)), "+ residual + relu")
+    # fused batchnorm + relu: the same epilogue arithmetic as the tile kernels (bit-identical to them)
+    mean, beta = (rng.integers(-4, 5, oc).astype(np.float32) for _ in range(2))
+    var = rng.uniform(0.5, 2.0, oc).astype(np.float32)
+    gamma = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    bn = up(rt, mean, var, gamma, beta)
+    fused = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, bn=bn, eps=1e-5, relu=True).numpy()
+    monkeypatch.setenv("SWC_HIP_CONV", "11_3m")
+    assert_bit_exact(fused, rt.conv2d(dx, df, db, fdims[1:3], strides, pads, bn=bn, eps=1e-5, relu=True).numpy(),
+                     "conv + bn + relu against the tile kernel")
+    monkeypatch.setenv("SWC_HIP_CONV", "strip")
+    # real-valued operands
+    xr = rng.standard_normal(idims).astype(np.float32)
+    fr = (rng.standard_normal(fdims) / np.sqrt(np.prod(fdims[1:]))).astype(np.float32)
+    br = rng.standard_normal(oc).astype(np.float32)
+    got = rt.conv2d(*up(rt, xr, fr, br), fdims[1:3], strides, pads, bn=bn, eps=1e-5, relu=True).numpy()
+    ref = oracle.relu(oracle.batchnormalization(oracle.conv2d(xr, fr, br, fdims[1:3], strides, pads), mean, var, gamma, beta, 1e-5))
+    mag = np.abs(oracle.batchnormalization(oracle.conv2d(np.abs(xr), np.abs(fr), np.abs(br), fdims[1:3], strides, pads),
+                                           -np.abs(mean), var, gamma, np.abs(beta), 1e-5))
+    assert np.max(np.abs(got - ref) / mag) < TOL
+
+
+@pytest.mark.parametrize("idims,oc", [((32, 56, 56, 64), 64), ((32, 56, 56, 64), 128), ((32, 28, 28, 128), 128)])
+def test_conv_block_layers_full_size_on_row_strips(rt, oracle, idims, oc):
+    """The convolutions of the ResNet-stage-like block at their full sizes, as the default dispatch runs them on
+    a whole MI355X (256 row-strip tiles, one per compute unit): integer-valued operands, three images through the
+    oracle bit for bit and the exact sum over the whole output."""
+    print("case conv block layer, full size", idims, oc, flush=True)
+    fdims = (oc, 3, 3, idims[3])
+    rng = np.random.default_rng(oc + idims[1])
+    x = rng.integers(-3, 4, idims).astype(np.float32)
+    f = rng.integers(-3, 4, fdims).astype(np.float32)
+    b = rng.integers(-3, 4, oc).astype(np.float32)
+    got = rt.conv2d(*up(rt, x, f, b), (3, 3), (1, 1), (1, 1, 1, 1)).numpy()
+    img = [0, 17, 31]
+    assert_bit_exact(got[img], oracle.conv2d(x[img], f, b, (3, 3), (1, 1), (1, 1, 1, 1)), "sampled images")
+    # sum over everything, exactly: each filter tap multiplies the sum of the input pixels it reaches
+    xs = x.astype(np.int64)
+    total = int(b.astype(np.int64).sum()) * idims[0] * idims[1] * idims[2]
+    fsum = f.astype(np.int64).sum(axis=0)                      # [3,3,C]
+    h, w = idims[1], idims[2]
+    for ky in range(3):
+        for kx in range(3):
+            ys = slice(max(0, ky - 1), min(h, h + ky - 1))
+            xs_ = slice(max(0, kx - 1), min(w, w + kx - 1))
+            total += int((xs[:, ys, xs_, :].sum(axis=(0, 1, 2)) * fsum[ky, kx]).sum())
+    assert int(got.astype(np.float64).sum()) == total
