@@ -520,8 +520,10 @@ int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGe
 
 // ------------------------------------------------------------ row-strip kernel (conv_strip.hpp)
 // Layers whose rows divide evenly over the compute units: whole output rows per workgroup, the input patch
-// resident in LDS, no scratch memory and no second kernel.  `min_eff`: the planner's estimate of useful matrix
-// time below which the tile kernels above, which balance by cutting tiles along K, are the better choice.
+// resident in LDS, no scratch memory and no second kernel.  Off by default (kStripDefault): on the layer shapes
+// measured so far its matrix cores are busy 77 % of the K loop and the tile kernels above, which balance by cutting
+// tiles along K, are level or ahead; SWC_HIP_CONV=strip takes it wherever the planner finds a tiling.
+constexpr bool kStripDefault = false;
 constexpr float kStripMinEff = 0.80f;
 
 // Whether a call with these operands runs on the row-strip kernel, and its plan.  SWC_HIP_CONV (test-only, read
@@ -540,13 +542,14 @@ bool takes_strip(const ConvGeom &g, const void *input, const void *filter, const
             strip::make_plan(g, num_cus(), R, BN, WM, p))
             return true;
     }
+    if (!force && !kStripDefault) return false;
     return strip::plan(g, num_cus(), p) && (force || p.eff >= kStripMinEff);
 }
 
-template <int TMW, int TNW, int LP>
+template <int TMW, int TNW>
 int launch_conv_strip_as(const float *in, const float *filt, float *out, const ConvGeom &g, const strip::Plan &p,
                          const Epilogue &ep) {
-    auto kern = strip::conv_strip<TMW, TNW, LP>;
+    auto kern = strip::conv_strip<TMW, TNW>;
     static bool attr_set = false;
     if (!attr_set) {
         SWC_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -562,19 +565,13 @@ int launch_conv_strip_as(const float *in, const float *filt, float *out, const C
 
 int launch_conv_strip(const float *in, const float *filt, float *out, const ConvGeom &g, const strip::Plan &p,
                       const Epilogue &ep) {
-    const int key = p.TMW * 100 + p.TNW * 10 + p.LP;
-    switch (key) {
-    case 711: return launch_conv_strip_as<7, 1, 1>(in, filt, out, g, p, ep);
-    case 712: return launch_conv_strip_as<7, 1, 2>(in, filt, out, g, p, ep);
-    case 721: return launch_conv_strip_as<7, 2, 1>(in, filt, out, g, p, ep);
-    case 722: return launch_conv_strip_as<7, 2, 2>(in, filt, out, g, p, ep);
-    case 741: return launch_conv_strip_as<7, 4, 1>(in, filt, out, g, p, ep);
-    case 742: return launch_conv_strip_as<7, 4, 2>(in, filt, out, g, p, ep);
-    case 1311: return launch_conv_strip_as<13, 1, 1>(in, filt, out, g, p, ep);
-    case 1312: return launch_conv_strip_as<13, 1, 2>(in, filt, out, g, p, ep);
-    case 1321: return launch_conv_strip_as<13, 2, 1>(in, filt, out, g, p, ep);
-    case 1322: return launch_conv_strip_as<13, 2, 2>(in, filt, out, g, p, ep);
-    default: return fail(SWC_HIP_ERUNTIME, "conv (row strips): no kernel for %d x %d blocks, %d loads", p.TMW, p.TNW, p.LP);
+    switch (p.TMW * 10 + p.TNW) {
+    case 71: return launch_conv_strip_as<7, 1>(in, filt, out, g, p, ep);
+    case 72: return launch_conv_strip_as<7, 2>(in, filt, out, g, p, ep);
+    case 74: return launch_conv_strip_as<7, 4>(in, filt, out, g, p, ep);
+    case 131: return launch_conv_strip_as<13, 1>(in, filt, out, g, p, ep);
+    case 132: return launch_conv_strip_as<13, 2>(in, filt, out, g, p, ep);
+    default: return fail(SWC_HIP_ERUNTIME, "conv (row strips): no kernel for %d x %d blocks", p.TMW, p.TNW);
     }
 }
 

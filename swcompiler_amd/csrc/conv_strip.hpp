@@ -2,19 +2,14 @@
 // layout, swizzles and the lane -> address maps are in conv_strip_index.hpp
 // (shared with the host-side emulation that checks them).
 //
-// Ring discipline.  A "slice" is one tap of one 16-channel chunk: 16 k.  Every
-// wavefront issues exactly LP + 1 direct-to-LDS loads per slice — LP blocks of
-// the NEXT chunk's patch (into the other patch buffer) and its block of the
-// filter slice kDepth slices ahead (into the stage read one slice ago) — a load
-// that has nothing to carry is issued all the same with an out-of-range offset,
-// into a per-wavefront dump block, so that the pending-load counter advances
-// identically in every slice.  Loads land in order, hence at the top of slice s
-//     s_waitcnt vmcnt((kDepth-1) * (LP+1));  s_barrier
-// certifies, for the wavefront and then for the workgroup, that everything
-// issued up to slice s - kDepth is in LDS — the filter slice s, and, at a chunk
-// boundary, the whole patch of the new chunk (the planner makes sure its last
-// real block is issued kDepth slices before the chunk ends) — and that nobody
-// still reads the stage and the patch buffer that this slice's loads overwrite.
+// Synchronisation.  K is walked chunk by chunk (16 channels x all taps).  At
+// the top of chunk c every wavefront waits for its own outstanding loads
+// (s_waitcnt vmcnt(0)) and the workgroup meets at a barrier: the patch and the
+// filter part of chunk c, requested one chunk earlier, are then in LDS for
+// everyone, and nobody reads the other pair of buffers any more — into which
+// the wavefronts at once request chunk c + 1, which has the whole of chunk c's
+// MFMAs (tens of thousands of cycles) to arrive.  Between barriers the
+// wavefronts run free.
 #pragma once
 #include "conv_strip_index.hpp"
 #include "mfma_dma.hpp"
@@ -44,7 +39,7 @@ __device__ __forceinline__ void settle(v4f (&acc)[TMW][TNW]) {
 #endif
 }
 
-template <int TMW, int TNW, int LP>
+template <int TMW, int TNW>
 __global__ __launch_bounds__(kThreads) void conv_strip(const float *__restrict__ in, const float *__restrict__ filt,
                                                        float *__restrict__ out, ConvGeom g, Plan p, unsigned in_bytes,
                                                        unsigned filt_bytes, mfma::Epilogue ep) {
@@ -64,29 +59,32 @@ __global__ __launch_bounds__(kThreads) void conv_strip(const float *__restrict__
     int px0[TMW];      // patch pixel under tap (0,0) of this lane's pixel in each of its blocks
 #pragma unroll
     for (int m = 0; m < TMW; ++m) px0[m] = lane_patch_px0(g, p, wb.blk0 + (m < wb.cnt ? m : 0), j);
-    int fbyte[TNW];    // byte offset of this lane's filter fragment inside a stage
+    int fbyte[TNW];    // byte offset of this lane's filter fragment inside tap 0 of a filter buffer
 #pragma unroll
     for (int n = 0; n < TNW; ++n) fbyte[n] = lane_filter_byte(wb.cb0 + n, j, q);
-    const int f_lane = filter_lane_byte(g, p, t, wave, lane);   // this wavefront's block of a filter slice
 
     char *const lds_b = reinterpret_cast<char *>(lds);
-    float *const dump = lds + lds_dump(p, wave);
 
-    // patch block `i` (of PW per wavefront) of channel chunk `chunk` into patch buffer `buf`; a block beyond PW
-    // or a chunk beyond the last goes to the dump block as an empty load
-    auto load_patch = [&](int i, int chunk, int buf) {
-        const bool real = i < p.PW && chunk < p.chunks;   // wavefront-uniform
-        const int blk = i * kWaves + wave;
-        const int v = real ? patch_lane_byte(g, p, t, blk, lane) : kNoByte;
-        float *dst = real ? lds + lds_patch(p, buf) + blk * kLoadFloats : dump;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, (lds_void_t *)dst, 16, v, chunk * kPxBytes, 0, 0);
-    };
-    // this wavefront's block of filter slice (tap, chunk) into ring stage `stage`
-    auto load_filter = [&](int tap, int chunk, int stage, bool exists) {
-        const bool real = exists && wave * kLoadPx < p.BN;
-        float *dst = real ? lds + lds_bstage(p, stage) + wave * kLoadFloats : dump;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_f, (lds_void_t *)dst, 16, real ? f_lane : kNoByte,
-                                                 (tap * g.C + chunk * kChunk) * 4, 0, 0);
+    // This wavefront's share of a chunk's loads: block i*8 + wave of the patch (i < PW) and of the filter part
+    // (i < FW).  The per-lane byte offsets do not depend on the chunk (a chunk adds 64 bytes as a scalar), so they
+    // are formed once; what is left per chunk is the load instructions themselves.
+    int pbyte[kMaxPW], fbyte_g[kMaxFW];
+#pragma unroll
+    for (int i = 0; i < kMaxPW; ++i) pbyte[i] = i < p.PW ? patch_lane_byte(g, p, t, i * kWaves + wave, lane) : kNoByte;
+#pragma unroll
+    for (int i = 0; i < kMaxFW; ++i) fbyte_g[i] = i < p.FW ? filter_lane_byte(g, p, t, i * kWaves + wave, lane) : kNoByte;
+    auto request_chunk = [&](int chunk, int buf) {
+        float *pdst = lds + lds_patch(p, buf) + wave * kLoadFloats, *fdst = lds + lds_filter(p, buf) + wave * kLoadFloats;
+#pragma unroll
+        for (int i = 0; i < kMaxPW; ++i)
+            if (i < p.PW)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, (lds_void_t *)(pdst + i * kWaves * kLoadFloats), 16, pbyte[i],
+                                                         chunk * kPxBytes, 0, 0);
+#pragma unroll
+        for (int i = 0; i < kMaxFW; ++i)
+            if (i < p.FW)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_f, (lds_void_t *)(fdst + i * kWaves * kLoadFloats), 16, fbyte_g[i],
+                                                         chunk * kPxBytes, 0, 0);
     };
 
     v4f acc[TMW][TNW];
@@ -95,60 +93,59 @@ __global__ __launch_bounds__(kThreads) void conv_strip(const float *__restrict__
 #pragma unroll
         for (int n = 0; n < TNW; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    // ---- prologue: the whole patch of chunk 0, then the loads of the kDepth slices "before" slice 0
-    for (int i = 0; i < p.PW; ++i) load_patch(i, 0, 0);
-    // (tap, chunk) of the filter slice to request next; slices run tap-fastest within a chunk
-    int ld_tap = 0, ld_chunk = 0, ld_stage = 0;
-    auto next_filter = [&]() {
-        load_filter(ld_tap, ld_chunk, ld_stage, ld_chunk < p.chunks);
-        if (++ld_tap == p.taps) ld_tap = 0, ++ld_chunk;
-        ld_stage = ld_stage + 1 == kBStages ? 0 : ld_stage + 1;
+    // Fragments of one tap: TNW of the filter, TMW of the pixels.  Those of tap t + 1 are read while tap t is
+    // multiplied — one read behind each block's MFMAs, pinned there by scheduling fences — so an LDS read has a
+    // whole tap (hundreds of MFMA cycles) to return; only the first tap after a barrier waits for its reads.
+    struct Frags {
+        v4f a[TNW], b[TMW];
     };
+    auto read_a = [&](Frags &f, const char *tap_b) {
 #pragma unroll
-    for (int d = 0; d < kDepth; ++d) {
-#pragma unroll
-        for (int l = 0; l < LP; ++l) load_patch(p.PW, 0, 0);   // empty: keeps the count per slice
-        next_filter();
-    }
+        for (int n = 0; n < TNW; ++n) f.a[n] = *reinterpret_cast<const v4f *>(tap_b + fbyte[n]);
+    };
+    auto read_b = [&](Frags &f, const char *patch_b, int tap_px, int m) {
+        const int pp = px0[m] + tap_px;
+        f.b[m] = *reinterpret_cast<const v4f *>(patch_b + swz_byte(pp, q));
+    };
+    const int taps = p.taps;
 
-    int rd_stage = 0;
+    request_chunk(0, 0);
     for (int chunk = 0; chunk < p.chunks; ++chunk) {
+        mfma::ring_sync<0>();   // chunk `chunk` is in LDS for everyone; the other buffer pair is free
+        if (chunk + 1 < p.chunks) request_chunk(chunk + 1, (chunk + 1) & 1);
         const char *patch_b = lds_b + lds_patch(p, chunk & 1) * 4;
-        int tap = 0;
-        for (int ky = 0; ky < g.kh; ++ky)
-            for (int kx = 0; kx < g.kw; ++kx, ++tap) {
-                mfma::ring_sync<(kDepth - 1) * (LP + 1)>();
-                // this slice's loads: LP blocks of the next chunk's patch, one block of the filter slice kDepth ahead
+        const char *tap_b = lds_b + lds_filter(p, chunk & 1) * 4;
+        Frags cur, nxt;
+        read_a(cur, tap_b);
 #pragma unroll
-                for (int l = 0; l < LP; ++l) load_patch(tap * LP + l, chunk + 1, (chunk + 1) & 1);
-                next_filter();
-
-                const char *stage_b = lds_b + lds_bstage(p, rd_stage) * 4;
-                v4f fa[TNW];   // filter fragments: four consecutive channels of this lane's output channel
-#pragma unroll
-                for (int n = 0; n < TNW; ++n) fa[n] = *reinterpret_cast<const v4f *>(stage_b + fbyte[n]);
-                const int tap_px = ky * p.Wp + kx;
-                auto pixel_frag = [&](int m) {
-                    const int pp = px0[m] + tap_px;
-                    return *reinterpret_cast<const v4f *>(patch_b + swz_byte(pp, q));
-                };
-                v4f fb = pixel_frag(0);
-#pragma unroll
-                for (int m = 0; m < TMW; ++m) {
-                    v4f fb_next = fb;
-                    if (m + 1 < TMW) fb_next = pixel_frag(m + 1);   // in flight behind this block's MFMAs
-                    if (m < wb.cnt) {
-#pragma unroll
-                        for (int s = 0; s < 4; ++s)
-#pragma unroll
-                            for (int n = 0; n < TNW; ++n) mfma16(acc[m][n], fa[n][s], fb[s]);
-                    }
-                    fb = fb_next;
-                }
-                rd_stage = rd_stage + 1 == kBStages ? 0 : rd_stage + 1;
+        for (int m = 0; m < TMW; ++m) read_b(cur, patch_b, 0, m);
+        int ky = 0, kx = 0;   // of the tap being multiplied
+        for (int tap = 0; tap < taps; ++tap) {
+            // the next tap's coordinates (the last tap of a chunk re-reads itself: harmless, never used)
+            int nky = ky, nkx = kx;
+            const bool more = tap + 1 < taps;
+            if (more) {
+                if (++nkx == g.kw) nkx = 0, ++nky;
+                tap_b += p.BN * kPxBytes;
             }
+            const int next_px = nky * p.Wp + nkx;
+            read_a(nxt, tap_b);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int m = 0; m < TMW; ++m) {
+                read_b(nxt, patch_b, next_px, m);
+                if (m < wb.cnt) {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+#pragma unroll
+                        for (int n = 0; n < TNW; ++n) mfma16(acc[m][n], cur.a[n][s], cur.b[m][s]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            cur = nxt;
+            ky = nky, kx = nkx;
+        }
     }
-    mfma::wait_vmcnt<0>();   // the trailing empty loads still target this workgroup's LDS
     settle<TMW, TNW>(acc);
 
     // ---- epilogue: lane (j, q) holds output channels 4q .. 4q+3 of pixel j of each of its blocks

@@ -10,8 +10,12 @@
 // 16 channels = 64 bytes each, zeros where the image ends — stay in LDS for all
 // kh*kw taps, so the input crosses from L2 into LDS once per chunk instead of
 // once per tap, and no address arithmetic is left in the tap loop: a tap is a
-// scalar offset into the patch.  The filter streams through a small ring, one
-// slice (BN x 16 floats) per tap.
+// scalar offset into the patch.  The filter's part for the chunk (kh*kw slices
+// of BN x 16 floats) sits beside it.  Both are double-buffered: the workgroup
+// meets at a barrier once per CHUNK — a barrier per tap left the matrix cores
+// of all four SIMDs idle together at every tap boundary (measured: 1300-2200
+// cycles per 3300-6400 cycles of MFMA work) — and between barriers its
+// wavefronts run free, so the two wavefronts of a SIMD fill each other's waits.
 //
 // Matrix blocks are 16 x 16 (v_mfma_f32_16x16x4_f32, the same flop rate as the
 // 32 x 32 x 2 form): with blocks of 16 pixels a tile of 392 pixels is 24.5
@@ -50,9 +54,9 @@ constexpr int kPxFloats = kChunk;          // floats per patch pixel
 constexpr int kPxBytes = kChunk * 4;       // 64
 constexpr int kLoadFloats = 256;           // one wavefront load: 64 lanes x 16 bytes
 constexpr int kLoadPx = kLoadFloats / kPxFloats;   // 16 patch pixels (or filter rows) per load
-constexpr int kDepth = 3;                  // filter slices in flight ahead of the one being multiplied
-constexpr int kBStages = kDepth + 1;
 constexpr int kMaxLds = 160 * 1024;
+constexpr int kMaxPW = 8;                  // patch loads per wavefront per chunk the kernel keeps offsets for
+constexpr int kMaxFW = 10;                 // the same for the filter part
 
 // How one layer is cut into tiles; filled by plan() on the host, read by the kernel.
 struct Plan {
@@ -60,14 +64,14 @@ struct Plan {
     int BN;           // output channels per tile (multiple of 16, divides OC)
     int WM, WN;       // wavefront grid: WM x WN = 8, rows split the pixel blocks, columns the channel blocks
     int TMW, TNW;     // pixel / channel blocks per wavefront (the kernel's template arguments)
-    int LP;           // patch loads per wavefront per slice (template argument)
     int P;            // R * OW
     int nblk;         // ceil(P / 16)
     int Rp, Wp;       // patch rows, columns: (R-1)*sh + kh, (OW-1)*sw + kw
     int patch_px;     // Rp * Wp
     int PW;           // patch loads per wavefront per chunk: ceil(ceil(patch_px / 16) / 8)
     int patch_floats; // floats of one patch buffer: PW * 8 * 256
-    int b_floats;     // floats of one filter stage: BN * 16
+    int FW;           // filter loads per wavefront per chunk: ceil(taps * BN / 16 / 8)
+    int b_floats;     // floats of one filter buffer: taps * BN * 16 (rounded up to whole rounds of loads)
     int tiles_m, tiles_n, strips_per_img;
     int taps, chunks, slices;
     float inv_wp;     // 1.0f / Wp
@@ -75,11 +79,10 @@ struct Plan {
     float eff;        // estimated share of the matrix cores' time that is useful work
 };
 
-// LDS layout in floats: patch[2], filter stages, then a dump block per wavefront for loads that carry nothing.
+// LDS layout in floats: patch[2], then filter[2]; a filter buffer is [tap][BN rows][16 floats].
 SWC_HD int lds_patch(const Plan &p, int buf) { return buf * p.patch_floats; }
-SWC_HD int lds_bstage(const Plan &p, int stage) { return 2 * p.patch_floats + stage * p.b_floats; }
-SWC_HD int lds_dump(const Plan &p, int wave) { return 2 * p.patch_floats + kBStages * p.b_floats + wave * kLoadFloats; }
-SWC_HD int lds_total_floats(const Plan &p) { return 2 * p.patch_floats + kBStages * p.b_floats + kWaves * kLoadFloats; }
+SWC_HD int lds_filter(const Plan &p, int buf) { return 2 * p.patch_floats + buf * p.b_floats; }
+SWC_HD int lds_total_floats(const Plan &p) { return 2 * p.patch_floats + 2 * p.b_floats; }
 
 // Swizzle: a row of 64 bytes (a patch pixel or a filter row of one slice) holds four 16-byte chunks; logical
 // chunk c of row r is stored at position c ^ key(r).  Sixteen lanes that read the same logical chunk of sixteen
@@ -130,7 +133,8 @@ SWC_HD int lane_patch_px0(const ConvGeom &g, const Plan &p, int blk, int j) {
     return r * g.sh * p.Wp + c * g.sw;
 }
 
-// ---- filter fragments (A operand): byte offset inside a filter stage of the lane's four channels
+// ---- filter fragments (A operand): byte offset inside tap 0 of a filter buffer of the lane's four channels (a
+// tap adds BN * 64 bytes; BN is a multiple of 16, so the swizzle key of a row does not depend on the tap)
 SWC_HD int lane_filter_byte(int cb, int j, int q) { return swz_byte(cb * 16 + j, q); }
 
 // ---- global -> LDS loads.  One wavefront load fills 1 KiB: lane l lands at byte 16*l of the block, i.e. row
@@ -148,13 +152,15 @@ SWC_HD int patch_lane_byte(const ConvGeom &g, const Plan &p, const TileOrigin &t
     return ok ? (((t.img * g.H + iy) * g.W + ix) * g.C + chunk * 4) * 4 : kNoByte;
 }
 
-// filter load of wavefront `wave` (filter rows 16*wave .. of the tile's BN): byte offset of the lane's 16 bytes
-// in the filter for tap 0, chunk 0 (a slice adds (tap*C + 16*chunk)*4 bytes as a scalar), or kNoByte
-SWC_HD int filter_lane_byte(const ConvGeom &g, const Plan &p, const TileOrigin &t, int wave, int lane) {
-    const int r = wave * kLoadPx + (lane >> 2);
+// filter load `blk` (sixteen rows 16*blk .. of the buffer's taps*BN rows; row = tap*BN + output channel): byte
+// offset of the lane's 16 bytes in the filter for channel chunk 0 (a later chunk adds 64 bytes per chunk as a
+// scalar), or kNoByte past the last tap
+SWC_HD int filter_lane_byte(const ConvGeom &g, const Plan &p, const TileOrigin &t, int blk, int lane) {
+    const int nb = p.BN / kLoadPx;                   // loads per tap
+    const int tap = blk / nb, r = (blk - tap * nb) * kLoadPx + (lane >> 2);
     const int chunk = (lane & 3) ^ swz_key(r);
-    const bool ok = r < p.BN && t.n0 + r < g.OC;
-    return ok ? ((t.n0 + r) * g.K + chunk * 4) * 4 : kNoByte;
+    const bool ok = tap < p.taps && t.n0 + r < g.OC;
+    return ok ? ((t.n0 + r) * g.K + tap * g.C + chunk * 4) * 4 : kNoByte;
 }
 
 // ---- host side: the plan
@@ -178,18 +184,14 @@ inline bool make_plan(const ConvGeom &g, int cus, int R, int BN, int WM, Plan &p
     if (p.patch_px >= (1 << 20)) return false;
     p.PW = ceil_div_i(ceil_div_i(p.patch_px, kLoadPx), kWaves);
     p.taps = g.kh * g.kw, p.chunks = g.C / kChunk, p.slices = p.taps * p.chunks;
-    // the patch of the next chunk must be on its way kDepth slices before the chunk ends
-    const int slots = p.taps - kDepth + 1;
-    if (slots < 1) return false;
-    p.LP = ceil_div_i(p.PW, slots);
-    if (p.LP > 2) return false;
     p.patch_floats = p.PW * kWaves * kLoadFloats;
-    p.b_floats = BN * kChunk;
+    p.FW = ceil_div_i(p.taps * BN / kLoadPx, kWaves);
+    p.b_floats = p.FW * kWaves * kLoadFloats;
     p.strips_per_img = g.OH / R;
     p.tiles_m = g.N * p.strips_per_img, p.tiles_n = g.OC / BN;
     p.inv_wp = 1.0f / (float)p.Wp;
     p.lds_bytes = lds_total_floats(p) * 4;
-    if (p.lds_bytes > kMaxLds) return false;
+    if (p.lds_bytes > kMaxLds || p.PW > kMaxPW || p.FW > kMaxFW) return false;
     // estimate: blocks on the busiest SIMD (wavefronts w and w + 4 share one) against the tile's average, times
     // how evenly the tiles fill the compute units
     int simd[4] = {0, 0, 0, 0};
@@ -198,14 +200,17 @@ inline bool make_plan(const ConvGeom &g, int cus, int R, int BN, int WM, Plan &p
     for (int s = 0; s < 4; ++s) crit = simd[s] > crit ? simd[s] : crit;
     const long tiles = (long)p.tiles_m * p.tiles_n;
     const long rounds = (tiles + cus - 1) / cus;
-    const double useful = (double)p.P / 16.0 * cblk / 4.0;
-    p.eff = (float)(useful / crit * (double)tiles / (double)(rounds * cus));
+    // in matrix-core cycles per SIMD: a block pair costs four MFMAs of 32 cycles per slice; a tile also pays for
+    // its first chunk's loads, its stores and its launch slot before and after (about 8000 cycles, measured)
+    const double per_block = 128.0 * p.slices, fixed = 8000.0;
+    const double useful = (double)p.P / 16.0 * cblk / 4.0 * per_block;
+    p.eff = (float)(useful * (double)tiles / ((double)rounds * cus * (crit * per_block + fixed)));
     return true;
 }
 
 // The best plan for the layer on `cus` compute units; false if the kernel does not apply.
 inline bool plan(const ConvGeom &g, int cus, Plan &best) {
-    if (g.C % kChunk || g.OC % 16 || g.M <= 0 || g.kh * g.kw < kDepth) return false;
+    if (g.C % kChunk || g.OC % 16 || g.M <= 0) return false;
     bool found = false;
     for (int R = 1; R <= g.OH; ++R) {
         if (g.OH % R) continue;
@@ -213,11 +218,14 @@ inline bool plan(const ConvGeom &g, int cus, Plan &best) {
             for (int WM = 1; WM <= kWaves; WM *= 2) {
                 Plan p;
                 if (!make_plan(g, cus, R, BN, WM, p)) continue;
-                // more useful matrix time first; on a tie (within 1 %) the plan with fewer LDS reads per MFMA:
-                // more channel blocks per wavefront, then more pixel blocks
-                const bool better = !found || p.eff > best.eff * 1.01f ||
-                                    (p.eff > best.eff * 0.99f &&
-                                     (p.TNW > best.TNW || (p.TNW == best.TNW && p.nblk > best.nblk)));
+                // A wavefront with one channel block reads a pixel fragment per four MFMAs, all four into the same
+                // accumulator; with two or four it reads one per eight or sixteen.  Plans of at least two channel
+                // blocks per wavefront come first unless they waste a tenth more of the matrix time; among equals
+                // (within 1 %) the wider tile, whose input patch is fetched by fewer workgroups.
+                const float score = p.eff * (p.TNW == 1 ? 0.9f : 1.0f);
+                const float best_score = found ? best.eff * (best.TNW == 1 ? 0.9f : 1.0f) : 0.f;
+                const bool better = !found || score > best_score * 1.01f ||
+                                    (score > best_score * 0.99f && (p.BN > best.BN || (p.BN == best.BN && p.TNW > best.TNW)));
                 if (better) best = p, found = true;
             }
         }

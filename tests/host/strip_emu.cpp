@@ -30,14 +30,14 @@ void dma_lane(std::vector<float> &lds, int dst_float, int lane, const float *bas
 
 extern "C" {
 
-// Fills `plan_out` (R, BN, WM, WN, TMW, TNW, LP, PW, lds_bytes, tiles, eff*1000) and returns 1 if the kernel
+// Fills `plan_out` (R, BN, WM, WN, TMW, TNW, FW, PW, lds_bytes, tiles, eff*1000) and returns 1 if the kernel
 // applies to the layer on `cus` compute units, else 0.
 int strip_emu_plan(const int *geom, int cus, int *plan_out) {
     ConvGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9], geom[10],
                geom[11], geom[12], geom[0] * geom[4] * geom[5], geom[7] * geom[8] * geom[3]};
     Plan p;
     if (!plan(g, cus, p)) return 0;
-    const int v[11] = {p.R, p.BN, p.WM, p.WN, p.TMW, p.TNW, p.LP, p.PW, p.lds_bytes, p.tiles_m * p.tiles_n, (int)(p.eff * 1000)};
+    const int v[11] = {p.R, p.BN, p.WM, p.WN, p.TMW, p.TNW, p.FW, p.PW, p.lds_bytes, p.tiles_m * p.tiles_n, (int)(p.eff * 1000)};
     std::memcpy(plan_out, v, sizeof(v));
     return 1;
 }
@@ -63,10 +63,9 @@ int strip_emu_conv(const float *in, const float *filt, const float *bias, float 
         auto A = [&](int w, int m, int n, int lane, int v) -> float & {
             return acc[((((size_t)w * p.TMW + m) * p.TNW + n) * 64 + lane) * 4 + v];
         };
-        int stage = 0;
         for (int chunk = 0; chunk < p.chunks; ++chunk) {
-            // the chunk's patch: PW loads per wavefront
-            for (int w = 0; w < kWaves; ++w)
+            // the chunk's patch and filter part: PW and FW loads per wavefront
+            for (int w = 0; w < kWaves; ++w) {
                 for (int i = 0; i < p.PW; ++i) {
                     const int blk = i * kWaves + w;
                     for (int lane = 0; lane < 64; ++lane) {
@@ -75,20 +74,20 @@ int strip_emu_conv(const float *in, const float *filt, const float *bias, float 
                                  v == kNoByte ? -1 : (long)v + chunk * kPxBytes);
                     }
                 }
+                for (int i = 0; i < p.FW; ++i) {
+                    const int blk = i * kWaves + w;
+                    for (int lane = 0; lane < 64; ++lane) {
+                        const int v = filter_lane_byte(g, p, t, blk, lane);
+                        dma_lane(lds, lds_filter(p, chunk & 1) + blk * kLoadFloats, lane, filt, filt_bytes,
+                                 v == kNoByte ? -1 : (long)v + chunk * kPxBytes);
+                    }
+                }
+            }
             int tap = 0;
             for (int ky = 0; ky < g.kh; ++ky)
                 for (int kx = 0; kx < g.kw; ++kx, ++tap) {
-                    // the filter slice into ring stage `stage`
-                    for (int w = 0; w < kWaves; ++w) {
-                        if (w * kLoadPx >= p.BN) continue;
-                        for (int lane = 0; lane < 64; ++lane) {
-                            const int v = filter_lane_byte(g, p, t, w, lane);
-                            dma_lane(lds, lds_bstage(p, stage) + w * kLoadFloats, lane, filt, filt_bytes,
-                                     v == kNoByte ? -1 : (long)v + (long)(tap * g.C + chunk * kChunk) * 4);
-                        }
-                    }
                     const char *lds_b = reinterpret_cast<const char *>(lds.data());
-                    const char *stage_b = lds_b + (size_t)lds_bstage(p, stage) * 4;
+                    const char *stage_b = lds_b + (size_t)lds_filter(p, chunk & 1) * 4 + (size_t)tap * p.BN * kPxBytes;
                     const char *patch_b = lds_b + (size_t)lds_patch(p, chunk & 1) * 4;
                     const int tap_px = ky * p.Wp + kx;
                     for (int w = 0; w < kWaves; ++w) {
@@ -114,7 +113,6 @@ int strip_emu_conv(const float *in, const float *filt, const float *bias, float 
                                         }
                             }
                     }
-                    stage = stage + 1 == kBStages ? 0 : stage + 1;
                 }
         }
         // epilogue: lane (j, q) holds output channels 4q .. 4q+3 of pixel j of each of its blocks

@@ -871,11 +871,14 @@ def test_conv_row_strips(rt, oracle, idims, fdims, strides, pads, monkeypatch):
 
 
 @pytest.mark.parametrize("idims,oc", [((32, 56, 56, 64), 64), ((32, 56, 56, 64), 128), ((32, 28, 28, 128), 128)])
-def test_conv_block_layers_full_size_on_row_strips(rt, oracle, idims, oc):
-    """The convolutions of the ResNet-stage-like block at their full sizes, as the default dispatch runs them on
-    a whole MI355X (256 row-strip tiles, one per compute unit): integer-valued operands, three images through the
-    oracle bit for bit and the exact sum over the whole output."""
-    print("case conv block layer, full size", idims, oc, flush=True)
+@pytest.mark.parametrize("variant", [None, "strip"])
+def test_conv_block_layers_full_size(rt, oracle, idims, oc, variant, monkeypatch):
+    """The convolutions of the ResNet-stage-like block at their full sizes, as the default dispatch runs them and
+    on the row-strip kernel (a whole number of tiles per compute unit on a whole MI355X): integer-valued operands,
+    three images through the oracle bit for bit and the exact sum over the whole output."""
+    print("case conv block layer, full size", idims, oc, variant, flush=True)
+    if variant:
+        monkeypatch.setenv("SWC_HIP_CONV", variant)
     fdims = (oc, 3, 3, idims[3])
     rng = np.random.default_rng(oc + idims[1])
     x = rng.integers(-3, 4, idims).astype(np.float32)
