@@ -25,7 +25,12 @@ Also in the line:
                 TFLOP/s or GB/s with the fraction of the MI355X peak)
                 plus `training_kernels`: conv2dGrad, reluGrad, sgd, maxpoolGrad at those sizes
   cpu_baseline  the reference's own CPU kernels (oracle/_ref, g++ -std=c++11 -O2,
-                one thread) on the first rows of the same batch
+                one thread) on the first rows of the same batch; every other configuration
+                carries its own under configs.cfgN.cpu_baseline (whole batch, same buffers)
+
+Ops never allocate: the harness sizes one scratch buffer with the library's
+swc_hip_*_workspace_bytes queries over every shape it runs and hands it over
+with swc_hip_set_workspace, as a generated program does.
 
 The CPU checker is used only for the cpu_baseline leg.
 """
@@ -303,22 +308,58 @@ def run_bn_pool_separately(rt, graphs, iters=20):
     return rows
 
 
-def cpu_baseline(graphs, rows=64):
-    """The reference's CPU kernels on the first `rows` rows of the headline batch."""
+def cpu_baselines(graphs, rows=64):
+    """The reference's CPU kernels (the unfused call sequence its generator emits, one thread, g++ -std=c++11 -O2,
+    src/codegen/MakefileBuilder.h:34) on the buffers of every configuration: the whole batch, three timed
+    iterations, for the MLP, LeNet and the bandwidth chain; one iteration for the conv block (about 10 s); the
+    first `rows` rows of the wide MLP's batch, whose whole batch would take about 11 minutes."""
     from oracle import binding
     if binding.ref_available():
         be, kind = binding.load_ref(), "reference"
     else:
         be, kind = binding.load_oracle(), "port"
-    t = graphs.make_inputs(2)
-    t["x"] = np.ascontiguousarray(t["x"][:rows])
-    t0 = time.perf_counter()
-    graphs.run(2, be, t, fused=False)
-    dt = time.perf_counter() - t0
-    return dict(value=rows / dt, unit="samples/s", cores=1, kind=kind, seconds=dt,
-                sample=f"first {rows} of the 4096 rows of the same batch through the whole graph "
-                       f"(matrixMatrixMul_f, batchedadd_f, relu_f, matrixSoftmax_f as the reference emits them), "
-                       f"one thread, g++ -std=c++11 -O2; {os.cpu_count()} host cpus visible")
+    out = {}
+    for cfg, iters in ((1, 3), (2, 1), (3, 3), (4, 1), (5, 3)):
+        t = graphs.make_inputs(cfg)
+        batch = graphs.batch_of(cfg, t)
+        sample = f"the whole batch of {batch}, {iters} timed iteration{'s' if iters > 1 else ''}"
+        if cfg == 2:
+            t["x"] = np.ascontiguousarray(t["x"][:rows])
+            sample = f"first {rows} of the {batch} rows of the same batch, one iteration"
+            batch = rows
+        times = []
+        for _ in range(iters):
+            t0 = time.perf_counter()
+            graphs.run(cfg, be, t, fused=False)
+            times.append(time.perf_counter() - t0)
+        dt = min(times)
+        out[f"cfg{cfg}"] = dict(value=batch / dt, unit="samples/s", cores=1, kind=kind, seconds=dt,
+                                seconds_all=times,
+                                sample=sample + "; the whole graph as the reference emits it (one kernels.h call per "
+                                       f"op node), one thread, g++ -std=c++11 -O2; {os.cpu_count()} host cpus visible")
+    return out
+
+
+def bench_workspace(rt, graphs):
+    """One scratch buffer for every op this harness runs: the maximum of the library's size queries over the FC
+    and convolution shapes of the five configurations and the training-kernel leg."""
+    need = 0
+    for m, n, k in ((8, 512, 784), (8, 10, 512), (4096, 4096, 784), (4096, 4096, 4096), (4096, 10, 4096),
+                    (256, 500, 800), (256, 10, 500)):
+        need = max(need, rt.gemm_workspace_bytes(m, n, k))
+    p1 = (1, 1, 1, 1)
+    convs = [((256, 28, 28, 1), (20, 5, 5, 1), (0,) * 4), ((256, 12, 12, 20), (50, 5, 5, 20), (0,) * 4),
+             ((32, 56, 56, 64), (64, 3, 3, 64), p1), ((32, 56, 56, 64), (128, 3, 3, 64), p1),
+             ((32, 28, 28, 128), (128, 3, 3, 128), p1)]
+    for xs, fs, pads in convs:
+        need = max(need, rt.conv2d_workspace_bytes(xs, fs, (1, 1), pads))
+    for xs, fs, pads in convs[2:]:
+        need = max(need, rt.conv2dGrad_workspace_bytes(xs, fs, (1, 1), pads))
+    if not need:
+        return None
+    ws = rt.empty((need // 4 + 64,))
+    rt.set_workspace(ws)
+    return ws
 
 
 def main():
@@ -337,8 +378,9 @@ def main():
         sys.exit("bench.py: this build runs on one GPU only (nothing is sharded); use --gpus 1")
 
     from swcompiler_amd import graphs
-    from swcompiler_amd.hip import runtime
-    rt = runtime()
+    from swcompiler_amd.hip import SwcHip
+    rt = SwcHip(0, auto_workspace=False)   # ops fail rather than allocate: the buffer below must cover them all
+    workspace = bench_workspace(rt, graphs)
 
     if args.calibrate:
         x = rt.upload(np.ones(1 << 26, np.float32))
@@ -354,10 +396,21 @@ def main():
     flop = sum(r["flop"] for r in gemm)
     secs = sum(r["ms"] for r in gemm) * 1e-3
     achieved = flop / secs / 1e12
-    traffic = None
+    # the kernel the roofline object names must be the one both large FC calls dispatched to in THIS run
+    ran = []
+    for x, w in ((rt.empty((4096, 784)), rt.empty((784, 4096))), (rt.empty((4096, 4096)), rt.empty((4096, 4096)))):
+        rt.fcbias(x, w, None, relu=True)
+        ran.append(rt.last_kernel())
+    rt.sync()
+    if any(name != ROOFLINE_KERNEL for name in ran):
+        sys.exit(f"bench.py: the large FC layers ran on {ran}, not on ROOFLINE_KERNEL = {ROOFLINE_KERNEL}: "
+                 f"update ROOFLINE_KERNEL and re-measure profiles/traffic.json before reporting a roofline")
+    traffic, traffic_source = None, None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):   # measured separately under rocprofv3 --pmc; see profiles/
-        traffic = json.load(open(tpath)).get(ROOFLINE_KERNEL, {}).get("bytes_per_launch")
+    if os.path.exists(tpath):   # measured separately under rocprofv3 --pmc (a counter run cannot share the timed run)
+        entry = json.load(open(tpath)).get(ROOFLINE_KERNEL, {})
+        traffic = entry.get("bytes_per_launch")
+        traffic_source = dict(file="profiles/traffic.json", **entry.get("measured", {}))
     out = {
         "metric": "samples/s per graph; TFLOP/s (FC/conv) & GB/s (eltwise) vs MI355X roofline",
         "value": head["samples_per_s"], "unit": "samples/s", "n_gpus": 1, "steps": args.steps,
@@ -367,7 +420,7 @@ def main():
                                "(BASELINE.json configs[1]), fused epilogues",
                    "global_batch": head["batch"], "device": rt.device_name()},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS_FP32_MFMA, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_TFLOPS_FP32_MFMA, "traffic": traffic,
+                     "frac": achieved / PEAK_TFLOPS_FP32_MFMA, "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": ROOFLINE_KERNEL + " (both launches per step: 4096x784x4096 and 4096x4096x4096)",
                      "flop_per_launch": flop / len(gemm), "avg_launch_ms": secs * 1e3 / len(gemm)},
         "gpu_ms_per_step": head["gpu_ms"] / args.steps,
@@ -389,7 +442,14 @@ def main():
         others["training_kernels"] = dict(kernels=run_training(rt))
         out["configs"] = others
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(graphs, args.cpu_rows)
+        cpu = cpu_baselines(graphs, args.cpu_rows)
+        out["cpu_baseline"] = cpu["cfg2"]
+        for name, entry in cpu.items():
+            if name != "cfg2" and "configs" in out:
+                out["configs"][name]["cpu_baseline"] = entry
+        out.setdefault("configs", {})["cfg2"] = dict(cpu_baseline=cpu["cfg2"], note="the headline workload: see the top level")
+    rt.sync()
+    rt.set_workspace(None)
     print(json.dumps(out))
 
 

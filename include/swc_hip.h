@@ -128,6 +128,10 @@ size_t swc_hip_conv2dGrad_workspace_bytes(const size_t *odims, const size_t *idi
 /* The same for a matrixSoftmaxWithLoss_f call over m rows of n (the rows' loss terms). */
 size_t swc_hip_matrixSoftmaxWithLoss_workspace_bytes(int m, int n);
 const char *swc_hip_last_error(void);         /* message of the last failure on this thread ("" if none) */
+/* Name of the kernel variant the last FC/GEMM or convolution call on this thread dispatched to, with its
+ * template arguments (e.g. "gemm_dma2<2,4,4,2,false,8>"; "" before the first such call): lets a harness check
+ * that the kernel it reports on is the one that ran. */
+const char *swc_hip_last_kernel(void);
 void *swc_hip_stream(void);                   /* the hipStream_t ops are launched on */
 int swc_hip_set_stream(void *hip_stream);     /* launch on a caller-owned stream (NULL: back to the library's own) */
 const char *swc_hip_device_name(void);        /* gcnArchName of the selected device */

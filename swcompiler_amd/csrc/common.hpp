@@ -23,6 +23,8 @@ int fail_code();   // the code of this thread's last fail() (for callers of help
 // The stream every op launches on; nullptr until swc_hip_init succeeded.
 hipStream_t stream();
 bool ready();
+// Records which kernel variant an op dispatched to (printf-style), for swc_hip_last_kernel().
+void note_kernel(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 int num_cus();   // of the initialised device (Device::computeUnits on a whole MI355X)
 // Scratch device memory for the current op (see runtime.hip); nullptr with the error recorded on failure.
 void *workspace(size_t bytes, const char *who);

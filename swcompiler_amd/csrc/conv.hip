@@ -506,6 +506,7 @@ int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGe
     const long tiles = (long)((g.M + T::BM - 1) / T::BM) * ((g.OC + T::BN - 1) / T::BN);
     const int nk = (g.K + BK - 1) / BK;
     const SkPlan p = conv_dma_plan<TM, TN, STAGES, MID>(g, scratch != nullptr);
+    note_kernel("conv_dma<%d,%d,%d,%s>%s", TM, TN, STAGES, MID ? "true" : "false", p.sk_wgs ? " + conv_sk_finish" : "");
     auto kern = conv_dma<TM, TN, STAGES, MID>;
     kern<<<(unsigned)(p.dp_tiles + p.sk_wgs), kThreads, T::kLdsBytes, stream()>>>(in, filt, out, g, (unsigned)in_bytes,
                                                                                   (unsigned)filt_bytes, ep, p, scratch);
@@ -549,6 +550,7 @@ bool takes_strip(const ConvGeom &g, const void *input, const void *filter, const
 template <int TMW, int TNW>
 int launch_conv_strip_as(const float *in, const float *filt, float *out, const ConvGeom &g, const strip::Plan &p,
                          const Epilogue &ep) {
+    note_kernel("conv_strip<%d,%d> R=%d BN=%d", TMW, TNW, p.R, p.BN);
     auto kern = strip::conv_strip<TMW, TNW>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -750,6 +752,7 @@ int launch_conv_direct(const float *in, const float *filt, const float *bias, fl
     const bool two = !four && (size_t)g.M >= (size_t)1024 * num_cus();
     const int pixels = four ? 4 : two ? 2 : 1;
     const unsigned blocks = ceil_div((size_t)g.M, (size_t)256 * pixels);
+    note_kernel("conv_direct<%d,%d>", ocq, pixels);
     auto launch = [&]<int OCQ>() {
         if constexpr (OCQ <= 5)
             if (four) return conv_direct<OCQ, 4><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep);
@@ -774,6 +777,7 @@ template <int TM, int TN>
 int launch_conv(bool vec, const float *in, const float *filt, float *out, const ConvGeom &g, const Epilogue &ep) {
     using T = Tile<TM, TN, true>;
     const long tiles = (long)((g.M + T::BM - 1) / T::BM) * ((g.OC + T::BN - 1) / T::BN);
+    note_kernel("conv_igemm<%d,%d,%s>", TM, TN, vec ? "true" : "false");
     auto kern = vec ? conv_igemm<TM, TN, true> : conv_igemm<TM, TN, false>;
     static bool attr_set[2] = {false, false};
     if (!attr_set[vec]) {

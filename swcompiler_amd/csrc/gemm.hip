@@ -443,6 +443,7 @@ int launch_tiled(bool vec, const float *a, const float *b, float *c, int m, int 
     using T = Tile<TM, TN, false>;
     const long tiles = (long)((m + T::BM - 1) / T::BM) * ((n + T::BN - 1) / T::BN);
     if (tiles > 0x7fffffffL) return fail(SWC_HIP_EINVAL, "gemm: too many tiles");
+    note_kernel("gemm_tiled<%d,%d,%s>", TM, TN, vec ? "true" : "false");
     auto kern = vec ? gemm_tiled<TM, TN, true> : gemm_tiled<TM, TN, false>;
     static bool attr_set[2] = {false, false};
     if (!attr_set[vec]) {
@@ -462,6 +463,7 @@ int launch_dma(const float *a, const float *b, float *c, int m, int n, int k, in
     using T = DmaTile<TM, TN, false, STAGES>;
     const long tiles = (long)((m + T::BM - 1) / T::BM) * ((n + T::BN - 1) / T::BN);
     if (tiles > 0x7fffffffL) return fail(SWC_HIP_EINVAL, "gemm: too many tiles");
+    note_kernel("gemm_dma<%d,%d,%d,%s>", TM, TN, STAGES, MID ? "true" : "false");
     auto kern = gemm_dma<TM, TN, STAGES, MID>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -483,6 +485,7 @@ int launch_dma2(const float *a, const float *b, float *c, int m, int n, int k, i
     using T = Dma2Tile<TM, TN, WM, STAGES, NW>;
     const long tiles = (long)((m + T::BM - 1) / T::BM) * ((n + T::BN - 1) / T::BN);
     if (tiles > 0x7fffffffL) return fail(SWC_HIP_EINVAL, "gemm: too many tiles");
+    note_kernel("gemm_dma2<%d,%d,%d,%d,%s,%d>", TM, TN, WM, STAGES, MID ? "true" : "false", NW);
     auto kern = gemm_dma2<TM, TN, WM, STAGES, MID, NW>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -512,6 +515,7 @@ int launch_splitk(const float *a, const float *b, float *c, int m, int n, int k,
         part = static_cast<float *>(workspace(need, "gemm (split-K)"));
         if (!part) return fail_code();   // (no workspace, one too small, or the allocation failed)
     }
+    note_kernel("gemm_dma2_splitk<%d,%d,%d,%d,false,4> x%d", TM, TN, WM, STAGES, splits);
     auto kern = gemm_dma2_splitk<TM, TN, WM, STAGES, false, 4>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -590,6 +594,7 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
         // 19.6 us against 22.0 with eight).
         const int waves = k <= 1024 ? 4 : kSkinnyMaxWaves;
         const unsigned blocks = ceil_div(m, 16);
+        note_kernel("gemm_skinny<%s>", vec ? "true" : "false");
         if (vec) gemm_skinny<true><<<blocks, 64 * waves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep, softmax);
         else gemm_skinny<false><<<blocks, 64 * waves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep, softmax);
         SWC_LAUNCH_CHECK();
@@ -598,6 +603,7 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
     const char *force = getenv("SWC_HIP_GEMM");
     // a handful of rows and a B of a few MB: one latency-bound pass over B (see gemm_fewrows)
     if (takes_fewrows(m, n, k) && (!force || !strcmp(force, "fewrows"))) {
+        note_kernel("gemm_fewrows");
         gemm_fewrows<<<ceil_div(n, 16), 64 * kFewRowsWaves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep);
         SWC_LAUNCH_CHECK();
         return SWC_HIP_OK;

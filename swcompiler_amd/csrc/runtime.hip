@@ -58,6 +58,13 @@ int fail(int code, const char *fmt, ...) {
     g_err_code = code;
     return code;
 }
+thread_local char g_kernel[96] = "";
+void note_kernel(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_kernel, sizeof(g_kernel), fmt, ap);
+    va_end(ap);
+}
 void clear_error() { g_err[0] = 0, g_err_code = SWC_HIP_OK; }
 int fail_code() { return g_err_code != SWC_HIP_OK ? g_err_code : SWC_HIP_ERUNTIME; }
 hipStream_t stream() { return g.cur; }
@@ -367,6 +374,8 @@ int swc_hip_sync(void) {
 }
 
 const char *swc_hip_last_error(void) { return g_err; }
+
+const char *swc_hip_last_kernel(void) { return g_kernel; }
 
 void *swc_hip_stream(void) { return (void *)g.cur; }
 

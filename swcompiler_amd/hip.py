@@ -20,7 +20,7 @@ EXPORTS = [
     "swc_hip_d2d", "swc_hip_copy_h2d_async", "swc_hip_copy_wait_ops", "swc_hip_ops_wait_copies", "swc_hip_copy_sync", "swc_hip_fill_f", "swc_hip_sync", "swc_hip_last_error", "swc_hip_stream",
     "swc_hip_set_stream", "swc_hip_device_name", "swc_hip_timer_begin", "swc_hip_timer_end",
     "swc_hip_timer_elapsed_ms", "swc_hip_event_record", "swc_hip_event_elapsed_ms", "swc_hip_graph_begin",
-    "swc_hip_graph_end", "swc_hip_graph_launch", "swc_hip_graph_destroy", "swc_hip_device_cus",
+    "swc_hip_graph_end", "swc_hip_graph_launch", "swc_hip_graph_destroy", "swc_hip_device_cus", "swc_hip_last_kernel",
     "swc_hip_enable_auto_workspace", "swc_hip_conv2dGrad_workspace_bytes", "swc_hip_matrixSoftmaxWithLoss_workspace_bytes",
     "swc_hip_matrixMatrixFCBias_noalloc_f",
     "swc_hip_matrixMatrixMul_f", "swc_hip_batchedadd_f", "swc_hip_relu_f",
@@ -80,6 +80,7 @@ def load_library():
         "swc_hip_graph_launch": (i32, [vp]),
         "swc_hip_graph_destroy": (i32, [vp]),
         "swc_hip_device_cus": (i32, []),
+        "swc_hip_last_kernel": (C.c_char_p, []),
         "swc_hip_enable_auto_workspace": (i32, [i32]),
         "swc_hip_conv2dGrad_workspace_bytes": (sz, [szp] * 6 + [sz]),
         "swc_hip_matrixSoftmaxWithLoss_workspace_bytes": (sz, [i32, i32]),
@@ -205,6 +206,10 @@ class SwcHip:
 
     def enable_auto_workspace(self, on):
         self._check(self.lib.swc_hip_enable_auto_workspace(int(on)), "swc_hip_enable_auto_workspace")
+
+    def last_kernel(self):
+        """the kernel variant the last FC/GEMM or convolution call dispatched to"""
+        return self.lib.swc_hip_last_kernel().decode()
 
     def device_cus(self):
         return int(self.lib.swc_hip_device_cus())
