@@ -389,7 +389,7 @@ def test_timed_hip_program(gen, oracle, tmp_path, graph):
     assert 0 < ms < 50
     want = oracle_run(oracle, "cfg3", 3, t)
     got = np.fromfile(os.path.join(tmp_path, "softmax_out_host.bin"), np.float32).reshape(want.shape)
-    assert strict_rel_err(got, want) < 5 * TOL
+    assert strict_rel_err(got, want) < TOL
 
 
 def test_graph_ir_and_passes_cpp_unit_tests(gen):
