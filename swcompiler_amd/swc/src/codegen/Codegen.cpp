@@ -1,6 +1,8 @@
 // CPU code generator and the machinery shared with the HIP target.
 #include "Codegen.h"
 
+#include "../pass/passes.h"
+
 #include <cassert>
 #include <cstdlib>
 #include <fstream>
@@ -173,6 +175,26 @@ void Codegen::emitEnvFinalize() { writer_ << "return 0;\n"; }
 
 // ------------------------------------------------------------------ driver
 std::string Codegen::generate() {
+    // Nested graphs (SubGraph nodes: the reference's route to a GPU, test/cuda/testGPUInfer.cpp, whose generator
+    // recurses into them, src/codegen/Codegen.cpp:1035-1077) are emitted in place of their node; on this one-device
+    // target every GPU they name is device Config::hip_device.
+    graph_->inlineSubGraphs(config_.hip_device);
+    // A program written for the reference's CUDA route (Config::cuda on a plain Codegen) or for the CPU, run with
+    // SWC_TARGET=hip or Config::hip: the hand-placed part keeps its Scatter/Gather nodes, what was left on the host
+    // is placed on the device as Engine::compile would, and the HIP generator writes the program.
+    if (!isHipGenerator()) {
+        const char *target = std::getenv("SWC_TARGET");
+        if (config_.hip || (target && std::string(target) == "hip")) {
+            Config cfg = config_;
+            cfg.hip = true;
+            cfg.cuda = cfg.cuda_stream = cfg.cublas = false;
+            graph_->setConfig(cfg);
+            pass::DeviceMemoryLoweringPass place(graph_, cfg.hip_device);
+            place.run();
+            HipCodegen hip(graph_, cfg);
+            return hip.generate();
+        }
+    }
     codeGenInit();
     emitHeader();
     headerWriter_ << "using namespace std;\n";

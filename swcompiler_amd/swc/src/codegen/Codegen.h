@@ -111,6 +111,7 @@ class Codegen {
     // Prints the program, writes ./Graph.cpp, ./G_Makefile and ./SW_Makefile,
     // returns the source text.
     std::string generate();
+    virtual bool isHipGenerator() const { return false; }
 
     virtual void initMakefileBuilder();
     virtual void emitHeader();
@@ -177,6 +178,7 @@ class HipCodegen : public Codegen {
 
   public:
     HipCodegen(IRGraph *graph, Config &config) : Codegen(graph, config) {}
+    bool isHipGenerator() const override { return true; }
     void initMakefileBuilder() override;
     void emitHeader() override;
     void emitEnvInit() override;

@@ -97,6 +97,21 @@ class IRGraph {
     std::string getCommTrace() const { return ""; }
     IRGraph *clone() const;
     void copyTo(IRGraph *empty) const;   // the same copy into a graph the caller has made
+
+    // The part of the graph between tensor `in` and tensor `out` moves into a nested graph behind a new SubGraph
+    // op node (reference: src/graphIR/IRGraph.cpp:99-223): inside, `in`, `out` and every parameter the part reads
+    // are represented by external mirror nodes of the same Tensor, joined to "<name>_sub" working copies by
+    // Scatter nodes (run-once for parameters) and a Gather node; outside, the SubGraph node reads `in` and the
+    // parameters and produces `out`.  Returns the node, or null if `out` does not depend on `in`.
+    OpNode *extractSubGraph(TensorNode *in, TensorNode *out);
+    // extractSubGraph, then `num` such SubGraph nodes side by side, each over 1/num of `in` along axis 0
+    // (reference: src/graphIR/IRGraph.cpp:47-97; SLICE along axis 0 only, as there).
+    bool buildSubGraphs(TensorNode *in, TensorNode *out, ParallelStrategy strategy, int axis = 0, int num = 2);
+    // Code generation on one device: every SubGraph node is replaced by the nodes of its nested graph (nested
+    // ones first), a mirror node becoming the outer node of the same Tensor, and every GPU label becomes device
+    // `device` — the op sequence a generator that recursed into the nested graphs at the SubGraph node's place
+    // (reference: src/codegen/Codegen.cpp:1035-1077) would emit.  Returns the number of nodes replaced.
+    int inlineSubGraphs(int device = 0);
 };
 
 template <typename V, typename N> void IRGraph::eraseNode(V &vec, N *node, const char *what) {

@@ -479,6 +479,8 @@ void DeviceMemoryLoweringPass::run() {
                 if (c->nodeType() == OP_NODE && static_cast<OpNode *>(c)->getOp()->getOpName() == "Dropout" &&
                     c->parentNum() > 1 && c->getParentNode(1) == t && c->getParentNode(0) != t)
                     continue;
+                // (a Scatter node placed by hand IS the upload of this host tensor: its operand stays on the host)
+                if (c->nodeType() == OP_NODE && static_cast<OpNode *>(c)->getOp()->getOpName() == "Scatter") continue;
                 if (onGpu(c) && std::find(gpuReaders.begin(), gpuReaders.end(), c) == gpuReaders.end())
                     gpuReaders.push_back(c);
             }
@@ -510,15 +512,21 @@ void DeviceMemoryLoweringPass::run() {
         } else {
             // 3. GPU tensor that leaves the device: host twin + Gather
             std::vector<IRNode *> hostReaders;
-            for (IRNode *c : t->getChildNodes())
+            for (IRNode *c : t->getChildNodes()) {
+                // (a Gather node placed by hand IS the download of this device tensor)
+                if (c->nodeType() == OP_NODE && static_cast<OpNode *>(c)->getOp()->getOpName() == "Gather") continue;
                 if (!onGpu(c) && std::find(hostReaders.begin(), hostReaders.end(), c) == hostReaders.end())
                     hostReaders.push_back(c);
+            }
+            bool gathered = false;   // already downloaded by a hand-placed Gather: no second copy as an output
+            for (IRNode *c : t->getChildNodes())
+                gathered |= c->nodeType() == OP_NODE && static_cast<OpNode *>(c)->getOp()->getOpName() == "Gather";
             // (a training graph marks its outputs — the updated parameters, the displayed loss; a gradient nobody
             // reads, such as the one a conv2dGrad computes for the data, is not one)
             bool isOutput = t->getLabel()->getIsOut() != 0 || (!cfg.train_mode && t->childNum() == 0);
             for (IRNode *lo : _graph->getLogicalOutNodes())
                 if (lo == t) isOutput = true;
-            if (hostReaders.empty() && !isOutput) continue;
+            if (hostReaders.empty() && (!isOutput || gathered)) continue;
             auto *twin = new TensorNode(t->name() + "_host", t->getTensor()->clone());
             twin->getTensor()->setTensorInit(TensorInitType::NONE);
             twin->getLabel()->setDeviceLabel(Device());

@@ -163,6 +163,86 @@ int main(int argc, char **argv) {
         GpT(graph, data0, weight0, bias0, data1, data2, weight1, bias1, data3, data4, top3_t);
         GpO(graph, fc0, tanh0, fc1, softmax, argmax_o, print_o);
         graph->addLogicalOutNodes(data4, top3_t);   // dump the probabilities and the top-3 table
+    } else if (model == "mnist8_subgraphs") {
+        // The reference's route to a GPU (test/cuda/testGPUInfer.cpp, test/old/testGraphPartition.cpp): the first
+        // layer of the MNIST example is cut out into two nested graphs, one per half of the batch, each labelled
+        // for a GPU of its own, and a plain Codegen is asked for the CUDA target.  On this one-device target
+        // (Config::hip, or SWC_TARGET=hip in the environment) both halves run on the one GPU.
+        TENSOR(data0, 8, 784);
+        TENSOR(weight0, 784, 512);
+        TENSOR(bias0, 512);
+        INIT(data0, TensorInitType::FILE, "mnist_images_8.bin");
+        INIT(weight0, TensorInitType::FILE, "mlp_weight0.bin");
+        INIT(bias0, TensorInitType::FILE, "mlp_bias0.bin");
+        OP(fc0, MatrixMatrixFCBiasOp);
+        LINKUPPER(fc0, data0, weight0, bias0);
+        TENSOR(data1, 8, 512);
+        LINKUPPER(data1, fc0);
+        OP(tanh0, MatrixTanhOp);
+        LINKUPPER(tanh0, data1);
+        TENSOR(data2, 8, 512);
+        LINKUPPER(data2, tanh0);
+        TENSOR(weight1, 512, 10);
+        TENSOR(bias1, 10);
+        INIT(weight1, TensorInitType::FILE, "mlp_weight1.bin");
+        INIT(bias1, TensorInitType::FILE, "mlp_bias1.bin");
+        OP(fc1, MatrixMatrixFCBiasOp);
+        LINKUPPER(fc1, data2, weight1, bias1);
+        TENSOR(data3, 8, 10);
+        LINKUPPER(data3, fc1);
+        OP(softmax, MatrixSoftmaxOp);
+        LINKUPPER(softmax, data3);
+        TENSOR(data4, 8, 10);
+        LINKUPPER(data4, softmax);
+        auto *argmax_o = new OpNode("argmax", new ArgMaxOp(3));
+        argmax_o->exlinkUpperNode(data4);
+        auto *top3_t = new TensorNode("top3", new Tensor({8, 3}, DataType::Int32_t), argmax_o);
+        auto *print_o = new OpNode("print", new DebugOp());
+        print_o->exlinkUpperNode(top3_t);
+        GpT(graph, data0, weight0, bias0, data1, data2, weight1, bias1, data3, data4, top3_t);
+        GpO(graph, fc0, tanh0, fc1, softmax, argmax_o, print_o);
+        graph->addLogicalOutNodes(data4, top3_t);
+
+        if (!graph->buildSubGraphs(data0, data2, ParallelStrategy::SLICE, 0, 2)) {
+            cerr << "buildSubGraphs failed" << endl;
+            return 1;
+        }
+        graph->findInOut();
+        graph->updateTopology();
+        pass::Optimizer opt(graph);
+        opt.runOptimizer();
+        int dev = 0;
+        for (int i = 0; i < graph->opNodeNum(); ++i) {
+            auto *sub = dynamic_cast<SubGraphOp *>(graph->getOpNode(i)->getOp());
+            if (!sub) continue;
+            IRGraph *inner = sub->getGraph();
+            // the second half of the batch: element offsets on the host side of its Scatter and Gather, as the
+            // reference's example sets them by hand (test/cuda/testGPUInfer.cpp:177-178, 205-206); the nodes of a
+            // cloned graph share their Op objects with the original, so these two get Ops of their own
+            if (dev == 1)
+                for (int j = 0; j < inner->opNodeNum(); ++j) {
+                    OpNode *o = inner->getOpNode(j);
+                    if (dynamic_cast<ScatterOp *>(o->getOp())) {
+                        if (!o->isRunOnce()) o->setOp(new ScatterOp(4 * 784));
+                    } else if (dynamic_cast<GatherOp *>(o->getOp())) {
+                        o->setOp(new GatherOp(4 * 512));
+                    }
+                }
+            inner->setDeviceLabel(Device(0, DeviceType::GPU, dev++));
+            inner->findInOut();
+            inner->updateTopology();
+            opt.setGraph(inner);
+            opt.runOptimizer();
+        }
+        Config config;
+        config.cuda = true;
+        config.cuda_stream = true;
+        config.cublas = true;
+        config.hip = target == "hip";   // (or SWC_TARGET=hip)
+        config.dump_outputs = true;
+        codegen::Codegen generator(graph, config);
+        cout << generator.generate();
+        return dev == 2 ? 0 : 1;
     } else if (model == "mnist_loader") {
         // the reference's test/engine/testEngineMLPInfer.cpp: batch loop over a record file,
         // FCBias -> Tanh -> FCBias -> Softmax -> ArgMax(1) -> Accuracy, counters printed at the end

@@ -138,6 +138,61 @@ static void testFusionAndPlacement() {
     CHECK(print->getLabel()->getDeviceLabel().type == DeviceType::CPU);
 }
 
+static void testSubGraphs() {
+    // x -> fc -> y -> tanh -> z -> relu -> r ; the part from x to z becomes nested graphs
+    TENSOR(x, 8, 32);
+    TENSOR(w, 32, 16);
+    TENSOR(b, 16);
+    OP(fc, MatrixMatrixFCBiasOp);
+    LINKUPPER(fc, x, w, b);
+    TENSOR(y, 8, 16);
+    LINKUPPER(y, fc);
+    OP(act, MatrixTanhOp);
+    LINKUPPER(act, y);
+    TENSOR(z, 8, 16);
+    LINKUPPER(z, act);
+    OP(relu, ReluOp);
+    LINKUPPER(relu, z);
+    TENSOR(r, 8, 16);
+    LINKUPPER(r, relu);
+    G(g);
+    GpT(g, x, w, b, y, z, r);
+    GpO(g, fc, act, relu);
+    CHECK(g->extractSubGraph(r, x) == nullptr);   // x does not depend on r
+    CHECK(g->buildSubGraphs(x, z, ParallelStrategy::SLICE, 0, 2));
+    CHECK(countOps(g, "SubGraph") == 2 && countOps(g, "MatrixMatrixFCBias") == 0 && countOps(g, "Relu") == 1);
+    CHECK(g->tensorNodeNum() == 5);               // x, w, b, z, r: y moved inside
+    int seen = 0;
+    for (int i = 0; i < g->opNodeNum(); ++i) {
+        auto *sub = dynamic_cast<SubGraphOp *>(g->getOpNode(i)->getOp());
+        if (!sub) continue;
+        OpNode *node = g->getOpNode(i);
+        CHECK(node->parentNum() == 3 && node->getParentNode(0) == x && node->childNum() == 1 && node->getChildNode(0) == z);
+        IRGraph *in = sub->getGraph();
+        CHECK(countOps(in, "Scatter") == 3 && countOps(in, "Gather") == 1 && countOps(in, "MatrixMatrixFCBias") == 1);
+        auto *xs = static_cast<TensorNode *>(in->getNodeByName("x_sub"));
+        auto *zs = static_cast<TensorNode *>(in->getNodeByName("z_sub"));
+        CHECK(xs && zs && xs->getDims() == (vector<size_t>{4, 32}) && zs->getDims() == (vector<size_t>{4, 16}));
+        auto *mirror = static_cast<TensorNode *>(in->getNodeByName("x"));
+        CHECK(mirror && mirror->isExternal() && mirror->getTensor() == x->getTensor());
+        in->setDeviceLabel(Device(0, DeviceType::GPU, seen));
+        CHECK(mirror->getLabel()->getDeviceLabel().type == DeviceType::CPU);   // mirrors keep the outer device
+        CHECK(xs->getLabel()->getDeviceLabel().id == seen);
+        ++seen;
+    }
+    CHECK(seen == 2);
+    CHECK(g->inlineSubGraphs(0) == 2);
+    CHECK(countOps(g, "SubGraph") == 0 && countOps(g, "MatrixMatrixFCBias") == 2 && countOps(g, "Scatter") == 6);
+    CHECK(z->parentNum() == 2 && z->getParentNode(0)->name() == "gather" && z->getParentNode(1)->name() == "gather");
+    CHECK(x->childNum() == 2 && w->childNum() == 2);
+    for (int i = 0; i < g->tensorNodeNum(); ++i) {
+        const Device d = g->getTensorNode(i)->getLabel()->getDeviceLabel();
+        CHECK(d.type == DeviceType::CPU || d.id == 0);   // every GPU label is the one device now
+        CHECK(!g->getTensorNode(i)->isExternal());
+    }
+    CHECK(g->topologyNum() == 11);   // x, scatter, x_sub, fc, y, tanh, z_sub, gather, z, relu, r: one level each
+}
+
 static void testElimination() {
     TENSOR(x, 2, 3, 4, 5);
     auto *t1 = new OpNode("t1", new TransposeOp(NCHW2NHWC));
@@ -323,6 +378,7 @@ int main() {
     testTopologyAndShapes();
     testLoweringAndRenaming();
     testFusionAndPlacement();
+    testSubGraphs();
     testElimination();
     testResidualBlockAndCounters();
     testAutodiff();

@@ -215,6 +215,35 @@ def test_mnist8_hip_program_prints_the_reference_labels(gen, tmp_path, golden):
     assert_bit_exact(top3, golden["mnist8_top3"], "dumped top-3")
 
 
+def test_subgraph_program_structure(gen, tmp_path):
+    """IRGraph::buildSubGraphs + SubGraph nodes labelled for two GPUs + a plain Codegen (the reference's route to a
+    GPU): on this target both nested graphs are emitted in place, on the one device"""
+    for f in os.listdir(os.path.join(ROOT, "tests", "golden", "mnist8")):
+        shutil.copy(os.path.join(ROOT, "tests", "golden", "mnist8", f), tmp_path)
+    code = generate(gen, "mnist8_subgraphs", "hip", tmp_path)
+    head, body = code.split("// call op routine functions")
+    assert head.count("swc_hip_h2d(weight0_sub") == 2 and head.count("swc_hip_h2d(bias0_sub") == 2
+    assert "swc_hip_h2d(data0_sub, data0, 12544)" in body and "swc_hip_h2d(data0_sub1, data0 + 3136, 12544)" in body
+    assert "swc_hip_d2h(data2, data2_sub, 8192)" in body and "swc_hip_d2h(data2 + 2048, data2_sub1, 8192)" in body
+    assert "SubGraph" not in body and "gpu1_baseptr" not in code
+    build_hip(tmp_path)
+
+
+@pytest.mark.gpu
+def test_subgraph_program_prints_the_reference_labels(gen, tmp_path, golden):
+    """the same program run: the reference's MNIST labels, and the probabilities of the un-partitioned program"""
+    for f in os.listdir(os.path.join(ROOT, "tests", "golden", "mnist8")):
+        shutil.copy(os.path.join(ROOT, "tests", "golden", "mnist8", f), tmp_path)
+    generate(gen, "mnist8_subgraphs", "hip", tmp_path)
+    exe = build_hip(tmp_path)
+    out = subprocess.run([exe], cwd=tmp_path, check=True, capture_output=True, text=True, timeout=120).stdout
+    rows = [[int(v) for v in line.split()] for line in out.strip().splitlines()]
+    assert [r[0] for r in rows] == [5, 0, 4, 1, 9, 2, 1, 3]
+    assert_bit_exact(np.array(rows, np.int32), golden["mnist8_top3"], "printed top-3")
+    prob = np.fromfile(os.path.join(tmp_path, "data4_host.bin"), np.float32).reshape(8, 10)
+    assert strict_rel_err(prob, golden["mnist8_prob"]) < TOL
+
+
 # ------------------------------------------------------ batch loop (dataloader)
 def write_record_file(tmp_path, samples, seed=5):
     """`samples` records of <1-byte label><784 fp32>; half of the images are the reference's eight

@@ -22,7 +22,7 @@ from tests.test_codegen import GEN, REF_UTILS, ROOT, SWC
 REF_TESTS = "/root/reference/test"
 pytestmark = pytest.mark.skipif(not os.path.isdir(REF_TESTS), reason="the reference tree is not here")
 
-MULTI_RANK = {"benchmark/benchParallelLowering", "old/testGraphPartition", "old/testParaMLPTraining", "parallel/testJointGraph",
+MULTI_RANK = {"benchmark/benchParallelLowering", "old/testParaMLPTraining", "parallel/testJointGraph",
               "parallel/testLenetDistTrain", "parallel/testMLPDistTrain", "parallel/testParallelInfer",
               "parallel/testParallelInferStrategyB", "parallel/testParallelInferStrategyC",
               "parallel/testParallelInferStrategyD", "testParallelPattern"}
@@ -46,11 +46,18 @@ def compile_program(name, lib, out=None):
     return subprocess.run(cmd, capture_output=True, text=True)
 
 
-def test_every_single_device_program_compiles(lib):
+def test_every_single_device_program_compiles_and_links(lib, tmp_path):
+    """compiled AND linked against libswc.a (a declaration without a definition would pass a syntax check)"""
     names = programs()
     assert len(names) >= 30 and MULTI_RANK <= set(names)
-    failed = {n: compile_program(n, lib).stderr.splitlines()[:3] for n in names if n not in MULTI_RANK}
-    failed = {n: e for n, e in failed.items() if e}
+    single = [n for n in names if n not in MULTI_RANK]
+    assert len(single) >= 22 and "cuda/testGPUInfer" in single and "old/testGraphPartition" in single
+    from concurrent.futures import ThreadPoolExecutor
+    def build(n):
+        r = compile_program(n, lib, os.path.join(tmp_path, n.replace("/", "_") + ".bin"))
+        return n, (r.stderr.splitlines()[:3] if r.returncode else None)
+    with ThreadPoolExecutor(4) as pool:
+        failed = {n: e for n, e in pool.map(build, single) if e}
     assert not failed, failed
 
 
@@ -77,12 +84,42 @@ def test_program_generates_code_that_builds(lib, tmp_path, name, calls):
     build_generated(tmp_path)
 
 
-def test_gpu_example_is_refused_with_a_message(lib, tmp_path):
-    """test/cuda/testGPUInfer.cpp asks for the CUDA target (Config::cuda): not part of this build, and said so"""
+def test_gpu_example_retargeted_by_the_environment(lib, tmp_path):
+    """test/cuda/testGPUInfer.cpp — the reference's only GPU example: two hand-built SubGraph nodes labelled for
+    GPU 0 and GPU 1, a plain Codegen with Config::cuda — unchanged, with SWC_TARGET=hip: the generator writes the
+    nested graphs' ops in place of their nodes, both on the one device, keeps the hand-placed Scatter/Gather nodes
+    with their offsets, and places the rest of the graph on the device too.  Without the variable the CUDA target
+    is refused with a message."""
+    from tests.test_codegen import build_hip
     exe = os.path.join(tmp_path, "program.bin")
     assert compile_program("cuda/testGPUInfer", lib, exe).returncode == 0
     r = subprocess.run([exe], cwd=tmp_path, capture_output=True, text=True, timeout=120)
     assert r.returncode != 0 and "use Config::hip" in r.stderr
+    subprocess.run([exe], cwd=tmp_path, check=True, capture_output=True, timeout=120, env=dict(os.environ, SWC_TARGET="hip"))
+    code = open(os.path.join(tmp_path, "Graph.cpp")).read()
+    head, body = code.split("// call op routine functions")
+    for name in ("weight0_gpu0, weight0", "weight0_gpu1, weight0", "bias0_gpu0, bias0", "bias0_gpu1, bias0"):
+        assert f"swc_hip_h2d({name}," in head            # parameters: uploaded once, to both copies
+    assert "swc_hip_h2d(data0_gpu0, data0, 12544)" in body and "swc_hip_h2d(data0_gpu1, data0 + 3136, 12544)" in body
+    assert "swc_hip_d2h(data2, data2_gpu0, 8192)" in body and "swc_hip_d2h(data2 + 2048, data2_gpu1, 8192)" in body
+    assert body.count("swc_hip_matrixMatrixMul_f(4, 512, 784,") == 2 and body.count("swc_hip_matrixTanh_f(4, 512,") == 2
+    assert "swc_hip_matrixSoftmax_f(8, 10," in body and "swc_hip_argMax_i(" in body
+    assert "cuda" not in code and "gpu1_baseptr" not in code   # one device, one arena
+    build_hip(tmp_path)
+
+
+def test_graph_partition_example(lib, tmp_path):
+    """test/old/testGraphPartition.cpp: IRGraph::buildSubGraphs cuts the first layer into two SubGraph nodes; the
+    program runs, and with SWC_TARGET=hip its graph becomes a HIP program that builds"""
+    from tests.test_codegen import build_hip
+    exe = os.path.join(tmp_path, "program.bin")
+    assert compile_program("old/testGraphPartition", lib, exe).returncode == 0
+    out = subprocess.run([exe], cwd=tmp_path, check=True, capture_output=True, text=True, timeout=120,
+                         env=dict(os.environ, SWC_TARGET="hip")).stdout
+    assert "build SubGraph Ok" in out and out.count("subGraph Node") == 2
+    code = open(os.path.join(tmp_path, "Graph.cpp")).read()
+    assert code.count("swc_hip_matrixTanh_f(4, 512,") == 2
+    build_hip(tmp_path)
 
 
 def test_engine_mlp_infer_example_retargeted_by_the_environment(lib, tmp_path):
