@@ -508,3 +508,116 @@ def test_lenet_and_vgg_import_hip_program(gen, oracle, tmp_path, make):
     want = run_net(oracle, predict, w, data)["gpu_0/softmax"]
     assert rel_err(prob, want) < TOL
     assert (top3[:, 0] == oracle.argMax(want, 1)[:, 0]).all()
+
+
+# ------------------------------------------------ the same files through the protobuf library
+# The fixtures above are written by this file's own encoder and read by the importer's own decoder: a shared
+# misreading of the reference's src/importer/caffe2.proto would pass.  Here the messages are built with the
+# protobuf library of the Python environment from descriptors that carry the field numbers and types of that
+# file (Argument: caffe2.proto:152-166, DeviceOption: 192-207, OperatorDef: 210-268, NetDef: 270-309), serialised
+# by the library — unpacked as proto2 declares the repeated scalars, and packed as newer writers emit them — and
+# printed by its text format; the importer must read them exactly as it reads the hand-written files.
+_CLASSES = {}
+
+
+def caffe2_classes(packed):
+    if packed not in _CLASSES:
+        _CLASSES[packed] = _caffe2_classes(packed)
+    return _CLASSES[packed]
+
+
+def _caffe2_classes(packed):
+    from google.protobuf import descriptor_pb2, descriptor_pool, message_factory
+    F = descriptor_pb2.FieldDescriptorProto
+    pkg = "c2p" if packed else "c2u"
+    fd = descriptor_pb2.FileDescriptorProto(name=pkg + ".proto", package=pkg, syntax="proto2")
+
+    def msg(name, fields):
+        m = fd.message_type.add(name=name)
+        for fname, number, ftype, label, type_name in fields:
+            f = m.field.add(name=fname, number=number, type=ftype, label=label)
+            if type_name:
+                f.type_name = "." + pkg + "." + type_name
+            if packed and label == F.LABEL_REPEATED and ftype in (F.TYPE_FLOAT, F.TYPE_INT64):
+                f.options.packed = True
+    O, R = F.LABEL_OPTIONAL, F.LABEL_REPEATED
+    msg("Argument", [("name", 1, F.TYPE_STRING, O, None), ("f", 2, F.TYPE_FLOAT, O, None), ("i", 3, F.TYPE_INT64, O, None),
+                     ("s", 4, F.TYPE_BYTES, O, None), ("floats", 5, F.TYPE_FLOAT, R, None), ("ints", 6, F.TYPE_INT64, R, None),
+                     ("strings", 7, F.TYPE_BYTES, R, None)])
+    msg("DeviceOption", [("device_type", 1, F.TYPE_INT32, O, None), ("device_id", 2, F.TYPE_INT32, O, None)])
+    msg("OperatorDef", [("input", 1, F.TYPE_STRING, R, None), ("output", 2, F.TYPE_STRING, R, None),
+                        ("name", 3, F.TYPE_STRING, O, None), ("type", 4, F.TYPE_STRING, O, None),
+                        ("arg", 5, F.TYPE_MESSAGE, R, "Argument"), ("device_option", 6, F.TYPE_MESSAGE, O, "DeviceOption"),
+                        ("engine", 7, F.TYPE_STRING, O, None), ("is_gradient_op", 9, F.TYPE_BOOL, O, None)])
+    msg("NetDef", [("name", 1, F.TYPE_STRING, O, None), ("op", 2, F.TYPE_MESSAGE, R, "OperatorDef"),
+                   ("type", 3, F.TYPE_STRING, O, None), ("device_option", 5, F.TYPE_MESSAGE, O, "DeviceOption"),
+                   ("arg", 6, F.TYPE_MESSAGE, R, "Argument"), ("external_input", 7, F.TYPE_STRING, R, None),
+                   ("external_output", 8, F.TYPE_STRING, R, None)])
+    pool = descriptor_pool.DescriptorPool()
+    pool.Add(fd)
+    return message_factory.GetMessageClass(pool.FindMessageTypeByName(pkg + ".NetDef"))
+
+
+def library_net(name, ops, packed):
+    net = caffe2_classes(packed)(name=name)
+    for o in ops:
+        op = net.op.add(name="", type=o["type"], engine="CUDNN", is_gradient_op=False)
+        op.input.extend(o["input"])
+        op.output.extend(o["output"])
+        op.device_option.device_type = 1
+        op.device_option.device_id = 0
+        for k, v in o.get("arg", {}).items():
+            a = op.arg.add(name=k)
+            if isinstance(v, float):
+                a.f = v
+            elif isinstance(v, int):
+                a.i = v
+            elif isinstance(v, str):
+                a.s = v.encode()
+            elif isinstance(v, np.ndarray):
+                a.floats.extend(float(x) for x in v.ravel())
+            else:
+                a.ints.extend(int(x) for x in v)
+    net.external_input.append("gpu_0/data")
+    return net
+
+
+def program_and_weights(gen, model, workdir):
+    code = generate(gen, model, "cpu", workdir, 2)
+    wdir = os.path.join(workdir, "weights")
+    return code, {f: open(os.path.join(wdir, f), "rb").read() for f in sorted(os.listdir(wdir))}
+
+
+def test_files_written_by_the_protobuf_library_import_identically(gen, tmp_path):
+    pytest.importorskip("google.protobuf")
+    from google.protobuf import text_format
+    w = make_weights()
+    predict, init = make_nets(w)
+    dirs = {}
+    for tag_ in ("hand", "lib_unpacked", "lib_packed", "lib_text"):
+        dirs[tag_] = os.path.join(tmp_path, tag_)
+        os.mkdir(dirs[tag_])
+        write_model(dirs[tag_], True)                       # (data.bin; its model files are replaced below)
+        if tag_ != "hand":
+            for f in ("predict_net.pb", "init_net.pb"):
+                os.remove(os.path.join(dirs[tag_], f))
+    for packed in (False, True):
+        d = dirs["lib_packed" if packed else "lib_unpacked"]
+        for fname, nm, ops in (("predict_net.pb", "mini_resnet", predict), ("init_net.pb", "mini_resnet_init", init)):
+            msg = library_net(nm, ops, packed)
+            open(os.path.join(d, fname), "wb").write(msg.SerializeToString())
+            # and the other way round: the library reads this file's own encoder's bytes as the same message
+            back = caffe2_classes(packed)()
+            back.ParseFromString(enc_net(nm, ops, packed))
+            plain = caffe2_classes(packed)()
+            plain.CopyFrom(msg)
+            for op in plain.op:
+                op.ClearField("device_option")          # (the hand encoder's binary files carry none)
+            assert back == plain, fname
+    for fname, nm, ops in (("predict_net.pbtxt", "mini_resnet", predict), ("init_net.pbtxt", "mini_resnet_init", init)):
+        open(os.path.join(dirs["lib_text"], fname), "w").write(text_format.MessageToString(library_net(nm, ops, False)))
+    want = program_and_weights(gen, "caffe2", dirs["hand"])
+    assert len(want[1]) == len(w)
+    assert program_and_weights(gen, "caffe2", dirs["lib_unpacked"]) == want
+    assert program_and_weights(gen, "caffe2", dirs["lib_packed"]) == want
+    assert program_and_weights(gen, "caffe2txt", dirs["lib_text"]) == want
