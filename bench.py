@@ -88,7 +88,10 @@ class Timed:
 def _gemm_work(res, a, b, *r, **kw):
     m, k = a.shape
     n = b.shape[1]
-    return dict(shape=f"{m}x{k}x{n}", flop=2.0 * m * n * k)
+    work = dict(shape=f"{m}x{k}x{n}", flop=2.0 * m * n * k)
+    if n <= 16:   # a classifier head: one pass over A is what bounds it, not the arithmetic
+        work["bytes"] = 4.0 * (m * k + k * n + m * n)
+    return work
 
 
 def _conv_work(res, x, f, *r, **kw):
@@ -116,7 +119,12 @@ WORK = {
 def rate(row):
     """adds achieved rate and roofline fraction to a kernel row"""
     s = row["ms"] * 1e-3
-    if "flop" in row:
+    if "flop" in row and "bytes" in row:   # GEMM with N <= 16: both figures, judged against the HBM roofline
+        row["tflops"] = row["flop"] / s / 1e12
+        row["gbs"] = row["bytes"] / s / 1e9
+        row["frac"] = row["gbs"] / PEAK_HBM_GBS
+        row["bound"] = "hbm"
+    elif "flop" in row:
         row["tflops"] = row["flop"] / s / 1e12
         row["frac"] = row["tflops"] / PEAK_TFLOPS_FP32_MFMA
         row["bound"] = "mfma"

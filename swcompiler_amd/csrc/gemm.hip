@@ -8,6 +8,8 @@
 //                v_mfma_f32_16x16x4_f32 straight from global memory (B is a few
 //                KB and stays in cache) and the partial 16x16 tiles are summed
 //                through LDS.
+//   gemm_skinny_stream  the same product for K above 1024: A and B by LDS-DMA
+//                into rings private to each wavefront, no barrier in the K loop.
 #include "common.hpp"
 #include "mfma_dma.hpp"
 #include "mfma_dma2.hpp"
@@ -384,6 +386,175 @@ __global__ __launch_bounds__(64 * kSkinnyMaxWaves) void gemm_skinny(const float 
     }
 }
 
+// ------------------------------------------------- skinny GEMM, long K, streamed
+// N <= 16 with K above 1024 (a classifier head behind a wide layer): one pass over A at close to the rate of a
+// plain read.  What holds gemm_skinny back on such shapes is not the arithmetic but the loads: it fetches B with
+// 32-bit gathers (four times as many load instructions as for A, each touching several cache lines) and its
+// wavefronts alternate between "all loads of a trip" and "all MFMAs of a trip".  Here
+//   * a workgroup still owns 16 rows and its sixteen wavefronts split K in groups of 32 (wavefront w takes groups
+//     w, w + 16, ...), but every group travels by LDS-DMA into a ring that is private to the wavefront: the A tile
+//     of the group (16 rows x 128 bytes: eight consecutive lanes fetch one whole cache line, streaming cache
+//     policy) and the 32 rows of B that go with it (32 x N consecutive floats since ldb == N);
+//   * no barrier inside the K loop: a wavefront waits for its own oldest group (s_waitcnt vmcnt), reads its
+//     fragments out of the slot, and requests the group kRing steps ahead into the slot it has just read;
+//   * workgroups start at different groups (rotated by the workgroup index), so that at any moment the chip
+//     reads from many 2-KiB windows of the rows and not from the same one in every row;
+//   * two MFMA chains (first and second 64 bytes of a row's line), added at the end.
+// k of a group is dealt to the four k-lanes of v_mfma_f32_16x16x4_f32 as q, step s -> 4q + 16(s / 4) + s % 4, the
+// same on the A and the B side.  The 16-byte pieces of a line are XOR-ed with the row inside a slot (bank spread).
+// Partial tiles are summed through LDS in wavefront order, as in gemm_skinny, with the same epilogue.
+constexpr int kStreamWaves = 16;
+constexpr int kStreamATile = 2048;   // bytes of a group's A tile in a slot; the B rows follow
+
+__host__ __device__ inline int stream_slot_bytes(int ldb) { return kStreamATile + ((32 * ldb * 4 + 15) & ~15); }
+
+template <int RING, bool B2>
+__global__ __launch_bounds__(64 * kStreamWaves) void gemm_skinny_stream(const float *__restrict__ A,
+                                                                         const float *__restrict__ B,
+                                                                         float *__restrict__ C, int M, int N, int K,
+                                                                         unsigned lda, int ldb, size_t ldc, Epilogue ep,
+                                                                         int softmax) {
+#if __HIP_DEVICE_COMPILE__
+    extern __shared__ __align__(16) float lds[];
+    constexpr int kNone = 0x7fffffff;   // byte offset outside every buffer: the load stores zeros
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int i = lane & 15, q = lane >> 4;
+    const size_t row0 = (size_t)blockIdx.x * 16;
+    const int rows = (M - (int)row0) < 16 ? (M - (int)row0) : 16;
+    const __amdgpu_buffer_rsrc_t rs_a = make_rsrc(A + row0 * lda, (unsigned)(((size_t)(rows - 1) * lda + K) * 4));
+    const __amdgpu_buffer_rsrc_t rs_b = make_rsrc(B, (unsigned)((size_t)K * ldb * 4));
+    const int slot_bytes = stream_slot_bytes(ldb);
+    char *const ring = reinterpret_cast<char *>(lds) + wave * (RING * slot_bytes);
+
+    // loads: lane = 8 * (row % 8) + piece; load h of a group takes rows 8h .. 8h + 7
+    const int r8 = lane >> 3, seg = (lane & 7) ^ r8;
+    const int a_lane = (int)((r8 * lda + 4 * seg) * 4);
+    const unsigned a_second = 8u * lda * 4u;
+    const bool b1_lane = lane * 16 < 32 * ldb * 4, b2_lane = 1024 + lane * 16 < 32 * ldb * 4;
+    // fragment reads: row i, pieces q and q + 4 of its line; B[4q + ..][column i]
+    const int i8 = i & 7;
+    const int rd0 = (i >> 3) * 1024 + (i8 * 8 + (q ^ i8)) * 16;
+    const int rd1 = (i >> 3) * 1024 + (i8 * 8 + ((q + 4) ^ i8)) * 16;
+    const bool col_ok = i < N;
+    const int rdb = kStreamATile + (4 * q * ldb + (col_ok ? i : 0)) * 4;
+
+    const int groups = (K + 31) / 32;
+    const int T = (groups - wave + kStreamWaves - 1) / kStreamWaves;   // groups of this wavefront (may be 0)
+    const int rot = T > 0 ? (int)(blockIdx.x % (unsigned)T) : 0;
+    auto request = [&](int t, int r) {
+        int tt = t + rot;
+        if (tt >= T) tt -= T;
+        const int k0 = (tt * kStreamWaves + wave) * 32;
+        char *slot = ring + r * slot_bytes;
+        if (b1_lane)   // (every lane for ldb >= 8; below that the rows of B end before the 1 KiB of a full load)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_void_t *)(slot + kStreamATile), 16, lane * 16, k0 * ldb * 4, 0, 0);
+        if (B2) {
+            if (b2_lane)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_void_t *)(slot + kStreamATile + 1024), 16, lane * 16,
+                                                         k0 * ldb * 4 + 1024, 0, 0);
+        }
+        const int voff = (k0 + 4 * seg < K) ? a_lane : kNone;   // K % 4 == 0: a piece is wholly inside a row or not
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_void_t *)(slot), 16, voff, k0 * 4, 0, 2);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_void_t *)(slot + 1024), 16, voff, k0 * 4 + a_second, 0, 2);
+    };
+    v4f acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+    auto consume = [&](int r, bool refill, int t_next) {
+        const char *slot = ring + r * slot_bytes;
+        const v4f x0 = *reinterpret_cast<const v4f *>(slot + rd0);
+        const v4f x1 = *reinterpret_cast<const v4f *>(slot + rd1);
+        float b[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) b[s] = *reinterpret_cast<const float *>(slot + rdb + (16 * (s >> 2) + (s & 3)) * ldb * 4);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slot has been read: it may be written again
+        if (refill) request(t_next, r);
+#pragma unroll
+        for (int s = 0; s < 8; ++s) b[s] = col_ok ? b[s] : 0.f;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(x0[s], b[s], acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(x1[s], b[4 + s], acc1, 0, 0, 0);
+        }
+    };
+    constexpr int kPer = B2 ? 4 : 3;   // loads per group
+    const int first = T < RING ? T : RING;
+    for (int t = 0; t < first; ++t) request(t, t);
+    int r = 0;
+    for (int t = 0; t + RING < T; ++t) {   // steady state: RING groups in flight, the oldest is waited for
+        wait_vmcnt<(RING - 1) * kPer>();
+        asm volatile("" ::: "memory");
+        consume(r, true, t + RING);
+        r = r + 1 == RING ? 0 : r + 1;
+    }
+    for (int left = first - 1; left >= 0; --left) {   // the last groups: nothing is requested any more
+        if (left >= 2) wait_vmcnt<2 * kPer>();
+        else if (left == 1) wait_vmcnt<kPer>();
+        else wait_vmcnt<0>();
+        asm volatile("" ::: "memory");
+        consume(r, false, 0);
+        r = r + 1 == RING ? 0 : r + 1;
+    }
+    acc0 += acc1;
+    __syncthreads();   // every ring is read out: the partial tiles go over them
+    float(*part)[16][17] = reinterpret_cast<float(*)[16][17]>(lds);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) part[wave][4 * q + v][i] = acc0[v];
+    __syncthreads();
+    if (tid < 256) {
+        const int pr = tid >> 4, c = tid & 15;
+        float s = 0.f;
+        for (int w = 0; w < kStreamWaves; ++w) s += part[w][pr][c];
+        const size_t grow = row0 + pr;
+        if (pr < rows && c < N) {
+            float x = s + (ep.bias ? ep.bias[c] : 0.f);
+            if (ep.relu) x = (x > 0.f) ? x : 0.f;
+            if (softmax) part[0][pr][c] = x;   // (this thread alone read part[.][pr][c])
+            else C[grow * ldc + c] = x;
+        }
+    }
+    if (softmax) {   // as gemm_skinny: one lane per row, the arithmetic of the stand-alone short-row kernel
+        __syncthreads();
+        if (tid < rows) {
+            const float *src = part[0][tid];
+            float *dst = C + (row0 + tid) * ldc;
+            float mx = src[0];
+            for (int j = 1; j < N; ++j) mx = fmaxf(mx, src[j]);
+            float sum = 0.f;
+            for (int j = 0; j < N; ++j) sum += fast_exp(src[j] - mx);
+            const float inv = 1.f / sum;
+            for (int j = 0; j < N; ++j) dst[j] = fast_exp(src[j] - mx) * inv;
+        }
+    }
+#endif
+}
+
+struct StreamArgs {
+    const float *a, *b;
+    float *c;
+    int m, n, k;
+    unsigned lda;
+    int ldb;
+    size_t ldc;
+    Epilogue ep;
+    int softmax;
+    unsigned blocks;
+    size_t lds;
+};
+
+template <int RING, bool B2> int launch_stream(const StreamArgs &x) {
+    auto kern = gemm_skinny_stream<RING, B2>;
+    static bool configured = false;
+    if (!configured) {
+        SWC_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)Device::ldsBytesPerCU));
+        configured = true;
+    }
+    note_kernel("gemm_skinny_stream<%d,%s>", RING, B2 ? "true" : "false");
+    kern<<<x.blocks, 64 * kStreamWaves, x.lds, stream()>>>(x.a, x.b, x.c, x.m, x.n, x.k, x.lda, x.ldb, x.ldc, x.ep, x.softmax);
+    SWC_LAUNCH_CHECK();
+    return SWC_HIP_OK;
+}
+
 // ------------------------------------------------------------ few-rows GEMM
 // M <= 16 (single-sample and small-batch inference) with a B of a few MB: the product is bound by the latency
 // of one pass over B.  A workgroup owns 16 columns of C; its sixteen wavefronts split K into contiguous ranges
@@ -594,6 +765,20 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
         // 19.6 us against 22.0 with eight).
         const int waves = k <= 1024 ? 4 : kSkinnyMaxWaves;
         const unsigned blocks = ceil_div(m, 16);
+        // Long K: the streamed kernel.  It wants whole 16-byte pieces (the vec conditions and a contiguous,
+        // aligned B) and 32-bit byte offsets inside the 16 rows of a workgroup and inside B.
+        const char *skinny = getenv("SWC_HIP_SKINNY");   // test-only: "plain" keeps gemm_skinny for every shape
+        const bool stream_ok = vec && k > 1024 && ldb == n && aligned16(b) && (size_t)lda * 64 < 0x7fff0000u &&
+                               (size_t)k * ldb * 4 < 0x7fff0000u && !(skinny && !strcmp(skinny, "plain"));
+        if (stream_ok) {
+            const int slot = stream_slot_bytes(ldb);
+            const int ring = (size_t)kStreamWaves * 3 * slot <= Device::ldsBytesPerCU ? 3 : 2;
+            const bool b2 = 32 * ldb * 4 > 1024;
+            const size_t lds = (size_t)kStreamWaves * ring * slot;
+            const StreamArgs sa{a, b, c, m, n, k, (unsigned)lda, ldb, (size_t)ldc, ep, softmax, blocks, lds};
+            if (ring == 3) return b2 ? launch_stream<3, true>(sa) : launch_stream<3, false>(sa);
+            return b2 ? launch_stream<2, true>(sa) : launch_stream<2, false>(sa);
+        }
         note_kernel("gemm_skinny<%s>", vec ? "true" : "false");
         if (vec) gemm_skinny<true><<<blocks, 64 * waves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep, softmax);
         else gemm_skinny<false><<<blocks, 64 * waves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep, softmax);

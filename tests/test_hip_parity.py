@@ -521,6 +521,54 @@ def test_fcbias_softmax_fused(rt, oracle, m, k, n):
                      "fused vs sequence, no bias")
 
 
+STREAMED_HEADS = [(4096, 4096, 10), (1000, 4096, 10), (33, 1028, 7), (16, 2048, 16), (257, 1056, 1), (100, 1200, 3),
+                  (17, 5000, 8), (50, 1444, 11), (1, 8192, 16), (130, 2052, 4), (48, 70000, 10)]
+
+
+@pytest.mark.parametrize("m,k,n", STREAMED_HEADS)
+def test_skinny_gemm_streamed_along_k(rt, oracle, m, k, n, monkeypatch):
+    """N <= 16 behind a K above 1024: A and B by LDS-DMA through per-wavefront rings.  Integer-valued operands make the
+    result exact whatever the order of summation, so every k, every row and every column is checked bit by bit (rows
+    and k past the end must come in as zeros, not as whatever the ring held); then real-valued data against the
+    oracle, and the fused softmax against the two calls in sequence, also with the plain kernel."""
+    print("case streamed head", m, k, n, flush=True)
+    rng = np.random.default_rng(m * 7 + k + n)
+    a = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    b = rng.integers(-4, 5, (k, n)).astype(np.float32)
+    bias = rng.integers(-8, 9, n).astype(np.float32)
+    want = (a.astype(np.int64) @ b.astype(np.int64) + bias.astype(np.int64)).astype(np.float32)
+    da, db, dbias = up(rt, a, b, bias)
+    got = rt.fcbias(da, db, dbias, relu=False).numpy()
+    assert rt.last_kernel().startswith("gemm_skinny_stream<"), rt.last_kernel()
+    assert_bit_exact(got, want, f"integer head {m}x{k}x{n}")
+    assert_bit_exact(rt.fcbias(da, db, dbias, relu=True).numpy(), np.maximum(want, 0), "with ReLU")
+    assert_bit_exact(rt.matrixMatrixMul(da, db).numpy(), want - bias, "no bias")
+    # a second call right after one on other data: nothing of the first may be left in the rings
+    a2 = np.where(rng.uniform(size=(m, k)) < 0.5, np.float32(np.inf), np.float32(1)).astype(np.float32)
+    rt.matrixMatrixMul(rt.upload(a2), db)
+    assert_bit_exact(rt.fcbias(da, db, dbias, relu=False).numpy(), want, "after a call full of infinities")
+    # real-valued
+    x = rng.uniform(0, 1, (m, k)).astype(np.float32)
+    w = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32)
+    c = rng.uniform(-0.01, 0.01, n).astype(np.float32)
+    dx, dw, dc = up(rt, x, w, c)
+    ref = oracle.fcbias(x, w, c) if m * k <= (1 << 23) else (x.astype(np.float64) @ w.astype(np.float64) + c).astype(np.float32)
+    assert scaled_err(rt.fcbias(dx, dw, dc).numpy(), ref, np.abs(x) @ np.abs(w) + np.abs(c)) < TOL
+    fused = rt.fcbias(dx, dw, dc, softmax=True).numpy()
+    assert_bit_exact(fused, rt.matrixSoftmax(rt.fcbias(dx, dw, dc)).numpy(), "fused softmax vs sequence")
+    assert np.allclose(fused.sum(axis=1), 1.0, atol=1e-5)
+    # rows of a wider matrix (lda > k)
+    wide = rng.integers(-4, 5, (m, k + 8)).astype(np.float32)
+    dwide, out = rt.upload(wide), rt.empty((m, n))
+    rt._check(rt.lib.swc_hip_matrixMatrixMul_f(m, n, k, dwide.ptr, k + 8, db.ptr, n, out.ptr, n), "matrixMatrixMul_f")
+    assert rt.last_kernel().startswith("gemm_skinny_stream<"), rt.last_kernel()
+    assert_bit_exact(out.numpy(), (wide[:, :k].astype(np.int64) @ b.astype(np.int64)).astype(np.float32), "lda > k")
+    # the plain kernel gives the same integers
+    monkeypatch.setenv("SWC_HIP_SKINNY", "plain")
+    assert_bit_exact(rt.fcbias(da, db, dbias, relu=False).numpy(), want, "plain kernel")
+    assert rt.last_kernel().startswith("gemm_skinny<"), rt.last_kernel()
+
+
 @pytest.mark.parametrize("m,k,n", [(1, 4100, 600), (7, 4096, 1000), (32, 2048, 1000), (32, 1030, 1028), (17, 3000, 404),
                                    (8, 25088, 512), (33, 2048, 1000), (64, 4100, 300), (50, 1111, 1000)])
 def test_gemm_of_up_to_64_rows_and_a_large_b(rt, oracle, m, k, n):
