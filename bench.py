@@ -97,6 +97,9 @@ def _gemm_work(res, a, b, *r, **kw):
 def _conv_work(res, x, f, *r, **kw):
     m = res.size // res.shape[3]
     k = f.shape[1] * f.shape[2] * f.shape[3]
+    if kw.get("pool"):   # the result is the pooled tensor: four convolution pixels per element
+        m *= 4
+        return dict(shape=f"{list(x.shape)}*{list(f.shape)} + maxpool 2x2", flop=2.0 * m * f.shape[0] * k)
     return dict(shape=f"{list(x.shape)}*{list(f.shape)}", flop=2.0 * m * f.shape[0] * k)
 
 
@@ -361,6 +364,8 @@ def bench_workspace(rt, graphs):
              ((32, 28, 28, 128), (128, 3, 3, 128), p1)]
     for xs, fs, pads in convs:
         need = max(need, rt.conv2d_workspace_bytes(xs, fs, (1, 1), pads))
+    for xs, fs, pads in convs[1:2] + convs[3:]:   # the layers that pool in their epilogue
+        need = max(need, rt.conv2d_maxpool_workspace_bytes(xs, fs, (1, 1), pads, ((2, 2), (2, 2))))
     for xs, fs, pads in convs[2:]:
         need = max(need, rt.conv2dGrad_workspace_bytes(xs, fs, (1, 1), pads))
     if not need:

@@ -383,6 +383,34 @@ int swc_hip_conv2dFusedAdd_f(float *output, const float *input, const float *fil
                              const float *bn_bias, float epsilon,
                              const float *residual, int relu);
 
+/* swc_hip_conv2dFused_f followed by maxpool_f (kernels.h:343-383) over its
+ * result, in one call: conv2d_f (kernels.h:177-243), optionally
+ * batchnormalization_f, optionally relu_f, then the pooling.  `cdims` are the
+ * convolution's output dims [N,OH,OW,oC] (that tensor is never stored), `pdims`
+ * the pooled output's [N,PH,PW,oC] = `output`.  For 2x2 windows with stride 2
+ * and no padding over even OH and OW the convolution kernel takes the maximum
+ * in its epilogue — the same bits as the two calls in sequence, one launch and
+ * the convolution's output neither written nor read back; any other pooling
+ * runs the two steps with the intermediate tensor in the workspace.
+ * Workspace: swc_hip_conv2dFusedMaxpool_workspace_bytes. */
+int swc_hip_conv2dFusedMaxpool_f(float *output, const float *input, const float *filter,
+                                 const float *bias, const size_t *cdims,
+                                 const size_t *idims, const size_t *fdims,
+                                 const size_t *bdims, const size_t *kernels,
+                                 const size_t *strides, const size_t *pads,
+                                 size_t group, const float *bn_mean,
+                                 const float *bn_var, const float *bn_scale,
+                                 const float *bn_bias, float epsilon, int relu,
+                                 const size_t *pdims, const size_t *pool_kernels,
+                                 const size_t *pool_strides, const size_t *pool_pads);
+size_t swc_hip_conv2dFusedMaxpool_workspace_bytes(const size_t *cdims, const size_t *idims,
+                                                  const size_t *fdims, const size_t *kernels,
+                                                  const size_t *strides, const size_t *pads,
+                                                  size_t group, const size_t *pdims,
+                                                  const size_t *pool_kernels,
+                                                  const size_t *pool_strides,
+                                                  const size_t *pool_pads);
+
 #ifdef __cplusplus
 }
 #endif

@@ -177,6 +177,110 @@ __global__ __launch_bounds__(kThreads) void conv_igemm(const float *__restrict__
     store_tile<TM, TN>(acc, out, (size_t)N, M, N, m0 + wave_m * 32 * TM, n0 + wave_n * 32 * TN, lane, ep);
 }
 
+// Row m of the GEMM view -> output pixel (see ConvGeom::win).
+__device__ __forceinline__ void pixel_of_row(const ConvGeom &g, int m, int &img, int &oy, int &ox) {
+    if (g.win) {
+        const int w = m >> 2, d = m & 3, pw = g.OW >> 1, ph = g.OH >> 1;
+        const int px = w % pw, t = w / pw;
+        const int py = t % ph;
+        img = t / ph;
+        oy = 2 * py + (d >> 1);
+        ox = 2 * px + (d & 1);
+    } else {
+        ox = m % g.OW;
+        const int t = m / g.OW;
+        oy = t % g.OH;
+        img = t / g.OH;
+    }
+}
+
+// The per-element epilogue of every convolution kernel here: bias, folded batchnorm, second summand, ReLU.
+struct ColumnParams {
+    float bias, mean, slope, beta;
+};
+__device__ __forceinline__ ColumnParams column_params(const Epilogue &ep, int col, bool ok) {
+    ColumnParams c{(ep.bias && ok) ? ep.bias[col] : 0.f, 0.f, 1.f, 0.f};
+    if (ep.bn_mean && ok) {   // slope formed in double and rounded once, as store_tile_impl
+        c.mean = ep.bn_mean[col];
+        c.slope = (float)((double)ep.bn_scale[col] / sqrt((double)(ep.bn_var[col] + ep.eps)));
+        c.beta = ep.bn_bias[col];
+    }
+    return c;
+}
+__device__ __forceinline__ float finish_element(float x, const ColumnParams &c, bool bn, bool relu) {
+    x += c.bias;
+    if (bn) x = fmaf(x - c.mean, c.slope, c.beta);
+    return relu ? ((x > 0.f) ? x : 0.f) : x;
+}
+// maxpool_f's choice among the taps of a window in its order (kernels.h:343-383: the first, then whatever is greater)
+__device__ __forceinline__ float window_max(float a, float b, float c, float d) {
+    float best = a;
+    if (b > best) best = b;
+    if (c > best) best = c;
+    if (d > best) best = d;
+    return best;
+}
+
+// A wavefront's 32 TM x 32 TN part of a tile whose rows are in window order (ConvGeom::win).  The four rows that a
+// lane holds in accumulator registers 4g .. 4g + 3 are the four pixels of one window.
+//   POOL == false: each goes to its own pixel of the [N, OH, OW, OC] output (the arithmetic of store_tile_impl);
+//   POOL == true:  the epilogue of each, then their maximum to the window's place in the [N, OH/2, OW/2, OC] output.
+// M is a multiple of 4 here, so a window is wholly inside or outside.
+template <int TM, int TN, bool POOL>
+__device__ __forceinline__ void store_tile_windows(const v16f (&acc)[TM][TN], float *__restrict__ out, const ConvGeom &g,
+                                                   int row0, int col0, int lane, const Epilogue &ep) {
+    const int l32 = lane & 31, h = lane >> 5;
+    const int N = g.OC, pw = g.OW >> 1, ph = g.OH >> 1;
+    const bool bn = ep.bn_mean != nullptr;
+    ColumnParams cp[TN];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) cp[tn] = column_params(ep, col0 + tn * 32 + l32, col0 + tn * 32 + l32 < N);
+    // this lane's windows: w0, w0 + 2, w0 + 4, ... (rows row0 + 4h + 8 * (g + 4 tm))
+    int w = (row0 >> 2) + h;
+    int px = w % pw, t = w / pw;
+    int py = t % ph, img = t / ph;
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (4 * w < g.M) {
+                const size_t pix = ((size_t)(img * g.OH + 2 * py) * g.OW + 2 * px);
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn) {
+                    const int col = col0 + tn * 32 + l32;
+                    if (col >= N) continue;
+                    float x[4];
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        x[d] = acc[tm][tn][4 * q + d] + cp[tn].bias;
+                        if (bn) x[d] = fmaf(x[d] - cp[tn].mean, cp[tn].slope, cp[tn].beta);
+                    }
+                    if (ep.residual) {
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) x[d] += ep.residual[(pix + (d >> 1) * g.OW + (d & 1)) * N + col];
+                    }
+                    if (ep.relu) {
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) x[d] = (x[d] > 0.f) ? x[d] : 0.f;
+                    }
+                    if (POOL) {
+                        out[(size_t)w * N + col] = window_max(x[0], x[1], x[2], x[3]);
+                    } else {
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) out[(pix + (d >> 1) * g.OW + (d & 1)) * N + col] = x[d];
+                    }
+                }
+            }
+            w += 2;
+            px += 2;
+            while (px >= pw) {
+                px -= pw;
+                if (++py == ph) py = 0, ++img;
+            }
+        }
+    }
+}
+
 // Direct-to-LDS variant (mfma_dma.hpp): the im2col gather is expressed as one
 // 32-bit byte offset per lane per load — out-of-image taps and rows past M get
 // the out-of-range offset and arrive in LDS as zeros.  Needs iC % 4 == 0,
@@ -216,7 +320,7 @@ template <int TM, int TN, int STAGES, bool MID = false>
 __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ in, const float *__restrict__ filt,
                                                      float *__restrict__ out, ConvGeom g, unsigned in_bytes,
                                                      unsigned filt_bytes, Epilogue ep, SkPlan sk,
-                                                     float *__restrict__ part) {
+                                                     float *__restrict__ part, int pool) {
 #if __HIP_DEVICE_COMPILE__   // the host pass only needs the launch stub
     using T = DmaTile<TM, TN, true, STAGES>;
     extern __shared__ __align__(16) float lds[];
@@ -261,10 +365,8 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
         for (int j = 0; j < T::kALoads; ++j) {
             const int m = m0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
             if (m < M) {
-                const int ox = m % g.OW;
-                const int t = m / g.OW;
-                const int oy = t % g.OH;
-                const int img = t / g.OH;
+                int img, oy, ox;
+                pixel_of_row(g, m, img, oy, ox);
                 iy0[j] = oy * g.sh - g.pt;
                 ix0[j] = ox * g.sw - g.pl;
                 row_off[j] = ((img * g.H + iy0[j]) * g.W + ix0[j]) * g.C;
@@ -358,7 +460,10 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
         wait_vmcnt<0>();   // the trailing dummy loads still target this workgroup's LDS
         acc_settle(acc);
         if (whole) {
-            store_tile<TM, TN>(acc, out, (size_t)N, M, N, m0 + (wave >> 1) * 32 * TM, n0 + (wave & 1) * 32 * TN, lane, ep);
+            const int row0 = m0 + (wave >> 1) * 32 * TM, col0 = n0 + (wave & 1) * 32 * TN;
+            if (!g.win) store_tile<TM, TN>(acc, out, (size_t)N, M, N, row0, col0, lane, ep);
+            else if (pool) store_tile_windows<TM, TN, true>(acc, out, g, row0, col0, lane, ep);
+            else store_tile_windows<TM, TN, false>(acc, out, g, row0, col0, lane, ep);
         } else {
             float *slot = part + (size_t)(2 * share + (piece ? 1 : 0)) * (T::BM * T::BN);
             store_tile_impl<TM, TN, false, false>(acc, slot, (size_t)T::BN, T::BM, T::BN, (wave >> 1) * 32 * TM,
@@ -369,10 +474,12 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
 }
 
 // Adds the pieces of every shared tile that more than one workgroup worked on (see conv_dma) in K order and
-// applies the epilogue.  blockIdx.x = shared tile, blockIdx.y = block of 16 rows of it.
+// applies the epilogue.  blockIdx.x = shared tile, blockIdx.y = block of 16 rows of it.  With `pool` (rows in window
+// order) the finished values of a window's four rows meet in LDS and their maximum is stored.
 template <int BM, int BN>
-__global__ __launch_bounds__(256) void conv_sk_finish(float *__restrict__ out, const float *__restrict__ part, int M,
-                                                      int N, int nk, SkPlan sk, Epilogue ep, int vec_ok) {
+__global__ __launch_bounds__(256) void conv_sk_finish(float *__restrict__ out, const float *__restrict__ part, ConvGeom g,
+                                                      int nk, SkPlan sk, Epilogue ep, int vec_ok, int pool) {
+    const int M = g.M, N = g.OC;
     const int t = blockIdx.x;
     const int first = t * nk, last = first + nk - 1;   // this tile's units, counted from the first shared unit
     const int big = sk.r * (sk.q + 1);                 // units held by the shares of q + 1
@@ -382,11 +489,8 @@ __global__ __launch_bounds__(256) void conv_sk_finish(float *__restrict__ out, c
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     int tile_m, tile_n;
     sk_tile_coords(sk.dp_tiles + t, sk.dp_tiles, tiles_m, tiles_n, tile_m, tile_n);
-    constexpr int kQuads = 16 * BN / 4;   // float4s in a block of 16 rows
-    for (int i = threadIdx.x; i < kQuads; i += 256) {
-        const int r = blockIdx.y * 16 + i / (BN / 4), c = (i % (BN / 4)) * 4;
-        const int row = tile_m * BM + r, col = tile_n * BN + c;
-        if (row >= M || col >= N) continue;
+    // the sum over the pieces of columns c .. c + 3 of row r of the tile
+    auto sum_pieces = [&](int r, int c) {
         float4 sum = {0.f, 0.f, 0.f, 0.f};
         for (int s0 = s_lo; s0 <= s_hi; s0 += 4) {   // four pieces' loads in flight, added in K order
             float4 v[4];
@@ -401,25 +505,73 @@ __global__ __launch_bounds__(256) void conv_sk_finish(float *__restrict__ out, c
             for (int i = 0; i < 4; ++i)
                 if (s0 + i <= s_hi) sum.x += v[i].x, sum.y += v[i].y, sum.z += v[i].z, sum.w += v[i].w;
         }
-        float x[4] = {sum.x, sum.y, sum.z, sum.w};
+        return sum;
+    };
+    // the epilogue of store_tile_impl on the four columns; `pix` = the row's pixel in the output
+    auto finish = [&](float4 sum, int col, size_t pix, float (&x)[4]) {
+        x[0] = sum.x, x[1] = sum.y, x[2] = sum.z, x[3] = sum.w;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            if (col + e >= N) break;   // same arithmetic as store_tile_impl
+            if (col + e >= N) break;
             float y = x[e] + (ep.bias ? ep.bias[col + e] : 0.f);
             if (ep.bn_mean) {
                 const float ve = ep.bn_var[col + e] + ep.eps;
                 const float slope = (float)((double)ep.bn_scale[col + e] / sqrt((double)ve));
                 y = fmaf(y - ep.bn_mean[col + e], slope, ep.bn_bias[col + e]);
             }
-            if (ep.residual) y += ep.residual[(size_t)row * N + col + e];
+            if (ep.residual) y += ep.residual[pix * N + col + e];
             if (ep.relu) y = (y > 0.f) ? y : 0.f;
             x[e] = y;
         }
-        float *dst = out + (size_t)row * N + col;
+    };
+    auto pixel = [&](int row) -> size_t {
+        if (!g.win) return (size_t)row;
+        int img, oy, ox;
+        pixel_of_row(g, row, img, oy, ox);
+        return ((size_t)img * g.OH + oy) * g.OW + ox;
+    };
+    auto store4 = [&](float *dst, int col, const float (&x)[4]) {
         if (vec_ok && col + 3 < N) {
             *reinterpret_cast<float4 *>(dst) = make_float4(x[0], x[1], x[2], x[3]);
         } else {
             for (int e = 0; e < 4 && col + e < N; ++e) dst[e] = x[e];
+        }
+    };
+    if (!pool) {
+        constexpr int kQuads = 16 * BN / 4;   // float4s in a block of 16 rows
+        for (int i = threadIdx.x; i < kQuads; i += 256) {
+            const int r = blockIdx.y * 16 + i / (BN / 4), c = (i % (BN / 4)) * 4;
+            const int row = tile_m * BM + r, col = tile_n * BN + c;
+            if (row >= M || col >= N) continue;
+            const size_t pix = pixel(row);
+            float x[4];
+            finish(sum_pieces(r, c), col, pix, x);
+            store4(out + pix * N + col, col, x);
+        }
+    } else {
+        // every thread finishes one row x four columns as above, into LDS; then the four rows of each window meet
+        __shared__ float done[16][BN];
+        constexpr int kQuads = 16 * BN / 4;
+        for (int i = threadIdx.x; i < kQuads; i += 256) {
+            const int rl = i / (BN / 4), c = (i % (BN / 4)) * 4;
+            const int r = blockIdx.y * 16 + rl;
+            const int row = tile_m * BM + r, col = tile_n * BN + c;
+            if (row >= M || col >= N) continue;
+            float x[4];
+            finish(sum_pieces(r, c), col, pixel(row), x);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) done[rl][c + e] = x[e];
+        }
+        __syncthreads();
+        constexpr int kWindowQuads = 4 * BN / 4;
+        for (int i = threadIdx.x; i < kWindowQuads; i += 256) {
+            const int rl = 4 * (i / (BN / 4)), c = (i % (BN / 4)) * 4;
+            const int row = tile_m * BM + blockIdx.y * 16 + rl, col = tile_n * BN + c;
+            if (row >= M || col >= N) continue;
+            float best[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) best[e] = window_max(done[rl][c + e], done[rl + 1][c + e], done[rl + 2][c + e], done[rl + 3][c + e]);
+            store4(out + (size_t)(row >> 2) * N + col, col, best);
         }
     }
 }
@@ -501,19 +653,20 @@ size_t conv_dma_scratch_bytes(const ConvGeom &g) {
 // `scratch` (may be null) receives the pieces of shared tiles; without it every tile is computed whole.
 template <int TM, int TN, int STAGES, bool MID = false>
 int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGeom &g, size_t in_bytes,
-                    size_t filt_bytes, const Epilogue &ep, float *scratch = nullptr) {
+                    size_t filt_bytes, const Epilogue &ep, float *scratch = nullptr, bool pool = false) {
     using T = DmaTile<TM, TN, true, STAGES>;
     const long tiles = (long)((g.M + T::BM - 1) / T::BM) * ((g.OC + T::BN - 1) / T::BN);
     const int nk = (g.K + BK - 1) / BK;
     const SkPlan p = conv_dma_plan<TM, TN, STAGES, MID>(g, scratch != nullptr);
-    note_kernel("conv_dma<%d,%d,%d,%s>%s", TM, TN, STAGES, MID ? "true" : "false", p.sk_wgs ? " + conv_sk_finish" : "");
+    note_kernel("conv_dma<%d,%d,%d,%s>%s%s", TM, TN, STAGES, MID ? "true" : "false", p.sk_wgs ? " + conv_sk_finish" : "",
+                pool ? " (pooled)" : "");
     auto kern = conv_dma<TM, TN, STAGES, MID>;
-    kern<<<(unsigned)(p.dp_tiles + p.sk_wgs), kThreads, T::kLdsBytes, stream()>>>(in, filt, out, g, (unsigned)in_bytes,
-                                                                                  (unsigned)filt_bytes, ep, p, scratch);
+    kern<<<(unsigned)(p.dp_tiles + p.sk_wgs), kThreads, T::kLdsBytes, stream()>>>(
+        in, filt, out, g, (unsigned)in_bytes, (unsigned)filt_bytes, ep, p, scratch, pool ? 1 : 0);
     SWC_LAUNCH_CHECK();
     if (p.sk_wgs) {
         conv_sk_finish<T::BM, T::BN><<<dim3((unsigned)(tiles - p.dp_tiles), T::BM / 16), 256, 0, stream()>>>(
-            out, scratch, g.M, g.OC, nk, p, ep, (g.OC % 4 == 0 && aligned16(out)) ? 1 : 0);
+            out, scratch, g, nk, p, ep, (g.OC % 4 == 0 && aligned16(out)) ? 1 : 0, pool ? 1 : 0);
         SWC_LAUNCH_CHECK();
     }
     return SWC_HIP_OK;
@@ -912,6 +1065,34 @@ size_t conv_total_scratch(const ConvGeom &g, const void *input, const void *filt
            conv_scratch_bytes(with_channels(g, cp), nullptr, nullptr);
 }
 
+// Rows of the GEMM view in 2 x 2 window order (ConvGeom::win) wherever the output has whole windows: a pooled
+// convolution needs it, and the plain one takes the same order so that the two put every pixel into the same tile
+// and add its products in the same sequence — the pooled result is then bit for bit the maximum of the plain one's.
+// SWC_HIP_CONV_ORDER=raster (test-only) keeps raster order.
+bool window_order(const ConvGeom &g) {
+    const char *e = getenv("SWC_HIP_CONV_ORDER");
+    return g.OH % 2 == 0 && g.OW % 2 == 0 && g.OH > 0 && g.OW > 0 && !(e && !strcmp(e, "raster"));
+}
+
+// Whether conv_dispatch would run this layer on the direct-to-LDS tile kernels, the ones that can pool in their
+// epilogue (the same tests in the same order as conv_dispatch).
+bool conv_pool_fusable(ConvGeom g, const void *input, const void *filter, const void *output) {
+    const char *force = getenv("SWC_HIP_CONV");
+    if (!window_order(g)) return false;
+    if (force && !strncmp(force, "reg", 3)) return false;
+    bool forced_dma = false;
+    if (force)
+        for (int v = 0; v < kVariants; ++v) forced_dma |= !strcmp(force, kDmaVariantName[v]);
+    if (!forced_dma && g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0) return false;
+    if (const int cp = padded_channels(g, force)) {
+        g = with_channels(g, cp);
+        input = filter = nullptr;   // the padded copies are aligned
+    }
+    strip::Plan sp;
+    if (takes_strip(g, input, filter, output, nullptr, sp)) return false;
+    return conv_uses_dma(g, input, filter, force);
+}
+
 int check_conv_dims(const char *who, const size_t *odims, const size_t *idims, const size_t *fdims,
                     const size_t *kernels, const size_t *strides, const size_t *pads, size_t group,
                     bool groups_ok = false) {
@@ -948,9 +1129,13 @@ ConvGeom make_geom(const size_t *odims, const size_t *idims, const size_t *fdims
 int conv_dispatch(const char *who, float *output, const float *input, const float *filter, const float *bias,
                   const size_t *odims, const size_t *idims, const size_t *fdims, const size_t *kernels,
                   const size_t *strides, const size_t *pads, size_t group, const Epilogue &ep_in,
-                  bool bias_optional = false, ConvScratch scratch = {nullptr, 0}) {
+                  bool bias_optional = false, ConvScratch scratch = {nullptr, 0}, bool pooled = false) {
+    // pooled: `output` is the [N, OH/2, OW/2, OC] result of a 2 x 2 / stride 2 max-pooling of the convolution, and
+    // the caller has made sure (conv_pool_fusable) that the layer runs on the direct-to-LDS tile kernels
     if (int rc = check_conv_dims(who, odims, idims, fdims, kernels, strides, pads, group, true)) return rc;
-    const ConvGeom g = make_geom(odims, idims, fdims, kernels, strides, pads);
+    ConvGeom g = make_geom(odims, idims, fdims, kernels, strides, pads);
+    g.win = window_order(g) ? 1 : 0;
+    const auto not_pooled = [&]() { return fail(SWC_HIP_EUNSUPPORTED, "%s: this kernel does not pool (internal error)", who); };
     const size_t M = (size_t)g.M;
     if (M == 0 || odims[3] == 0) return SWC_HIP_OK;
     if (!output || !input || !filter || (!bias && !bias_optional)) return fail(SWC_HIP_EINVAL, "%s: null pointer", who);
@@ -969,7 +1154,7 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
                                                                                  (int)group);
         SWC_LAUNCH_CHECK();
         return conv_dispatch(who, output, input, masked, bias, odims, idims, fdims, kernels, strides, pads, 1, ep_in,
-                             bias_optional, ConvScratch{reinterpret_cast<float *>(base + f_b), need - f_b});
+                             bias_optional, ConvScratch{reinterpret_cast<float *>(base + f_b), need - f_b}, pooled);
     }
     Epilogue ep = ep_in;
     ep.bias = bias;
@@ -977,6 +1162,7 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
     const size_t M_in = idims[0] * idims[1] * idims[2];
     const size_t in_bytes = M_in * idims[3] * 4, filt_bytes = odims[3] * (size_t)g.K * 4;
     const char *force = getenv("SWC_HIP_CONV");   // forces a kernel variant (tests, tuning): reg22 reg21 reg12 reg11 | 22_2 21_3 12_3 11_3 11_4 | 11_3m 21_3m 12_3m 22_3m (m: ring hand-over in mid-slice)
+    if (force && pooled && !strncmp(force, "reg", 3)) return not_pooled();
     if (force) {
         if (!strcmp(force, "reg22")) return launch_conv<2, 2>(vec, input, filter, output, g, ep);
         if (!strcmp(force, "reg21")) return launch_conv<2, 1>(vec, input, filter, output, g, ep);
@@ -987,7 +1173,7 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
     if (force)
         for (int v = 0; v < kVariants; ++v) forced_dma |= !strcmp(force, kDmaVariantName[v]);
     if (!forced_dma && !(force && !strncmp(force, "reg", 3)) && g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0)
-        return launch_conv_direct(input, filter, bias, output, g, ep);
+        return pooled ? not_pooled() : launch_conv_direct(input, filter, bias, output, g, ep);
     if (const int cp = forced_dma || !(force && !strncmp(force, "reg", 3)) ? padded_channels(g, force) : 0) {
         // zero-padded copies of input and filter, then the same convolution with a channel count of cp
         const size_t in_b = align256(M_in * cp * 4), f_b = align256((size_t)g.OC * g.kh * g.kw * cp * 4);
@@ -1008,14 +1194,16 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
             const size_t p_idims[4] = {idims[0], idims[1], idims[2], (size_t)cp};
             const size_t p_fdims[4] = {fdims[0], fdims[1], fdims[2], (size_t)cp};
             return conv_dispatch(who, output, in_p, f_p, bias, odims, p_idims, p_fdims, kernels, strides, pads, group, ep_in,
-                                 bias_optional, ConvScratch{reinterpret_cast<float *>(base + in_b + f_b), need - in_b - f_b});
+                                 bias_optional, ConvScratch{reinterpret_cast<float *>(base + in_b + f_b), need - in_b - f_b},
+                                 pooled);
         }
     }
     // Whole rows per workgroup where the planner finds an even division ("strip" forces it wherever a plan exists,
     // any other forced variant rules it out)
     {
         strip::Plan sp;
-        if (takes_strip(g, input, filter, output, ep.residual, sp)) return launch_conv_strip(input, filter, output, g, sp, ep);
+        if (takes_strip(g, input, filter, output, ep.residual, sp))
+            return pooled ? not_pooled() : launch_conv_strip(input, filter, output, g, sp, ep);
     }
     if (conv_uses_dma(g, input, filter, force)) {
         // the pieces of shared tiles go into the caller's region when it gave one (and none are made if that
@@ -1034,9 +1222,10 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
             }
         }
         return with_dma_variant(pick_dma_variant(g, force, shared), [&]<int TM, int TN, int STAGES, bool MID>() {
-            return launch_conv_dma<TM, TN, STAGES, MID>(input, filter, output, g, in_bytes, filt_bytes, ep, pieces);
+            return launch_conv_dma<TM, TN, STAGES, MID>(input, filter, output, g, in_bytes, filt_bytes, ep, pieces, pooled);
         });
     }
+    if (pooled) return not_pooled();
     const long tiles_m128 = (M + 127) / 128;
     if (g.OC > 64 && tiles_m128 * ((g.OC + 127) / 128) >= num_cus())
         return launch_conv<2, 2>(vec, input, filter, output, g, ep);
@@ -1686,6 +1875,73 @@ int swc_hip_conv2dFusedAdd_f(float *output, const float *input, const float *fil
     Epilogue ep{nullptr, bn_mean, bn_var, bn_scale, bn_bias, epsilon, relu, residual};
     return conv_dispatch("swc_hip_conv2dFusedAdd_f", output, input, filter, bias, odims, idims, fdims, kernels, strides,
                          pads, group, ep);
+}
+
+// ---- convolution (+ batchnorm) (+ ReLU) + max-pooling in one call
+namespace {
+
+// The pooling the tile kernels can do in their epilogue: 2 x 2 windows, stride 2, no padding, over an output with
+// whole windows only.
+bool pool_is_2x2(const size_t *cdims, const size_t *pdims, const size_t *pk, const size_t *ps, const size_t *pp) {
+    return pk[0] == 2 && pk[1] == 2 && ps[0] == 2 && ps[1] == 2 && pp[0] == 0 && pp[1] == 0 && cdims[1] % 2 == 0 &&
+           cdims[2] % 2 == 0 && pdims[1] == cdims[1] / 2 && pdims[2] == cdims[2] / 2;
+}
+
+int check_pool_after_conv(const char *who, const size_t *cdims, const size_t *pdims, const size_t *pk, const size_t *ps,
+                          const size_t *pp) {
+    if (!pdims || !pk || !ps || !pp) return fail(SWC_HIP_EINVAL, "%s: null shape array", who);
+    if (pdims[0] != cdims[0] || pdims[3] != cdims[3])
+        return fail(SWC_HIP_EINVAL, "%s: pooled batch/channels differ from the convolution's", who);
+    return SWC_HIP_OK;
+}
+
+} // namespace
+
+size_t swc_hip_conv2dFusedMaxpool_workspace_bytes(const size_t *cdims, const size_t *idims, const size_t *fdims,
+                                                  const size_t *kernels, const size_t *strides, const size_t *pads,
+                                                  size_t group, const size_t *pdims, const size_t *pool_kernels,
+                                                  const size_t *pool_strides, const size_t *pool_pads) {
+    const char *who = "swc_hip_conv2dFusedMaxpool_workspace_bytes";
+    if (!ready() || check_conv_dims(who, cdims, idims, fdims, kernels, strides, pads, group, true) ||
+        check_pool_after_conv(who, cdims, pdims, pool_kernels, pool_strides, pool_pads))
+        return 0;
+    const size_t conv = swc_hip_conv2d_workspace_bytes(cdims, idims, fdims, kernels, strides, pads, group);
+    const ConvGeom g = make_geom(cdims, idims, fdims, kernels, strides, pads);
+    if (g.M == 0 || g.OC == 0) return 0;
+    if (pool_is_2x2(cdims, pdims, pool_kernels, pool_strides, pool_pads) && conv_pool_fusable(g, nullptr, nullptr, nullptr))
+        return conv;
+    return align256((size_t)g.M * g.OC * 4) + conv;   // the convolution's own output, then pooled by maxpool_f's kernel
+}
+
+int swc_hip_conv2dFusedMaxpool_f(float *output, const float *input, const float *filter, const float *bias,
+                                 const size_t *cdims, const size_t *idims, const size_t *fdims, const size_t *bdims,
+                                 const size_t *kernels, const size_t *strides, const size_t *pads, size_t group,
+                                 const float *bn_mean, const float *bn_var, const float *bn_scale, const float *bn_bias,
+                                 float epsilon, int relu, const size_t *pdims, const size_t *pool_kernels,
+                                 const size_t *pool_strides, const size_t *pool_pads) {
+    SWC_REQUIRE_INIT();
+    (void)bdims;
+    const char *who = "swc_hip_conv2dFusedMaxpool_f";
+    if (bn_mean || bn_var || bn_scale || bn_bias)
+        SWC_ARG(bn_mean && bn_var && bn_scale && bn_bias);
+    if (int rc = check_conv_dims(who, cdims, idims, fdims, kernels, strides, pads, group, true)) return rc;
+    if (int rc = check_pool_after_conv(who, cdims, pdims, pool_kernels, pool_strides, pool_pads)) return rc;
+    Epilogue ep{nullptr, bn_mean, bn_var, bn_scale, bn_bias, epsilon, relu};
+    const ConvGeom g = make_geom(cdims, idims, fdims, kernels, strides, pads);
+    if (g.M == 0 || g.OC == 0) return SWC_HIP_OK;
+    if (pool_is_2x2(cdims, pdims, pool_kernels, pool_strides, pool_pads) && conv_pool_fusable(g, input, filter, output))
+        return conv_dispatch(who, output, input, filter, bias, cdims, idims, fdims, kernels, strides, pads, group, ep, false,
+                             ConvScratch{nullptr, 0}, true);
+    // any other pooling, or a layer for another kernel: the two steps, the convolution's output in the workspace
+    const size_t inter = align256((size_t)g.M * g.OC * 4);
+    const size_t need = inter + swc_hip_conv2d_workspace_bytes(cdims, idims, fdims, kernels, strides, pads, group);
+    char *base = static_cast<char *>(workspace(need, who));
+    if (!base) return fail_code();
+    float *conv_out = reinterpret_cast<float *>(base);
+    if (int rc = conv_dispatch(who, conv_out, input, filter, bias, cdims, idims, fdims, kernels, strides, pads, group, ep,
+                               false, ConvScratch{reinterpret_cast<float *>(base + inter), need - inter}))
+        return rc;
+    return swc_hip_maxpool_f(conv_out, output, cdims, pdims, pool_kernels, pool_strides, pool_pads);
 }
 
 size_t swc_hip_conv2d_workspace_bytes(const size_t *odims, const size_t *idims, const size_t *fdims,

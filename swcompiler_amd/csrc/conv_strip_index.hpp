@@ -43,6 +43,11 @@ struct ConvGeom {
     int OH, OW, OC;      // output
     int kh, kw, sh, sw, pt, pl;
     int M, K;            // GEMM view: output pixels, kh*kw*C
+    // Order in which the rows of the GEMM view walk the output pixels.  0: raster order (image, row, column).
+    // 1: by 2 x 2 windows — row m is pixel (2py + d/2, 2px + d%2) of window m/4 = (image, py, px) in raster order
+    // of the windows, d = m%4 — so that every aligned group of four rows is one window of a 2 x 2 / stride 2
+    // pooling (even OH and OW only).
+    int win = 0;
 };
 
 namespace strip {

@@ -7,8 +7,9 @@ checker on numpy arrays.  `unfused` sequences are call-for-call what the
 reference's code generator emits for the graph (FCBias lowered to
 matrixMatrixMul + batchedadd, src/op/dlOp/dlOpEinsum.cpp:154-237; one call per
 op node in topological order, src/codegen/Codegen.cpp:1035-1060).  `fused`
-sequences are what the HIP target emits: bias/BN/ReLU folded into the GEMM or
-conv epilogue and BN+ReLU(+pool) into one pass.
+sequences are what the HIP target emits: bias/BN/ReLU (and a 2x2 max-pooling
+behind them) folded into the GEMM or conv epilogue and BN+ReLU(+pool) into one
+pass.
 
 Activations are NHWC and conv filters [oC,kH,kW,iC] (the reference's layout,
 src/tensor/tensor.h:96-98); the "NCHW" shapes quoted for the configurations
@@ -126,6 +127,9 @@ def run(cfg, be, t, fused=False, ws=None):
     if cfg == 3:
         h = t["x"]
         for i in (1, 2):
+            if fused and i == 2:   # 20 input channels: a layer of the tile kernels, which pool in their epilogue
+                h = w(f"c{i}", be.conv2d, h, t[f"f{i}"], t[f"cb{i}"], relu=True, pool=((2, 2), (2, 2)))
+                continue
             if fused:
                 h = w(f"c{i}", be.conv2d, h, t[f"f{i}"], t[f"cb{i}"], relu=True)
             else:
@@ -139,6 +143,10 @@ def run(cfg, be, t, fused=False, ws=None):
         h = t["x"]
         for i in (1, 2, 3, 4):
             bn = _bn(t, f"bn{i}")
+            if fused and i in (2, 4):   # the pooling in the convolution's epilogue
+                h = w(f"c{i}", be.conv2d, h, t[f"f{i}"], t[f"cb{i}"], pads=(1, 1, 1, 1), bn=bn, eps=EPS, relu=True,
+                      pool=((2, 2), (2, 2)))
+                continue
             if fused:
                 h = w(f"c{i}", be.conv2d, h, t[f"f{i}"], t[f"cb{i}"], pads=(1, 1, 1, 1), bn=bn, eps=EPS, relu=True)
             else:

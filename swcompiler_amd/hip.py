@@ -29,6 +29,7 @@ EXPORTS = [
     "swc_hip_matrixSoftmax_f", "swc_hip_matrixTanh_f", "swc_hip_argMax_i", "swc_hip_accuracy_i", "swc_hip_fill_i",
     "swc_hip_matrixMatrixFCBias_f", "swc_hip_vecAddRelu_f", "swc_hip_batchnormRelu_f",
     "swc_hip_batchnormReluMaxpool_f", "swc_hip_conv2dFused_f", "swc_hip_conv2dFusedAdd_f",
+    "swc_hip_conv2dFusedMaxpool_f", "swc_hip_conv2dFusedMaxpool_workspace_bytes",
     "swc_hip_set_workspace", "swc_hip_matrixMatrixFCBiasSoftmax_f", "swc_hip_gemm_workspace_bytes", "swc_hip_conv2d_workspace_bytes", "swc_hip_host_malloc", "swc_hip_host_free", "swc_hip_matrixTrans_f", "swc_hip_matrixTanhGrad_f", "swc_hip_matrixSoftmaxWithLoss_f",
     "swc_hip_matrixSoftmaxGrad_f", "swc_hip_matrixSoftmaxWithLossGrad_f", "swc_hip_conv2dGrad_f",
     "swc_hip_maxpoolGrad_f", "swc_hip_batchedreduceadd_f", "swc_hip_sgd_f", "swc_hip_reluGrad_f",
@@ -110,6 +111,9 @@ def load_library():
                                         vp, vp, vp, vp, f32, i32]),
         "swc_hip_conv2dFusedAdd_f": (i32, [vp, vp, vp, vp, szp, szp, szp, szp, szp, szp, szp, sz,
                                         vp, vp, vp, vp, f32, vp, i32]),
+        "swc_hip_conv2dFusedMaxpool_f": (i32, [vp, vp, vp, vp, szp, szp, szp, szp, szp, szp, szp, sz,
+                                            vp, vp, vp, vp, f32, i32, szp, szp, szp, szp]),
+        "swc_hip_conv2dFusedMaxpool_workspace_bytes": (sz, [szp] * 6 + [sz] + [szp] * 4),
         "swc_hip_set_workspace": (i32, [vp, sz]),
         "swc_hip_host_malloc": (vp, [sz]),
         "swc_hip_host_free": (i32, [vp]),
@@ -414,12 +418,25 @@ class SwcHip:
         return t
 
     def conv2d(self, x, filt, bias, kernels=None, strides=(1, 1), pads=(0, 0, 0, 0), group=1, bn=None,
-               eps=1e-5, relu=False, out=None, residual=None):
-        """bn = (mean, var, scale, bias) DeviceArrays to fuse inference batchnorm."""
+               eps=1e-5, relu=False, out=None, residual=None, pool=None):
+        """bn = (mean, var, scale, bias) DeviceArrays to fuse inference batchnorm; pool = (kernels, strides[, pads])
+        to max-pool the result in the same call (the result is then the pooled tensor)."""
         if kernels is None:
             kernels = filt.shape[1:3]
         n, oh, ow, _ = pool_out_dims(x.shape, kernels, strides, pads)
         odims = (n, oh, ow, filt.shape[0])
+        if pool is not None:
+            assert residual is None
+            pk, ps = pool[0], pool[1]
+            pp = pool[2] if len(pool) > 2 else (0, 0, 0, 0)
+            pdims = pool_out_dims(odims, pk, ps, pp)
+            out = out if out is not None else self.empty(pdims)
+            ptrs = [p.ptr for p in bn] if bn is not None else [None] * 4
+            self._check(self.lib.swc_hip_conv2dFusedMaxpool_f(
+                out.ptr, x.ptr, filt.ptr, bias.ptr, _dims(odims), _dims(x.shape), _dims(filt.shape), _dims(bias.shape),
+                _dims(kernels), _dims(strides), _dims(pads), group, *ptrs, eps, int(relu), _dims(pdims), _dims(pk),
+                _dims(ps), _dims(pp)), "conv2dFusedMaxpool_f")
+            return out
         out = out if out is not None else self.empty(odims)
         shp = (_dims(odims), _dims(x.shape), _dims(filt.shape), _dims(bias.shape), _dims(kernels),
                _dims(strides), _dims(pads))
@@ -561,6 +578,16 @@ class SwcHip:
     def gemm_workspace_bytes(self, m, n, k):
         """scratch bytes an m x n x k FC/GEMM call uses on this device (0 unless it is split over K)"""
         return int(self.lib.swc_hip_gemm_workspace_bytes(m, n, k))
+
+    def conv2d_maxpool_workspace_bytes(self, xshape, fshape, strides, pads, pool, group=1):
+        n, oh, ow, _ = pool_out_dims(xshape, fshape[1:3], strides, pads)
+        odims = (n, oh, ow, fshape[0])
+        pk, ps = pool[0], pool[1]
+        pp = pool[2] if len(pool) > 2 else (0, 0, 0, 0)
+        pdims = pool_out_dims(odims, pk, ps, pp)
+        return int(self.lib.swc_hip_conv2dFusedMaxpool_workspace_bytes(
+            _dims(odims), _dims(xshape), _dims(fshape), _dims(fshape[1:3]), _dims(strides), _dims(pads), group, _dims(pdims),
+            _dims(pk), _dims(ps), _dims(pp)))
 
     def conv2d_workspace_bytes(self, xshape, fshape, strides=(1, 1), pads=(0, 0, 0, 0), group=1):
         """scratch bytes a conv2d call of these shapes uses on this device (0 if every tile is computed whole)"""

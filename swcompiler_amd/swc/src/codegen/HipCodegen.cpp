@@ -90,6 +90,16 @@ void HipCodegen::emitWorkspace() {
               << arrayDef("k", conv->getKernels()) << arrayDef("s", conv->getStrides()) << arrayDef("p", conv->getPads())
               << "gpu0_ws_bytes = std::max(gpu0_ws_bytes, swc_hip_conv2d_workspace_bytes(o, i, f, k, s, p, "
               << conv->getGroup() << "));\n}\n";
+        } else if (type == "Conv2dMaxPool") {
+            auto *conv = static_cast<Conv2dMaxPoolOp *>(op->getOp());
+            Tensor *y = static_cast<TensorNode *>(op->getChildNode(0))->getTensor();
+            q << "{\n"
+              << arrayDef("o", conv->convOutDims(T(0)->getDims(), T(1)->getDim(0))) << arrayDef("i", T(0)->getDims())
+              << arrayDef("f", T(1)->getDims()) << arrayDef("k", conv->getKernels()) << arrayDef("s", conv->getStrides())
+              << arrayDef("p", conv->getPads()) << arrayDef("po", y->getDims()) << arrayDef("pk", conv->getPoolKernels())
+              << arrayDef("ps", conv->getPoolStrides()) << arrayDef("pp", conv->getPoolPads())
+              << "gpu0_ws_bytes = std::max(gpu0_ws_bytes, swc_hip_conv2dFusedMaxpool_workspace_bytes(o, i, f, k, s, p, "
+              << conv->getGroup() << ", po, pk, ps, pp));\n}\n";
         } else if (type == "Conv2dGrad") {   // parents: input, filter, outputGrad
             auto *conv = static_cast<Conv2dGradOp *>(op->getOp());
             q << "{\n"
@@ -618,6 +628,27 @@ void HipCodegen::emitHipCall(OpNode *op) {
         writer_ << "SWC_HIP_CHECK(swc_hip_conv2dFused_f(" << convArgs(conv) << ", " << nameOf(in(5)) << ", "
                 << nameOf(in(6)) << ", " << nameOf(in(3)) << ", " << nameOf(in(4)) << ", " << std::setprecision(12)
                 << conv->getEpsilon() << ", " << (conv->hasRelu() ? 1 : 0) << "));\n";
+    } else if (type == "Conv2dMaxPool") {
+        // parents: input, filter, bias [, bn scale, bn bias, bn mean, bn var]; the child is the pooled tensor
+        auto *conv = static_cast<Conv2dMaxPoolOp *>(op->getOp());
+        writer_ << arrayDef(nm + "_inDims", T(in(0))->getDims())
+                << arrayDef(nm + "_convDims", conv->convOutDims(T(in(0))->getDims(), T(in(1))->getDim(0)))
+                << arrayDef(nm + "_outDims", T(out(0))->getDims()) << arrayDef(nm + "_filterDims", T(in(1))->getDims())
+                << arrayDef(nm + "_biasDims", T(in(2))->getDims()) << arrayDef(nm + "_filterSizes", conv->getKernels())
+                << arrayDef(nm + "_strides", conv->getStrides()) << arrayDef(nm + "_pads", conv->getPads())
+                << arrayDef(nm + "_poolSizes", conv->getPoolKernels()) << arrayDef(nm + "_poolStrides", conv->getPoolStrides())
+                << arrayDef(nm + "_poolPads", conv->getPoolPads());
+        writer_ << "SWC_HIP_CHECK(swc_hip_conv2dFusedMaxpool_f(" << nameOf(out(0)) << ", " << nameOf(in(0)) << ", "
+                << nameOf(in(1)) << ", " << nameOf(in(2)) << ", " << nm << "_convDims, " << nm << "_inDims, " << nm
+                << "_filterDims, " << nm << "_biasDims, " << nm << "_filterSizes, " << nm << "_strides, " << nm << "_pads, "
+                << conv->getGroup() << ", ";
+        if (conv->hasBatchNorm())
+            writer_ << nameOf(in(5)) << ", " << nameOf(in(6)) << ", " << nameOf(in(3)) << ", " << nameOf(in(4)) << ", "
+                    << std::setprecision(12) << conv->getEpsilon();
+        else
+            writer_ << "NULL, NULL, NULL, NULL, 0.f";
+        writer_ << ", " << (conv->hasRelu() ? 1 : 0) << ", " << nm << "_outDims, " << nm << "_poolSizes, " << nm
+                << "_poolStrides, " << nm << "_poolPads));\n";
     } else if (type == "Conv2dAdd") {
         // parents: input, filter, bias, [bn scale, bn bias, bn mean, bn var,] the other summand
         auto *conv = static_cast<Conv2dAddOp *>(op->getOp());

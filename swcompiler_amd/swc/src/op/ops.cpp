@@ -76,6 +76,13 @@ void BatchNormReluMaxPoolOp::outTensorShapeGen(OpNode *node, size_t, TensorShape
     const auto idims = dimsOfParent(node, 0);
     shape->setShape(windowedShape(idims, kernels_, strides_, pads_, idims[3]));
 }
+std::vector<size_t> Conv2dMaxPoolOp::convOutDims(const std::vector<size_t> &idims, size_t oc) const {
+    return windowedShape(idims, kernels_, strides_, pads_, oc);
+}
+void Conv2dMaxPoolOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *shape) {
+    const auto cdims = convOutDims(dimsOfParent(node, 0), dimsOfParent(node, 1)[0]);
+    shape->setShape(windowedShape(cdims, pool_kernels_, pool_strides_, pool_pads_, cdims[3]));
+}
 void AvgPoolOp::outTensorShapeGen(OpNode *node, size_t, TensorShape *shape) {
     const auto idims = dimsOfParent(node, 0);
     shape->setShape(windowedShape(idims, kernels_, strides_, pads_, idims[3]));

@@ -385,6 +385,28 @@ class Conv2dAddOp : public Conv2dOp {
     bool hasBatchNorm() const { return bn_; }
     bool hasRelu() const { return relu_; }
 };
+// Conv2d (+ BatchNormalization) (+ Relu) followed by MaxPool: parents as Conv2d (3) or Conv2dBatchNorm (7); the
+// output is the pooled tensor, the convolution's own output never exists.  swc_hip_conv2dFusedMaxpool_f
+class Conv2dMaxPoolOp : public Conv2dOp {
+    float epsilon_;
+    bool bn_, relu_;
+    std::vector<size_t> pool_kernels_, pool_strides_, pool_pads_;
+
+  public:
+    Conv2dMaxPoolOp(std::vector<size_t> &kernels, std::vector<size_t> &strides, std::vector<size_t> &pads, bool bn, float eps,
+                    bool relu, std::vector<size_t> pk, std::vector<size_t> ps, std::vector<size_t> pp)
+        : Conv2dOp("Conv2dMaxPool", bn ? 7 : 3, kernels, strides, pads), epsilon_(eps), bn_(bn), relu_(relu),
+          pool_kernels_(std::move(pk)), pool_strides_(std::move(ps)), pool_pads_(std::move(pp)) {}
+    float getEpsilon() const { return epsilon_; }
+    bool hasBatchNorm() const { return bn_; }
+    bool hasRelu() const { return relu_; }
+    std::vector<size_t> getPoolKernels() const { return pool_kernels_; }
+    std::vector<size_t> getPoolStrides() const { return pool_strides_; }
+    std::vector<size_t> getPoolPads() const { return pool_pads_; }
+    // dims of the convolution's output for an input of `idims` and `oc` filters
+    std::vector<size_t> convOutDims(const std::vector<size_t> &idims, size_t oc) const;
+    void outTensorShapeGen(OpNode *node, size_t index, TensorShape *shape) override;
+};
 
 } // namespace op
 } // namespace swc

@@ -371,6 +371,28 @@ void spliceAdd(IRGraph *g, OpNode *producer, OpNode *add, IRNode *other, Op *fus
 
 } // namespace
 
+// The MaxPool that may move into the epilogue of the convolution `conv` feeding it: 2 x 2 windows, stride 2, no
+// padding, over a convolution output with even height and width, and an input-channel count the MFMA tile kernels
+// take as it is (a multiple of 4) — what swc_hip_conv2dFusedMaxpool_f does in one launch.
+static OpNode *poolBehind(OpNode *conv, IRGraph *g) {
+    OpNode *pool = soleConsumer(conv, "MaxPool", g);
+    if (!pool) return nullptr;
+    auto *mp = static_cast<MaxPoolOp *>(pool->getOp());
+    const auto k = mp->getKernels(), s = mp->getStrides(), p = mp->getPads();
+    if (k != std::vector<size_t>{2, 2} || s != std::vector<size_t>{2, 2}) return nullptr;
+    for (size_t v : p)
+        if (v) return nullptr;
+    Tensor *y = static_cast<TensorNode *>(conv->getChildNode(0))->getTensor();
+    Tensor *x = static_cast<TensorNode *>(conv->getParentNode(0))->getTensor();
+    if (y->getNDim() != 4 || y->getDim(1) % 2 || y->getDim(2) % 2 || x->getDim(3) % 4) return nullptr;
+    return pool;
+}
+static Op *pooledConv(Conv2dOp *conv, bool bn, float eps, bool relu, OpNode *pool) {
+    auto *mp = static_cast<MaxPoolOp *>(pool->getOp());
+    auto k = conv->getKernels(), s = conv->getStrides(), p = conv->getPads();
+    return new Conv2dMaxPoolOp(k, s, p, bn, eps, relu, mp->getKernels(), mp->getStrides(), mp->getPads());
+}
+
 void HipFusionPass::run() {
     bool changed = true;
     while (changed) {
@@ -400,10 +422,27 @@ void HipFusionPass::run() {
                 } else if (IRNode *other = nullptr; OpNode *add = soleAddConsumer(o, _graph, other)) {
                     spliceAdd(_graph, o, add, other, new Conv2dAddOp(k, s, p, false, 0.f, isType(add, "ElementAddRelu")));
                     changed = true;
+                } else if (OpNode *pool = poolBehind(o, _graph)) {
+                    splice(_graph, o, pool, pooledConv(conv, false, 0.f, false, pool));
+                    changed = true;
+                }
+            } else if (type == "Conv2dWithActivation") {
+                auto *ca = static_cast<Conv2dWithActivationOp *>(o->getOp());
+                if (ca->getGroup() != 1 || ca->getActivationType() != SWC_ACTIVATION_RELU) continue;
+                if (OpNode *pool = poolBehind(o, _graph)) {
+                    splice(_graph, o, pool, pooledConv(ca, false, 0.f, true, pool));
+                    changed = true;
                 }
             } else if (type == "Conv2dBatchNorm") {
                 auto *cb = static_cast<Conv2dBatchNormOp *>(o->getOp());
-                if (cb->hasRelu()) continue;
+                if (cb->hasRelu()) {
+                    if (OpNode *pool = poolBehind(o, _graph)) {
+                        splice(_graph, o, pool, pooledConv(cb, true, cb->getEpsilon(), true, pool));
+                        changed = true;
+                        ++fused_;
+                    }
+                    continue;
+                }
                 auto k = cb->getKernels(), s = cb->getStrides(), p = cb->getPads();
                 if (OpNode *r = soleConsumer(o, "Relu", _graph)) {
                     splice(_graph, o, r, new Conv2dBatchNormOp(k, s, p, cb->getEpsilon(), true));
@@ -411,6 +450,9 @@ void HipFusionPass::run() {
                 } else if (IRNode *other = nullptr; OpNode *add = soleAddConsumer(o, _graph, other)) {
                     spliceAdd(_graph, o, add, other,
                               new Conv2dAddOp(k, s, p, true, cb->getEpsilon(), isType(add, "ElementAddRelu")));
+                    changed = true;
+                } else if (OpNode *pool = poolBehind(o, _graph)) {
+                    splice(_graph, o, pool, pooledConv(cb, true, cb->getEpsilon(), false, pool));
                     changed = true;
                 }
             } else if (type == "BatchNormalization") {
@@ -444,7 +486,7 @@ bool DeviceMemoryLoweringPass::runsOnGpu(const std::string &t) {
     static const std::set<std::string> gpu = {
         "MatrixMatrixMul", "MatrixVectorAdd", "BatchedAdd", "MatrixMatrixFCBias", "MatrixMatrixFCBiasRelu",
         "MatrixMatrixFCBiasSoftmax", "Reshape", "TensorDescend", "TensorAscend", "MatrixTanh", "MatrixSoftmax", "ElementAdd", "ElementAddRelu", "Relu", "Dropout",
-        "Conv2d", "Conv2dWithActivation", "Conv2dBatchNorm", "Conv2dAdd", "MaxPool", "AveragePool", "Transpose",
+        "Conv2d", "Conv2dWithActivation", "Conv2dBatchNorm", "Conv2dAdd", "Conv2dMaxPool", "MaxPool", "AveragePool", "Transpose",
         "BatchNormalization",
         "BatchNormalizationRelu", "BatchNormReluMaxPool", "ArgMax", "Accuracy",
         "MatrixSoftmaxWithLoss", "MatrixSoftmaxWithLossGrad", "MatrixSoftmaxGrad", "BatchedReduceAdd", "MatrixTanhGrad", "ReluGrad",

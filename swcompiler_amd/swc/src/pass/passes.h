@@ -107,6 +107,8 @@ class ElimTransposePass : public OptimizePass {
 //   BatchNormalizationRelu -> MaxPool             => BatchNormReluMaxPool
 //   ElementAdd -> Relu                            => ElementAddRelu
 //   Conv2d | Conv2dBatchNorm -> ElementAdd[Relu]  => Conv2dAdd (the other summand becomes its last operand)
+//   Conv2d | Conv2dWithActivation | Conv2dBatchNorm -> MaxPool 2x2/2, no padding, over an even-sized output of a
+//       convolution with iC % 4 == 0                 => Conv2dMaxPool (the pooling in the convolution's epilogue)
 // Each right-hand side is one kernel launch of libswc_hip whose result equals
 // the left-hand sequence of reference kernels.
 class HipFusionPass : public OptimizePass {

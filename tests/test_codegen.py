@@ -130,9 +130,16 @@ def test_mnist8_cpu_program_prints_the_reference_labels(gen, tmp_path, golden):
 
 def test_hip_program_structure_and_build(gen, tmp_path):
     code = generate(gen, "cfg4", "hip", tmp_path, 2)
-    # fused: four conv+bn+relu launches, two pools, nothing else on the device
-    assert code.count("swc_hip_conv2dFused_f(") == 4 and "swc_hip_batchnorm" not in code and "swc_hip_relu_f" not in code
-    assert code.count("swc_hip_maxpool_f(") == 2
+    # fused: four launches — conv+bn+relu twice, conv+bn+relu with the 2x2 pooling in its epilogue twice — and
+    # nothing else on the device
+    assert code.count("swc_hip_conv2dFused_f(") == 2 and code.count("swc_hip_conv2dFusedMaxpool_f(") == 2
+    assert "swc_hip_batchnorm" not in code and "swc_hip_relu_f" not in code and "swc_hip_maxpool_f(" not in code
+    assert "const size_t conv2_convDims[] = {2, 56, 56, 128};" in code and "const size_t conv2_outDims[] = {2, 28, 28, 128};" in code
+    assert re.search(r"swc_hip_conv2dFusedMaxpool_f\(\w+, \w+, \w+, \w+, conv2_convDims, conv2_inDims, conv2_filterDims, "
+                     r"conv2_biasDims, conv2_filterSizes, conv2_strides, conv2_pads, 1, \w+, \w+, \w+, \w+, [0-9.e-]+, 1, "
+                     r"conv2_outDims, conv2_poolSizes, conv2_poolStrides, conv2_poolPads\)", code)
+    # the convolution's own output is no tensor of the program any more
+    assert code.count("swc_hip_conv2dFusedMaxpool_workspace_bytes(o, i, f, k, s, p, 1, po, pk, ps, pp)") == 2
     # every device tensor sits on a 256-byte boundary of the arena
     offs = [int(v) for v in re.findall(r"gpu0_baseptr \+ (\d+)\)", code)]
     assert offs and all(o % 256 == 0 for o in offs)
@@ -162,11 +169,13 @@ def test_hip_program_structure_and_build(gen, tmp_path):
     assert mlp.index("swc_hip_set_workspace(gpu0_ws, gpu0_ws_bytes)") < mlp.index("// call op routine functions")
     assert mlp.index("swc_hip_set_workspace(nullptr, 0)") < mlp.index("swc_hip_free(gpu0_ws)")
     # ... and of its convolutions: one query per conv, with the conv's own shape arrays
-    assert code.count("swc_hip_conv2d_workspace_bytes(o, i, f, k, s, p, 1)") == 4
+    assert code.count("swc_hip_conv2d_workspace_bytes(o, i, f, k, s, p, 1)") == 2
     assert "const size_t o[] = {2, 56, 56, 64};" in code and "const size_t f[] = {128, 3, 3, 64};" in code
     assert code.index("swc_hip_set_workspace(gpu0_ws, gpu0_ws_bytes)") < code.index("// call op routine functions")
     lenet = generate(gen, "cfg3", "hip", tmp_path, 4)
-    assert lenet.count("swc_hip_conv2dFused_f(") == 2 and "swc_hip_matrixMatrixFCBias_f(4, 500, 800" in lenet
+    # LeNet: the first layer (one input channel) keeps its pooling kernel, the second (20 channels) pools in its epilogue
+    assert lenet.count("swc_hip_conv2dFused_f(") == 1 and lenet.count("swc_hip_conv2dFusedMaxpool_f(") == 1
+    assert lenet.count("swc_hip_maxpool_f(") == 1 and "swc_hip_matrixMatrixFCBias_f(4, 500, 800" in lenet
     bnpool = generate(gen, "cfg5c", "hip", tmp_path, 1)
     assert bnpool.count("swc_hip_batchnormReluMaxpool_f(") == 1 and "swc_hip_maxpool_f" not in bnpool
     assert "swc_hip_batchnormRelu_f" not in bnpool and "swc_hip_batchnormalization_f" not in bnpool

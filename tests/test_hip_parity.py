@@ -13,6 +13,7 @@ product differ by ~k*eps*sum|a||b| however small the cancelled result is; so
 both against 1e-4, and integer-valued operands (exact in any order) are asserted
 bit-exact.
 """
+import ctypes
 import itertools
 import os
 
@@ -519,6 +520,91 @@ def test_fcbias_softmax_fused(rt, oracle, m, k, n):
     # no bias
     assert_bit_exact(rt.fcbias(da, dw, None, softmax=True).numpy(), rt.matrixSoftmax(rt.fcbias(da, dw, None)).numpy(),
                      "fused vs sequence, no bias")
+
+
+POOLED_CONVS = [
+    # idims, fdims, pads: the two layers of the conv block that a pooling follows, at full size
+    ((32, 56, 56, 64), (128, 3, 3, 64), (1, 1, 1, 1)),
+    ((32, 28, 28, 128), (128, 3, 3, 128), (1, 1, 1, 1)),
+    ((2, 8, 12, 8), (24, 3, 3, 8), (1, 1, 1, 1)),       # one partial tile, 24 of 64 columns
+    ((3, 10, 6, 16), (70, 3, 3, 16), (1, 1, 1, 1)),     # columns over two tiles, rows end inside a tile
+    ((5, 16, 16, 12), (64, 5, 5, 12), (2, 2, 2, 2)),
+    ((1, 2, 2, 4), (4, 1, 1, 4), (0, 0, 0, 0)),         # a single window
+    ((2, 18, 20, 32), (96, 3, 3, 32), (0, 0, 0, 0)),    # 16 x 18 output
+]
+
+
+@pytest.mark.parametrize("idims,fdims,pads", POOLED_CONVS)
+@pytest.mark.parametrize("slots", [None, "7"])
+def test_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, pads, slots, monkeypatch):
+    """conv (+BN) (+ReLU) + 2x2/2 max-pooling in one call is bit for bit the pooling of the separate convolution:
+    both put a pixel into the same tile (rows in window order) and add its products in the same sequence, whole
+    tiles and tiles cut along K alike (slots = 7 pretends a chip of seven workgroups, so that most tiles are cut)."""
+    print("case pooled conv", idims, fdims, pads, slots, flush=True)
+    if slots:
+        monkeypatch.setenv("SWC_HIP_CONV_SLOTS", slots)
+    rng = np.random.default_rng(sum(idims) + sum(fdims))
+    oc, c = fdims[0], fdims[3]
+    x = rng.standard_normal(idims).astype(np.float32)
+    f = (rng.standard_normal(fdims) / np.sqrt(fdims[1] * fdims[2] * c)).astype(np.float32)
+    b = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    bn = [rng.uniform(-0.1, 0.1, oc).astype(np.float32), rng.uniform(0.5, 2.0, oc).astype(np.float32),
+          rng.uniform(0.5, 1.5, oc).astype(np.float32), rng.uniform(-0.1, 0.1, oc).astype(np.float32)]   # mean var scale bias
+    dx, df, db = up(rt, x, f, b)
+    dbn = up(rt, *bn)
+    pool = ((2, 2), (2, 2))
+    for with_bn, relu in [(True, True), (False, True), (False, False), (True, False)]:
+        kw = dict(pads=pads, bn=dbn if with_bn else None, eps=1e-5, relu=relu)
+        fused = rt.conv2d(dx, df, db, pool=pool, **kw)
+        assert rt.last_kernel().startswith("conv_dma<") and rt.last_kernel().endswith("(pooled)"), rt.last_kernel()
+        plain = rt.conv2d(dx, df, db, **kw)
+        assert rt.last_kernel().startswith("conv_dma<"), rt.last_kernel()
+        want = rt.maxpool(plain, *pool).numpy()
+        assert_bit_exact(fused.numpy(), want, f"pooled in the epilogue vs conv then maxpool (bn {with_bn}, relu {relu})")
+    # against the oracle (full-size layers: the first image only)
+    n = 1 if idims[0] * idims[1] * idims[2] * fdims[0] > (1 << 22) else idims[0]
+    ref = oracle.conv2d(x[:n], f, b, pads=pads)
+    ref = oracle.maxpool(oracle.relu(oracle.batchnormalization(ref, *bn, 1e-5)), *pool)
+    got = rt.conv2d(dx, df, db, pads=pads, bn=dbn, eps=1e-5, relu=True, pool=pool).numpy()[:n]
+    # (signed operands: the error of a sum is judged against the sum of the magnitudes of its terms, here carried
+    # through the batchnorm's slope and the pooling)
+    slope = np.abs(bn[2] / np.sqrt(bn[1] + np.float32(1e-5)))
+    scale = oracle.maxpool(oracle.conv2d(np.abs(x[:n]), np.abs(f), np.abs(b), pads=pads) * slope + np.abs(bn[3]), *pool)
+    assert scaled_err(got, ref, scale) < TOL
+    # raster order of the rows gives the same values up to the order of summation of the tiles cut along K
+    monkeypatch.setenv("SWC_HIP_CONV_ORDER", "raster")
+    raster = rt.maxpool(rt.conv2d(dx, df, db, pads=pads, bn=dbn, eps=1e-5, relu=True), *pool).numpy()[:n]
+    assert scaled_err(raster, ref, scale) < TOL
+    if not slots and rt.last_kernel().find("conv_sk_finish") < 0:
+        assert_bit_exact(raster, got, "window order vs raster order, every tile whole")
+
+
+def test_conv_with_a_pooling_the_epilogue_cannot_do(rt, oracle):
+    """odd output sizes, 3x3 windows, a layer for the direct kernel: conv into the workspace, then maxpool_f's kernel"""
+    rng = np.random.default_rng(5)
+    cases = [((2, 9, 9, 8), (16, 3, 3, 8), (1, 1, 1, 1), ((2, 2), (2, 2))),          # 9 x 9 output
+             ((2, 12, 12, 8), (16, 3, 3, 8), (1, 1, 1, 1), ((3, 3), (2, 2))),        # 3 x 3 windows
+             ((2, 12, 12, 8), (16, 3, 3, 8), (1, 1, 1, 1), ((2, 2), (2, 2), (1, 1, 1, 1))),   # padded pooling
+             ((4, 28, 28, 1), (20, 5, 5, 1), (0, 0, 0, 0), ((2, 2), (2, 2)))]        # the direct kernel's layer
+    for idims, fdims, pads, pool in cases:
+        print("case conv + other pooling", idims, fdims, pads, pool, flush=True)
+        x = rng.standard_normal(idims).astype(np.float32)
+        f = (rng.standard_normal(fdims) / 8).astype(np.float32)
+        b = (rng.standard_normal(fdims[0]) * 0.1).astype(np.float32)
+        dx, df, db = up(rt, x, f, b)
+        assert rt.conv2d_maxpool_workspace_bytes(idims, fdims, (1, 1), pads, pool) >= 4 * np.prod(idims[:3]) * fdims[0] // 2
+        fused = rt.conv2d(dx, df, db, pads=pads, relu=True, pool=pool).numpy()
+        assert not rt.last_kernel().endswith("(pooled)"), rt.last_kernel()
+        assert_bit_exact(fused, rt.maxpool(rt.conv2d(dx, df, db, pads=pads, relu=True), *pool).numpy(), "two steps")
+        assert rel_err(fused, oracle.maxpool(oracle.relu(oracle.conv2d(x, f, b, pads=pads)), *pool)) < TOL
+    # error paths
+    dx, df, db = up(rt, np.zeros((1, 4, 4, 4), np.float32), np.zeros((4, 1, 1, 4), np.float32), np.zeros(4, np.float32))
+    out = rt.empty((1, 2, 2, 8))
+    d = lambda *v: (ctypes.c_size_t * len(v))(*v)
+    rc = rt.lib.swc_hip_conv2dFusedMaxpool_f(out.ptr, dx.ptr, df.ptr, db.ptr, d(1, 4, 4, 4), d(1, 4, 4, 4), d(4, 1, 1, 4),
+                                             d(4), d(1, 1), d(1, 1), d(0, 0, 0, 0), 1, None, None, None, None, 0.0, 1,
+                                             d(1, 2, 2, 8), d(2, 2), d(2, 2), d(0, 0, 0, 0))
+    assert rc != 0 and b"pooled batch/channels" in rt.lib.swc_hip_last_error()
 
 
 STREAMED_HEADS = [(4096, 4096, 10), (1000, 4096, 10), (33, 1028, 7), (16, 2048, 16), (257, 1056, 1), (100, 1200, 3),
