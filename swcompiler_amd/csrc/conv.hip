@@ -207,10 +207,29 @@ __device__ __forceinline__ ColumnParams column_params(const Epilogue &ep, int co
     }
     return c;
 }
-__device__ __forceinline__ float finish_element(float x, const ColumnParams &c, bool bn, bool relu) {
-    x += c.bias;
-    if (bn) x = fmaf(x - c.mean, c.slope, c.beta);
-    return relu ? ((x > 0.f) ? x : 0.f) : x;
+// The same in two steps, for a kernel that requests the parameters at its start and needs them at its end: the raw
+// loads (nothing waits for them), and, once they have arrived, the arithmetic.
+struct ColumnRaw {
+    float bias, mean, var, scale, beta;
+};
+__device__ __forceinline__ ColumnRaw column_raw(const Epilogue &ep, int col, bool ok) {
+    ColumnRaw r{(ep.bias && ok) ? ep.bias[col] : 0.f, 0.f, 1.f, 1.f, 0.f};
+    if (ep.bn_mean && ok) {
+        r.mean = ep.bn_mean[col];
+        r.var = ep.bn_var[col];
+        r.scale = ep.bn_scale[col];
+        r.beta = ep.bn_bias[col];
+    }
+    return r;
+}
+__device__ __forceinline__ ColumnParams column_params(const Epilogue &ep, const ColumnRaw &r) {
+    ColumnParams c{r.bias, 0.f, 1.f, 0.f};
+    if (ep.bn_mean) {
+        c.mean = r.mean;
+        c.slope = (float)((double)r.scale / sqrt((double)(r.var + ep.eps)));
+        c.beta = r.beta;
+    }
+    return c;
 }
 // maxpool_f's choice among the taps of a window in its order (kernels.h:343-383: the first, then whatever is greater)
 __device__ __forceinline__ float window_max(float a, float b, float c, float d) {
@@ -228,13 +247,11 @@ __device__ __forceinline__ float window_max(float a, float b, float c, float d) 
 // M is a multiple of 4 here, so a window is wholly inside or outside.
 template <int TM, int TN, bool POOL>
 __device__ __forceinline__ void store_tile_windows(const v16f (&acc)[TM][TN], float *__restrict__ out, const ConvGeom &g,
-                                                   int row0, int col0, int lane, const Epilogue &ep) {
+                                                   int row0, int col0, int lane, const Epilogue &ep,
+                                                   const ColumnParams (&cp)[TN]) {
     const int l32 = lane & 31, h = lane >> 5;
     const int N = g.OC, pw = g.OW >> 1, ph = g.OH >> 1;
     const bool bn = ep.bn_mean != nullptr;
-    ColumnParams cp[TN];
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn) cp[tn] = column_params(ep, col0 + tn * 32 + l32, col0 + tn * 32 + l32 < N);
     // this lane's windows: w0, w0 + 2, w0 + 4, ... (rows row0 + 4h + 8 * (g + 4 tm))
     int w = (row0 >> 2) + h;
     int px = w % pw, t = w / pw;
@@ -356,6 +373,27 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
         sk_tile_coords(pid, sk.dp_tiles, tiles_m, tiles_n, tile_m, tile_n);
         const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
         const int k_limit = (kt_end * BK < K) ? kt_end * BK : K;
+        // The three workgroups of a CU run in step (they start together and take equally long), so the start and
+        // the end of a tile are not covered by the others' matrix work: both are kept short and run at a raised
+        // wavefront priority, the K loop at the lowest.  The epilogue's per-column parameters are requested here,
+        // ahead of the ring's loads (older loads complete first, so the ring's counts are unaffected), and
+        // turned into bias / slope / offset after the first slice has landed.
+        __builtin_amdgcn_s_setprio(3);
+        const int col_first = n0 + (wave & 1) * 32 * TN + (lane & 31);
+        ColumnRaw raw[TN];
+        ColumnParams cp[TN];
+        if (whole && g.win) {
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn) raw[tn] = column_raw(ep, col_first + tn * 32, col_first + tn * 32 < N);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        auto first_slice_landed = [&]() {
+            if (whole && g.win) {
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn) cp[tn] = column_params(ep, raw[tn]);
+            }
+            __builtin_amdgcn_s_setprio(0);
+        };
 
         // Per load, the output pixel this lane gathers for: element offset of its
         // window's top-left tap (may be negative) and that tap's coordinates; rows
@@ -436,6 +474,7 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
         int rd_stage = 0, wr_stage = STAGES - 1;
         if constexpr (MID) {   // ring hand-over after the first MFMA group of a slice (dma_step_mid)
             ring_sync<(STAGES - 2) * T::kLoads>();   // the first slice has landed
+            first_slice_landed();
             Frag<TM, TN> frag[2];
             load_frag_swz<TM, TN, true>(frag[0], lds, lds + T::kAFloats, 0, wave >> 1, wave & 1, lane & 31, lane >> 5);
             for (int kt = kt_begin; kt < kt_end; ++kt) {
@@ -450,6 +489,7 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
         } else {
             for (int kt = kt_begin; kt < kt_end; ++kt) {
                 ring_sync<(STAGES - 2) * T::kLoads>();
+                if (kt == kt_begin) first_slice_landed();
                 next_offsets();
                 dma_step<TM, TN, true, STAGES>(lds + wr_stage * T::kStageFloats, lds + rd_stage * T::kStageFloats, rsrc_a,
                                                rsrc_b, va, vb, acc, wave, lane);
@@ -457,19 +497,494 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
                 wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
             }
         }
+        __builtin_amdgcn_s_setprio(3);
         wait_vmcnt<0>();   // the trailing dummy loads still target this workgroup's LDS
         acc_settle(acc);
         if (whole) {
             const int row0 = m0 + (wave >> 1) * 32 * TM, col0 = n0 + (wave & 1) * 32 * TN;
             if (!g.win) store_tile<TM, TN>(acc, out, (size_t)N, M, N, row0, col0, lane, ep);
-            else if (pool) store_tile_windows<TM, TN, true>(acc, out, g, row0, col0, lane, ep);
-            else store_tile_windows<TM, TN, false>(acc, out, g, row0, col0, lane, ep);
+            else if (pool) store_tile_windows<TM, TN, true>(acc, out, g, row0, col0, lane, ep, cp);
+            else store_tile_windows<TM, TN, false>(acc, out, g, row0, col0, lane, ep, cp);
         } else {
             float *slot = part + (size_t)(2 * share + (piece ? 1 : 0)) * (T::BM * T::BN);
             store_tile_impl<TM, TN, false, false>(acc, slot, (size_t)T::BN, T::BM, T::BN, (wave >> 1) * 32 * TM,
                                            (wave & 1) * 32 * TN, lane, Epilogue{});
         }
     }
+#endif
+}
+
+#if __HIP_DEVICE_COMPILE__
+// The four loads of a wavefront for one slice of a 64 x 64 tile into stage `wr` (conv_dma_lean): per-lane offsets
+// va/vb, the position inside the tap (A) and along K (B) as scalar offsets.
+__device__ __forceinline__ void lean_request(char *__restrict__ wr, __amdgpu_buffer_rsrc_t rsrc_a, __amdgpu_buffer_rsrc_t rsrc_b,
+                                             int va0, int va1, int vb0, int vb1, int soff_a, int soff_b, int wave) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t *)(wr + wave * 1024), 16, va0, soff_a, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t *)(wr + (4 + wave) * 1024), 16, va1, soff_a, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_t *)(wr + 8192 + wave * 1024), 16, vb0, soff_b, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_t *)(wr + 8192 + (4 + wave) * 1024), 16, vb1, soff_b, 0, 0);
+}
+__device__ __forceinline__ void lean_read(Frag<1, 1> &f, const char *__restrict__ stage, int a_addr, int b_addr) {
+    const float4 a = *reinterpret_cast<const float4 *>(stage + a_addr);
+    const float4 b = *reinterpret_cast<const float4 *>(stage + b_addr);
+    f.a[0][0] = a.x, f.a[0][1] = a.y, f.a[0][2] = a.z, f.a[0][3] = a.w;
+    f.b[0][0] = b.x, f.b[0][1] = b.y, f.b[0][2] = b.z, f.b[0][3] = b.w;
+}
+// One slice out of stage `rd`; behind the barrier the loads of the slice two on go into `wr`; the first fragments of
+// the next slice come out of `nx` (see dma_step_mid).  The three stages are distinct, which is what __restrict__ says:
+// without it every LDS read behind a load would wait for ALL outstanding loads.
+__device__ __forceinline__ void lean_step(char *__restrict__ wr, const char *__restrict__ rd, const char *__restrict__ nx,
+                                          __amdgpu_buffer_rsrc_t rsrc_a, __amdgpu_buffer_rsrc_t rsrc_b, int va0, int va1,
+                                          int vb0, int vb1, int soff_a, int soff_b, const int (&a_addr)[4],
+                                          const int (&b_addr)[4], v16f (&acc)[1][1], Frag<1, 1> (&frag)[2], int wave) {
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+        if (gq == 1) {
+            ring_sync<0>();
+            lean_request(wr, rsrc_a, rsrc_b, va0, va1, vb0, vb1, soff_a, soff_b, wave);
+        }
+        if (gq < 3) lean_read(frag[(gq + 1) & 1], rd, a_addr[gq + 1], b_addr[gq + 1]);
+        else lean_read(frag[0], nx, a_addr[0], b_addr[0]);
+        __builtin_amdgcn_sched_barrier(0);
+        const Frag<1, 1> &f = frag[gq & 1];
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) mfma_acc(acc[0][0], f.a[0][s4], f.b[0][s4]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+#endif
+
+// conv_dma<1,1,3,true> with next to no vector-ALU work in its K loop, for layers whose channel count is a multiple
+// of 32 (a K slice then lies inside one filter tap, the same for every lane).
+// Why.  On this chip the vector ALU and the matrix pipe of a SIMD do not run side by side: a microbenchmark of three
+// wavefronts per SIMD, each issuing 16 dependent v_mfma_f32_32x32x2_f32 per iteration, loses 2 - 5 cycles of MFMA
+// throughput for every VALU instruction that any of the three executes (v_mov 2.2, v_fma 3.1, v_cmp 4.9; LDS reads
+// and scalar instructions under half a cycle).  conv_dma spends about 60 VALU instructions per slice of 16 MFMAs
+// on gather offsets (bounds tests, tap stepping) and LDS addresses — a fifth of the slice's 1024 MFMA cycles — and
+// that, not its memory traffic, is most of what its matrix cores wait for.
+// What differs here:
+//   * the gather offset of a row changes with the tap only: within a tap the channel position travels in the load's
+//     scalar offset, so the per-lane offsets (with their bounds tests) are recomputed once per tap, C/32 slices;
+//   * the filter rows' offsets never change (the k position is the scalar offset);
+//   * the K loop is unrolled over the three ring stages, so every LDS address is a lane constant (eight registers,
+//     one per operand and group of 8 k) plus an immediate.
+// Pieces, slots, ring discipline, epilogues and results are conv_dma's.
+__global__ __launch_bounds__(kThreads) void conv_dma_lean(const float *__restrict__ in, const float *__restrict__ filt,
+                                                          float *__restrict__ out, ConvGeom g, unsigned in_bytes,
+                                                          unsigned filt_bytes, Epilogue ep, SkPlan sk,
+                                                          float *__restrict__ part, int pool) {
+#if __HIP_DEVICE_COMPILE__
+    constexpr int TM = 1, TN = 1, STAGES = 3;
+    using T = DmaTile<TM, TN, true, STAGES>;
+    static_assert(T::kALoads == 2 && T::kBLoads == 2, "");
+    extern __shared__ __align__(16) float lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int M = g.M, N = g.OC, K = g.K;
+    const int tiles_m = (M + T::BM - 1) / T::BM, tiles_n = (N + T::BN - 1) / T::BN;
+    const int nk = K / BK;   // C % 32 == 0
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(in, in_bytes);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(filt, filt_bytes);
+    char *const lds_b = reinterpret_cast<char *>(lds);
+
+    // LDS byte addresses of this lane's fragments inside a stage, per group of 8 k (see load_frag_swz)
+    int a_addr[4], b_addr[4];
+    {
+        const int l32 = lane & 31, h = lane >> 5, swz = (l32 >> 1) & 7;
+        const int row_a = (wave >> 1) * 32 + l32, row_b = (wave & 1) * 32 + l32;
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+            a_addr[gq] = (row_a * BK + (((2 * gq + h) ^ swz) << 2)) * 4;
+            b_addr[gq] = (T::kAFloats + row_b * BK + (((2 * gq + h) ^ swz) << 2)) * 4;
+        }
+    }
+    const int chunk16 = kc_chunk(lane, wave) * 16;   // byte position of this lane's 16 bytes inside a slice of a row
+
+    int u0, u1, share = -1;
+    if ((int)blockIdx.x < sk.dp_tiles) {
+        u0 = blockIdx.x * nk;
+        u1 = u0 + nk;
+    } else {
+        share = blockIdx.x - sk.dp_tiles;
+        u0 = sk.dp_tiles * nk + share * sk.q + (share < sk.r ? share : sk.r);
+        u1 = u0 + sk.q + (share < sk.r ? 1 : 0);
+    }
+    for (int piece = 0; u0 < u1; ++piece) {
+        const int pid = u0 / nk;
+        const int kt_begin = u0 - pid * nk;
+        const int kt_end = (u1 - u0 < nk - kt_begin) ? kt_begin + (u1 - u0) : nk;
+        const bool whole = kt_begin == 0 && kt_end == nk;
+        u0 += kt_end - kt_begin;
+        if (piece) __builtin_amdgcn_s_barrier();   // every wavefront is done reading the ring of the previous piece
+
+        int tile_m, tile_n;
+        sk_tile_coords(pid, sk.dp_tiles, tiles_m, tiles_n, tile_m, tile_n);
+        const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
+        __builtin_amdgcn_s_setprio(3);
+        const int col_first = n0 + (wave & 1) * 32 + (lane & 31);
+        ColumnRaw raw[TN];
+        ColumnParams cp[TN];
+        if (whole && g.win) raw[0] = column_raw(ep, col_first, col_first < N);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // per-lane constants of the two rows of A and of B that this lane gathers for
+        int row_off[2], iy0[2], ix0[2], vb[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int m = m0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
+            if (m < M) {
+                int img, oy, ox;
+                pixel_of_row(g, m, img, oy, ox);
+                iy0[j] = oy * g.sh - g.pt;
+                ix0[j] = ox * g.sw - g.pl;
+                row_off[j] = (((img * g.H + iy0[j]) * g.W + ix0[j]) * g.C) * 4 + chunk16;
+            } else {
+                iy0[j] = ix0[j] = -(1 << 20);
+                row_off[j] = 0;
+            }
+            const int n = n0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
+            vb[j] = n < N ? n * K * 4 + chunk16 : kOutOfRange;
+        }
+        // the loads' position: slice lk of the piece = tap (ky, kx), channels ci .. ci + 31
+        int lk = kt_begin, ky, kx, ci;
+        {
+            const int tap = (lk * BK) / g.C;
+            ci = lk * BK - tap * g.C;
+            ky = tap / g.kw;
+            kx = tap - ky * g.kw;
+        }
+        int va[2];
+        auto retap = [&]() {   // the rows' offsets under tap (ky, kx), or out of range
+            const int tap_off = (ky * g.W + kx) * g.C * 4;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const bool ok = (unsigned)(iy0[j] + ky) < (unsigned)g.H && (unsigned)(ix0[j] + kx) < (unsigned)g.W;
+                va[j] = ok ? row_off[j] + tap_off : kOutOfRange;
+            }
+        };
+        retap();
+        // moves the loads' position on by a slice; past the piece's end the loads are empty
+        auto advance = [&]() {
+            ++lk;
+            ci += BK;
+            if (lk == kt_end) {
+                va[0] = va[1] = vb[0] = vb[1] = kOutOfRange;
+            } else if (ci == g.C) {
+                asm volatile("" ::: "memory");   // keeps this a (wavefront-uniform) branch: as selects it would run every slice
+                ci = 0;
+                if (++kx == g.kw) {
+                    kx = 0;
+                    ++ky;
+                }
+                retap();
+            }
+        };
+        constexpr int kStageBytes = T::kStageFloats * 4;
+        char *const st0 = lds_b, *const st1 = lds_b + kStageBytes, *const st2 = lds_b + 2 * kStageBytes;
+
+        v16f acc[1][1];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[0][0][v] = 0.f;
+        Frag<1, 1> frag[2];
+        // a step out of stage RD: its loads go into stage (RD + 2) % 3, the next slice sits in (RD + 1) % 3
+        auto step = [&](char *wr, const char *rd, const char *nx) {
+            lean_step(wr, rd, nx, rsrc_a, rsrc_b, va[0], va[1], vb[0], vb[1], ci * 4, lk * BK * 4, a_addr, b_addr, acc, frag, wave);
+            advance();
+        };
+
+        lean_request(st0, rsrc_a, rsrc_b, va[0], va[1], vb[0], vb[1], ci * 4, lk * BK * 4, wave);
+        advance();
+        lean_request(st1, rsrc_a, rsrc_b, va[0], va[1], vb[0], vb[1], ci * 4, lk * BK * 4, wave);
+        advance();
+        ring_sync<T::kLoads>();   // the first slice has landed
+        if (whole && g.win) cp[0] = column_params(ep, raw[0]);
+        __builtin_amdgcn_s_setprio(0);
+        lean_read(frag[0], st0, a_addr[0], b_addr[0]);
+        int kt = kt_begin;
+        for (; kt + 3 <= kt_end; kt += 3) {
+            step(st2, st0, st1);
+            step(st0, st1, st2);
+            step(st1, st2, st0);
+        }
+        if (kt < kt_end) step(st2, st0, st1);
+        if (kt + 1 < kt_end) step(st0, st1, st2);
+
+        __builtin_amdgcn_s_setprio(3);
+        wait_vmcnt<0>();   // the trailing empty loads still target this workgroup's LDS
+        acc_settle(acc);
+        if (whole) {
+            const int row0 = m0 + (wave >> 1) * 32, col0 = n0 + (wave & 1) * 32;
+            if (!g.win) store_tile<1, 1>(acc, out, (size_t)N, M, N, row0, col0, lane, ep);
+            else if (pool) store_tile_windows<1, 1, true>(acc, out, g, row0, col0, lane, ep, cp);
+            else store_tile_windows<1, 1, false>(acc, out, g, row0, col0, lane, ep, cp);
+        } else {
+            float *slot = part + (size_t)(2 * share + (piece ? 1 : 0)) * (T::BM * T::BN);
+            store_tile_impl<1, 1, false, false>(acc, slot, (size_t)T::BN, T::BM, T::BN, (wave >> 1) * 32, (wave & 1) * 32, lane,
+                                                Epilogue{});
+        }
+    }
+#endif
+}
+
+// conv_dma for workgroups that stay (opt-in, SWC_HIP_CONV_STREAM=1): as many workgroups as the chip holds at a time,
+// each walking its own list of work — first its share of the tiles cut along K (if it has one), then the whole tiles
+// w, w + G, w + 2G, ... — with the LDS ring running on across the boundaries between pieces: the loads of the next
+// piece's first slices are requested while the last slices of the current one are multiplied, the gather offsets of
+// the next tile are computed in the shadow of those MFMAs, the epilogue's parameters are requested a piece ahead, and
+// the epilogue itself is the accumulator read-out and the stores.  The units, the pieces' slots in `part` and
+// conv_sk_finish are those of conv_dma, and so are the results, bit for bit.
+// Why it is not the default.  A timeline of conv_dma (wall clock per workgroup) shows the start of a tile (gather
+// offsets, two slices requested, the wait for the first: 2 us on an idle chip, a median of 5 - 10 us later on) and
+// its end (3 us) taking a third of a workgroup's lifetime on a K of 576, and the three workgroups of a CU doing both
+// in step — which suggested that workgroups without those phases would run a fifth faster.  Measured, 56x56x64->64 /
+// ->128 / 28x28x128->128 take 94.5 / 177.6 / 88.0 us this way against 91.1 / 172.3 / 85.2 us: per slice a workgroup
+// here needs 2.0 us where conv_dma's need 1.3 - 1.6 us while all three are in their K loops.  Neither a fourth
+// ring stage (two slices of loads in flight, two workgroups per CU: 98.8 / 184.5 / 96.4 us), nor 128x64 or 64x128
+// tiles (171 / 169 us for the second layer), nor start times spread over a slice period changed that.  What the
+// ablations of conv_dma's K loop say instead: without its loads 82 / 156 / 76 us, without its fragment reads 86 /
+// 167 / 81, without the offset arithmetic 84 / 159 / 77, without all three and without the barrier still 76.5 / 142 /
+// 71 — against 47 / 94 / 47 us of pure matrix work: the larger part of the loss is not in the K loop's memory
+// traffic at all.
+template <int TM, int TN, int STAGES>
+__global__ __launch_bounds__(kThreads) void conv_dma_stream(const float *__restrict__ in, const float *__restrict__ filt,
+                                                            float *__restrict__ out, ConvGeom g, unsigned in_bytes,
+                                                            unsigned filt_bytes, Epilogue ep, SkPlan sk,
+                                                            float *__restrict__ part, int pool) {
+#if __HIP_DEVICE_COMPILE__
+    using T = DmaTile<TM, TN, true, STAGES>;
+    static_assert(STAGES >= 3, "ring hand-over in mid-slice");
+    extern __shared__ __align__(16) float lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int M = g.M, N = g.OC, K = g.K;
+    const int tiles_m = (M + T::BM - 1) / T::BM, tiles_n = (N + T::BN - 1) / T::BN;
+    const int nk = (K + BK - 1) / BK;
+    const int entries = sk.sk_wgs + sk.dp_tiles;   // entry e < sk_wgs: share e of the cut tiles; else whole tile e - sk_wgs
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(in, in_bytes);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(filt, filt_bytes);
+
+    // A walk over this workgroup's pieces, in order: entry e (then e + G, e + 2G, ...), of which units [u0, u1) are
+    // left; `share` is the entry's share of the cut tiles or -1 for a whole tile, `done` the pieces handed out of it.
+    // Two walks run, the loads' (ahead) and the multiplications'.  (Plain integers by reference, no structures: a
+    // structure here ends up in scratch memory, whose accesses count as vector-memory operations and would stall
+    // on the ring's outstanding loads.)
+    const int stride = gridDim.x;
+    auto open_entry = [&](int e, int &u0, int &u1, int &share, int &done) {
+        done = 0;
+        if (e >= sk.sk_wgs) {
+            share = -1;
+            u0 = (e - sk.sk_wgs) * nk;
+            u1 = u0 + nk;
+        } else {
+            share = e;
+            u0 = sk.dp_tiles * nk + e * sk.q + (e < sk.r ? e : sk.r);
+            u1 = u0 + sk.q + (e < sk.r ? 1 : 0);
+        }
+    };
+    // the next piece as (tile, first slice, end slice, slot in `part`); false when the list is exhausted
+    auto next_piece = [&](int &e, int &u0, int &u1, int &share, int &done, int &pid, int &kt_begin, int &kt_end, int &slot) {
+        if (u0 >= u1) {
+            if (e >= entries) return false;
+            e += stride;
+            if (e >= entries) return false;
+            open_entry(e, u0, u1, share, done);
+        }
+        pid = u0 / nk;
+        kt_begin = u0 - pid * nk;
+        kt_end = (u1 - u0 < nk - kt_begin) ? kt_begin + (u1 - u0) : nk;
+        slot = 2 * share + (done ? 1 : 0);
+        u0 += kt_end - kt_begin;
+        ++done;
+        return true;
+    };
+
+    // ---- the loads' side
+    int l_e = blockIdx.x, l_u0 = 0, l_u1 = 0, l_share = -1, l_done = 0;
+    int l_pid = 0, l_kt_begin = 0, l_kt_end = 0, l_slot = 0;
+    bool l_more;          // a piece is open on the loads' side
+    int l_left = 0;       // slices of it not yet requested
+    int row_off[T::kALoads], iy0[T::kALoads], ix0[T::kALoads], f_base[T::kBLoads];
+    int kpos = 0, ky = 0, kx = 0, ci = 0, k_limit = 0;
+    int va[T::kALoads], vb[T::kBLoads];
+    auto open_load_piece = [&]() {   // gather data of piece lp: as at the top of a piece in conv_dma
+        int tile_m, tile_n;
+        sk_tile_coords(l_pid, sk.dp_tiles, tiles_m, tiles_n, tile_m, tile_n);
+        const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
+        k_limit = (l_kt_end * BK < K) ? l_kt_end * BK : K;
+#pragma unroll
+        for (int j = 0; j < T::kALoads; ++j) {
+            const int m = m0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
+            if (m < M) {
+                int img, oy, ox;
+                pixel_of_row(g, m, img, oy, ox);
+                iy0[j] = oy * g.sh - g.pt;
+                ix0[j] = ox * g.sw - g.pl;
+                row_off[j] = ((img * g.H + iy0[j]) * g.W + ix0[j]) * g.C;
+            } else {
+                iy0[j] = ix0[j] = -(1 << 20);
+                row_off[j] = 0;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < T::kBLoads; ++j) {
+            const int n = n0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
+            f_base[j] = n < N ? n * K * 4 : kOutOfRange;
+        }
+        kpos = l_kt_begin * BK + kc_chunk(lane, wave) * 4;
+        const int tap = kpos / g.C;
+        ci = kpos - tap * g.C;
+        ky = tap / g.kw;
+        kx = tap - ky * g.kw;
+        l_left = l_kt_end - l_kt_begin;
+    };
+    // offsets of the next slice in the workgroup's order (all out of range once its list is exhausted)
+    auto next_offsets = [&]() {
+        if (l_more && l_left == 0) {
+            l_more = next_piece(l_e, l_u0, l_u1, l_share, l_done, l_pid, l_kt_begin, l_kt_end, l_slot);
+            if (l_more) open_load_piece();
+        }
+        if (!l_more) {
+#pragma unroll
+            for (int j = 0; j < T::kALoads; ++j) va[j] = kOutOfRange;
+#pragma unroll
+            for (int j = 0; j < T::kBLoads; ++j) vb[j] = kOutOfRange;
+            return;
+        }
+        const bool k_ok = kpos < k_limit;
+        const int tap_off = (ky * g.W + kx) * g.C + ci;
+#pragma unroll
+        for (int j = 0; j < T::kALoads; ++j) {
+            const bool ok = k_ok && (unsigned)(iy0[j] + ky) < (unsigned)g.H && (unsigned)(ix0[j] + kx) < (unsigned)g.W;
+            va[j] = ok ? (row_off[j] + tap_off) * 4 : kOutOfRange;
+        }
+#pragma unroll
+        for (int j = 0; j < T::kBLoads; ++j) vb[j] = (k_ok && f_base[j] != kOutOfRange) ? f_base[j] + kpos * 4 : kOutOfRange;
+        kpos += BK;
+        ci += BK;
+        while (ci >= g.C) {
+            ci -= g.C;
+            if (++kx == g.kw) {
+                kx = 0;
+                ++ky;
+            }
+        }
+        --l_left;
+    };
+    auto request = [&](float *wr) {
+#pragma unroll
+        for (int j = 0; j < T::kALoads; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t *)(wr + (4 * j + wave) * 256), 16, va[j], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < T::kBLoads; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_t *)(wr + T::kAFloats + (4 * j + wave) * 256), 16,
+                                                     vb[j], 0, 0, 0);
+    };
+
+    // ---- the multiplications' side
+    int c_e = blockIdx.x, c_u0 = 0, c_u1 = 0, c_share = -1, c_done = 0;
+    int c_pid = 0, c_kt_begin = 0, c_kt_end = 0, c_slot = 0;   // the piece being multiplied
+    int c_left = 0;        // slices of it still to multiply
+    int c_m0 = 0, c_n0 = 0;
+    ColumnRaw raw[TN];     // its epilogue parameters, requested when it is opened
+    auto open_compute_piece = [&]() {
+        int tile_m, tile_n;
+        sk_tile_coords(c_pid, sk.dp_tiles, tiles_m, tiles_n, tile_m, tile_n);
+        c_m0 = tile_m * T::BM;
+        c_n0 = tile_n * T::BN;
+        c_left = c_kt_end - c_kt_begin;
+        if (c_kt_begin == 0 && c_kt_end == nk && g.win) {
+            const int col_first = c_n0 + (wave & 1) * 32 * TN + (lane & 31);
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn) raw[tn] = column_raw(ep, col_first + tn * 32, col_first + tn * 32 < N);
+        }
+    };
+
+    v16f acc[TM][TN];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    };
+    auto finish_piece = [&]() {
+        acc_settle(acc);
+        if (c_kt_begin == 0 && c_kt_end == nk) {
+            const int row0 = c_m0 + (wave >> 1) * 32 * TM, col0 = c_n0 + (wave & 1) * 32 * TN;
+            if (!g.win) {
+                store_tile<TM, TN>(acc, out, (size_t)N, M, N, row0, col0, lane, ep);
+            } else {
+                ColumnParams cp[TN];
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn) cp[tn] = column_params(ep, raw[tn]);
+                if (pool) store_tile_windows<TM, TN, true>(acc, out, g, row0, col0, lane, ep, cp);
+                else store_tile_windows<TM, TN, false>(acc, out, g, row0, col0, lane, ep, cp);
+            }
+        } else {
+            float *slot = part + (size_t)c_slot * (T::BM * T::BN);
+            store_tile_impl<TM, TN, false, false>(acc, slot, (size_t)T::BN, T::BM, T::BN, (wave >> 1) * 32 * TM,
+                                                  (wave & 1) * 32 * TN, lane, Epilogue{});
+        }
+    };
+
+    // total slices of this workgroup
+    int total = 0;
+    {
+        int e = blockIdx.x, u0 = 0, u1 = 0, share = -1, done = 0, pid, kb, ke, slot;
+        if (e < entries) {
+            open_entry(e, u0, u1, share, done);
+            while (next_piece(e, u0, u1, share, done, pid, kb, ke, slot)) total += ke - kb;
+        }
+    }
+    if (total == 0) return;
+
+    __builtin_amdgcn_s_setprio(3);
+    open_entry(l_e, l_u0, l_u1, l_share, l_done);
+    l_more = next_piece(l_e, l_u0, l_u1, l_share, l_done, l_pid, l_kt_begin, l_kt_end, l_slot);
+    open_load_piece();
+    open_entry(c_e, c_u0, c_u1, c_share, c_done);
+    next_piece(c_e, c_u0, c_u1, c_share, c_done, c_pid, c_kt_begin, c_kt_end, c_slot);
+    open_compute_piece();
+    __builtin_amdgcn_sched_barrier(0);   // the parameter loads are older than every load of the ring
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) {
+        next_offsets();
+        request(lds + s * T::kStageFloats);
+    }
+    clear_acc();
+    int rd_stage = 0, wr_stage = STAGES - 1;
+    ring_sync<(STAGES - 2) * T::kLoads>();   // the first slice has landed
+    __builtin_amdgcn_s_setprio(0);
+    Frag<TM, TN> frag[2];
+    load_frag_swz<TM, TN, true>(frag[0], lds, lds + T::kAFloats, 0, wave >> 1, wave & 1, lane & 31, lane >> 5);
+    next_offsets();
+    for (int t = 0; t < total; ++t) {
+        const int nx_stage = rd_stage + 1 == STAGES ? 0 : rd_stage + 1;
+        dma_step_mid<TM, TN, true, STAGES>(lds + wr_stage * T::kStageFloats, lds + rd_stage * T::kStageFloats,
+                                           lds + nx_stage * T::kStageFloats, rsrc_a, rsrc_b, va, vb, acc, frag, wave, lane);
+        next_offsets();   // of the slice the next step requests
+        rd_stage = nx_stage;
+        wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
+        if (--c_left == 0) {
+            __builtin_amdgcn_s_setprio(3);
+            finish_piece();
+            if (next_piece(c_e, c_u0, c_u1, c_share, c_done, c_pid, c_kt_begin, c_kt_end, c_slot)) {
+                open_compute_piece();
+                clear_acc();
+            }
+            // No load into registers may be outstanding when the K loop resumes: the compiler, which cannot know
+            // that the parameter loads above never return into the registers the loop's LDS reads write, would
+            // otherwise wait for ALL vector-memory operations — the ring's loads included — at the top of every
+            // iteration.
+            wait_vmcnt<0>();
+            __builtin_amdgcn_s_setprio(0);
+        }
+    }
+    wait_vmcnt<0>();   // the trailing empty loads still target this workgroup's LDS
 #endif
 }
 
@@ -637,6 +1152,25 @@ int conv_dma_slots() {
     return per_cu * num_cus();
 }
 
+// The same for conv_dma_stream, whose grid is exactly this number.
+template <int TM, int TN, int STAGES>
+int conv_stream_slots() {
+    static int per_cu = 0;
+    if (!per_cu) {
+        using T = DmaTile<TM, TN, true, STAGES>;
+        auto kern = conv_dma_stream<TM, TN, STAGES>;
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)T::kLdsBytes);
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, kThreads, T::kLdsBytes) != hipSuccess || n < 1) {
+            (void)hipGetLastError();
+            n = 1;
+        }
+        per_cu = n;
+    }
+    return per_cu * num_cus();
+}
+
 template <int TM, int TN, int STAGES, bool MID>
 SkPlan conv_dma_plan(const ConvGeom &g, bool allow_shared) {
     using T = DmaTile<TM, TN, true, STAGES>;
@@ -658,12 +1192,40 @@ int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGe
     const long tiles = (long)((g.M + T::BM - 1) / T::BM) * ((g.OC + T::BN - 1) / T::BN);
     const int nk = (g.K + BK - 1) / BK;
     const SkPlan p = conv_dma_plan<TM, TN, STAGES, MID>(g, scratch != nullptr);
-    note_kernel("conv_dma<%d,%d,%d,%s>%s%s", TM, TN, STAGES, MID ? "true" : "false", p.sk_wgs ? " + conv_sk_finish" : "",
-                pool ? " (pooled)" : "");
-    auto kern = conv_dma<TM, TN, STAGES, MID>;
-    kern<<<(unsigned)(p.dp_tiles + p.sk_wgs), kThreads, T::kLdsBytes, stream()>>>(
-        in, filt, out, g, (unsigned)in_bytes, (unsigned)filt_bytes, ep, p, scratch, pool ? 1 : 0);
-    SWC_LAUNCH_CHECK();
+    // Workgroups that stay and walk a list of pieces (conv_dma_stream): off unless SWC_HIP_CONV_STREAM=1 (test-only) —
+    // on the layer shapes measured it is 2 - 4 % behind one workgroup per tile (see the kernel's comment).
+    bool staying = false;
+    if constexpr (MID) {
+        const char *e = getenv("SWC_HIP_CONV_STREAM");
+        const int slots = conv_stream_slots<TM, TN, STAGES>();
+        staying = e && e[0] == '1' && p.dp_tiles + p.sk_wgs > slots;
+        if (staying) {
+            note_kernel("conv_dma_stream<%d,%d,%d>%s%s", TM, TN, STAGES, p.sk_wgs ? " + conv_sk_finish" : "",
+                        pool ? " (pooled)" : "");
+            conv_dma_stream<TM, TN, STAGES><<<(unsigned)slots, kThreads, T::kLdsBytes, stream()>>>(
+                in, filt, out, g, (unsigned)in_bytes, (unsigned)filt_bytes, ep, p, scratch, pool ? 1 : 0);
+            SWC_LAUNCH_CHECK();
+        }
+    }
+    bool lean = false;   // the variant with a K loop free of vector-ALU work (conv_dma_lean); SWC_HIP_CONV_LEAN=0 (test-only) rules it out
+    if constexpr (TM == 1 && TN == 1 && STAGES == 3 && MID) {
+        const char *e = getenv("SWC_HIP_CONV_LEAN");
+        lean = !staying && g.C % BK == 0 && !(e && e[0] == '0');
+        if (lean) {
+            note_kernel("conv_dma_lean%s%s", p.sk_wgs ? " + conv_sk_finish" : "", pool ? " (pooled)" : "");
+            conv_dma_lean<<<(unsigned)(p.dp_tiles + p.sk_wgs), kThreads, T::kLdsBytes, stream()>>>(
+                in, filt, out, g, (unsigned)in_bytes, (unsigned)filt_bytes, ep, p, scratch, pool ? 1 : 0);
+            SWC_LAUNCH_CHECK();
+        }
+    }
+    if (!staying && !lean) {
+        note_kernel("conv_dma<%d,%d,%d,%s>%s%s", TM, TN, STAGES, MID ? "true" : "false", p.sk_wgs ? " + conv_sk_finish" : "",
+                    pool ? " (pooled)" : "");
+        auto kern = conv_dma<TM, TN, STAGES, MID>;
+        kern<<<(unsigned)(p.dp_tiles + p.sk_wgs), kThreads, T::kLdsBytes, stream()>>>(
+            in, filt, out, g, (unsigned)in_bytes, (unsigned)filt_bytes, ep, p, scratch, pool ? 1 : 0);
+        SWC_LAUNCH_CHECK();
+    }
     if (p.sk_wgs) {
         conv_sk_finish<T::BM, T::BN><<<dim3((unsigned)(tiles - p.dp_tiles), T::BM / 16), 256, 0, stream()>>>(
             out, scratch, g, nk, p, ep, (g.OC % 4 == 0 && aligned16(out)) ? 1 : 0, pool ? 1 : 0);

@@ -556,9 +556,9 @@ def test_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, pads, s
     for with_bn, relu in [(True, True), (False, True), (False, False), (True, False)]:
         kw = dict(pads=pads, bn=dbn if with_bn else None, eps=1e-5, relu=relu)
         fused = rt.conv2d(dx, df, db, pool=pool, **kw)
-        assert rt.last_kernel().startswith("conv_dma<") and rt.last_kernel().endswith("(pooled)"), rt.last_kernel()
+        assert rt.last_kernel().startswith("conv_dma") and rt.last_kernel().endswith("(pooled)"), rt.last_kernel()
         plain = rt.conv2d(dx, df, db, **kw)
-        assert rt.last_kernel().startswith("conv_dma<"), rt.last_kernel()
+        assert rt.last_kernel().startswith("conv_dma"), rt.last_kernel()
         want = rt.maxpool(plain, *pool).numpy()
         assert_bit_exact(fused.numpy(), want, f"pooled in the epilogue vs conv then maxpool (bn {with_bn}, relu {relu})")
     # against the oracle (full-size layers: the first image only)
@@ -577,6 +577,50 @@ def test_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, pads, s
     assert scaled_err(raster, ref, scale) < TOL
     if not slots and rt.last_kernel().find("conv_sk_finish") < 0:
         assert_bit_exact(raster, got, "window order vs raster order, every tile whole")
+
+
+@pytest.mark.parametrize("idims,fdims,pads", [((32, 56, 56, 64), (128, 3, 3, 64), (1, 1, 1, 1)),
+                                              ((32, 28, 28, 128), (128, 3, 3, 128), (1, 1, 1, 1)),
+                                              ((3, 10, 6, 32), (70, 3, 3, 32), (1, 1, 1, 1)),
+                                              ((2, 9, 11, 96), (64, 5, 5, 96), (2, 2, 2, 2)),     # odd output: raster order
+                                              ((4, 16, 16, 64), (64, 1, 1, 64), (0, 0, 0, 0))])
+@pytest.mark.parametrize("slots", [None, "7"])
+def test_conv_kernel_forms_agree_bit_for_bit(rt, idims, fdims, pads, slots, monkeypatch):
+    """The three forms of the 64x64-tile kernel — conv_dma, conv_dma_lean (channel counts that are multiples of 32:
+    no vector-ALU work in the K loop) and conv_dma_stream (workgroups that stay, opt-in) — walk K in the same order
+    and cut the same tiles: the same bits, whole and cut tiles, plain and pooled."""
+    print("case conv kernel forms", idims, fdims, pads, slots, flush=True)
+    if slots:
+        monkeypatch.setenv("SWC_HIP_CONV_SLOTS", slots)
+    rng = np.random.default_rng(sum(idims) * 3 + sum(fdims))
+    oc = fdims[0]
+    x = rng.standard_normal(idims).astype(np.float32)
+    f = (rng.standard_normal(fdims) / np.sqrt(np.prod(fdims[1:]))).astype(np.float32)
+    b = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    bn = up(rt, rng.uniform(-0.1, 0.1, oc).astype(np.float32), rng.uniform(0.5, 2.0, oc).astype(np.float32),
+            rng.uniform(0.5, 1.5, oc).astype(np.float32), rng.uniform(-0.1, 0.1, oc).astype(np.float32))
+    dx, df, db = up(rt, x, f, b)
+    kw = dict(pads=pads, bn=bn, eps=1e-5, relu=True)
+    lean = rt.conv2d(dx, df, db, **kw).numpy()
+    if slots and not rt.last_kernel().startswith("conv_dma_lean"):
+        pytest.skip("on a chip of seven workgroups the planner gives this layer another tile shape: " + rt.last_kernel())
+    assert rt.last_kernel().startswith("conv_dma_lean"), rt.last_kernel()
+    monkeypatch.setenv("SWC_HIP_CONV_LEAN", "0")
+    plain = rt.conv2d(dx, df, db, **kw).numpy()
+    assert rt.last_kernel().startswith("conv_dma<1,1,3,true>"), rt.last_kernel()
+    assert_bit_exact(lean, plain, "conv_dma_lean vs conv_dma")
+    monkeypatch.setenv("SWC_HIP_CONV_STREAM", "1")
+    staying = rt.conv2d(dx, df, db, **kw).numpy()
+    assert_bit_exact(staying, plain, "conv_dma_stream vs conv_dma")
+    if idims[1] % 2 == 0 and idims[2] % 2 == 0 and fdims[1] != 5:
+        pool = ((2, 2), (2, 2))
+        staying_pooled = rt.conv2d(dx, df, db, pool=pool, **kw).numpy()
+        monkeypatch.delenv("SWC_HIP_CONV_STREAM")
+        monkeypatch.delenv("SWC_HIP_CONV_LEAN")
+        lean_pooled = rt.conv2d(dx, df, db, pool=pool, **kw).numpy()
+        assert rt.last_kernel().startswith("conv_dma_lean") and rt.last_kernel().endswith("(pooled)"), rt.last_kernel()
+        assert_bit_exact(lean_pooled, rt.maxpool(rt.upload(plain), *pool).numpy(), "pooled, lean")
+        assert_bit_exact(staying_pooled, lean_pooled, "pooled, staying")
 
 
 def test_conv_with_a_pooling_the_epilogue_cannot_do(rt, oracle):
