@@ -628,14 +628,40 @@ __global__ __launch_bounds__(kThreads) void conv_dma_lean(const float *__restric
         if (whole && g.win) raw[0] = column_raw(ep, col_first, col_first < N);
         __builtin_amdgcn_sched_barrier(0);
 
-        // per-lane constants of the two rows of A and of B that this lane gathers for
+        // per-lane constants of the two rows of A and of B that this lane gathers for.  In window order with at
+        // least eight windows per output row the pixel of row m0 + r follows from the tile's first window (one
+        // division on scalars) by at most two carries — the general map costs four divisions per row, and vector
+        // instructions here are paid for in matrix-core time.
+        const int pw = g.OW >> 1, ph = g.OH >> 1;
+        const bool near = g.win && pw >= 8;
+        int img_t = 0, py_t = 0, px_t = 0;
+        if (near) {
+            const int w0 = m0 >> 2, t0 = w0 / pw;
+            px_t = w0 - t0 * pw;
+            img_t = t0 / ph;
+            py_t = t0 - img_t * ph;
+        }
         int row_off[2], iy0[2], ix0[2], vb[2];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            const int m = m0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
+            const int r = (4 * j + wave) * 8 + kc_row_in_load(lane);
+            const int m = m0 + r;
             if (m < M) {
                 int img, oy, ox;
-                pixel_of_row(g, m, img, oy, ox);
+                if (near) {
+                    int px = px_t + (r >> 2), py = py_t;
+                    img = img_t;
+#pragma unroll
+                    for (int c = 0; c < 2; ++c)
+                        if (px >= pw) {
+                            px -= pw;
+                            if (++py == ph) py = 0, ++img;
+                        }
+                    oy = 2 * py + ((r >> 1) & 1);
+                    ox = 2 * px + (r & 1);
+                } else {
+                    pixel_of_row(g, m, img, oy, ox);
+                }
                 iy0[j] = oy * g.sh - g.pt;
                 ix0[j] = ox * g.sw - g.pl;
                 row_off[j] = (((img * g.H + iy0[j]) * g.W + ix0[j]) * g.C) * 4 + chunk16;

@@ -332,7 +332,31 @@ void HipCodegen::emitExecute() {
                 auto *op = static_cast<OpNode *>(node);
                 if (!op->isRunOnce() && op->getOp()->getOpName() == "Scatter") uploads.push_back(op);
             }
-        const bool prefetch = config_.hip_prefetch && !uploads.empty();
+        // With prefetching the loader overwrites its host buffers with batch i+1 as soon as the graph of batch i has
+        // been launched.  A host op of the iteration, or a displayed tensor, that reads one of those buffers would see
+        // the next batch: such a program keeps the plain loop.
+        auto hostReadsLoaderBuffers = [&]() {
+            Tensor *lt = T(loaderLabelNode()), *dt = T(loaderDataNode());
+            for (int i = 0; i < graph_->topologyNum(); ++i)
+                for (int j = 0; j < graph_->getNumInTopoLevel(i); ++j) {
+                    IRNode *node = graph_->getNodeInTopo(i, j);
+                    if (node->nodeType() != OP_NODE) continue;
+                    auto *op = static_cast<OpNode *>(node);
+                    const std::string type = op->getOp()->getOpName();
+                    if (op->isRunOnce() || isDeviceComputeOp(op) || type == "Scatter" || type == "Gather") continue;
+                    for (IRNode *p : op->getParentNodes())
+                        if (p->nodeType() == TENSOR_NODE && (T(p) == lt || T(p) == dt)) return true;
+                }
+            if (config_.display > 0)
+                for (TensorNode *tn : graph_->getDisplayTensorNodes())
+                    if (tn->getTensor() == lt || tn->getTensor() == dt) return true;
+            return false;
+        };
+        bool prefetch = config_.hip_prefetch && !uploads.empty();
+        if (prefetch && hostReadsLoaderBuffers()) {
+            prefetch = false;
+            writer_ << "// (hip_prefetch: a host op or a displayed tensor reads the loader's host buffers: no prefetching)\n";
+        }
         const std::string next = "loader.next(" + nameOf(loaderLabelNode()) + ", " + nameOf(loaderDataNode()) + ")";
         auto stageName = [&](OpNode *u) { return nameOf(u->getChildNode(0)) + "_stage"; };
         auto bytesOf = [&](OpNode *u) {

@@ -110,6 +110,9 @@ int main(int argc, char **argv) {
         return 2;
     }
     string model = argv[1];
+    // "mnist_loader+labels": the data-loader model with the label batch among the displayed tensors
+    const bool show_labels = model == "mnist_loader+labels";
+    if (show_labels) model = "mnist_loader";
     const string target = argv[2];
     const size_t batch = argc > 3 ? strtoul(argv[3], nullptr, 10) : 0;
     const size_t iters = argc > 4 ? strtoul(argv[4], nullptr, 10) : 0;
@@ -284,6 +287,7 @@ int main(int argc, char **argv) {
         GpO(graph, fc0, tanh0, fc1, softmax, argmax_o, accuracy_o);
         graph->setInferDataNodes(label, data0);
         graph->addDisplayTensorNodes(accuracy_t);
+        if (show_labels) graph->addDisplayTensorNodes(label);   // the display block then reads the loader's host buffer
     } else if (training) {
         // Training programs in the style of the reference's test/engine/testEngineLenetDistTrain.cpp (one process,
         // no MPI): the inference graph ends in MatrixSoftmaxWithLoss, the parameters are marked for training, and

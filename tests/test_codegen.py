@@ -362,6 +362,19 @@ def test_prefetching_batch_loop_structure(gen, tmp_path):
     build_hip(tmp_path)
 
 
+def test_prefetching_is_dropped_when_the_host_reads_the_loaders_buffers(gen, tmp_path):
+    """With prefetching the loader refills its host buffers right after the graph launch; a displayed tensor (or a host
+    op) that reads one of them would show the next batch, so such a program keeps the plain loop."""
+    code = generate(gen, "mnist_loader+labels", "hip", tmp_path, 44, prefetch=True)
+    assert "no prefetching" in code and "swc_hip_copy_h2d_async" not in code and "_stage" not in code
+    assert "while(loader.next(" in code and "swc_hip_graph_launch(swc_graph)" in code
+    body = code[code.index("while(loader.next("):]
+    assert "printMatrix(selected" in body.replace("cpu0_", "") or "printMatrix(" in body
+    build_hip(tmp_path)
+    # the same model without the label on display prefetches
+    assert "swc_hip_copy_h2d_async" in generate(gen, "mnist_loader", "hip", tmp_path, 44, prefetch=True)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("graph,prefetch", [(False, False), (True, False), (True, True)])
 def test_batch_loop_hip_program(gen, oracle, tmp_path, graph, prefetch):
