@@ -515,6 +515,75 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
 }
 
 #if __HIP_DEVICE_COMPILE__
+// store_tile_windows with as few vector instructions as the arithmetic allows (they are paid for in matrix-core time):
+// stores through a buffer descriptor of the output — one 32-bit offset per window and column block, the four pixels of
+// a window at scalar offsets from it — and the window's coordinates from one division on scalars.  No second summand;
+// the output below 2 GiB.
+template <int TM, int TN, bool POOL>
+__device__ __forceinline__ void store_tile_windows_buf(const v16f (&acc)[TM][TN], __amdgpu_buffer_rsrc_t rsrc_out,
+                                                       const ConvGeom &g, int row0, int col0, int lane, const Epilogue &ep,
+                                                       const ColumnParams (&cp)[TN]) {
+    const int l32 = lane & 31, h = lane >> 5;
+    const int N = g.OC, pw = g.OW >> 1, ph = g.OH >> 1;
+    const bool bn = ep.bn_mean != nullptr;
+    const int s_px = N * 4, s_row = g.OW * N * 4;   // byte steps to the window's right and lower pixels
+    // this lane's windows: w0, w0 + 2, ... with w0 = row0 / 4 + h (row0 is the same for the whole wavefront)
+    int w = row0 >> 2;
+    int px, py, img;
+    {
+        const int t = w / pw;
+        px = w - t * pw;
+        img = t / ph;
+        py = t - img * ph;
+    }
+    w += h;
+    px += h;
+    if (px >= pw) {
+        px -= pw;
+        if (++py == ph) py = 0, ++img;
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (4 * w < g.M) {
+                const int base = POOL ? w * N : ((img * g.OH + 2 * py) * g.OW + 2 * px) * N;
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn) {
+                    const int col = col0 + tn * 32 + l32;
+                    if (col >= N) continue;
+                    const int voff = (base + col) * 4;
+                    float x[4];
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        x[d] = acc[tm][tn][4 * q + d] + cp[tn].bias;
+                        if (bn) x[d] = fmaf(x[d] - cp[tn].mean, cp[tn].slope, cp[tn].beta);
+                    }
+                    if (ep.relu) {
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) x[d] = (x[d] > 0.f) ? x[d] : 0.f;
+                    }
+                    if (POOL) {
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, window_max(x[0], x[1], x[2], x[3])),
+                                                              rsrc_out, voff, 0, 0);
+                    } else {
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[0]), rsrc_out, voff, 0, 0);
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[1]), rsrc_out, voff, s_px, 0);
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[2]), rsrc_out, voff, s_row, 0);
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[3]), rsrc_out, voff, s_row + s_px, 0);
+                    }
+                }
+            }
+            w += 2;
+            px += 2;
+            while (px >= pw) {
+                px -= pw;
+                if (++py == ph) py = 0, ++img;
+            }
+        }
+    }
+}
+
 // The four loads of a wavefront for one slice of a 64 x 64 tile into stage `wr` (conv_dma_lean): per-lane offsets
 // va/vb, the position inside the tap (A) and along K (B) as scalar offsets.
 __device__ __forceinline__ void lean_request(char *__restrict__ wr, __amdgpu_buffer_rsrc_t rsrc_a, __amdgpu_buffer_rsrc_t rsrc_b,
@@ -572,8 +641,9 @@ __device__ __forceinline__ void lean_step(char *__restrict__ wr, const char *__r
 __global__ __launch_bounds__(kThreads) void conv_dma_lean(const float *__restrict__ in, const float *__restrict__ filt,
                                                           float *__restrict__ out, ConvGeom g, unsigned in_bytes,
                                                           unsigned filt_bytes, Epilogue ep, SkPlan sk,
-                                                          float *__restrict__ part, int pool) {
+                                                          float *__restrict__ part, int pool, unsigned out_bytes) {
 #if __HIP_DEVICE_COMPILE__
+    // out_bytes: size of the output if it is below 2 GiB (stores then go through a buffer descriptor), else 0
     constexpr int TM = 1, TN = 1, STAGES = 3;
     using T = DmaTile<TM, TN, true, STAGES>;
     static_assert(T::kALoads == 2 && T::kBLoads == 2, "");
@@ -741,9 +811,17 @@ __global__ __launch_bounds__(kThreads) void conv_dma_lean(const float *__restric
         acc_settle(acc);
         if (whole) {
             const int row0 = m0 + (wave >> 1) * 32, col0 = n0 + (wave & 1) * 32;
-            if (!g.win) store_tile<1, 1>(acc, out, (size_t)N, M, N, row0, col0, lane, ep);
-            else if (pool) store_tile_windows<1, 1, true>(acc, out, g, row0, col0, lane, ep, cp);
-            else store_tile_windows<1, 1, false>(acc, out, g, row0, col0, lane, ep, cp);
+            if (!g.win) {
+                store_tile<1, 1>(acc, out, (size_t)N, M, N, row0, col0, lane, ep);
+            } else if (out_bytes && !ep.residual) {
+                const __amdgpu_buffer_rsrc_t rsrc_out = make_rsrc(out, out_bytes);
+                if (pool) store_tile_windows_buf<1, 1, true>(acc, rsrc_out, g, row0, col0, lane, ep, cp);
+                else store_tile_windows_buf<1, 1, false>(acc, rsrc_out, g, row0, col0, lane, ep, cp);
+            } else if (pool) {
+                store_tile_windows<1, 1, true>(acc, out, g, row0, col0, lane, ep, cp);
+            } else {
+                store_tile_windows<1, 1, false>(acc, out, g, row0, col0, lane, ep, cp);
+            }
         } else {
             float *slot = part + (size_t)(2 * share + (piece ? 1 : 0)) * (T::BM * T::BN);
             store_tile_impl<1, 1, false, false>(acc, slot, (size_t)T::BN, T::BM, T::BN, (wave >> 1) * 32, (wave & 1) * 32, lane,
@@ -1239,8 +1317,10 @@ int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGe
         lean = !staying && g.C % BK == 0 && !(e && e[0] == '0');
         if (lean) {
             note_kernel("conv_dma_lean%s%s", p.sk_wgs ? " + conv_sk_finish" : "", pool ? " (pooled)" : "");
+            const size_t out_bytes = (size_t)(pool ? g.M / 4 : g.M) * g.OC * 4;
             conv_dma_lean<<<(unsigned)(p.dp_tiles + p.sk_wgs), kThreads, T::kLdsBytes, stream()>>>(
-                in, filt, out, g, (unsigned)in_bytes, (unsigned)filt_bytes, ep, p, scratch, pool ? 1 : 0);
+                in, filt, out, g, (unsigned)in_bytes, (unsigned)filt_bytes, ep, p, scratch, pool ? 1 : 0,
+                out_bytes < kMaxDmaBytes ? (unsigned)out_bytes : 0u);
             SWC_LAUNCH_CHECK();
         }
     }
