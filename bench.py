@@ -15,7 +15,9 @@ Also in the line:
                 with HIP events on the library's stream inside the timed region
   kernels       per-launch times of the headline graph
   graph_replay  the same K steps replayed as one HIP graph per step (no per-kernel
-                events in the loop): what a launch-bound small graph gains
+                events in the loop): what a launch-bound small graph gains; `shader_clock_ghz`: the clock the
+                chip ran at meanwhile (one-wavefront watcher of the bench-only library on a stream of its own;
+                the datasheet peaks assume 2.4 GHz)
   incl_transfers  the step with the input batch uploaded and the result downloaded
                 each time (never the headline value); `overlapped_uploads`: the same with
                 the next batch's upload on a second stream while this batch is computed
@@ -251,10 +253,14 @@ def run_config(rt, graphs, cfg, steps, warmup):
         rt.graph_launch(handle)
     rt.sync()
     graph_wall = time.perf_counter() - t0
+    # the shader clock while that graph replays back to back (the datasheet peaks assume 2.4 GHz; under sustained
+    # matrix work the chip settles lower, by an amount that depends on the kernel and on the data)
+    clock = rt.shader_clock_ghz(lambda: rt.graph_launch(handle), graph_wall * 1e3 / steps)
     rt.graph_destroy(handle)
     return dict(batch=batch, wall_s=wall, gpu_ms=gpu_ms, ms_per_step=wall * 1e3 / steps,
                 samples_per_s=batch * steps / wall, kernels=rows,
-                graph_replay=dict(ms_per_step=graph_wall * 1e3 / steps, samples_per_s=batch * steps / graph_wall))
+                graph_replay=dict(ms_per_step=graph_wall * 1e3 / steps, samples_per_s=batch * steps / graph_wall,
+                                  shader_clock_ghz=clock))
 
 
 def run_training(rt, iters=20):
@@ -435,7 +441,10 @@ def main():
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS_FP32_MFMA, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_TFLOPS_FP32_MFMA, "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": ROOFLINE_KERNEL + " (both launches per step: 4096x784x4096 and 4096x4096x4096)",
-                     "flop_per_launch": flop / len(gemm), "avg_launch_ms": secs * 1e3 / len(gemm)},
+                     "flop_per_launch": flop / len(gemm), "avg_launch_ms": secs * 1e3 / len(gemm),
+                     # for information, not part of frac: the clock the step ran at and the MFMA peak at that clock
+                     "shader_clock_ghz": head["graph_replay"]["shader_clock_ghz"],
+                     "peak_at_that_clock": PEAK_TFLOPS_FP32_MFMA * head["graph_replay"]["shader_clock_ghz"] / 2.4},
         "gpu_ms_per_step": head["gpu_ms"] / args.steps,
         "graph_replay": head["graph_replay"],
         "incl_transfers": with_transfers(rt, graphs, 2, max(5, min(args.steps, 20))),

@@ -21,6 +21,16 @@ extern "C" {
 int swc_hip_bench_probe_mfma_f32(void *hip_stream, int cus, float *scratch_dev, size_t scratch_floats, int iters,
                                  float *ms_out, double *flop_out);
 
+/* The shader clock while other work runs.  _start launches, on a stream of the bench library's own (default
+ * priority), ONE wavefront that writes n pairs (100 MHz wall-clock ticks, shader-clock counter) into samples_dev
+ * (2 n 64-bit words of device memory), sleeping sleeps x 8128 shader cycles (about 3.5 us each) between pairs,
+ * and returns at once; the watcher ends by itself after its n pairs.  The harness then enqueues the work it
+ * wants watched on its own stream, calls _wait, and reads the clock off consecutive pairs:
+ * GHz = 0.1 x (shader difference) / (wall difference).  One wavefront on one CU does not disturb a kernel that
+ * fills the chip.  1 < n <= 65536, 1 <= sleeps <= 64.  Return 0, or a non-zero hipError_t. */
+int swc_hip_bench_clock_watch_start(unsigned long long *samples_dev, int n, int sleeps);
+int swc_hip_bench_clock_watch_wait(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -31,6 +31,23 @@ __global__ __launch_bounds__(256) void mfma_rate_probe(float *out, int iters, fl
 #endif
 }
 
+// One wavefront that notes the 100 MHz wall clock and the shader clock counter side by side, `n` times, sleeping
+// `sleeps` x 8128 shader cycles in between, and ends by itself.
+__global__ __launch_bounds__(64) void clock_watch(unsigned long long *samples, int n, int sleeps) {
+#if __HIP_DEVICE_COMPILE__
+    for (int i = 0; i < n; ++i) {
+        const unsigned long long wall = wall_clock64(), shader = clock64();
+        if (threadIdx.x == 0) {
+            samples[2 * i] = wall;
+            samples[2 * i + 1] = shader;
+        }
+        for (int s = 0; s < sleeps; ++s) __builtin_amdgcn_s_sleep(127);
+    }
+#endif
+}
+
+hipStream_t g_watch_stream = nullptr;
+
 } // namespace
 
 #define PROBE_TRY(expr)                  \
@@ -60,5 +77,19 @@ extern "C" int swc_hip_bench_probe_mfma_f32(void *hip_stream, int cus, float *sc
     (void)hipEventDestroy(e1);
     // 32x32x2 MFMA = 2*32*32*2 = 4096 flop per wavefront instruction
     *flop_out = (double)blocks * 4 * (double)iters * kProbeUnroll * kProbeAcc * 4096.0;
+    return 0;
+}
+
+extern "C" int swc_hip_bench_clock_watch_start(unsigned long long *samples_dev, int n, int sleeps) {
+    if (!samples_dev || n <= 1 || n > (1 << 16) || sleeps < 1 || sleeps > 64) return (int)hipErrorInvalidValue;
+    if (!g_watch_stream) PROBE_TRY(hipStreamCreateWithFlags(&g_watch_stream, hipStreamNonBlocking));
+    clock_watch<<<1, 64, 0, g_watch_stream>>>(samples_dev, n, sleeps);
+    PROBE_TRY(hipGetLastError());
+    return 0;
+}
+
+extern "C" int swc_hip_bench_clock_watch_wait(void) {
+    if (!g_watch_stream) return (int)hipErrorInvalidValue;
+    PROBE_TRY(hipStreamSynchronize(g_watch_stream));
     return 0;
 }

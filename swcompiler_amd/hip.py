@@ -279,9 +279,8 @@ class SwcHip:
     def copy_sync(self):
         self._check(self.lib.swc_hip_copy_sync(), "swc_hip_copy_sync")
 
-    def probe_mfma_tflops(self, iters=2000):
-        """fp32 MFMA rate a register-only loop sustains (TFLOP/s) and its duration in ms; runs the bench-only
-        helper library (include/swc_hip_bench.h) on the library's stream"""
+    def _bench(self):
+        """the bench-only helper library (include/swc_hip_bench.h), loaded on first use"""
         if self._bench_lib is None:
             path = os.path.join(_HERE, "libswc_hip_bench.so")
             if not os.path.exists(path):
@@ -290,6 +289,41 @@ class SwcHip:
             self._bench_lib.swc_hip_bench_probe_mfma_f32.restype = C.c_int
             self._bench_lib.swc_hip_bench_probe_mfma_f32.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_size_t, C.c_int,
                                                                      C.POINTER(C.c_float), C.POINTER(C.c_double)]
+            self._bench_lib.swc_hip_bench_clock_watch_start.restype = C.c_int
+            self._bench_lib.swc_hip_bench_clock_watch_start.argtypes = [C.c_void_p, C.c_int, C.c_int]
+            self._bench_lib.swc_hip_bench_clock_watch_wait.restype = C.c_int
+            self._bench_lib.swc_hip_bench_clock_watch_wait.argtypes = []
+        return self._bench_lib
+
+    def shader_clock_ghz(self, fn, op_ms, watch_ms=4.0):
+        """The shader clock (GHz) while `fn` — which enqueues one op of about op_ms on the library's stream — runs
+        back to back: a one-wavefront watcher of the bench-only library notes the 100 MHz wall clock and the shader
+        clock counter every ~3.5 us on a stream of its own for watch_ms; fn is enqueued often enough to outlast it;
+        the figure is the median over consecutive samples of the middle 80 % of the watch."""
+        import numpy as np
+        lib = self._bench()
+        n = max(16, int(watch_ms * 1e3 / 3.6))
+        samples = self.empty((4 * n,))          # 2 n 64-bit words
+        self.sync()
+        rc = lib.swc_hip_bench_clock_watch_start(samples.ptr, n, 1)
+        if rc != 0:
+            raise SwcHipError(f"swc_hip_bench_clock_watch_start failed (hipError {rc})")
+        for _ in range(max(3, int(1.5 * watch_ms / max(op_ms, 1e-3)) + 2)):
+            fn()
+        rc = lib.swc_hip_bench_clock_watch_wait()
+        self.sync()
+        if rc != 0:
+            raise SwcHipError(f"swc_hip_bench_clock_watch_wait failed (hipError {rc})")
+        s = samples.numpy().view(np.uint64).reshape(n, 2).astype(np.float64)
+        samples.free()
+        s = s[n // 10: n - n // 10]
+        d = np.diff(s, axis=0)
+        return float(np.median(0.1 * d[:, 1] / d[:, 0]))
+
+    def probe_mfma_tflops(self, iters=2000):
+        """fp32 MFMA rate a register-only loop sustains (TFLOP/s) and its duration in ms; runs the bench-only
+        helper library (include/swc_hip_bench.h) on the library's stream"""
+        self._bench()
         self.sync()
         scratch = self.empty((512 * 512,))
         ms, flop = C.c_float(), C.c_double()
