@@ -26,6 +26,20 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
 
 
+def test_bench_library_exports_its_header():
+    """include/swc_hip_bench.h (measurement helpers, not part of the drop-in ABI) against libswc_hip_bench.so"""
+    import ctypes
+    text = open(os.path.join(ROOT, "include", "swc_hip_bench.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(swc_hip_bench_\w+)\s*\(", text)))
+    assert names == ["swc_hip_bench_clock_watch_start", "swc_hip_bench_clock_watch_wait", "swc_hip_bench_probe_mfma_f32"]
+    lib = ctypes.CDLL(os.path.join(ROOT, "swcompiler_amd", "libswc_hip_bench.so"))
+    for name in names:
+        assert hasattr(lib, name), name
+    # nothing of it leaks into the product header
+    assert "swc_hip_bench" not in open(os.path.join(ROOT, "include", "swc_hip.h")).read()
+
+
 def test_calls_fail_cleanly_without_device_or_init():
     if os.path.exists("/dev/kfd"):
         pytest.skip("a GPU is present; the no-device path cannot be forced")

@@ -194,3 +194,19 @@ def test_library_workspace_is_not_replaced_under_a_recorded_graph(rt):
         rt.graph_destroy(handle)
     rt.fcbias(a2, w2, None)                     # the graph is gone: the buffer may grow now
     rt.sync()
+
+
+@pytest.mark.gpu
+def test_shader_clock_watcher(rt):
+    """The bench-only library's one-wavefront clock watcher (swc_hip_bench_clock_watch_*): it ends by itself, the
+    work enqueued beside it runs undisturbed and correctly, and the clock it reads is a plausible shader clock —
+    no higher under a long matrix product than on an idle chip."""
+    idle = rt.shader_clock_ghz(lambda: None, 1.0, watch_ms=1.0)
+    assert 0.5 < idle < 3.0, idle
+    rng = np.random.default_rng(3)
+    a, b = rng.standard_normal((1024, 1024)).astype(np.float32), rng.standard_normal((1024, 1024)).astype(np.float32)
+    da, db, out = rt.upload(a), rt.upload(b), rt.empty((1024, 1024))
+    busy = rt.shader_clock_ghz(lambda: rt.matrixMatrixMul(da, db, out=out), 0.03, watch_ms=1.0)
+    assert 0.5 < busy <= idle + 0.05, (busy, idle)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    assert np.max(np.abs(out.numpy() - want)) < 1e-2
