@@ -2227,7 +2227,7 @@ __global__ __launch_bounds__(1024) void wgrad_small(float *__restrict__ part, co
 }
 
 // ---- bias gradient: masked column sums of outputG [M, OC]
-constexpr int kBiasRows = 256;   // rows per partial sum (enough workgroups to fill the chip at the sizes of interest)
+constexpr int kBiasRows = 128;   // rows per partial sum: 128 measured best on the cfg4 layers (256: 183 / 307 / 169 us for conv2dGrad, 128: 181 / 304 / 163, 64: 184 / 304 / 160)
 // A workgroup sums kBiasRows rows: thread = (VEC columns, row phase), the pixel coordinates of its rows kept
 // incrementally (no division in the loop); the 256/colsq phases of a column are combined in a fixed order.
 // colsq * VEC columns per workgroup in x (colsq a power of two), row chunks in y.
