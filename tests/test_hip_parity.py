@@ -188,6 +188,49 @@ def test_conv_vs_oracle(rt, oracle, idims, fdims, strides, pads):
                           oracle.relu(oracle.conv2d(xp, fp, b, fdims[1:3], strides, pads))) < TOL
 
 
+def _random_conv_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        c = int(rng.choice([1, 3, 4, 8, 20, 32, 36, 64, 96, 128]))
+        kh, kw = (int(v) for v in rng.choice([1, 2, 3, 5], 2))
+        sh, sw = (int(v) for v in rng.choice([1, 1, 2], 2))
+        pads = tuple(int(v) for v in rng.integers(0, 3, 4))      # top, left, bottom, right
+        n, h, w = int(rng.integers(1, 4)), int(rng.integers(4, 23)), int(rng.integers(4, 23))
+        oc = int(rng.choice([3, 16, 40, 64, 70, 128, 136]))
+        if h + pads[0] + pads[2] < kh or w + pads[1] + pads[3] < kw:
+            continue
+        cases.append(((n, h, w, c), (oc, kh, kw, c), (sh, sw), pads, [None, "7", "3"][len(cases) % 3]))
+    return cases
+
+
+@pytest.mark.parametrize("idims,fdims,strides,pads,slots", _random_conv_cases(48, 2024))
+def test_conv_random_shapes_integer_exact(rt, oracle, idims, fdims, strides, pads, slots, monkeypatch):
+    """Random layer shapes (channel counts for every kernel form, ragged tiles, strides, uneven padding), on a chip
+    pretended to hold 7 or 3 workgroups for two thirds of them so that tiles are cut along K: small-integer operands
+    make every order of summation exact, so the result must equal the oracle's bit for bit — plain, with ReLU and a
+    second summand, and with the 2x2 pooling where the output allows it."""
+    print("case random conv", idims, fdims, strides, pads, slots, flush=True)
+    if slots:
+        monkeypatch.setenv("SWC_HIP_CONV_SLOTS", slots)
+    rng = np.random.default_rng(sum(idims) * 7 + sum(fdims) * 3 + sum(pads))
+    x = rng.integers(-3, 4, idims).astype(np.float32)
+    f = rng.integers(-3, 4, fdims).astype(np.float32)
+    b = rng.integers(-3, 4, fdims[0]).astype(np.float32)
+    dx, df, db = up(rt, x, f, b)
+    want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
+    got = rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy()
+    kernel = rt.last_kernel()
+    assert_bit_exact(got, want, f"conv on integers [{kernel}]")
+    res = rng.integers(-3, 4, want.shape).astype(np.float32)
+    got = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True, residual=rt.upload(res)).numpy()
+    assert_bit_exact(got, oracle.relu(want + res), f"conv + summand + ReLU on integers [{rt.last_kernel()}]")
+    if want.shape[1] % 2 == 0 and want.shape[2] % 2 == 0:
+        pool = ((2, 2), (2, 2))
+        got = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True, pool=pool).numpy()
+        assert_bit_exact(got, oracle.maxpool(oracle.relu(want), *pool), f"conv + ReLU + pool on integers [{rt.last_kernel()}]")
+
+
 def test_conv_integer_valued_is_exact(rt):
     rng = np.random.default_rng(9)
     for idims, fdims, pads in [((2, 9, 10, 8), (40, 3, 3, 8), (1, 1, 1, 1)), ((1, 12, 12, 3), (70, 5, 5, 3), (2, 2, 2, 2))]:

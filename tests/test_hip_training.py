@@ -195,6 +195,43 @@ def test_conv2dGrad_vs_oracle(rt, oracle, idims, fdims, st, pd):
         assert_bit_exact(g, w, f"integer {name}")
 
 
+def _random_grad_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        c = int(rng.choice([1, 3, 4, 8, 20, 32, 64, 96]))
+        kh, kw = (int(v) for v in rng.choice([1, 2, 3, 5], 2))
+        st = tuple(int(v) for v in rng.choice([1, 1, 2], 2))
+        pd = tuple(int(v) for v in rng.integers(0, 3, 4))
+        n, h, w = int(rng.integers(1, 4)), int(rng.integers(4, 20)), int(rng.integers(4, 20))
+        oc = int(rng.choice([3, 16, 40, 64, 70, 128]))
+        if h + pd[0] + pd[2] < kh or w + pd[1] + pd[3] < kw:
+            continue
+        cases.append(((n, h, w, c), (oc, kh, kw, c), st, pd, [None, "7"][len(cases) % 2]))
+    return cases
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("idims,fdims,st,pd,slots", _random_grad_cases(32, 777))
+def test_conv2dGrad_random_shapes_integer_exact(rt, oracle, idims, fdims, st, pd, slots, monkeypatch):
+    """Random layer shapes (strides, uneven padding, channel counts for every kernel form of the three gradients; on
+    a chip pretended to hold seven workgroups for every other one): with small-integer operands any order of
+    summation is exact, so inputG, filterG and biasG must equal the oracle's bit for bit."""
+    print("case random conv2dGrad", idims, fdims, st, pd, slots, flush=True)
+    if slots:
+        monkeypatch.setenv("SWC_HIP_CONV_SLOTS", slots)
+    rng = np.random.default_rng(sum(idims) * 11 + sum(fdims) * 5 + sum(pd))
+    n, oh, ow, _ = pool_out_dims(idims, fdims[1:3], st, pd)
+    odims = (n, oh, ow, fdims[0])
+    x = rng.integers(-3, 4, idims).astype(np.float32)
+    f = rng.integers(-3, 4, fdims).astype(np.float32)
+    og = rng.integers(-3, 4, odims).astype(np.float32)
+    want = oracle.conv2dGrad(x, f, og, fdims[1:3], st, pd)
+    got = [t.numpy() for t in rt.conv2dGrad(*up(rt, x, f, og), fdims[1:3], st, pd)]
+    for g, w, name in zip(got, want, ("inputG", "filterG", "biasG")):
+        assert_bit_exact(g, w, f"integer {name}")
+
+
 @pytest.mark.parametrize("tag", ["p1", "s2", "k5", "asym", "c32"])
 def test_conv2dGrad_golden(rt, oracle, golden, tag):
     x, f, og = golden[f"cgrad_{tag}_x"], golden[f"cgrad_{tag}_f"], golden[f"cgrad_{tag}_og"]
