@@ -117,6 +117,31 @@ def test_gemm_integer_valued_is_exact(rt, m, k, n):
     assert_bit_exact(rt.matrixMatrixMul(da, db).numpy(), want, "integer gemm")
 
 
+def _random_gemm_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    ms = [1, 3, 8, 16, 40, 64, 100, 128, 256, 300, 513, 1024]
+    ks = [1, 4, 30, 64, 100, 500, 800, 1024, 1500, 2048, 4100]
+    ns = [1, 3, 10, 16, 20, 64, 100, 128, 256, 500, 1000]
+    return [(int(rng.choice(ms)), int(rng.choice(ks)), int(rng.choice(ns))) for _ in range(count)]
+
+
+@pytest.mark.parametrize("m,k,n", _random_gemm_cases(40, 99))
+def test_gemm_random_shapes_integer_exact(rt, m, k, n):
+    """Random (rows, K, columns) across every FC kernel's territory (few rows, heads of up to 16 columns streamed or
+    not, K split over the chip, ragged tiles): small integers make every order of summation exact, so the product,
+    with bias and ReLU in the epilogue, must equal integer arithmetic bit for bit."""
+    print("case random gemm", m, k, n, flush=True)
+    rng = np.random.default_rng(m * 7 + k * 3 + n)
+    a = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    b = rng.integers(-4, 5, (k, n)).astype(np.float32)
+    bias = rng.integers(-4, 5, n).astype(np.float32)
+    want = a.astype(np.int64) @ b.astype(np.int64)
+    da, db, dbias = up(rt, a, b, bias)
+    assert_bit_exact(rt.matrixMatrixMul(da, db).numpy(), want.astype(np.float32), f"integer gemm [{rt.last_kernel()}]")
+    got = rt.fcbias(da, db, dbias, relu=True).numpy()
+    assert_bit_exact(got, np.maximum(want + bias.astype(np.int64), 0).astype(np.float32), f"integer FC + bias + ReLU [{rt.last_kernel()}]")
+
+
 @pytest.mark.parametrize("tag", ["a", "b", "c", "d", "e"])
 def test_gemm_golden(rt, golden, tag):
     da, db, dbias = up(rt, golden[f"gemm_{tag}_a"], golden[f"gemm_{tag}_b"], golden[f"gemm_{tag}_bias"])
