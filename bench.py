@@ -2,6 +2,7 @@
 """Benchmark of the SWCompiler inference path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--headline-only] [--no-cpu]
+    python bench.py --clocks        (the shader clock under single kernels, a line of its own)
 
 Headline workload (the configuration the metric is quoted on): the wide MLP,
 batch 4096 x 784 -> FC 4096 + ReLU -> FC 4096 + ReLU -> FC 10 + softmax (one call), fp32,
@@ -325,6 +326,49 @@ def run_bn_pool_separately(rt, graphs, iters=20):
     return rows
 
 
+def clock_report(rt):
+    """--clocks: the shader clock (GHz) the chip holds under single kernels in a loop, by operand distribution: the
+    4096^3 product and the three cfg4 convolution shapes.  One JSON line; not part of the benchmark line."""
+    rng = np.random.default_rng(0)
+
+    def timed(fn, n):
+        for _ in range(3):
+            fn()
+        rt.sync()
+        rt.event_record(0)
+        for _ in range(n):
+            fn()
+        rt.event_record(1)
+        rt.sync()
+        return rt.event_elapsed_ms(0, 1) / n
+
+    kinds = [("normal", lambda s: rng.standard_normal(s)), ("relu(normal)", lambda s: np.maximum(rng.standard_normal(s), 0)),
+             ("ones", lambda s: np.ones(s))]
+    rows = [dict(work="idle", clock_ghz=rt.shader_clock_ghz(lambda: None, 1.0))]
+    b = rt.upload((rng.standard_normal((4096, 4096)) / 64).astype(np.float32))
+    c = rt.empty((4096, 4096))
+    for name, make in kinds:
+        a = rt.upload(make((4096, 4096)).astype(np.float32))
+        fn = lambda: rt.matrixMatrixMul(a, b, out=c)   # noqa: E731
+        ms = timed(fn, 10)
+        rows.append(dict(work="gemm 4096^3", a=name, us=ms * 1e3, tflops=2 * 4096 ** 3 / ms / 1e9,
+                         clock_ghz=rt.shader_clock_ghz(fn, ms), kernel=rt.last_kernel()))
+        a.free()
+    for idims, oc in (((32, 56, 56, 64), 64), ((32, 56, 56, 64), 128), ((32, 28, 28, 128), 128)):
+        f = rt.upload((rng.standard_normal((oc, 3, 3, idims[3])) / np.sqrt(9 * idims[3])).astype(np.float32))
+        bias = rt.upload(np.zeros(oc, np.float32))
+        out = rt.empty(idims[:3] + (oc,))
+        for name, make in kinds[:2]:
+            x = rt.upload(make(idims).astype(np.float32))
+            fn = lambda: rt.conv2d(x, f, bias, out=out, pads=(1, 1, 1, 1), relu=True)   # noqa: E731
+            ms = timed(fn, 20)
+            rows.append(dict(work=f"conv {list(idims)} -> {oc}, 3x3", input=name, us=ms * 1e3,
+                             tflops=2.0 * np.prod(idims[:3]) * oc * 9 * idims[3] / ms / 1e9,
+                             clock_ghz=rt.shader_clock_ghz(fn, ms), kernel=rt.last_kernel()))
+            x.free()
+    return dict(shader_clock=rows, datasheet_clock_ghz=2.4)
+
+
 def cpu_baselines(graphs, rows=64):
     """The reference's CPU kernels (the unfused call sequence its generator emits, one thread, g++ -std=c++11 -O2,
     src/codegen/MakefileBuilder.h:34) on the buffers of every configuration: the whole batch, three timed
@@ -392,6 +436,8 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch relu_f on 2^26 floats three times: a plain 256 MiB-in/256 MiB-out pass whose "
                          "FETCH_SIZE/WRITE_SIZE readings calibrate the counters for the traffic figures")
+    ap.add_argument("--clocks", action="store_true",
+                    help="instead of the benchmark: print the shader clock held under single kernels, by operand distribution")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (nothing is sharded); use --gpus 1")
@@ -400,6 +446,11 @@ def main():
     from swcompiler_amd.hip import SwcHip
     rt = SwcHip(0, auto_workspace=False)   # ops fail rather than allocate: the buffer below must cover them all
     workspace = bench_workspace(rt, graphs)
+    if args.clocks:
+        print(json.dumps(clock_report(rt)))
+        rt.sync()
+        rt.set_workspace(None)
+        return
 
     if args.calibrate:
         x = rt.upload(np.ones(1 << 26, np.float32))
