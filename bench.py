@@ -414,7 +414,7 @@ def bench_workspace(rt, graphs):
              ((32, 28, 28, 128), (128, 3, 3, 128), p1)]
     for xs, fs, pads in convs:
         need = max(need, rt.conv2d_workspace_bytes(xs, fs, (1, 1), pads))
-    for xs, fs, pads in convs[1:2] + convs[3:]:   # the layers that pool in their epilogue
+    for xs, fs, pads in convs[:2] + convs[3:]:   # the layers that pool in their epilogue
         need = max(need, rt.conv2d_maxpool_workspace_bytes(xs, fs, (1, 1), pads, ((2, 2), (2, 2))))
     for xs, fs, pads in convs[2:]:
         need = max(need, rt.conv2dGrad_workspace_bytes(xs, fs, (1, 1), pads))

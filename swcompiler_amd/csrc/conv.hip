@@ -1411,7 +1411,10 @@ int launch_conv_strip(const float *in, const float *filt, float *out, const Conv
 constexpr int kDirectMaxK = 128;
 constexpr int kDirectMaxOC = 32;
 
-template <int OCQ, int P>   // output channels rounded up to 4*OCQ; pixels per thread
+// POOL (OH and OW even): the pixels are numbered in 2 x 2 window order (pixel m is pixel m % 4 of window m / 4), so
+// four neighbouring threads hold a window; their finished values meet in the staging block, and what is stored is
+// maxpool_f's choice among them, at the window's place in the pooled tensor.
+template <int OCQ, int P, bool POOL = false>   // output channels rounded up to 4*OCQ; pixels per thread
 __global__ __launch_bounds__(256) void conv_direct(const float *__restrict__ in, const float *__restrict__ filt,
                                                    const float *__restrict__ bias, float *__restrict__ out,
                                                    ConvGeom g, Epilogue ep) {
@@ -1444,12 +1447,22 @@ __global__ __launch_bounds__(256) void conv_direct(const float *__restrict__ in,
     for (int p = 0; p < P; ++p) {
         const int m = first + p * 256 + threadIdx.x;
         const int mm = m < g.M ? m : 0;
-        const int ox = mm % g.OW;
-        const int t = mm / g.OW;
-        const int oy = t % g.OH;
+        int ox, oy, img;
+        if (POOL) {   // pixel mm % 4 of window mm / 4: (2 py + d / 2, 2 px + d % 2)
+            const int w = mm >> 2, d = mm & 3, pw = g.OW >> 1, ph = g.OH >> 1;
+            const int px = w % pw, t = w / pw;
+            ox = 2 * px + (d & 1);
+            oy = 2 * (t % ph) + (d >> 1);
+            img = t / ph;
+        } else {
+            ox = mm % g.OW;
+            const int t = mm / g.OW;
+            oy = t % g.OH;
+            img = t / g.OH;
+        }
         iy0[p] = m < g.M ? oy * g.sh - g.pt : -(1 << 20);   // pixels past M: no tap in bounds
         ix0[p] = ox * g.sw - g.pl;
-        img_base[p] = (long)(t / g.OH) * g.H;
+        img_base[p] = (long)img * g.H;
     }
     float acc[P][OCP];
 #pragma unroll
@@ -1550,6 +1563,15 @@ __global__ __launch_bounds__(256) void conv_direct(const float *__restrict__ in,
         }
         __syncthreads();
         const int pixels = (g.M - base < 256) ? (g.M - base) : 256;   // may be <= 0
+        if (POOL) {   // (M is a multiple of 4: whole windows only)
+            float *o = out + (size_t)(base >> 2) * OC;
+            if (lane_px < per_step)
+                for (int wl = wave * per_step + lane_px; 4 * wl < pixels; wl += 4 * per_step) {
+                    const float *q = &stage[4 * wl * stride + lane_oc];
+                    o[wl * OC + lane_oc] = window_max(q[0], q[stride], q[2 * stride], q[3 * stride]);
+                }
+            continue;
+        }
         float *o = out + (size_t)base * OC;
         const float *res = ep.residual ? ep.residual + (size_t)base * OC : nullptr;
         if (lane_px < per_step)
@@ -1564,8 +1586,11 @@ __global__ __launch_bounds__(256) void conv_direct(const float *__restrict__ in,
     }
 }
 
+// Whether the direct kernel can take the 2 x 2 / stride 2 pooling of its layer along.
+bool direct_pools(const ConvGeom &g) { return g.OH % 2 == 0 && g.OW % 2 == 0 && g.OH > 0 && g.OW > 0; }
+
 int launch_conv_direct(const float *in, const float *filt, const float *bias, float *out, const ConvGeom &g,
-                       const Epilogue &ep) {
+                       const Epilogue &ep, bool pool = false) {
     const int ocq = (g.OC + 3) / 4;
     // four (two) pixels per thread while that leaves at least two workgroups per CU; four only while the
     // accumulators leave room for two wavefronts per SIMD
@@ -1573,12 +1598,16 @@ int launch_conv_direct(const float *in, const float *filt, const float *bias, fl
     const bool two = !four && (size_t)g.M >= (size_t)1024 * num_cus();
     const int pixels = four ? 4 : two ? 2 : 1;
     const unsigned blocks = ceil_div((size_t)g.M, (size_t)256 * pixels);
-    note_kernel("conv_direct<%d,%d>", ocq, pixels);
+    note_kernel("conv_direct<%d,%d>%s", ocq, pixels, pool ? " (pooled)" : "");
     auto launch = [&]<int OCQ>() {
-        if constexpr (OCQ <= 5)
-            if (four) return conv_direct<OCQ, 4><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep);
-        if (two) return conv_direct<OCQ, 2><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep);
-        return conv_direct<OCQ, 1><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep);
+        auto with_pool = [&]<bool POOL>() {
+            if constexpr (OCQ <= 5)
+                if (four) return conv_direct<OCQ, 4, POOL><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep);
+            if (two) return conv_direct<OCQ, 2, POOL><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep);
+            return conv_direct<OCQ, 1, POOL><<<blocks, 256, 0, stream()>>>(in, filt, bias, out, g, ep);
+        };
+        if (pool) with_pool.template operator()<true>();
+        else with_pool.template operator()<false>();
     };
     switch (ocq) {
     case 1: launch.template operator()<1>(); break;
@@ -1751,7 +1780,7 @@ bool conv_pool_fusable(ConvGeom g, const void *input, const void *filter, const 
     bool forced_dma = false;
     if (force)
         for (int v = 0; v < kVariants; ++v) forced_dma |= !strcmp(force, kDmaVariantName[v]);
-    if (!forced_dma && g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0) return false;
+    if (!forced_dma && g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0) return direct_pools(g);   // the direct kernel's layer
     if (const int cp = padded_channels(g, force)) {
         g = with_channels(g, cp);
         input = filter = nullptr;   // the padded copies are aligned
@@ -1841,7 +1870,7 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
     if (force)
         for (int v = 0; v < kVariants; ++v) forced_dma |= !strcmp(force, kDmaVariantName[v]);
     if (!forced_dma && !(force && !strncmp(force, "reg", 3)) && g.K <= kDirectMaxK && g.OC <= kDirectMaxOC && g.C % 4 != 0)
-        return pooled ? not_pooled() : launch_conv_direct(input, filter, bias, output, g, ep);
+        return pooled && !direct_pools(g) ? not_pooled() : launch_conv_direct(input, filter, bias, output, g, ep, pooled);
     if (const int cp = forced_dma || !(force && !strncmp(force, "reg", 3)) ? padded_channels(g, force) : 0) {
         // zero-padded copies of input and filter, then the same convolution with a channel count of cp
         const size_t in_b = align256(M_in * cp * 4), f_b = align256((size_t)g.OC * g.kh * g.kw * cp * 4);

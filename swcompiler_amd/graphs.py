@@ -127,14 +127,11 @@ def run(cfg, be, t, fused=False, ws=None):
     if cfg == 3:
         h = t["x"]
         for i in (1, 2):
-            if fused and i == 2:   # 20 input channels: a layer of the tile kernels, which pool in their epilogue
+            if fused:   # ReLU and the 2x2 pooling in the convolution's epilogue (the direct kernel's and the tile kernels')
                 h = w(f"c{i}", be.conv2d, h, t[f"f{i}"], t[f"cb{i}"], relu=True, pool=((2, 2), (2, 2)))
                 continue
-            if fused:
-                h = w(f"c{i}", be.conv2d, h, t[f"f{i}"], t[f"cb{i}"], relu=True)
-            else:
-                h = w(f"c{i}", be.conv2d, h, t[f"f{i}"], t[f"cb{i}"])
-                h = w(f"r{i}", be.relu, h)
+            h = w(f"c{i}", be.conv2d, h, t[f"f{i}"], t[f"cb{i}"])
+            h = w(f"r{i}", be.relu, h)
             h = w(f"p{i}", be.maxpool, h, (2, 2), (2, 2))
         h = h.reshape(h.shape[0], -1)  # ReshapeOp alias, (h,w,c) order
         h = _fc(be, w, "fc1", h, t["w1"], t["b1"], True, fused)

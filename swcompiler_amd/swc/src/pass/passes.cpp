@@ -384,7 +384,14 @@ static OpNode *poolBehind(OpNode *conv, IRGraph *g) {
         if (v) return nullptr;
     Tensor *y = static_cast<TensorNode *>(conv->getChildNode(0))->getTensor();
     Tensor *x = static_cast<TensorNode *>(conv->getParentNode(0))->getTensor();
-    if (y->getNDim() != 4 || y->getDim(1) % 2 || y->getDim(2) % 2 || x->getDim(3) % 4) return nullptr;
+    if (y->getNDim() != 4 || y->getDim(1) % 2 || y->getDim(2) % 2) return nullptr;
+    // channel counts the tile kernels take as they are, or a first layer for the direct kernel (a short filter and up
+    // to 20 output channels: a thread then holds a window's four pixels); any other layer would pool in a second
+    // kernel anyway
+    Tensor *f = static_cast<TensorNode *>(conv->getParentNode(1))->getTensor();
+    const size_t taps = f->getNDim() == 4 ? f->getDim(1) * f->getDim(2) * f->getDim(3) : 0;
+    const bool direct = taps && taps <= 128 && y->getDim(3) <= 20;
+    if (x->getDim(3) % 4 && !direct) return nullptr;
     return pool;
 }
 static Op *pooledConv(Conv2dOp *conv, bool bn, float eps, bool relu, OpNode *pool) {

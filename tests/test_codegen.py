@@ -173,9 +173,9 @@ def test_hip_program_structure_and_build(gen, tmp_path):
     assert "const size_t o[] = {2, 56, 56, 64};" in code and "const size_t f[] = {128, 3, 3, 64};" in code
     assert code.index("swc_hip_set_workspace(gpu0_ws, gpu0_ws_bytes)") < code.index("// call op routine functions")
     lenet = generate(gen, "cfg3", "hip", tmp_path, 4)
-    # LeNet: the first layer (one input channel) keeps its pooling kernel, the second (20 channels) pools in its epilogue
-    assert lenet.count("swc_hip_conv2dFused_f(") == 1 and lenet.count("swc_hip_conv2dFusedMaxpool_f(") == 1
-    assert lenet.count("swc_hip_maxpool_f(") == 1 and "swc_hip_matrixMatrixFCBias_f(4, 500, 800" in lenet
+    # LeNet: both layers pool in their epilogue (the first in the direct kernel, the second in the tile kernel)
+    assert lenet.count("swc_hip_conv2dFused_f(") == 0 and lenet.count("swc_hip_conv2dFusedMaxpool_f(") == 2
+    assert lenet.count("swc_hip_maxpool_f(") == 0 and "swc_hip_matrixMatrixFCBias_f(4, 500, 800" in lenet
     bnpool = generate(gen, "cfg5c", "hip", tmp_path, 1)
     assert bnpool.count("swc_hip_batchnormReluMaxpool_f(") == 1 and "swc_hip_maxpool_f" not in bnpool
     assert "swc_hip_batchnormRelu_f" not in bnpool and "swc_hip_batchnormalization_f" not in bnpool

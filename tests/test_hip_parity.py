@@ -691,13 +691,46 @@ def test_conv_kernel_forms_agree_bit_for_bit(rt, idims, fdims, pads, slots, monk
         assert_bit_exact(staying_pooled, lean_pooled, "pooled, staying")
 
 
+@pytest.mark.parametrize("idims,fdims,pads", [((256, 28, 28, 1), (20, 5, 5, 1), (0, 0, 0, 0)),      # LeNet's first layer
+                                              ((3, 10, 14, 3), (8, 3, 3, 3), (1, 1, 1, 1)),
+                                              ((2, 6, 6, 1), (3, 3, 3, 1), (1, 1, 1, 1)),
+                                              ((1, 8, 8, 2), (20, 3, 3, 2), (0, 0, 0, 0)),
+                                              ((2, 12, 12, 3), (30, 3, 3, 3), (1, 1, 1, 1)),
+                                              ((300, 28, 28, 3), (16, 3, 3, 3), (1, 1, 1, 1))])        # two pixels per thread
+def test_direct_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, pads):
+    """first layers (the direct kernel: four neighbouring threads hold a window): bit-exact with the oracle's
+    conv2d_f -> relu_f -> maxpool_f, with and without ReLU and batchnorm, and with the two calls in sequence"""
+    print("case direct pooled conv", idims, fdims, pads, flush=True)
+    rng = np.random.default_rng(sum(idims) + sum(fdims))
+    oc = fdims[0]
+    x = rng.standard_normal(idims).astype(np.float32)
+    f = (rng.standard_normal(fdims) / 4).astype(np.float32)
+    b = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    dx, df, db = up(rt, x, f, b)
+    pool = ((2, 2), (2, 2))
+    n = min(idims[0], 8)
+    want = oracle.conv2d(x[:n], f, b, pads=pads)
+    got = rt.conv2d(dx, df, db, pads=pads, pool=pool)
+    assert rt.last_kernel().startswith("conv_direct") and rt.last_kernel().endswith("(pooled)"), rt.last_kernel()
+    assert rt.conv2d_maxpool_workspace_bytes(idims, fdims, (1, 1), pads, pool) == 0
+    assert_bit_exact(got.numpy()[:n], oracle.maxpool(want, *pool), "conv + pool")
+    assert_bit_exact(got.numpy(), rt.maxpool(rt.conv2d(dx, df, db, pads=pads), *pool).numpy(), "one call vs two")
+    got = rt.conv2d(dx, df, db, pads=pads, relu=True, pool=pool).numpy()
+    assert_bit_exact(got[:n], oracle.maxpool(oracle.relu(want), *pool), "conv + ReLU + pool")
+    bn = up(rt, rng.uniform(-0.1, 0.1, oc).astype(np.float32), rng.uniform(0.5, 2.0, oc).astype(np.float32),
+            rng.uniform(0.5, 1.5, oc).astype(np.float32), rng.uniform(-0.1, 0.1, oc).astype(np.float32))
+    kw = dict(pads=pads, bn=bn, eps=1e-5, relu=True)
+    assert_bit_exact(rt.conv2d(dx, df, db, pool=pool, **kw).numpy(), rt.maxpool(rt.conv2d(dx, df, db, **kw), *pool).numpy(),
+                     "conv + BN + ReLU + pool, one call vs two")
+
+
 def test_conv_with_a_pooling_the_epilogue_cannot_do(rt, oracle):
     """odd output sizes, 3x3 windows, a layer for the direct kernel: conv into the workspace, then maxpool_f's kernel"""
     rng = np.random.default_rng(5)
     cases = [((2, 9, 9, 8), (16, 3, 3, 8), (1, 1, 1, 1), ((2, 2), (2, 2))),          # 9 x 9 output
              ((2, 12, 12, 8), (16, 3, 3, 8), (1, 1, 1, 1), ((3, 3), (2, 2))),        # 3 x 3 windows
              ((2, 12, 12, 8), (16, 3, 3, 8), (1, 1, 1, 1), ((2, 2), (2, 2), (1, 1, 1, 1))),   # padded pooling
-             ((4, 28, 28, 1), (20, 5, 5, 1), (0, 0, 0, 0), ((2, 2), (2, 2)))]        # the direct kernel's layer
+             ((4, 27, 27, 1), (20, 5, 5, 1), (0, 0, 0, 0), ((2, 2), (2, 2), (0, 0, 1, 1)))]   # the direct kernel's layer, 23 x 23 output
     for idims, fdims, pads, pool in cases:
         print("case conv + other pooling", idims, fdims, pads, pool, flush=True)
         x = rng.standard_normal(idims).astype(np.float32)
