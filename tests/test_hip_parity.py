@@ -696,7 +696,8 @@ def test_conv_kernel_forms_agree_bit_for_bit(rt, idims, fdims, pads, slots, monk
                                               ((2, 6, 6, 1), (3, 3, 3, 1), (1, 1, 1, 1)),
                                               ((1, 8, 8, 2), (20, 3, 3, 2), (0, 0, 0, 0)),
                                               ((2, 12, 12, 3), (30, 3, 3, 3), (1, 1, 1, 1)),
-                                              ((300, 28, 28, 3), (16, 3, 3, 3), (1, 1, 1, 1))])        # two pixels per thread
+                                              ((400, 28, 28, 3), (16, 3, 3, 3), (1, 1, 1, 1)),        # two pixels per thread
+                                              ((700, 28, 28, 1), (20, 5, 5, 1), (2, 2, 2, 2))])        # four pixels per thread
 def test_direct_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, pads):
     """first layers (the direct kernel: four neighbouring threads hold a window): bit-exact with the oracle's
     conv2d_f -> relu_f -> maxpool_f, with and without ReLU and batchnorm, and with the two calls in sequence"""
@@ -712,6 +713,8 @@ def test_direct_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, 
     want = oracle.conv2d(x[:n], f, b, pads=pads)
     got = rt.conv2d(dx, df, db, pads=pads, pool=pool)
     assert rt.last_kernel().startswith("conv_direct") and rt.last_kernel().endswith("(pooled)"), rt.last_kernel()
+    per_thread = 4 if idims[0] >= 700 else 2 if idims[0] >= 400 else 1
+    assert rt.last_kernel() == f"conv_direct<{(oc + 3) // 4},{per_thread}> (pooled)", rt.last_kernel()
     assert rt.conv2d_maxpool_workspace_bytes(idims, fdims, (1, 1), pads, pool) == 0
     assert_bit_exact(got.numpy()[:n], oracle.maxpool(want, *pool), "conv + pool")
     assert_bit_exact(got.numpy(), rt.maxpool(rt.conv2d(dx, df, db, pads=pads), *pool).numpy(), "one call vs two")
