@@ -557,7 +557,9 @@ template <int RING, bool B2> int launch_stream(const StreamArgs &x) {
 
 // ------------------------------------------------------------ few-rows GEMM
 // M <= 16 (single-sample and small-batch inference) with a B of a few MB: the product is bound by the latency
-// of one pass over B.  A workgroup owns 16 columns of C; its sixteen wavefronts split K into contiguous ranges
+// of one pass over B.  (Also up to 128 rows in blocks of 16 over blockIdx.y while K fits one trip and the blocks'
+// passes over B stay within 16 MB of L2 traffic: one launch where the tiled kernels need a split-K pair.)
+// A workgroup owns 16 columns of C; its sixteen wavefronts split K into contiguous ranges
 // and feed v_mfma_f32_16x16x4_f32 straight from global memory (A is a few KB and stays in cache), all operands
 // of a trip requested before its first MFMA — for K up to 1024 a single trip, i.e. one memory latency.  The
 // sixteen partial 16x16 tiles are summed through LDS in wavefront order.  One launch where the tiled kernels
@@ -573,9 +575,9 @@ __global__ __launch_bounds__(64 * kFewRowsWaves) void gemm_fewrows(const float *
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int j = lane & 15, kk = lane >> 4;   // as operand A the lane's row is j, as operand B its column
-    const int col = blockIdx.x * 16 + j;
-    const bool col_ok = col < N, row_ok = j < M;
-    const float *arow = A + (size_t)(row_ok ? j : 0) * lda;
+    const int col = blockIdx.x * 16 + j, row0 = blockIdx.y * 16;
+    const bool col_ok = col < N, row_ok = row0 + j < M;
+    const float *arow = A + (size_t)(row_ok ? row0 + j : 0) * lda;
     // this wavefront's range of K, a multiple of 4 long
     const int chunk = ((K + kFewRowsWaves - 1) / kFewRowsWaves + 3) & ~3;
     const int k_begin = wave * chunk, k_end = (k_begin + chunk < K) ? k_begin + chunk : K;
@@ -600,10 +602,10 @@ __global__ __launch_bounds__(64 * kFewRowsWaves) void gemm_fewrows(const float *
         float s = 0.f;
         for (int w = 0; w < kFewRowsWaves; ++w) s += part[w][r][c];
         const int gc = blockIdx.x * 16 + c;
-        if (r < M && gc < N) {
+        if (row0 + r < M && gc < N) {
             float x = s + (ep.bias ? ep.bias[gc] : 0.f);
             if (ep.relu) x = (x > 0.f) ? x : 0.f;
-            C[(size_t)r * ldc + gc] = x;
+            C[(size_t)(row0 + r) * ldc + gc] = x;
         }
     }
 }
@@ -708,7 +710,14 @@ int launch_splitk(const float *a, const float *b, float *c, int m, int n, int k,
 
 // Split-K plan of an m x n x k product on this device: true with the number of splits and the K slices per
 // split when the shape has too few output tiles to fill the chip.
-bool takes_fewrows(int m, int n, int k) { return m <= 16 && k > 0 && (size_t)k * n <= ((size_t)2 << 20); }
+bool takes_fewrows(int m, int n, int k) {
+    if (k <= 0) return false;
+    if (m <= 16) return (size_t)k * n <= ((size_t)2 << 20);
+    // blocks of 16 rows: K in one trip of the sixteen wavefronts, the blocks' passes over B within 16 MB.  Measured
+    // against the split-K pair: 32 x 784 x 512 10.6 against 12.7 us, 64 x 1024 x 1024 12.8 against 15.8, 128 x 512 x 256
+    // 8.7 against 11.8; level at 256 x 800 x 500 (17.5 us both) and behind beyond, so 128 rows are the limit
+    return m <= 128 && k <= 64 * kFewRowsWaves && (size_t)((m + 15) / 16) * k * n <= ((size_t)4 << 20);
+}
 
 // Up to 64 rows (small-batch inference: the product streams B once and is bound by that): tiles of 32 x 256
 // or 64 x 256 instead of 128 x 128, so that no matrix-core work goes into rows that do not exist — with
@@ -789,7 +798,7 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
     // a handful of rows and a B of a few MB: one latency-bound pass over B (see gemm_fewrows)
     if (takes_fewrows(m, n, k) && (!force || !strcmp(force, "fewrows"))) {
         note_kernel("gemm_fewrows");
-        gemm_fewrows<<<ceil_div(n, 16), 64 * kFewRowsWaves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep);
+        gemm_fewrows<<<dim3(ceil_div(n, 16), ceil_div(m, 16)), 64 * kFewRowsWaves, 0, stream()>>>(a, b, c, m, n, k, lda, ldb, ldc, ep);
         SWC_LAUNCH_CHECK();
         return SWC_HIP_OK;
     }
