@@ -319,9 +319,11 @@ def test_text_and_binary_files_give_the_same_program(gen, tmp_path):
 def test_import_hip_program_structure(gen, tmp_path):
     write_model(tmp_path, True)
     code = generate(gen, "caffe2", "hip", tmp_path, 2)
-    # conv+BN+ReLU is one call, and so is conv+BN+Sum+ReLU (the other summand, pool1, is the call's `residual`);
-    # the weight transposes run once, before the op sequence
-    assert code.count("swc_hip_conv2dFused_f(") == 1 and "swc_hip_vecAdd" not in code
+    # conv+BN+ReLU with the pooling behind it is one call (a first layer: the direct kernel pools in its epilogue), and
+    # so is conv+BN+Sum+ReLU (the other summand, pool1, is the call's `residual`); the weight transposes run once,
+    # before the op sequence
+    assert code.count("swc_hip_conv2dFusedMaxpool_f(") == 1 and code.count("swc_hip_conv2dFused_f(") == 0
+    assert "swc_hip_vecAdd" not in code and "swc_hip_maxpool_f(" not in code
     assert code.count("swc_hip_conv2dFusedAdd_f(") == 1 and "1e-05, gpu_0_pool1, 1));" in code
     head, body = code.split("// call op routine functions")
     assert head.count("swc_hip_transpose4d_f(") == 2 and head.count("swc_hip_transpose2d_f(") == 1
