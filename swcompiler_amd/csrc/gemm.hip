@@ -557,8 +557,8 @@ template <int RING, bool B2> int launch_stream(const StreamArgs &x) {
 
 // ------------------------------------------------------------ few-rows GEMM
 // M <= 16 (single-sample and small-batch inference) with a B of a few MB: the product is bound by the latency
-// of one pass over B.  (Also up to 128 rows in blocks of 16 over blockIdx.y while K fits one trip and the blocks'
-// passes over B stay within 16 MB of L2 traffic: one launch where the tiled kernels need a split-K pair.)
+// of one pass over B.  (Also up to 256 rows in blocks of 16 over blockIdx.y while K fits one trip and the blocks'
+// passes over B stay within 32 MB of L2 traffic: one launch where the tiled kernels need a split-K pair.)
 // A workgroup owns 16 columns of C; its sixteen wavefronts split K into contiguous ranges
 // and feed v_mfma_f32_16x16x4_f32 straight from global memory (A is a few KB and stays in cache), all operands
 // of a trip requested before its first MFMA — for K up to 1024 a single trip, i.e. one memory latency.  The
@@ -582,14 +582,24 @@ __global__ __launch_bounds__(64 * kFewRowsWaves) void gemm_fewrows(const float *
     const int chunk = ((K + kFewRowsWaves - 1) / kFewRowsWaves + 3) & ~3;
     const int k_begin = wave * chunk, k_end = (k_begin + chunk < K) ? k_begin + chunk : K;
     v4f acc = {0.f, 0.f, 0.f, 0.f};
+    // Which four k an MFMA adds up is free (a sum).  In blocks of 16 k, step s of a block gives lane (j, kk) the
+    // element k = 16 t + 4 kk + s: the lane's four A operands of a block are then 16 contiguous bytes of its row
+    // (one 128-bit load where the row allows it, a quarter of the load instructions), and B follows the same k.
+    const bool a_vec = (lda % 4 == 0) && ((reinterpret_cast<size_t>(A) & 15) == 0) && (k_begin % 4 == 0);
     for (int kb = k_begin; kb < k_end; kb += 4 * kFewRowsUnroll) {
         float a[kFewRowsUnroll], b[kFewRowsUnroll];
 #pragma unroll
-        for (int u = 0; u < kFewRowsUnroll; ++u) {
-            const int k = kb + 4 * u + kk;
-            const bool k_ok = k < k_end;
-            b[u] = (k_ok && col_ok) ? B[(size_t)k * ldb + col] : 0.f;
-            a[u] = (k_ok && row_ok) ? arow[k] : 0.f;
+        for (int t = 0; t < kFewRowsUnroll / 4; ++t) {
+            const int k0 = kb + 16 * t + 4 * kk;   // this lane's four k of block t
+            if (a_vec && row_ok && k0 + 3 < k_end) {
+                const float4 q = *reinterpret_cast<const float4 *>(arow + k0);
+                a[4 * t] = q.x, a[4 * t + 1] = q.y, a[4 * t + 2] = q.z, a[4 * t + 3] = q.w;
+            } else {
+#pragma unroll
+                for (int s4 = 0; s4 < 4; ++s4) a[4 * t + s4] = (row_ok && k0 + s4 < k_end) ? arow[k0 + s4] : 0.f;
+            }
+#pragma unroll
+            for (int s4 = 0; s4 < 4; ++s4) b[4 * t + s4] = (col_ok && k0 + s4 < k_end) ? B[(size_t)(k0 + s4) * ldb + col] : 0.f;
         }
 #pragma unroll
         for (int u = 0; u < kFewRowsUnroll; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u], b[u], acc, 0, 0, 0);
@@ -713,10 +723,11 @@ int launch_splitk(const float *a, const float *b, float *c, int m, int n, int k,
 bool takes_fewrows(int m, int n, int k) {
     if (k <= 0) return false;
     if (m <= 16) return (size_t)k * n <= ((size_t)2 << 20);
-    // blocks of 16 rows: K in one trip of the sixteen wavefronts, the blocks' passes over B within 16 MB.  Measured
-    // against the split-K pair: 32 x 784 x 512 10.6 against 12.7 us, 64 x 1024 x 1024 12.8 against 15.8, 128 x 512 x 256
-    // 8.7 against 11.8; level at 256 x 800 x 500 (17.5 us both) and behind beyond, so 128 rows are the limit
-    return m <= 128 && k <= 64 * kFewRowsWaves && (size_t)((m + 15) / 16) * k * n <= ((size_t)4 << 20);
+    // blocks of 16 rows: K in one trip of the sixteen wavefronts (and long enough to give each of them work), the
+    // blocks' passes over B within 32 MB.  Between events, against the split-K pair: 32 x 784 x 512 7.6 against 12.8 us,
+    // 64 x 1024 x 1024 8.8 against 15.9, 128 x 512 x 256 7.3 against 12.0, 256 x 800 x 500 13.1 against 17.7,
+    // 256 x 1024 x 512 12.6 against 17.9; 200 x 300 x 1000 is better off on the tiled kernel (14.3 against 12.5)
+    return m <= 256 && k >= 512 && k <= 64 * kFewRowsWaves && (size_t)((m + 15) / 16) * k * n <= ((size_t)8 << 20);
 }
 
 // Up to 64 rows (small-batch inference: the product streams B once and is bound by that): tiles of 32 x 256

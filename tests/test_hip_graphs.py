@@ -172,15 +172,15 @@ def test_library_workspace_is_not_replaced_under_a_recorded_graph(rt):
     rng = np.random.default_rng(3)
     rt.sync()
     rt.set_workspace(None)                      # drop whatever earlier tests grew
-    a = rt.upload(rng.standard_normal((160, 512)).astype(np.float32))
-    w = rt.upload(rng.standard_normal((512, 200)).astype(np.float32))
+    a = rt.upload(rng.standard_normal((160, 448)).astype(np.float32))
+    w = rt.upload(rng.standard_normal((448, 200)).astype(np.float32))
     out = rt.empty((160, 200))
-    small, big = rt.gemm_workspace_bytes(160, 200, 512), rt.gemm_workspace_bytes(256, 500, 800)
+    small, big = rt.gemm_workspace_bytes(160, 200, 448), rt.gemm_workspace_bytes(256, 500, 1600)
     assert 0 < small < big - (1 << 20)          # (the library rounds its buffer up to 1 MiB)
     rt.fcbias(a, w, None, out=out)              # eager: the library allocates `small`
     eager = out.numpy().copy()
     handle = rt.capture(lambda: rt.fcbias(a, w, None, out=out))
-    a2, w2 = rt.empty((256, 800)), rt.empty((800, 500))
+    a2, w2 = rt.empty((256, 1600)), rt.empty((1600, 500))
     try:
         with pytest.raises(SwcHipError, match="recorded graph"):
             rt.fcbias(a2, w2, None)             # would need `big`

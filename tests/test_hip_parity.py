@@ -829,9 +829,10 @@ def test_gemm_of_up_to_64_rows_and_a_large_b(rt, oracle, m, k, n):
 
 @pytest.mark.parametrize("m,k,n", [(8, 784, 512), (1, 784, 512), (16, 1000, 100), (3, 5, 17), (16, 1, 33), (7, 64, 520),
                                    (8, 4096, 512), (2, 130, 4099),
-                                   (32, 784, 512), (40, 700, 300), (128, 512, 256), (100, 1000, 90), (17, 1024, 33)])   # blocks of 16 rows
+                                   (32, 784, 512), (40, 700, 300), (128, 512, 256), (100, 1000, 90), (17, 1024, 33), (256, 800, 500),
+                                   (250, 513, 37)])   # blocks of 16 rows
 def test_gemm_of_a_few_rows(rt, oracle, m, k, n):
-    """M <= 16 with a small B (or up to 128 rows of a K of up to 1024, in blocks of 16 rows): one launch, K split
+    """M <= 16 with a small B (or up to 256 rows of a K of 512 to 1024, in blocks of 16 rows): one launch, K split
     over the wavefronts of a workgroup"""
     print("case few-rows gemm", m, k, n, flush=True)
     rng = np.random.default_rng(m * 7 + k + n)
@@ -857,7 +858,7 @@ def test_gemm_split_over_k_uses_exactly_the_size_it_reports(rt, oracle):
     from swcompiler_amd.hip import SwcHipError
     assert rt.gemm_workspace_bytes(4096, 4096, 784) == 0 and rt.gemm_workspace_bytes(8, 10, 512) == 0
     assert rt.gemm_workspace_bytes(8, 512, 784) == 0   # a handful of rows: the one-pass kernel, no scratch
-    assert rt.gemm_workspace_bytes(32, 512, 784) == 0  # up to 128 rows of a short K: the same kernel in blocks of 16 rows
+    assert rt.gemm_workspace_bytes(32, 512, 784) == 0  # up to 256 rows of a K of up to 1024: the same kernel in blocks of 16 rows
     m, n, k = 32, 512, 1568
     need = rt.gemm_workspace_bytes(m, n, k)
     assert need > 0 and need % (m * n * 4) == 0

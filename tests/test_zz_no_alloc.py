@@ -28,8 +28,8 @@ def _operands(rt, rng, m, n, k):
 
 def test_noalloc_matches_workspace_entry_point_twice(rt, oracle):
     rng = np.random.default_rng(0x5C0DE)
-    # LeNet's 256 x 800 x 500 layer (25 ranges of K, 12.8 MB of partial tiles), then a smaller product (16 ranges)
-    for (m, n, k), relu in (((256, 500, 800), True), ((160, 200, 512), False)):
+    # a product of 33 ranges of K (12.7 MB of partial tiles), then a smaller one (16 ranges)
+    for (m, n, k), relu in (((192, 500, 1056), True), ((160, 200, 448), False)):
         need = rt.gemm_workspace_bytes(m, n, k)
         assert 0 < need <= NOALLOC_SCRATCH_BYTES, (m, n, k, need)   # the shape does use the scratch array
         a, w, b, da, dw, db = _operands(rt, rng, m, n, k)
@@ -49,7 +49,7 @@ def test_noalloc_without_any_workspace(rt):
     """works where the ordinary entry point is refused: no workspace set, none allocated on demand"""
     from swcompiler_amd.hip import SwcHipError
     rng = np.random.default_rng(7)
-    m, n, k = 256, 500, 800
+    m, n, k = 192, 500, 1056
     a, w, b, da, dw, db = _operands(rt, rng, m, n, k)
     want = rt.fcbias(da, dw, db).numpy()
     rt.sync()
