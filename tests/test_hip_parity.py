@@ -256,6 +256,42 @@ def test_conv_random_shapes_integer_exact(rt, oracle, idims, fdims, strides, pad
         assert_bit_exact(got, oracle.maxpool(oracle.relu(want), *pool), f"conv + ReLU + pool on integers [{rt.last_kernel()}]")
 
 
+def _random_wide_lean_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        c, oc = int(rng.choice([32, 64])), int(rng.choice([8, 64, 72, 128]))
+        k, s = int(rng.choice([1, 3])), int(rng.choice([1, 1, 2]))
+        n, h, w = int(rng.integers(1, 4)), int(rng.integers(8, 40)), int(rng.integers(16, 70))
+        oh, ow = (h + 2 * (k // 2) - k) // s + 1, (w + 2 * (k // 2) - k) // s + 1
+        if oh % 2 or ow % 2 or ow < 16:
+            continue
+        cases.append(((n, h, w, c), (oc, k, k, c), (s, s), (k // 2,) * 4, [None, "7", "20"][len(cases) % 3]))
+    return cases
+
+
+@pytest.mark.parametrize("idims,fdims,strides,pads,slots", _random_wide_lean_cases(18, 31))
+def test_conv_lean_wide_images_integer_exact(rt, oracle, idims, fdims, strides, pads, slots, monkeypatch):
+    """conv_dma_lean on images of at least eight 2x2 windows per output row, where the pixel of a row follows from the
+    tile's first window by carries (ragged last tiles, strides, tiles cut along K): integer operands, the oracle's bits,
+    plain and with the pooled epilogue."""
+    print("case wide lean conv", idims, fdims, strides, pads, slots, flush=True)
+    if slots:
+        monkeypatch.setenv("SWC_HIP_CONV_SLOTS", slots)
+    rng = np.random.default_rng(sum(idims) * 13 + sum(fdims))
+    x = rng.integers(-3, 4, idims).astype(np.float32)
+    f = rng.integers(-3, 4, fdims).astype(np.float32)
+    b = rng.integers(-3, 4, fdims[0]).astype(np.float32)
+    dx, df, db = up(rt, x, f, b)
+    want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
+    got = rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy()
+    assert rt.last_kernel().startswith("conv_dma_lean"), rt.last_kernel()
+    assert_bit_exact(got, want, f"conv on integers [{rt.last_kernel()}]")
+    pool = ((2, 2), (2, 2))
+    got = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True, pool=pool).numpy()
+    assert_bit_exact(got, oracle.maxpool(oracle.relu(want), *pool), f"conv + ReLU + pool on integers [{rt.last_kernel()}]")
+
+
 def test_conv_integer_valued_is_exact(rt):
     rng = np.random.default_rng(9)
     for idims, fdims, pads in [((2, 9, 10, 8), (40, 3, 3, 8), (1, 1, 1, 1)), ((1, 12, 12, 3), (70, 5, 5, 3), (2, 2, 2, 2))]:
