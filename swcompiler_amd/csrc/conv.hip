@@ -2307,6 +2307,53 @@ __global__ __launch_bounds__(256) void bias_partials(float *__restrict__ part, c
     }
 }
 
+// outputG [M, OC] -> its transpose ogT [OC, lda] (what the filter gradient's GEMM reads), and in the same pass over
+// outputG the bias gradient's masked column sums of chunks of kBiasRows rows (see bias_partials for the mask): one read
+// of outputG instead of two.  A workgroup moves kBiasRows / 32 tiles of 32 rows x 32 columns through a 32 x 33 LDS tile
+// (matrix_trans's); thread (tx, ty) sees rows ty, ty + 8, ... of column tx and keeps its pixel coordinates
+// incrementally; the eight partial sums of a column are added in order.  grid: (chunks, OC / 32 rounded up).
+__global__ __launch_bounds__(256) void trans_bias_partials(float *__restrict__ ogT, size_t lda, float *__restrict__ part,
+                                                           const float *__restrict__ og, ConvGeom g) {
+    __shared__ float tile[32][33];
+    __shared__ float red[8][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 32 x 8
+    const int c0 = blockIdx.y * 32, m0 = blockIdx.x * kBiasRows;
+    int m = m0 + ty;
+    int ox = m % g.OW, oy = (m / g.OW) % g.OH;
+    const int step_y = 8 / g.OW, step_x = 8 - step_y * g.OW;   // eight rows further on
+    float acc = 0.f;
+    for (int r0 = m0; r0 < m0 + kBiasRows && r0 < g.M; r0 += 32) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int r = r0 + ty + 8 * k, c = c0 + tx;
+            if (r < g.M && c < g.OC) {
+                const float v = og[(size_t)r * g.OC + c];
+                tile[ty + 8 * k][tx] = v;
+                const bool counts = (unsigned)(oy * g.sh - g.pt) < (unsigned)g.H && (unsigned)(ox * g.sw - g.pl) < (unsigned)g.W;
+                if (counts) acc += v;
+            }
+            ox += step_x;
+            oy += step_y;
+            if (ox >= g.OW) ox -= g.OW, ++oy;
+            while (oy >= g.OH) oy -= g.OH;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int c = c0 + ty + 8 * k, r = r0 + tx;   // output row c, column r
+            if (c < g.OC && r < g.M) ogT[(size_t)c * lda + r] = tile[tx][ty + 8 * k];
+        }
+        __syncthreads();
+    }
+    red[ty][tx] = acc;
+    __syncthreads();
+    if (ty == 0 && c0 + tx < g.OC) {
+        float t = red[0][tx];
+        for (int q = 1; q < 8; ++q) t += red[q][tx];
+        part[(size_t)blockIdx.x * g.OC + c0 + tx] = t;
+    }
+}
+
 size_t wgrad_small_lds(const ConvGeom &g, int rows) {
     return ((size_t)rows * g.OW * g.OC + ((size_t)(rows - 1) * g.sh + g.kh) * g.W * g.C) * sizeof(float);
 }
@@ -2443,8 +2490,15 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
     float *dgrad_pieces = reinterpret_cast<float *>(ws + turned_b + ogt_b + part_b + bias_b);
     float *og_padded = reinterpret_cast<float *>(ws + turned_b + ogt_b + part_b + bias_b + dgrad_b);
 
-    // ---- bias gradient
-    {
+    // ---- bias gradient (with the filter gradient's transposed outputG in the same pass where that is needed)
+    if (wgrad_mfma) {
+        // the 128-bit loads of the last k chunk reach into the row padding: it must hold zeros, not stale bits
+        if ((size_t)lda != M) {
+            const int rc0 = swc_hip_fill_f(ogT, 0.f, (size_t)g.OC * lda);
+            if (rc0 != SWC_HIP_OK) return rc0;
+        }
+        trans_bias_partials<<<dim3(bias_chunks, (g.OC + 31) / 32), 256, 0, stream()>>>(ogT, (size_t)lda, bias_part, outputG, g);
+    } else {
         const bool vec4 = g.OC % 4 == 0 && aligned16(outputG);
         const int quads = vec4 ? g.OC / 4 : g.OC;
         int colsq = 1;
@@ -2497,13 +2551,6 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
 
     // ---- filter gradient
     if (wgrad_mfma) {
-        // the 128-bit loads of the last k chunk reach into the row padding: it must hold zeros, not stale bits
-        if ((size_t)lda != M) {
-            const int rc0 = swc_hip_fill_f(ogT, 0.f, (size_t)g.OC * lda);
-            if (rc0 != SWC_HIP_OK) return rc0;
-        }
-        const int rc = swc_hip_matrixTrans_f((int)M, g.OC, outputG, g.OC, ogT, lda);
-        if (rc != SWC_HIP_OK) return rc;
         const Im2colB bsrc{input, (unsigned)(in_elems * 4), g.H, g.W, g.C, g.OH, g.OW, g.kw, g.sh, g.sw, g.pt, g.pl, g.N,
                            BK / g.OW, BK % g.OW};
         float *dst = splits > 1 ? part : filterG;
