@@ -23,7 +23,8 @@ Also in the line:
                 each time (never the headline value); `overlapped_uploads`: the same with
                 the next batch's upload on a second stream while this batch is computed
   peaks_measured  fp32 MFMA rate of a register-only loop and a streaming copy on this
-                device, beside the datasheet peaks the fractions are computed from
+                device, beside the datasheet peaks the fractions are computed from; and what a pair of
+                events reads with nothing / a 1 KB kernel between them (the floor under every per-op figure)
   configs       the other synthetic configurations (samples/s and, per kernel,
                 TFLOP/s or GB/s with the fraction of the MI355X peak)
                 plus `training_kernels`: conv2dGrad, reluGrad, sgd, maxpoolGrad at those sizes
@@ -214,7 +215,24 @@ def measured_peaks(rt):
         times.append(rt.event_elapsed_ms(0, 1))
     x.free()
     y.free()
-    return dict(mfma_f32_tflops_short=short[0], mfma_f32_short_ms=short[1], mfma_f32_tflops_sustained=long_[0],
+    # what a pair of events costs by itself: every per-op figure below carries it (it matters for kernels of a few us)
+    gaps = []
+    for i in range(20):
+        rt.event_record(0)
+        rt.event_record(1)
+        rt.sync()
+        gaps.append(rt.event_elapsed_ms(0, 1) * 1e3)
+    tiny = rt.upload(np.ones(256, np.float32))
+    tiny_out = rt.empty((256,))
+    around_tiny = []
+    for i in range(20):
+        rt.event_record(0)
+        rt.relu(tiny, out=tiny_out)
+        rt.event_record(1)
+        rt.sync()
+        around_tiny.append(rt.event_elapsed_ms(0, 1) * 1e3)
+    return dict(event_pair_empty_us=float(np.median(gaps)), event_pair_around_a_1kb_kernel_us=float(np.median(around_tiny)),
+                mfma_f32_tflops_short=short[0], mfma_f32_short_ms=short[1], mfma_f32_tflops_sustained=long_[0],
                 mfma_f32_sustained_ms=long_[1], stream_copy_gbs=2 * (1 << 28) / (min(times) * 1e-3) / 1e9,
                 datasheet=dict(mfma_f32_tflops=PEAK_TFLOPS_FP32_MFMA, hbm_gbs=PEAK_HBM_GBS))
 
