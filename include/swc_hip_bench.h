@@ -27,7 +27,8 @@ int swc_hip_bench_probe_mfma_f32(void *hip_stream, int cus, float *scratch_dev, 
  * and returns at once; the watcher ends by itself after its n pairs.  The harness then enqueues the work it
  * wants watched on its own stream, calls _wait, and reads the clock off consecutive pairs:
  * GHz = 0.1 x (shader difference) / (wall difference).  One wavefront on one CU does not disturb a kernel that
- * fills the chip.  1 < n <= 65536, 1 <= sleeps <= 64.  Return 0, or a non-zero hipError_t. */
+ * fills the chip.  1 < n <= 65536, 1 <= sleeps <= 64, n x sleeps <= 262144 (the watcher then ends within a second).
+ * Return 0, or a non-zero hipError_t. */
 int swc_hip_bench_clock_watch_start(unsigned long long *samples_dev, int n, int sleeps);
 int swc_hip_bench_clock_watch_wait(void);
 

@@ -81,7 +81,8 @@ extern "C" int swc_hip_bench_probe_mfma_f32(void *hip_stream, int cus, float *sc
 }
 
 extern "C" int swc_hip_bench_clock_watch_start(unsigned long long *samples_dev, int n, int sleeps) {
-    if (!samples_dev || n <= 1 || n > (1 << 16) || sleeps < 1 || sleeps > 64) return (int)hipErrorInvalidValue;
+    if (!samples_dev || n <= 1 || n > (1 << 16) || sleeps < 1 || sleeps > 64 || (long)n * sleeps > (1L << 18))   // under a second
+        return (int)hipErrorInvalidValue;
     if (!g_watch_stream) PROBE_TRY(hipStreamCreateWithFlags(&g_watch_stream, hipStreamNonBlocking));
     clock_watch<<<1, 64, 0, g_watch_stream>>>(samples_dev, n, sleeps);
     PROBE_TRY(hipGetLastError());
