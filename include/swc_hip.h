@@ -132,6 +132,10 @@ const char *swc_hip_last_error(void);         /* message of the last failure on 
  * template arguments (e.g. "gemm_dma2<2,4,4,2,false,8>"; "" before the first such call): lets a harness check
  * that the kernel it reports on is the one that ran. */
 const char *swc_hip_last_kernel(void);
+/* The SWC_HIP_* environment variables (test and tuning switches that force kernel variants; none is part of the
+ * contract) are read once, by swc_hip_init; no op reads the environment.  A test process that changes them calls
+ * this to have them read again — not while a graph is being recorded.  No counterpart in the reference. */
+int swc_hip_reload_switches(void);
 void *swc_hip_stream(void);                   /* the hipStream_t ops are launched on */
 int swc_hip_set_stream(void *hip_stream);     /* launch on a caller-owned stream (NULL: back to the library's own) */
 const char *swc_hip_device_name(void);        /* gcnArchName of the selected device */

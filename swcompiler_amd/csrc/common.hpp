@@ -32,6 +32,23 @@ void *workspace(size_t bytes, const char *who);
 // that allocates nothing (gemm.hip); called once per device by swc_hip_init.
 int gemm_noalloc_setup(int device);
 
+// Test and tuning switches (the SWC_HIP_* environment variables; none is part of the contract).  swc_hip_init reads
+// them ONCE into this record (swc_hip_reload_switches reads them again, for a test process that changes them): no
+// op touches the environment, so a size query, a warm-up run and a recorded graph all see the same choice.
+struct Switches {
+    const char *gemm = nullptr;   // SWC_HIP_GEMM: forces a GEMM kernel variant ("splitk", "fewrows", "reg", "22_2", ...)
+    const char *conv = nullptr;   // SWC_HIP_CONV: forces a convolution kernel variant ("reg22", "11_3m", ...)
+    bool skinny_plain = false;    // SWC_HIP_SKINNY=plain: gemm_skinny for every classifier head
+    bool conv_share = true;       // SWC_HIP_CONV_SHARE=0: every convolution tile computed whole
+    bool conv_raster = false;     // SWC_HIP_CONV_ORDER=raster: rows of the GEMM view in raster order
+    bool conv_lean = true;        // SWC_HIP_CONV_LEAN=0: the general tile kernel where the lean one would run
+    int conv_share_all = 0;       // SWC_HIP_CONV_SHARE_ALL=n: slices per tile from which a short layer is cut (unset 0: default; "0" -> -1: never)
+    int conv_slots = 0;           // SWC_HIP_CONV_SLOTS=n: pretend the chip holds n workgroups at a time (0: ask the device)
+    int conv_piece_min = 0;       // SWC_HIP_CONV_PIECE_MIN=n: least K slices per piece of a tile cut along K (0: default)
+    int wgrad_bn = 0;             // SWC_HIP_WGRAD_BN=128|256: tile width of the filter gradient (0: planner's choice)
+};
+const Switches &switches();
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 inline unsigned ceil_div(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }

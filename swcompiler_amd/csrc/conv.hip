@@ -11,7 +11,6 @@
 // from the FC GEMM.  When iC % 4 == 0 four consecutive k's lie in one tap, so
 // the gather uses 128-bit loads; otherwise (first layer, iC = 1 or 3) 32-bit.
 #include "common.hpp"
-#include "conv_strip.hpp"
 #include "mfma_dma.hpp"
 #include "mfma_dma2.hpp"
 #include "mfma_tile.hpp"
@@ -22,6 +21,18 @@ using namespace swc_hip;
 using namespace swc_hip::mfma;
 
 namespace {
+
+struct ConvGeom {
+    int N, H, W, C;      // input NHWC
+    int OH, OW, OC;      // output
+    int kh, kw, sh, sw, pt, pl;
+    int M, K;            // GEMM view: output pixels, kh*kw*C
+    // Order in which the rows of the GEMM view walk the output pixels.  0: raster order (image, row, column).
+    // 1: by 2 x 2 windows — row m is pixel (2py + d/2, 2px + d%2) of window m/4 = (image, py, px) in raster order
+    // of the windows, d = m%4 — so that every aligned group of four rows is one window of a 2 x 2 / stride 2
+    // pooling (even OH and OW only).
+    int win = 0;
+};
 
 template <int TM, int TN, bool VEC>
 __global__ __launch_bounds__(kThreads) void conv_igemm(const float *__restrict__ in, const float *__restrict__ filt,
@@ -303,12 +314,17 @@ __device__ __forceinline__ void store_tile_windows(const v16f (&acc)[TM][TN], fl
 // the out-of-range offset and arrive in LDS as zeros.  Needs iC % 4 == 0,
 // 16-byte-aligned tensors and input/filter below 2 GiB.
 //
-// Work is counted in units of one K slice of one tile.  The first `dp_tiles`
-// workgroups each take a whole tile.  The tiles that are left — fewer than the
-// chip holds workgroups at a time, so that handing them out whole would leave
-// most CUs idle while a few finish — are cut along K: their units form one
-// sequence that `sk_wgs` further workgroups share evenly (the first `r` take
-// q + 1 units, the others q).  A workgroup whose share covers a whole tile
+// Work is counted in units of one K slice of one tile.  `dp_tiles` workgroups
+// each take a whole tile.  The tiles that are left — fewer than the chip holds
+// workgroups at a time, so that handing them out whole would leave most CUs
+// idle while a few finish — are cut along K: their units form one sequence
+// that `sk_wgs` further workgroups share evenly (the first `r` take q + 1
+// units, the others q).  The sharing workgroups have the LOWEST workgroup
+// numbers: they start first, are done after a few slices, and whole tiles take
+// their places, so that the kernel ends with every slot finishing a whole tile
+// at about the same time.  (With the short pieces last, most of the chip idled
+// while they ran: 85 / 153 / 77 / 77 us against 80 / 136 / 70 / 67 us for the
+// four layers of the ResNet-like block, 84 against 71 us for 7x7x512->512.)  A workgroup whose share covers a whole tile
 // stores it as usual; otherwise it stores the raw partial sums of its piece in
 // slot 2s (the piece its share begins with) or 2s + 1 (the piece it ends with)
 // of `part`, and conv_sk_finish adds the pieces of each tile in K order.
@@ -353,11 +369,11 @@ __global__ __launch_bounds__(kThreads) void conv_dma(const float *__restrict__ i
 
     // this workgroup's units [u0, u1) of the sequence (tile 0: units 0..nk-1, tile 1: nk..2nk-1, ...)
     int u0, u1, share = -1;
-    if ((int)blockIdx.x < sk.dp_tiles) {
-        u0 = blockIdx.x * nk;
+    if ((int)blockIdx.x >= sk.sk_wgs) {
+        u0 = ((int)blockIdx.x - sk.sk_wgs) * nk;
         u1 = u0 + nk;
     } else {
-        share = blockIdx.x - sk.dp_tiles;
+        share = blockIdx.x;
         u0 = sk.dp_tiles * nk + share * sk.q + (share < sk.r ? share : sk.r);
         u1 = u0 + sk.q + (share < sk.r ? 1 : 0);
     }
@@ -672,11 +688,11 @@ __global__ __launch_bounds__(kThreads) void conv_dma_lean(const float *__restric
     const int chunk16 = kc_chunk(lane, wave) * 16;   // byte position of this lane's 16 bytes inside a slice of a row
 
     int u0, u1, share = -1;
-    if ((int)blockIdx.x < sk.dp_tiles) {
-        u0 = blockIdx.x * nk;
+    if ((int)blockIdx.x >= sk.sk_wgs) {
+        u0 = ((int)blockIdx.x - sk.sk_wgs) * nk;
         u1 = u0 + nk;
     } else {
-        share = blockIdx.x - sk.dp_tiles;
+        share = blockIdx.x;
         u0 = sk.dp_tiles * nk + share * sk.q + (share < sk.r ? share : sk.r);
         u1 = u0 + sk.q + (share < sk.r ? 1 : 0);
     }
@@ -831,267 +847,6 @@ __global__ __launch_bounds__(kThreads) void conv_dma_lean(const float *__restric
 #endif
 }
 
-// conv_dma for workgroups that stay (opt-in, SWC_HIP_CONV_STREAM=1): as many workgroups as the chip holds at a time,
-// each walking its own list of work — first its share of the tiles cut along K (if it has one), then the whole tiles
-// w, w + G, w + 2G, ... — with the LDS ring running on across the boundaries between pieces: the loads of the next
-// piece's first slices are requested while the last slices of the current one are multiplied, the gather offsets of
-// the next tile are computed in the shadow of those MFMAs, the epilogue's parameters are requested a piece ahead, and
-// the epilogue itself is the accumulator read-out and the stores.  The units, the pieces' slots in `part` and
-// conv_sk_finish are those of conv_dma, and so are the results, bit for bit.
-// Why it is not the default.  A timeline of conv_dma (wall clock per workgroup) shows the start of a tile (gather
-// offsets, two slices requested, the wait for the first: 2 us on an idle chip, a median of 5 - 10 us later on) and
-// its end (3 us) taking a third of a workgroup's lifetime on a K of 576, and the three workgroups of a CU doing both
-// in step — which suggested that workgroups without those phases would run a fifth faster.  Measured, 56x56x64->64 /
-// ->128 / 28x28x128->128 take 94.5 / 177.6 / 88.0 us this way against 91.1 / 172.3 / 85.2 us: per slice a workgroup
-// here needs 2.0 us where conv_dma's need 1.3 - 1.6 us while all three are in their K loops.  Neither a fourth
-// ring stage (two slices of loads in flight, two workgroups per CU: 98.8 / 184.5 / 96.4 us), nor 128x64 or 64x128
-// tiles (171 / 169 us for the second layer), nor start times spread over a slice period changed that.  What the
-// ablations of conv_dma's K loop say instead: without its loads 82 / 156 / 76 us, without its fragment reads 86 /
-// 167 / 81, without the offset arithmetic 84 / 159 / 77, without all three and without the barrier still 76.5 / 142 /
-// 71 — against 47 / 94 / 47 us of pure matrix work: the larger part of the loss is not in the K loop's memory
-// traffic at all.
-template <int TM, int TN, int STAGES>
-__global__ __launch_bounds__(kThreads) void conv_dma_stream(const float *__restrict__ in, const float *__restrict__ filt,
-                                                            float *__restrict__ out, ConvGeom g, unsigned in_bytes,
-                                                            unsigned filt_bytes, Epilogue ep, SkPlan sk,
-                                                            float *__restrict__ part, int pool) {
-#if __HIP_DEVICE_COMPILE__
-    using T = DmaTile<TM, TN, true, STAGES>;
-    static_assert(STAGES >= 3, "ring hand-over in mid-slice");
-    extern __shared__ __align__(16) float lds[];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int M = g.M, N = g.OC, K = g.K;
-    const int tiles_m = (M + T::BM - 1) / T::BM, tiles_n = (N + T::BN - 1) / T::BN;
-    const int nk = (K + BK - 1) / BK;
-    const int entries = sk.sk_wgs + sk.dp_tiles;   // entry e < sk_wgs: share e of the cut tiles; else whole tile e - sk_wgs
-
-    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(in, in_bytes);
-    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(filt, filt_bytes);
-
-    // A walk over this workgroup's pieces, in order: entry e (then e + G, e + 2G, ...), of which units [u0, u1) are
-    // left; `share` is the entry's share of the cut tiles or -1 for a whole tile, `done` the pieces handed out of it.
-    // Two walks run, the loads' (ahead) and the multiplications'.  (Plain integers by reference, no structures: a
-    // structure here ends up in scratch memory, whose accesses count as vector-memory operations and would stall
-    // on the ring's outstanding loads.)
-    const int stride = gridDim.x;
-    auto open_entry = [&](int e, int &u0, int &u1, int &share, int &done) {
-        done = 0;
-        if (e >= sk.sk_wgs) {
-            share = -1;
-            u0 = (e - sk.sk_wgs) * nk;
-            u1 = u0 + nk;
-        } else {
-            share = e;
-            u0 = sk.dp_tiles * nk + e * sk.q + (e < sk.r ? e : sk.r);
-            u1 = u0 + sk.q + (e < sk.r ? 1 : 0);
-        }
-    };
-    // the next piece as (tile, first slice, end slice, slot in `part`); false when the list is exhausted
-    auto next_piece = [&](int &e, int &u0, int &u1, int &share, int &done, int &pid, int &kt_begin, int &kt_end, int &slot) {
-        if (u0 >= u1) {
-            if (e >= entries) return false;
-            e += stride;
-            if (e >= entries) return false;
-            open_entry(e, u0, u1, share, done);
-        }
-        pid = u0 / nk;
-        kt_begin = u0 - pid * nk;
-        kt_end = (u1 - u0 < nk - kt_begin) ? kt_begin + (u1 - u0) : nk;
-        slot = 2 * share + (done ? 1 : 0);
-        u0 += kt_end - kt_begin;
-        ++done;
-        return true;
-    };
-
-    // ---- the loads' side
-    int l_e = blockIdx.x, l_u0 = 0, l_u1 = 0, l_share = -1, l_done = 0;
-    int l_pid = 0, l_kt_begin = 0, l_kt_end = 0, l_slot = 0;
-    bool l_more;          // a piece is open on the loads' side
-    int l_left = 0;       // slices of it not yet requested
-    int row_off[T::kALoads], iy0[T::kALoads], ix0[T::kALoads], f_base[T::kBLoads];
-    int kpos = 0, ky = 0, kx = 0, ci = 0, k_limit = 0;
-    int va[T::kALoads], vb[T::kBLoads];
-    auto open_load_piece = [&]() {   // gather data of piece lp: as at the top of a piece in conv_dma
-        int tile_m, tile_n;
-        sk_tile_coords(l_pid, sk.dp_tiles, tiles_m, tiles_n, tile_m, tile_n);
-        const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
-        k_limit = (l_kt_end * BK < K) ? l_kt_end * BK : K;
-#pragma unroll
-        for (int j = 0; j < T::kALoads; ++j) {
-            const int m = m0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
-            if (m < M) {
-                int img, oy, ox;
-                pixel_of_row(g, m, img, oy, ox);
-                iy0[j] = oy * g.sh - g.pt;
-                ix0[j] = ox * g.sw - g.pl;
-                row_off[j] = ((img * g.H + iy0[j]) * g.W + ix0[j]) * g.C;
-            } else {
-                iy0[j] = ix0[j] = -(1 << 20);
-                row_off[j] = 0;
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < T::kBLoads; ++j) {
-            const int n = n0 + (4 * j + wave) * 8 + kc_row_in_load(lane);
-            f_base[j] = n < N ? n * K * 4 : kOutOfRange;
-        }
-        kpos = l_kt_begin * BK + kc_chunk(lane, wave) * 4;
-        const int tap = kpos / g.C;
-        ci = kpos - tap * g.C;
-        ky = tap / g.kw;
-        kx = tap - ky * g.kw;
-        l_left = l_kt_end - l_kt_begin;
-    };
-    // offsets of the next slice in the workgroup's order (all out of range once its list is exhausted)
-    auto next_offsets = [&]() {
-        if (l_more && l_left == 0) {
-            l_more = next_piece(l_e, l_u0, l_u1, l_share, l_done, l_pid, l_kt_begin, l_kt_end, l_slot);
-            if (l_more) open_load_piece();
-        }
-        if (!l_more) {
-#pragma unroll
-            for (int j = 0; j < T::kALoads; ++j) va[j] = kOutOfRange;
-#pragma unroll
-            for (int j = 0; j < T::kBLoads; ++j) vb[j] = kOutOfRange;
-            return;
-        }
-        const bool k_ok = kpos < k_limit;
-        const int tap_off = (ky * g.W + kx) * g.C + ci;
-#pragma unroll
-        for (int j = 0; j < T::kALoads; ++j) {
-            const bool ok = k_ok && (unsigned)(iy0[j] + ky) < (unsigned)g.H && (unsigned)(ix0[j] + kx) < (unsigned)g.W;
-            va[j] = ok ? (row_off[j] + tap_off) * 4 : kOutOfRange;
-        }
-#pragma unroll
-        for (int j = 0; j < T::kBLoads; ++j) vb[j] = (k_ok && f_base[j] != kOutOfRange) ? f_base[j] + kpos * 4 : kOutOfRange;
-        kpos += BK;
-        ci += BK;
-        while (ci >= g.C) {
-            ci -= g.C;
-            if (++kx == g.kw) {
-                kx = 0;
-                ++ky;
-            }
-        }
-        --l_left;
-    };
-    auto request = [&](float *wr) {
-#pragma unroll
-        for (int j = 0; j < T::kALoads; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t *)(wr + (4 * j + wave) * 256), 16, va[j], 0, 0, 0);
-#pragma unroll
-        for (int j = 0; j < T::kBLoads; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_t *)(wr + T::kAFloats + (4 * j + wave) * 256), 16,
-                                                     vb[j], 0, 0, 0);
-    };
-
-    // ---- the multiplications' side
-    int c_e = blockIdx.x, c_u0 = 0, c_u1 = 0, c_share = -1, c_done = 0;
-    int c_pid = 0, c_kt_begin = 0, c_kt_end = 0, c_slot = 0;   // the piece being multiplied
-    int c_left = 0;        // slices of it still to multiply
-    int c_m0 = 0, c_n0 = 0;
-    ColumnRaw raw[TN];     // its epilogue parameters, requested when it is opened
-    auto open_compute_piece = [&]() {
-        int tile_m, tile_n;
-        sk_tile_coords(c_pid, sk.dp_tiles, tiles_m, tiles_n, tile_m, tile_n);
-        c_m0 = tile_m * T::BM;
-        c_n0 = tile_n * T::BN;
-        c_left = c_kt_end - c_kt_begin;
-        if (c_kt_begin == 0 && c_kt_end == nk && g.win) {
-            const int col_first = c_n0 + (wave & 1) * 32 * TN + (lane & 31);
-#pragma unroll
-            for (int tn = 0; tn < TN; ++tn) raw[tn] = column_raw(ep, col_first + tn * 32, col_first + tn * 32 < N);
-        }
-    };
-
-    v16f acc[TM][TN];
-    auto clear_acc = [&]() {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-    };
-    auto finish_piece = [&]() {
-        acc_settle(acc);
-        if (c_kt_begin == 0 && c_kt_end == nk) {
-            const int row0 = c_m0 + (wave >> 1) * 32 * TM, col0 = c_n0 + (wave & 1) * 32 * TN;
-            if (!g.win) {
-                store_tile<TM, TN>(acc, out, (size_t)N, M, N, row0, col0, lane, ep);
-            } else {
-                ColumnParams cp[TN];
-#pragma unroll
-                for (int tn = 0; tn < TN; ++tn) cp[tn] = column_params(ep, raw[tn]);
-                if (pool) store_tile_windows<TM, TN, true>(acc, out, g, row0, col0, lane, ep, cp);
-                else store_tile_windows<TM, TN, false>(acc, out, g, row0, col0, lane, ep, cp);
-            }
-        } else {
-            float *slot = part + (size_t)c_slot * (T::BM * T::BN);
-            store_tile_impl<TM, TN, false, false>(acc, slot, (size_t)T::BN, T::BM, T::BN, (wave >> 1) * 32 * TM,
-                                                  (wave & 1) * 32 * TN, lane, Epilogue{});
-        }
-    };
-
-    // total slices of this workgroup
-    int total = 0;
-    {
-        int e = blockIdx.x, u0 = 0, u1 = 0, share = -1, done = 0, pid, kb, ke, slot;
-        if (e < entries) {
-            open_entry(e, u0, u1, share, done);
-            while (next_piece(e, u0, u1, share, done, pid, kb, ke, slot)) total += ke - kb;
-        }
-    }
-    if (total == 0) return;
-
-    __builtin_amdgcn_s_setprio(3);
-    open_entry(l_e, l_u0, l_u1, l_share, l_done);
-    l_more = next_piece(l_e, l_u0, l_u1, l_share, l_done, l_pid, l_kt_begin, l_kt_end, l_slot);
-    open_load_piece();
-    open_entry(c_e, c_u0, c_u1, c_share, c_done);
-    next_piece(c_e, c_u0, c_u1, c_share, c_done, c_pid, c_kt_begin, c_kt_end, c_slot);
-    open_compute_piece();
-    __builtin_amdgcn_sched_barrier(0);   // the parameter loads are older than every load of the ring
-#pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s) {
-        next_offsets();
-        request(lds + s * T::kStageFloats);
-    }
-    clear_acc();
-    int rd_stage = 0, wr_stage = STAGES - 1;
-    ring_sync<(STAGES - 2) * T::kLoads>();   // the first slice has landed
-    __builtin_amdgcn_s_setprio(0);
-    Frag<TM, TN> frag[2];
-    load_frag_swz<TM, TN, true>(frag[0], lds, lds + T::kAFloats, 0, wave >> 1, wave & 1, lane & 31, lane >> 5);
-    next_offsets();
-    for (int t = 0; t < total; ++t) {
-        const int nx_stage = rd_stage + 1 == STAGES ? 0 : rd_stage + 1;
-        dma_step_mid<TM, TN, true, STAGES>(lds + wr_stage * T::kStageFloats, lds + rd_stage * T::kStageFloats,
-                                           lds + nx_stage * T::kStageFloats, rsrc_a, rsrc_b, va, vb, acc, frag, wave, lane);
-        next_offsets();   // of the slice the next step requests
-        rd_stage = nx_stage;
-        wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
-        if (--c_left == 0) {
-            __builtin_amdgcn_s_setprio(3);
-            finish_piece();
-            if (next_piece(c_e, c_u0, c_u1, c_share, c_done, c_pid, c_kt_begin, c_kt_end, c_slot)) {
-                open_compute_piece();
-                clear_acc();
-            }
-            // No load into registers may be outstanding when the K loop resumes: the compiler, which cannot know
-            // that the parameter loads above never return into the registers the loop's LDS reads write, would
-            // otherwise wait for ALL vector-memory operations — the ring's loads included — at the top of every
-            // iteration.
-            wait_vmcnt<0>();
-            __builtin_amdgcn_s_setprio(0);
-        }
-    }
-    wait_vmcnt<0>();   // the trailing empty loads still target this workgroup's LDS
-#endif
-}
-
 // Adds the pieces of every shared tile that more than one workgroup worked on (see conv_dma) in K order and
 // applies the epilogue.  blockIdx.x = shared tile, blockIdx.y = block of 16 rows of it.  With `pool` (rows in window
 // order) the finished values of a window's four rows meet in LDS and their maximum is stored.
@@ -1206,11 +961,11 @@ __global__ __launch_bounds__(256) void conv_sk_finish(float *__restrict__ out, c
 // less (one image: 16 tiles of 32 slices for 14 x 14 x 1024 -> 256, 24 us as whole tiles) K = 512 is long enough.
 constexpr int kShareAllMinSlices = 64;   // K >= 2048: below that the pieces and the second kernel cost what the idle CUs do
 int share_all_min_slices() {
-    if (const char *e = getenv("SWC_HIP_CONV_SHARE_ALL"))   // tuning: slices per tile from which a short layer is cut (0: never)
-        return atoi(e) > 0 ? atoi(e) : 1 << 30;
-    return kShareAllMinSlices;
+    const int n = switches().conv_share_all;   // tuning: slices per tile from which a short layer is cut
+    return n > 0 ? n : n < 0 ? 1 << 30 : kShareAllMinSlices;
 }
 
+constexpr int kPieceMinSlices = 4;
 SkPlan sk_plan(long tiles, int nk, int slots, bool allow_shared) {
     SkPlan p{(int)tiles, 0, 0, 0};
     if (!allow_shared || tiles == 0) return p;
@@ -1226,7 +981,9 @@ SkPlan sk_plan(long tiles, int nk, int slots, bool allow_shared) {
     }
     const long units = rest * nk;
     long wgs = slots;
-    if (units < 4 * wgs) wgs = units / 4;   // at least four slices per share: a piece costs a ring start and a tile store
+    // at least kPieceMinSlices slices per share: a piece costs a ring start and a tile store
+    const int piece_min = switches().conv_piece_min > 0 ? switches().conv_piece_min : kPieceMinSlices;
+    if (units < piece_min * wgs) wgs = units / piece_min;
     if (wgs <= rest) return p;              // shares of a tile or more each: nothing to gain
     p.dp_tiles = (int)(tiles - rest);
     p.sk_wgs = (int)wgs;
@@ -1238,31 +995,11 @@ SkPlan sk_plan(long tiles, int nk, int slots, bool allow_shared) {
 // Workgroups of one kernel variant that the chip holds at a time (its LDS and registers decide).
 template <int TM, int TN, int STAGES, bool MID>
 int conv_dma_slots() {
-    if (const char *e = getenv("SWC_HIP_CONV_SLOTS"))   // tests: pretend the chip holds this many workgroups
-        if (atoi(e) > 0) return atoi(e);
+    if (switches().conv_slots > 0) return switches().conv_slots;   // tests: pretend the chip holds this many workgroups
     static int per_cu = 0;
     if (!per_cu) {
         using T = DmaTile<TM, TN, true, STAGES>;
         auto kern = conv_dma<TM, TN, STAGES, MID>;
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)T::kLdsBytes);
-        int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, kThreads, T::kLdsBytes) != hipSuccess || n < 1) {
-            (void)hipGetLastError();
-            n = 1;
-        }
-        per_cu = n;
-    }
-    return per_cu * num_cus();
-}
-
-// The same for conv_dma_stream, whose grid is exactly this number.
-template <int TM, int TN, int STAGES>
-int conv_stream_slots() {
-    static int per_cu = 0;
-    if (!per_cu) {
-        using T = DmaTile<TM, TN, true, STAGES>;
-        auto kern = conv_dma_stream<TM, TN, STAGES>;
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)T::kLdsBytes);
         int n = 0;
@@ -1296,25 +1033,9 @@ int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGe
     const long tiles = (long)((g.M + T::BM - 1) / T::BM) * ((g.OC + T::BN - 1) / T::BN);
     const int nk = (g.K + BK - 1) / BK;
     const SkPlan p = conv_dma_plan<TM, TN, STAGES, MID>(g, scratch != nullptr);
-    // Workgroups that stay and walk a list of pieces (conv_dma_stream): off unless SWC_HIP_CONV_STREAM=1 (test-only) —
-    // on the layer shapes measured it is 2 - 4 % behind one workgroup per tile (see the kernel's comment).
-    bool staying = false;
-    if constexpr (MID) {
-        const char *e = getenv("SWC_HIP_CONV_STREAM");
-        const int slots = conv_stream_slots<TM, TN, STAGES>();
-        staying = e && e[0] == '1' && p.dp_tiles + p.sk_wgs > slots;
-        if (staying) {
-            note_kernel("conv_dma_stream<%d,%d,%d>%s%s", TM, TN, STAGES, p.sk_wgs ? " + conv_sk_finish" : "",
-                        pool ? " (pooled)" : "");
-            conv_dma_stream<TM, TN, STAGES><<<(unsigned)slots, kThreads, T::kLdsBytes, stream()>>>(
-                in, filt, out, g, (unsigned)in_bytes, (unsigned)filt_bytes, ep, p, scratch, pool ? 1 : 0);
-            SWC_LAUNCH_CHECK();
-        }
-    }
     bool lean = false;   // the variant with a K loop free of vector-ALU work (conv_dma_lean); SWC_HIP_CONV_LEAN=0 (test-only) rules it out
     if constexpr (TM == 1 && TN == 1 && STAGES == 3 && MID) {
-        const char *e = getenv("SWC_HIP_CONV_LEAN");
-        lean = !staying && g.C % BK == 0 && !(e && e[0] == '0');
+        lean = g.C % BK == 0 && switches().conv_lean;
         if (lean) {
             note_kernel("conv_dma_lean%s%s", p.sk_wgs ? " + conv_sk_finish" : "", pool ? " (pooled)" : "");
             const size_t out_bytes = (size_t)(pool ? g.M / 4 : g.M) * g.OC * 4;
@@ -1324,7 +1045,7 @@ int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGe
             SWC_LAUNCH_CHECK();
         }
     }
-    if (!staying && !lean) {
+    if (!lean) {
         note_kernel("conv_dma<%d,%d,%d,%s>%s%s", TM, TN, STAGES, MID ? "true" : "false", p.sk_wgs ? " + conv_sk_finish" : "",
                     pool ? " (pooled)" : "");
         auto kern = conv_dma<TM, TN, STAGES, MID>;
@@ -1338,64 +1059,6 @@ int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGe
         SWC_LAUNCH_CHECK();
     }
     return SWC_HIP_OK;
-}
-
-// ------------------------------------------------------------ row-strip kernel (conv_strip.hpp)
-// Layers whose rows divide evenly over the compute units: whole output rows per workgroup, the input patch
-// resident in LDS, no scratch memory and no second kernel.  Off by default (kStripDefault): on the layer shapes
-// measured so far its matrix cores are busy 77 % of the K loop and the tile kernels above, which balance by cutting
-// tiles along K, are level or ahead; SWC_HIP_CONV=strip takes it wherever the planner finds a tiling.
-constexpr bool kStripDefault = false;
-constexpr float kStripMinEff = 0.80f;
-
-// Whether a call with these operands runs on the row-strip kernel, and its plan.  SWC_HIP_CONV (test-only, read
-// per call) = "strip" takes it wherever a plan exists; any other value rules it out.
-bool takes_strip(const ConvGeom &g, const void *input, const void *filter, const void *output, const void *residual,
-                 strip::Plan &p) {
-    const char *force = getenv("SWC_HIP_CONV");
-    if (force && strcmp(force, "strip")) return false;
-    const size_t in_bytes = (size_t)g.N * g.H * g.W * g.C * 4, filt_bytes = (size_t)g.OC * g.K * 4;
-    if (!(aligned16(input) && aligned16(filter) && aligned16(output) && aligned16(residual) && in_bytes < kMaxDmaBytes &&
-          filt_bytes < kMaxDmaBytes))
-        return false;
-    if (const char *e = getenv("SWC_HIP_STRIP_PLAN")) {   // test-only: "R,BN,WM" takes that tiling if the kernel can
-        int R = 0, BN = 0, WM = 0;
-        if (sscanf(e, "%d,%d,%d", &R, &BN, &WM) == 3 && g.C % strip::kChunk == 0 && g.OC % 16 == 0 &&
-            strip::make_plan(g, num_cus(), R, BN, WM, p))
-            return true;
-    }
-    if (!force && !kStripDefault) return false;
-    return strip::plan(g, num_cus(), p) && (force || p.eff >= kStripMinEff);
-}
-
-template <int TMW, int TNW>
-int launch_conv_strip_as(const float *in, const float *filt, float *out, const ConvGeom &g, const strip::Plan &p,
-                         const Epilogue &ep) {
-    note_kernel("conv_strip<%d,%d> R=%d BN=%d", TMW, TNW, p.R, p.BN);
-    auto kern = strip::conv_strip<TMW, TNW>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        SWC_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                        strip::kMaxLds));
-        attr_set = true;
-    }
-    const unsigned in_bytes = (unsigned)((size_t)g.N * g.H * g.W * g.C * 4), filt_bytes = (unsigned)((size_t)g.OC * g.K * 4);
-    kern<<<(unsigned)(p.tiles_m * p.tiles_n), strip::kThreads, (size_t)p.lds_bytes, stream()>>>(in, filt, out, g, p, in_bytes,
-                                                                                                  filt_bytes, ep);
-    SWC_LAUNCH_CHECK();
-    return SWC_HIP_OK;
-}
-
-int launch_conv_strip(const float *in, const float *filt, float *out, const ConvGeom &g, const strip::Plan &p,
-                      const Epilogue &ep) {
-    switch (p.TMW * 10 + p.TNW) {
-    case 71: return launch_conv_strip_as<7, 1>(in, filt, out, g, p, ep);
-    case 72: return launch_conv_strip_as<7, 2>(in, filt, out, g, p, ep);
-    case 74: return launch_conv_strip_as<7, 4>(in, filt, out, g, p, ep);
-    case 131: return launch_conv_strip_as<13, 1>(in, filt, out, g, p, ep);
-    case 132: return launch_conv_strip_as<13, 2>(in, filt, out, g, p, ep);
-    default: return fail(SWC_HIP_ERUNTIME, "conv (row strips): no kernel for %d x %d blocks", p.TMW, p.TNW);
-    }
 }
 
 // ------------------------------------------------------------ small direct conv
@@ -1661,8 +1324,7 @@ template <class F> auto with_dma_variant(int v, F &&f) {
 
 // Whether the leftover tiles are cut along K (SWC_HIP_CONV_SHARE=0 turns it off; read per call).
 bool share_tiles() {
-    const char *e = getenv("SWC_HIP_CONV_SHARE");
-    return !(e && e[0] == '0');
+    return switches().conv_share;
 }
 
 // Variant for a geometry the direct-to-LDS kernels can take; `forced` = SWC_HIP_CONV.
@@ -1725,10 +1387,7 @@ __global__ __launch_bounds__(256) void mask_filter_groups(float *dst, const floa
 
 // Scratch bytes the forward convolution of this geometry uses (0: none).
 size_t conv_scratch_bytes(const ConvGeom &g, const void *input, const void *filter) {
-    const char *force = getenv("SWC_HIP_CONV");
-    strip::Plan sp;
-    if (takes_strip(g, input, filter, nullptr, nullptr, sp)) return 0;   // (output taken as 16-byte aligned: a call whose
-                                                                        // output is not computes every tile whole)
+    const char *force = switches().conv;
     if (!share_tiles() || !conv_uses_dma(g, input, filter, force)) return 0;
     return with_dma_variant(pick_dma_variant(g, force, true), [&]<int TM, int TN, int STAGES, bool MID>() {
         return conv_dma_scratch_bytes<TM, TN, STAGES, MID>(g);
@@ -1756,7 +1415,7 @@ ConvGeom with_channels(ConvGeom g, int c) {
 
 // Scratch bytes a forward convolution uses in all: padded copies (if any) and the pieces of shared tiles.
 size_t conv_total_scratch(const ConvGeom &g, const void *input, const void *filter) {
-    const int cp = padded_channels(g, getenv("SWC_HIP_CONV"));
+    const int cp = padded_channels(g, switches().conv);
     if (!cp) return conv_scratch_bytes(g, input, filter);
     return align256((size_t)g.N * g.H * g.W * cp * 4) + align256((size_t)g.OC * g.kh * g.kw * cp * 4) +
            conv_scratch_bytes(with_channels(g, cp), nullptr, nullptr);
@@ -1767,14 +1426,13 @@ size_t conv_total_scratch(const ConvGeom &g, const void *input, const void *filt
 // and add its products in the same sequence — the pooled result is then bit for bit the maximum of the plain one's.
 // SWC_HIP_CONV_ORDER=raster (test-only) keeps raster order.
 bool window_order(const ConvGeom &g) {
-    const char *e = getenv("SWC_HIP_CONV_ORDER");
-    return g.OH % 2 == 0 && g.OW % 2 == 0 && g.OH > 0 && g.OW > 0 && !(e && !strcmp(e, "raster"));
+    return g.OH % 2 == 0 && g.OW % 2 == 0 && g.OH > 0 && g.OW > 0 && !switches().conv_raster;
 }
 
 // Whether conv_dispatch would run this layer on the direct-to-LDS tile kernels, the ones that can pool in their
 // epilogue (the same tests in the same order as conv_dispatch).
 bool conv_pool_fusable(ConvGeom g, const void *input, const void *filter, const void *output) {
-    const char *force = getenv("SWC_HIP_CONV");
+    const char *force = switches().conv;
     if (!window_order(g)) return false;
     if (force && !strncmp(force, "reg", 3)) return false;
     bool forced_dma = false;
@@ -1785,8 +1443,6 @@ bool conv_pool_fusable(ConvGeom g, const void *input, const void *filter, const 
         g = with_channels(g, cp);
         input = filter = nullptr;   // the padded copies are aligned
     }
-    strip::Plan sp;
-    if (takes_strip(g, input, filter, output, nullptr, sp)) return false;
     return conv_uses_dma(g, input, filter, force);
 }
 
@@ -1858,7 +1514,7 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
     const bool vec = (g.C % 4 == 0) && aligned16(input) && aligned16(filter);
     const size_t M_in = idims[0] * idims[1] * idims[2];
     const size_t in_bytes = M_in * idims[3] * 4, filt_bytes = odims[3] * (size_t)g.K * 4;
-    const char *force = getenv("SWC_HIP_CONV");   // forces a kernel variant (tests, tuning): reg22 reg21 reg12 reg11 | 22_2 21_3 12_3 11_3 11_4 | 11_3m 21_3m 12_3m 22_3m (m: ring hand-over in mid-slice)
+    const char *force = switches().conv;   // forces a kernel variant (tests, tuning): reg22 reg21 reg12 reg11 | 22_2 21_3 12_3 11_3 11_4 | 11_3m 21_3m 12_3m 22_3m (m: ring hand-over in mid-slice)
     if (force && pooled && !strncmp(force, "reg", 3)) return not_pooled();
     if (force) {
         if (!strcmp(force, "reg22")) return launch_conv<2, 2>(vec, input, filter, output, g, ep);
@@ -1894,13 +1550,6 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
                                  bias_optional, ConvScratch{reinterpret_cast<float *>(base + in_b + f_b), need - in_b - f_b},
                                  pooled);
         }
-    }
-    // Whole rows per workgroup where the planner finds an even division ("strip" forces it wherever a plan exists,
-    // any other forced variant rules it out)
-    {
-        strip::Plan sp;
-        if (takes_strip(g, input, filter, output, ep.residual, sp))
-            return pooled ? not_pooled() : launch_conv_strip(input, filter, output, g, sp, ep);
     }
     if (conv_uses_dma(g, input, filter, force)) {
         // the pieces of shared tiles go into the caller's region when it gave one (and none are made if that
@@ -2386,8 +2035,8 @@ GradLayout grad_layout(const ConvGeom &g, const size_t *odims, const size_t *idi
     // with over a tenth fewer: 576 columns are 768 on three wide tiles, 640 on five narrow ones)
     L.narrow = g.OC <= 64;
     L.narrow128 = L.narrow && ((Kf + 127) / 128 * 128) * 11 < ((Kf + 255) / 256 * 256) * 10;
-    if (const char *e = getenv("SWC_HIP_WGRAD_BN"))   // test-only: 128 or 256 forces the width for narrow layers
-        L.narrow128 = L.narrow && atoi(e) == 128;
+    if (switches().wgrad_bn)   // test-only: 128 or 256 forces the width for narrow layers
+        L.narrow128 = L.narrow && switches().wgrad_bn == 128;
     const int bm = L.narrow ? 64 : 128, bn = L.narrow && !L.narrow128 ? 256 : 128;
     const int tiles = ((g.OC + bm - 1) / bm) * (int)((Kf + bn - 1) / bn);
     const int nk = (int)((M + BK - 1) / BK);

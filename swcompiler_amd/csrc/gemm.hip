@@ -761,10 +761,9 @@ bool splitk_plan(int m, int n, int k, int &splits, int &sps, bool forced = false
 
 // The one decision function for "is this product cut along K, and how": the dispatch, swc_hip_gemm_workspace_bytes
 // and the entry point with fixed scratch all ask it, so a size query always matches what the call then does.
-// SWC_HIP_GEMM is a test-only variable (it forces a kernel variant; read per call so that one test process can run
-// every variant): "splitk" forces the cut for shapes the plan would leave whole, any other value rules it out.
+// SWC_HIP_GEMM is a test-only variable (it forces a kernel variant; read once at swc_hip_init, see Switches): "splitk" forces the cut for shapes the plan would leave whole, any other value rules it out.
 bool splitk_decision(int m, int n, int k, int &splits, int &sps) {
-    const char *force = getenv("SWC_HIP_GEMM");
+    const char *force = switches().gemm;
     if (force && strcmp(force, "splitk")) return false;
     return splitk_plan(m, n, k, splits, sps, force != nullptr);
 }
@@ -787,9 +786,8 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
         const unsigned blocks = ceil_div(m, 16);
         // Long K: the streamed kernel.  It wants whole 16-byte pieces (the vec conditions and a contiguous,
         // aligned B) and 32-bit byte offsets inside the 16 rows of a workgroup and inside B.
-        const char *skinny = getenv("SWC_HIP_SKINNY");   // test-only: "plain" keeps gemm_skinny for every shape
         const bool stream_ok = vec && k > 1024 && ldb == n && aligned16(b) && (size_t)lda * 64 < 0x7fff0000u &&
-                               (size_t)k * ldb * 4 < 0x7fff0000u && !(skinny && !strcmp(skinny, "plain"));
+                               (size_t)k * ldb * 4 < 0x7fff0000u && !switches().skinny_plain;   // (test-only switch: gemm_skinny for every shape)
         if (stream_ok) {
             const int slot = stream_slot_bytes(ldb);
             const int ring = (size_t)kStreamWaves * 3 * slot <= Device::ldsBytesPerCU ? 3 : 2;
@@ -805,7 +803,7 @@ int gemm_dispatch(const char *who, int m, int n, int k, const float *a, int lda,
         SWC_LAUNCH_CHECK();
         return SWC_HIP_OK;
     }
-    const char *force = getenv("SWC_HIP_GEMM");
+    const char *force = switches().gemm;
     // a handful of rows and a B of a few MB: one latency-bound pass over B (see gemm_fewrows)
     if (takes_fewrows(m, n, k) && (!force || !strcmp(force, "fewrows"))) {
         note_kernel("gemm_fewrows");

@@ -4,6 +4,7 @@
 // generator prints (src/codegen/Codegen.cpp:154-172, 504-521, 1134-1169).
 #include "common.hpp"
 
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -42,6 +43,40 @@ struct State {
     int n_graphs_on_own_ws = 0;
 } g;
 
+Switches g_switches;
+char g_switch_gemm[32], g_switch_conv[32];
+
+// Reads the SWC_HIP_* variables into g_switches (see Switches).
+void load_switches() {
+    auto text = [](const char *name, char (&buf)[32]) -> const char * {
+        const char *e = getenv(name);
+        if (!e || !e[0]) return nullptr;
+        snprintf(buf, sizeof(buf), "%s", e);
+        return buf;
+    };
+    auto number = [](const char *name) {
+        const char *e = getenv(name);
+        const int v = e ? atoi(e) : 0;
+        return v > 0 ? v : 0;
+    };
+    auto is = [](const char *name, const char *value) {
+        const char *e = getenv(name);
+        return e && !strcmp(e, value);
+    };
+    Switches s;
+    s.gemm = text("SWC_HIP_GEMM", g_switch_gemm);
+    s.conv = text("SWC_HIP_CONV", g_switch_conv);
+    s.skinny_plain = is("SWC_HIP_SKINNY", "plain");
+    s.conv_share = !is("SWC_HIP_CONV_SHARE", "0");
+    s.conv_raster = is("SWC_HIP_CONV_ORDER", "raster");
+    s.conv_lean = !is("SWC_HIP_CONV_LEAN", "0");
+    s.conv_share_all = getenv("SWC_HIP_CONV_SHARE_ALL") ? (number("SWC_HIP_CONV_SHARE_ALL") ? number("SWC_HIP_CONV_SHARE_ALL") : -1) : 0;
+    s.conv_slots = number("SWC_HIP_CONV_SLOTS");
+    s.conv_piece_min = number("SWC_HIP_CONV_PIECE_MIN");
+    s.wgrad_bn = number("SWC_HIP_WGRAD_BN");
+    g_switches = s;
+}
+
 template <typename T> __global__ void fill_kernel(T *__restrict__ dst, T v, size_t n) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t step = (size_t)gridDim.x * blockDim.x;
@@ -67,6 +102,7 @@ void note_kernel(const char *fmt, ...) {
 }
 void clear_error() { g_err[0] = 0, g_err_code = SWC_HIP_OK; }
 int fail_code() { return g_err_code != SWC_HIP_OK ? g_err_code : SWC_HIP_ERUNTIME; }
+const Switches &switches() { return g_switches; }
 hipStream_t stream() { return g.cur; }
 bool ready() { return g.ready; }
 int num_cus() { return g.cus; }
@@ -131,6 +167,7 @@ extern "C" {
 
 int swc_hip_init(int device) {
     std::lock_guard<std::mutex> lk(g.mu);
+    load_switches();
     if (g.ready) {
         if (device != g.device)
             return fail(SWC_HIP_EINVAL, "swc_hip_init: already initialised on device %d", g.device);
@@ -159,6 +196,13 @@ int swc_hip_init(int device) {
     g.device = device;
     g.ready = true;
     clear_error();
+    return SWC_HIP_OK;
+}
+
+int swc_hip_reload_switches(void) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (g.capturing) return fail(SWC_HIP_EINVAL, "swc_hip_reload_switches: not while a graph is being recorded");
+    load_switches();
     return SWC_HIP_OK;
 }
 

@@ -20,7 +20,7 @@ EXPORTS = [
     "swc_hip_d2d", "swc_hip_copy_h2d_async", "swc_hip_copy_wait_ops", "swc_hip_ops_wait_copies", "swc_hip_copy_sync", "swc_hip_fill_f", "swc_hip_sync", "swc_hip_last_error", "swc_hip_stream",
     "swc_hip_set_stream", "swc_hip_device_name", "swc_hip_timer_begin", "swc_hip_timer_end",
     "swc_hip_timer_elapsed_ms", "swc_hip_event_record", "swc_hip_event_elapsed_ms", "swc_hip_graph_begin",
-    "swc_hip_graph_end", "swc_hip_graph_launch", "swc_hip_graph_destroy", "swc_hip_device_cus", "swc_hip_last_kernel",
+    "swc_hip_graph_end", "swc_hip_graph_launch", "swc_hip_graph_destroy", "swc_hip_device_cus", "swc_hip_last_kernel", "swc_hip_reload_switches",
     "swc_hip_enable_auto_workspace", "swc_hip_conv2dGrad_workspace_bytes", "swc_hip_matrixSoftmaxWithLoss_workspace_bytes",
     "swc_hip_matrixMatrixFCBias_noalloc_f",
     "swc_hip_matrixMatrixMul_f", "swc_hip_batchedadd_f", "swc_hip_relu_f",
@@ -56,6 +56,7 @@ def load_library():
     sig = {
         "swc_hip_init": (i32, [i32]),
         "swc_hip_shutdown": (i32, []),
+        "swc_hip_reload_switches": (i32, []),
         "swc_hip_malloc": (vp, [sz]),
         "swc_hip_free": (i32, [vp]),
         "swc_hip_h2d": (i32, [vp, vp, sz]),
@@ -217,6 +218,10 @@ class SwcHip:
 
     def device_cus(self):
         return int(self.lib.swc_hip_device_cus())
+
+    def reload_switches(self):
+        """have the library read the SWC_HIP_* environment variables again (it reads them once, at init)"""
+        self._check(self.lib.swc_hip_reload_switches(), "swc_hip_reload_switches")
 
     # -- plumbing --------------------------------------------------------
     def _check(self, rc, what):

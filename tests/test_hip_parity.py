@@ -230,14 +230,14 @@ def _random_conv_cases(count, seed):
 
 
 @pytest.mark.parametrize("idims,fdims,strides,pads,slots", _random_conv_cases(48, 2024))
-def test_conv_random_shapes_integer_exact(rt, oracle, idims, fdims, strides, pads, slots, monkeypatch):
+def test_conv_random_shapes_integer_exact(rt, oracle, idims, fdims, strides, pads, slots, switch_env):
     """Random layer shapes (channel counts for every kernel form, ragged tiles, strides, uneven padding), on a chip
     pretended to hold 7 or 3 workgroups for two thirds of them so that tiles are cut along K: small-integer operands
     make every order of summation exact, so the result must equal the oracle's bit for bit — plain, with ReLU and a
     second summand, and with the 2x2 pooling where the output allows it."""
     print("case random conv", idims, fdims, strides, pads, slots, flush=True)
     if slots:
-        monkeypatch.setenv("SWC_HIP_CONV_SLOTS", slots)
+        switch_env.setenv("SWC_HIP_CONV_SLOTS", slots)
     rng = np.random.default_rng(sum(idims) * 7 + sum(fdims) * 3 + sum(pads))
     x = rng.integers(-3, 4, idims).astype(np.float32)
     f = rng.integers(-3, 4, fdims).astype(np.float32)
@@ -271,13 +271,13 @@ def _random_wide_lean_cases(count, seed):
 
 
 @pytest.mark.parametrize("idims,fdims,strides,pads,slots", _random_wide_lean_cases(18, 31))
-def test_conv_lean_wide_images_integer_exact(rt, oracle, idims, fdims, strides, pads, slots, monkeypatch):
+def test_conv_lean_wide_images_integer_exact(rt, oracle, idims, fdims, strides, pads, slots, switch_env):
     """conv_dma_lean on images of at least eight 2x2 windows per output row, where the pixel of a row follows from the
     tile's first window by carries (ragged last tiles, strides, tiles cut along K): integer operands, the oracle's bits,
     plain and with the pooled epilogue."""
     print("case wide lean conv", idims, fdims, strides, pads, slots, flush=True)
     if slots:
-        monkeypatch.setenv("SWC_HIP_CONV_SLOTS", slots)
+        switch_env.setenv("SWC_HIP_CONV_SLOTS", slots)
     rng = np.random.default_rng(sum(idims) * 13 + sum(fdims))
     x = rng.integers(-3, 4, idims).astype(np.float32)
     f = rng.integers(-3, 4, fdims).astype(np.float32)
@@ -581,9 +581,9 @@ GEMM_VARIANTS = ["reg", "22_2", "22_3", "21_3", "12_3", "11_3", "11_4", "11_3m",
 
 
 @pytest.mark.parametrize("variant", GEMM_VARIANTS)
-def test_gemm_every_variant(rt, oracle, variant, monkeypatch):
+def test_gemm_every_variant(rt, oracle, variant, switch_env):
     print("case gemm variant", variant, flush=True)
-    monkeypatch.setenv("SWC_HIP_GEMM", variant)
+    switch_env.setenv("SWC_HIP_GEMM", variant)
     rng = np.random.default_rng(11)
     for m, k, n in [(300, 200, 260), (128, 64, 128), (70, 36, 132), (64, 4, 64)]:
         a = rng.integers(-8, 9, (m, k)).astype(np.float32)
@@ -640,13 +640,13 @@ POOLED_CONVS = [
 
 @pytest.mark.parametrize("idims,fdims,pads", POOLED_CONVS)
 @pytest.mark.parametrize("slots", [None, "7"])
-def test_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, pads, slots, monkeypatch):
+def test_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, pads, slots, switch_env):
     """conv (+BN) (+ReLU) + 2x2/2 max-pooling in one call is bit for bit the pooling of the separate convolution:
     both put a pixel into the same tile (rows in window order) and add its products in the same sequence, whole
     tiles and tiles cut along K alike (slots = 7 pretends a chip of seven workgroups, so that most tiles are cut)."""
     print("case pooled conv", idims, fdims, pads, slots, flush=True)
     if slots:
-        monkeypatch.setenv("SWC_HIP_CONV_SLOTS", slots)
+        switch_env.setenv("SWC_HIP_CONV_SLOTS", slots)
     rng = np.random.default_rng(sum(idims) + sum(fdims))
     oc, c = fdims[0], fdims[3]
     x = rng.standard_normal(idims).astype(np.float32)
@@ -676,7 +676,7 @@ def test_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, pads, s
     scale = oracle.maxpool(oracle.conv2d(np.abs(x[:n]), np.abs(f), np.abs(b), pads=pads) * slope + np.abs(bn[3]), *pool)
     assert scaled_err(got, ref, scale) < TOL
     # raster order of the rows gives the same values up to the order of summation of the tiles cut along K
-    monkeypatch.setenv("SWC_HIP_CONV_ORDER", "raster")
+    switch_env.setenv("SWC_HIP_CONV_ORDER", "raster")
     raster = rt.maxpool(rt.conv2d(dx, df, db, pads=pads, bn=dbn, eps=1e-5, relu=True), *pool).numpy()[:n]
     assert scaled_err(raster, ref, scale) < TOL
     if not slots and rt.last_kernel().find("conv_sk_finish") < 0:
@@ -688,14 +688,15 @@ def test_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, pads, s
                                               ((3, 10, 6, 32), (70, 3, 3, 32), (1, 1, 1, 1)),
                                               ((2, 9, 11, 96), (64, 5, 5, 96), (2, 2, 2, 2)),     # odd output: raster order
                                               ((4, 16, 16, 64), (64, 1, 1, 64), (0, 0, 0, 0))])
-@pytest.mark.parametrize("slots", [None, "7"])
-def test_conv_kernel_forms_agree_bit_for_bit(rt, idims, fdims, pads, slots, monkeypatch):
-    """The three forms of the 64x64-tile kernel — conv_dma, conv_dma_lean (channel counts that are multiples of 32:
-    no vector-ALU work in the K loop) and conv_dma_stream (workgroups that stay, opt-in) — walk K in the same order
-    and cut the same tiles: the same bits, whole and cut tiles, plain and pooled."""
+@pytest.mark.parametrize("slots", [None, "11"])
+def test_conv_kernel_forms_agree_bit_for_bit(rt, idims, fdims, pads, slots, switch_env):
+    """The two forms of the 64x64-tile kernel — conv_dma and conv_dma_lean (channel counts that are multiples of 32:
+    no vector-ALU work in the K loop) — walk K in the same order and cut the same tiles: the same bits, whole and
+    cut tiles, plain and pooled.  (Eleven slots: every layer here then stays on the 64x64 tiles, and the two
+    full-size ones have tiles cut along K.)"""
     print("case conv kernel forms", idims, fdims, pads, slots, flush=True)
     if slots:
-        monkeypatch.setenv("SWC_HIP_CONV_SLOTS", slots)
+        switch_env.setenv("SWC_HIP_CONV_SLOTS", slots)
     rng = np.random.default_rng(sum(idims) * 3 + sum(fdims))
     oc = fdims[0]
     x = rng.standard_normal(idims).astype(np.float32)
@@ -706,25 +707,21 @@ def test_conv_kernel_forms_agree_bit_for_bit(rt, idims, fdims, pads, slots, monk
     dx, df, db = up(rt, x, f, b)
     kw = dict(pads=pads, bn=bn, eps=1e-5, relu=True)
     lean = rt.conv2d(dx, df, db, **kw).numpy()
-    if slots and not rt.last_kernel().startswith("conv_dma_lean"):
-        pytest.skip("on a chip of seven workgroups the planner gives this layer another tile shape: " + rt.last_kernel())
     assert rt.last_kernel().startswith("conv_dma_lean"), rt.last_kernel()
-    monkeypatch.setenv("SWC_HIP_CONV_LEAN", "0")
+    if slots and idims[0] >= 32:
+        assert "conv_sk_finish" in rt.last_kernel(), rt.last_kernel()
+    switch_env.setenv("SWC_HIP_CONV_LEAN", "0")
     plain = rt.conv2d(dx, df, db, **kw).numpy()
     assert rt.last_kernel().startswith("conv_dma<1,1,3,true>"), rt.last_kernel()
     assert_bit_exact(lean, plain, "conv_dma_lean vs conv_dma")
-    monkeypatch.setenv("SWC_HIP_CONV_STREAM", "1")
-    staying = rt.conv2d(dx, df, db, **kw).numpy()
-    assert_bit_exact(staying, plain, "conv_dma_stream vs conv_dma")
     if idims[1] % 2 == 0 and idims[2] % 2 == 0 and fdims[1] != 5:
         pool = ((2, 2), (2, 2))
-        staying_pooled = rt.conv2d(dx, df, db, pool=pool, **kw).numpy()
-        monkeypatch.delenv("SWC_HIP_CONV_STREAM")
-        monkeypatch.delenv("SWC_HIP_CONV_LEAN")
+        plain_pooled = rt.conv2d(dx, df, db, pool=pool, **kw).numpy()
+        switch_env.delenv("SWC_HIP_CONV_LEAN")
         lean_pooled = rt.conv2d(dx, df, db, pool=pool, **kw).numpy()
         assert rt.last_kernel().startswith("conv_dma_lean") and rt.last_kernel().endswith("(pooled)"), rt.last_kernel()
         assert_bit_exact(lean_pooled, rt.maxpool(rt.upload(plain), *pool).numpy(), "pooled, lean")
-        assert_bit_exact(staying_pooled, lean_pooled, "pooled, staying")
+        assert_bit_exact(plain_pooled, lean_pooled, "pooled, general form")
 
 
 @pytest.mark.parametrize("idims,fdims,pads", [((256, 28, 28, 1), (20, 5, 5, 1), (0, 0, 0, 0)),      # LeNet's first layer
@@ -796,7 +793,7 @@ STREAMED_HEADS = [(4096, 4096, 10), (1000, 4096, 10), (33, 1028, 7), (16, 2048, 
 
 
 @pytest.mark.parametrize("m,k,n", STREAMED_HEADS)
-def test_skinny_gemm_streamed_along_k(rt, oracle, m, k, n, monkeypatch):
+def test_skinny_gemm_streamed_along_k(rt, oracle, m, k, n, switch_env):
     """N <= 16 behind a K above 1024: A and B by LDS-DMA through per-wavefront rings.  Integer-valued operands make the
     result exact whatever the order of summation, so every k, every row and every column is checked bit by bit (rows
     and k past the end must come in as zeros, not as whatever the ring held); then real-valued data against the
@@ -834,7 +831,7 @@ def test_skinny_gemm_streamed_along_k(rt, oracle, m, k, n, monkeypatch):
     assert rt.last_kernel().startswith("gemm_skinny_stream<"), rt.last_kernel()
     assert_bit_exact(out.numpy(), (wide[:, :k].astype(np.int64) @ b.astype(np.int64)).astype(np.float32), "lda > k")
     # the plain kernel gives the same integers
-    monkeypatch.setenv("SWC_HIP_SKINNY", "plain")
+    switch_env.setenv("SWC_HIP_SKINNY", "plain")
     assert_bit_exact(rt.fcbias(da, db, dbias, relu=False).numpy(), want, "plain kernel")
     assert rt.last_kernel().startswith("gemm_skinny<"), rt.last_kernel()
 
@@ -916,9 +913,9 @@ def test_gemm_split_over_k_uses_exactly_the_size_it_reports(rt, oracle):
 
 
 @pytest.mark.parametrize("variant", ["reg22", "reg21", "reg12", "reg11", "22_2", "21_3", "12_3", "11_3", "11_4", "11_3m", "21_3m", "12_3m", "22_3m"])
-def test_conv_every_variant(rt, oracle, variant, monkeypatch):
+def test_conv_every_variant(rt, oracle, variant, switch_env):
     print("case conv variant", variant, flush=True)
-    monkeypatch.setenv("SWC_HIP_CONV", variant)
+    switch_env.setenv("SWC_HIP_CONV", variant)
     rng = np.random.default_rng(12)
     for idims, fdims, strides, pads in [((2, 9, 10, 8), (40, 3, 3, 8), (1, 1), (1, 1, 1, 1)),
                                         ((1, 13, 11, 20), (70, 5, 5, 20), (2, 1), (2, 2, 2, 2)),
@@ -940,10 +937,10 @@ SHARED_CONV_CASES = [((2, 20, 20, 32), (70, 3, 3, 32), (1, 1), (1, 1, 1, 1)),   
 
 
 @pytest.mark.parametrize("variant", [None, "11_3m", "11_4", "21_3", "12_3m", "22_2", "22_3m"])
-def test_conv_tiles_shared_along_k(rt, oracle, variant, monkeypatch):
+def test_conv_tiles_shared_along_k(rt, oracle, variant, switch_env):
     print("case conv shared tiles, variant", variant, flush=True)
     if variant:
-        monkeypatch.setenv("SWC_HIP_CONV", variant)
+        switch_env.setenv("SWC_HIP_CONV", variant)
     rng = np.random.default_rng(31)
     for idims, fdims, strides, pads in SHARED_CONV_CASES:
         oc = fdims[0]
@@ -956,13 +953,13 @@ def test_conv_tiles_shared_along_k(rt, oracle, variant, monkeypatch):
         dx, df, db = up(rt, x, f, b)
         bn = up(rt, mean, var, gamma, beta)
         want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
-        monkeypatch.setenv("SWC_HIP_CONV_SHARE", "0")
+        switch_env.setenv("SWC_HIP_CONV_SHARE", "0")
         assert rt.conv2d_workspace_bytes(idims, fdims, strides, pads) == 0
         whole = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, bn=bn, eps=1e-5, relu=True).numpy()
-        monkeypatch.setenv("SWC_HIP_CONV_SHARE", "1")
+        switch_env.setenv("SWC_HIP_CONV_SHARE", "1")
         shared = 0
         for slots in (3, 4, 5, 6, 7, 9, 11, 13, 17, 19, 23, 29, 37, 47):
-            monkeypatch.setenv("SWC_HIP_CONV_SLOTS", str(slots))
+            switch_env.setenv("SWC_HIP_CONV_SLOTS", str(slots))
             shared += rt.conv2d_workspace_bytes(idims, fdims, strides, pads) > 0
             plain = rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy()
             fused = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, bn=bn, eps=1e-5, relu=True).numpy()
@@ -970,11 +967,11 @@ def test_conv_tiles_shared_along_k(rt, oracle, variant, monkeypatch):
             # reference's, and the fused epilogue sees the same sums whether a tile was cut or not
             assert_bit_exact(plain, want, f"shared tiles {idims} {variant} slots {slots}")
             assert_bit_exact(fused, whole, f"shared tiles, fused epilogue {idims} {variant} slots {slots}")
-        monkeypatch.delenv("SWC_HIP_CONV_SLOTS")
+        switch_env.delenv("SWC_HIP_CONV_SLOTS")
         assert shared, f"{idims} {variant}: no slot count made this case share tiles"
     # real-valued operands: the usual tolerance
     idims, fdims, strides, pads = SHARED_CONV_CASES[1]
-    monkeypatch.setenv("SWC_HIP_CONV_SLOTS", "4")
+    switch_env.setenv("SWC_HIP_CONV_SLOTS", "4")
     x = rng.standard_normal(idims).astype(np.float32)
     f = rng.standard_normal(fdims).astype(np.float32)
     b = rng.standard_normal(fdims[0]).astype(np.float32)
@@ -988,7 +985,7 @@ def test_conv_tiles_shared_along_k(rt, oracle, variant, monkeypatch):
                                                       ((1, 9, 9, 2048), (64, 1, 1, 2048), (1, 1), (0, 0, 0, 0)),   # 1x1, 2 tiles of 64 slices
                                                       ((3, 14, 14, 96), (72, 3, 3, 96), (2, 2), (1, 1, 1, 1)),      # 6 tiles of 27 slices: few enough tiles
                                                       ((3, 14, 14, 32), (72, 3, 3, 32), (2, 2), (1, 1, 1, 1))])     # 9 slices: below the limit
-def test_conv_layers_of_few_tiles_and_a_long_k_are_cut_throughout(rt, oracle, idims, fdims, strides, pads, monkeypatch):
+def test_conv_layers_of_few_tiles_and_a_long_k_are_cut_throughout(rt, oracle, idims, fdims, strides, pads, switch_env):
     """Fewer tiles than the chip holds workgroups and K >= 2048 (K >= 512 for a twelfth of a round or less): every
     tile is cut along K (no whole tiles at all)."""
     print("case conv, all tiles shared", idims, fdims, flush=True)
@@ -1002,15 +999,15 @@ def test_conv_layers_of_few_tiles_and_a_long_k_are_cut_throughout(rt, oracle, id
     dx, df, db = up(rt, x, f, b)
     for slots in (None, 5, 9, 37, 100):
         if slots:
-            monkeypatch.setenv("SWC_HIP_CONV_SLOTS", str(slots))
+            switch_env.setenv("SWC_HIP_CONV_SLOTS", str(slots))
         assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy(), want, f"all tiles shared, slots {slots}")
         assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True).numpy(), oracle.relu(want),
                          f"all tiles shared + relu, slots {slots}")
-    monkeypatch.delenv("SWC_HIP_CONV_SLOTS")
-    monkeypatch.setenv("SWC_HIP_CONV_SHARE_ALL", "0")
+    switch_env.delenv("SWC_HIP_CONV_SLOTS")
+    switch_env.setenv("SWC_HIP_CONV_SHARE_ALL", "0")
     assert rt.conv2d_workspace_bytes(idims, fdims, strides, pads) == 0
     assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy(), want, "whole tiles")
-    monkeypatch.setenv("SWC_HIP_CONV_SHARE_ALL", "8")
+    switch_env.setenv("SWC_HIP_CONV_SHARE_ALL", "8")
     assert rt.conv2d_workspace_bytes(idims, fdims, strides, pads) > 0
     xr = rng.standard_normal(idims).astype(np.float32)
     fr = rng.standard_normal(fdims).astype(np.float32)
@@ -1063,11 +1060,11 @@ RESIDUAL_CONV_CASES = [((2, 14, 14, 64), (256, 1, 1, 64), (1, 1), (0, 0, 0, 0)),
 
 @pytest.mark.parametrize("idims,fdims,strides,pads", RESIDUAL_CONV_CASES)
 @pytest.mark.parametrize("variant", [None, "reg11", "22_3m"])
-def test_conv_with_a_second_summand(rt, oracle, idims, fdims, strides, pads, variant, monkeypatch):
+def test_conv_with_a_second_summand(rt, oracle, idims, fdims, strides, pads, variant, switch_env):
     """conv2dFusedAdd_f = conv2d_f, batchnormalization_f, vecAdd_f with the other branch, relu_f."""
     print("case conv + residual", idims, fdims, variant, flush=True)
     if variant:
-        monkeypatch.setenv("SWC_HIP_CONV", variant)
+        switch_env.setenv("SWC_HIP_CONV", variant)
     rng = np.random.default_rng(sum(idims) + sum(fdims))
     oc = fdims[0]
     x = rng.integers(-4, 5, idims).astype(np.float32)
@@ -1103,10 +1100,10 @@ def test_conv_with_a_second_summand(rt, oracle, idims, fdims, strides, pads, var
     assert np.max(np.abs(fused - want) / mag) < TOL
 
 
-def test_conv_shared_tiles_in_a_caller_workspace(rt, oracle, monkeypatch):
+def test_conv_shared_tiles_in_a_caller_workspace(rt, oracle, switch_env):
     from swcompiler_amd.hip import SwcHipError
     idims, fdims, strides, pads = SHARED_CONV_CASES[0]
-    monkeypatch.setenv("SWC_HIP_CONV_SLOTS", "19")
+    switch_env.setenv("SWC_HIP_CONV_SLOTS", "19")
     need = rt.conv2d_workspace_bytes(idims, fdims, strides, pads)
     assert need > 0
     rng = np.random.default_rng(32)
@@ -1143,66 +1140,15 @@ def test_small_direct_conv_is_bit_exact(rt, oracle, idims, fdims, strides, pads)
     assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True).numpy(), oracle.relu(want), "direct conv + relu")
 
 
-# ---------------------------------------------------------------- row-strip convolution kernel
-# Layers with channel counts that are multiples of 16 whose rows divide evenly over the compute units run on
-# a kernel that gives every workgroup whole output rows (the planner decides; SWC_HIP_CONV=strip takes it
-# wherever a plan exists, so small shapes can exercise it).
-STRIP_CONV_CASES = [((2, 8, 8, 16), (16, 3, 3, 16), (1, 1), (1, 1, 1, 1)),
-                    ((3, 14, 14, 32), (32, 3, 3, 32), (1, 1), (1, 1, 1, 1)),      # 196 pixels per image: 12.25 blocks of 16
-                    ((1, 12, 10, 16), (48, 3, 3, 16), (1, 1), (0, 0, 0, 0)),      # no padding, 48 output channels
-                    ((2, 9, 9, 16), (32, 5, 5, 16), (1, 1), (2, 2, 2, 2)),        # 5 x 5 taps
-                    ((2, 13, 11, 16), (16, 3, 3, 16), (2, 2), (1, 1, 1, 1)),      # stride 2
-                    ((5, 14, 14, 64), (128, 3, 3, 64), (1, 1), (1, 1, 1, 1)),     # four channel chunks, eight column blocks
-                    ((2, 28, 28, 128), (64, 3, 3, 128), (1, 1), (1, 1, 1, 1))]
-
-
-@pytest.mark.parametrize("idims,fdims,strides,pads", STRIP_CONV_CASES)
-def test_conv_row_strips(rt, oracle, idims, fdims, strides, pads, monkeypatch):
-    print("case conv row strips", idims, fdims, strides, flush=True)
-    monkeypatch.setenv("SWC_HIP_CONV", "strip")
-    assert rt.conv2d_workspace_bytes(idims, fdims, strides, pads) == 0    # no scratch memory, no second kernel
-    rng = np.random.default_rng(sum(idims) + sum(fdims))
-    oc = fdims[0]
-    x = rng.integers(-4, 5, idims).astype(np.float32)
-    f = rng.integers(-4, 5, fdims).astype(np.float32)
-    b = rng.integers(-4, 5, oc).astype(np.float32)
-    dx, df, db = up(rt, x, f, b)
-    want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
-    assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy(), want, "integer-valued")
-    assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True).numpy(), oracle.relu(want), "+ relu")
-    res = rng.integers(-40, 41, want.shape).astype(np.float32)
-    assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads, residual=rt.upload(res), relu=True).numpy(),
-                     oracle.relu(oracle.vecAdd(want.ravel(), res.ravel()).reshape(want.shape)), "+ residual + relu")
-    # fused batchnorm + relu: the same epilogue arithmetic as the tile kernels (bit-identical to them)
-    mean, beta = (rng.integers(-4, 5, oc).astype(np.float32) for _ in range(2))
-    var = rng.uniform(0.5, 2.0, oc).astype(np.float32)
-    gamma = rng.uniform(0.5, 1.5, oc).astype(np.float32)
-    bn = up(rt, mean, var, gamma, beta)
-    fused = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, bn=bn, eps=1e-5, relu=True).numpy()
-    monkeypatch.setenv("SWC_HIP_CONV", "11_3m")
-    assert_bit_exact(fused, rt.conv2d(dx, df, db, fdims[1:3], strides, pads, bn=bn, eps=1e-5, relu=True).numpy(),
-                     "conv + bn + relu against the tile kernel")
-    monkeypatch.setenv("SWC_HIP_CONV", "strip")
-    # real-valued operands
-    xr = rng.standard_normal(idims).astype(np.float32)
-    fr = (rng.standard_normal(fdims) / np.sqrt(np.prod(fdims[1:]))).astype(np.float32)
-    br = rng.standard_normal(oc).astype(np.float32)
-    got = rt.conv2d(*up(rt, xr, fr, br), fdims[1:3], strides, pads, bn=bn, eps=1e-5, relu=True).numpy()
-    ref = oracle.relu(oracle.batchnormalization(oracle.conv2d(xr, fr, br, fdims[1:3], strides, pads), mean, var, gamma, beta, 1e-5))
-    mag = np.abs(oracle.batchnormalization(oracle.conv2d(np.abs(xr), np.abs(fr), np.abs(br), fdims[1:3], strides, pads),
-                                           -np.abs(mean), var, gamma, np.abs(beta), 1e-5))
-    assert np.max(np.abs(got - ref) / mag) < TOL
-
-
 @pytest.mark.parametrize("idims,oc", [((32, 56, 56, 64), 64), ((32, 56, 56, 64), 128), ((32, 28, 28, 128), 128)])
-@pytest.mark.parametrize("variant", [None, "strip"])
-def test_conv_block_layers_full_size(rt, oracle, idims, oc, variant, monkeypatch):
+@pytest.mark.parametrize("variant", [None, "11_3m"])
+def test_conv_block_layers_full_size(rt, oracle, idims, oc, variant, switch_env):
     """The convolutions of the ResNet-stage-like block at their full sizes, as the default dispatch runs them and
-    on the row-strip kernel (a whole number of tiles per compute unit on a whole MI355X): integer-valued operands,
-    three images through the oracle bit for bit and the exact sum over the whole output."""
+    on the general form of the tile kernel: integer-valued operands, three images through the oracle bit for bit
+    and the exact sum over the whole output."""
     print("case conv block layer, full size", idims, oc, variant, flush=True)
     if variant:
-        monkeypatch.setenv("SWC_HIP_CONV", variant)
+        switch_env.setenv("SWC_HIP_CONV", variant)
     fdims = (oc, 3, 3, idims[3])
     rng = np.random.default_rng(oc + idims[1])
     x = rng.integers(-3, 4, idims).astype(np.float32)

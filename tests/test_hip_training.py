@@ -213,13 +213,13 @@ def _random_grad_cases(count, seed):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("idims,fdims,st,pd,slots", _random_grad_cases(32, 777))
-def test_conv2dGrad_random_shapes_integer_exact(rt, oracle, idims, fdims, st, pd, slots, monkeypatch):
+def test_conv2dGrad_random_shapes_integer_exact(rt, oracle, idims, fdims, st, pd, slots, switch_env):
     """Random layer shapes (strides, uneven padding, channel counts for every kernel form of the three gradients; on
     a chip pretended to hold seven workgroups for every other one): with small-integer operands any order of
     summation is exact, so inputG, filterG and biasG must equal the oracle's bit for bit."""
     print("case random conv2dGrad", idims, fdims, st, pd, slots, flush=True)
     if slots:
-        monkeypatch.setenv("SWC_HIP_CONV_SLOTS", slots)
+        switch_env.setenv("SWC_HIP_CONV_SLOTS", slots)
     rng = np.random.default_rng(sum(idims) * 11 + sum(fdims) * 5 + sum(pd))
     n, oh, ow, _ = pool_out_dims(idims, fdims[1:3], st, pd)
     odims = (n, oh, ow, fdims[0])
@@ -259,7 +259,7 @@ def test_conv2dGrad_many_pixels_split_k(rt, oracle):
 @pytest.mark.gpu
 @pytest.mark.parametrize("width", ["128", "256", None])
 @pytest.mark.parametrize("fdims", [(24, 3, 3, 32), (40, 1, 1, 128), (24, 1, 1, 256), (24, 3, 3, 128), (24, 1, 1, 1408)])
-def test_conv2dGrad_narrow_layer_tile_widths(rt, oracle, monkeypatch, width, fdims):
+def test_conv2dGrad_narrow_layer_tile_widths(rt, oracle, switch_env, width, fdims):
     """up to 64 output channels: the filter gradient runs on 64 x 128 or 64 x 256 tiles (SWC_HIP_WGRAD_BN forces one;
     unset, the narrow tiles are taken where they cover the kh*kw*iC columns with over a tenth fewer: 288 and 128
     columns take them; 256 columns fill one wide tile exactly and keep it; 1152 columns (nine narrow tiles against
@@ -267,9 +267,9 @@ def test_conv2dGrad_narrow_layer_tile_widths(rt, oracle, monkeypatch, width, fdi
     0.917) just on the wide side).  Integer-valued operands: the gradients equal the oracle's bit for bit on either."""
     print("case conv2dGrad tile width", width, fdims, flush=True)
     if width is None:
-        monkeypatch.delenv("SWC_HIP_WGRAD_BN", raising=False)
+        switch_env.delenv("SWC_HIP_WGRAD_BN", raising=False)
     else:
-        monkeypatch.setenv("SWC_HIP_WGRAD_BN", width)
+        switch_env.setenv("SWC_HIP_WGRAD_BN", width)
     rng = np.random.default_rng(fdims[0])
     k = fdims[1]
     pads = (k // 2,) * 4
