@@ -19,7 +19,7 @@ BENCH_LIB = os.path.join(HERE, "libswc_hip_bench.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "-Wno-unused-command-line-argument", "-Wno-unknown-attributes"]
+         "-Wno-unused-command-line-argument", "-Wno-unknown-attributes"] + os.environ.get("SWC_HIP_HIPCC_FLAGS", "").split()
 
 
 def sources():

@@ -14,8 +14,10 @@
 #include "mfma_dma.hpp"
 #include "mfma_dma2.hpp"
 #include "mfma_tile.hpp"
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
 
 using namespace swc_hip;
 using namespace swc_hip::mfma;
@@ -334,19 +336,21 @@ struct SkPlan {
     int q, r;       // units per sharing workgroup: q, and one more for the first r
 };
 
-// Tile number -> tile coordinates (see tile_coords): the whole tiles are renumbered for the 8 XCDs, the
-// shared ones are taken in order.
-__device__ __forceinline__ void sk_tile_coords(int pid, int dp_tiles, int tiles_m, int tiles_n, int &tile_m, int &tile_n) {
+// Tile number -> tile coordinates.  Workgroups are dealt round-robin to the 8 XCDs, each with its own L2; the whole
+// tiles (all but the last few) are renumbered so that the ones one XCD works on are consecutive; consecutive numbers
+// walk the column tiles of one block of rows, then the next block of rows: the tiles an XCD holds at a time share
+// their rows of the gathered operand (the filter, a few hundred KB, stays in every L2 anyway).  The shared tiles are
+// taken in order.
+__device__ __forceinline__ int xcd_renumbered(int pid, int dp_tiles) {
     constexpr int kXcd = Device::xcds;
-    if (pid < dp_tiles && dp_tiles % kXcd == 0) pid = (pid % kXcd) * (dp_tiles / kXcd) + pid / kXcd;
-    constexpr int kGroup = 8;
-    const int per_group = kGroup * tiles_n;
-    const int group = pid / per_group;
-    const int first_m = group * kGroup;
-    const int rows = (tiles_m - first_m < kGroup) ? (tiles_m - first_m) : kGroup;
-    const int in_group = pid - group * per_group;
-    tile_m = first_m + in_group % rows;
-    tile_n = in_group / rows;
+    const int full = dp_tiles - dp_tiles % kXcd;
+    return pid < full ? (pid % kXcd) * (full / kXcd) + pid / kXcd : pid;
+}
+__device__ __forceinline__ void sk_tile_coords(int pid, int dp_tiles, int tiles_m, int tiles_n, int &tile_m, int &tile_n) {
+    (void)tiles_m;
+    pid = xcd_renumbered(pid, dp_tiles);
+    tile_m = pid / tiles_n;
+    tile_n = pid - tile_m * tiles_n;
 }
 
 template <int TM, int TN, int STAGES, bool MID = false>
@@ -847,6 +851,363 @@ __global__ __launch_bounds__(kThreads) void conv_dma_lean(const float *__restric
 #endif
 }
 
+// ------------------------------------------------------------------------------------------------ conv_win
+// The tile kernel of the layers that matter most: output with whole 2 x 2 windows (rows in window order), a channel
+// count that is a multiple of 32, tensors below 2 GiB.  Tile (64 x 64), ring, swizzle, MFMA order, pieces, slots and
+// epilogue arithmetic are conv_dma<1,1,3,true>'s — the same bits — but a vector-ALU instruction issued by ANY
+// wavefront of a SIMD costs that SIMD 2-5 cycles of matrix throughput, so everything around the MFMAs is cut down to
+// what the arithmetic needs:
+//   * all geometry comes from one argument record in the kernel-argument segment; tile and window coordinates are
+//     scalar arithmetic with precomputed multiply-shift divisions (no division runs in the vector unit, no
+//     argument is kept in a vector register across the K loop);
+//   * the gather offset of a row is lane constant + scalar: the descriptor starts (pt*W + pl) pixels below the
+//     input, which makes a row's top-left tap offset non-negative, and the tap position travels in the load's
+//     scalar offset with the channel position.  A change of filter tap only re-selects between that constant and
+//     "out of range" (3 instructions per row: the column test; the row test is a lane mask kept per filter row);
+//   * the K loop holds no vector-ALU instruction at all: its LDS reads are assembly with immediate offsets;
+//   * the pixel of a window follows from its number w by one division: 2 x 2 windows in raster order make the
+//     output offset of window w's first pixel 2 OC (w + floor(w / pw) pw) — no image or row coordinates.
+// Measured against conv_dma_lean in alternating runs on one box, the four layers of the ResNet-like block:
+// 73.5 / 133.2 / 69.1 / 67.5 -> 68.2 / 120.2 / 64.9 / 63.7 us.  Tried with it and dropped: 128 x 64 tiles (a wavefront
+// owning 64 x 32; three ring stages with two workgroups per CU, or two stages with three): 77.4 / 123.8 / 72.2 / 71.4 and
+// 71.4 / 122.9 / 75.2 / 74.1 us — fewer bytes per MFMA buy nothing here.
+struct Magic {   // x / d for 0 <= x < 2^31 as (umulhi(x, mul) + x) >> shift
+    unsigned mul, shift;
+};
+Magic magic_of(unsigned d) {
+    unsigned shift = 0;
+    while ((1ull << shift) < d) ++shift;
+    return Magic{(unsigned)(((1ull << 32) * ((1ull << shift) - d)) / d + 1), shift};
+}
+__device__ __forceinline__ int magic_div(int x, Magic m) { return (int)((__umulhi((unsigned)x, m.mul) + (unsigned)x) >> m.shift); }
+
+struct WinArgs {
+    const float *in, *filt;
+    float *out;
+    float *part;                        // slots for the pieces of tiles cut along K
+    Epilogue ep;
+    SkPlan sk;
+    unsigned in_bytes, filt_bytes, out_bytes;   // out_bytes: of the tensor that is written (pooled or not)
+    int shift_bytes;                    // (pt * W + pl) * C * 4: how far below the input its descriptor starts
+    int N, K, C, H, W, kw, sh, sw, pt, pl, OW;
+    int pw, ph, nwin;                   // windows per output row and column, windows in all (M / 4)
+    int tiles_n, nk, cpt;               // column tiles, K slices per tile, slices per filter tap (C / 32)
+    Magic d_pw, d_ph, d_tn;
+    int last_round;                     // workgroups from this number on finish together (see the K loop)
+};
+
+#if __HIP_DEVICE_COMPILE__
+// The K loop's LDS reads are written as assembly: the compiler cannot tell which ring stage a direct-to-LDS load
+// targets and would make every LDS read behind one wait for ALL outstanding loads; it also re-derives addresses
+// it could keep.  The ring's real ordering is the explicit s_waitcnt vmcnt + s_barrier (ring_sync); these reads are
+// ordered among themselves and against the MFMAs by lds_wait, which takes the fragments as operands.
+typedef float f4v __attribute__((ext_vector_type(4)));
+template <int OFF> __device__ __forceinline__ void lds_read128(f4v &dst, int addr) {   // addr + OFF: LDS byte address
+    static_assert(OFF >= 0 && OFF < 65536, "the instruction's offset field has 16 bits");
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+struct WinFrag {
+    f4v a, b;
+};
+// waits until at most PENDING LDS reads are outstanding; the fragments' registers are operands so that no use of
+// them moves above the wait
+template <int PENDING> __device__ __forceinline__ void lds_wait(WinFrag &f) {
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(f.a), "+v"(f.b) : "n"(PENDING));
+}
+// if_set where the lane's bit of `mask` is set, else if_clear (the mask stays in scalar registers)
+__device__ __forceinline__ int select_by_mask(unsigned long long mask, int if_set, int if_clear) {
+    int r;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(if_clear), "v"(if_set), "s"(mask));
+    return r;
+}
+#endif
+
+template <bool POOL, bool RES>
+__global__ __launch_bounds__(kThreads) void conv_win(const WinArgs a) {
+#if __HIP_DEVICE_COMPILE__
+    // A new wavefront is the youngest on its SIMD and the CU serves the oldest first: without a raised priority its
+    // first instructions wait behind the MFMAs of the workgroups that are in their K loops.
+    __builtin_amdgcn_s_setprio(3);
+    constexpr int BM = 64, BN = 64;
+    constexpr int kLoads = 4;                                // 1-KiB loads per wavefront per slice: two of A, two of B
+    constexpr int kBBytes = BN * 128, kABytes = BM * 128;   // a stage: the filter rows, then the gathered rows
+    constexpr int kStageBytes = kABytes + kBBytes;
+    extern __shared__ __align__(16) float lds[];
+    char *const lds_b = reinterpret_cast<char *>(lds);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, h = lane >> 5;
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const int nk = a.nk;
+    const int chunk16 = kc_chunk(lane, wave) * 16;   // byte position of this lane's 16 bytes inside a slice of a row
+    const int row_in_load = kc_row_in_load(lane);
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(reinterpret_cast<const char *>(a.in) - a.shift_bytes, a.in_bytes + a.shift_bytes);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(a.filt, a.filt_bytes);
+
+    int u0, u1, share = -1;
+    if ((int)blockIdx.x >= a.sk.sk_wgs) {
+        u0 = ((int)blockIdx.x - a.sk.sk_wgs) * nk;
+        u1 = u0 + nk;
+    } else {
+        share = blockIdx.x;
+        u0 = a.sk.dp_tiles * nk + share * a.sk.q + (share < a.sk.r ? share : a.sk.r);
+        u1 = u0 + a.sk.q + (share < a.sk.r ? 1 : 0);
+    }
+    for (int piece = 0; u0 < u1; ++piece) {
+        int pid, kt_begin, kt_end;
+        if (share < 0) {
+            pid = (int)blockIdx.x - a.sk.sk_wgs, kt_begin = 0, kt_end = nk;
+        } else {
+            pid = u0 / nk;
+            kt_begin = u0 - pid * nk;
+            kt_end = (u1 - u0 < nk - kt_begin) ? kt_begin + (u1 - u0) : nk;
+        }
+        const bool whole = kt_begin == 0 && kt_end == nk;
+        u0 += kt_end - kt_begin;
+        if (piece) {
+            __builtin_amdgcn_s_barrier();   // every wavefront is done reading the ring of the previous piece
+            __builtin_amdgcn_s_setprio(3);
+        }
+        pid = xcd_renumbered(pid, a.sk.dp_tiles);
+        const int tile_m = magic_div(pid, a.d_tn), tile_n = pid - tile_m * a.tiles_n;
+        const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+        // The filter rows' loads of the first two slices go out before anything else is computed (load j of a
+        // wavefront fills the 1-KiB block 4j + wave of its operand's part of a stage).
+        int vb[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int n = n0 + (4 * j + wave) * 8 + row_in_load;
+            vb[j] = n < a.N ? n * a.K * 4 + chunk16 : kOutOfRange;
+        }
+        int soff_b = kt_begin * BK * 4;
+        auto request_b = [&](int stage, int soff) {
+            char *const wr = lds_b + stage * kStageBytes;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_t *)(wr + (4 * j + wave) * 1024), 16, vb[j], soff, 0, 0);
+        };
+        const bool two = kt_begin + 1 < kt_end;
+        request_b(0, soff_b);
+        if (two) request_b(1, soff_b + BK * 4);
+        // the epilogue's per-column parameters (a whole tile's): requested here — older loads complete first, so the
+        // count below of the loads that may still be pending is unaffected — and turned into bias / slope / offset
+        // once the first slice has landed
+        const int col = n0 + wave_n * 32 + l32;
+        ColumnRaw raw;
+        ColumnParams cp;
+        if (whole) raw = column_raw(a.ep, col, col < a.N);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // per A load: the lane's row is row (4j + wave) * 8 + lane / 8 of the tile = pixel d of window w
+        int row_off[2], iy0[2], ix0[2], va[2];
+        const int d = row_in_load & 3;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int w = (m0 >> 2) + 8 * j + 2 * wave + (row_in_load >> 2);
+            const int t = magic_div(w, a.d_pw), px = w - t * a.pw;
+            const int img = magic_div(t, a.d_ph), py = t - img * a.ph;
+            const int y = (2 * py + (d >> 1)) * a.sh - a.pt;
+            ix0[j] = (2 * px + (d & 1)) * a.sw - a.pl;
+            iy0[j] = w < a.nwin ? y : -(1 << 20);   // rows past M: no filter row brings them inside the image
+            row_off[j] = ((img * a.H + y) * a.W + ix0[j]) * a.C * 4 + chunk16 + a.shift_bytes;
+        }
+        // the loads' position: slice lk = slice cs of tap (ky, kx)
+        int lk = kt_begin, ky = 0, kx = 0, cs = 0;
+        if (kt_begin) {
+            const int tap = kt_begin / a.cpt;
+            cs = kt_begin - tap * a.cpt;
+            ky = tap / a.kw;
+            kx = tap - ky * a.kw;
+        }
+        unsigned long long y_ok[2];
+        auto refilter_row = [&]() {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) y_ok[j] = __builtin_amdgcn_ballot_w64((unsigned)(iy0[j] + ky) < (unsigned)a.H);
+        };
+        auto retap = [&]() {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const unsigned long long ok = y_ok[j] & __builtin_amdgcn_ballot_w64((unsigned)(ix0[j] + kx) < (unsigned)a.W);
+                va[j] = select_by_mask(ok, row_off[j], kOutOfRange);
+            }
+        };
+        refilter_row();
+        retap();
+        int soff_a = ((ky * a.W + kx) * a.C + cs * BK) * 4;
+        // moves the loads' position on by a slice (the array va has ONE place that writes it: two would be merged
+        // into a store at a variable index, and the array would live in scratch memory)
+        auto advance = [&]() {
+            ++lk, ++cs;
+            soff_a += BK * 4, soff_b += BK * 4;
+            if (lk < kt_end && cs == a.cpt) {
+                cs = 0;
+                asm volatile("" : "+s"(cs));   // keeps this a (wavefront-uniform) branch: as selects it would run every slice
+                if (++kx == a.kw) {
+                    kx = 0, ++ky;
+                    refilter_row();
+                }
+                soff_a = (ky * a.W + kx) * a.C * 4;
+                retap();
+            }
+        };
+        auto request_a = [&](int stage) {
+            char *const wr = lds_b + stage * kStageBytes + kBBytes;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t *)(wr + (4 * j + wave) * 1024), 16, va[j], soff_a, 0, 0);
+        };
+        request_a(0);
+        advance();
+        if (two) request_a(1);
+        advance();
+        __builtin_amdgcn_sched_barrier(0);
+
+        // LDS byte addresses of this lane's fragments in stage 0, per group of 8 k (see load_frag_swz)
+        int a_addr[4], b_addr[4];
+        {
+            const int base = (int)(unsigned)(uintptr_t)(lds_void_t *)lds_b, swz = (l32 >> 1) & 7;
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                const int chunk = ((2 * gq + h) ^ swz) << 4;
+                a_addr[gq] = base + kBBytes + (wave_m * 32 + l32) * 128 + chunk;
+                b_addr[gq] = base + (wave_n * 32 + l32) * 128 + chunk;
+                asm volatile("" : "+v"(a_addr[gq]), "+v"(b_addr[gq]));   // eight registers, kept: not re-derived from shared parts at every use
+            }
+        }
+
+        v16f acc[1][1];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[0][0][v] = 0.f;
+        WinFrag frag[2];
+        auto read_frags = [&](WinFrag &f, auto stage_c, auto gq_c) {
+            constexpr int kStage = decltype(stage_c)::value * kStageBytes, GQ = decltype(gq_c)::value;
+            lds_read128<kStage>(f.a, a_addr[GQ]);
+            lds_read128<kStage>(f.b, b_addr[GQ]);
+        };
+        using G0 = std::integral_constant<int, 0>;
+        using G1 = std::integral_constant<int, 1>;
+        using G2 = std::integral_constant<int, 2>;
+        using G3 = std::integral_constant<int, 3>;
+        // the MFMAs of group GQ of a slice out of frag[GQ & 1], behind the reads of the next group's fragments
+        auto group = [&](auto gq_c, auto rd_c, auto nx_c) {
+            constexpr int GQ = decltype(gq_c)::value;
+            if constexpr (GQ == 0) read_frags(frag[1], rd_c, G1{});
+            else if constexpr (GQ == 1) read_frags(frag[0], rd_c, G2{});
+            else if constexpr (GQ == 2) read_frags(frag[1], rd_c, G3{});
+            else read_frags(frag[0], nx_c, G0{});
+            WinFrag &f = frag[GQ & 1];
+            lds_wait<2>(f);   // the fragments read a group ago are here
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s4 = 0; s4 < 4; ++s4) mfma_acc(acc[0][0], f.a[s4], f.b[s4]);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        // A CU serves its wavefronts by priority, then oldest first: left alone, the workgroups of a CU finish one
+        // after the other and the last runs by itself for a third of its K range — and a single workgroup cannot
+        // hide the loads' latency behind one slice.  Where all whole tiles are on the chip at once (a single round)
+        // they therefore lower their priority as they get on (3, 2, 1, 0 by quarters of the K range): whoever is
+        // behind is served first and they finish together (2 % on the 28 x 28 x 128 layers).  With several rounds the
+        // staggered ends are wanted — they hide the starts of the workgroups that follow (the same rule there: 68 ->
+        // 75 us on 56 x 56 x 64 -> 64) — and every K loop runs at the lowest priority.
+        const bool fair = (int)blockIdx.x >= a.last_round;
+        const int quarter = (kt_end - kt_begin + 3) >> 2;
+        int done = 0, next_drop = quarter;
+        // One slice out of stage RD.  Behind the barrier (every wavefront's part of the next slice has landed,
+        // nobody reads the slice before this one any more) the loads of the slice two on go into stage WR; the
+        // first fragments of the next slice come out of stage NX.
+        auto step = [&](auto rd_c, auto wr_c, auto nx_c) {
+            group(G0{}, rd_c, nx_c);
+            ring_sync<0>();
+            if (lk < kt_end) {   // (past the piece's end there is nothing to load)
+                request_a(decltype(wr_c)::value);
+                request_b(decltype(wr_c)::value, soff_b);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            group(G1{}, rd_c, nx_c);
+            group(G2{}, rd_c, nx_c);
+            group(G3{}, rd_c, nx_c);
+            advance();
+            if (fair && ++done == next_drop) {
+                next_drop += quarter;
+                if (done == quarter) __builtin_amdgcn_s_setprio(2);
+                else if (done == 2 * quarter) __builtin_amdgcn_s_setprio(1);
+                else __builtin_amdgcn_s_setprio(0);
+            }
+        };
+        using S0 = std::integral_constant<int, 0>;
+        using S1 = std::integral_constant<int, 1>;
+        using S2 = std::integral_constant<int, 2>;
+        if (two) ring_sync<2>();   // all but the second slice's gathered rows — the last two loads — have landed
+        else ring_sync<0>();
+        if (whole) cp = column_params(a.ep, raw);
+        if (!fair) __builtin_amdgcn_s_setprio(0);
+        read_frags(frag[0], S0{}, G0{});
+        int kt = kt_begin;
+        for (; kt + 3 <= kt_end; kt += 3) {
+            step(S0{}, S2{}, S1{});
+            step(S1{}, S0{}, S2{});
+            step(S2{}, S1{}, S0{});
+        }
+        if (kt < kt_end) step(S0{}, S2{}, S1{});
+        if (kt + 1 < kt_end) step(S1{}, S0{}, S2{});
+
+        __builtin_amdgcn_s_setprio(3);
+        lds_wait<0>(frag[0]);   // the fragments read ahead for a slice that does not follow
+        acc_settle(acc);
+        if (whole) {
+            // Lane (l32, h) holds column `col` of the windows wbase + 2 q, four pixels each (accumulator registers
+            // 4q .. 4q + 3).  One 32-bit offset per window; the window's other pixels (and those of the second
+            // summand) at scalar offsets from it.
+            const __amdgpu_buffer_rsrc_t rsrc_out = make_rsrc(a.out, a.out_bytes);
+            const int N = a.N, s_px = N * 4, s_row = a.OW * N * 4;
+            const int wbase = (m0 >> 2) + wave_m * 8 + h;
+            const bool bn = a.ep.bn_mean != nullptr;
+            int voff[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int w = wbase + 2 * q;
+                const int at = POOL ? (w * N + col) * 4 : ((w + magic_div(w, a.d_pw) * a.pw) * 2 * N + col) * 4;
+                voff[q] = (w < a.nwin && col < N) ? at : kOutOfRange;
+            }
+            float add[4][4];
+            if constexpr (RES) {
+                const __amdgpu_buffer_rsrc_t rsrc_res = make_rsrc(a.ep.residual, (unsigned)a.nwin * 16u * (unsigned)N);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    add[q][0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_res, voff[q], 0, 0));
+                    add[q][1] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_res, voff[q], s_px, 0));
+                    add[q][2] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_res, voff[q], s_row, 0));
+                    add[q][3] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_res, voff[q], s_row + s_px, 0));
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float x[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    x[e] = acc[0][0][4 * q + e] + cp.bias;
+                    if (bn) x[e] = fmaf(x[e] - cp.mean, cp.slope, cp.beta);
+                    if constexpr (RES) x[e] += add[q][e];
+                    if (a.ep.relu) x[e] = (x[e] > 0.f) ? x[e] : 0.f;
+                }
+                if constexpr (POOL) {
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, window_max(x[0], x[1], x[2], x[3])), rsrc_out, voff[q], 0, 0);
+                } else {
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[0]), rsrc_out, voff[q], 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[1]), rsrc_out, voff[q], s_px, 0);
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[2]), rsrc_out, voff[q], s_row, 0);
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[3]), rsrc_out, voff[q], s_row + s_px, 0);
+                }
+            }
+        } else {
+            float *slot = a.part + (size_t)(2 * share + (piece ? 1 : 0)) * (BM * BN);
+            store_tile_impl<1, 1, false, false>(acc, slot, (size_t)BN, BM, BN, wave_m * 32, wave_n * 32, lane, Epilogue{});
+        }
+    }
+#endif
+}
+
 // Adds the pieces of every shared tile that more than one workgroup worked on (see conv_dma) in K order and
 // applies the epilogue.  blockIdx.x = shared tile, blockIdx.y = block of 16 rows of it.  With `pool` (rows in window
 // order) the finished values of a window's four rows meet in LDS and their maximum is stored.
@@ -965,25 +1326,34 @@ int share_all_min_slices() {
     return n > 0 ? n : n < 0 ? 1 << 30 : kShareAllMinSlices;
 }
 
-constexpr int kPieceMinSlices = 4;
+// A compute unit serves its resident workgroups oldest first at the rate of its matrix cores: what has to be even
+// is the work per CU.  With at least as many tiles as CUs, every CU gets the same number of whole tiles (the
+// dispatcher refills slots as they free up) and the tiles beyond a multiple of the CU count are cut into one piece
+// per CU, started first (the first workgroups of a launch land on distinct CUs): with pieces of four slices or more on
+// only some CUs those CUs finished 4-5 us after the others (traced per workgroup: 65.5 against 61 us on 28x28x128->128).
+constexpr int kPieceMinSlices = 2;   // a piece costs a ring start and a tile store
 SkPlan sk_plan(long tiles, int nk, int slots, bool allow_shared) {
     SkPlan p{(int)tiles, 0, 0, 0};
     if (!allow_shared || tiles == 0) return p;
-    long rest = tiles % slots;
-    if (tiles < slots) {
-        // (a nearly full round: leave it; a twelfth of a round or less — single images — is cut from K = 512 on)
+    const int piece_min = switches().conv_piece_min > 0 ? switches().conv_piece_min : kPieceMinSlices;
+    const long cus = num_cus() < slots ? num_cus() : slots;   // (tests pretend a smaller chip through `slots`)
+    long rest, wgs;
+    if (tiles < cus) {
+        // fewer tiles than CUs: all are cut if K is long (a nearly full round: leave it; a twelfth of a round or
+        // less — single images — is cut from K = 512 on), into as many pieces as the chip holds workgroups
         const int min_slices = share_all_min_slices();
         const bool long_k = nk >= min_slices || (min_slices == kShareAllMinSlices && 12 * tiles <= slots && nk >= 16);
-        if (!long_k || 4 * tiles > 3 * slots) return p;
+        if (!long_k) return p;
         rest = tiles;
-    } else if (rest == 0 || 2 * rest > slots) {
-        return p;
+        wgs = slots;
+        if (rest * nk < 4 * wgs) wgs = rest * nk / 4;
+    } else {
+        rest = tiles % cus;
+        if (rest == 0 || nk < 8) return p;
+        wgs = cus;
+        if (rest * nk < piece_min * wgs) wgs = rest * nk / piece_min;
     }
     const long units = rest * nk;
-    long wgs = slots;
-    // at least kPieceMinSlices slices per share: a piece costs a ring start and a tile store
-    const int piece_min = switches().conv_piece_min > 0 ? switches().conv_piece_min : kPieceMinSlices;
-    if (units < piece_min * wgs) wgs = units / piece_min;
     if (wgs <= rest) return p;              // shares of a tile or more each: nothing to gain
     p.dp_tiles = (int)(tiles - rest);
     p.sk_wgs = (int)wgs;
@@ -1056,6 +1426,71 @@ int launch_conv_dma(const float *in, const float *filt, float *out, const ConvGe
     if (p.sk_wgs) {
         conv_sk_finish<T::BM, T::BN><<<dim3((unsigned)(tiles - p.dp_tiles), T::BM / 16), 256, 0, stream()>>>(
             out, scratch, g, nk, p, ep, (g.OC % 4 == 0 && aligned16(out)) ? 1 : 0, pool ? 1 : 0);
+        SWC_LAUNCH_CHECK();
+    }
+    return SWC_HIP_OK;
+}
+
+// ------------------------------------------------------------ conv_win: host side
+constexpr size_t kWinLdsBytes = 3 * (64 + 64) * 128;
+
+int conv_win_slots() {
+    if (switches().conv_slots > 0) return switches().conv_slots;   // tests: pretend the chip holds this many workgroups
+    static int per_cu = 0;
+    if (!per_cu) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_win<false, false>, kThreads, kWinLdsBytes) != hipSuccess || n < 1) {
+            (void)hipGetLastError();
+            n = 1;
+        }
+        per_cu = n;
+    }
+    return per_cu * num_cus();
+}
+
+SkPlan conv_win_plan(const ConvGeom &g, bool allow_shared) {
+    const long tiles = (long)((g.M + 63) / 64) * ((g.OC + 63) / 64);
+    return sk_plan(tiles, g.K / BK, conv_win_slots(), allow_shared);
+}
+
+size_t conv_win_scratch_bytes(const ConvGeom &g) { return (size_t)2 * conv_win_plan(g, true).sk_wgs * 64 * 64 * sizeof(float); }
+
+// Whether a layer runs on conv_win.  SWC_HIP_CONV=win forces it where it applies (test-only); any other forced variant,
+// or SWC_HIP_CONV_LEAN=0, rules the kernel out.  `g.win` must have been set.
+bool takes_win(const ConvGeom &g, const void *input, const void *filter) {
+    const char *force = switches().conv;
+    if ((force && strcmp(force, "win")) || !switches().conv_lean) return false;
+    if (!g.win || g.C % BK != 0 || g.M % 4 != 0 || (g.OW >> 1) < 1) return false;
+    const size_t in_bytes = (size_t)g.N * g.H * g.W * g.C * 4, filt_bytes = (size_t)g.OC * g.K * 4;
+    const size_t out_bytes = (size_t)g.M * g.OC * 4, shift = ((size_t)g.pt * g.W + g.pl) * g.C * 4;
+    return aligned16(input) && aligned16(filter) && in_bytes + shift < kMaxDmaBytes && filt_bytes < kMaxDmaBytes &&
+           out_bytes < kMaxDmaBytes;
+}
+
+int launch_conv_win(const float *in, const float *filt, float *out, const ConvGeom &g, const Epilogue &ep, float *scratch, bool pool) {
+    constexpr int BM = 64, BN = 64;
+    const long tiles = (long)((g.M + BM - 1) / BM) * ((g.OC + BN - 1) / BN);
+    const SkPlan p = conv_win_plan(g, scratch != nullptr);
+    WinArgs a{};
+    a.in = in, a.filt = filt, a.out = out, a.part = scratch, a.ep = ep, a.sk = p;
+    a.in_bytes = (unsigned)((size_t)g.N * g.H * g.W * g.C * 4);
+    a.filt_bytes = (unsigned)((size_t)g.OC * g.K * 4);
+    a.out_bytes = (unsigned)((size_t)(pool ? g.M / 4 : g.M) * g.OC * 4);
+    a.shift_bytes = (g.pt * g.W + g.pl) * g.C * 4;
+    a.N = g.OC, a.K = g.K, a.C = g.C, a.H = g.H, a.W = g.W, a.kw = g.kw, a.sh = g.sh, a.sw = g.sw, a.pt = g.pt, a.pl = g.pl;
+    a.OW = g.OW, a.pw = g.OW >> 1, a.ph = g.OH >> 1, a.nwin = g.M >> 2;
+    a.tiles_n = (g.OC + BN - 1) / BN, a.nk = g.K / BK, a.cpt = g.C / BK;
+    a.d_pw = magic_of((unsigned)a.pw), a.d_ph = magic_of((unsigned)a.ph), a.d_tn = magic_of((unsigned)a.tiles_n);
+    a.last_round = switches().conv_fair && p.dp_tiles <= conv_win_slots() ? p.sk_wgs : 1 << 30;
+    note_kernel("conv_win%s%s", p.sk_wgs ? " + conv_sk_finish" : "", pool ? " (pooled)" : "");
+    const unsigned grid = (unsigned)(p.dp_tiles + p.sk_wgs);
+    if (pool) conv_win<true, false><<<grid, kThreads, kWinLdsBytes, stream()>>>(a);
+    else if (ep.residual) conv_win<false, true><<<grid, kThreads, kWinLdsBytes, stream()>>>(a);
+    else conv_win<false, false><<<grid, kThreads, kWinLdsBytes, stream()>>>(a);
+    SWC_LAUNCH_CHECK();
+    if (p.sk_wgs) {
+        conv_sk_finish<BM, BN><<<dim3((unsigned)(tiles - p.dp_tiles), BM / 16), 256, 0, stream()>>>(
+            out, scratch, g, a.nk, p, ep, (g.OC % 4 == 0 && aligned16(out)) ? 1 : 0, pool ? 1 : 0);
         SWC_LAUNCH_CHECK();
     }
     return SWC_HIP_OK;
@@ -1385,10 +1820,15 @@ __global__ __launch_bounds__(256) void mask_filter_groups(float *dst, const floa
     }
 }
 
+bool window_order(const ConvGeom &g);
+
 // Scratch bytes the forward convolution of this geometry uses (0: none).
 size_t conv_scratch_bytes(const ConvGeom &g, const void *input, const void *filter) {
     const char *force = switches().conv;
     if (!share_tiles() || !conv_uses_dma(g, input, filter, force)) return 0;
+    ConvGeom gw = g;
+    gw.win = window_order(g) ? 1 : 0;
+    if (takes_win(gw, input, filter)) return conv_win_scratch_bytes(gw);
     return with_dma_variant(pick_dma_variant(g, force, true), [&]<int TM, int TN, int STAGES, bool MID>() {
         return conv_dma_scratch_bytes<TM, TN, STAGES, MID>(g);
     });
@@ -1567,6 +2007,7 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
                 if (!pieces) return fail_code();
             }
         }
+        if (takes_win(g, input, filter)) return launch_conv_win(input, filter, output, g, ep, pieces, pooled);
         return with_dma_variant(pick_dma_variant(g, force, shared), [&]<int TM, int TN, int STAGES, bool MID>() {
             return launch_conv_dma<TM, TN, STAGES, MID>(input, filter, output, g, in_bytes, filt_bytes, ep, pieces, pooled);
         });

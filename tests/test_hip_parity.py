@@ -256,26 +256,35 @@ def test_conv_random_shapes_integer_exact(rt, oracle, idims, fdims, strides, pad
         assert_bit_exact(got, oracle.maxpool(oracle.relu(want), *pool), f"conv + ReLU + pool on integers [{rt.last_kernel()}]")
 
 
-def _random_wide_lean_cases(count, seed):
+def _random_window_order_cases(count, seed):
+    """layers for conv_win: channel counts that are multiples of 32, outputs with whole 2x2 windows of every size
+    (one window per row up to wide images), any stride, kernel and padding, ragged tiles in both directions"""
     rng = np.random.default_rng(seed)
     cases = []
     while len(cases) < count:
-        c, oc = int(rng.choice([32, 64])), int(rng.choice([8, 64, 72, 128]))
-        k, s = int(rng.choice([1, 3])), int(rng.choice([1, 1, 2]))
-        n, h, w = int(rng.integers(1, 4)), int(rng.integers(8, 40)), int(rng.integers(16, 70))
-        oh, ow = (h + 2 * (k // 2) - k) // s + 1, (w + 2 * (k // 2) - k) // s + 1
-        if oh % 2 or ow % 2 or ow < 16:
+        c, oc = int(rng.choice([32, 64, 96])), int(rng.choice([8, 64, 70, 128, 136]))
+        kh, kw = int(rng.choice([1, 3, 5])), int(rng.choice([1, 3, 3]))
+        sh, sw = int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2, 3]))
+        pads = tuple(int(v) for v in rng.integers(0, 3, 4))
+        small = len(cases) % 2 == 0
+        n = int(rng.integers(1, 6))
+        h, w = (int(rng.integers(2, 14)), int(rng.integers(2, 14))) if small else (int(rng.integers(8, 40)), int(rng.integers(16, 70)))
+        if h + pads[0] + pads[2] < kh or w + pads[1] + pads[3] < kw:
             continue
-        cases.append(((n, h, w, c), (oc, k, k, c), (s, s), (k // 2,) * 4, [None, "7", "20"][len(cases) % 3]))
+        oh, ow = (h + pads[0] + pads[2] - kh) // sh + 1, (w + pads[1] + pads[3] - kw) // sw + 1
+        if oh % 2 or ow % 2 or oh < 2 or ow < 2:
+            continue
+        cases.append(((n, h, w, c), (oc, kh, kw, c), (sh, sw), pads, [None, "7", "20"][len(cases) % 3]))
     return cases
 
 
-@pytest.mark.parametrize("idims,fdims,strides,pads,slots", _random_wide_lean_cases(18, 31))
-def test_conv_lean_wide_images_integer_exact(rt, oracle, idims, fdims, strides, pads, slots, switch_env):
-    """conv_dma_lean on images of at least eight 2x2 windows per output row, where the pixel of a row follows from the
-    tile's first window by carries (ragged last tiles, strides, tiles cut along K): integer operands, the oracle's bits,
-    plain and with the pooled epilogue."""
-    print("case wide lean conv", idims, fdims, strides, pads, slots, flush=True)
+@pytest.mark.parametrize("idims,fdims,strides,pads,slots", _random_window_order_cases(36, 31))
+def test_conv_win_integer_exact(rt, oracle, idims, fdims, strides, pads, slots, switch_env):
+    """conv_win (rows in 2x2 window order, channel counts that are multiples of 32) over random layer shapes — from one
+    window per output row to wide images, ragged last tiles, strides, uneven padding, tiles cut along K on a chip
+    pretended to hold 7 or 20 workgroups: integer operands, the oracle's bits, plain, with a second summand and ReLU,
+    and with the pooled epilogue."""
+    print("case conv_win", idims, fdims, strides, pads, slots, flush=True)
     if slots:
         switch_env.setenv("SWC_HIP_CONV_SLOTS", slots)
     rng = np.random.default_rng(sum(idims) * 13 + sum(fdims))
@@ -285,10 +294,15 @@ def test_conv_lean_wide_images_integer_exact(rt, oracle, idims, fdims, strides, 
     dx, df, db = up(rt, x, f, b)
     want = oracle.conv2d(x, f, b, fdims[1:3], strides, pads)
     got = rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy()
-    assert rt.last_kernel().startswith("conv_dma_lean"), rt.last_kernel()
+    assert rt.last_kernel().startswith("conv_win"), rt.last_kernel()
     assert_bit_exact(got, want, f"conv on integers [{rt.last_kernel()}]")
+    res = rng.integers(-3, 4, want.shape).astype(np.float32)
+    got = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True, residual=rt.upload(res)).numpy()
+    assert rt.last_kernel().startswith("conv_win"), rt.last_kernel()
+    assert_bit_exact(got, oracle.relu(want + res), f"conv + summand + ReLU on integers [{rt.last_kernel()}]")
     pool = ((2, 2), (2, 2))
     got = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True, pool=pool).numpy()
+    assert rt.last_kernel().startswith("conv_win") and rt.last_kernel().endswith("(pooled)"), rt.last_kernel()
     assert_bit_exact(got, oracle.maxpool(oracle.relu(want), *pool), f"conv + ReLU + pool on integers [{rt.last_kernel()}]")
 
 
@@ -660,9 +674,9 @@ def test_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, pads, s
     for with_bn, relu in [(True, True), (False, True), (False, False), (True, False)]:
         kw = dict(pads=pads, bn=dbn if with_bn else None, eps=1e-5, relu=relu)
         fused = rt.conv2d(dx, df, db, pool=pool, **kw)
-        assert rt.last_kernel().startswith("conv_dma") and rt.last_kernel().endswith("(pooled)"), rt.last_kernel()
+        assert rt.last_kernel().startswith(("conv_dma", "conv_win")) and rt.last_kernel().endswith("(pooled)"), rt.last_kernel()
         plain = rt.conv2d(dx, df, db, **kw)
-        assert rt.last_kernel().startswith("conv_dma"), rt.last_kernel()
+        assert rt.last_kernel().startswith(("conv_dma", "conv_win")), rt.last_kernel()
         want = rt.maxpool(plain, *pool).numpy()
         assert_bit_exact(fused.numpy(), want, f"pooled in the epilogue vs conv then maxpool (bn {with_bn}, relu {relu})")
     # against the oracle (full-size layers: the first image only)
@@ -690,10 +704,10 @@ def test_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, pads, s
                                               ((4, 16, 16, 64), (64, 1, 1, 64), (0, 0, 0, 0))])
 @pytest.mark.parametrize("slots", [None, "11"])
 def test_conv_kernel_forms_agree_bit_for_bit(rt, idims, fdims, pads, slots, switch_env):
-    """The two forms of the 64x64-tile kernel — conv_dma and conv_dma_lean (channel counts that are multiples of 32:
-    no vector-ALU work in the K loop) — walk K in the same order and cut the same tiles: the same bits, whole and
-    cut tiles, plain and pooled.  (Eleven slots: every layer here then stays on the 64x64 tiles, and the two
-    full-size ones have tiles cut along K.)"""
+    """The three forms of the 64x64-tile kernel — conv_dma (any channel count that is a multiple of 4), conv_dma_lean
+    (multiples of 32: gather offsets per filter tap) and conv_win (rows in window order, no vector-ALU work in the K
+    loop) — walk K in the same order and cut the same tiles: the same bits, whole and cut tiles, plain and pooled.
+    (Eleven slots: every layer here then stays on the 64x64 tiles, and the two full-size ones have tiles cut along K.)"""
     print("case conv kernel forms", idims, fdims, pads, slots, flush=True)
     if slots:
         switch_env.setenv("SWC_HIP_CONV_SLOTS", slots)
@@ -706,22 +720,31 @@ def test_conv_kernel_forms_agree_bit_for_bit(rt, idims, fdims, pads, slots, swit
             rng.uniform(0.5, 1.5, oc).astype(np.float32), rng.uniform(-0.1, 0.1, oc).astype(np.float32))
     dx, df, db = up(rt, x, f, b)
     kw = dict(pads=pads, bn=bn, eps=1e-5, relu=True)
-    lean = rt.conv2d(dx, df, db, **kw).numpy()
-    assert rt.last_kernel().startswith("conv_dma_lean"), rt.last_kernel()
+    windows = idims[1] % 2 == 0 and idims[2] % 2 == 0 and fdims[1] != 5   # (the 5x5 layer's output is 9 x 11: raster order)
+    default = rt.conv2d(dx, df, db, **kw).numpy()
+    assert rt.last_kernel().startswith("conv_win" if windows else "conv_dma_lean"), rt.last_kernel()
     if slots and idims[0] >= 32:
         assert "conv_sk_finish" in rt.last_kernel(), rt.last_kernel()
+    switch_env.setenv("SWC_HIP_CONV", "11_3m")
+    lean = rt.conv2d(dx, df, db, **kw).numpy()
+    assert rt.last_kernel().startswith("conv_dma_lean"), rt.last_kernel()
+    assert_bit_exact(default, lean, "default vs conv_dma_lean")
     switch_env.setenv("SWC_HIP_CONV_LEAN", "0")
     plain = rt.conv2d(dx, df, db, **kw).numpy()
     assert rt.last_kernel().startswith("conv_dma<1,1,3,true>"), rt.last_kernel()
     assert_bit_exact(lean, plain, "conv_dma_lean vs conv_dma")
-    if idims[1] % 2 == 0 and idims[2] % 2 == 0 and fdims[1] != 5:
+    if windows:
         pool = ((2, 2), (2, 2))
         plain_pooled = rt.conv2d(dx, df, db, pool=pool, **kw).numpy()
         switch_env.delenv("SWC_HIP_CONV_LEAN")
         lean_pooled = rt.conv2d(dx, df, db, pool=pool, **kw).numpy()
         assert rt.last_kernel().startswith("conv_dma_lean") and rt.last_kernel().endswith("(pooled)"), rt.last_kernel()
-        assert_bit_exact(lean_pooled, rt.maxpool(rt.upload(plain), *pool).numpy(), "pooled, lean")
-        assert_bit_exact(plain_pooled, lean_pooled, "pooled, general form")
+        switch_env.delenv("SWC_HIP_CONV")
+        win_pooled = rt.conv2d(dx, df, db, pool=pool, **kw).numpy()
+        assert rt.last_kernel().startswith("conv_win") and rt.last_kernel().endswith("(pooled)"), rt.last_kernel()
+        assert_bit_exact(win_pooled, rt.maxpool(rt.upload(plain), *pool).numpy(), "pooled, conv_win")
+        assert_bit_exact(lean_pooled, win_pooled, "pooled, conv_dma_lean")
+        assert_bit_exact(plain_pooled, win_pooled, "pooled, general form")
 
 
 @pytest.mark.parametrize("idims,fdims,pads", [((256, 28, 28, 1), (20, 5, 5, 1), (0, 0, 0, 0)),      # LeNet's first layer
