@@ -14,7 +14,14 @@ Also in the line:
   roofline      the dominant kernel (the tiled fp32-MFMA GEMM gemm_dma2<2,4,4,2,false,8>: both of its
                 launches per step, 4096x784x4096 and 4096x4096x4096), timed
                 with HIP events on the library's stream inside the timed region
-  kernels       per-launch times of the headline graph
+  kernels       per-launch times of the headline graph.  Every kernel row carries two durations: `ms`, between
+                events around the single launch inside the eager step (which adds the 2-5 us a pair of events
+                costs), and `ms_loop`, the average over 20 back-to-back launches of that op between ONE pair of
+                events; `frac`, `tflops`, `gbs` come from `ms_loop`, `frac_in_step` from `ms`
+  parity        measured distance between what the timed graph computed on the GPU and what the reference's own
+                CPU kernels computed from the same buffers in the cpu_baseline leg (strict on significant outputs,
+                floored, max norm, bit-exact), with its bar; configs.cfgN.parity for the other configurations; the
+                run exits non-zero after printing if a bar is broken
   graph_replay  the same K steps replayed as one HIP graph per step (no per-kernel
                 events in the loop): what a launch-bound small graph gains; `shader_clock_ghz`: the clock the
                 chip ran at meanwhile (one-wavefront watcher of the bench-only library on a stream of its own;
@@ -52,6 +59,69 @@ import numpy as np  # noqa: E402
 PEAK_TFLOPS_FP32_MFMA = 157.3
 PEAK_HBM_GBS = 8000.0
 ROOFLINE_KERNEL = "gemm_dma2<2,4,4,2,false,8>"   # 256x256 tiles, eight wavefronts: what both large FCs dispatch to
+# the sources of that kernel: profiles/traffic.json records their hash when its counters are read, and a figure
+# measured on other sources is not reported
+ROOFLINE_SOURCES = ["swcompiler_amd/csrc/gemm.hip", "swcompiler_amd/csrc/mfma_dma2.hpp", "swcompiler_amd/csrc/mfma_dma.hpp",
+                    "swcompiler_amd/csrc/mfma_tile.hpp"]
+
+
+def sources_sha256():
+    import hashlib
+    h = hashlib.sha256()
+    for rel in ROOFLINE_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def traffic_from_counters(fetch_csv, write_csv):
+    """--traffic-from: reads the two rocprofv3 --pmc runs of `bench.py --headline-only --no-cpu --calibrate` (FETCH_SIZE,
+    then WRITE_SIZE; KiB per dispatch), scales each by what the same counter reads for the calibration pass (relu_f
+    over 2^26 floats: 256 MiB read, 256 MiB written) and writes profiles/traffic.json with the hash of the kernel's
+    sources."""
+    import csv
+    import datetime
+    import re
+
+    def short(name):   # "void (anonymous namespace)::gemm_dma2<2, 4, 4, 2, false, 8>(float const*, ...)" -> "gemm_dma2<2,4,4,2,false,8>"
+        name = re.sub(r"\(anonymous namespace\)::", "", name.replace("void ", ""))
+        depth, out = 0, ""
+        for ch in name:
+            if ch == "(" and depth == 0:
+                break
+            depth += ch == "<"
+            depth -= ch == ">"
+            out += ch
+        return out.replace(" ", "")
+
+    def per_kernel(path, counter):
+        vals = {}
+        for row in csv.DictReader(open(path)):
+            if row["Counter_Name"] == counter:
+                vals.setdefault((short(row["Kernel_Name"]), int(row["Grid_Size"])), []).append(float(row["Counter_Value"]))
+        return vals
+
+    fetch, write = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
+    cal = ("flat_vec4<OpRelu,true>", 1 << 24)   # 2^26 floats, four per thread
+    true_kib = float(1 << 18)
+    f_scale = true_kib / (sum(fetch[cal]) / len(fetch[cal]))
+    w_scale = true_kib / (sum(write[cal]) / len(write[cal]))
+    out = {"_comment": "HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (written by bench.py --traffic-from; "
+                       "the commands are in profiles/wide_mlp_gemm.txt); bench.py copies the figure of the dominant kernel "
+                       "into roofline.traffic while the kernel's sources still hash to sources_sha256"}
+    for kernel in (ROOFLINE_KERNEL, "gemm_skinny_stream<3,true>"):
+        f = [v for (k, _), vs in fetch.items() if k == kernel for v in vs]
+        w = [v for (k, _), vs in write.items() if k == kernel for v in vs]
+        if not f or not w:
+            continue
+        fk, wk = sum(f) / len(f), sum(w) / len(w)
+        out[kernel] = dict(fetch_kib_counter=fk, fetch_scale=f_scale, write_kib_counter=wk, write_scale=w_scale,
+                           bytes_per_launch=int((fk * f_scale + wk * w_scale) * 1024), dispatches=len(f),
+                           measured=dict(date=datetime.date.today().isoformat(), sources_sha256=sources_sha256(),
+                                         sources=ROOFLINE_SOURCES, command="see profiles/wide_mlp_gemm.txt"))
+    with open(os.path.join(ROOT, "profiles", "traffic.json"), "w") as fh:
+        json.dump(out, fh, indent=1)
+    print(json.dumps(out, indent=1))
 
 
 class Timed:
@@ -74,7 +144,7 @@ class Timed:
             self.rt.event_record(s0)
             out = fn(*a, **kw)
             self.rt.event_record(s0 + 1)
-            self.log.append((name, s0, s0 + 1, work_fn(out, *a, **kw)))
+            self.log.append((name, s0, s0 + 1, work_fn(out, *a, **kw), lambda: fn(*a, **kw)))
             return out
         return call
 
@@ -83,10 +153,25 @@ class Timed:
 
     def results(self):
         rows = []
-        for name, s0, s1, work in self.log:
+        for name, s0, s1, work, _ in self.log:
             ms = self.rt.event_elapsed_ms(s0, s1)
             rows.append(dict(op=name, ms=ms, **work))
         return rows
+
+    def loop_times(self, iters=20, warm=3):
+        """Average duration of one launch of every op of the last logged step, over `iters` back-to-back launches
+        of that op between ONE pair of events: the op's kernels and the gaps between its launches, without the
+        2-5 us that a pair of events around a single launch adds."""
+        out = []
+        for _, _, _, _, again in self.log:
+            for _ in range(warm):
+                again()
+            self.rt.event_record(0)
+            for _ in range(iters):
+                again()
+            self.rt.event_record(1)
+            out.append(self.rt.event_elapsed_ms(0, 1) / iters)
+        return out
 
 
 def _gemm_work(res, a, b, *r, **kw):
@@ -124,8 +209,13 @@ WORK = {
 
 
 def rate(row):
-    """adds achieved rate and roofline fraction to a kernel row"""
-    s = row["ms"] * 1e-3
+    """adds achieved rate and roofline fraction to a kernel row: from `ms_loop` (average launch duration over
+    back-to-back launches) where the row has one, else from `ms`; rows with both also get `frac_in_step`, the same
+    fraction from the events around the single launch inside the eager step"""
+    if "ms_loop" in row:
+        in_step = rate(dict((k, v) for k, v in row.items() if k != "ms_loop"))
+        row["frac_in_step"] = in_step["frac"]
+    s = row.get("ms_loop", row["ms"]) * 1e-3
     if "flop" in row and "bytes" in row:   # GEMM with N <= 16: both figures, judged against the HBM roofline
         row["tflops"] = row["flop"] / s / 1e12
         row["gbs"] = row["bytes"] / s / 1e9
@@ -142,16 +232,19 @@ def rate(row):
     return row
 
 
-def merge_rows(all_rows):
-    """average per-launch rows of repeated steps (same op order every step)"""
+def merge_rows(all_rows, loop_ms=None):
+    """average per-launch rows of repeated steps (same op order every step); loop_ms: per op, the average launch
+    duration over back-to-back launches (Timed.loop_times)"""
     n = len(all_rows)
     out = []
     for i, row in enumerate(all_rows[0]):
         r = dict(row)
         times = sorted(step[i]["ms"] for step in all_rows)
-        r["ms"] = sum(times) / n          # the average: what the rates below are computed from
+        r["ms"] = sum(times) / n          # events around the single launch inside the step, averaged over the steps
         r["ms_median"] = times[n // 2]
         r["ms_min"] = times[0]
+        if loop_ms is not None:
+            r["ms_loop"] = loop_ms[i]
         out.append(rate(r))
     return out
 
@@ -261,7 +354,10 @@ def run_config(rt, graphs, cfg, steps, warmup):
     for log in per_step:
         timed.log = log
         all_rows.append(timed.results())
-    rows = merge_rows(all_rows)
+    timed.log = per_step[-1]
+    rows = merge_rows(all_rows, timed.loop_times())
+    result = graphs.run(cfg, rt, dt, fused=True, ws=ws)   # what the timed steps computed, for the parity figures
+    result = {k: v.numpy() for k, v in result.items()} if isinstance(result, dict) else result.numpy()
     # the same step as one HIP graph: K replays, nothing else in the loop
     handle = rt.capture(lambda: graphs.run(cfg, rt, dt, fused=True, ws=ws))
     for _ in range(3):
@@ -277,7 +373,7 @@ def run_config(rt, graphs, cfg, steps, warmup):
     clock = rt.shader_clock_ghz(lambda: rt.graph_launch(handle), graph_wall * 1e3 / steps)
     rt.graph_destroy(handle)
     return dict(batch=batch, wall_s=wall, gpu_ms=gpu_ms, ms_per_step=wall * 1e3 / steps,
-                samples_per_s=batch * steps / wall, kernels=rows,
+                samples_per_s=batch * steps / wall, kernels=rows, result=result,
                 graph_replay=dict(ms_per_step=graph_wall * 1e3 / steps, samples_per_s=batch * steps / graph_wall,
                                   shader_clock_ghz=clock))
 
@@ -397,7 +493,7 @@ def cpu_baselines(graphs, rows=64):
         be, kind = binding.load_ref(), "reference"
     else:
         be, kind = binding.load_oracle(), "port"
-    out = {}
+    out, results = {}, {}
     for cfg, iters in ((1, 3), (2, 1), (3, 3), (4, 1), (5, 3)):
         t = graphs.make_inputs(cfg)
         batch = graphs.batch_of(cfg, t)
@@ -409,14 +505,61 @@ def cpu_baselines(graphs, rows=64):
         times = []
         for _ in range(iters):
             t0 = time.perf_counter()
-            graphs.run(cfg, be, t, fused=False)
+            results[f"cfg{cfg}"] = graphs.run(cfg, be, t, fused=False)
             times.append(time.perf_counter() - t0)
         dt = min(times)
         out[f"cfg{cfg}"] = dict(value=batch / dt, unit="samples/s", cores=1, kind=kind, seconds=dt,
                                 seconds_all=times,
                                 sample=sample + "; the whole graph as the reference emits it (one kernels.h call per "
                                        f"op node), one thread, g++ -std=c++11 -O2; {os.cpu_count()} host cpus visible")
-    return out
+    return out, results
+
+
+def distance(got, want):
+    """Measured distance between the device's and the reference's result of one graph output (the definitions of
+    tests/util.py and tests/test_parity_report.py): strict_on_significant = max |g-r|/|r| over the outputs with
+    |r| >= 1e-3 max|r|; floored = max |g-r| / max(|r|, 1e-3 max|r|) over all outputs; max_norm = max|g-r| / max|r|."""
+    g, r = np.asarray(got, np.float64).ravel(), np.asarray(want, np.float64).ravel()
+    top = float(np.max(np.abs(r)))
+    big = np.abs(r) >= 1e-3 * top
+    diff = np.abs(g - r)
+    same = bool(np.array_equal(np.ascontiguousarray(got, np.float32).view(np.uint32), np.ascontiguousarray(want, np.float32).view(np.uint32)))
+    return dict(strict_on_significant=float(np.max(diff[big] / np.abs(r[big]))),
+                floored=float(np.max(diff / np.maximum(np.abs(r), 1e-3 * top))),
+                max_norm=float(np.max(diff)) / top, bit_exact=same, outputs=int(r.size))
+
+
+def parity_report(device, reference, cpu_rows):
+    """Per configuration: the distances between what the timed (fused) graphs computed on the GPU and what the
+    reference's own kernels computed from the same buffers in the cpu_baseline leg, with the bar each is held to.
+    Softmax outputs (cfg1-3, cfg5a) and BN+ReLU+max-pool (cfg5c): 1e-4 strict on the significant outputs and floored;
+    add+ReLU (cfg5b): bit-exact; the conv block (cfg4: four chained contractions of K = 576-1152 on N(0,1) data, each
+    followed by BN and ReLU): 1e-4 in the max norm — the per-layer bars are held by the tests."""
+    report, failed = {}, []
+    for name in sorted(reference):
+        got, want = device[name], reference[name]
+        if name == "cfg2":
+            got = got[:cpu_rows]
+        if isinstance(want, dict):
+            rows = {k: distance(got[k], want[k]) for k in sorted(want)}
+            rows["a"]["bar"], rows["b"]["bar"], rows["c"]["bar"] = "strict, floored < 1e-4", "bit-exact", "strict, floored < 1e-4"
+            ok = (rows["a"]["strict_on_significant"] < 1e-4 and rows["a"]["floored"] < 1e-4 and rows["b"]["bit_exact"] and
+                  rows["c"]["strict_on_significant"] < 1e-4 and rows["c"]["floored"] < 1e-4)
+            entry = dict(outputs=rows, ok=ok)
+        elif name == "cfg4":
+            entry = distance(got, want)
+            entry["bar"] = "max_norm < 1e-4"
+            entry["ok"] = entry["max_norm"] < 1e-4
+        else:
+            entry = distance(got, want)
+            entry["bar"] = "strict_on_significant, floored < 1e-4"
+            entry["ok"] = entry["strict_on_significant"] < 1e-4 and entry["floored"] < 1e-4
+        if name == "cfg2":
+            entry["rows"] = f"the first {cpu_rows} of the batch's 4096 rows"
+        if not entry["ok"]:
+            failed.append(name)
+        report[name] = entry
+    return report, failed
 
 
 def bench_workspace(rt, graphs):
@@ -454,11 +597,16 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch relu_f on 2^26 floats three times: a plain 256 MiB-in/256 MiB-out pass whose "
                          "FETCH_SIZE/WRITE_SIZE readings calibrate the counters for the traffic figures")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="instead of the benchmark: write profiles/traffic.json from two rocprofv3 --pmc counter files")
     ap.add_argument("--clocks", action="store_true",
                     help="instead of the benchmark: print the shader clock held under single kernels, by operand distribution")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (nothing is sharded); use --gpus 1")
+    if args.traffic_from:
+        traffic_from_counters(*args.traffic_from)
+        return
 
     from swcompiler_amd import graphs
     from swcompiler_amd.hip import SwcHip
@@ -480,6 +628,7 @@ def main():
         y.free()
 
     head = run_config(rt, graphs, 2, args.steps, args.warmup)
+    device_results = {"cfg2": head.pop("result")}
     gemm = [r for r in head["kernels"] if r["op"] == "fcbias" and not r["shape"].endswith("x10")]
     flop = sum(r["flop"] for r in gemm)
     secs = sum(r["ms"] for r in gemm) * 1e-3
@@ -497,8 +646,11 @@ def main():
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):   # measured separately under rocprofv3 --pmc (a counter run cannot share the timed run)
         entry = json.load(open(tpath)).get(ROOFLINE_KERNEL, {})
-        traffic = entry.get("bytes_per_launch")
         traffic_source = dict(file="profiles/traffic.json", **entry.get("measured", {}))
+        if traffic_source.get("sources_sha256") == sources_sha256():
+            traffic = entry.get("bytes_per_launch")
+        else:   # the kernel's sources changed since its counters were read: no figure rather than a stale one
+            traffic_source["stale"] = "the kernel's sources no longer hash to sources_sha256: re-measure (bench.py --traffic-from)"
     out = {
         "metric": "samples/s per graph; TFLOP/s (FC/conv) & GB/s (eltwise) vs MI355X roofline",
         "value": head["samples_per_s"], "unit": "samples/s", "n_gpus": 1, "steps": args.steps,
@@ -526,22 +678,34 @@ def main():
         for cfg in (1, 3, 4, 5):
             steps = max(5, min(args.steps, 20))
             r = run_config(rt, graphs, cfg, steps, max(2, min(args.warmup, 5)))
+            device_results[f"cfg{cfg}"] = r.pop("result")
             others[f"cfg{cfg}"] = dict(batch=r["batch"], samples_per_s=r["samples_per_s"], ms_per_step=r["ms_per_step"],
                                        gpu_ms_per_step=r["gpu_ms"] / steps, graph_replay=r["graph_replay"],
                                        kernels=r["kernels"])
         others["cfg5"]["kernels_unfused"] = run_bn_pool_separately(rt, graphs)
         others["training_kernels"] = dict(kernels=run_training(rt))
         out["configs"] = others
+    failed = []
     if not args.no_cpu:
-        cpu = cpu_baselines(graphs, args.cpu_rows)
+        cpu, reference = cpu_baselines(graphs, args.cpu_rows)
+        if args.headline_only:
+            reference = {"cfg2": reference["cfg2"]}
+        report, failed = parity_report(device_results, reference, args.cpu_rows)
+        out["parity"] = report["cfg2"]
+        for name, entry in report.items():
+            if name != "cfg2" and "configs" in out:
+                out["configs"][name]["parity"] = entry
         out["cpu_baseline"] = cpu["cfg2"]
         for name, entry in cpu.items():
             if name != "cfg2" and "configs" in out:
                 out["configs"][name]["cpu_baseline"] = entry
-        out.setdefault("configs", {})["cfg2"] = dict(cpu_baseline=cpu["cfg2"], note="the headline workload: see the top level")
+        out.setdefault("configs", {})["cfg2"] = dict(cpu_baseline=cpu["cfg2"], parity=report["cfg2"],
+                                                     note="the headline workload: see the top level")
     rt.sync()
     rt.set_workspace(None)
     print(json.dumps(out))
+    if failed:
+        sys.exit(f"bench.py: the device results of {failed} are outside their parity bar (see `parity` in the line above)")
 
 
 if __name__ == "__main__":
