@@ -2043,19 +2043,25 @@ int conv_dispatch(const char *who, float *output, const float *input, const floa
 // a different order.
 
 // turned[ci][ky][kx][co] = filter[co][kh-1-ky][kw-1-kx][ci]; rows of OCP >= OC floats, the tail zero
-__global__ __launch_bounds__(256) void turn_filter(const float *__restrict__ filt, float *__restrict__ turned, int OC,
-                                                   int OCP, int kh, int kw, int C) {
-    const int total = OCP * kh * kw * C;
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
-        const int co = i % OCP;
-        int t = i / OCP;
-        const int kx = t % kw;
-        t /= kw;
-        const int ky = t % kh;
-        const int ci = t / kh;
-        turned[i] = co < OC ? filt[((co * kh + (kh - 1 - ky)) * kw + (kw - 1 - kx)) * C + ci] : 0.f;
+struct TurnJob {
+    const float *filt;
+    float *turned;
+    int OC, OCP, kh, kw, C;
+};
+// (block `block` of `blocks` workgroups of 256 threads)
+__device__ __forceinline__ void turn_filter_part(const TurnJob &j, int block, int blocks) {
+    const int total = j.OCP * j.kh * j.kw * j.C;
+    for (int i = block * 256 + threadIdx.x; i < total; i += blocks * 256) {
+        const int co = i % j.OCP;
+        int t = i / j.OCP;
+        const int kx = t % j.kw;
+        t /= j.kw;
+        const int ky = t % j.kh;
+        const int ci = t / j.kh;
+        j.turned[i] = co < j.OC ? j.filt[((co * j.kh + (j.kh - 1 - ky)) * j.kw + (j.kw - 1 - kx)) * j.C + ci] : 0.f;
     }
 }
+__global__ __launch_bounds__(256) void turn_filter(TurnJob j) { turn_filter_part(j, blockIdx.x, gridDim.x); }
 
 // any stride: one thread per input element gathers the taps that reach it
 __global__ __launch_bounds__(256) void dgrad_direct(float *__restrict__ ig, const float *__restrict__ og,
@@ -2143,6 +2149,12 @@ __global__ __launch_bounds__(256) void dgrad_few_channels(float *__restrict__ ig
 }
 
 // ---- filter gradient: B operand = im2col(input), gathered
+// (Tried and dropped: the pixel arithmetic on the scalar unit — a load instruction covers one or two pixels of the
+// [32 pixels][BN columns] tile, so coordinates, bounds tests and the pixel's offset are wavefront-uniform, and per lane
+// a load needs an add and a select instead of some twenty vector instructions.  Bit-identical, but the scalar chains
+// (a wavefront issues in order: its MFMAs wait behind them) and the spilled scalar registers cost more than the
+// vector instructions saved: 215.6 / 339.6 / 182.0 us against 174.6 / 299.8 / 166.2 us for conv2dGrad_f on the three
+// layer shapes of the ResNet-like block, alternating runs on one box.)
 struct Im2colB {
     const float *in;
     unsigned bytes;
@@ -2194,24 +2206,24 @@ struct Im2colB {
 #endif
 };
 
-template <int TM, int TN, int WM, int STAGES, bool MID, int NW>
+template <int TM, int TN, int WM, int STAGES, bool MID, int NW, class BSrc>
 __global__ __launch_bounds__(64 * NW) void conv_wgrad(const float *__restrict__ ogT, unsigned a_bytes, int lda,
-                                                       Im2colB bsrc, float *__restrict__ part, size_t split_stride,
+                                                       BSrc bsrc, float *__restrict__ part, size_t split_stride,
                                                        int OC, int Kf, int M, int slices_per_split) {
 #if __HIP_DEVICE_COMPILE__
     const int k_begin = blockIdx.y * slices_per_split * BK;
     const int k_stop = k_begin + slices_per_split * BK;
     const Epilogue ep{nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
-    dma2_tile_body<TM, TN, WM, STAGES, MID, NW>(ogT, a_bytes, lda, bsrc, part + blockIdx.y * split_stride, (size_t)Kf, OC,
-                                                Kf, k_begin, k_stop < M ? k_stop : M, ep);
+    dma2_tile_body<TM, TN, WM, STAGES, MID, NW, BSrc, true>(ogT, a_bytes, lda, bsrc, part + blockIdx.y * split_stride, (size_t)Kf,
+                                                            OC, Kf, k_begin, k_stop < M ? k_stop : M, ep);
 #endif
 }
 
-template <int TM, int TN, int WM, int STAGES, bool MID, int NW>
-int launch_wgrad(const float *ogT, size_t a_bytes, int lda, const Im2colB &bsrc, float *part, int OC, int Kf, int M,
-                 int splits, int sps) {
+template <int TM, int TN, int WM, int STAGES, bool MID, int NW, class BSrc>
+int launch_wgrad_as(const float *ogT, size_t a_bytes, int lda, const BSrc &bsrc, float *part, int OC, int Kf, int M, int splits,
+                    int sps) {
     using T = Dma2Tile<TM, TN, WM, STAGES, NW>;
-    auto kern = conv_wgrad<TM, TN, WM, STAGES, MID, NW>;
+    auto kern = conv_wgrad<TM, TN, WM, STAGES, MID, NW, BSrc>;
     static bool attr_set = false;
     if (!attr_set) {
         SWC_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -2225,15 +2237,29 @@ int launch_wgrad(const float *ogT, size_t a_bytes, int lda, const Im2colB &bsrc,
     return SWC_HIP_OK;
 }
 
+template <int TM, int TN, int WM, int STAGES, bool MID, int NW>
+int launch_wgrad(const float *ogT, size_t a_bytes, int lda, const Im2colB &b, float *part, int OC, int Kf, int M, int splits, int sps) {
+    note_kernel("conv_wgrad<%d,%d,%d,%d,%s,%d>", TM, TN, WM, STAGES, MID ? "true" : "false", NW);
+    return launch_wgrad_as<TM, TN, WM, STAGES, MID, NW>(ogT, a_bytes, lda, b, part, OC, Kf, M, splits, sps);
+}
+
 // out[i] = sum over splits of part[split][i], in a fixed order: PH threads share an element, thread p adds
 // splits p, p+PH, p+2PH, ... four loads at a time (PH independent chains instead of one long one), then the PH
 // partial sums are added in order.  PH = 8 for a few splits of many elements, 32 for hundreds of splits.
+struct SumJob {
+    float *out;
+    const float *part;
+    size_t n;
+    int splits;
+};
 template <int PH>
-__global__ __launch_bounds__(32 * PH) void sum_splits(float *__restrict__ out, const float *__restrict__ part, size_t n,
-                                                      int splits) {
+__device__ __forceinline__ void sum_splits_part(const SumJob &j, unsigned block, unsigned blocks) {
     __shared__ float red[PH][33];
     const int e = threadIdx.x & 31, p = threadIdx.x >> 5;
-    for (size_t base = (size_t)blockIdx.x * 32; base < n; base += (size_t)gridDim.x * 32) {
+    const float *__restrict__ part = j.part;
+    const size_t n = j.n;
+    const int splits = j.splits;
+    for (size_t base = (size_t)block * 32; base < n; base += (size_t)blocks * 32) {
         const size_t i = base + e;
         float s = 0.f;
         if (i < n) {
@@ -2251,18 +2277,28 @@ __global__ __launch_bounds__(32 * PH) void sum_splits(float *__restrict__ out, c
             float t = red[0][e];
 #pragma unroll
             for (int q = 1; q < PH; ++q) t += red[q][e];
-            out[i] = t;
+            j.out[i] = t;
         }
         __syncthreads();
     }
 }
+// The first blocks_a workgroups sum job a, the others (if any) job b: two reductions of one call in one launch.
+template <int PH>
+__global__ __launch_bounds__(32 * PH) void sum_splits(SumJob a, SumJob b, unsigned blocks_a) {
+    if (blockIdx.x < blocks_a) sum_splits_part<PH>(a, blockIdx.x, blocks_a);
+    else sum_splits_part<PH>(b, blockIdx.x - blocks_a, gridDim.x - blocks_a);
+}
 
-// launches sum_splits with the number of chains that suits `splits`
-int launch_sum_splits(float *out, const float *part, size_t n, int splits) {
+// launches sum_splits with the number of chains that suits the number of splits; `also`: a second reduction for
+// the same launch
+int launch_sum_splits(float *out, const float *part, size_t n, int splits, const SumJob *also = nullptr) {
     unsigned blocks = ceil_div(n, 32);
     blocks = blocks > 16384 ? 16384 : blocks;
-    if (splits >= 128) sum_splits<32><<<blocks, 1024, 0, stream()>>>(out, part, n, splits);
-    else sum_splits<8><<<blocks, 256, 0, stream()>>>(out, part, n, splits);
+    unsigned more = also ? ceil_div(also->n, 32) : 0;
+    more = more > 16384 ? 16384 : more;
+    const SumJob a{out, part, n, splits}, b = also ? *also : SumJob{nullptr, nullptr, 0, 0};
+    if (splits >= 128 || b.splits >= 128) sum_splits<32><<<blocks + more, 1024, 0, stream()>>>(a, b, blocks);
+    else sum_splits<8><<<blocks + more, 256, 0, stream()>>>(a, b, blocks);
     SWC_LAUNCH_CHECK();
     return SWC_HIP_OK;
 }
@@ -2402,8 +2438,14 @@ __global__ __launch_bounds__(256) void bias_partials(float *__restrict__ part, c
 // of outputG instead of two.  A workgroup moves kBiasRows / 32 tiles of 32 rows x 32 columns through a 32 x 33 LDS tile
 // (matrix_trans's); thread (tx, ty) sees rows ty, ty + 8, ... of column tx and keeps its pixel coordinates
 // incrementally; the eight partial sums of a column are added in order.  grid: (chunks, OC / 32 rounded up).
+// Workgroups with blockIdx.x >= chunks (if any) turn the filter for the input gradient's convolution instead: one
+// launch of a few microseconds less in a call whose small kernels add up to a sixth of its time.
 __global__ __launch_bounds__(256) void trans_bias_partials(float *__restrict__ ogT, size_t lda, float *__restrict__ part,
-                                                           const float *__restrict__ og, ConvGeom g) {
+                                                           const float *__restrict__ og, ConvGeom g, int chunks, TurnJob turn) {
+    if ((int)blockIdx.x >= chunks) {
+        turn_filter_part(turn, ((int)blockIdx.x - chunks) * gridDim.y + blockIdx.y, ((int)gridDim.x - chunks) * gridDim.y);
+        return;
+    }
     __shared__ float tile[32][33];
     __shared__ float red[8][33];
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 32 x 8
@@ -2587,7 +2629,10 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
             const int rc0 = swc_hip_fill_f(ogT, 0.f, (size_t)g.OC * lda);
             if (rc0 != SWC_HIP_OK) return rc0;
         }
-        trans_bias_partials<<<dim3(bias_chunks, (g.OC + 31) / 32), 256, 0, stream()>>>(ogT, (size_t)lda, bias_part, outputG, g);
+        // (with the input gradient's filter turned by a few extra workgroups of the same launch)
+        const unsigned turn_x = dgrad_conv ? ceil_div(ceil_div(idims[3] * fdims[1] * fdims[2] * ocp, 256), (g.OC + 31) / 32) : 0;
+        trans_bias_partials<<<dim3(bias_chunks + (turn_x > 64 ? 64 : turn_x), (g.OC + 31) / 32), 256, 0, stream()>>>(
+            ogT, (size_t)lda, bias_part, outputG, g, bias_chunks, TurnJob{filter, turned, g.OC, (int)ocp, g.kh, g.kw, g.C});
     } else {
         const bool vec4 = g.OC % 4 == 0 && aligned16(outputG);
         const int quads = vec4 ? g.OC / 4 : g.OC;
@@ -2598,13 +2643,19 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
         else bias_partials<1><<<grid, 256, 0, stream()>>>(bias_part, outputG, g, colsq, 256 / colsq);
     }
     SWC_LAUNCH_CHECK();
-    if (int rc = launch_sum_splits(biasG, bias_part, (size_t)g.OC, bias_chunks)) return rc;
+    // the partial sums of the bias gradient are added up in the launch that adds up the filter gradient's, if there is one
+    const bool sums_together = wgrad_mfma && splits > 1;
+    const SumJob bias_sum{biasG, bias_part, (size_t)g.OC, bias_chunks};
+    if (!sums_together)
+        if (int rc = launch_sum_splits(biasG, bias_part, (size_t)g.OC, bias_chunks)) return rc;
 
     // ---- input gradient
     if (dgrad_conv) {
         unsigned blocks = ceil_div(idims[3] * fdims[1] * fdims[2] * ocp, 256);
-        turn_filter<<<blocks > 1024 ? 1024 : blocks, 256, 0, stream()>>>(filter, turned, g.OC, (int)ocp, g.kh, g.kw, g.C);
-        SWC_LAUNCH_CHECK();
+        if (!wgrad_mfma) {   // (otherwise the launch above has turned the filter)
+            turn_filter<<<blocks > 1024 ? 1024 : blocks, 256, 0, stream()>>>(TurnJob{filter, turned, g.OC, (int)ocp, g.kh, g.kw, g.C});
+            SWC_LAUNCH_CHECK();
+        }
         const float *og_in = outputG;
         if (ogp_b) {
             blocks = ceil_div(M * ocp, 256);
@@ -2650,7 +2701,7 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
                                   : launch_wgrad<1, 4, 4, 2, false, 4>(ogT, a_bytes, lda, bsrc, dst, g.OC, (int)Kf, (int)M, splits, sps);
         if (rc2 != SWC_HIP_OK) return rc2;
         if (splits > 1) {
-            if (int rc3 = launch_sum_splits(filterG, part, f_elems, splits)) return rc3;
+            if (int rc3 = launch_sum_splits(filterG, part, f_elems, splits, &bias_sum)) return rc3;
         }
     } else if (wgrad_rows) {
         const dim3 grid((unsigned)g.N, (unsigned)((g.OH + wgrad_rows - 1) / wgrad_rows));

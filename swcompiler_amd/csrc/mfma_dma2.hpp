@@ -152,7 +152,9 @@ struct DenseB {
 };
 
 #if __HIP_DEVICE_COMPILE__
-template <int TM, int TN, int WM, int STAGES, bool MID, int NW, class BSrc>
+// SKIP: a wavefront whose columns all lie outside the matrix (the last column tile of an N that is no multiple of the
+// tile width) takes part in the loads and barriers but issues no MFMA and reads no fragment.
+template <int TM, int TN, int WM, int STAGES, bool MID, int NW, class BSrc, bool SKIP = false>
 __device__ __forceinline__ void dma2_tile_body(const float *__restrict__ A, unsigned a_bytes, int lda, const BSrc &bsrc,
                                                float *__restrict__ C, size_t ldc, int M, int N, int k_begin, int k_end,
                                                const Epilogue &ep) {
@@ -258,11 +260,21 @@ __device__ __forceinline__ void dma2_tile_body(const float *__restrict__ A, unsi
     }
     const int nk = (k_end - k_begin + BK - 1) / BK;
     int rd_stage = 0, wr_stage = STAGES - 1;
+    const bool computes = !SKIP || n0 + col0 < N;   // (wavefront-uniform)
     for (int kt = 0; kt < nk; ++kt) {
         const int nx_stage = rd_stage + 1 == STAGES ? 0 : rd_stage + 1;
         float *__restrict__ wr = lds + wr_stage * T::kStageFloats;
         const float *__restrict__ rd = lds + rd_stage * T::kStageFloats;
         const float *__restrict__ nx = lds + nx_stage * T::kStageFloats;
+        if (SKIP && !computes) {   // the slice's barrier and this wavefront's share of the loads, nothing else
+            ring_sync<MID ? (STAGES - 3) * T::kLoads : (STAGES - 2) * T::kLoads>();
+#pragma unroll
+            for (int j = 0; j < T::kLoads; ++j) issue(wr, j);
+            k0 += BK;
+            rd_stage = nx_stage;
+            wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
+            continue;
+        }
         if constexpr (!MID) {
             ring_sync<(STAGES - 2) * T::kLoads>();
 #pragma unroll
