@@ -269,11 +269,36 @@ bool IRGraph::buildSubGraphs(TensorNode *in, TensorNode *out, ParallelStrategy s
             }
         return true;
     };
+    // Slice i reads rows [i, i + 1) * whole[0] / num of `in` and writes the same rows of `out`: its Scatter and Gather
+    // nodes get ops of their own (a clone shares its ops with the original) with the slice's element offset, as the
+    // reference's two-GPU example sets them by hand (test/cuda/testGPUInfer.cpp:177-178, 205-206).  The reference's
+    // buildSubGraphs leaves every offset at zero (src/graphIR/IRGraph.cpp:47-96): all its slices read and write the
+    // first one's rows.
+    size_t in_slice = 1, out_slice = 1;
+    for (size_t d : part_dims) in_slice *= d;
+    const std::vector<size_t> out_dims = out->getDims();
+    if (out_dims.empty() || out_dims[0] % (size_t)num) return false;
+    for (size_t d : out_dims) out_slice *= d;
+    out_slice /= (size_t)num;
+    auto place_slice = [&](IRGraph *g, int i) {
+        IRNode *work_in = g->getNodeByName(in->name() + "_sub"), *work_out = g->getNodeByName(out->name() + "_sub");
+        if (!work_in || !work_out || work_in->parentNum() != 1 || work_out->childNum() < 1) return false;
+        auto *scatter = static_cast<OpNode *>(work_in->getParentNode(0));
+        OpNode *gather = nullptr;
+        for (int c = 0; c < work_out->childNum(); ++c) {
+            auto *reader = static_cast<OpNode *>(work_out->getChildNode(c));
+            if (reader->nodeType() == OP_NODE && reader->getOp()->getOpName() == "Gather") gather = reader;
+        }
+        if (scatter->getOp()->getOpName() != "Scatter" || !gather) return false;
+        scatter->setOp(new op::ScatterOp((size_t)i * in_slice));
+        gather->setOp(new op::GatherOp((size_t)i * out_slice));
+        return true;
+    };
     IRGraph *inner = static_cast<op::SubGraphOp *>(first->getOp())->getGraph();
-    if (!reshape_inner(inner)) return false;
+    if (!reshape_inner(inner) || !place_slice(inner, 0)) return false;
     for (int i = 1; i < num; ++i) {
         IRGraph *copy = inner->clone();
-        if (!reshape_inner(copy)) return false;
+        if (!reshape_inner(copy) || !place_slice(copy, i)) return false;
         auto *sub_op = new op::SubGraphOp();
         sub_op->setGraph(copy);
         auto *node = new OpNode("subG", sub_op);

@@ -219,18 +219,8 @@ int main(int argc, char **argv) {
             auto *sub = dynamic_cast<SubGraphOp *>(graph->getOpNode(i)->getOp());
             if (!sub) continue;
             IRGraph *inner = sub->getGraph();
-            // the second half of the batch: element offsets on the host side of its Scatter and Gather, as the
-            // reference's example sets them by hand (test/cuda/testGPUInfer.cpp:177-178, 205-206); the nodes of a
-            // cloned graph share their Op objects with the original, so these two get Ops of their own
-            if (dev == 1)
-                for (int j = 0; j < inner->opNodeNum(); ++j) {
-                    OpNode *o = inner->getOpNode(j);
-                    if (dynamic_cast<ScatterOp *>(o->getOp())) {
-                        if (!o->isRunOnce()) o->setOp(new ScatterOp(4 * 784));
-                    } else if (dynamic_cast<GatherOp *>(o->getOp())) {
-                        o->setOp(new GatherOp(4 * 512));
-                    }
-                }
+            // (buildSubGraphs has given the second slice's Scatter and Gather the element offsets of its rows: what the
+            // reference's two-GPU example sets by hand, test/cuda/testGPUInfer.cpp:177-178, 205-206)
             inner->setDeviceLabel(Device(0, DeviceType::GPU, dev++));
             inner->findInOut();
             inner->updateTopology();

@@ -119,6 +119,9 @@ def test_graph_partition_example(lib, tmp_path):
     assert "build SubGraph Ok" in out and out.count("subGraph Node") == 2
     code = open(os.path.join(tmp_path, "Graph.cpp")).read()
     assert code.count("swc_hip_matrixTanh_f(4, 512,") == 2
+    # each slice reads and writes ITS rows (the reference's buildSubGraphs leaves both at the first slice's)
+    assert "swc_hip_h2d(data0_sub, data0, 12544)" in code and "swc_hip_h2d(data0_sub1, data0 + 3136, 12544)" in code
+    assert "swc_hip_d2h(data2, data2_sub, 8192)" in code and "swc_hip_d2h(data2 + 2048, data2_sub1, 8192)" in code
     build_hip(tmp_path)
 
 
