@@ -34,7 +34,9 @@ Also in the line:
                 events reads with nothing / a 1 KB kernel between them (the floor under every per-op figure)
   configs       the other synthetic configurations (samples/s and, per kernel,
                 TFLOP/s or GB/s with the fraction of the MI355X peak)
-                plus `training_kernels`: conv2dGrad, reluGrad, sgd, maxpoolGrad at those sizes
+                plus `training_kernels`: conv2dGrad, reluGrad, sgd, maxpoolGrad at those sizes, and `resnet50_b32`:
+                ResNet-50 (synthetic weights) imported from Caffe2 model files, fused and run as a HIP graph by the
+                generated program, with a table of its layers by class
   cpu_baseline  the reference's own CPU kernels (oracle/_ref, g++ -std=c++11 -O2,
                 one thread) on the first rows of the same batch; every other configuration
                 carries its own under configs.cfgN.cpu_baseline (whole batch, same buffers)
@@ -417,6 +419,154 @@ def run_training(rt, iters=20):
     return rows
 
 
+def run_resnet50(rt, workspace, batch=32, iters=20):
+    """The import path at a real workload (reference: test/importer/testResnetImport.cpp:19-51): ResNet-50 as the Caffe2
+    model zoo stores it, with synthetic weights (25.6 M parameters), written as a pair of .pb files, imported by
+    Caffe2Importer, fused, emitted by the HIP generator, built and run as one HIP graph per batch: `ms_per_batch` is
+    the program's own timer over `iters` replays.  Beside it, per class of layer, the layers of that class timed
+    through the C ABI as the program calls them (fused epilogues; average over back-to-back launches): what share
+    of the matrix or HBM peak each class reaches."""
+    import shutil
+    import subprocess
+    import tempfile
+    from swcompiler_amd.caffe2_files import enc_net, make_resnet50
+    swc = os.path.join(ROOT, "swcompiler_amd", "swc")
+    gen = os.path.join(swc, "test", "bin", "genGraphs")
+    if not os.path.exists(gen) or shutil.which("g++") is None:
+        return dict(error="genGraphs is not built or there is no g++ here")
+    predict, init, w = make_resnet50()
+    out = dict(model="ResNet-50, Caffe2 model-zoo structure, synthetic weights, 224 x 224 x 3, fp32", batch=batch,
+               parameters=int(sum(v.size for v in w.values())))
+    work = tempfile.mkdtemp(prefix="swc_resnet50_")
+    try:
+        open(os.path.join(work, "predict_net.pb"), "wb").write(enc_net("resnet50", predict, packed=True))
+        open(os.path.join(work, "init_net.pb"), "wb").write(enc_net("resnet50_init", init, packed=True))
+        np.random.default_rng(11).standard_normal((batch, 224, 224, 3)).astype(np.float32).tofile(os.path.join(work, "data.bin"))
+        libdir = os.path.join(ROOT, "swcompiler_amd")
+        subprocess.run([gen, "caffe2@224", "hip", str(batch), str(iters), "graph"], cwd=work, check=True, capture_output=True, timeout=120)
+        subprocess.run(["g++", "-std=c++11", "-O2", "-I", os.path.join(ROOT, "include"), "Graph.cpp", "-L", libdir,
+                        "-Wl,-rpath," + libdir, "-lswc_hip", "-o", "net_hip.bin"], cwd=work, check=True, capture_output=True, timeout=120)
+        rt.sync()
+        res = subprocess.run([os.path.join(work, "net_hip.bin")], cwd=work, check=True, capture_output=True, text=True, timeout=300).stdout
+        ms = float(res.split("swc_time_ms_per_iter")[1].split()[0])
+        out.update(ms_per_batch=ms, samples_per_s=batch / ms * 1e3)
+    except Exception as e:
+        out["error"] = f"{type(e).__name__}: {str(e)[:300]}"
+    finally:
+        shutil.rmtree(work, ignore_errors=True)
+
+    # ---- the layers by class, as the generated program calls them
+    def timed(fn, n=10):
+        for _ in range(2):
+            fn()
+        rt.event_record(0)
+        for _ in range(n):
+            fn()
+        rt.event_record(1)
+        return rt.event_elapsed_ms(0, 1) / n
+
+    rng = np.random.default_rng(5)
+    shape = {"gpu_0/data": (224, 224, 3)}
+    need = rt.gemm_workspace_bytes(batch, 1000, 2048)
+    for op in predict:   # one scratch buffer for the layers of this leg, as the generated program sets one
+        if op["type"] == "Conv":
+            src, (oc, ic, k) = shape[op["input"][0]], w[op["input"][1]].shape[:3]
+            s, pad = op["arg"]["stride"], op["arg"]["pad"]
+            need = max(need, rt.conv2d_workspace_bytes((batch,) + src, (oc, k, k, ic), (s, s), (pad,) * 4))
+            shape[op["output"][0]] = ((src[0] + 2 * pad - k) // s + 1,) * 2 + (oc,)
+        elif op["type"] in ("MaxPool", "AveragePool"):
+            src, a = shape[op["input"][0]], op["arg"]
+            shape[op["output"][0]] = ((src[0] + 2 * a.get("pad", 0) - a["kernel"]) // a["stride"] + 1,) * 2 + (src[2],)
+        else:
+            shape[op["output"][0]] = shape[op["input"][0]]
+    scratch = rt.empty((need // 4 + 64,))
+    rt.set_workspace(scratch)
+    shape = {"gpu_0/data": (224, 224, 3)}
+    relu_after, summed = set(), set()
+    for op in predict:
+        if op["type"] == "Relu":
+            relu_after.add(op["input"][0])
+        if op["type"] == "Sum":
+            summed.add(op["input"][0])
+    classes, seen, total_flop = {}, {}, 0.0
+
+    def add(cls, ms, flop=0.0, nbytes=0.0):
+        c = classes.setdefault(cls, dict(layers=0, ms=0.0, flop=0.0, bytes=0.0))
+        c["layers"] += 1
+        c["ms"] += ms
+        c["flop"] += flop
+        c["bytes"] += nbytes
+
+    for op in predict:
+        a, src = op.get("arg", {}), shape[op["input"][0]]
+        if op["type"] == "Conv":
+            oc, ic, k = w[op["input"][1]].shape[:3]
+            s, pad = a["stride"], a["pad"]
+            oh = (src[0] + 2 * pad - k) // s + 1
+            name = op["output"][0]
+            shape[name] = (oh, oh, oc)
+            bn = name + "_bn"
+            key = (src, oc, k, s, bn in relu_after, bn in summed)
+            flop = 2.0 * batch * oh * oh * oc * ic * k * k
+            total_flop += flop
+            if key not in seen:
+                x = rt.upload(rng.standard_normal((batch,) + src).astype(np.float32))
+                f = rt.upload((rng.standard_normal((oc, k, k, ic)) * np.sqrt(2.0 / (ic * k * k))).astype(np.float32))
+                b = rt.upload(np.zeros(oc, np.float32))
+                par = [rt.upload(rng.uniform(0.5, 1.5, oc).astype(np.float32)) for _ in range(4)]
+                y = rt.empty((batch, oh, oh, oc))
+                res = rt.upload(rng.standard_normal((batch, oh, oh, oc)).astype(np.float32)) if key[5] else None
+                fn = lambda: rt.conv2d(x, f, b, (k, k), (s, s), (pad,) * 4, bn=par, eps=1e-5, relu=key[4] or key[5],   # noqa: E731
+                                       residual=res, out=y)
+                seen[key] = (timed(fn), rt.last_kernel())
+                for t in [x, f, b, y] + par + ([res] if res is not None else []):
+                    t.free()
+            cls = "conv 7x7 stride 2 (first layer)" if k == 7 else f"conv {k}x{k}" + (f" stride {s}" if s > 1 else "")
+            add(cls, seen[key][0], flop=flop)
+        elif op["type"] in ("MaxPool", "AveragePool"):
+            k, s, pad = a["kernel"], a["stride"], a.get("pad", 0)
+            oh = (src[0] + 2 * pad - k) // s + 1
+            shape[op["output"][0]] = (oh, oh, src[2])
+            x = rt.upload(rng.standard_normal((batch,) + src).astype(np.float32))
+            y = rt.empty((batch, oh, oh, src[2]))
+            pool = rt.maxpool if op["type"] == "MaxPool" else rt.avgpool
+            ms = timed(lambda: pool(x, (k, k), (s, s), (pad,) * 4, out=y))
+            add(f"{'max' if op['type'] == 'MaxPool' else 'average'} pooling {k}x{k} stride {s}", ms, nbytes=4.0 * (x.size + y.size))
+            x.free(), y.free()
+        elif op["type"] == "FC":
+            n, kdim = w[op["input"][1]].shape
+            x, wt, b = rt.upload(rng.standard_normal((batch, kdim)).astype(np.float32)), rt.upload(rng.standard_normal((kdim, n)).astype(np.float32)), rt.upload(np.zeros(n, np.float32))
+            y = rt.empty((batch, n))
+            ms = timed(lambda: rt.fcbias(x, wt, b, softmax=True, out=y))
+            add("FC 2048 -> 1000 + softmax", ms, flop=2.0 * batch * n * kdim, nbytes=4.0 * (kdim * n + n + batch * (kdim + n)))
+            total_flop += 2.0 * batch * n * kdim
+            shape[op["output"][0]] = src
+            for t in (x, wt, b, y):
+                t.free()
+        else:
+            shape[op["output"][0]] = src
+    rt.set_workspace(workspace)
+    scratch.free()
+    table = []
+    for cls, c in classes.items():
+        row = dict(layer_class=cls, layers=c["layers"], ms=c["ms"])
+        if c["flop"] and not cls.startswith("FC"):
+            row.update(flop=c["flop"], tflops=c["flop"] / c["ms"] / 1e9, frac=c["flop"] / c["ms"] / 1e9 / PEAK_TFLOPS_FP32_MFMA, bound="mfma")
+        else:   # pools, and the FC of 32 rows (one pass over its 8 MB of weights)
+            row.update(bytes=c["bytes"], gbs=c["bytes"] / c["ms"] / 1e6, frac=c["bytes"] / c["ms"] / 1e6 / PEAK_HBM_GBS, bound="hbm")
+        table.append(row)
+    out["layer_classes"] = table
+    out["flop_per_batch"] = total_flop
+    out["layers_ms_sum"] = sum(c["ms"] for c in classes.values())
+    out["conv_shapes"] = [dict(input=list(k[0]), oc=k[1], k=k[2], stride=k[3], relu=k[4], residual=k[5], ms=ms, kernel=name,
+                               frac=2.0 * batch * ((k[0][0] - 1) // k[3] + 1) ** 2 * k[1] * k[0][2] * k[2] ** 2 / ms / 1e9 / PEAK_TFLOPS_FP32_MFMA)
+                          for k, (ms, name) in seen.items()]
+    if "ms_per_batch" in out:
+        out["tflops"] = total_flop / out["ms_per_batch"] / 1e9
+        out["frac_of_mfma_peak"] = out["tflops"] / PEAK_TFLOPS_FP32_MFMA
+    return out
+
+
 def run_bn_pool_separately(rt, graphs, iters=20):
     """BN+ReLU and max-pool of the bandwidth configuration as two launches (the target emits one fused call,
     which is what that configuration's step times): the two kernels' own rates against the HBM roofline."""
@@ -599,6 +749,8 @@ def main():
                          "FETCH_SIZE/WRITE_SIZE readings calibrate the counters for the traffic figures")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="instead of the benchmark: write profiles/traffic.json from two rocprofv3 --pmc counter files")
+    ap.add_argument("--resnet50", action="store_true",
+                    help="instead of the benchmark: only the `resnet50_b32` leg (the import path), printed as its own JSON line")
     ap.add_argument("--clocks", action="store_true",
                     help="instead of the benchmark: print the shader clock held under single kernels, by operand distribution")
     args = ap.parse_args()
@@ -614,6 +766,12 @@ def main():
     workspace = bench_workspace(rt, graphs)
     if args.clocks:
         print(json.dumps(clock_report(rt)))
+        rt.sync()
+        rt.set_workspace(None)
+        return
+
+    if args.resnet50:
+        print(json.dumps(run_resnet50(rt, workspace)))
         rt.sync()
         rt.set_workspace(None)
         return
@@ -684,6 +842,7 @@ def main():
                                        kernels=r["kernels"])
         others["cfg5"]["kernels_unfused"] = run_bn_pool_separately(rt, graphs)
         others["training_kernels"] = dict(kernels=run_training(rt))
+        others["resnet50_b32"] = run_resnet50(rt, workspace)
         out["configs"] = others
     failed = []
     if not args.no_cpu:
