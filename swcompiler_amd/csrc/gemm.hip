@@ -311,6 +311,46 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 constexpr int kSkinnyMaxWaves = 16;
 constexpr int kSkinnyUnroll = 4;
 
+// The end of both skinny kernels, entered by every thread of the workgroup behind the barrier after which the
+// partial 16x16 tile of wavefront w lies at part + w * wave_stride as [row][17]: thread 16 * row + column adds the
+// tiles in wavefront order and applies bias and ReLU (the wavefronts past the fourth have nothing left to do).
+// softmax != 0: the workgroup holds whole rows, so the row softmax of matrixSoftmax_f is stored instead, with the
+// arithmetic of the stand-alone kernel for short rows (row maximum; exp(x - max) summed over the columns in
+// ascending order; exp(x - max) times the reciprocal of that sum).  The sixteen lanes of a row work together:
+// the maximum by lane exchange (any order gives the same maximum), each lane the exponential of its own column,
+// the sum by every lane over the row's values in LDS.  No further barrier: a thread overwrites only the element
+// of the first tile that it alone has read, and a row's sixteen lanes are in one wavefront, whose LDS accesses
+// are served in program order.
+__device__ inline float skinny_bias(const Epilogue &ep, int tid, int N) {   // asked for at kernel entry: a cold load
+    return (ep.bias && tid < 256 && (tid & 15) < N) ? ep.bias[tid & 15] : 0.f;
+}
+
+__device__ inline void skinny_finish(float *part, int wave_stride, int waves, int tid, size_t row0, int rows, int N,
+                                     float *C, size_t ldc, const Epilogue &ep, float bias, int softmax) {
+    if (tid >= 256) return;
+    const int r = tid >> 4, c = tid & 15;
+    const bool live = r < rows && c < N;
+    float *mine = part + r * 17 + c;
+    float x = 0.f;
+    for (int w = 0; w < waves; ++w) x += mine[w * wave_stride];
+    x += bias;
+    if (ep.relu) x = (x > 0.f) ? x : 0.f;
+    if (!softmax) {
+        if (live) C[(row0 + r) * ldc + c] = x;
+        return;
+    }
+    float mx = live ? x : -__builtin_inff();
+#pragma unroll
+    for (int o = 8; o; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 16));
+    const float e = fast_exp(x - mx);
+    *mine = e;
+    __builtin_amdgcn_wave_barrier();
+    float sum = 0.f;
+    for (int j = 0; j < N; ++j) sum += part[r * 17 + j];
+    const float inv = 1.f / sum;
+    if (live) C[(row0 + r) * ldc + c] = e * inv;
+}
+
 // v_mfma_f32_16x16x4_f32: A[i][kk] i = l%16, kk = l/16; B[kk][j] j = l%16, kk = l/16;
 // D[i][j] in VGPR v: j = l%16, i = 4*(l/16) + v.
 // K is walked in groups of 32: quarter-wave q = l/16 takes k = 8q..8q+7, so a
@@ -329,6 +369,7 @@ __global__ __launch_bounds__(64 * kSkinnyMaxWaves) void gemm_skinny(const float 
     const bool row_ok = row < M;
     const bool col_ok = i < N;   // as B operand, lane's column j = i
     const float *arow = A + (size_t)(row_ok ? row : 0) * lda;
+    const float bias = skinny_bias(ep, tid, N);
     v4f acc = {0.f, 0.f, 0.f, 0.f};
     // kSkinnyUnroll groups of 32 k per trip: all of a trip's loads are issued
     // before its first MFMA, so a wavefront keeps 8 KB of A in flight.
@@ -358,32 +399,8 @@ __global__ __launch_bounds__(64 * kSkinnyMaxWaves) void gemm_skinny(const float 
 #pragma unroll
     for (int v = 0; v < 4; ++v) part[wave][4 * q + v][i] = acc[v];
     __syncthreads();
-    if (tid < 256) {
-        const int r = tid >> 4, c = tid & 15;
-        float s = 0.f;
-        for (int w = 0; w < waves; ++w) s += part[w][r][c];
-        const int grow = blockIdx.x * 16 + r;
-        if (grow < M && c < N) {
-            float x = s + (ep.bias ? ep.bias[c] : 0.f);
-            if (ep.relu) x = (x > 0.f) ? x : 0.f;
-            if (softmax) part[0][r][c] = x;   // (this thread alone read part[.][r][c])
-            else C[(size_t)grow * ldc + c] = x;
-        }
-    }
-    if (softmax) {   // the workgroup holds whole rows: the row softmax of matrixSoftmax_f, one lane per row,
-        __syncthreads();   // with the arithmetic of the stand-alone kernel for short rows
-        const int grow = blockIdx.x * 16 + tid;
-        if (tid < 16 && grow < M) {
-            const float *src = part[0][tid];
-            float *dst = C + (size_t)grow * ldc;
-            float mx = src[0];
-            for (int j = 1; j < N; ++j) mx = fmaxf(mx, src[j]);
-            float sum = 0.f;
-            for (int j = 0; j < N; ++j) sum += fast_exp(src[j] - mx);
-            const float inv = 1.f / sum;
-            for (int j = 0; j < N; ++j) dst[j] = fast_exp(src[j] - mx) * inv;
-        }
-    }
+    const int rows = (M - (int)blockIdx.x * 16) < 16 ? (M - (int)blockIdx.x * 16) : 16;
+    skinny_finish(&part[0][0][0], 16 * 17, waves, tid, (size_t)blockIdx.x * 16, rows, N, C, ldc, ep, bias, softmax);
 }
 
 // ------------------------------------------------- skinny GEMM, long K, streamed
@@ -403,6 +420,13 @@ __global__ __launch_bounds__(64 * kSkinnyMaxWaves) void gemm_skinny(const float 
 // k of a group is dealt to the four k-lanes of v_mfma_f32_16x16x4_f32 as q, step s -> 4q + 16(s / 4) + s % 4, the
 // same on the A and the B side.  The 16-byte pieces of a line are XOR-ed with the row inside a slot (bank spread).
 // Partial tiles are summed through LDS in wavefront order, as in gemm_skinny, with the same epilogue.
+// Where the time goes at 4096 x 4096 x 10 with the row softmax (13.3 us with A resident in the last-level cache,
+// 14.1 us out of HBM, on a box where a plain read of the 64 MiB takes 8.5 / 11.0 us), measured by leaving parts out:
+// the A loads alone 10.5 / 12.0 us; the B rows (every workgroup passes over all of B: 40 MB out of L2) +0.8 us;
+// the MFMAs +1.0 us (what the last groups of a SIMD's four wavefronts still hold when the stream ends: N = 10 fills
+// 10 of the 16 columns of every v_mfma_f32_16x16x4_f32, and every fp32 MFMA shape has the same rate); the reduction,
+// the store of C and the end of the kernel behind it +1.0 us.  Tried and slower: each wavefront a contiguous range of
+// K instead of every sixteenth group (+0.7 us), no rotation of the starting group (+1.0 us).
 constexpr int kStreamWaves = 16;
 constexpr int kStreamATile = 2048;   // bytes of a group's A tile in a slot; the B rows follow
 
@@ -422,6 +446,7 @@ __global__ __launch_bounds__(64 * kStreamWaves) void gemm_skinny_stream(const fl
     const int i = lane & 15, q = lane >> 4;
     const size_t row0 = (size_t)blockIdx.x * 16;
     const int rows = (M - (int)row0) < 16 ? (M - (int)row0) : 16;
+    const float bias = skinny_bias(ep, tid, N);
     const __amdgpu_buffer_rsrc_t rs_a = make_rsrc(A + row0 * lda, (unsigned)(((size_t)(rows - 1) * lda + K) * 4));
     const __amdgpu_buffer_rsrc_t rs_b = make_rsrc(B, (unsigned)((size_t)K * ldb * 4));
     const int slot_bytes = stream_slot_bytes(ldb);
@@ -495,36 +520,12 @@ __global__ __launch_bounds__(64 * kStreamWaves) void gemm_skinny_stream(const fl
         r = r + 1 == RING ? 0 : r + 1;
     }
     acc0 += acc1;
-    __syncthreads();   // every ring is read out: the partial tiles go over them
-    float(*part)[16][17] = reinterpret_cast<float(*)[16][17]>(lds);
+    // a wavefront's partial tile goes over the start of its own ring, which no other wavefront touches
+    float(*part)[17] = reinterpret_cast<float(*)[17]>(ring);
 #pragma unroll
-    for (int v = 0; v < 4; ++v) part[wave][4 * q + v][i] = acc0[v];
+    for (int v = 0; v < 4; ++v) part[4 * q + v][i] = acc0[v];
     __syncthreads();
-    if (tid < 256) {
-        const int pr = tid >> 4, c = tid & 15;
-        float s = 0.f;
-        for (int w = 0; w < kStreamWaves; ++w) s += part[w][pr][c];
-        const size_t grow = row0 + pr;
-        if (pr < rows && c < N) {
-            float x = s + (ep.bias ? ep.bias[c] : 0.f);
-            if (ep.relu) x = (x > 0.f) ? x : 0.f;
-            if (softmax) part[0][pr][c] = x;   // (this thread alone read part[.][pr][c])
-            else C[grow * ldc + c] = x;
-        }
-    }
-    if (softmax) {   // as gemm_skinny: one lane per row, the arithmetic of the stand-alone short-row kernel
-        __syncthreads();
-        if (tid < rows) {
-            const float *src = part[0][tid];
-            float *dst = C + (row0 + tid) * ldc;
-            float mx = src[0];
-            for (int j = 1; j < N; ++j) mx = fmaxf(mx, src[j]);
-            float sum = 0.f;
-            for (int j = 0; j < N; ++j) sum += fast_exp(src[j] - mx);
-            const float inv = 1.f / sum;
-            for (int j = 0; j < N; ++j) dst[j] = fast_exp(src[j] - mx) * inv;
-        }
-    }
+    skinny_finish(lds, RING * slot_bytes / 4, kStreamWaves, tid, row0, rows, N, C, ldc, ep, bias, softmax);
 #endif
 }
 
