@@ -749,6 +749,7 @@ def main():
                          "FETCH_SIZE/WRITE_SIZE readings calibrate the counters for the traffic figures")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="instead of the benchmark: write profiles/traffic.json from two rocprofv3 --pmc counter files")
+    ap.add_argument("--no-resnet", action="store_true", help="skip the `resnet50_b32` leg (the only one that starts other programs)")
     ap.add_argument("--resnet50", action="store_true",
                     help="instead of the benchmark: only the `resnet50_b32` leg (the import path), printed as its own JSON line")
     ap.add_argument("--clocks", action="store_true",
@@ -842,7 +843,8 @@ def main():
                                        kernels=r["kernels"])
         others["cfg5"]["kernels_unfused"] = run_bn_pool_separately(rt, graphs)
         others["training_kernels"] = dict(kernels=run_training(rt))
-        others["resnet50_b32"] = run_resnet50(rt, workspace)
+        if not args.no_resnet:
+            others["resnet50_b32"] = run_resnet50(rt, workspace)
         out["configs"] = others
     failed = []
     if not args.no_cpu:

@@ -45,6 +45,7 @@ struct Switches {
     int conv_share_all = 0;       // SWC_HIP_CONV_SHARE_ALL=n: slices per tile from which a short layer is cut (unset 0: default; "0" -> -1: never)
     int conv_slots = 0;           // SWC_HIP_CONV_SLOTS=n: pretend the chip holds n workgroups at a time (0: ask the device)
     int conv_piece_min = 0;       // SWC_HIP_CONV_PIECE_MIN=n: least K slices per piece of a tile cut along K (0: default)
+    int conv_min_idle = -1;       // SWC_HIP_CONV_MIN_IDLE=n: tiles are cut along K only if whole tiles would leave the average CU idle for n slices + 1/16 per cut tile (0: no such test; -1: default)
     bool conv_fair = true;        // SWC_HIP_CONV_FAIR=0: the last round's workgroups keep one priority (see conv_win)
     int wgrad_bn = 0;             // SWC_HIP_WGRAD_BN=128|256: tile width of the filter gradient (0: planner's choice)
 };

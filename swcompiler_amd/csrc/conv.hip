@@ -1332,11 +1332,23 @@ int share_all_min_slices() {
 // per CU, started first (the first workgroups of a launch land on distinct CUs): with pieces of four slices or more on
 // only some CUs those CUs finished 4-5 us after the others (traced per workgroup: 65.5 against 61 us on 28x28x128->128).
 constexpr int kPieceMinSlices = 2;   // a piece costs a ring start and a tile store
+// The pieces need a second kernel (5-6 us with the gap before it) and their own stores, the more of them the more
+// tiles are cut: cutting pays only if whole tiles would leave the average CU idle for longer than that while the
+// busiest one works through its last tile.  Idle time in slices = (rounds of the busiest CU - tiles per CU) x slices
+// per tile; tiles are cut from 12 slices + 1/16 per cut tile on.  Measured at batch 32, whole against cut (idle
+// slices, cut tiles): 28x28x512 -> 256 1x1/2 (7.5, 136) 21.0 / 26.4 us; 14x14x1024 -> 256 1x1 (15, 136) 37.5 / 39.4;
+// 7x7x2048 -> 512 1x1 (14, 200) 41.2 / 44.3; 56x56x64 -> 128 3x3 (13.5, 64) 125.9 / 124.0; 7x7x512 -> 2048 1x1 (14, 32)
+// 44.0 / 40.8; 56x56x64 -> 64 3x3 (15.8, 32) 74.1 / 71.9; 14x14x1024 -> 2048 1x1/2 (28, 32) 78.1 / 65.7; 28x28x128 -> 128 3x3
+// (34, 16) 77.7 / 67.6; 14x14x256 -> 256 3x3 (34, 136) 75.5 / 69.7; 14x14x512 -> 512 3x3 (68, 136) 271 / 215.
+constexpr int kMinIdleSlices = 12;
 SkPlan sk_plan(long tiles, int nk, int slots, bool allow_shared) {
     SkPlan p{(int)tiles, 0, 0, 0};
     if (!allow_shared || tiles == 0) return p;
     const int piece_min = switches().conv_piece_min > 0 ? switches().conv_piece_min : kPieceMinSlices;
     const long cus = num_cus() < slots ? num_cus() : slots;   // (tests pretend a smaller chip through `slots`)
+    const int min_idle = switches().conv_min_idle >= 0 ? switches().conv_min_idle : kMinIdleSlices;
+    const long cut = tiles < cus ? tiles : tiles % cus;
+    if (min_idle > 0 && ((tiles + cus - 1) / cus * cus - tiles) * nk * 16 < (min_idle * 16 + cut) * cus) return p;
     long rest, wgs;
     if (tiles < cus) {
         // fewer tiles than CUs: all are cut if K is long (a nearly full round: leave it; a twelfth of a round or

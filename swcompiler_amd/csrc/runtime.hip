@@ -73,6 +73,7 @@ void load_switches() {
     s.conv_share_all = getenv("SWC_HIP_CONV_SHARE_ALL") ? (number("SWC_HIP_CONV_SHARE_ALL") ? number("SWC_HIP_CONV_SHARE_ALL") : -1) : 0;
     s.conv_slots = number("SWC_HIP_CONV_SLOTS");
     s.conv_piece_min = number("SWC_HIP_CONV_PIECE_MIN");
+    s.conv_min_idle = getenv("SWC_HIP_CONV_MIN_IDLE") ? number("SWC_HIP_CONV_MIN_IDLE") : -1;
     s.conv_fair = !is("SWC_HIP_CONV_FAIR", "0");
     s.wgrad_bn = number("SWC_HIP_WGRAD_BN");
     g_switches = s;

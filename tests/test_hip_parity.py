@@ -238,6 +238,7 @@ def test_conv_random_shapes_integer_exact(rt, oracle, idims, fdims, strides, pad
     print("case random conv", idims, fdims, strides, pads, slots, flush=True)
     if slots:
         switch_env.setenv("SWC_HIP_CONV_SLOTS", slots)
+        switch_env.setenv("SWC_HIP_CONV_MIN_IDLE", "0")   # cut tiles however little that saves
     rng = np.random.default_rng(sum(idims) * 7 + sum(fdims) * 3 + sum(pads))
     x = rng.integers(-3, 4, idims).astype(np.float32)
     f = rng.integers(-3, 4, fdims).astype(np.float32)
@@ -287,6 +288,7 @@ def test_conv_win_integer_exact(rt, oracle, idims, fdims, strides, pads, slots, 
     print("case conv_win", idims, fdims, strides, pads, slots, flush=True)
     if slots:
         switch_env.setenv("SWC_HIP_CONV_SLOTS", slots)
+        switch_env.setenv("SWC_HIP_CONV_MIN_IDLE", "0")   # cut tiles however little that saves
     rng = np.random.default_rng(sum(idims) * 13 + sum(fdims))
     x = rng.integers(-3, 4, idims).astype(np.float32)
     f = rng.integers(-3, 4, fdims).astype(np.float32)
@@ -661,6 +663,7 @@ def test_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, pads, s
     print("case pooled conv", idims, fdims, pads, slots, flush=True)
     if slots:
         switch_env.setenv("SWC_HIP_CONV_SLOTS", slots)
+        switch_env.setenv("SWC_HIP_CONV_MIN_IDLE", "0")   # cut tiles however little that saves
     rng = np.random.default_rng(sum(idims) + sum(fdims))
     oc, c = fdims[0], fdims[3]
     x = rng.standard_normal(idims).astype(np.float32)
@@ -711,6 +714,7 @@ def test_conv_kernel_forms_agree_bit_for_bit(rt, idims, fdims, pads, slots, swit
     print("case conv kernel forms", idims, fdims, pads, slots, flush=True)
     if slots:
         switch_env.setenv("SWC_HIP_CONV_SLOTS", slots)
+        switch_env.setenv("SWC_HIP_CONV_MIN_IDLE", "0")   # cut tiles however little that saves
     rng = np.random.default_rng(sum(idims) * 3 + sum(fdims))
     oc = fdims[0]
     x = rng.standard_normal(idims).astype(np.float32)
@@ -983,6 +987,7 @@ def test_conv_tiles_shared_along_k(rt, oracle, variant, switch_env):
         shared = 0
         for slots in (3, 4, 5, 6, 7, 9, 11, 13, 17, 19, 23, 29, 37, 47):
             switch_env.setenv("SWC_HIP_CONV_SLOTS", str(slots))
+            switch_env.setenv("SWC_HIP_CONV_MIN_IDLE", "0")   # cut tiles however little that saves
             shared += rt.conv2d_workspace_bytes(idims, fdims, strides, pads) > 0
             plain = rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy()
             fused = rt.conv2d(dx, df, db, fdims[1:3], strides, pads, bn=bn, eps=1e-5, relu=True).numpy()
@@ -995,6 +1000,7 @@ def test_conv_tiles_shared_along_k(rt, oracle, variant, switch_env):
     # real-valued operands: the usual tolerance
     idims, fdims, strides, pads = SHARED_CONV_CASES[1]
     switch_env.setenv("SWC_HIP_CONV_SLOTS", "4")
+    switch_env.setenv("SWC_HIP_CONV_MIN_IDLE", "0")   # cut tiles however little that saves
     x = rng.standard_normal(idims).astype(np.float32)
     f = rng.standard_normal(fdims).astype(np.float32)
     b = rng.standard_normal(fdims[0]).astype(np.float32)
@@ -1023,11 +1029,13 @@ def test_conv_layers_of_few_tiles_and_a_long_k_are_cut_throughout(rt, oracle, id
     for slots in (None, 5, 9, 37, 100):
         if slots:
             switch_env.setenv("SWC_HIP_CONV_SLOTS", str(slots))
+            switch_env.setenv("SWC_HIP_CONV_MIN_IDLE", "0")   # cut tiles however little that saves
         assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy(), want, f"all tiles shared, slots {slots}")
         assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads, relu=True).numpy(), oracle.relu(want),
                          f"all tiles shared + relu, slots {slots}")
     switch_env.delenv("SWC_HIP_CONV_SLOTS")
     switch_env.setenv("SWC_HIP_CONV_SHARE_ALL", "0")
+    switch_env.setenv("SWC_HIP_CONV_MIN_IDLE", "0")   # cut tiles however little that saves
     assert rt.conv2d_workspace_bytes(idims, fdims, strides, pads) == 0
     assert_bit_exact(rt.conv2d(dx, df, db, fdims[1:3], strides, pads).numpy(), want, "whole tiles")
     switch_env.setenv("SWC_HIP_CONV_SHARE_ALL", "8")
@@ -1127,6 +1135,7 @@ def test_conv_shared_tiles_in_a_caller_workspace(rt, oracle, switch_env):
     from swcompiler_amd.hip import SwcHipError
     idims, fdims, strides, pads = SHARED_CONV_CASES[0]
     switch_env.setenv("SWC_HIP_CONV_SLOTS", "19")
+    switch_env.setenv("SWC_HIP_CONV_MIN_IDLE", "0")   # cut tiles however little that saves
     need = rt.conv2d_workspace_bytes(idims, fdims, strides, pads)
     assert need > 0
     rng = np.random.default_rng(32)
