@@ -2170,12 +2170,31 @@ __global__ __launch_bounds__(256) void dgrad_few_channels(float *__restrict__ ig
 struct Im2colB {
     const float *in;
     unsigned bytes;
-    int H, W, C, OH, OW, kw, sh, sw, pt, pl, nimg;
-    int q32, r32;   // 32 / OW, 32 % OW: how a slice of 32 pixels moves (oy, ox)
+    int H, W, nimg, kw, C, OH, OW, sh, sw, pt, pl;
+    // A lane follows its pixel from slice to slice (+32 pixels) by additions and selects only: multiplications, and
+    // divergent branches between the MFMAs of a slice, cost the matrix pipe more than the loads they feed.
+    int ys_end, xs_end;          // OH * sh, OW * sw: where the scaled row / column wraps
+    int dxs, dys, dimg, doff;    // a slice's step: columns (x sw), rows (x sh), images, bytes — before carries
+    int row_carry, img_carry;    // bytes added when the column wraps into the next row / the row into the next image
     struct Lane {
-        int img, oy, ox, ty, tx, cbase, krow;
+        int img, ys, xs, off;    // image, oy * sh, ox * sw, byte offset of input pixel (img, ys, xs)
+        int ty, tx, tap, krow;   // tap row - pt, tap column - pl, byte offset of the tap and channel (+ descriptor shift), row in the slice
         bool ok;
     };
+    static Im2colB of(const float *in, size_t in_bytes, const ConvGeom &g) {
+        Im2colB b{};
+        b.in = in, b.bytes = (unsigned)in_bytes;
+        b.H = g.H, b.W = g.W, b.nimg = g.N, b.kw = g.kw, b.C = g.C, b.OH = g.OH, b.OW = g.OW;
+        b.sh = g.sh, b.sw = g.sw, b.pt = g.pt, b.pl = g.pl;
+        b.ys_end = g.OH * g.sh, b.xs_end = g.OW * g.sw;
+        const int per_img = g.OH * g.OW, qi = BK / per_img, qy = BK % per_img / g.OW, rx = BK % per_img % g.OW;
+        const int px = g.C * 4;   // bytes per input pixel
+        b.dxs = rx * g.sw, b.dys = qy * g.sh, b.dimg = qi;
+        b.doff = ((qi * g.H + qy * g.sh) * g.W + rx * g.sw) * px;
+        b.row_carry = (g.sh * g.W - g.OW * g.sw) * px;
+        b.img_carry = (g.H - g.OH * g.sh) * g.W * px;
+        return b;
+    }
 #if __HIP_DEVICE_COMPILE__
     __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc() const {
         return make_rsrc(reinterpret_cast<const char *>(in) - kImmSpan, bytes + kImmSpan);
@@ -2184,36 +2203,38 @@ struct Im2colB {
     __device__ __forceinline__ Lane init(int krow, int col, bool col_ok, int imm, int k_begin) const {
         Lane s;
         const int pix = k_begin + krow;
-        s.ox = pix % OW;
-        const int t = pix / OW;
-        s.oy = t % OH;
+        const int ox = pix % OW, t = pix / OW, oy = t % OH;
         s.img = t / OH;
-        const int tap = col / C;
-        s.ty = tap / kw;
-        s.tx = tap - s.ty * kw;
-        s.cbase = (col - tap * C) * 4 + kImmSpan - imm;
+        s.ys = oy * sh;
+        s.xs = ox * sw;
+        s.off = ((s.img * H + s.ys) * W + s.xs) * C * 4;
+        const int tap = col / C, ky = tap / kw;
+        s.ty = ky - pt;
+        s.tx = tap - ky * kw - pl;
+        s.tap = ((s.ty * W + s.tx) * C + (col - tap * C)) * 4 + kImmSpan - imm;
         s.krow = krow;
         s.ok = col_ok;
         return s;
     }
     __device__ __forceinline__ int voffset(const Lane &s, int k0, int k_end) const {
-        const int iy = s.oy * sh - pt + s.ty, ix = s.ox * sw - pl + s.tx;
-        const bool valid = s.ok && k0 + s.krow < k_end && s.img < nimg && (unsigned)iy < (unsigned)H &&
-                           (unsigned)ix < (unsigned)W;
-        return valid ? ((s.img * H + iy) * W + ix) * C * 4 + s.cbase : kOutOfRange;
+        const int iy = s.ys + s.ty, ix = s.xs + s.tx;
+        const bool valid = s.ok & (k0 + s.krow < k_end) & (s.img < nimg) & ((unsigned)iy < (unsigned)H) &
+                           ((unsigned)ix < (unsigned)W);
+        const int off = s.off + s.tap;
+        return valid ? off : kOutOfRange;
     }
     __device__ __forceinline__ int soffset(int) const { return 0; }
     __device__ __forceinline__ void advance(Lane &s) const {
-        s.ox += r32;
-        s.oy += q32;
-        if (s.ox >= OW) {
-            s.ox -= OW;
-            ++s.oy;
-        }
-        while (s.oy >= OH) {
-            s.oy -= OH;
-            ++s.img;
-        }
+        s.xs += dxs;
+        s.off += doff;
+        const bool cx = s.xs >= xs_end;
+        s.xs -= cx ? xs_end : 0;
+        s.off += cx ? row_carry : 0;
+        s.ys += dys + (cx ? sh : 0);
+        const bool cy = s.ys >= ys_end;
+        s.ys -= cy ? ys_end : 0;
+        s.off += cy ? img_carry : 0;
+        s.img += dimg + (cy ? 1 : 0);
     }
 #endif
 };
@@ -2704,8 +2725,7 @@ int conv_grad(float *inputG, float *filterG, float *biasG, const float *outputG,
 
     // ---- filter gradient
     if (wgrad_mfma) {
-        const Im2colB bsrc{input, (unsigned)(in_elems * 4), g.H, g.W, g.C, g.OH, g.OW, g.kw, g.sh, g.sw, g.pt, g.pl, g.N,
-                           BK / g.OW, BK % g.OW};
+        const Im2colB bsrc = Im2colB::of(input, in_elems * 4, g);
         float *dst = splits > 1 ? part : filterG;
         const size_t a_bytes = ((size_t)(g.OC - 1) * lda + M) * 4;
         const int rc2 = narrow128 ? launch_wgrad<1, 2, 2, 2, false, 4>(ogT, a_bytes, lda, bsrc, dst, g.OC, (int)Kf, (int)M, splits, sps)

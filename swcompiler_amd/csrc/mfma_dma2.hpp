@@ -261,20 +261,26 @@ __device__ __forceinline__ void dma2_tile_body(const float *__restrict__ A, unsi
     const int nk = (k_end - k_begin + BK - 1) / BK;
     int rd_stage = 0, wr_stage = STAGES - 1;
     const bool computes = !SKIP || n0 + col0 < N;   // (wavefront-uniform)
+    if (SKIP && !computes) {
+        // The slices' barriers and this wavefront's share of the loads, nothing else.  (A loop of its own: as a branch
+        // inside the loop below it made the compiler carry the accumulators through the loop in VGPRs and copy them
+        // into the AGPRs in every slice.)
+        for (int kt = 0; kt < nk; ++kt) {
+            float *__restrict__ wr = lds + wr_stage * T::kStageFloats;
+            ring_sync<MID ? (STAGES - 3) * T::kLoads : (STAGES - 2) * T::kLoads>();
+#pragma unroll
+            for (int j = 0; j < T::kLoads; ++j) issue(wr, j);
+            k0 += BK;
+            wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
+        }
+        wait_vmcnt<0>();
+        return;   // (nothing of this wavefront's tile lies inside the matrix)
+    }
     for (int kt = 0; kt < nk; ++kt) {
         const int nx_stage = rd_stage + 1 == STAGES ? 0 : rd_stage + 1;
         float *__restrict__ wr = lds + wr_stage * T::kStageFloats;
         const float *__restrict__ rd = lds + rd_stage * T::kStageFloats;
         const float *__restrict__ nx = lds + nx_stage * T::kStageFloats;
-        if (SKIP && !computes) {   // the slice's barrier and this wavefront's share of the loads, nothing else
-            ring_sync<MID ? (STAGES - 3) * T::kLoads : (STAGES - 2) * T::kLoads>();
-#pragma unroll
-            for (int j = 0; j < T::kLoads; ++j) issue(wr, j);
-            k0 += BK;
-            rd_stage = nx_stage;
-            wr_stage = wr_stage + 1 == STAGES ? 0 : wr_stage + 1;
-            continue;
-        }
         if constexpr (!MID) {
             ring_sync<(STAGES - 2) * T::kLoads>();
 #pragma unroll
