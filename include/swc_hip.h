@@ -104,9 +104,12 @@ int swc_hip_set_workspace(void *dptr, size_t bytes);
  * fails instead, and so does swc_hip_set_workspace). */
 int swc_hip_enable_auto_workspace(int enable);
 /* No counterpart in the reference.  Workspace a matrixMatrixMul_f /
- * matrixMatrixFCBias_f call of this shape uses on the initialised device (0 for most shapes: only products with few output tiles and a K
- * of hundreds are split over K).  A generated program takes the maximum over its
- * calls and provides that much with swc_hip_set_workspace. */
+ * matrixMatrixFCBias_f call of this shape uses on the initialised device (0 for
+ * most shapes: only products with few output tiles and a K of hundreds are
+ * split over K, and only on operands the direct-to-LDS kernels take — rows on
+ * 16-byte boundaries; for others the call needs none and the figure is an upper
+ * bound).  A generated program takes the maximum over its calls and provides
+ * that much with swc_hip_set_workspace. */
 size_t swc_hip_gemm_workspace_bytes(int m, int n, int k);
 /* The same for a conv2d_f / conv2dFused_f call of these shapes (arguments as in
  * swc_hip_conv2d_f, tensors assumed 16-byte aligned): the output tiles that are
@@ -114,8 +117,9 @@ size_t swc_hip_gemm_workspace_bytes(int m, int n, int k);
  * their partial sums kept here; a layer whose input-channel count is no multiple
  * of 4 (and that is too large for the direct first-layer kernel) is computed on
  * zero-padded copies of input and filter, which live here too, and so does the
- * filter copy of a call with more than one group.  Without a workspace large
- * enough the library allocates its own at the first such call. */
+ * filter copy of a call with more than one group.  The size queries do not see
+ * the pointers: each answers for whichever alignment of the operands (on
+ * 16-byte boundaries or not) needs the most. */
 size_t swc_hip_conv2d_workspace_bytes(const size_t *odims, const size_t *idims, const size_t *fdims,
                                       const size_t *kernels, const size_t *strides, const size_t *pads,
                                       size_t group);

@@ -2825,9 +2825,10 @@ size_t swc_hip_conv2dFusedMaxpool_workspace_bytes(const size_t *cdims, const siz
     const size_t conv = swc_hip_conv2d_workspace_bytes(cdims, idims, fdims, kernels, strides, pads, group);
     const ConvGeom g = make_geom(cdims, idims, fdims, kernels, strides, pads);
     if (g.M == 0 || g.OC == 0) return 0;
-    if (pool_is_2x2(cdims, pdims, pool_kernels, pool_strides, pool_pads) && conv_pool_fusable(g, nullptr, nullptr, nullptr))
-        return conv;
-    return align256((size_t)g.M * g.OC * 4) + conv;   // the convolution's own output, then pooled by maxpool_f's kernel
+    // The pool runs in the convolution's epilogue only for operands on 16-byte boundaries; otherwise the convolution's
+    // own output goes through the workspace and maxpool_f's kernel pools it.  The query does not see the pointers, so
+    // it answers for the case that needs more.
+    return align256((size_t)g.M * g.OC * 4) + conv;
 }
 
 int swc_hip_conv2dFusedMaxpool_f(float *output, const float *input, const float *filter, const float *bias,
@@ -2881,10 +2882,14 @@ size_t swc_hip_conv2dGrad_workspace_bytes(const size_t *odims, const size_t *idi
     const ConvGeom g = make_geom(odims, idims, fdims, kernels, strides, pads);
     const size_t f_elems = fdims[0] * fdims[1] * fdims[2] * fdims[3];
     if (g.M == 0 || g.OC == 0 || f_elems == 0 || idims[0] * idims[1] * idims[2] * idims[3] == 0) return 0;
-    // operands on 16-byte boundaries (every tensor of a generated program) or not: the larger of the two layouts
-    const size_t a = grad_layout(g, odims, idims, fdims, kernels, true, true, true).total();
-    const size_t u = grad_layout(g, odims, idims, fdims, kernels, false, false, false).total();
-    return (group > 1 ? align256(f_elems * 4) : 0) + (a > u ? a : u);
+    // each of the three alignment tests of the call (16-byte boundaries or not) picks kernels with their own needs, and
+    // the query does not see the pointers: the largest of the eight layouts
+    size_t most = 0;
+    for (int c = 0; c < 8; ++c) {
+        const size_t t = grad_layout(g, odims, idims, fdims, kernels, c & 1, c & 2, c & 4).total();
+        most = t > most ? t : most;
+    }
+    return (group > 1 ? align256(f_elems * 4) : 0) + most;
 }
 
 int swc_hip_conv2dGrad_f(float *inputG, float *filterG, float *biasG, const float *outputG, const float *input,

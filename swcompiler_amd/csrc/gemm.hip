@@ -691,9 +691,11 @@ int launch_splitk(const float *a, const float *b, float *c, int m, int n, int k,
     using T = Dma2Tile<TM, TN, WM, STAGES, 4>;
     const size_t need = (size_t)splits * m * n * sizeof(float);
     float *part = fixed.ptr;
-    if (part) {
+    if (part) {   // (the entry point that allocates nothing: refused here, where the kernel is known, before any launch)
         if (need > fixed.bytes)
-            return fail(SWC_HIP_EINVAL, "gemm (split-K): the partial tiles take %zu bytes, the fixed scratch holds %zu",
+            return fail(SWC_HIP_EINVAL, "swc_hip_matrixMatrixFCBias_noalloc_f: a %d x %d x %d product is cut into %d ranges of K "
+                        "whose partial tiles take %zu bytes, more than the %zu bytes of fixed scratch "
+                        "(SWC_HIP_NOALLOC_SCRATCH_BYTES); use swc_hip_matrixMatrixFCBias_f with a workspace", m, n, k, splits,
                         need, fixed.bytes);
     } else {
         part = static_cast<float *>(workspace(need, "gemm (split-K)"));
@@ -907,14 +909,8 @@ int swc_hip_matrixMatrixFCBias_noalloc_f(int m, int n, int k, const float *a, in
     const char *who = "swc_hip_matrixMatrixFCBias_noalloc_f";
     float *fixed = (g_scratch_device >= 0 && g_scratch_device < kMaxDevices) ? g_scratch_ptr[g_scratch_device] : nullptr;
     if (!fixed) return fail(SWC_HIP_ERUNTIME, "%s: the fixed scratch array was not located at swc_hip_init", who);
-    if (m > 0 && n > 0 && k > 0) {   // refused before anything is launched
-        int splits = 0, sps = 0;
-        if (splitk_decision(m, n, k, splits, sps) && (size_t)splits * m * n * sizeof(float) > SWC_HIP_NOALLOC_SCRATCH_BYTES)
-            return fail(SWC_HIP_EINVAL, "%s: a %d x %d x %d product is cut into %d ranges of K whose partial tiles take %zu "
-                        "bytes, more than the %zu bytes of fixed scratch (SWC_HIP_NOALLOC_SCRATCH_BYTES); use "
-                        "swc_hip_matrixMatrixFCBias_f with a workspace", who, m, n, k, splits,
-                        (size_t)splits * m * n * sizeof(float), (size_t)SWC_HIP_NOALLOC_SCRATCH_BYTES);
-    }
+    // (a product whose partial tiles exceed the array is refused by the dispatch, at the one place that knows which
+    // kernel the shape and the operands' alignment select, before anything is launched)
     return gemm_dispatch(who, m, n, k, a, lda, b, ldb, bias, c, ldc, relu, 0,
                          PartialStore{fixed, (size_t)SWC_HIP_NOALLOC_SCRATCH_BYTES});
 }

@@ -654,6 +654,40 @@ POOLED_CONVS = [
 ]
 
 
+@pytest.mark.parametrize("shift", [0, 1])
+def test_pooled_conv_query_covers_unaligned_operands(rt, oracle, shift):
+    """swc_hip_conv2dFusedMaxpool_workspace_bytes does not see the pointers: an input that is not on a 16-byte boundary
+    takes the call off the pooling epilogue (the convolution's own output then goes through the workspace).  With
+    auto-workspace off and a buffer of exactly the queried size the call must run either way."""
+    print("case pooled conv query, shift", shift, flush=True)
+    idims, fdims, pads, pool = (2, 12, 12, 32), (64, 3, 3, 32), (1, 1, 1, 1), ((2, 2), (2, 2))
+    rng = np.random.default_rng(5)
+    x = rng.integers(-3, 4, idims).astype(np.float32)
+    f = rng.integers(-2, 3, fdims).astype(np.float32)
+    b = rng.integers(-2, 3, fdims[0]).astype(np.float32)
+    want = oracle.maxpool(oracle.relu(oracle.conv2d(x, f, b, pads=pads)), *pool)
+    base = rt.empty((x.size + 4,))
+    dx = base.offset_view(shift, idims)
+    rt.upload_into(dx, x)
+    df, db = up(rt, f, b)
+    out = rt.empty(want.shape)
+    need = rt.conv2d_maxpool_workspace_bytes(idims, fdims, (1, 1), pads, pool)
+    ws = rt.empty((max(need, 4) // 4,))
+    rt.sync()
+    rt.set_workspace(ws)
+    rt.enable_auto_workspace(False)
+    try:
+        rt.conv2d(dx, df, db, pads=pads, relu=True, pool=pool, out=out)
+        name = rt.last_kernel()
+        got = out.numpy()
+    finally:
+        rt.sync()
+        rt.set_workspace(None)
+        rt.enable_auto_workspace(True)
+    assert name.endswith("(pooled)") == (shift == 0), name
+    assert_bit_exact(got, want, f"pooled conv, input shifted by {shift} floats")   # integer-valued data: exact in any order
+
+
 @pytest.mark.parametrize("idims,fdims,pads", POOLED_CONVS)
 @pytest.mark.parametrize("slots", [None, "7"])
 def test_conv_with_the_pooling_in_its_epilogue(rt, oracle, idims, fdims, pads, slots, switch_env):

@@ -383,3 +383,48 @@ def test_conv2dGrad_full_size_properties(rt, oracle):
     ig3, fg3, bg3 = (t.numpy() for t in rt.conv2dGrad(dx, df, rt.upload(og + og2), (3, 3), (1, 1), (1, 1, 1, 1)))
     assert_bit_exact(ig3, ig + ig2, "inputG linear")
     assert_bit_exact(fg3, fg + fg2, "filterG linear")
+
+
+# ------------------------------------------------------------ the size queries hold for any operand alignment
+def _shifted(rt, host, shift):
+    """`host` on the device, `shift` floats past a 256-byte boundary (shift % 4 != 0: not on a 16-byte boundary)"""
+    base = rt.empty((host.size + shift,))
+    view = base.offset_view(shift, host.shape)
+    rt.upload_into(view, host)
+    return base, view
+
+
+@pytest.mark.parametrize("case", range(8))
+def test_conv2dGrad_query_covers_every_alignment(rt, oracle, case):
+    """The query does not see the pointers; each of the call's three alignment tests (input, outputG, filterG) picks
+    kernels with their own scratch needs.  With auto-workspace off and a buffer of exactly the queried size the call
+    must run — and give the same gradients — for all eight combinations."""
+    print("case conv2dGrad alignment", case, flush=True)
+    idims, fdims, st, pd = (2, 14, 14, 8), (12, 3, 3, 8), (1, 1), (1, 1, 1, 1)
+    rng = np.random.default_rng(77)
+    n, oh, ow, _ = pool_out_dims(idims, fdims[1:3], st, pd)
+    x = rng.integers(-3, 4, idims).astype(np.float32)
+    f = rng.integers(-2, 3, fdims).astype(np.float32)
+    og = rng.integers(-2, 3, (n, oh, ow, fdims[0])).astype(np.float32)
+    want = oracle.conv2dGrad(x, f, og, fdims[1:3], st, pd)
+    keep = []
+    xb, dx = _shifted(rt, x, 1 if case & 1 else 0)
+    ob, dog = _shifted(rt, og, 1 if case & 2 else 0)
+    fgb = rt.empty((f.size + 1,))
+    fg = fgb.offset_view(1 if case & 4 else 0, fdims)
+    df, ig, bg = rt.upload(f), rt.empty(idims), rt.empty((fdims[0],))
+    keep += [xb, ob, fgb]
+    need = rt.conv2dGrad_workspace_bytes(idims, fdims, st, pd)
+    ws = rt.empty((max(need, 4) // 4,))
+    rt.sync()
+    rt.set_workspace(ws)
+    rt.enable_auto_workspace(False)
+    try:
+        rt.conv2dGrad(dx, df, dog, fdims[1:3], st, pd, out=(ig, fg, bg))
+        got = [ig.numpy(), fg.numpy(), bg.numpy()]
+    finally:
+        rt.sync()
+        rt.set_workspace(None)
+        rt.enable_auto_workspace(True)
+    for g, w, name in zip(got, want, ("inputG", "filterG", "biasG")):
+        assert_bit_exact(g, w, f"{name}, alignment case {case}")   # integer-valued data: exact in any order

@@ -21,7 +21,8 @@ asserts what can hold: the device result is no farther from the float64 value
 than the reference's own result is (to within a quarter, both being maxima over
 a tensor: the excess over 1e-4 is the rounding noise both share, not an error
 of the device — in the rows below the device is usually the closer one), and
-the two never differ by more than 1e-3 floored.  ReLU, add and max-pool must be bit-exact.  Batches are reduced where the single-threaded oracle would
+the distance stays within 1.25 x the figure pinned for that row (PINNED; the
+measured table is kept in profiles/parity_report.txt).  ReLU, add and max-pool must be bit-exact.  Batches are reduced where the single-threaded oracle would
 take minutes; the wide MLP additionally runs at its FULL size on the GPU with
 twelve sampled rows through the oracle, so that the very launches the headline
 figure times (4096 x 784 x 4096 and 4096^3 on 256 x 256 tiles) have oracle rows
@@ -43,6 +44,29 @@ def rt():
     return runtime()
 
 
+# Today's distance (the larger of strict and floored) of every row that exceeds 1e-4 for the reason given in the
+# module text.  A row may drift to 1.25 x its figure (a different split of K reorders the sums); beyond that, or for
+# a row that is not listed, the test fails: a regression below the generic 1e-3 does not pass unnoticed.
+PINNED = {
+    'cfg1 FC 8x784x512 (+bias)': 1.36e-04,
+    'cfg2 FC 64x784x4096 (+bias)': 3.15e-04,
+    'cfg2 FC 64x4096x4096 (+bias)': 5.29e-04,
+    'cfg2 FC 64x4096x10 (+bias)': 1.93e-04,
+    'cfg3 FC 32x800x500 (+bias)': 1.53e-04,
+    'cfg2 full size, layer 1 (784->4096), 12 rows': 1.30e-04,
+    'cfg2 full size, layer 2 (4096->4096), 12 rows': 4.71e-04,
+    'cfg2 full size, layer 3 (4096->10), 12 rows': 3.71e-04,
+    'cfg3 conv2 [16, 12, 12, 20] * [50, 5, 5, 20]': 2.37e-04,
+    'cfg4 conv1 [2, 56, 56, 64] * [64, 3, 3, 64]': 1.69e-04,
+    'cfg4 conv1+BN+ReLU fused': 1.53e-04,
+    'cfg4 conv2 [2, 56, 56, 64] * [128, 3, 3, 64]': 1.14e-04,
+    'cfg4 conv3 [2, 28, 28, 128] * [128, 3, 3, 128]': 4.95e-04,
+    'cfg4 conv3+BN+ReLU fused': 4.07e-04,
+    'cfg4 conv4 [2, 28, 28, 128] * [128, 3, 3, 128]': 2.37e-04,
+    'cfg4 conv4+BN+ReLU fused': 3.03e-04,
+}
+
+
 def strict_on_significant(got, want):
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
     big = np.abs(want) >= 1e-3 * np.max(np.abs(want))
@@ -59,7 +83,8 @@ def check(name, got, want, exact=None):
     assert exact is not None, f"{name}: strict {s:.2e}, floored {f:.2e} exceed 1e-4"
     dev64, ref64 = rel_err(got, exact), rel_err(want, exact)
     print(line + f"  | vs float64: device {dev64:9.2e}  reference {ref64:9.2e}", flush=True)
-    assert f < 1e-3, f"{name}: floored {f:.2e}"
+    assert name in PINNED, f"{name}: strict {s:.2e}, floored {f:.2e} exceed 1e-4 and the row has no pinned figure"
+    assert max(s, f) <= 1.25 * PINNED[name], f"{name}: {max(s, f):.2e} against the pinned {PINNED[name]:.2e}"
     # (maxima over a tensor: two evaluations of equal quality tie within a few percent of each other)
     assert dev64 <= 1.25 * ref64, f"{name}: the device result is farther from float64 ({dev64:.2e}) than the reference's ({ref64:.2e})"
 

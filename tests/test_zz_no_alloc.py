@@ -80,3 +80,76 @@ def test_noalloc_rejects_sizes_beyond_the_scratch(rt):
     da, dw, out = rt.empty((m, k)), rt.empty((k, n)), rt.empty((m, n))   # never read: the call is refused first
     with pytest.raises(SwcHipError, match="SWC_HIP_NOALLOC_SCRATCH_BYTES"):
         rt.fcbias_noalloc(da, dw, None, out=out)
+
+
+def test_noalloc_recorded_in_a_graph(rt):
+    """the use the header names: the call recorded into a HIP graph with no workspace anywhere, replayed several times
+    with eager work and synchronisations in between; every replay gives the eager result"""
+    rng = np.random.default_rng(21)
+    m, n, k = 192, 500, 1056
+    assert rt.gemm_workspace_bytes(m, n, k) > 0
+    a, w, b, da, dw, db = _operands(rt, rng, m, n, k)
+    want = rt.fcbias_noalloc(da, dw, db, relu=True).numpy()
+    out, other = rt.empty((m, n)), rt.empty((m, n))
+    rt.sync()
+    rt.set_workspace(None)
+    rt.enable_auto_workspace(False)
+    try:
+        graph = rt.capture(lambda: rt.fcbias_noalloc(da, dw, db, relu=True, out=out))
+        for replay in range(4):
+            rt.relu(other, out=out)                        # eager work between replays: overwrites the graph's output,
+            rt.fcbias_noalloc(da, dw, db, out=other)       # and uses the same scratch array
+            rt.sync()
+            rt.graph_launch(graph)
+            rt.sync()
+            assert_bit_exact(out.numpy(), want, f"replay {replay}")
+        rt.graph_destroy(graph)
+    finally:
+        rt.enable_auto_workspace(True)
+
+
+def test_noalloc_leaves_free_device_memory_unchanged(rt):
+    """hipMemGetInfo before and after a series of calls (after one warm-up call, which loads the kernels)"""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    rng = np.random.default_rng(22)
+    a, w, b, da, dw, db = _operands(rt, rng, 192, 500, 1056)
+    out = rt.empty((192, 500))
+    rt.sync()
+    rt.set_workspace(None)
+    rt.enable_auto_workspace(False)
+
+    def free_bytes():
+        free, total = C.c_size_t(), C.c_size_t()
+        assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value
+
+    try:
+        rt.fcbias_noalloc(da, dw, db, out=out)
+        rt.sync()
+        before = free_bytes()
+        for _ in range(5):
+            rt.fcbias_noalloc(da, dw, db, relu=True, out=out)
+        rt.sync()
+        assert free_bytes() == before
+    finally:
+        rt.enable_auto_workspace(True)
+
+
+def test_noalloc_takes_operands_whose_kernel_needs_no_scratch(rt):
+    """a shape whose split would overflow the array, on an A that is not on a 16-byte boundary: such operands run on
+    the register-staged kernel, which is never split — the call is served, with the ordinary entry point's bits"""
+    rng = np.random.default_rng(23)
+    m, n, k = 64, 4096, 4096
+    assert rt.gemm_workspace_bytes(m, n, k) > NOALLOC_SCRATCH_BYTES
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    w = (rng.standard_normal((k, n), dtype=np.float32) / np.sqrt(k)).astype(np.float32)
+    base = rt.empty((m * k + 4,))
+    da = base.offset_view(1, (m, k))
+    rt.upload_into(da, a)
+    dw = rt.upload(w)
+    want = rt.fcbias(da, dw, None).numpy()
+    name = rt.last_kernel()
+    assert "splitk" not in name, name
+    got = rt.fcbias_noalloc(da, dw, None).numpy()
+    assert_bit_exact(got, want, "noalloc on an unaligned A")
