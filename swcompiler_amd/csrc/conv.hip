@@ -2825,9 +2825,14 @@ size_t swc_hip_conv2dFusedMaxpool_workspace_bytes(const size_t *cdims, const siz
     const size_t conv = swc_hip_conv2d_workspace_bytes(cdims, idims, fdims, kernels, strides, pads, group);
     const ConvGeom g = make_geom(cdims, idims, fdims, kernels, strides, pads);
     if (g.M == 0 || g.OC == 0) return 0;
-    // The pool runs in the convolution's epilogue only for operands on 16-byte boundaries; otherwise the convolution's
-    // own output goes through the workspace and maxpool_f's kernel pools it.  The query does not see the pointers, so
-    // it answers for the case that needs more.
+    // Where the tile kernels pool in their epilogue they do so only for operands on 16-byte boundaries; otherwise the
+    // convolution's own output goes through the workspace and maxpool_f's kernel pools it.  The query does not see the
+    // pointers: it answers for the alignment that needs more (the direct kernel of first layers, and layers computed on
+    // padded copies, pool whatever the alignment).
+    const void *off_grid = reinterpret_cast<const void *>(4);
+    if (pool_is_2x2(cdims, pdims, pool_kernels, pool_strides, pool_pads) && conv_pool_fusable(g, nullptr, nullptr, nullptr) &&
+        conv_pool_fusable(g, off_grid, off_grid, off_grid))
+        return conv;
     return align256((size_t)g.M * g.OC * 4) + conv;
 }
 
