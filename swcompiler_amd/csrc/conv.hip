@@ -922,6 +922,17 @@ __device__ __forceinline__ int select_by_mask(unsigned long long mask, int if_se
 }
 #endif
 
+// The argument record as it lies in the kernel-argument segment, for the fields that are needed only once the K loop
+// is over: read again there (scalar loads that hit the scalar cache) instead of kept in scalar registers across the
+// loop, which has none to spare — the compiler parked them in lanes of a vector register (44 v_writelane at the
+// start, some 60 v_readlane behind the loop, per workgroup: vector instructions that take matrix-pipe cycles).
+typedef const __attribute__((address_space(4))) WinArgs *WinArgsInSegment;
+__device__ __forceinline__ WinArgsInSegment win_args_again() {
+    WinArgsInSegment p = (WinArgsInSegment)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(p));   // a value the compiler cannot trace back to the loads at the kernel's entry
+    return p;
+}
+
 template <bool POOL, bool RES>
 __global__ __launch_bounds__(kThreads) void conv_win(const WinArgs a) {
 #if __HIP_DEVICE_COMPILE__
@@ -1159,20 +1170,24 @@ __global__ __launch_bounds__(kThreads) void conv_win(const WinArgs a) {
             // Lane (l32, h) holds column `col` of the windows wbase + 2 q, four pixels each (accumulator registers
             // 4q .. 4q + 3).  One 32-bit offset per window; the window's other pixels (and those of the second
             // summand) at scalar offsets from it.
-            const __amdgpu_buffer_rsrc_t rsrc_out = make_rsrc(a.out, a.out_bytes);
-            const int N = a.N, s_px = N * 4, s_row = a.OW * N * 4;
+            const WinArgsInSegment z = win_args_again();
+            const Magic d_pw{z->d_pw.mul, z->d_pw.shift};
+            const int pw = z->pw, nwin = z->nwin;
+            const bool relu = z->ep.relu != 0;
+            const __amdgpu_buffer_rsrc_t rsrc_out = make_rsrc(z->out, z->out_bytes);
+            const int N = z->N, s_px = N * 4, s_row = z->OW * N * 4;
             const int wbase = (m0 >> 2) + wave_m * 8 + h;
-            const bool bn = a.ep.bn_mean != nullptr;
+            const bool bn = z->ep.bn_mean != nullptr;
             int voff[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int w = wbase + 2 * q;
-                const int at = POOL ? (w * N + col) * 4 : ((w + magic_div(w, a.d_pw) * a.pw) * 2 * N + col) * 4;
-                voff[q] = (w < a.nwin && col < N) ? at : kOutOfRange;
+                const int at = POOL ? (w * N + col) * 4 : ((w + magic_div(w, d_pw) * pw) * 2 * N + col) * 4;
+                voff[q] = (w < nwin && col < N) ? at : kOutOfRange;
             }
             float add[4][4];
             if constexpr (RES) {
-                const __amdgpu_buffer_rsrc_t rsrc_res = make_rsrc(a.ep.residual, (unsigned)a.nwin * 16u * (unsigned)N);
+                const __amdgpu_buffer_rsrc_t rsrc_res = make_rsrc(z->ep.residual, (unsigned)nwin * 16u * (unsigned)N);
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     add[q][0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_res, voff[q], 0, 0));
@@ -1181,27 +1196,38 @@ __global__ __launch_bounds__(kThreads) void conv_win(const WinArgs a) {
                     add[q][3] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_res, voff[q], s_row + s_px, 0));
                 }
             }
+            // (batchnorm and ReLU or not: four straight-line copies behind wavefront-uniform branches — as selects on the
+            // two flags they were two more vector instructions for every one of the 16 elements)
+            auto finish = [&](auto bn_c, auto relu_c) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                float x[4];
+                for (int q = 0; q < 4; ++q) {
+                    float x[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    x[e] = acc[0][0][4 * q + e] + cp.bias;
-                    if (bn) x[e] = fmaf(x[e] - cp.mean, cp.slope, cp.beta);
-                    if constexpr (RES) x[e] += add[q][e];
-                    if (a.ep.relu) x[e] = (x[e] > 0.f) ? x[e] : 0.f;
+                    for (int e = 0; e < 4; ++e) {
+                        x[e] = acc[0][0][4 * q + e] + cp.bias;
+                        if constexpr (decltype(bn_c)::value) x[e] = fmaf(x[e] - cp.mean, cp.slope, cp.beta);
+                        if constexpr (RES) x[e] += add[q][e];
+                        if constexpr (decltype(relu_c)::value) x[e] = (x[e] > 0.f) ? x[e] : 0.f;
+                    }
+                    if constexpr (POOL) {
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, window_max(x[0], x[1], x[2], x[3])), rsrc_out, voff[q], 0, 0);
+                    } else {
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[0]), rsrc_out, voff[q], 0, 0);
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[1]), rsrc_out, voff[q], s_px, 0);
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[2]), rsrc_out, voff[q], s_row, 0);
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[3]), rsrc_out, voff[q], s_row + s_px, 0);
+                    }
                 }
-                if constexpr (POOL) {
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, window_max(x[0], x[1], x[2], x[3])), rsrc_out, voff[q], 0, 0);
-                } else {
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[0]), rsrc_out, voff[q], 0, 0);
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[1]), rsrc_out, voff[q], s_px, 0);
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[2]), rsrc_out, voff[q], s_row, 0);
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[3]), rsrc_out, voff[q], s_row + s_px, 0);
-                }
+            };
+            if (bn) {
+                if (relu) finish(std::true_type{}, std::true_type{});
+                else finish(std::true_type{}, std::false_type{});
+            } else {
+                if (relu) finish(std::false_type{}, std::true_type{});
+                else finish(std::false_type{}, std::false_type{});
             }
         } else {
-            float *slot = a.part + (size_t)(2 * share + (piece ? 1 : 0)) * (BM * BN);
+            float *slot = win_args_again()->part + (size_t)(2 * share + (piece ? 1 : 0)) * (BM * BN);
             store_tile_impl<1, 1, false, false>(acc, slot, (size_t)BN, BM, BN, wave_m * 32, wave_n * 32, lane, Epilogue{});
         }
     }
