@@ -1253,33 +1253,52 @@ __global__ __launch_bounds__(256) void conv_sk_finish(float *__restrict__ out, c
     // the sum over the pieces of columns c .. c + 3 of row r of the tile
     auto sum_pieces = [&](int r, int c) {
         float4 sum = {0.f, 0.f, 0.f, 0.f};
-        for (int s0 = s_lo; s0 <= s_hi; s0 += 4) {   // four pieces' loads in flight, added in K order
-            float4 v[4];
+        // sixteen pieces' loads in flight (a tile is cut into 8 or 16 pieces on a whole chip: one round trip to memory
+        // instead of two to four, in a kernel that is little else), added in K order
+        constexpr int kAtOnce = 16;
+        for (int s0 = s_lo; s0 <= s_hi; s0 += kAtOnce) {
+            float4 v[kAtOnce];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int i = 0; i < kAtOnce; ++i) {
                 const int s = s0 + i;
                 const int begin = s * sk.q + (s < sk.r ? s : sk.r);
                 const float *slot = part + (size_t)(2 * s + (begin < first ? 1 : 0)) * (BM * BN);
                 v[i] = s <= s_hi ? *reinterpret_cast<const float4 *>(slot + r * BN + c) : make_float4(0.f, 0.f, 0.f, 0.f);
             }
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < kAtOnce; ++i)
                 if (s0 + i <= s_hi) sum.x += v[i].x, sum.y += v[i].y, sum.z += v[i].z, sum.w += v[i].w;
         }
         return sum;
     };
-    // the epilogue of store_tile_impl on the four columns; `pix` = the row's pixel in the output
-    auto finish = [&](float4 sum, int col, size_t pix, float (&x)[4]) {
+    // the epilogue of store_tile_impl on the four columns; `pix` = the row's pixel in the output.  The columns'
+    // parameters are fetched (and the batchnorm slope formed) before the pieces are asked for, so that their latency
+    // and arithmetic run beside the pieces' loads instead of behind them.
+    struct Columns {
+        float bias[4], mean[4], slope[4], beta[4];
+    };
+    auto columns = [&](int col) {
+        Columns p;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const bool in = col + e < N;
+            p.bias[e] = (in && ep.bias) ? ep.bias[col + e] : 0.f;
+            p.mean[e] = p.beta[e] = 0.f, p.slope[e] = 1.f;
+            if (in && ep.bn_mean) {
+                const float ve = ep.bn_var[col + e] + ep.eps;
+                p.slope[e] = (float)((double)ep.bn_scale[col + e] / sqrt((double)ve));
+                p.mean[e] = ep.bn_mean[col + e], p.beta[e] = ep.bn_bias[col + e];
+            }
+        }
+        return p;
+    };
+    auto finish = [&](float4 sum, const Columns &p, int col, size_t pix, float (&x)[4]) {
         x[0] = sum.x, x[1] = sum.y, x[2] = sum.z, x[3] = sum.w;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             if (col + e >= N) break;
-            float y = x[e] + (ep.bias ? ep.bias[col + e] : 0.f);
-            if (ep.bn_mean) {
-                const float ve = ep.bn_var[col + e] + ep.eps;
-                const float slope = (float)((double)ep.bn_scale[col + e] / sqrt((double)ve));
-                y = fmaf(y - ep.bn_mean[col + e], slope, ep.bn_bias[col + e]);
-            }
+            float y = x[e] + p.bias[e];
+            if (ep.bn_mean) y = fmaf(y - p.mean[e], p.slope[e], p.beta[e]);
             if (ep.residual) y += ep.residual[pix * N + col + e];
             if (ep.relu) y = (y > 0.f) ? y : 0.f;
             x[e] = y;
@@ -1304,9 +1323,10 @@ __global__ __launch_bounds__(256) void conv_sk_finish(float *__restrict__ out, c
             const int r = blockIdx.y * 16 + i / (BN / 4), c = (i % (BN / 4)) * 4;
             const int row = tile_m * BM + r, col = tile_n * BN + c;
             if (row >= M || col >= N) continue;
+            const Columns p = columns(col);
             const size_t pix = pixel(row);
             float x[4];
-            finish(sum_pieces(r, c), col, pix, x);
+            finish(sum_pieces(r, c), p, col, pix, x);
             store4(out + pix * N + col, col, x);
         }
     } else {
@@ -1318,8 +1338,9 @@ __global__ __launch_bounds__(256) void conv_sk_finish(float *__restrict__ out, c
             const int r = blockIdx.y * 16 + rl;
             const int row = tile_m * BM + r, col = tile_n * BN + c;
             if (row >= M || col >= N) continue;
+            const Columns p = columns(col);
             float x[4];
-            finish(sum_pieces(r, c), col, pixel(row), x);
+            finish(sum_pieces(r, c), p, col, pixel(row), x);
 #pragma unroll
             for (int e = 0; e < 4; ++e) done[rl][c + e] = x[e];
         }
