@@ -2221,10 +2221,10 @@ struct Im2colB {
     // A lane follows its pixel from slice to slice (+32 pixels) by additions and selects only: multiplications, and
     // divergent branches between the MFMAs of a slice, cost the matrix pipe more than the loads they feed.
     int ys_end, xs_end;          // OH * sh, OW * sw: where the scaled row / column wraps
-    int dxs, dys, dimg, doff;    // a slice's step: columns (x sw), rows (x sh), images, bytes — before carries
+    int dxs, dys, doff;          // a slice's step: columns (x sw), rows (x sh), bytes (whole images included) — before carries
     int row_carry, img_carry;    // bytes added when the column wraps into the next row / the row into the next image
     struct Lane {
-        int img, ys, xs, off;    // image, oy * sh, ox * sw, byte offset of input pixel (img, ys, xs)
+        int ys, xs, off;         // oy * sh, ox * sw, byte offset of the input pixel (image, ys, xs)
         int ty, tx, tap, krow;   // tap row - pt, tap column - pl, byte offset of the tap and channel (+ descriptor shift), row in the slice
         bool ok;
     };
@@ -2236,7 +2236,7 @@ struct Im2colB {
         b.ys_end = g.OH * g.sh, b.xs_end = g.OW * g.sw;
         const int per_img = g.OH * g.OW, qi = BK / per_img, qy = BK % per_img / g.OW, rx = BK % per_img % g.OW;
         const int px = g.C * 4;   // bytes per input pixel
-        b.dxs = rx * g.sw, b.dys = qy * g.sh, b.dimg = qi;
+        b.dxs = rx * g.sw, b.dys = qy * g.sh;
         b.doff = ((qi * g.H + qy * g.sh) * g.W + rx * g.sw) * px;
         b.row_carry = (g.sh * g.W - g.OW * g.sw) * px;
         b.img_carry = (g.H - g.OH * g.sh) * g.W * px;
@@ -2250,11 +2250,10 @@ struct Im2colB {
     __device__ __forceinline__ Lane init(int krow, int col, bool col_ok, int imm, int k_begin) const {
         Lane s;
         const int pix = k_begin + krow;
-        const int ox = pix % OW, t = pix / OW, oy = t % OH;
-        s.img = t / OH;
+        const int ox = pix % OW, t = pix / OW, oy = t % OH, img = t / OH;
         s.ys = oy * sh;
         s.xs = ox * sw;
-        s.off = ((s.img * H + s.ys) * W + s.xs) * C * 4;
+        s.off = ((img * H + s.ys) * W + s.xs) * C * 4;
         const int tap = col / C, ky = tap / kw;
         s.ty = ky - pt;
         s.tx = tap - ky * kw - pl;
@@ -2265,8 +2264,8 @@ struct Im2colB {
     }
     __device__ __forceinline__ int voffset(const Lane &s, int k0, int k_end) const {
         const int iy = s.ys + s.ty, ix = s.xs + s.tx;
-        const bool valid = s.ok & (k0 + s.krow < k_end) & (s.img < nimg) & ((unsigned)iy < (unsigned)H) &
-                           ((unsigned)ix < (unsigned)W);
+        // (k_end is at most the pixel count, so a row of the slice below k_end lies in one of the images)
+        const bool valid = s.ok & (k0 + s.krow < k_end) & ((unsigned)iy < (unsigned)H) & ((unsigned)ix < (unsigned)W);
         const int off = s.off + s.tap;
         return valid ? off : kOutOfRange;
     }
@@ -2281,7 +2280,6 @@ struct Im2colB {
         const bool cy = s.ys >= ys_end;
         s.ys -= cy ? ys_end : 0;
         s.off += cy ? img_carry : 0;
-        s.img += dimg + (cy ? 1 : 0);
     }
 #endif
 };
