@@ -2265,7 +2265,7 @@ struct Im2colB {
     __device__ __forceinline__ int voffset(const Lane &s, int k0, int k_end) const {
         const int iy = s.ys + s.ty, ix = s.xs + s.tx;
         // (k_end is at most the pixel count, so a row of the slice below k_end lies in one of the images)
-        const bool valid = s.ok & (k0 + s.krow < k_end) & ((unsigned)iy < (unsigned)H) & ((unsigned)ix < (unsigned)W);
+        const bool valid = s.ok & (s.krow < k_end - k0) & ((unsigned)iy < (unsigned)H) & ((unsigned)ix < (unsigned)W);   // (k_end - k0: scalar)
         const int off = s.off + s.tap;
         return valid ? off : kOutOfRange;
     }
